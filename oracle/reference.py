@@ -1,0 +1,362 @@
+"""CPU oracle for the quantized linear-layer path (TEST INFRASTRUCTURE ONLY).
+
+This module restates, in plain numpy, the arithmetic that iMMIQ/orinfer's E8P
+Q4A8 / Q2A8 / W8A8 kernels implement.  It is the checker for the HIP kernels
+and the timed CPU baseline; it is never imported by the product package
+(`orinfer_amd`).  Only tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg may import it.
+
+Every function cites the reference file:line it follows.  Pinning status:
+
+* basis()                pinned by tests/golden/e8p_basis.npy (written from the
+                         reference's own basis()), plus closed-form invariants
+* e8p_decode()           pinned by the scalar formula, the palette decoders and
+                         the XOR/nibble identities of the reference's test_vq.py
+* q4_integers()          pinned by the exhaustive 65 536-code fixture
+* a8()                   pinned by closed-form edge cases (ties, clamp, floor)
+* project()/rescale()    pinned by brute-force int64 dots and power-of-two KATs
+* router_topk()/metadata pinned by stable argsort / enumeration
+* swiglu(), combine()    pinned by direct formula on tiny inputs
+"""
+
+import itertools
+
+import numpy as np
+
+# Coordinate j of a codeword takes its sign from bit SIGN_BITS[j] of the
+# parity-adjusted low byte (python/orinfer_build/quantization/vq.py:17).
+SIGN_BITS = (0, 4, 1, 5, 2, 6, 3, 7)
+SEED = 20261002  # python/orinfer_build/compiler/cuda/common.py:18
+
+
+# --------------------------------------------------------------------------
+# Codebook
+# --------------------------------------------------------------------------
+def basis():
+    """256x8 int8 E8P basis (python/orinfer_build/quantization/e8p.py:15-25).
+
+    Inner rows: magnitudes in {2,6,10}, lexicographic product order, squared
+    norm <= 160 (227 rows).  Outer rows: 29 patterns of five 6s and three 2s,
+    taken at positions i*56//29 of the 56 five-subsets of range(8).  The last
+    coordinate is negated when sum(row)//4 is odd.
+    """
+    inner = [r for r in itertools.product((2, 6, 10), repeat=8) if sum(v * v for v in r) <= 160]
+    subsets = list(itertools.combinations(range(8), 5))
+    outer = []
+    for i in range(29):
+        chosen = subsets[i * len(subsets) // 29]
+        outer.append(tuple(6 if j in chosen else 2 for j in range(8)))
+    rows = np.array(inner + outer, dtype=np.int16)
+    flip = (rows.sum(axis=1) // 4) % 2 == 1
+    rows[flip, 7] = -rows[flip, 7]
+    assert rows.shape == (256, 8)
+    return rows.astype(np.int8)
+
+
+def e8p_decode(codes, table):
+    """u16 code -> 8 int8 lattice coordinates (vq.py:34-43, docs/quantization.md:66-72).
+
+    b = code>>8, u = code&255, p = popcount(u)&1, m = u^p,
+    q[j] = table[b,j] * (1 - 2*bit(m, SIGN_BITS[j])) + (1 - 2p).
+    """
+    c = np.asarray(codes).astype(np.uint16).astype(np.int32)
+    u = c & 255
+    p = np.zeros_like(u)
+    for bit in range(8):
+        p ^= (u >> bit) & 1
+    m = u ^ p
+    sign = np.stack([1 - 2 * ((m >> s) & 1) for s in SIGN_BITS], axis=-1)
+    t = np.asarray(table).astype(np.int32)[c >> 8]
+    return (t * sign + (1 - 2 * p)[..., None]).astype(np.int8)
+
+
+def e8p_decode_scalar(code, table):
+    """Pure-Python scalar decode of one code (test_vq.py:132-147); small cases only."""
+    code = int(code)
+    u = code & 255
+    p = bin(u).count("1") & 1
+    m = u ^ p
+    return [
+        int(table[code >> 8][j]) * (-1 if (m >> SIGN_BITS[j]) & 1 else 1) + (1 - 2 * p)
+        for j in range(8)
+    ]
+
+
+def selector_table(table):
+    """(256,1) u32 selector LUT the engine binds as `Book` (vq.py:74-93).
+
+    Nibble j = magnitude id ((|t|-2)/4, or 3 for zero) | 4 if t<0.
+    """
+    t = np.asarray(table)
+    if t.dtype != np.int8 or t.shape != (256, 8) or not np.isin(t, (-10, -6, -2, 0, 2, 6, 10)).all():
+        raise ValueError("selector table needs values in {0,+-2,+-6,+-10}")
+    v = t.astype(np.int64)
+    ident = np.where(v == 0, 3, (np.abs(v) - 2) // 4) + 4 * (v < 0)
+    word = np.zeros(256, np.uint64)
+    for j in range(8):
+        word |= ident[:, j].astype(np.uint64) << np.uint64(4 * j)
+    return word.astype(np.uint32).reshape(256, 1)
+
+
+def basis_words(table):
+    """(256,2) u32 raw int8 basis view used by the single-token Q2 kernel (vq.py:203)."""
+    return np.ascontiguousarray(np.asarray(table, np.int8)).view("<u4").reshape(256, 2)
+
+
+# --------------------------------------------------------------------------
+# Weights
+# --------------------------------------------------------------------------
+def q4_integers(packed, table, coefficients=(4, 1)):
+    """Two-stage Q4 int8 weights (quantization/e8p_q4.py:61-67).
+
+    packed u32 [N, K/8]: low half = coarse code, high half = residual code.
+    w = a*decode(lo) + b*decode(hi); (a,b)=(4,1) gives |w| <= 55.
+    """
+    packed = np.asarray(packed)
+    if packed.dtype != np.uint32 or packed.ndim != 2:
+        raise ValueError("expected u32 [N, K/8]")
+    a, b = coefficients
+    lo = e8p_decode((packed & 0xFFFF).astype(np.uint16), table).astype(np.int16)
+    hi = e8p_decode((packed >> 16).astype(np.uint16), table).astype(np.int16)
+    w = a * lo + b * hi
+    assert np.abs(w).max() <= 127
+    return w.reshape(packed.shape[0], packed.shape[1] * 8).astype(np.int8)
+
+
+def q2_integers(indices, table):
+    """Single-stage int8 weights from u16 [N, K/8] (vq.py:185-195, without patches)."""
+    indices = np.asarray(indices)
+    if indices.dtype != np.uint16 or indices.ndim != 2:
+        raise ValueError("expected u16 [N, K/8]")
+    return e8p_decode(indices, table).reshape(indices.shape[0], indices.shape[1] * 8)
+
+
+def q4_pack_k(packed, packed_k):
+    """Row-major (N,K/8) u32 -> K-major (K/pk, N, pk/8) (models/qwen35/storage.py:69-76)."""
+    n, vectors = packed.shape
+    per = packed_k // 8
+    return np.ascontiguousarray(packed.reshape(n, vectors // per, per).transpose(1, 0, 2))
+
+
+def q2_pack_k128(indices):
+    """(N,K/8) u16 -> (K/128, N, 16) (vq.py:199-202)."""
+    n, vectors = indices.shape
+    return np.ascontiguousarray(indices.reshape(n, vectors // 16, 16).transpose(1, 0, 2))
+
+
+def q2_repack_k64(packed):
+    """(E,K/128,N,16) u16 -> (E,K/64,N,8), codes unchanged (vq.py:121-128)."""
+    e, g, n, _ = packed.shape
+    return np.ascontiguousarray(packed.reshape(e, g, n, 2, 8).transpose(0, 1, 3, 2, 4)).reshape(
+        e, g * 2, n, 8
+    )
+
+
+# --------------------------------------------------------------------------
+# Activations
+# --------------------------------------------------------------------------
+def a8(x, group=None):
+    """fp16 -> int8 codes + fp16 scale per (row, group).
+
+    quantization/reference_math.py:6-20 and
+    kernels/cuda/operators/op30_activation_quantization.py:14-18,49-65:
+    scale = fp16(max(amax/127, 2^-24)) or 1 when amax == 0;
+    code = clamp(rint(x / fp32(scale)), -127, 127), ties to even.
+    Returns (codes int8 [M,K], scale fp16 [M, groups]).
+    """
+    x = np.asarray(x).astype(np.float16).astype(np.float32)
+    if x.ndim != 2 or not np.isfinite(x).all():
+        raise ValueError("a8 wants a finite 2-D fp16 matrix")
+    width = x.shape[1] if group is None else group
+    if x.shape[1] % width:
+        raise ValueError("group must divide K")
+    g = x.reshape(x.shape[0], -1, width)
+    amax = np.abs(g).max(axis=-1)
+    floor = np.float32(2.0**-24)
+    raw = np.maximum(amax / np.float32(127.0), floor).astype(np.float32)
+    scale = np.where(amax > 0, raw, np.float32(1.0)).astype(np.float16)
+    ratio = g / scale.astype(np.float32)[..., None]
+    codes = np.clip(np.rint(ratio), -127, 127).astype(np.int8)
+    return codes.reshape(x.shape), scale
+
+
+def swiglu_fp16(gu):
+    """fp16 [M,2I] -> fp16 [M,I]: silu(gate)*up in fp32 with a stable sigmoid, one fp16 cast.
+
+    kernels/cuda/operators/op04_swiglu.py:6-17, reference_math.py:31-35.
+    """
+    gu = np.asarray(gu).astype(np.float16).astype(np.float32)
+    g, u = np.split(gu, 2, axis=-1)
+    e = np.exp(-np.abs(g)).astype(np.float32)
+    one = np.float32(1.0)
+    sig = np.where(g >= 0, one / (one + e), e / (one + e)).astype(np.float32)
+    return ((g * sig) * u).astype(np.float16)
+
+
+# --------------------------------------------------------------------------
+# Contraction + epilogue
+# --------------------------------------------------------------------------
+def int_dot(a_q, w_q):
+    """Exact int32 accumulators [M,N] via fp64 BLAS (tests/cuda/operators/quantized_reference.py:12-15).
+
+    Exact because |sum| <= 128*128*K < 2^53 for every K on this path.
+    """
+    a = np.asarray(a_q)
+    w = np.asarray(w_q)
+    assert a.dtype == np.int8 and w.dtype == np.int8 and a.shape[1] == w.shape[1]
+    dot = a.astype(np.float64) @ w.astype(np.float64).T
+    return dot.astype(np.int64).astype(np.int32)
+
+
+def int_dot_bruteforce(a_q, w_q):
+    """Pure integer dot, no floating point anywhere; for pinning int_dot on small shapes."""
+    a = np.asarray(a_q).astype(np.int64)
+    w = np.asarray(w_q).astype(np.int64)
+    return np.einsum("mk,nk->mn", a, w).astype(np.int32)
+
+
+def rescale(acc, weight_scale, token_scale, out_dtype=np.float16):
+    """(fp32(acc) * fp32(ws)) * fp32(as), one cast (kernels/cuda/model/integer_core.py:19-22)."""
+    value = np.asarray(acc).astype(np.float32) * np.asarray(weight_scale).astype(np.float32)[None, :]
+    value = value * np.asarray(token_scale).astype(np.float32).reshape(-1)[:, None]
+    return value.astype(out_dtype)
+
+
+def project(a_q, a_scale, w_q, w_scale, out_dtype=np.float16):
+    """int8 x int8 -> int32 -> rescale (tests/cuda/operators/flash_next_quantized.py:30-37)."""
+    return rescale(int_dot(a_q, w_q), w_scale, a_scale, out_dtype)
+
+
+# --------------------------------------------------------------------------
+# MoE routing (kernels/cuda/model/moe.py)
+# --------------------------------------------------------------------------
+def router_topk(logits, top_k, renormalize=True):
+    """fp32 logits [M,E] -> ids int32 [M,k], prob fp32 [M,k] (moe.py:413-494).
+
+    Descending logit, exact ties -> lower id, -0 == +0 (stable descending
+    argsort, tests/cuda/operators/moe.py:51-57).  prob = exp(l-max)/den with
+    den over the selected experts (renormalize) or over all E.
+    """
+    logits = np.asarray(logits, np.float32)
+    m, e = logits.shape
+    key = np.where(logits == 0, np.float32(0.0), logits)  # fold signed zero
+    ids = np.argsort(-key.astype(np.float64), axis=1, kind="stable")[:, :top_k].astype(np.int32)
+    top = logits.max(axis=1, keepdims=True)
+    picked = np.take_along_axis(logits, ids.astype(np.int64), axis=1)
+    num = np.exp((picked - top).astype(np.float32)).astype(np.float32)
+    if renormalize:
+        den = num.sum(axis=1, keepdims=True, dtype=np.float32)
+    else:
+        den = np.exp((logits - top).astype(np.float32)).sum(axis=1, keepdims=True, dtype=np.float32)
+    return ids, (num / den).astype(np.float32)
+
+
+def expert_histogram(ids, experts):
+    """Counts[E], RelativeSlot[M,k]; assignment order token-major, rank-minor (moe.py:177-210)."""
+    ids = np.asarray(ids, np.int32)
+    counts = np.zeros(experts, np.int32)
+    relative = np.zeros_like(ids)
+    for row in range(ids.shape[0]):
+        for rank in range(ids.shape[1]):
+            e = int(ids[row, rank])
+            relative[row, rank] = counts[e]
+            counts[e] += 1
+    return counts, relative
+
+
+def expert_offsets(counts, block_m):
+    """RowOffsets, TileOffsets (exclusive prefixes) and TileCount (moe.py:214-244)."""
+    counts = np.asarray(counts, np.int64)
+    tiles = (counts + block_m - 1) // block_m
+    rows = np.cumsum(counts) - counts
+    tile_offsets = np.cumsum(tiles) - tiles
+    return rows.astype(np.int32), tile_offsets.astype(np.int32), np.array([tiles.sum()], np.int32)
+
+
+def expert_tiles(counts, tile_offsets, block_m, capacity):
+    """(TileExpert, TileRow) lists; entries beyond TileCount stay -1 here (moe.py:248-282)."""
+    tile_expert = np.full(capacity, -1, np.int32)
+    tile_row = np.full(capacity, -1, np.int32)
+    for e, c in enumerate(np.asarray(counts)):
+        for t in range((int(c) + block_m - 1) // block_m):
+            tile_expert[tile_offsets[e] + t] = e
+            tile_row[tile_offsets[e] + t] = t * block_m
+    return tile_expert, tile_row
+
+
+def tile_capacity(assignments, experts, block_m):
+    """ceil(M*k/bm) + min(E, M*k) (moe.py:263-264)."""
+    return (assignments + block_m - 1) // block_m + min(experts, assignments)
+
+
+def expert_dispatch(a_q, a_scale, ids, relative, row_offsets):
+    """Copy int8 rows + scales to expert-sorted slots; returns (D, DS, SlotMap) (moe.py:286-329)."""
+    m, k = ids.shape
+    slot_map = (np.asarray(row_offsets)[ids] + relative).astype(np.int32)
+    d = np.zeros((m * k, a_q.shape[1]), np.int8)
+    scale = np.asarray(a_scale).reshape(m, -1)
+    ds = np.zeros((m * k, scale.shape[1]), np.float16)
+    for row in range(m):
+        for rank in range(k):
+            d[slot_map[row, rank]] = a_q[row]
+            ds[slot_map[row, rank]] = scale[row]
+    return d, ds, slot_map
+
+
+def moe_combine(expert_out, slot_map, prob, shared=None, shared_gate=None):
+    """out = sum_rank fp32(Expert[slot])*prob (+ sigmoid(gate)*shared), one fp16 cast (moe.py:498-554).
+
+    fp32 accumulation in rank order; slots < 0 or >= slots are skipped.
+    """
+    expert_out = np.asarray(expert_out)
+    slots = expert_out.shape[0]
+    m, k = slot_map.shape
+    acc = np.zeros((m, expert_out.shape[1]), np.float32)
+    for rank in range(k):
+        s = slot_map[:, rank]
+        ok = (s >= 0) & (s < slots)
+        rows = expert_out[np.clip(s, 0, slots - 1)].astype(np.float32)
+        term = (rows * np.asarray(prob, np.float32)[:, rank : rank + 1]).astype(np.float32)
+        acc = np.where(ok[:, None], (acc + term).astype(np.float32), acc)
+    if shared is not None:
+        gate = np.asarray(shared_gate).astype(np.float32)
+        sig = (np.float32(1.0) / (np.float32(1.0) + np.exp(-gate).astype(np.float32))).astype(np.float32)
+        acc = (acc + sig[:, None] * np.asarray(shared).astype(np.float32)).astype(np.float32)
+    return acc.astype(np.float16)
+
+
+def grouped_project(d, ds, weights_int8, weight_scales, counts, row_offsets):
+    """Per-expert project over the sorted rows (integer_vq.py:205-214 epilogue)."""
+    out = np.zeros((d.shape[0], weights_int8.shape[1]), np.float16)
+    for e, c in enumerate(np.asarray(counts)):
+        if c:
+            lo = int(row_offsets[e])
+            out[lo : lo + c] = project(d[lo : lo + c], ds[lo : lo + c, 0], weights_int8[e], weight_scales[e])
+    return out
+
+
+def moe_layer(x, logits, gate_up_codes, gate_up_scales, down_codes, down_scales, table, top_k, block_m=16):
+    """Whole Q2A8 expert layer in the reference's program order
+    (tests/cuda/operators/flash_next_quantized.py:117-135; kernels/cuda/model/moe.py):
+    top-k -> histogram/offsets -> A8 -> dispatch -> grouped gate_up -> SwiGLU fp16 -> A8 ->
+    grouped down -> weighted combine.
+
+    gate_up_codes u16 [E, 2I, H/8], down_codes u16 [E, H, I/8] (row-major per expert).
+    Returns a dict of every intermediate so kernels can be checked stage by stage.
+    """
+    e = gate_up_codes.shape[0]
+    ids, prob = router_topk(logits, top_k, True)
+    counts, relative = expert_histogram(ids, e)
+    row_offsets, tile_offsets, tile_count = expert_offsets(counts, block_m)
+    a_q, a_s = a8(x)
+    d, ds, slot_map = expert_dispatch(a_q, a_s, ids, relative, row_offsets)
+    w1 = np.stack([q2_integers(gate_up_codes[i], table) for i in range(e)])
+    w2 = np.stack([q2_integers(down_codes[i], table) for i in range(e)])
+    gu = grouped_project(d, ds, w1, gate_up_scales, counts, row_offsets)
+    act = swiglu_fp16(gu)
+    h_q, h_s = a8(act)
+    dn = grouped_project(h_q, h_s, w2, down_scales, counts, row_offsets)
+    out = moe_combine(dn, slot_map, prob)
+    return dict(ids=ids, prob=prob, counts=counts, relative=relative, row_offsets=row_offsets,
+                tile_offsets=tile_offsets, tile_count=tile_count, a_q=a_q, a_s=a_s, d=d, ds=ds,
+                slot_map=slot_map, gate_up=gu, act=act, h_q=h_q, h_s=h_s, down=dn, out=out)

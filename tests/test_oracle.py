@@ -1,0 +1,398 @@
+"""Pins the CPU oracle (oracle/reference.py, oracle/e8p_oracle.c) before anything trusts it.
+
+Each check is chosen so that a plausible mistake fails: a wrong SIGN_BITS entry, a
+dropped parity shift, a transposed table, a wrong outer-row spread, reciprocal
+instead of divide in A8, swapped scale order in the epilogue.
+"""
+import ctypes
+import itertools
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from oracle import reference as orc
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+@pytest.fixture(scope="module")
+def table():
+    return orc.basis()
+
+
+@pytest.fixture(scope="module")
+def clib():
+    so = ROOT / "oracle" / "libe8p_oracle.so"
+    if not so.exists():
+        subprocess.check_call(["make", "-C", str(ROOT / "oracle")])
+    return ctypes.CDLL(str(so))
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+# ---- codebook ------------------------------------------------------------
+def test_basis_matches_reference_golden(table, golden_basis):
+    # Row ORDER is fixed only by the reference's source; the golden holds its output.
+    np.testing.assert_array_equal(table, golden_basis)
+
+
+def test_basis_closed_form_invariants(table):
+    t = table.astype(np.int32)
+    assert table.shape == (256, 8) and table.dtype == np.int8
+    assert set(np.unique(np.abs(t))) == {2, 6, 10}
+    norms = (t * t).sum(1)
+    inner, outer = t[:227], t[227:]
+    assert (norms[:227] <= 160).all() and (norms[227:] == 192).all()
+    n6 = (np.abs(inner) == 6).sum(1)
+    n10 = (np.abs(inner) == 10).sum(1)
+    # docs/quantization.md:44-50: 163 rows without a 10, 64 with exactly one 10
+    assert ((n10 == 0) & (n6 <= 4)).sum() == 163
+    assert ((n10 == 1) & (n6 <= 1)).sum() == 64
+    assert ((np.abs(outer) == 6).sum(1) == 5).all() and len(outer) == 29
+    # only the last coordinate is ever negative, and sum(B/4 ... ) parity rule holds
+    assert (t[:, :7] > 0).all()
+    assert ((np.abs(t).sum(1) // 4) % 2 == (t[:, 7] < 0)).all()
+    assert (((t.sum(1)) // 4) % 2 == 0).all()  # canonical representative: even sum(B)/4
+    assert len({tuple(r) for r in np.abs(t)}) == 256
+
+
+def test_c_basis_agrees(table, clib):
+    out = np.zeros((256, 8), np.int8)
+    clib.orc_basis(_ptr(out))
+    np.testing.assert_array_equal(out, table)
+
+
+# ---- decoder ------------------------------------------------------------
+ALL = np.arange(65536, dtype=np.uint16)
+
+
+def test_decode_all_codes_unique_and_odd(table):
+    grid = orc.e8p_decode(ALL, table)
+    assert grid.shape == (65536, 8)
+    assert (grid.astype(np.int32) % 2 != 0).all() and np.abs(grid.astype(np.int32)).max() == 11
+    assert len(np.unique(grid, axis=0)) == 65536  # test_e8p.py:12-13
+
+
+def test_decode_known_answers_by_hand(table):
+    # code 0: basis row 0 = all 2, no flips, parity 0 -> all 3
+    assert orc.e8p_decode(np.array([0], np.uint16), table)[0].tolist() == [3] * 8
+    # code 1: u=1, p=1, m=0 -> no flips, shift -1 -> all 1
+    assert orc.e8p_decode(np.array([1], np.uint16), table)[0].tolist() == [1] * 8
+    # code 3: u=3, p=0, m=3 -> bits 0,1 flip coords 0 and 2 -> [-1,3,-1,3,3,3,3,3]
+    assert orc.e8p_decode(np.array([3], np.uint16), table)[0].tolist() == [-1, 3, -1, 3, 3, 3, 3, 3]
+    # code 0x10: u=16, p=1, m=17 -> bits 0,4 flip coords 0 and 1, shift -1
+    assert orc.e8p_decode(np.array([0x10], np.uint16), table)[0].tolist() == [-3, -3, 1, 1, 1, 1, 1, 1]
+
+
+def test_decode_against_scalar_formula_random_table():
+    # same construction as test_vq.py:132-147 (random even table incl. zeros and negatives)
+    rng = np.random.default_rng(orc.SEED)
+    t = (rng.integers(-5, 6, (256, 8)) * 2).astype(np.int8)
+    codes = np.array([0, 1, 127, 128, 255, 256, 32768, 65535], np.uint16)
+    want = [orc.e8p_decode_scalar(c, t) for c in codes]
+    np.testing.assert_array_equal(orc.e8p_decode(codes, t), want)
+    some = rng.integers(0, 65536, 512).astype(np.uint16)
+    np.testing.assert_array_equal(orc.e8p_decode(some, t), [orc.e8p_decode_scalar(c, t) for c in some])
+
+
+def test_decode_against_palette_decoder():
+    # literal palettes from test_vq.py:32-36: an independent statement of the decoder
+    rng = np.random.default_rng(orc.SEED)
+    t = rng.choice(np.array([-10, -6, -2, 0, 2, 6, 10], np.int8), (256, 8))
+    book = orc.selector_table(t)
+    parity = np.array([bin(int(c) & 255).count("1") & 1 for c in ALL], np.uint32)
+    even = np.array([3, 7, 11, 1, -1, -5, -9, 1], np.int8)
+    odd = np.array([1, 5, 9, -1, -3, -7, -11, -1], np.int8)
+    got = np.empty((65536, 8), np.int8)
+    base = book[ALL >> 8, 0]
+    for lane, bit in enumerate(orc.SIGN_BITS):
+        sel = ((base >> np.uint32(4 * lane)) & 7) ^ ((((ALL ^ parity) >> bit) & 1) * 4)
+        got[:, lane] = np.where(parity == 1, odd[sel], even[sel])
+    np.testing.assert_array_equal(got, orc.e8p_decode(ALL, t))
+
+
+def test_decode_against_xor_nibble_identity(table):
+    # v=(q-1)/2 equals h ^ mask with h=t/2, mask = (flip?0xE:0)^(parity?1:0): the identity behind
+    # the reference's nibble decoder (test_vq.py:70-95, magic 0xEEE00E00) on the real basis.
+    q = orc.e8p_decode(ALL, table).astype(np.int32)
+    u = ALL.astype(np.int32) & 255
+    p = np.array([bin(int(x)).count("1") & 1 for x in u])
+    m = u ^ p
+    h = table.astype(np.int32)[ALL >> 8] // 2
+    for j, bit in enumerate(orc.SIGN_BITS):
+        mask = np.where((m >> bit) & 1, 0xE, 0) ^ p
+        v = ((h[:, j] & 15) ^ mask)
+        v = np.where(v >= 8, v - 16, v)
+        np.testing.assert_array_equal(2 * v + 1, q[:, j])
+
+
+def test_decode_negation_symmetry(table):
+    # lattice fact: flipping all 8 sign bits and the parity bit negates the vector
+    q = orc.e8p_decode(ALL, table).astype(np.int32)
+    neg = orc.e8p_decode((ALL ^ np.uint16(0xFE)).astype(np.uint16), table).astype(np.int32)
+    np.testing.assert_array_equal(neg, -q)
+
+
+def test_c_decode_agrees(table, clib):
+    out = np.zeros((65536, 8), np.int8)
+    clib.orc_decode_all(_ptr(table), _ptr(ALL), ctypes.c_int64(65536), _ptr(out))
+    np.testing.assert_array_equal(out, orc.e8p_decode(ALL, table))
+
+
+def test_selector_table_roundtrip_and_rejects(table):
+    book = orc.selector_table(table)
+    assert book.shape == (256, 1) and book.dtype == np.uint32 and book.nbytes == 1024
+    mags = np.array([2, 6, 10, 0, -2, -6, -10, 0])
+    back = np.stack([mags[(book[:, 0] >> np.uint32(4 * j)) & 7] for j in range(8)], 1)
+    np.testing.assert_array_equal(back, table)
+    assert not (book & np.uint32(0x88888888)).any()
+    bad = table.copy()
+    bad[0, 0] = 4
+    with pytest.raises(ValueError):
+        orc.selector_table(bad)
+
+
+# ---- Q4 two-stage -------------------------------------------------------
+def test_q4_exhaustive_fixture(table, clib):
+    # quantization/test_e8p_q4.py:13-30: every coarse code once, residual by an LCG
+    first = np.arange(65536, dtype=np.uint32).reshape(4096, 16)
+    second = (first * np.uint32(32771) + np.uint32(97)) & np.uint32(65535)
+    packed = first | (second << np.uint32(16))
+    for a, b in ((3, 1), (4, 1), (7, 2)):
+        w = orc.q4_integers(packed, table, (a, b))
+        want = (a * orc.e8p_decode(first.astype(np.uint16), table).astype(np.int16)
+                + b * orc.e8p_decode(second.astype(np.uint16), table).astype(np.int16)).reshape(4096, 128)
+        np.testing.assert_array_equal(w, want)
+        assert np.abs(want).max() <= 127
+        cw = np.zeros((4096, 128), np.int8)
+        clib.orc_q4_integers(_ptr(table), _ptr(packed), ctypes.c_int64(4096), ctypes.c_int64(128),
+                             ctypes.c_int(a), ctypes.c_int(b), _ptr(cw))
+        np.testing.assert_array_equal(cw, w)
+    w41 = orc.q4_integers(packed, table, (4, 1)).astype(np.int32)
+    assert np.abs(w41).max() == 55 and (w41 % 2 != 0).all()  # 4*odd + odd is odd, |.| <= 44+11
+
+
+def test_k_major_layouts_are_lossless():
+    rng = np.random.default_rng(orc.SEED)
+    packed = rng.integers(0, 2**32, (17, 48), dtype=np.uint64).astype(np.uint32)
+    for pk in (64, 128):
+        km = orc.q4_pack_k(packed, pk)
+        assert km.shape == (48 * 8 // pk, 17, pk // 8)
+        np.testing.assert_array_equal(km.transpose(1, 0, 2).reshape(17, 48), packed)
+    idx = rng.integers(0, 65536, (5, 32), dtype=np.uint16)
+    k128 = orc.q2_pack_k128(idx)
+    assert k128.shape == (2, 5, 16)
+    np.testing.assert_array_equal(k128.transpose(1, 0, 2).reshape(5, 32), idx)
+    src = rng.integers(0, 65536, (2, 3, 17, 16), dtype=np.uint16)
+    k64 = orc.q2_repack_k64(src)
+    np.testing.assert_array_equal(k64.reshape(2, 3, 2, 17, 8).transpose(0, 1, 3, 2, 4).reshape(src.shape), src)
+
+
+# ---- A8 ------------------------------------------------------------------
+def test_a8_edge_cases():
+    x = np.zeros((4, 8), np.float16)
+    x[1] = [127, -127, 63.5, 0.5, 1.5, 2.5, -0.5, -2.5]     # scale exactly 1: ties go to even
+    x[2] = [1e-7, 0, 0, 0, 0, 0, 0, 0]                       # amax/127 under the 2^-24 floor
+    x[3] = [254, 1, -1, 3, -3, 5, 127, -254]                 # scale exactly 2: halves tie
+    q, s = orc.a8(x)
+    assert s.dtype == np.float16 and s.shape == (4, 1) and q.dtype == np.int8
+    assert s[0, 0] == 1 and (q[0] == 0).all()
+    assert s[1, 0] == 1 and q[1].tolist() == [127, -127, 64, 0, 2, 2, 0, -2]
+    assert s[2, 0] == np.float16(2.0**-24)
+    assert q[2, 0] == int(np.rint(np.float32(np.float16(1e-7)) / np.float32(2.0**-24)))
+    assert s[3, 0] == 2 and q[3].tolist() == [127, 0, 0, 2, -2, 2, 64, -127]
+
+
+def test_a8_scale_is_divide_then_fp16_and_codes_clamp():
+    rng = np.random.default_rng(orc.SEED)
+    x = rng.normal(size=(64, 256)).astype(np.float16)
+    x[0, 0] = 65504  # fp16 max
+    q, s = orc.a8(x)
+    amax = np.abs(x.astype(np.float32)).max(1)
+    np.testing.assert_array_equal(s[:, 0], (amax / np.float32(127)).astype(np.float16))
+    assert np.abs(q.astype(np.int32)).max() <= 127
+    # fp16 rounding of the scale can push |x|/scale above 127.5: the clamp must catch it
+    ratio = np.abs(x.astype(np.float32)) / s.astype(np.float32)
+    assert (np.abs(q.astype(np.int32)) == np.minimum(np.rint(ratio), 127)).all()
+    # grouped form
+    qg, sg = orc.a8(x, 64)
+    assert sg.shape == (64, 4)
+    q0, s0 = orc.a8(x[:, :64])
+    np.testing.assert_array_equal(qg[:, :64], q0)
+    np.testing.assert_array_equal(sg[:, :1], s0)
+
+
+def test_c_a8_agrees(clib):
+    rng = np.random.default_rng(orc.SEED + 1)
+    x = rng.normal(size=(9, 384)).astype(np.float16)
+    x[3] = 0
+    xf = np.ascontiguousarray(x.astype(np.float32))
+    raw = np.zeros(9, np.float32)
+    clib.orc_a8_scale(_ptr(xf), ctypes.c_int64(9), ctypes.c_int64(384), _ptr(raw))
+    s16 = raw.astype(np.float16)
+    sf = np.ascontiguousarray(s16.astype(np.float32))
+    q = np.zeros((9, 384), np.int8)
+    clib.orc_a8_codes(_ptr(xf), _ptr(sf), ctypes.c_int64(9), ctypes.c_int64(384), _ptr(q))
+    wq, ws = orc.a8(x)
+    np.testing.assert_array_equal(s16, ws[:, 0])
+    np.testing.assert_array_equal(q, wq)
+
+
+# ---- contraction + epilogue ---------------------------------------------
+def test_int_dot_matches_bruteforce_at_extremes(clib):
+    rng = np.random.default_rng(orc.SEED)
+    a = rng.integers(-128, 128, (5, 640), dtype=np.int64).astype(np.int8)
+    w = rng.integers(-128, 128, (7, 640), dtype=np.int64).astype(np.int8)
+    a[0] = -128
+    w[0] = -128
+    a[1] = 127
+    w[1] = -128
+    np.testing.assert_array_equal(orc.int_dot(a, w), orc.int_dot_bruteforce(a, w))
+    assert orc.int_dot(a, w)[0, 0] == 128 * 128 * 640
+    c = np.zeros((5, 7), np.int32)
+    clib.orc_int_dot(_ptr(a), _ptr(w), ctypes.c_int64(5), ctypes.c_int64(7), ctypes.c_int64(640), _ptr(c))
+    np.testing.assert_array_equal(c, orc.int_dot(a, w))
+
+
+def test_project_power_of_two_scales_are_exact():
+    # tests/cuda/operators/int8_projection.py:25-41: with 2^-6 and 2^-7 every product is exact
+    rng = np.random.default_rng(orc.SEED)
+    for m, n, k in ((1, 48, 2560), (3, 65, 128), (17, 129, 640)):
+        a = rng.integers(-128, 128, (m, k), dtype=np.int64).astype(np.int8)
+        w = rng.integers(-128, 128, (n, k), dtype=np.int64).astype(np.int8)
+        ws = np.full(n, 0.015625, np.float16)
+        ts = np.full(m, 0.0078125, np.float16)
+        out32 = orc.project(a, ts, w, ws, np.float32)
+        exact = orc.int_dot_bruteforce(a, w).astype(np.float64) * 2.0**-13
+        np.testing.assert_array_equal(out32.astype(np.float64), exact)
+        np.testing.assert_array_equal(orc.project(a, ts, w, ws), exact.astype(np.float16))
+
+
+def test_rescale_order_is_weight_scale_first(clib):
+    # (acc*ws)*as and acc*(ws*as) differ in fp32 for suitable values: pin the order
+    acc = np.array([[16777217 // 3]], np.int32)
+    ws = np.array([0.0123], np.float16)
+    ts = np.array([0.0071], np.float16)
+    got = orc.rescale(acc, ws, ts, np.float32)[0, 0]
+    want = np.float32(np.float32(np.float32(acc[0, 0]) * np.float32(ws[0])) * np.float32(ts[0]))
+    assert got == want
+    found = False
+    rng = np.random.default_rng(1)
+    for _ in range(2000):
+        a = np.int32(rng.integers(1, 2**24))
+        s1, s2 = np.float16(rng.uniform(0.005, 0.02)), np.float16(rng.uniform(0.001, 0.01))
+        x = np.float32(np.float32(a) * np.float32(s1)) * np.float32(s2)
+        y = np.float32(a) * np.float32(np.float32(s1) * np.float32(s2))
+        if x != y:
+            assert orc.rescale(np.array([[a]], np.int32), np.array([s1]), np.array([s2]), np.float32)[0, 0] == x
+            out = np.zeros(1, np.float32)
+            clib.orc_rescale(_ptr(np.array([a], np.int32)), _ptr(np.array([s1], np.float32)),
+                             _ptr(np.array([s2], np.float32)), ctypes.c_int64(1), ctypes.c_int64(1), _ptr(out))
+            assert out[0] == x
+            found = True
+            break
+    assert found
+
+
+def test_q4_dot_fused_c_path_agrees(table, clib):
+    rng = np.random.default_rng(orc.SEED)
+    packed = rng.integers(0, 2**32, (33, 32), dtype=np.uint64).astype(np.uint32)
+    a = rng.integers(-128, 128, (3, 256), dtype=np.int64).astype(np.int8)
+    acc = np.zeros((3, 33), np.int32)
+    clib.orc_q4_dot(_ptr(table), _ptr(packed), _ptr(a), ctypes.c_int64(3), ctypes.c_int64(33),
+                    ctypes.c_int64(256), _ptr(acc))
+    np.testing.assert_array_equal(acc, orc.int_dot(a, orc.q4_integers(packed, table)))
+
+
+# ---- MoE -----------------------------------------------------------------
+def test_router_topk_ties_signed_zero_and_extremes():
+    # tests/cuda/operators/moe.py:25-57
+    rng = np.random.default_rng(orc.SEED)
+    for m, e, k in ((1, 512, 10), (8, 512, 10), (17, 37, 10), (3, 5, 5), (1, 1, 1)):
+        logits = (rng.normal(size=(m, e)) * 5).astype(np.float32)
+        logits[0] = 0
+        if m > 1:
+            logits[1] = -10000
+            logits[1, -1] = 10000
+        if m > 2:
+            logits[2] = -1
+            logits[2, :k] = 0
+            logits[2, 0] = -0.0
+        for renorm in (False, True):
+            ids, prob = orc.router_topk(logits, k, renorm)
+            assert ids[0].tolist() == list(range(k))
+            if m > 1:
+                assert ids[1, 0] == e - 1 and ids[1, 1:].tolist() == list(range(k - 1))
+            if m > 2:
+                assert ids[2].tolist() == list(range(k))
+            for row in range(m):
+                order = sorted(range(e), key=lambda j: (-float(logits[row, j]) + 0.0, j))[:k]
+                assert ids[row].tolist() == order
+            soft = np.exp(logits.astype(np.float64) - logits.max(1, keepdims=True))
+            soft /= soft.sum(1, keepdims=True)
+            want = np.take_along_axis(soft, ids.astype(np.int64), 1)
+            if renorm:
+                want /= want.sum(1, keepdims=True)
+            np.testing.assert_allclose(prob, want, atol=2e-6)
+
+
+def test_routing_metadata_by_enumeration():
+    rng = np.random.default_rng(orc.SEED)
+    m, e, k, bm = 37, 16, 4, 8
+    ids = np.stack([rng.permutation(e)[:k] for _ in range(m)]).astype(np.int32)
+    counts, rel = orc.expert_histogram(ids, e)
+    np.testing.assert_array_equal(counts, np.bincount(ids.ravel(), minlength=e))
+    flat = ids.ravel()
+    for i, ex in enumerate(flat):
+        assert rel.ravel()[i] == (flat[:i] == ex).sum()
+    rows, tiles, total = orc.expert_offsets(counts, bm)
+    assert rows[0] == 0 and (np.diff(rows) == counts[:-1]).all()
+    assert total[0] == sum(-(-int(c) // bm) for c in counts)
+    cap = orc.tile_capacity(m * k, e, bm)
+    te, tr = orc.expert_tiles(counts, tiles, bm, cap)
+    listed = [(int(a), int(b)) for a, b in zip(te[: total[0]], tr[: total[0]])]
+    assert listed == [(ex, t * bm) for ex in range(e) for t in range(-(-int(counts[ex]) // bm))]
+    assert total[0] <= cap
+    a_q = rng.integers(-127, 128, (m, 64), dtype=np.int64).astype(np.int8)
+    a_s = rng.uniform(0.01, 0.02, (m, 1)).astype(np.float16)
+    d, ds, slot = orc.expert_dispatch(a_q, a_s, ids, rel, rows)
+    assert sorted(slot.ravel().tolist()) == list(range(m * k))  # a permutation of the slots
+    for row, rank in itertools.product(range(m), range(k)):
+        s = slot[row, rank]
+        assert rows[ids[row, rank]] <= s < rows[ids[row, rank]] + counts[ids[row, rank]]
+        np.testing.assert_array_equal(d[s], a_q[row])
+        assert ds[s, 0] == a_s[row, 0]
+
+
+def test_combine_skips_invalid_slots_and_matches_formula():
+    rng = np.random.default_rng(orc.SEED)
+    m, h, slots, k = 5, 33, 12, 3
+    ex = rng.normal(size=(slots, h)).astype(np.float16)
+    sm = rng.integers(0, slots, (m, k)).astype(np.int32)
+    sm[0, :2] = [-1, slots]
+    prob = rng.uniform(0, 1, (m, k)).astype(np.float32)
+    shared = rng.normal(size=(m, h)).astype(np.float16)
+    gate = rng.normal(size=m).astype(np.float16)
+    got = orc.moe_combine(ex, sm, prob, shared, gate)
+    want = np.zeros((m, h), np.float64)
+    for r in range(m):
+        for j in range(k):
+            if 0 <= sm[r, j] < slots:
+                want[r] += ex[sm[r, j]].astype(np.float64) * prob[r, j]
+        want[r] += shared[r].astype(np.float64) / (1 + np.exp(-float(gate[r])))
+    np.testing.assert_allclose(got.astype(np.float64), want, atol=2e-3, rtol=2e-3)
+    nos = orc.moe_combine(ex, sm, prob)
+    assert nos.dtype == np.float16 and nos.shape == (m, h)
+
+
+def test_swiglu_matches_closed_form():
+    g = np.array([[-20, -1, 0, 1, 20, 3.5]], np.float16)
+    u = np.array([[2, 2, 2, 2, 2, -1.25]], np.float16)
+    got = orc.swiglu_fp16(np.concatenate([g, u], 1)).astype(np.float64)
+    gf, uf = g.astype(np.float64), u.astype(np.float64)
+    np.testing.assert_allclose(got, gf / (1 + np.exp(-gf)) * uf, rtol=2e-3, atol=1e-7)
+    assert got[0, 2] == 0 and abs(got[0, 4] - 40) < 0.05
