@@ -1,0 +1,87 @@
+/* orx.h -- C ABI of liborx.so: MI355X (gfx950) kernels for orinfer's quantized linear path.
+ *
+ * The orinfer engine launches every device kernel through one data-driven entry
+ * point: a `Kernel` record (symbol, grid, block, shared bytes, ordered args) is
+ * resolved to a function handle and launched with `cuLaunchKernel(f, grid, block,
+ * shared, stream, void** args, NULL)`.  This header is that entry point for HIP.
+ * Nothing here allocates, synchronises or touches the host after the launch is
+ * enqueued; every kernel reads its tables, scales and routing metadata from device
+ * memory at run time, so a launch can be captured in a hipGraph and replayed after
+ * the caller changed buffer contents.
+ *
+ * Argument convention (crates/orinfer-engine/src/backend/cuda/mod.rs:282-299,319):
+ * args[i] points at an 8-byte device pointer or at a 4-byte scalar.  The ORDER of
+ * arguments per symbol is the generated host ABI of the reference (buffer names in
+ * ASCII order, then scalars; dynamic-row kernels take `int32 m` last) and is
+ * published by orx_arg_name() and orx_catalog().
+ *
+ * Thread model: one thread per device session, one explicit stream
+ * (backend/cuda/mod.rs:1-3).  Calls are re-entrant across distinct streams.
+ */
+#ifndef ORX_H
+#define ORX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Return codes.  0 = success.  Values 1..9999 are hipError_t values passed through
+ * unchanged (the reference returns the driver's numeric code, mod.rs:48-55);
+ * values >= 10000 are raised by the catalog itself before anything is enqueued. */
+#define ORX_OK 0
+#define ORX_ERR_UNKNOWN_SYMBOL 10001   /* no kernel of that name in the catalog            */
+#define ORX_ERR_BAD_VARIANT 10002      /* variant JSON unparsable or geometry not supported */
+#define ORX_ERR_BAD_GEOMETRY 10003     /* grid/block/shared do not fit the resolved kernel   */
+#define ORX_ERR_BAD_ARGUMENT 10004     /* null handle, null args, misaligned pointer         */
+#define ORX_ERR_ROWS 10005             /* dynamic rows outside 1..capacity                   */
+
+typedef struct orx_function* orx_fn;
+
+/* Replaces Catalog::resolve = cuModuleLoadData + cuModuleGetFunction + attribute checks
+ * (crates/orinfer-engine/src/backend/cuda/kernels.rs:114-192).  `symbol` is a kernel
+ * family of the catalog; `variant_json` is a flat JSON object carrying what the
+ * reference bakes into a cubin at compile time (shape, tile, layout, dtype), the way
+ * package `Definition`s do (crates/orinfer-model-sdk/src/catalog.rs:32-50).
+ * Example: orx_resolve("e8p_q4_projection",
+ *                      "{\"M\":1,\"N\":9728,\"K\":2560,\"algorithm\":\"gemv\"}", &f). */
+int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out);
+
+/* Drops a handle (cuModuleUnload in Session::cleanup). */
+int orx_release(orx_fn f);
+
+/* Replaces cuFuncGetAttribute(MAX_THREADS_PER_BLOCK / SHARED_SIZE_BYTES)
+ * (kernels.rs:150-170): limits the caller validates its launch record against. */
+int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes);
+
+/* The launch geometry a package would record for this kernel: the static grid of a
+ * fixed-row kernel, or the RowExpression result of a dynamic one for `rows` live rows
+ * (crates/orinfer-model-sdk/src/operators/dynamic.rs:93-118).  rows <= 0 means the
+ * variant's own M.  Fails with ORX_ERR_ROWS when rows exceeds the capacity. */
+int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes);
+
+/* Argument list of the resolved kernel, in launch order (contracts/abi.py:26-80 parses
+ * the same from the generated host.txt).  kind: 0 = device pointer, 1 = int32 scalar. */
+int orx_arg_count(orx_fn f);
+const char* orx_arg_name(orx_fn f, int index);
+int orx_arg_kind(orx_fn f, int index);
+
+/* Replaces launch_kernel = cuLaunchKernel (backend/cuda/mod.rs:312-341).  Enqueues the
+ * kernel on `hip_stream` (a hipStream_t, may be 0).  grid/block/shared must equal what
+ * orx_geometry() returns for the row count passed in `m` (validated; the reference
+ * validates records in kernels.rs:47-61).  Never blocks, never allocates. */
+int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+               void* hip_stream, void** args);
+
+/* Thread-local text of the last failure on this thread (mod.rs:48-55 formats
+ * "<op>: CUDA error <code>").  Never NULL. */
+const char* orx_last_error(void);
+
+/* JSON text listing every symbol, its variant keys and its argument order. Static storage. */
+const char* orx_catalog(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ORX_H */

@@ -1,0 +1,172 @@
+// Device-side E8P decode helpers shared by every kernel of liborx (gfx950 only).
+//
+// A u16 code is b = code>>8 (basis row), u = code&255 (sign bits + parity).
+// With p = popcount(u)&1 and m = u^p, coordinate j decodes to
+//     q_j = t[b][j] * (1 - 2*bit(m, SIGN_BITS[j])) + (1 - 2p),   SIGN_BITS = {0,4,1,5,2,6,3,7}
+// (python/orinfer_build/quantization/vq.py:17,34-43).  Every basis value t is
+// +-2, +-6 or +-10, i.e. t = 2h with h odd, and q = 2v+1 with
+//     v_j = h_j XOR mask_j,   mask_j = (bit(m,..) ? 0xE : 0) ^ p          (4-bit two's complement)
+// so one code decodes with two table reads and one XOR: a per-basis word and a
+// per-low-byte word.  The same identity on whole bytes gives q_j = t_j ^ mask3_j with
+// mask3 in {0x01, 0xFD, 0x03, 0xFF}.  The reference's nibble decoder rests on the same
+// identity (quantization/vq.py:105-118); it needs a basis without zeros, which the E8P
+// basis is (quantization/e8p.py:15-25).
+//
+// `Book` as bound by the engine is the (256,1) u32 selector table: nibble j =
+// magnitude id {0:2, 1:6, 2:10, 3:0} | 4 when negative (vq.py:74-93).  The tables below
+// are rebuilt from it in LDS by every workgroup, so swapping Book between graph replays
+// is honoured.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace orx {
+
+// Nibble position of coordinate j inside a packed 8-nibble word: coordinates 0..3 sit in
+// the even nibbles (low nibble of bytes 0..3), coordinates 4..7 in the odd nibbles.
+// (word & 0x0F0F0F0F) is then the byte vector of coordinates 0..3 and
+// ((word >> 4) & 0x0F0F0F0F) that of coordinates 4..7.
+__device__ __forceinline__ int nibble_slot(int j) { return j < 4 ? 2 * j : 2 * (j - 4) + 1; }
+
+// h = t/2 of coordinate j from a selector word; 0 for the "zero" id (unsupported basis).
+__device__ __forceinline__ int selector_half(uint32_t selector, int j) {
+    const uint32_t id = (selector >> (4 * j)) & 7u;
+    const int mag = (int)(id & 3u);
+    const int h = mag == 3 ? 0 : 2 * mag + 1;
+    return (id & 4u) ? -h : h;
+}
+
+// Sign bit of coordinate j in the parity-adjusted low byte m.
+__device__ __forceinline__ uint32_t sign_bit(uint32_t m, int j) {
+    const int bit = (j & 1) ? 4 + (j >> 1) : (j >> 1);
+    return (m >> bit) & 1u;
+}
+
+// ---- nibble tables (GEMV path): v word = nib[b] ^ msk[u], signed 4-bit v per coordinate ----
+__device__ __forceinline__ uint32_t nibble_basis_word(uint32_t selector, uint32_t bias) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        word |= (((uint32_t)selector_half(selector, j) ^ bias) & 15u) << (4 * nibble_slot(j));
+    return word;
+}
+
+__device__ __forceinline__ uint32_t nibble_mask_word(uint32_t u) {
+    const uint32_t p = __popc(u) & 1u;
+    const uint32_t m = u ^ p;
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        word |= ((sign_bit(m, j) ? 0xEu : 0u) ^ p) << (4 * nibble_slot(j));
+    return word;
+}
+
+// ---- byte tables: 8 bytes per entry in coordinate order ---------------------------------
+// "biased nibble" form: byte j = ((h_j ^ 8) & 15) << shift and mask_j << shift.  XOR of a basis
+// entry and a mask entry is (v_j + 8) << shift, an unsigned value that never carries out of
+// its byte for shift <= 3.
+__device__ __forceinline__ uint2 byte_basis_biased(uint32_t selector, int shift) {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        lo |= ((((uint32_t)selector_half(selector, j) ^ 8u) & 15u) << shift) << (8 * j);
+        hi |= ((((uint32_t)selector_half(selector, j + 4) ^ 8u) & 15u) << shift) << (8 * j);
+    }
+    return make_uint2(lo, hi);
+}
+
+__device__ __forceinline__ uint2 byte_mask_biased(uint32_t u, int shift) {
+    const uint32_t p = __popc(u) & 1u;
+    const uint32_t m = u ^ p;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        lo |= (((sign_bit(m, j) ? 0xEu : 0u) ^ p) << shift) << (8 * j);
+        hi |= (((sign_bit(m, j + 4) ? 0xEu : 0u) ^ p) << shift) << (8 * j);
+    }
+    return make_uint2(lo, hi);
+}
+
+// "signed byte" form (single-stage Q2): byte j = t_j and mask3_j; XOR is q_j itself.
+__device__ __forceinline__ uint2 byte_basis_signed(uint32_t selector) {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        lo |= ((uint32_t)(2 * selector_half(selector, j)) & 255u) << (8 * j);
+        hi |= ((uint32_t)(2 * selector_half(selector, j + 4)) & 255u) << (8 * j);
+    }
+    return make_uint2(lo, hi);
+}
+
+__device__ __forceinline__ uint2 byte_mask_signed(uint32_t u) {
+    const uint32_t p = __popc(u) & 1u;
+    const uint32_t m = u ^ p;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t a = sign_bit(m, j) ? (p ? 0xFFu : 0xFDu) : (p ? 0x03u : 0x01u);
+        const uint32_t b = sign_bit(m, j + 4) ? (p ? 0xFFu : 0xFDu) : (p ? 0x03u : 0x01u);
+        lo |= a << (8 * j);
+        hi |= b << (8 * j);
+    }
+    return make_uint2(lo, hi);
+}
+
+// LDS tables for the byte decoders.
+struct Q4ByteTables {   // w = 4*q0 + q1 = 8*(v0+8) + 2*(v1+8) - 75
+    uint2 basis0[256];  // (h^8) << 3
+    uint2 mask0[256];   // mask << 3
+    uint2 basis1[256];  // (h^8) << 1
+    uint2 mask1[256];   // mask << 1
+};
+struct Q2ByteTables {
+    uint2 basis[256];   // t
+    uint2 mask[256];    // mask3
+};
+
+__device__ __forceinline__ void build_tables(Q4ByteTables& t, const uint32_t* __restrict__ book, int tid, int threads) {
+    for (int i = tid; i < 256; i += threads) {
+        const uint32_t s = book[i];
+        t.basis0[i] = byte_basis_biased(s, 3);
+        t.basis1[i] = byte_basis_biased(s, 1);
+        t.mask0[i] = byte_mask_biased((uint32_t)i, 3);
+        t.mask1[i] = byte_mask_biased((uint32_t)i, 1);
+    }
+}
+
+__device__ __forceinline__ void build_tables(Q2ByteTables& t, const uint32_t* __restrict__ book, int tid, int threads) {
+    for (int i = tid; i < 256; i += threads) {
+        t.basis[i] = byte_basis_signed(book[i]);
+        t.mask[i] = byte_mask_signed((uint32_t)i);
+    }
+}
+
+// One u32 two-stage code -> 8 int8 weights (two words: coordinates 0..3 and 4..7).
+// (x0 + x1 + 53) is w+128 in every byte, in [73,183]: no carry between bytes; the XOR
+// turns offset binary into two's complement.
+__device__ __forceinline__ uint2 decode_q4(const Q4ByteTables& t, uint32_t code) {
+    const uint2 b0 = t.basis0[(code >> 8) & 255u];
+    const uint2 m0 = t.mask0[code & 255u];
+    const uint2 b1 = t.basis1[code >> 24];
+    const uint2 m1 = t.mask1[(code >> 16) & 255u];
+    uint2 w;
+    w.x = ((b0.x ^ m0.x) + (b1.x ^ m1.x) + 0x35353535u) ^ 0x80808080u;
+    w.y = ((b0.y ^ m0.y) + (b1.y ^ m1.y) + 0x35353535u) ^ 0x80808080u;
+    return w;
+}
+
+// One u16 single-stage code -> 8 int8 weights.
+__device__ __forceinline__ uint2 decode_q2(const Q2ByteTables& t, uint32_t code) {
+    const uint2 b = t.basis[(code >> 8) & 255u];
+    const uint2 m = t.mask[code & 255u];
+    return make_uint2(b.x ^ m.x, b.y ^ m.y);
+}
+
+// fp32 epilogue shared by every projection: (float(acc) * ws) * as, two separate roundings
+// (kernels/cuda/model/integer_core.py:19-22).  The volatile-free form below relies on the
+// build flags forbidding reassociation; there is no add, so contraction cannot apply.
+__device__ __forceinline__ float rescale(int acc, float weight_scale, float token_scale) {
+    return ((float)acc * weight_scale) * token_scale;
+}
+
+}  // namespace orx

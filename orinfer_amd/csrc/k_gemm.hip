@@ -1,0 +1,530 @@
+// int8 MFMA projections: E8P-Q4 (decode fused), single-stage E8P-Q2 experts (grouped) and W8A8.
+//
+// Reference counterparts: kernels/cuda/model/integer_core.py:162-272 (tile loop, weight loader,
+// epilogue), kernels/cuda/model/e8p_q4.py:143-264 (Q4 projection + ABI), int8_projection.py:15-62
+// (W8A8 ABI), integer_vq.py:58-260 / e8p_decode.py:36-245 (routed Q2 ABI), e8p_q4.py:267-302
+// (unpack).  Arithmetic: exact int32 accumulation over full K, then (float(acc)*ws)*as.
+//
+// MI355X design.  A workgroup of four wave64 owns a BM x BN output tile and walks K in steps
+// of 128.  Activations go HBM -> registers -> LDS as int8; weight codes go HBM -> registers,
+// are decoded with two 8-byte LDS table reads and XORs per code (e8p_device.h), and land in
+// LDS as an int8 [BN][128] tile, so v_mfma_i32_32x32x32_i8 reads both operands as 16-byte,
+// K-contiguous lane fragments.  Rows in LDS are padded to 144 bytes so that the sixteen lanes of
+// one ds_read_b128 phase hit distinct banks.  Global loads for tile t+1 are issued before the
+// MFMAs of tile t.  Grouped (expert) tiles take (expert, first row, count) from device lists.
+#include <hip/hip_fp16.h>
+
+#include "e8p_device.h"
+#include "orx_internal.h"
+
+namespace orx {
+
+// from k_gemv.hip
+int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
+                const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out);
+int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
+int gemv_configure(orx_function* f, int codec, int passes_override);
+int gemv_prepare_device();
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
+enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2 };
+
+constexpr int kBK = 128;        // K bytes per tile step
+constexpr int kPitch = kBK + 16;  // LDS row pitch in bytes
+
+struct GemmParams {
+    const int8_t* a;
+    const void* w;
+    const uint32_t* book;
+    const __half* ws;
+    const __half* as;
+    void* out;
+    int n, k, stride, m;
+    int packed_k;  // 0 row-major codes, 128 K-major blocks
+    int out_f32;
+    // grouped only
+    const int* counts;
+    const int* offsets;
+    const int* tile_expert;
+    const int* tile_row;
+    const int* tile_count;
+    int64_t expert_weight_stride;  // bytes between experts in w
+};
+
+template <int CODEC>
+struct Tables {
+    typedef Q4ByteTables type;
+};
+template <>
+struct Tables<kQ2> {
+    typedef Q2ByteTables type;
+};
+template <>
+struct Tables<kW8> {
+    struct type {};
+};
+
+// Number of 16-byte global chunks of weight stream per output row per K step.
+template <int CODEC>
+__host__ __device__ constexpr int weight_chunks() {
+    return CODEC == kQ4 ? 4 : CODEC == kQ2 ? 2 : 8;
+}
+
+template <int CODEC, int BM, int BN, int WAVES_M, bool GROUPED>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
+    constexpr int WAVES_N = 4 / WAVES_M;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
+    constexpr int A_CHUNKS = BM * 8 / 256;                        // uint4 per thread for A
+    constexpr int W_CHUNKS = BN * weight_chunks<CODEC>() / 256;   // uint4 per thread for weights
+    static_assert(A_CHUNKS >= 1 && W_CHUNKS >= 1, "tile too small for 256 threads");
+
+    __shared__ __align__(16) int8_t lds_a[BM * kPitch];
+    __shared__ __align__(16) int8_t lds_w[BN * kPitch];
+    __shared__ typename Tables<CODEC>::type tables;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int n0 = blockIdx.x * BN;
+    int row0, rows_here;
+    const int8_t* w_base = reinterpret_cast<const int8_t*>(p.w);
+    const __half* ws = p.ws;
+    if (GROUPED) {
+        const int tile = blockIdx.y;
+        if (tile >= p.tile_count[0]) return;
+        const int expert = p.tile_expert[tile];
+        const int first = p.tile_row[tile];
+        row0 = p.offsets[expert] + first;
+        rows_here = min(BM, p.counts[expert] - first);
+        if (rows_here <= 0) return;
+        w_base += (int64_t)expert * p.expert_weight_stride;
+        ws += (int64_t)expert * p.n;
+    } else {
+        row0 = blockIdx.y * BM;
+        rows_here = min(BM, p.m - row0);
+    }
+
+    if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, 256);
+
+    const int k_tiles = p.k / kBK;
+    uint4 reg_a[A_CHUNKS], reg_w[W_CHUNKS];
+
+    auto load_tile = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            const int r = min(c >> 3, rows_here - 1), kc = c & 7;
+            reg_a[i] = *reinterpret_cast<const uint4*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            constexpr int PER_ROW = weight_chunks<CODEC>();
+            const int nn = min(n0 + c / PER_ROW, p.n - 1), q = c % PER_ROW;
+            int64_t byte;
+            if (CODEC == kW8)
+                byte = (int64_t)nn * p.k + kt * kBK + q * 16;
+            else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
+                byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
+            else  // (N, K/8 codes)
+                byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
+            reg_w[i] = *reinterpret_cast<const uint4*>(w_base + byte);
+        }
+    };
+
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            *reinterpret_cast<uint4*>(lds_a + (c >> 3) * kPitch + (c & 7) * 16) = reg_a[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            constexpr int PER_ROW = weight_chunks<CODEC>();
+            const int nn = c / PER_ROW, q = c % PER_ROW;
+            if constexpr (CODEC == kW8) {
+                *reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
+            } else if constexpr (CODEC == kQ4) {
+                // 4 u32 codes -> 32 weights at k offset q*32
+                const uint2 d0 = decode_q4(tables, reg_w[i].x), d1 = decode_q4(tables, reg_w[i].y);
+                const uint2 d2 = decode_q4(tables, reg_w[i].z), d3 = decode_q4(tables, reg_w[i].w);
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 32);
+                dst[0] = make_uint4(d0.x, d0.y, d1.x, d1.y);
+                dst[1] = make_uint4(d2.x, d2.y, d3.x, d3.y);
+            } else {
+                // 8 u16 codes -> 64 weights at k offset q*64
+                const uint32_t pair[4] = {reg_w[i].x, reg_w[i].y, reg_w[i].z, reg_w[i].w};
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 64);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint2 lo = decode_q2(tables, pair[j] & 0xFFFFu), hi = decode_q2(tables, pair[j] >> 16);
+                    dst[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                }
+            }
+        }
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    load_tile(0);
+    __syncthreads();  // tables ready
+    for (int kt = 0; kt < k_tiles; ++kt) {
+        store_tile();
+        __syncthreads();
+        if (kt + 1 < k_tiles) load_tile(kt + 1);
+        const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
+#pragma unroll
+        for (int ks = 0; ks < kBK / 32; ++ks) {
+            v4i fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                fa[i] = *reinterpret_cast<const v4i*>(lds_a + ((wave_m * TM + i) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                fb[j] = *reinterpret_cast<const v4i*>(lds_w + ((wave_n * TN + j) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane&31) and rows 8*(r/4) + 4*(lane>>5) + r%4 of each 32x32 block
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = n0 + (wave_n * TN + j) * 32 + (lane & 31);
+        if (col >= p.n) continue;
+        const float wscale = __half2float(ws[col]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int local = (wave_m * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (local < rows_here) {
+                    const int64_t row = row0 + local;
+                    const float value = rescale(acc[i][j][r], wscale, __half2float(p.as[row]));
+                    if (p.out_f32)
+                        reinterpret_cast<float*>(p.out)[row * p.stride + col] = value;
+                    else
+                        reinterpret_cast<__half*>(p.out)[row * p.stride + col] = __float2half_rn(value);
+                }
+            }
+        }
+    }
+}
+
+// Whole-matrix decode to int8 (diagnostic; e8p_q4.py:267-302).  One thread per code.
+template <int CODEC>
+__global__ __launch_bounds__(256) void unpack_kernel(const void* __restrict__ w, const uint32_t* __restrict__ book,
+                                                     uint2* __restrict__ out, int n, int k, int packed_k) {
+    __shared__ typename Tables<CODEC>::type tables;
+    build_tables(tables, book, threadIdx.x, 256);
+    __syncthreads();
+    const int64_t total = (int64_t)n * (k / 8);
+    const int64_t index = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (index >= total) return;
+    const int row = (int)(index / (k / 8)), vec = (int)(index % (k / 8));
+    int64_t src = index;
+    if (packed_k) {
+        const int per = packed_k / 8;
+        src = ((int64_t)(vec / per) * n + row) * per + vec % per;
+    }
+    if constexpr (CODEC == kQ4)
+        out[index] = decode_q4(tables, reinterpret_cast<const uint32_t*>(w)[src]);
+    else
+        out[index] = decode_q2(tables, reinterpret_cast<const uint16_t*>(w)[src]);
+}
+
+// ---- host side -----------------------------------------------------------------------------
+// slots: M/capacity, N, K, stride, packed_k, algorithm, block_m (gemv passes), flags (codec),
+// E/tiles (grouped), out_f32.
+
+int pick_bm(int rows) { return rows <= 32 ? 32 : rows <= 64 ? 64 : 128; }
+
+template <int CODEC, bool GROUPED>
+int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stream) {
+    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    switch (bm) {
+        case 32:
+            hipLaunchKernelGGL((gemm_kernel<CODEC, 32, 128, 1, GROUPED>), grid, block, 0, stream, p);
+            break;
+        case 64:
+            hipLaunchKernelGGL((gemm_kernel<CODEC, 64, 128, 2, GROUPED>), grid, block, 0, stream, p);
+            break;
+        default:
+            hipLaunchKernelGGL((gemm_kernel<CODEC, 128, 128, 2, GROUPED>), grid, block, 0, stream, p);
+            break;
+    }
+    return hip_check(hipGetLastError(), "launch projection (mfma)");
+}
+
+bool use_gemv(const orx_function& f, int rows) {
+    return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
+}
+
+int projection_geometry(const orx_function& f, int rows, Geometry* g) {
+    if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
+    const int bm = f.tiles ? f.tiles : pick_bm(rows);
+    g->grid[0] = ceil_div((uint32_t)f.N, 128u);
+    g->grid[1] = ceil_div((uint32_t)rows, (uint32_t)bm);
+    g->block[0] = 256;
+    g->shared = 0;
+    return ORX_OK;
+}
+
+// E8P-Q4: A, AS, Book, Out, S, W[, m]   (e8p_q4.py:248-255 in generated-ABI order)
+int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.as = pointer_arg<const __half>(args, 1);
+    p.book = pointer_arg<const uint32_t>(args, 2);
+    p.out = pointer_arg<void>(args, 3);
+    p.ws = pointer_arg<const __half>(args, 4);
+    p.w = pointer_arg<const void>(args, 5);
+    p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
+    if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
+}
+
+// W8A8: A, Output, TokenScale, Weight, WeightScale[, m]   (int8_projection.py:51-57)
+int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.out = pointer_arg<void>(args, 1);
+    p.as = pointer_arg<const __half>(args, 2);
+    p.w = pointer_arg<const void>(args, 3);
+    p.ws = pointer_arg<const __half>(args, 4);
+    p.book = nullptr;
+    p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = 0, p.out_f32 = f.out_f32;
+    if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
+}
+
+int make_projection(const Variant& v, orx_function* f, int codec) {
+    bool bad = false;
+    f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    f->stride = (int)v.integer("output_stride", f->N, &bad);
+    f->packed_k = (int)v.integer("packed_k", 0, &bad);
+    f->tiles = (int)v.integer("block_m", 0, &bad);  // forced MFMA row tile, 0 = by row count
+    const int passes = (int)v.integer("gemv_passes", 0, &bad);
+    const std::string dtype = v.string("output_dtype", "float16", &bad);
+    const std::string algorithm = v.string("algorithm", "auto", &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    const char* name = f->symbol.c_str();
+    // validate_shape + K*128*127 < 2^31 (q4_projection.py:33-35, int8_projection.py:29)
+    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % kBK || (int64_t)f->K * 128 * 128 > 2147483647LL) {
+        set_error("%s: need M,N,K > 0, K a multiple of 128 and K*2^14 < 2^31", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->stride < f->N) {
+        set_error("%s: output_stride must contain the entire row", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (dtype != "float16" && dtype != "float32") {
+        set_error("%s: output_dtype must be float16 or float32", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->packed_k != 0 && (f->packed_k != 128 || codec == kW8)) {
+        set_error("%s: packed_k must be 0 or 128 (codes only)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->tiles != 0 && f->tiles != 32 && f->tiles != 64 && f->tiles != 128) {
+        set_error("%s: block_m must be 32, 64 or 128", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->out_f32 = dtype == "float32";
+    f->capacity = f->M;
+    f->flags = codec;
+    f->algorithm = algorithm == "gemv" ? kGemv : algorithm == "mfma" ? kMfma : algorithm == "auto" ? kAuto : -1;
+    if (f->algorithm < 0) {
+        set_error("%s: algorithm must be auto, gemv or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kGemv && f->packed_k != 0) {
+        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kGemv || (f->algorithm == kAuto && f->packed_k == 0)) {
+        orx_function probe = *f;
+        if (probe.capacity > 4) probe.capacity = 4;
+        int code = gemv_configure(&probe, codec, passes);
+        if (code != ORX_OK) {
+            if (f->algorithm == kGemv) return code;
+            f->algorithm = kMfma;
+        } else {
+            if (f->algorithm == kGemv && f->capacity > 4) return gemv_configure(f, codec, passes);  // reports the error
+            f->block_m = probe.block_m;
+        }
+    }
+    f->geometry = projection_geometry;
+    f->device_function = reinterpret_cast<const void*>(&gemm_kernel<kW8, 128, 128, 2, false>);
+    return ORX_OK;
+}
+
+int make_q4_projection(const Variant& v, orx_function* f) {
+    int code = make_projection(v, f, kQ4);
+    if (code != ORX_OK) return code;
+    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4},
+               {"Out", ArgPointer, 2}, {"S", ArgPointer, 2},  {"W", ArgPointer, 16}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->launch = q4_launch;
+    return ORX_OK;
+}
+
+int make_w8_projection(const Variant& v, orx_function* f) {
+    int code = make_projection(v, f, kW8);
+    if (code != ORX_OK) return code;
+    f->args = {{"A", ArgPointer, 16},     {"Output", ArgPointer, 2},      {"TokenScale", ArgPointer, 2},
+               {"Weight", ArgPointer, 16}, {"WeightScale", ArgPointer, 2}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->launch = w8_launch;
+    return ORX_OK;
+}
+
+// ---- routed single-stage experts -----------------------------------------------------------
+// A, AS, Book, C, Counts, Offsets, P, TileCount, TileExpert, TileRow, WS
+// (tests/cuda/operators/e8p_decode.py:72-84; kernels/cuda/model/e8p_decode.py:60-73 without Patch)
+int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)f.N, 128u);
+    g->grid[1] = (uint32_t)f.tiles;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.as = pointer_arg<const __half>(args, 1);
+    p.book = pointer_arg<const uint32_t>(args, 2);
+    p.out = pointer_arg<void>(args, 3);
+    p.counts = pointer_arg<const int>(args, 4);
+    p.offsets = pointer_arg<const int>(args, 5);
+    p.w = pointer_arg<const void>(args, 6);
+    p.tile_count = pointer_arg<const int>(args, 7);
+    p.tile_expert = pointer_arg<const int>(args, 8);
+    p.tile_row = pointer_arg<const int>(args, 9);
+    p.ws = pointer_arg<const __half>(args, 10);
+    p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
+    p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
+    return launch_mfma<kQ2, true>(f.block_m, p, g, stream);
+}
+
+int make_q2_grouped(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("rows", 0, &bad);
+    f->E = (int)v.integer("E", 0, &bad);
+    f->tiles = (int)v.integer("tiles", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->block_m = (int)v.integer("block_m", 32, &bad);
+    f->packed_k = (int)v.integer("packed_k", 128, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    const char* name = f->symbol.c_str();
+    if (f->M <= 0 || f->E <= 0 || f->tiles <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 ||
+        (int64_t)f->K * 128 * 128 > 2147483647LL) {
+        set_error("%s: invalid E8P decode geometry", name);  // e8p_decode.py:52
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->block_m != 32 && f->block_m != 64 && f->block_m != 128) {
+        set_error("%s: block_m must be 32, 64 or 128 (rows per routed tile)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->packed_k != 128 && f->packed_k != 0) {
+        set_error("%s: packed_k must be 128 (K-major) or 0 (row-major per expert)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"A", ArgPointer, 16},         {"AS", ArgPointer, 2},         {"Book", ArgPointer, 4},
+               {"C", ArgPointer, 2},          {"Counts", ArgPointer, 4},     {"Offsets", ArgPointer, 4},
+               {"P", ArgPointer, 16},         {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
+               {"TileRow", ArgPointer, 4},    {"WS", ArgPointer, 2}};
+    f->geometry = grouped_geometry;
+    f->launch = grouped_launch;
+    f->device_function = reinterpret_cast<const void*>(&gemm_kernel<kQ2, 32, 128, 1, true>);
+    return ORX_OK;
+}
+
+// ---- unpack ----------------------------------------------------------------------------------
+// Book, Output, W
+int unpack_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)((int64_t)f.N * (f.K / 8)), 256u);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int unpack_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    const uint32_t* book = pointer_arg<const uint32_t>(args, 0);
+    uint2* out = pointer_arg<uint2>(args, 1);
+    const void* w = pointer_arg<const void>(args, 2);
+    if (f.flags == kQ4)
+        hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k);
+    else
+        hipLaunchKernelGGL((unpack_kernel<kQ2>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k);
+    return hip_check(hipGetLastError(), "launch unpack");
+}
+
+int make_unpack(const Variant& v, orx_function* f, int codec) {
+    bool bad = false;
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->packed_k = (int)v.integer("packed_k", 0, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->N <= 0 || f->K <= 0 || f->K % 128 || (f->packed_k != 0 && f->packed_k != 64 && f->packed_k != 128)) {
+        set_error("%s: need N,K > 0, K a multiple of 128, packed_k in {0,64,128}", f->symbol.c_str());
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->capacity = 1;
+    f->flags = codec;
+    f->args = {{"Book", ArgPointer, 4}, {"Output", ArgPointer, 8}, {"W", ArgPointer, 4}};
+    f->geometry = unpack_geometry;
+    f->launch = unpack_launch;
+    f->device_function = reinterpret_cast<const void*>(&unpack_kernel<kQ4>);
+    return ORX_OK;
+}
+int make_q4_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f, kQ4); }
+int make_q2_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f, kQ2); }
+
+}  // namespace
+
+const Registration* gemm_registrations(int* count) {
+    static const Registration rows[] = {
+    {"e8p_q4_projection", make_q4_projection,
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, packed_k=0|128, output_dtype=float16|float32, "
+     "output_stride=N, block_m=0|32|64|128, gemv_passes=0",
+     "A,AS,Book,Out,S,W[,m]"},
+    {"int8_projection", make_w8_projection,
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, output_dtype=float16|float32, output_stride=N, "
+     "block_m=0|32|64|128",
+     "A,Output,TokenScale,Weight,WeightScale[,m]"},
+    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0",
+     "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
+    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0",
+     "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
+    {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
+    {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
+    };
+    *count = 6;
+    return rows;
+}
+
+}  // namespace orx

@@ -1,0 +1,411 @@
+// MoE routing, dispatch and weighted combine around the grouped expert projections.
+//
+// Reference: kernels/cuda/model/moe.py -- router_topk (:413-494), expert_histogram (:177-210),
+// expert_offsets (:214-244), expert_tiles (:248-282), expert_dispatch (:286-329),
+// moe_combine (:498-554).  All metadata is int32, assignment order is token-major /
+// rank-minor, and nothing here uses atomics: each output element has exactly one writer, so
+// the result is deterministic and every kernel is replayable inside a captured graph.
+#include <hip/hip_fp16.h>
+
+#include "orx_internal.h"
+
+namespace orx {
+namespace {
+
+// Total order on finite fp32 with -0 == +0 (moe.py:449-465): larger key = larger score.
+__device__ __forceinline__ uint32_t ordered_key(float value) {
+    const uint32_t bits = __float_as_uint(value);
+    if (value == 0.f) return 0x80000000u;
+    return (bits & 0x80000000u) ? ~bits : bits ^ 0x80000000u;
+}
+__device__ __forceinline__ float key_value(uint32_t ordered) {
+    return __uint_as_float((ordered & 0x80000000u) ? ordered ^ 0x80000000u : ~ordered);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        const unsigned long long other = __shfl_xor(v, offset, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+    return v;
+}
+
+// One wave per row; each lane keeps ceil(E/64) keys in registers.  Key = ordered score in the
+// high word, (E - id) in the low word, so one max picks the score and the lowest id on ties.
+constexpr int kMaxLocal = 16;  // E <= 1024
+__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids,
+                                                          float* __restrict__ prob, int m, int e, int top_k,
+                                                          int renormalize) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= m) return;
+    unsigned long long keys[kMaxLocal];
+    float all_exp = 0.f;
+    float local_max = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < kMaxLocal; ++j) {
+        const int id = j * 64 + lane;
+        keys[j] = 0ull;
+        if (id < e) {
+            const float v = logits[(int64_t)row * e + id];
+            keys[j] = ((unsigned long long)ordered_key(v) << 32) | (unsigned long long)(uint32_t)(e - id);
+            local_max = fmaxf(local_max, v);
+        }
+    }
+    float global_max = local_max;
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, offset, 64));
+    if (!renormalize) {
+#pragma unroll
+        for (int j = 0; j < kMaxLocal; ++j) {
+            const int id = j * 64 + lane;
+            if (id < e) all_exp += expf(logits[(int64_t)row * e + id] - global_max);
+        }
+        all_exp = wave_sum(all_exp);
+    }
+    float mine = 0.f;  // numerator of rank == lane
+    for (int rank = 0; rank < top_k; ++rank) {
+        unsigned long long best = 0ull;
+#pragma unroll
+        for (int j = 0; j < kMaxLocal; ++j) best = keys[j] > best ? keys[j] : best;
+        best = wave_max_u64(best);
+        const int id = e - (int)(uint32_t)(best & 0xFFFFFFFFull);
+        const float score = key_value((uint32_t)(best >> 32));
+#pragma unroll
+        for (int j = 0; j < kMaxLocal; ++j)
+            if (j * 64 + lane == id) keys[j] = 0ull;
+        if (lane == rank) {
+            ids[(int64_t)row * top_k + rank] = id;
+            mine = expf(score - global_max);
+        }
+    }
+    const float selected_sum = wave_sum(lane < top_k ? mine : 0.f);
+    if (lane < top_k) prob[(int64_t)row * top_k + lane] = __fdiv_rn(mine, renormalize ? selected_sum : all_exp);
+}
+
+// Block-wide exclusive prefix of a 0/1 flag; returns this thread's prefix and the block total.
+__device__ __forceinline__ int block_flag_scan(bool flag, int* wave_totals, int* total) {
+    const unsigned long long ballot = __ballot(flag);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int within = __popcll(ballot & ((1ull << lane) - 1ull));
+    __syncthreads();  // previous round's readers are done with wave_totals
+    if (lane == 0) wave_totals[wave] = __popcll(ballot);
+    __syncthreads();
+    int before = 0, sum = 0;
+    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) {
+        const int t = wave_totals[w];
+        if (w < wave) before += t;
+        sum += t;
+    }
+    *total = sum;
+    return before + within;
+}
+
+// grid E: expert e scans every assignment in token-major order.
+__global__ __launch_bounds__(256) void expert_histogram_kernel(const int* __restrict__ ids, int* __restrict__ counts,
+                                                               int* __restrict__ relative, int assignments) {
+    __shared__ int wave_totals[4];
+    const int expert = blockIdx.x;
+    int base = 0;
+    for (int first = 0; first < assignments; first += 256) {
+        const int i = first + threadIdx.x;
+        const bool match = i < assignments && ids[i] == expert;
+        int total;
+        const int prefix = block_flag_scan(match, wave_totals, &total);
+        if (match) relative[i] = base + prefix;
+        base += total;
+    }
+    if (threadIdx.x == 0) counts[expert] = base;
+}
+
+// one block: exclusive prefixes of counts and of ceil(counts/bm); TileCount = total tiles.
+__global__ __launch_bounds__(256) void expert_offsets_kernel(const int* __restrict__ counts, int* __restrict__ row_offsets,
+                                                             int* __restrict__ tile_count, int* __restrict__ tile_offsets,
+                                                             int experts, int block_m) {
+    __shared__ int rows_scan[256], tiles_scan[256];
+    int row_base = 0, tile_base = 0;
+    for (int first = 0; first < experts; first += 256) {
+        const int e = first + threadIdx.x;
+        const int c = e < experts ? counts[e] : 0;
+        const int t = (c + block_m - 1) / block_m;
+        rows_scan[threadIdx.x] = c;
+        tiles_scan[threadIdx.x] = t;
+        __syncthreads();
+        for (int offset = 1; offset < 256; offset <<= 1) {
+            const int r = threadIdx.x >= offset ? rows_scan[threadIdx.x - offset] : 0;
+            const int s = threadIdx.x >= offset ? tiles_scan[threadIdx.x - offset] : 0;
+            __syncthreads();
+            rows_scan[threadIdx.x] += r;
+            tiles_scan[threadIdx.x] += s;
+            __syncthreads();
+        }
+        if (e < experts) {
+            row_offsets[e] = row_base + rows_scan[threadIdx.x] - c;
+            tile_offsets[e] = tile_base + tiles_scan[threadIdx.x] - t;
+        }
+        row_base += rows_scan[255];
+        tile_base += tiles_scan[255];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) tile_count[0] = tile_base;
+}
+
+// grid E
+__global__ __launch_bounds__(256) void expert_tiles_kernel(const int* __restrict__ counts, int* __restrict__ tile_expert,
+                                                           const int* __restrict__ tile_offsets, int* __restrict__ tile_row,
+                                                           int block_m) {
+    const int e = blockIdx.x;
+    const int c = counts[e], base = tile_offsets[e];
+    for (int tile = threadIdx.x; tile * block_m < c; tile += 256) {
+        tile_expert[base + tile] = e;
+        tile_row[base + tile] = tile * block_m;
+    }
+}
+
+// grid M*top_k: copy one int8 row and its scales to the expert-sorted slot.
+__global__ __launch_bounds__(256) void expert_dispatch_kernel(const int8_t* __restrict__ a, int8_t* __restrict__ d,
+                                                              __half* __restrict__ ds, const int* __restrict__ ids,
+                                                              const int* __restrict__ relative,
+                                                              const int* __restrict__ row_offsets,
+                                                              const __half* __restrict__ scale, int* __restrict__ slot_map,
+                                                              int h, int groups, int top_k) {
+    const int assignment = blockIdx.x;
+    const int row = assignment / top_k;
+    const int slot = row_offsets[ids[assignment]] + relative[assignment];
+    if (threadIdx.x == 0) slot_map[assignment] = slot;
+    const int8_t* src = a + (int64_t)row * h;
+    int8_t* dst = d + (int64_t)slot * h;
+    if ((h & 15) == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(d)) & 15) == 0) {
+        for (int i = threadIdx.x; i < h / 16; i += 256)
+            reinterpret_cast<uint4*>(dst)[i] = reinterpret_cast<const uint4*>(src)[i];
+    } else {
+        for (int i = threadIdx.x; i < h; i += 256) dst[i] = src[i];
+    }
+    for (int g = threadIdx.x; g < groups; g += 256) ds[(int64_t)slot * groups + g] = scale[(int64_t)row * groups + g];
+}
+
+// grid (M, ceil(H/256)): fp32 accumulate in rank order, one fp16 cast.
+__global__ __launch_bounds__(256) void moe_combine_kernel(const __half* __restrict__ expert, __half* __restrict__ output,
+                                                          const float* __restrict__ prob, const __half* __restrict__ shared,
+                                                          const __half* __restrict__ shared_gate,
+                                                          const int* __restrict__ slot_map, int h, int slots, int top_k) {
+    const int row = blockIdx.x;
+    const int col = blockIdx.y * 256 + threadIdx.x;
+    if (col >= h) return;
+    float acc = 0.f;
+    for (int rank = 0; rank < top_k; ++rank) {
+        const int slot = slot_map[(int64_t)row * top_k + rank];
+        if (slot >= 0 && slot < slots)
+            acc += __half2float(expert[(int64_t)slot * h + col]) * prob[(int64_t)row * top_k + rank];
+    }
+    if (shared != nullptr) {
+        const float gate = __fdiv_rn(1.0f, 1.0f + expf(-__half2float(shared_gate[row])));
+        acc = acc + gate * __half2float(shared[(int64_t)row * h + col]);
+    }
+    output[(int64_t)row * h + col] = __float2half_rn(acc);
+}
+
+// ---- host side -----------------------------------------------------------------------------
+bool geometry_fields(const Variant& v, orx_function* f, bool need_m) {
+    bool bad = false;
+    f->M = (int)v.integer("M", need_m ? 0 : 1, &bad);
+    f->E = (int)v.integer("E", 512, &bad);
+    f->top_k = (int)v.integer("top_k", 10, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    f->capacity = f->M;
+    return !bad;
+}
+
+int rows_geometry_router(const orx_function&, int rows, Geometry* g) {
+    g->grid[0] = ceil_div((uint32_t)rows, 4u);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int router_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(router_topk_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const float>(args, 1),
+                       pointer_arg<int>(args, 0), pointer_arg<float>(args, 2), rows, f.E, f.top_k, f.flags);
+    return hip_check(hipGetLastError(), "launch router_topk");
+}
+int make_router(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->flags = v.boolean("renormalize", true, &bad) ? 1 : 0;
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || f->top_k > 64 || f->E > 64 * kMaxLocal) {
+        set_error("router_topk: invalid MoE router dimensions (need top_k <= min(E,64), E <= 1024)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"IDs", ArgPointer, 4}, {"Logits", ArgPointer, 4}, {"Prob", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = rows_geometry_router;
+    f->launch = router_launch;
+    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel);
+    return ORX_OK;
+}
+
+int histogram_geometry(const orx_function& f, int, Geometry* g) {
+    g->grid[0] = (uint32_t)f.E;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int histogram_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(expert_histogram_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 1),
+                       pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), rows * f.top_k);
+    return hip_check(hipGetLastError(), "launch expert_histogram");
+}
+int make_histogram(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E) {
+        set_error("expert_histogram: invalid MoE dispatch dimensions");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"Counts", ArgPointer, 4}, {"IDs", ArgPointer, 4}, {"RelativeSlot", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = histogram_geometry;
+    f->launch = histogram_launch;
+    f->device_function = reinterpret_cast<const void*>(&expert_histogram_kernel);
+    return ORX_OK;
+}
+
+int one_block_geometry(const orx_function&, int, Geometry* g) {
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int offsets_launch(const orx_function& f, int, const Geometry&, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(expert_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 0),
+                       pointer_arg<int>(args, 1), pointer_arg<int>(args, 2), pointer_arg<int>(args, 3), f.E, f.block_m);
+    return hip_check(hipGetLastError(), "launch expert_offsets");
+}
+bool valid_block_m(int bm) { return bm == 8 || bm == 16 || bm == 32 || bm == 64 || bm == 128 || bm == 256; }
+int make_offsets(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->E = (int)v.integer("E", 512, &bad);
+    f->block_m = (int)v.integer("block_m", 16, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->E <= 0 || !valid_block_m(f->block_m)) {
+        set_error("expert_offsets: invalid MoE expert prefix dimensions");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->capacity = 1;
+    f->args = {{"Counts", ArgPointer, 4}, {"RowOffsets", ArgPointer, 4}, {"TileCount", ArgPointer, 4},
+               {"TileOffsets", ArgPointer, 4}};
+    f->geometry = one_block_geometry;
+    f->launch = offsets_launch;
+    f->device_function = reinterpret_cast<const void*>(&expert_offsets_kernel);
+    return ORX_OK;
+}
+
+int tiles_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(expert_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 0),
+                       pointer_arg<int>(args, 1), pointer_arg<const int>(args, 2), pointer_arg<int>(args, 3), f.block_m);
+    return hip_check(hipGetLastError(), "launch expert_tiles");
+}
+int make_tiles(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->block_m = (int)v.integer("block_m", 16, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->E <= 0 || f->top_k <= 0 || !valid_block_m(f->block_m)) {
+        set_error("expert_tiles: invalid MoE tile dimensions");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->dynamic_rows = false;
+    f->args = {{"Counts", ArgPointer, 4}, {"TileExpert", ArgPointer, 4}, {"TileOffsets", ArgPointer, 4},
+               {"TileRow", ArgPointer, 4}};
+    f->geometry = histogram_geometry;
+    f->launch = tiles_launch;
+    f->device_function = reinterpret_cast<const void*>(&expert_tiles_kernel);
+    return ORX_OK;
+}
+
+int dispatch_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)(rows * f.top_k);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int dispatch_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(expert_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int8_t>(args, 0),
+                       pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 2), pointer_arg<const int>(args, 3),
+                       pointer_arg<const int>(args, 4), pointer_arg<const int>(args, 5),
+                       pointer_arg<const __half>(args, 6), pointer_arg<int>(args, 7), f.H, f.H / f.group, f.top_k);
+    return hip_check(hipGetLastError(), "launch expert_dispatch");
+}
+int make_dispatch(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->H = (int)v.integer("H", 0, &bad);
+    f->group = (int)v.integer("scale_group", f->H, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->H <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || f->group <= 0 || f->H % f->group) {
+        set_error("expert_dispatch: invalid MoE activation dispatch dimensions");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"A", ArgPointer, 1},          {"D", ArgPointer, 1},          {"DS", ArgPointer, 2},
+               {"IDs", ArgPointer, 4},        {"RelativeSlot", ArgPointer, 4}, {"RowOffsets", ArgPointer, 4},
+               {"Scale", ArgPointer, 2},      {"SlotMap", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = dispatch_geometry;
+    f->launch = dispatch_launch;
+    f->device_function = reinterpret_cast<const void*>(&expert_dispatch_kernel);
+    return ORX_OK;
+}
+
+int combine_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->grid[1] = ceil_div((uint32_t)f.H, 256u);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int combine_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    // dynamic decode has exactly top_k assignments per live row (moe.py:514-517)
+    const int slots = f.dynamic_rows ? rows * f.top_k : f.slots;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
+                       pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), pointer_arg<const float>(args, 2),
+                       pointer_arg<const __half>(args, 3), pointer_arg<const __half>(args, 4),
+                       pointer_arg<const int>(args, 5), f.H, slots, f.top_k);
+    return hip_check(hipGetLastError(), "launch moe_combine");
+}
+int make_combine(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->H = (int)v.integer("H", 0, &bad);
+    f->slots = (int)v.integer("slots", f->M * f->top_k, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->H <= 0 || f->slots <= 0 || f->top_k <= 0) {
+        set_error("moe_combine: invalid MoE mixture dimensions");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    // Shared / SharedGate may be null device pointers: then no shared expert is added
+    f->args = {{"Expert", ArgPointer, 2},     {"Output", ArgPointer, 2},           {"Prob", ArgPointer, 4},
+               {"Shared", ArgPointer, 0x80000002u}, {"SharedGate", ArgPointer, 0x80000002u}, {"SlotMap", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = combine_geometry;
+    f->launch = combine_launch;
+    f->device_function = reinterpret_cast<const void*>(&moe_combine_kernel);
+    return ORX_OK;
+}
+
+}  // namespace
+
+const Registration* moe_registrations(int* count) {
+    static const Registration rows[] = {
+    {"router_topk", make_router, "M, E=512, top_k=10, renormalize=true, dynamic_rows=false", "IDs,Logits,Prob[,m]"},
+    {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
+    {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
+    {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
+    {"expert_dispatch", make_dispatch, "M, H, E=512, top_k=10, scale_group=H, dynamic_rows=false",
+     "A,D,DS,IDs,RelativeSlot,RowOffsets,Scale,SlotMap[,m]"},
+    {"moe_combine", make_combine, "M, H, slots=M*top_k, top_k=10, dynamic_rows=false",
+     "Expert,Output,Prob,Shared,SharedGate,SlotMap[,m]"},
+    };
+    *count = 6;
+    return rows;
+}
+
+}  // namespace orx

@@ -1,0 +1,213 @@
+// Activation A8 quantiser and the fp16 SwiGLU boundary in front of it.
+//
+// activation_quantization follows kernels/cuda/operators/op30_activation_quantization.py:
+// per (row, group): amax -> scale = fp16(max(amax/127, 2^-24)) (1 when amax == 0) ->
+// code = clamp(rint(x / fp32(scale)), -127, 127) with a correctly rounded divide and
+// ties-to-even (:14-18, :49-65, contract text :71-78).  `fused` quantises
+// fp16(silu(gate)*up) read from X[rows, 2K] (:43-46, op04_swiglu.py:6-17).
+// The kernel is memory-bound: one fp16 read (twice, second pass from L2) and one int8 write.
+#include <hip/hip_fp16.h>
+
+#include "orx_internal.h"
+
+namespace orx {
+namespace {
+
+__device__ __forceinline__ float swiglu_value(__half gate, __half up) {
+    const float g = __half2float(gate), u = __half2float(up);
+    const float e = expf(-fabsf(g));
+    const float sigmoid = g >= 0.f ? __fdiv_rn(1.0f, 1.0f + e) : __fdiv_rn(e, 1.0f + e);
+    // one fp16 rounding here: the value a downstream quantiser sees is the materialised fp16
+    return __half2float(__float2half_rn((g * sigmoid) * u));
+}
+
+template <bool FUSED, bool MASKED>
+__device__ __forceinline__ float load_value(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
+                                            int64_t row_base, int k, int col) {
+    float v;
+    if (FUSED)
+        v = swiglu_value(x[row_base + col], x[row_base + k + col]);
+    else
+        v = __half2float(x[row_base + col]);
+    if (MASKED && mask[col] != 0) v = 0.f;
+    return v;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, 64));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    const int waves = (blockDim.x + 63) >> 6;
+    float r = scratch[0];
+    for (int i = 1; i < waves; ++i) r = fmaxf(r, scratch[i]);
+    return r;
+}
+
+__device__ __forceinline__ int8_t quantise(float value, float scale) {
+    const float r = rintf(__fdiv_rn(value, scale));
+    return (int8_t)fmaxf(-127.f, fminf(127.f, r));
+}
+
+// grid (rows, groups), 256 threads.
+template <bool FUSED, bool MASKED>
+__global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
+                                                 int8_t* __restrict__ q, __half* __restrict__ s, int k, int group,
+                                                 int groups) {
+    __shared__ float scratch[4];
+    const int row = blockIdx.x, g = blockIdx.y;
+    const int first = g * group;
+    const int width = min(group, k - first);
+    const int64_t in_base = (int64_t)row * (FUSED ? 2 * k : k);
+    const int64_t out_base = (int64_t)row * k;
+    // 8 halves per thread per step when everything is 16-byte aligned and unmasked/unfused
+    const bool vector = !FUSED && !MASKED && (k % 8 == 0) && (group % 8 == 0) &&
+                        ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
+    float amax = 0.f;
+    if (vector) {
+        const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
+        for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
+            const uint4 raw = src[i];
+            const __half2* h = reinterpret_cast<const __half2*>(&raw);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float2 f = __half22float2(h[j]);
+                amax = fmaxf(amax, fmaxf(fabsf(f.x), fabsf(f.y)));
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x)
+            amax = fmaxf(amax, fabsf(load_value<FUSED, MASKED>(x, mask, in_base, k, first + i)));
+    }
+    amax = block_max(amax, scratch);
+    const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
+    const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
+    if (threadIdx.x == 0) s[(int64_t)row * groups + g] = stored;
+    const float scale = __half2float(stored);
+    if (vector) {
+        const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
+        uint2* dst = reinterpret_cast<uint2*>(q + out_base + first);
+        for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
+            const uint4 raw = src[i];
+            const __half* h = reinterpret_cast<const __half*>(&raw);
+            uint32_t lo = 0, hi = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                lo |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
+                hi |= ((uint32_t)(uint8_t)quantise(__half2float(h[j + 4]), scale)) << (8 * j);
+            }
+            dst[i] = make_uint2(lo, hi);
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x)
+            q[out_base + first + i] = quantise(load_value<FUSED, MASKED>(x, mask, in_base, k, first + i), scale);
+    }
+}
+
+// fp16 [rows, 2I] -> fp16 [rows, I].  grid (rows, ceil(I/256)).
+__global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ x, __half* __restrict__ y, int width) {
+    const int row = blockIdx.x;
+    const int col = blockIdx.y * 256 + threadIdx.x;
+    if (col < width) {
+        const int64_t base = (int64_t)row * 2 * width;
+        y[(int64_t)row * width + col] = __float2half_rn(swiglu_value(x[base + col], x[base + width + col]));
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------
+// slots used: K, group, flags (bit0 masked, bit1 fused), capacity
+int a8_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->grid[1] = ceil_div((uint32_t)f.K, (uint32_t)f.group);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    const uint8_t* mask = pointer_arg<const uint8_t>(args, 0);
+    int8_t* q = pointer_arg<int8_t>(args, 1);
+    __half* s = pointer_arg<__half>(args, 2);
+    const __half* x = pointer_arg<const __half>(args, 3);
+    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    const int groups = (int)g.grid[1];
+    const bool masked = f.flags & 1, fused = f.flags & 2;
+    if (fused && masked)
+        hipLaunchKernelGGL((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+    else if (fused)
+        hipLaunchKernelGGL((a8_kernel<true, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+    else if (masked)
+        hipLaunchKernelGGL((a8_kernel<false, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+    else
+        hipLaunchKernelGGL((a8_kernel<false, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+    return hip_check(hipGetLastError(), "launch activation_quantization");
+}
+
+int make_a8(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("K", 0, &bad);
+    f->group = (int)v.integer("group_size", f->K, &bad);
+    const bool masked = v.boolean("masked", false, &bad);
+    const bool fused = v.boolean("fused", false, &bad);
+    f->capacity = (int)v.integer("M", 1 << 24, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->K <= 0 || f->group <= 0 || f->group > f->K || f->capacity < 1) {
+        set_error("activation_quantization: need K > 0 and 0 < group_size <= K");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = (masked ? 1 : 0) | (fused ? 2 : 0);
+    f->dynamic_rows = true;
+    // Mask may be null unless masked (the reference ignores it then, op30:75-76)
+    f->args = {{"Mask", ArgPointer, masked ? 1u : 0x80000001u}, {"Q", ArgPointer, 1}, {"S", ArgPointer, 2},
+               {"X", ArgPointer, 2}, {"rows", ArgI32, 4}};
+    f->device_function = reinterpret_cast<const void*>(&a8_kernel<false, false>);
+    f->geometry = a8_geometry;
+    f->launch = a8_launch;
+    return ORX_OK;
+}
+
+int swiglu_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->grid[1] = ceil_div((uint32_t)f.N, 256u);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int swiglu_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    hipLaunchKernelGGL(swiglu_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream,
+                       pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), f.N);
+    return hip_check(hipGetLastError(), "launch swiglu");
+}
+
+int make_swiglu(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->N = (int)v.integer("I", 0, &bad);
+    f->capacity = (int)v.integer("M", 1 << 24, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->N <= 0) {
+        set_error("swiglu: need I > 0");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->dynamic_rows = true;
+    f->args = {{"X", ArgPointer, 2}, {"Y", ArgPointer, 2}, {"rows", ArgI32, 4}};
+    f->device_function = reinterpret_cast<const void*>(&swiglu_kernel);
+    f->geometry = swiglu_geometry;
+    f->launch = swiglu_launch;
+    return ORX_OK;
+}
+
+}  // namespace
+
+const Registration* quant_registrations(int* count) {
+    static const Registration rows[] = {
+    {"activation_quantization", make_a8, "K, group_size=null, masked=false, fused=false, M=capacity",
+     "Mask,Q,S,X,rows"},
+    {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
+    };
+    *count = 2;
+    return rows;
+}
+
+}  // namespace orx

@@ -1,0 +1,366 @@
+// liborx C ABI: resolve + launch, the HIP stand-in for orinfer's Catalog::resolve
+// (crates/orinfer-engine/src/backend/cuda/kernels.rs:114-192) and launch_kernel
+// (crates/orinfer-engine/src/backend/cuda/mod.rs:312-341).
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <cmath>
+
+#include "orx_internal.h"
+
+namespace orx {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* format, ...) {
+    va_list ap;
+    va_start(ap, format);
+    vsnprintf(g_error, sizeof g_error, format, ap);
+    va_end(ap);
+}
+
+int hip_check(hipError_t code, const char* operation) {
+    if (code == hipSuccess) return ORX_OK;
+    // Same text shape as the reference's check(): "<op>: CUDA error <code>" (mod.rs:48-55).
+    set_error("%s: HIP error %d (%s)", operation, (int)code, hipGetErrorName(code));
+    return (int)code;
+}
+
+// ---- flat JSON object parser -------------------------------------------------------------
+namespace {
+struct Cursor {
+    const char* p;
+    void skip() {
+        while (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r') ++p;
+    }
+};
+
+bool parse_string(Cursor& c, std::string* out) {
+    if (*c.p != '"') return false;
+    ++c.p;
+    out->clear();
+    while (*c.p && *c.p != '"') {
+        if (*c.p == '\\') {
+            ++c.p;
+            if (!*c.p) return false;
+        }
+        out->push_back(*c.p++);
+    }
+    if (*c.p != '"') return false;
+    ++c.p;
+    return true;
+}
+}  // namespace
+
+bool parse_variant(const char* json, Variant* out, std::string* error) {
+    out->fields.clear();
+    if (json == nullptr) return true;
+    Cursor c{json};
+    c.skip();
+    if (*c.p == 0) return true;
+    if (*c.p != '{') {
+        *error = "variant must be a JSON object";
+        return false;
+    }
+    ++c.p;
+    c.skip();
+    if (*c.p == '}') return true;
+    for (;;) {
+        c.skip();
+        std::string key;
+        if (!parse_string(c, &key)) {
+            *error = "expected a string key";
+            return false;
+        }
+        c.skip();
+        if (*c.p != ':') {
+            *error = "expected ':' after key " + key;
+            return false;
+        }
+        ++c.p;
+        c.skip();
+        Value v;
+        if (*c.p == '"') {
+            v.kind = Value::String;
+            if (!parse_string(c, &v.text)) {
+                *error = "bad string value for " + key;
+                return false;
+            }
+        } else if (!strncmp(c.p, "true", 4)) {
+            v.kind = Value::Bool;
+            v.number = 1;
+            c.p += 4;
+        } else if (!strncmp(c.p, "false", 5)) {
+            v.kind = Value::Bool;
+            v.number = 0;
+            c.p += 5;
+        } else if (!strncmp(c.p, "null", 4)) {
+            v.kind = Value::Null;
+            c.p += 4;
+        } else {
+            char* end = nullptr;
+            v.number = strtod(c.p, &end);
+            if (end == c.p) {
+                *error = "bad value for " + key;
+                return false;
+            }
+            v.kind = Value::Number;
+            c.p = end;
+        }
+        if (out->fields.count(key)) {
+            *error = "duplicate key " + key;
+            return false;
+        }
+        out->fields[key] = v;
+        c.skip();
+        if (*c.p == ',') {
+            ++c.p;
+            continue;
+        }
+        if (*c.p == '}') {
+            ++c.p;
+            c.skip();
+            if (*c.p != 0) {
+                *error = "trailing text after the object";
+                return false;
+            }
+            return true;
+        }
+        *error = "expected ',' or '}'";
+        return false;
+    }
+}
+
+long long Variant::integer(const char* key, long long fallback, bool* bad) const {
+    auto it = fields.find(key);
+    if (it == fields.end() || it->second.kind == Value::Null) return fallback;
+    if (it->second.kind != Value::Number || std::floor(it->second.number) != it->second.number) {
+        *bad = true;
+        set_error("variant field %s must be an integer", key);
+        return fallback;
+    }
+    return (long long)it->second.number;
+}
+
+bool Variant::boolean(const char* key, bool fallback, bool* bad) const {
+    auto it = fields.find(key);
+    if (it == fields.end() || it->second.kind == Value::Null) return fallback;
+    if (it->second.kind != Value::Bool) {
+        *bad = true;
+        set_error("variant field %s must be true or false", key);
+        return fallback;
+    }
+    return it->second.number != 0;
+}
+
+std::string Variant::string(const char* key, const char* fallback, bool* bad) const {
+    auto it = fields.find(key);
+    if (it == fields.end() || it->second.kind == Value::Null) return fallback;
+    if (it->second.kind != Value::String) {
+        *bad = true;
+        set_error("variant field %s must be a string", key);
+        return fallback;
+    }
+    return it->second.text;
+}
+
+// ---- catalog -------------------------------------------------------------------------------
+namespace {
+struct Table {
+    const Registration* rows;
+    int count;
+};
+void tables(Table out[4]) {
+    out[0].rows = quant_registrations(&out[0].count);
+    out[1].rows = gemv_registrations(&out[1].count);
+    out[2].rows = gemm_registrations(&out[2].count);
+    out[3].rows = moe_registrations(&out[3].count);
+}
+const Registration* find(const char* symbol) {
+    Table t[4];
+    tables(t);
+    for (auto& table : t)
+        for (int i = 0; i < table.count; ++i)
+            if (!strcmp(table.rows[i].symbol, symbol)) return &table.rows[i];
+    return nullptr;
+}
+}  // namespace
+}  // namespace orx
+
+using namespace orx;
+
+extern "C" {
+
+int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
+    if (out == nullptr || symbol == nullptr) {
+        set_error("orx_resolve: null symbol or output");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    *out = nullptr;
+    const Registration* r = find(symbol);
+    if (r == nullptr) {
+        set_error("orx_resolve: unknown symbol %s", symbol);
+        return ORX_ERR_UNKNOWN_SYMBOL;
+    }
+    Variant variant;
+    std::string why;
+    if (!parse_variant(variant_json, &variant, &why)) {
+        set_error("orx_resolve %s: %s", symbol, why.c_str());
+        return ORX_ERR_BAD_VARIANT;
+    }
+    orx_function* f = new orx_function();
+    f->symbol = symbol;
+    int code = r->factory(variant, f);
+    if (code != ORX_OK) {
+        delete f;
+        return code;
+    }
+    if (f->geometry == nullptr || f->launch == nullptr || f->args.empty()) {
+        delete f;
+        set_error("orx_resolve %s: incomplete kernel record", symbol);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    *out = f;
+    return ORX_OK;
+}
+
+int orx_release(orx_fn f) {
+    delete f;
+    return ORX_OK;
+}
+
+int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
+    if (f == nullptr) {
+        set_error("orx_query: null handle");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    hipFuncAttributes attr;
+    memset(&attr, 0, sizeof attr);
+    if (f->device_function != nullptr) {
+        int code = hip_check(hipFuncGetAttributes(&attr, f->device_function), "hipFuncGetAttributes");
+        if (code != ORX_OK) return code;
+    } else {
+        attr.maxThreadsPerBlock = 1024;
+    }
+    if (max_threads_per_block) *max_threads_per_block = (uint32_t)attr.maxThreadsPerBlock;
+    if (static_lds_bytes) *static_lds_bytes = (uint32_t)attr.sharedSizeBytes;
+    return ORX_OK;
+}
+
+int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes) {
+    if (f == nullptr) {
+        set_error("orx_geometry: null handle");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    int live = rows <= 0 ? f->capacity : rows;
+    if (live > f->capacity || (!f->dynamic_rows && live != f->capacity)) {
+        // DynamicBatchKernel::launch rejects rows outside 1..capacity (operators/dynamic.rs:96-98).
+        set_error("%s: rows %d outside the kernel capacity %d", f->symbol.c_str(), live, f->capacity);
+        return ORX_ERR_ROWS;
+    }
+    Geometry g;
+    int code = f->geometry(*f, live, &g);
+    if (code != ORX_OK) return code;
+    for (int i = 0; i < 3; ++i) {
+        if (grid) grid[i] = g.grid[i];
+        if (block) block[i] = g.block[i];
+    }
+    if (shared_bytes) *shared_bytes = g.shared;
+    return ORX_OK;
+}
+
+int orx_arg_count(orx_fn f) { return f ? (int)f->args.size() : 0; }
+
+const char* orx_arg_name(orx_fn f, int index) {
+    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return "";
+    return f->args[index].name;
+}
+
+int orx_arg_kind(orx_fn f, int index) {
+    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return -1;
+    return (int)f->args[index].kind;
+}
+
+int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+               void* hip_stream, void** args) {
+    if (f == nullptr || grid == nullptr || block == nullptr || args == nullptr) {
+        set_error("orx_launch: null handle, geometry or argument list");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    const int count = (int)f->args.size();
+    for (int i = 0; i < count; ++i) {
+        if (args[i] == nullptr) {
+            set_error("launch %s: argument %d (%s) is null", f->symbol.c_str(), i, f->args[i].name);
+            return ORX_ERR_BAD_ARGUMENT;
+        }
+        if (f->args[i].kind == ArgPointer) {
+            const uint64_t address = *reinterpret_cast<uint64_t*>(args[i]);
+            if (address == 0 && !(f->args[i].alignment & 0x80000000u)) {
+                set_error("launch %s: buffer %s is a null device pointer", f->symbol.c_str(), f->args[i].name);
+                return ORX_ERR_BAD_ARGUMENT;
+            }
+            const uint32_t alignment = f->args[i].alignment & 0x7fffffffu;
+            if (alignment > 1 && address % alignment) {
+                set_error("launch %s: buffer %s is not %u-byte aligned", f->symbol.c_str(), f->args[i].name,
+                          alignment);
+                return ORX_ERR_BAD_ARGUMENT;
+            }
+        }
+    }
+    int rows = f->capacity;
+    if (f->dynamic_rows) {
+        rows = int_arg(args, count - 1);
+        if (rows < 1 || rows > f->capacity) {
+            set_error("launch %s: rows %d outside the kernel capacity %d", f->symbol.c_str(), rows, f->capacity);
+            return ORX_ERR_ROWS;
+        }
+    }
+    Geometry want;
+    int code = f->geometry(*f, rows, &want);
+    if (code != ORX_OK) return code;
+    for (int i = 0; i < 3; ++i) {
+        if (grid[i] != want.grid[i] || block[i] != want.block[i]) {
+            set_error("launch %s: geometry grid(%u,%u,%u) block(%u,%u,%u) does not fit the kernel, which needs "
+                      "grid(%u,%u,%u) block(%u,%u,%u) for %d rows",
+                      f->symbol.c_str(), grid[0], grid[1], grid[2], block[0], block[1], block[2], want.grid[0],
+                      want.grid[1], want.grid[2], want.block[0], want.block[1], want.block[2], rows);
+            return ORX_ERR_BAD_GEOMETRY;
+        }
+    }
+    if (shared_bytes != want.shared) {
+        set_error("launch %s: dynamic shared bytes %u, kernel needs %u", f->symbol.c_str(), shared_bytes, want.shared);
+        return ORX_ERR_BAD_GEOMETRY;
+    }
+    return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), args);
+}
+
+const char* orx_last_error(void) { return g_error; }
+
+const char* orx_catalog(void) {
+    static std::string text;
+    if (text.empty()) {
+        std::string s = "{\"kernels\":[";
+        Table t[4];
+        tables(t);
+        bool first = true;
+        for (auto& table : t)
+            for (int i = 0; i < table.count; ++i) {
+                if (!first) s += ",";
+                first = false;
+                s += "{\"symbol\":\"";
+                s += table.rows[i].symbol;
+                s += "\",\"variant_keys\":\"";
+                s += table.rows[i].variant_keys;
+                s += "\",\"arguments\":\"";
+                s += table.rows[i].arguments;
+                s += "\"}";
+            }
+        s += "]}";
+        text = s;
+    }
+    return text.c_str();
+}
+
+}  // extern "C"

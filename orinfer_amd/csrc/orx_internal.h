@@ -1,0 +1,95 @@
+// Host-side internals of liborx: the resolved-function record and the registration
+// interface each kernel file implements.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/orx.h"
+
+namespace orx {
+
+// One value of the flat variant JSON object.
+struct Value {
+    enum Kind { Null, Bool, Number, String } kind = Null;
+    double number = 0;
+    std::string text;
+};
+
+struct Variant {
+    std::map<std::string, Value> fields;
+    bool has(const char* key) const { return fields.count(key) != 0; }
+    // Integer field with a default; sets `bad` if the field exists but is not an integer.
+    long long integer(const char* key, long long fallback, bool* bad) const;
+    bool boolean(const char* key, bool fallback, bool* bad) const;
+    std::string string(const char* key, const char* fallback, bool* bad) const;
+};
+
+bool parse_variant(const char* json, Variant* out, std::string* error);
+
+enum ArgKind { ArgPointer = 0, ArgI32 = 1 };
+struct ArgSpec {
+    const char* name;
+    ArgKind kind;
+    uint32_t alignment;  // bytes the pointer must be aligned to (dtype alignment only)
+};
+
+struct Geometry {
+    uint32_t grid[3] = {1, 1, 1};
+    uint32_t block[3] = {1, 1, 1};
+    uint32_t shared = 0;
+};
+
+}  // namespace orx
+
+// The handle behind orx_fn.  Shape parameters are generic integer slots so that one record
+// type serves every kernel family; each family documents which slots it reads.
+struct orx_function {
+    std::string symbol;
+    std::vector<orx::ArgSpec> args;
+    bool dynamic_rows = false;  // last argument is `int32 m`
+    int capacity = 0;           // largest row count (M of the variant)
+    // shape / configuration
+    int M = 0, N = 0, K = 0, E = 0, top_k = 0, H = 0, stride = 0, group = 0, tiles = 0, slots = 0;
+    int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0;
+    bool out_f32 = false;
+    const void* device_function = nullptr;  // for hipFuncGetAttributes
+    // rows -> geometry; returns ORX_OK or an error code
+    int (*geometry)(const orx_function&, int rows, orx::Geometry*) = nullptr;
+    // enqueue on stream; args already validated for count/alignment
+    int (*launch)(const orx_function&, int rows, const orx::Geometry&, hipStream_t, void** args) = nullptr;
+};
+
+namespace orx {
+
+void set_error(const char* format, ...);
+int hip_check(hipError_t code, const char* operation);
+
+// Each kernel file exports one factory per symbol: fills `f` from the variant or returns an
+// error code after set_error().
+typedef int (*Factory)(const Variant&, orx_function* f);
+struct Registration {
+    const char* symbol;
+    Factory factory;
+    const char* variant_keys;  // human-readable list for orx_catalog()
+    const char* arguments;     // launch order, comma separated
+};
+
+// Implemented by the kernel translation units (host functions, so the tables never reach device code).
+const Registration* quant_registrations(int* count);
+const Registration* gemv_registrations(int* count);
+const Registration* gemm_registrations(int* count);
+const Registration* moe_registrations(int* count);
+
+template <typename T>
+static inline T* pointer_arg(void** args, int index) {
+    return *reinterpret_cast<T**>(args[index]);
+}
+static inline int int_arg(void** args, int index) { return *reinterpret_cast<int32_t*>(args[index]); }
+
+static inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+}  // namespace orx

@@ -1,0 +1,366 @@
+"""GPU parity: decode, A8 and the dense Q4A8 / W8A8 projections against the CPU oracle.
+
+Integer results (decoded weights, int8 activations, int32 accumulators) must be bit-exact.
+fp16/fp32 outputs are produced by the same two fp32 multiplies as the oracle, so they are
+compared for equality as well; the contract tolerance (1e-3 relative / 1e-2 absolute) is
+asserted separately so a reader sees the stated bar.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import reference as orc
+from orinfer_amd import codebook, workloads
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+TABLE = orc.basis()
+RTOL, ATOL = 1e-3, 1e-2  # fp16 output tolerance stated by the benchmark contract
+
+
+def assert_close_fp16(got, want):
+    got = np.asarray(got, np.float32)
+    want = np.asarray(want, np.float32)
+    assert np.isfinite(got).all()
+    assert (np.abs(got - want) <= ATOL + RTOL * np.abs(want)).all()
+
+
+def exhaustive_q4():
+    first = np.arange(65536, dtype=np.uint32).reshape(4096, 16)
+    second = (first * np.uint32(32771) + np.uint32(97)) & np.uint32(65535)
+    return first | (second << np.uint32(16))
+
+
+# ---- decode ---------------------------------------------------------------
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
+def test_q4_unpack_every_code(packed_k):
+    packed = exhaustive_q4()  # every coarse code once, residual by an LCG (test_e8p_q4.py:13-30)
+    want = orc.q4_integers(packed, TABLE)
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
+    out = torch.zeros((4096, 128), dtype=torch.int8, device=gu.DEV)
+    gu.kernel("e8p_q4_unpack", N=4096, K=128, packed_k=packed_k)(Book=gu.book(), Output=out, W=gu.dev(stored))
+    np.testing.assert_array_equal(gu.host(out), want)
+
+
+def test_q4_unpack_residual_every_code():
+    # swap the halves so that every code also appears as the residual stage
+    packed = exhaustive_q4()
+    swapped = (packed >> np.uint32(16)) | (packed << np.uint32(16))
+    out = torch.zeros((4096, 128), dtype=torch.int8, device=gu.DEV)
+    gu.kernel("e8p_q4_unpack", N=4096, K=128)(Book=gu.book(), Output=out, W=gu.dev(swapped))
+    np.testing.assert_array_equal(gu.host(out), orc.q4_integers(swapped, TABLE))
+
+
+def test_q2_unpack_every_code():
+    codes = np.arange(65536, dtype=np.uint16).reshape(4096, 16)
+    out = torch.zeros((4096, 128), dtype=torch.int8, device=gu.DEV)
+    gu.kernel("e8p_q2_unpack", N=4096, K=128)(Book=gu.book(), Output=out, W=gu.dev(codes))
+    np.testing.assert_array_equal(gu.host(out), orc.q2_integers(codes, TABLE))
+    k128 = orc.q2_pack_k128(codes)
+    out.zero_()
+    gu.kernel("e8p_q2_unpack", N=4096, K=128, packed_k=128)(Book=gu.book(), Output=out, W=gu.dev(k128))
+    np.testing.assert_array_equal(gu.host(out), orc.q2_integers(codes, TABLE))
+
+
+# ---- A8 -------------------------------------------------------------------
+def test_a8_edges_and_random():
+    rng = np.random.default_rng(orc.SEED)
+    x = rng.normal(size=(67, 2560)).astype(np.float16)
+    x[0] = 0
+    x[1, :8] = [127, -127, 63.5, 0.5, 1.5, 2.5, -0.5, -2.5]
+    x[1, 8:] = 0
+    x[2] = 0
+    x[2, 5] = 1e-7
+    x[3, :8] = [254, 1, -1, 3, -3, 5, 127, -254]
+    x[3, 8:] = 0
+    x[4, 0] = 65504
+    x[5] *= 20
+    q, s = gu.a8(gu.dev(x))
+    wq, ws = orc.a8(x)
+    np.testing.assert_array_equal(gu.host(s), ws)
+    np.testing.assert_array_equal(gu.host(q), wq)
+
+
+@pytest.mark.parametrize("k,group", [(2560, 64), (384, 128), (100, 25), (7, 7)])
+def test_a8_groups_and_odd_shapes(k, group):
+    rng = np.random.default_rng(orc.SEED + k)
+    x = (rng.normal(size=(5, k)) * 3).astype(np.float16)
+    q, s = gu.a8(gu.dev(x), group=group)
+    wq, ws = orc.a8(x, group)
+    np.testing.assert_array_equal(gu.host(s), ws)
+    np.testing.assert_array_equal(gu.host(q), wq)
+
+
+def test_a8_masked_columns():
+    rng = np.random.default_rng(orc.SEED)
+    x = rng.normal(size=(9, 512)).astype(np.float16)
+    mask = (rng.uniform(size=512) < 0.1).astype(np.uint8)
+    x[:, 3] = 1000  # would dominate amax if the mask were ignored
+    mask[3] = 7
+    q, s = gu.a8(gu.dev(x), masked=gu.dev(mask))
+    xm = x.copy()
+    xm[:, mask != 0] = 0
+    wq, ws = orc.a8(xm)
+    np.testing.assert_array_equal(gu.host(s), ws)
+    np.testing.assert_array_equal(gu.host(q), wq)
+
+
+def test_swiglu_then_a8_and_fused_form_agree():
+    rng = np.random.default_rng(orc.SEED)
+    gu_in = (rng.normal(size=(33, 2 * 512)) * 2).astype(np.float16)
+    x = gu.dev(gu_in)
+    y = torch.empty((33, 512), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("swiglu", I=512)(X=x, Y=y, rows=33)
+    want = orc.swiglu_fp16(gu_in)
+    got = gu.host(y)
+    # exp() differs by an ulp between libraries: tolerance on the fp16 boundary value
+    np.testing.assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=1e-6)
+    assert (got == want).mean() > 0.99
+    q1, s1 = gu.a8(y)
+    wq, ws = orc.a8(got)  # the quantiser itself must be exact on the GPU's own fp16 values
+    np.testing.assert_array_equal(gu.host(q1), wq)
+    np.testing.assert_array_equal(gu.host(s1), ws)
+    q2, s2 = gu.a8(x, fused=True)
+    assert torch.equal(q1, q2) and torch.equal(s1, s2)
+
+
+# ---- Q4A8 projections -----------------------------------------------------
+def q4_case(rng, m, n, k):
+    x = (rng.normal(size=(m, k))).astype(np.float16)
+    a_q, a_s = orc.a8(x)
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    return a_q, a_s[:, 0].copy(), packed, scales
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("n,k", [(65, 256), (257, 2560), (1024, 5120)])
+def test_q4_gemv_matches_oracle(m, n, k):
+    rng = np.random.default_rng(orc.SEED + m + n)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :4] = [-128, -1, 0, 127]  # extremes outside the A8 range must still be exact
+    w = orc.q4_integers(packed, TABLE)
+    acc = orc.int_dot(a_q, w)
+    ones_n, ones_m = np.ones(n, np.float16), np.ones(m, np.float16)
+    got_acc = gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(packed), gu.dev(ones_n), dtype=torch.float32,
+                            algorithm="gemv")
+    np.testing.assert_array_equal(gu.host(got_acc).astype(np.int64), acc.astype(np.int64))
+    got = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), algorithm="gemv")
+    want = orc.rescale(acc, scales, a_s)
+    assert_close_fp16(gu.host(got), want)
+    np.testing.assert_array_equal(gu.host(got), want)
+
+
+@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("m", [1, 7, 32, 33, 64, 65, 128, 129, 300])
+def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
+    # check_e8p_q4.py:123-193: N=65, K=256, fp32 out, stride N+3, sentinel 91 beyond the tails
+    rng = np.random.default_rng(orc.SEED + m)
+    n, k = 65, 256
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
+                  dtype=torch.float32, algorithm="mfma", packed_k=packed_k)
+    got = gu.host(storage)
+    want = orc.project(a_q, a_s, orc.q4_integers(packed, TABLE), scales, np.float32)
+    np.testing.assert_array_equal(got[:m, :n], want)
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+
+
+@pytest.mark.parametrize("block_m", [32, 64, 128])
+def test_q4_mfma_tiles_and_accumulators(block_m):
+    rng = np.random.default_rng(orc.SEED + block_m)
+    m, n, k = 200, 384, 1024
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    acc = orc.int_dot(a_q, orc.q4_integers(packed, TABLE))
+    got = gu.q4_project(gu.dev(a_q), gu.dev(np.ones(m, np.float16)), gu.dev(packed), gu.dev(np.ones(n, np.float16)),
+                        dtype=torch.float32, algorithm="mfma", block_m=block_m)
+    np.testing.assert_array_equal(gu.host(got).astype(np.int64), acc.astype(np.int64))
+    got16 = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), algorithm="mfma", block_m=block_m)
+    np.testing.assert_array_equal(gu.host(got16), orc.rescale(acc, scales, a_s))
+
+
+def test_q4_dynamic_rows_one_handle_many_lengths():
+    rng = np.random.default_rng(orc.SEED)
+    n, k, cap = 257, 640 + 128, 128
+    _, _, packed, scales = q4_case(rng, 1, n, k)
+    w = orc.q4_integers(packed, TABLE)
+    for m in (1, 2, 4, 5, 31, 64, 127, 128):
+        x = rng.normal(size=(m, k)).astype(np.float16)
+        a_q, a_s = orc.a8(x)
+        out = torch.full((cap + 1, n), 7.0, dtype=torch.float16, device=gu.DEV)
+        gu.q4_project(gu.dev(a_q), gu.dev(a_s[:, 0].copy()), gu.dev(packed), gu.dev(scales), dynamic=True,
+                      capacity=cap, out=out)
+        got = gu.host(out)
+        np.testing.assert_array_equal(got[:m], orc.project(a_q, a_s[:, 0], w, scales))
+        assert (got[m:] == 7).all()
+
+
+# ---- W8A8 -----------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k", [(1, 48, 2560), (3, 65, 128), (17, 129, 640)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("algorithm", ["auto", "mfma"])
+def test_w8_power_of_two_scales_exact(m, n, k, dtype, algorithm):
+    # tests/cuda/operators/int8_projection.py:25-41
+    rng = np.random.default_rng(orc.SEED + m)
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    ws = np.full(n, 0.015625, np.float16)
+    ts = np.full(m, 0.0078125, np.float16)
+    out = torch.full((m + 1, n), 99.0, dtype=dtype, device=gu.DEV)
+    gu.w8_project(gu.dev(x), gu.dev(ts), gu.dev(w), gu.dev(ws), out=out, dtype=dtype, algorithm=algorithm)
+    want = orc.project(x, ts, w, ws, np.float32 if dtype == torch.float32 else np.float16)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:m], want)
+    assert (got[m] == 99).all()
+
+
+@pytest.mark.parametrize("m", [1, 3, 17, 63, 65, 129, 511])
+def test_w8_dynamic_capacity_stride_extremes(m):
+    # int8_projection.py:125-193: capacity 512, N=257, stride 272, forced extremes, ws[0]=0
+    rng = np.random.default_rng(orc.SEED + m)
+    n, k, stride = 257, 640, 272
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    x[:, :4] = [-128, -1, 0, 127]
+    ws = (rng.uniform(size=n) * 0.003).astype(np.float16)
+    ts = (rng.uniform(size=m) * 0.005).astype(np.float16)
+    ws[0] = 0
+    storage = torch.full((m + 2, stride), 99.0, dtype=torch.float16, device=gu.DEV)
+    gu.w8_project(gu.dev(x), gu.dev(ts), gu.dev(w), gu.dev(ws), dynamic=True, capacity=512, out=storage, stride=stride)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(x, ts, w, ws))
+    assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
+
+
+def test_w8_mid_size_accumulators():
+    rng = np.random.default_rng(orc.SEED)
+    m, n, k = 384, 512, 4096
+    x = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    got = gu.w8_project(gu.dev(x), gu.dev(np.ones(m, np.float16)), gu.dev(w), gu.dev(np.ones(n, np.float16)),
+                        dtype=torch.float32)
+    acc = orc.int_dot(x, w)
+    assert np.abs(acc).max() < 2**24
+    np.testing.assert_array_equal(gu.host(got).astype(np.int64), acc.astype(np.int64))
+
+
+# ---- launch contract -------------------------------------------------------
+def test_graph_capture_replays_with_changed_contents():
+    # Every reference operator test captures once and replays after mutating inputs in place.
+    rng = np.random.default_rng(orc.SEED)
+    m, n, k = 3, 129, 512
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    ta, ts_, tw, tsc = gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales)
+    book = gu.book()
+    out = torch.empty((m, n), dtype=torch.float16, device=gu.DEV)
+    for algorithm in ("gemv", "mfma"):
+        kern = gu.kernel("e8p_q4_projection", M=m, N=n, K=k, algorithm=algorithm)
+        args = dict(A=ta, AS=ts_, Book=book, Out=out, S=tsc, W=tw)
+        kern(**args)  # warm-up outside capture
+        gu.sync()
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                kern(stream=stream.cuda_stream, **args)
+        w = orc.q4_integers(packed, TABLE)
+        for step in range(3):
+            out.fill_(float("nan"))
+            graph.replay()
+            gu.sync()
+            np.testing.assert_array_equal(gu.host(out), orc.project(gu.host(ta), gu.host(ts_), w, gu.host(tsc)))
+            ta.copy_(gu.dev(rng.integers(-127, 128, (m, k), dtype=np.int8)))  # new contents, same addresses
+            tsc.mul_(1.5)
+        ta.zero_()
+        graph.replay()
+        gu.sync()
+        assert bool((out == 0).all())  # zero-input replay (backend/cuda/mod.rs:649-678)
+        ta.copy_(gu.dev(a_q))
+        tsc.copy_(gu.dev(scales))
+
+
+def test_launch_rejects_bad_geometry_rows_and_alignment():
+    from orinfer_amd import lib
+
+    kern = gu.kernel("e8p_q4_projection", M=8, N=128, K=256, dynamic_rows=True)
+    a = torch.zeros((8, 256), dtype=torch.int8, device=gu.DEV)
+    s = torch.ones(8, dtype=torch.float16, device=gu.DEV)
+    w = torch.zeros((128, 32), dtype=torch.int32, device=gu.DEV)
+    ws = torch.ones(128, dtype=torch.float16, device=gu.DEV)
+    out = torch.zeros((8, 128), dtype=torch.float16, device=gu.DEV)
+    values = [a, s, gu.book(), out, ws, w, 8]
+    grid, block, shared = kern.geometry(8)
+    stream = torch.cuda.current_stream().cuda_stream
+    with pytest.raises(lib.OrxError) as e:
+        kern.launch_raw((grid[0] + 1, 1, 1), block, shared, stream, values)
+    assert e.value.code == lib.ORX_ERR_BAD_GEOMETRY
+    with pytest.raises(lib.OrxError) as e:
+        kern.launch_raw(grid, block, shared, stream, values[:-1] + [9])
+    assert e.value.code == lib.ORX_ERR_ROWS
+    with pytest.raises(lib.OrxError) as e:
+        kern.launch_raw(grid, block, shared, stream, [a.data_ptr() + 1] + values[1:])
+    assert e.value.code == lib.ORX_ERR_BAD_ARGUMENT
+    kern.launch_raw(grid, block, shared, stream, values)
+    gu.sync()
+
+
+# ---- benchmark configurations at full size ---------------------------------
+def test_config0_full_size_bit_exact():
+    c = workloads.config0()
+    x = gu.dev(c["x"])
+    a_q, a_s = gu.a8(x)
+    wq, ws = orc.a8(c["x"])
+    np.testing.assert_array_equal(gu.host(a_q), wq)
+    np.testing.assert_array_equal(gu.host(a_s), ws)
+    out = gu.q4_project(a_q, a_s, gu.dev(c["packed"]), gu.dev(c["scales"]))
+    w = orc.q4_integers(c["packed"], TABLE)
+    want = orc.project(wq, ws[:, 0], w, c["scales"])
+    assert_close_fp16(gu.host(out), want)
+    np.testing.assert_array_equal(gu.host(out), want)
+
+
+@pytest.mark.parametrize("rows", [1, 8, 32, 128, 512])
+def test_config1_full_size_bit_exact(rows):
+    c = workloads.config1(rows)
+    a_q, a_s = gu.a8(gu.dev(c["x"]))
+    wq, ws = orc.a8(c["x"])
+    np.testing.assert_array_equal(gu.host(a_q), wq)
+    out = gu.q4_project(a_q, a_s, gu.dev(c["packed"]), gu.dev(c["scales"]))
+    w = _config1_weights(c)
+    want = orc.project(wq, ws[:, 0], w, c["scales"])
+    assert_close_fp16(gu.host(out), want)
+    np.testing.assert_array_equal(gu.host(out), want)
+
+
+_weights_cache = {}
+
+
+def _config1_weights(c):
+    if "w" not in _weights_cache:
+        _weights_cache["w"] = orc.q4_integers(c["packed"], TABLE)
+    return _weights_cache["w"]
+
+
+def test_config2_full_size_sampled_rows_and_linearity():
+    c = workloads.config2()
+    a_q, a_s = gu.a8(gu.dev(c["x"]))
+    out = gu.w8_project(a_q, a_s, gu.dev(c["weight"]), gu.dev(c["scales"]))
+    rows = np.random.default_rng(0).choice(c["rows"], 96, replace=False)
+    wq, ws = orc.a8(c["x"][rows])
+    np.testing.assert_array_equal(gu.host(a_q)[rows], wq)
+    want = orc.project(wq, ws[:, 0], c["weight"], c["scales"])
+    np.testing.assert_array_equal(gu.host(out)[rows], want)
+    # size-independent property on ALL rows: the int32 accumulators are linear in the activations,
+    # so acc(a) + acc(-a) == 0 and acc(a) with unit scales summed over N equals a . colsum(W)
+    ones_m = torch.ones(c["rows"], dtype=torch.float16, device=gu.DEV)
+    ones_n = torch.ones(c["n"], dtype=torch.float16, device=gu.DEV)
+    acc = gu.w8_project(a_q, ones_m, gu.dev(c["weight"]), ones_n, dtype=torch.float32)
+    neg = gu.w8_project(-a_q, ones_m, gu.dev(c["weight"]), ones_n, dtype=torch.float32)
+    assert bool((acc + neg == 0).all())
+    colsum = c["weight"].astype(np.int64).sum(0)
+    checksum = gu.host(a_q).astype(np.int64) @ colsum
+    np.testing.assert_array_equal(gu.host(acc.double().sum(1)).astype(np.int64), checksum)
