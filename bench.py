@@ -1,0 +1,274 @@
+"""Benchmark of the quantized linear-layer path on one MI355X.
+
+Contract line (one JSON object on stdout): metric = Q4A8 GEMV achieved HBM GB/s on
+BASELINE configuration 1 at M=1 (K=5120, N=17408), one step = A8 quantisation of the token row
+plus the E8P-Q4 projection, weights rotating over enough distinct copies that they cannot stay
+in the 256 MB Infinity Cache.  `roofline` prices the projection kernel alone against 8 TB/s;
+`extra` carries the other configurations (GEMV config 0, the M sweep, W8A8 and layer GEMM TOPS
+against the int8 MFMA peak, the MoE layer).  `cpu_baseline` times the numpy oracle on the same
+workload on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA (5.0 POP/s)
+CACHE_BYTES = 256 << 20        # Infinity Cache
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=240)
+    p.add_argument("--warmup", type=int, default=24)
+    p.add_argument("--no-extra", action="store_true", help="only the contract workload")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    return p.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    from orinfer_amd import codebook, lib, workloads
+    from orinfer_amd.lib import Kernel
+
+    lib.library()
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream()
+
+    def dev(a):
+        a = np.ascontiguousarray(a)
+        view = {np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32}.get(a.dtype)
+        return torch.from_numpy(a.view(view) if view else a).cuda()
+
+    def timed_graph(enqueue, launches, replays=3):
+        """Captures `launches` calls of enqueue(i) in one graph; returns best seconds per launch."""
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            enqueue(0, side.cuda_stream)  # warm-up outside capture (first-launch setup)
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(launches):
+                    enqueue(i, side.cuda_stream)
+        best = float("inf")
+        for _ in range(replays + 1):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record()
+            graph.replay()
+            stop.record()
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(stop) * 1e-3 / launches)
+        return best
+
+    book = dev(codebook.book())
+
+    class Q4Case:
+        """One Q4A8 linear at (rows, n, k) with `copies` distinct weight tensors."""
+
+        def __init__(self, case, copies, algorithm="auto"):
+            self.rows, self.n, self.k = case["rows"], case["n"], case["k"]
+            rng = np.random.default_rng(7)
+            self.weights = [dev(case["packed"])]
+            for _ in range(copies - 1):  # same shape and statistics, different bits
+                self.weights.append(dev(rng.integers(0, 2**32, case["packed"].shape, dtype=np.uint32)))
+            self.scales = dev(case["scales"])
+            self.x = dev(case["x"])
+            self.a_q = torch.empty((self.rows, self.k), dtype=torch.int8, device="cuda")
+            self.a_s = torch.empty((self.rows, 1), dtype=torch.float16, device="cuda")
+            self.out = torch.empty((self.rows, self.n), dtype=torch.float16, device="cuda")
+            self.quant = Kernel("activation_quantization", K=self.k)
+            self.proj = Kernel("e8p_q4_projection", M=self.rows, N=self.n, K=self.k, algorithm=algorithm)
+
+        def quantize(self, s):
+            self.quant(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=self.x, rows=self.rows)
+
+        def project(self, i, s):
+            self.proj(stream=s, A=self.a_q, AS=self.a_s, Book=book, Out=self.out, S=self.scales,
+                      W=self.weights[i % len(self.weights)])
+
+        def step(self, i, s):
+            self.quantize(s)
+            self.project(i, s)
+
+    # ---- contract workload: config 1, M=1 ----
+    c1 = workloads.config1(1)
+    bytes_c1 = workloads.algorithmic_bytes_q4(1, c1["n"], c1["k"])
+    copies = -(-2 * CACHE_BYTES // (c1["n"] * c1["k"] // 2))  # aggregate footprint >= 2x the cache
+    main_case = Q4Case(c1, copies)
+    for i in range(args.warmup):
+        main_case.step(i, stream.cuda_stream)
+    torch.cuda.synchronize()
+    # exactly K steps, bracketed by synchronize on both sides, replayed as one graph
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(args.steps):
+                main_case.step(i, side.cuda_stream)
+    graph.replay()  # graph upload
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    step_seconds = (time.perf_counter() - t0) / args.steps
+    kernel_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(args.steps, copies))
+    main_case.quantize(stream.cuda_stream)
+    achieved = bytes_c1 / kernel_seconds / 1e9
+    result = {
+        "metric": "Q4A8 GEMV HBM GB/s (% of peak) + GEMM int8 TOPS (% MFMA peak), 1 GPU",
+        "value": round(bytes_c1 / step_seconds / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_seconds * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 x int8 -> int32 (u16 E8P codes), fp16 rescale",
+        "data": "synthetic (seeded uniform codes, N(0,1) activations, random-init scales)",
+        "config": {"workload": "BASELINE config 1: Q4A8 linear K=5120 N=17408, M=1 decode GEMV, step = A8 + projection",
+                   "weight_copies_rotated": copies, "algorithmic_bytes_per_step": bytes_c1},
+        "roofline": {"bound": "hbm", "kernel": "gemv_rowmajor_kernel<Q4,1>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": MEASURED_TRAFFIC_BYTES},
+    }
+
+    extra = {}
+    if not args.no_extra:
+        # config 0 GEMV
+        c0 = workloads.config0()
+        b0 = workloads.algorithmic_bytes_q4(1, c0["n"], c0["k"])
+        case0 = Q4Case(c0, -(-2 * CACHE_BYTES // (c0["n"] * c0["k"] // 2)))
+        t = timed_graph(lambda i, s: case0.project(i, s), 480)
+        extra["config0_q4a8_gemv_m1"] = {"us": round(t * 1e6, 3), "GBps": round(b0 / t / 1e9, 1),
+                                         "frac_hbm": round(b0 / t / 1e9 / HBM_PEAK_GBS, 4), "bytes": b0}
+        del case0
+        # config 1 sweep
+        sweep = {}
+        for rows in (1, 8, 32, 128, 512):
+            case = Q4Case(workloads.config1(rows), copies)
+            t = timed_graph(lambda i, s: case.project(i, s), 2 * copies)
+            b = workloads.algorithmic_bytes_q4(rows, case.n, case.k)
+            ops = workloads.algorithmic_ops(rows, case.n, case.k)
+            sweep[str(rows)] = {"us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
+                                "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4), "TOPS": round(ops / t / 1e12, 2),
+                                "frac_int8": round(ops / t / 1e12 / INT8_PEAK_TOPS, 4)}
+            del case
+        extra["config1_q4a8_sweep"] = sweep
+        del main_case
+        torch.cuda.empty_cache()
+        # config 2 W8A8
+        c2 = workloads.config2()
+        x2 = dev(c2["x"])
+        a2 = torch.empty((c2["rows"], c2["k"]), dtype=torch.int8, device="cuda")
+        s2 = torch.empty((c2["rows"], 1), dtype=torch.float16, device="cuda")
+        o2 = torch.empty((c2["rows"], c2["n"]), dtype=torch.float16, device="cuda")
+        w2, ws2 = dev(c2["weight"]), dev(c2["scales"])
+        quant2 = Kernel("activation_quantization", K=c2["k"])
+        proj2 = Kernel("int8_projection", M=c2["rows"], N=c2["n"], K=c2["k"])
+        quant2(Mask=None, Q=a2, S=s2, X=x2, rows=c2["rows"])
+        t = timed_graph(lambda i, s: proj2(stream=s, A=a2, Output=o2, TokenScale=s2, Weight=w2, WeightScale=ws2), 20)
+        tq = timed_graph(lambda i, s: quant2(stream=s, Mask=None, Q=a2, S=s2, X=x2, rows=c2["rows"]), 20)
+        ops = workloads.algorithmic_ops(c2["rows"], c2["n"], c2["k"])
+        extra["config2_w8a8_gemm"] = {"us": round(t * 1e6, 2), "TOPS": round(ops / t / 1e12, 1),
+                                      "frac_int8": round(ops / t / 1e12 / INT8_PEAK_TOPS, 4),
+                                      "a8_us": round(tq * 1e6, 2)}
+        del x2, a2, s2, o2, w2
+        torch.cuda.empty_cache()
+        # config 3 MoE layer
+        from orinfer_amd import programs
+
+        c3 = workloads.config3()
+        layer = programs.MoeLayer(c3["tokens"], c3["experts"], c3["top_k"], c3["hidden"], c3["intermediate"],
+                                  c3["gate_up"], c3["gate_up_scales"], c3["down"], c3["down_scales"], block_m=32)
+        x3, l3 = dev(c3["x"]), dev(c3["logits"])
+        t = timed_graph(lambda i, s: layer.run(x3, l3, stream=s), 20)
+        counts = layer.counts.cpu().numpy()
+        touched = int((counts > 0).sum())
+        code_bytes = touched * (c3["hidden"] * 2 * c3["intermediate"] + c3["intermediate"] * c3["hidden"]) // 4
+        extra["config3_moe_q2a8_layer"] = {"us": round(t * 1e6, 2), "experts_touched": touched,
+                                           "code_bytes_touched": code_bytes,
+                                           "GBps_codes": round(code_bytes / t / 1e9, 1)}
+        del layer
+        torch.cuda.empty_cache()
+        # config 4 layer linears
+        c4 = workloads.config4()
+        layer_us, per = 0.0, {}
+        for name, spec in c4.items():
+            rows, n, k = spec["rows"], spec["n"], spec["k"]
+            x = dev(spec["x"])
+            a = torch.empty((rows, k), dtype=torch.int8, device="cuda")
+            sc = torch.empty((rows, 1), dtype=torch.float16, device="cuda")
+            o = torch.empty((rows, n), dtype=torch.float16, device="cuda")
+            ws = dev(spec["scales"])
+            quant = Kernel("activation_quantization", K=k)
+            if spec["codec"] == "q4":
+                w = dev(spec["packed"])
+                proj = Kernel("e8p_q4_projection", M=rows, N=n, K=k)
+                run = lambda i, s: proj(stream=s, A=a, AS=sc, Book=book, Out=o, S=ws, W=w)
+            else:
+                w = dev(spec["weight"])
+                proj = Kernel("int8_projection", M=rows, N=n, K=k)
+                run = lambda i, s: proj(stream=s, A=a, Output=o, TokenScale=sc, Weight=w, WeightScale=ws)
+            tq = timed_graph(lambda i, s: quant(stream=s, Mask=None, Q=a, S=sc, X=x, rows=rows), 5)
+            tp = timed_graph(run, 5)
+            ops = workloads.algorithmic_ops(rows, n, k)
+            per[name] = {"codec": spec["codec"], "a8_us": round(tq * 1e6, 1), "gemm_us": round(tp * 1e6, 1),
+                         "TOPS": round(ops / tp / 1e12, 1), "frac_int8": round(ops / tp / 1e12 / INT8_PEAK_TOPS, 4)}
+            layer_us += (tq + tp) * 1e6
+            del x, a, o, w
+            torch.cuda.empty_cache()
+        extra["config4_layer_linears_m8192"] = {"layer_us": round(layer_us, 1), "per_gemm": per}
+    result["extra"] = extra
+
+    # ---- CPU baseline: the numpy oracle on the contract workload (one full call) ----
+    if not args.no_cpu:
+        from oracle import reference as orc
+
+        try:
+            from threadpoolctl import threadpool_limits
+        except Exception:  # pragma: no cover
+            threadpool_limits = None
+        table = orc.basis()
+
+        def cpu_once():
+            a_q, a_s = orc.a8(c1["x"])
+            w = orc.q4_integers(c1["packed"], table)
+            return orc.project(a_q, a_s[:, 0], w, c1["scales"])
+
+        ctx = threadpool_limits(limits=1) if threadpool_limits else None
+        t0 = time.perf_counter()
+        cpu_once()
+        cpu_seconds = time.perf_counter() - t0
+        if ctx is not None:
+            ctx.unregister() if hasattr(ctx, "unregister") else None
+        result["cpu_baseline"] = {
+            "value": round(bytes_c1 / cpu_seconds / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "seconds_per_call": round(cpu_seconds, 3), "host_cpus": os.cpu_count(),
+            "sample": "one full call of the numpy oracle on config 1, M=1 (decode 11.1M two-stage codes, "
+                      "fp64 dot, rescale), single thread",
+        }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

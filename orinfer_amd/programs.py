@@ -1,0 +1,144 @@
+"""Kernel programs: ordered launch lists for one quantized linear and for one MoE expert layer.
+
+The engine runs a *program* -- an ordered list of kernel records whose buffers it owns
+(crates/orinfer-engine/src/backend/cuda/executor.rs:1095-1124).  These classes are that list for
+the paths of this library, with every buffer allocated once up front (torch is used only for
+device memory and the stream), so `run()` only enqueues and can be captured in a graph.
+Program order of the expert layer follows python/orinfer_build/models/flash_next (router top-k,
+histogram, offsets, tiles, A8, dispatch, grouped gate_up, SwiGLU->A8, grouped down, combine).
+"""
+import numpy as np
+import torch
+
+from . import codebook
+from .lib import Kernel
+
+
+def _dev(array):
+    a = np.ascontiguousarray(array)
+    view = {np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32}.get(a.dtype)
+    return torch.from_numpy(a.view(view) if view else a).cuda()
+
+
+class QuantizedLinear:
+    """A8 quantiser + one projection (E8P-Q4 or W8A8) with a dynamic row count up to `capacity`."""
+
+    def __init__(self, codec, weight, scales, capacity, *, packed_k=0, algorithm="auto", block_m=0, book=None):
+        if codec not in ("q4", "w8"):
+            raise ValueError("codec must be q4 or w8")
+        self.codec, self.capacity = codec, capacity
+        scales = np.asarray(scales)
+        self.n = scales.shape[0]
+        weight = np.asarray(weight)
+        if codec == "q4":
+            self.k = weight.shape[1] * 8
+            stored = codebook.q4_to_k_major(weight, 128) if packed_k == 128 else weight
+        else:
+            self.k = weight.shape[1]
+            stored = weight
+        self.weight = _dev(stored)
+        self.scales = _dev(scales)
+        self.book = _dev(codebook.book() if book is None else book)
+        self.a_q = torch.empty((capacity, self.k), dtype=torch.int8, device="cuda")
+        self.a_s = torch.empty((capacity, 1), dtype=torch.float16, device="cuda")
+        self.out = torch.empty((capacity, self.n), dtype=torch.float16, device="cuda")
+        self.quantizer = Kernel("activation_quantization", K=self.k)
+        variant = dict(M=capacity, N=self.n, K=self.k, dynamic_rows=True, algorithm=algorithm)
+        if block_m:
+            variant["block_m"] = block_m
+        if codec == "q4":
+            if packed_k:
+                variant["packed_k"] = packed_k
+            self.projection = Kernel("e8p_q4_projection", **variant)
+        else:
+            self.projection = Kernel("int8_projection", **variant)
+
+    def quantize(self, x16, stream=None):
+        rows = x16.shape[0]
+        self.quantizer(stream=stream, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=rows)
+        return rows
+
+    def project(self, rows, stream=None):
+        if self.codec == "q4":
+            self.projection(stream=stream, A=self.a_q, AS=self.a_s, Book=self.book, Out=self.out, S=self.scales,
+                            W=self.weight, m=rows)
+        else:
+            self.projection(stream=stream, A=self.a_q, Output=self.out, TokenScale=self.a_s, Weight=self.weight,
+                            WeightScale=self.scales, m=rows)
+        return self.out[:rows]
+
+    def run(self, x16, stream=None):
+        return self.project(self.quantize(x16, stream), stream)
+
+
+class MoeLayer:
+    """Q2A8 expert layer: token-sort, grouped gate_up, SwiGLU->A8, grouped down, weighted combine."""
+
+    def __init__(self, tokens, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales,
+                 block_m=32, packed_k=128):
+        self.tokens, self.experts, self.top_k = tokens, experts, top_k
+        self.hidden, self.inter, self.block_m = hidden, intermediate, block_m
+        assignments = tokens * top_k
+        self.assignments = assignments
+        # capacity bound of the tile list (kernels/cuda/model/moe.py:263-264)
+        self.tile_capacity = (assignments + block_m - 1) // block_m + min(experts, assignments)
+        gate_up, down = np.asarray(gate_up), np.asarray(down)
+        if packed_k == 128:
+            gate_up, down = codebook.q2_to_k_major(gate_up), codebook.q2_to_k_major(down)
+        self.w1, self.w2 = _dev(gate_up), _dev(down)
+        self.s1, self.s2 = _dev(gate_up_scales), _dev(down_scales)
+        self.book = _dev(codebook.book())
+        i32 = dict(dtype=torch.int32, device="cuda")
+        f16 = dict(dtype=torch.float16, device="cuda")
+        i8 = dict(dtype=torch.int8, device="cuda")
+        self.ids = torch.empty((tokens, top_k), **i32)
+        self.prob = torch.empty((tokens, top_k), dtype=torch.float32, device="cuda")
+        self.counts = torch.empty(experts, **i32)
+        self.relative = torch.empty((tokens, top_k), **i32)
+        self.row_offsets = torch.empty(experts, **i32)
+        self.tile_offsets = torch.empty(experts, **i32)
+        self.tile_count = torch.empty(1, **i32)
+        self.tile_expert = torch.empty(self.tile_capacity, **i32)
+        self.tile_row = torch.empty(self.tile_capacity, **i32)
+        self.slot_map = torch.empty((tokens, top_k), **i32)
+        self.a_q = torch.empty((tokens, hidden), **i8)
+        self.a_s = torch.empty((tokens, 1), **f16)
+        self.d = torch.empty((assignments, hidden), **i8)
+        self.ds = torch.empty((assignments, 1), **f16)
+        self.gate_up_out = torch.empty((assignments, 2 * intermediate), **f16)
+        self.h_q = torch.empty((assignments, intermediate), **i8)
+        self.h_s = torch.empty((assignments, 1), **f16)
+        self.down_out = torch.empty((assignments, hidden), **f16)
+        self.out = torch.empty((tokens, hidden), **f16)
+        common = dict(M=tokens, E=experts, top_k=top_k)
+        self.k_router = Kernel("router_topk", renormalize=True, **common)
+        self.k_histogram = Kernel("expert_histogram", **common)
+        self.k_offsets = Kernel("expert_offsets", E=experts, block_m=block_m)
+        self.k_tiles = Kernel("expert_tiles", block_m=block_m, **common)
+        self.k_a8 = Kernel("activation_quantization", K=hidden)
+        self.k_dispatch = Kernel("expert_dispatch", H=hidden, **common)
+        grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k)
+        self.k_gate_up = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, **grouped)
+        self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
+        self.k_down = Kernel("e8p_decode_grouped", N=hidden, K=intermediate, **grouped)
+        self.k_combine = Kernel("moe_combine", H=hidden, slots=assignments, **common)
+
+    def run(self, x16, logits, stream=None):
+        s = stream
+        self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
+        self.k_histogram(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative)
+        self.k_offsets(stream=s, Counts=self.counts, RowOffsets=self.row_offsets, TileCount=self.tile_count,
+                       TileOffsets=self.tile_offsets)
+        self.k_tiles(stream=s, Counts=self.counts, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
+                     TileRow=self.tile_row)
+        self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=self.tokens)
+        self.k_dispatch(stream=s, A=self.a_q, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
+                        RowOffsets=self.row_offsets, Scale=self.a_s, SlotMap=self.slot_map)
+        routed = dict(Book=self.book, Counts=self.counts, Offsets=self.row_offsets, TileCount=self.tile_count,
+                      TileExpert=self.tile_expert, TileRow=self.tile_row)
+        self.k_gate_up(stream=s, A=self.d, AS=self.ds, C=self.gate_up_out, P=self.w1, WS=self.s1, **routed)
+        self.k_swiglu_a8(stream=s, Mask=None, Q=self.h_q, S=self.h_s, X=self.gate_up_out, rows=self.assignments)
+        self.k_down(stream=s, A=self.h_q, AS=self.h_s, C=self.down_out, P=self.w2, WS=self.s2, **routed)
+        self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
+                       SlotMap=self.slot_map)
+        return self.out
