@@ -36,18 +36,17 @@ __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }
 
-// LDS: nib[256] | msk[256] | sums[4] | planes.  For Q4/Q2 the planes are hi then lo nibble
-// words, MR x K/8 each; for W8 they are the raw int8 rows, MR x K bytes.
+// LDS: static nib[256], msk[256], sums[4]; dynamic activation planes.  For Q4/Q2 the planes are hi
+// then lo nibble words, MR x K/8 each; for W8 they are the raw int8 rows, MR x K bytes.
 template <int CODEC, int MR>
 __global__ __launch_bounds__(kThreads) void gemv_rowmajor_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
     int m, int passes, int out_f32) {
-    extern __shared__ __align__(16) uint32_t lds[];
-    uint32_t* nib = lds;
-    uint32_t* msk = lds + 256;
-    int* sums = reinterpret_cast<int*>(lds + 512);
-    uint32_t* planes = lds + 512 + 4;  // 16-byte aligned: (512+4)*4 = 2064
+    extern __shared__ __align__(16) uint32_t planes[];
+    __shared__ uint32_t nib[256];
+    __shared__ uint32_t msk[256];
+    __shared__ int sums[4];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int sub = lane & (kLanesPerRow - 1);  // which chunks of the row
@@ -57,109 +56,171 @@ __global__ __launch_bounds__(kThreads) void gemv_rowmajor_kernel(
     const int chunks = row_bytes / 16;
     const int groups = k / 8;
 
+    // Row owned by this lane group in the first pass; its first chunks are requested right after
+    // the small setup reads below (the memory counter retires in order, so the setup reads must
+    // be older than the bulk stream to be waited on alone) and land while the tables are built.
+    // Stream loads are never predicated:
+    // indices beyond the row are clamped to its last chunk (a cache hit) and simply not consumed,
+    // which keeps the loop free of divergent branches and lets the hardware counters track
+    // exactly which request each consume step waits for.
+    constexpr int D = 4;  // register ring of 16-byte chunks per lane
+    const int per_lane = (chunks - sub + kLanesPerRow - 1) / kLanesPerRow;       // chunks this lane owns
+    const int steps = (chunks + kLanesPerRow - 1) / kLanesPerRow;                // wave-uniform trip count
+    auto row_of = [&](int pass) {
+        return (blockIdx.x * passes + pass) * kRowsPerPass + wave * kRowsPerWave + row_in_wave;
+    };
+    auto fetch = [&](const uint4* src, int step) { return src[min(sub + step * kLanesPerRow, chunks - 1)]; };
+    uint4 ring[D];
+
     // ---- workgroup setup: tables, activation planes, activation sums ----
+    // Every global read of the setup is issued up front (selector word, activation groups, the
+    // row's scales) so that the kernel pays one memory latency, not one per dependent step.
+    const int first_row = row_of(0);
+    // raw bits now, conversion in the epilogue: a conversion here would wait for the load at once
+    // (unconditional, clamped indices: a conditional load would merge with a constant and be
+    // waited for at the merge)
+    const unsigned short ws_first = reinterpret_cast<const unsigned short*>(ws)[min(first_row, n - 1)];
+    unsigned short as_bits[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) as_bits[r] = reinterpret_cast<const unsigned short*>(as)[min(r, m - 1)];
+    const uint32_t selector = CODEC != kW8 ? book[tid & 255] : 0u;
     if (tid < 4) sums[tid] = 0;
-    if (CODEC != kW8) {
-        for (int i = tid; i < 256; i += kThreads) {
-            nib[i] = nibble_basis_word(book[i], 0u);
-            msk[i] = nibble_mask_word((uint32_t)i);
-        }
-    }
-    __syncthreads();
     if (CODEC != kW8) {
         uint32_t* hi = planes;
         uint32_t* lo = planes + MR * groups;
-        for (int r = 0; r < MR; ++r) {
-            int partial = 0;
-            for (int g = tid; g < groups; g += kThreads) {
-                uint2 raw = make_uint2(0u, 0u);
-                if (r < m) raw = *reinterpret_cast<const uint2*>(a + (int64_t)r * k + 8 * g);
-                // hi nibbles: coordinates 0..3 to even nibble slots, 4..7 to odd slots
-                hi[r * groups + g] = ((raw.x >> 4) & 0x0F0F0F0Fu) | (raw.y & 0xF0F0F0F0u);
-                lo[r * groups + g] = ((raw.x & 0x0F0F0F0Fu) | ((raw.y << 4) & 0xF0F0F0F0u)) ^ 0x88888888u;
-                partial = sdot4(raw.x, 0x01010101u, partial);
-                partial = sdot4(raw.y, 0x01010101u, partial);
+        constexpr int GR = 2;  // activation groups per thread per round
+        for (int g0 = 0; g0 < groups; g0 += GR * kThreads) {
+            uint2 raw[MR][GR];
+#pragma unroll
+            for (int r = 0; r < MR; ++r)
+#pragma unroll
+                for (int i = 0; i < GR; ++i) {
+                    const int g = g0 + i * kThreads + tid;
+                    raw[r][i] = (r < m && g < groups) ? *reinterpret_cast<const uint2*>(a + (int64_t)r * k + 8 * g)
+                                                     : make_uint2(0u, 0u);
+                }
+            if (g0 == 0) {  // bulk stream behind the setup reads, ahead of any wait
+                const uint4* src = w + (int64_t)(first_row < n ? first_row : 0) * chunks;
+#pragma unroll
+                for (int d = 0; d < D; ++d) ring[d] = fetch(src, d);
             }
-            if (partial != 0) atomicAdd(&sums[r], partial);
+            if (g0 == 0 && tid < 256) {  // table entries while the loads are in flight
+                nib[tid] = nibble_basis_word(selector, 0u);
+                msk[tid] = nibble_mask_word((uint32_t)tid);
+            }
+            if (g0 == 0) __syncthreads();  // sums[] is zero before the first add below
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                int partial = 0;
+#pragma unroll
+                for (int i = 0; i < GR; ++i) {
+                    const int g = g0 + i * kThreads + tid;
+                    const uint2 v = raw[r][i];
+                    if (g < groups) {
+                        // hi nibbles: coordinates 0..3 to even nibble slots, 4..7 to odd slots
+                        hi[r * groups + g] = ((v.x >> 4) & 0x0F0F0F0Fu) | (v.y & 0xF0F0F0F0u);
+                        lo[r * groups + g] = ((v.x & 0x0F0F0F0Fu) | ((v.y << 4) & 0xF0F0F0F0u)) ^ 0x88888888u;
+                    }
+                    partial = sdot4(v.x, 0x01010101u, partial);
+                    partial = sdot4(v.y, 0x01010101u, partial);
+                }
+#pragma unroll
+                for (int offset = 32; offset > 0; offset >>= 1) partial += __shfl_xor(partial, offset, 64);
+                if (lane == 0 && partial != 0) atomicAdd(&sums[r], partial);
+            }
         }
     } else {
+        {
+            const uint4* src = w + (int64_t)(first_row < n ? first_row : 0) * chunks;
+#pragma unroll
+            for (int d = 0; d < D; ++d) ring[d] = fetch(src, d);
+        }
         for (int r = 0; r < MR; ++r)
             for (int i = tid; i < k / 4; i += kThreads)
                 planes[r * (k / 4) + i] = r < m ? reinterpret_cast<const uint32_t*>(a + (int64_t)r * k)[i] : 0u;
     }
     __syncthreads();
 
-    for (int pass = 0; pass < passes; ++pass) {
-        const int row = (blockIdx.x * passes + pass) * kRowsPerPass + wave * kRowsPerWave + row_in_wave;
-        const bool live = row < n;
-        const uint4* src = w + (int64_t)(live ? row : 0) * chunks;
-        int acc_h0[MR], acc_l0[MR], acc_h1[MR], acc_l1[MR];
-        int acc_v0 = 0, acc_v1 = 0;
+    // One 16-byte chunk of the weight stream against every activation row.
+    int acc_h0[MR], acc_l0[MR], acc_h1[MR], acc_l1[MR];
+    int acc_v0, acc_v1;
+    auto consume = [&](const uint4& cur, int j) {
+        if (CODEC == kQ4) {
+            const uint32_t code[4] = {cur.x, cur.y, cur.z, cur.w};
+            uint4 ph[MR], pl[MR];
 #pragma unroll
-        for (int r = 0; r < MR; ++r) acc_h0[r] = acc_l0[r] = acc_h1[r] = acc_l1[r] = 0;
-
-        if (live) {
-            uint4 next = sub < chunks ? src[sub] : make_uint4(0, 0, 0, 0);
-            for (int j = sub; j < chunks; j += kLanesPerRow) {
-                const uint4 cur = next;
-                if (j + kLanesPerRow < chunks) next = src[j + kLanesPerRow];
-                if (CODEC == kQ4) {
-                    const uint32_t code[4] = {cur.x, cur.y, cur.z, cur.w};
-                    uint4 ph[MR], pl[MR];
+            for (int r = 0; r < MR; ++r) {
+                ph[r] = *reinterpret_cast<const uint4*>(planes + r * groups + 4 * j);
+                pl[r] = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 4 * j);
+            }
 #pragma unroll
-                    for (int r = 0; r < MR; ++r) {
-                        ph[r] = *reinterpret_cast<const uint4*>(planes + r * groups + 4 * j);
-                        pl[r] = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 4 * j);
-                    }
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t c = code[i];
+                const uint32_t v0 = nib[(c >> 8) & 255u] ^ msk[c & 255u];
+                const uint32_t v1 = nib[c >> 24] ^ msk[(c >> 16) & 255u];
+                acc_v0 = sdot8(v0, 0x11111111u, acc_v0);
+                acc_v1 = sdot8(v1, 0x11111111u, acc_v1);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t c = code[i];
-                        const uint32_t v0 = nib[(c >> 8) & 255u] ^ msk[c & 255u];
-                        const uint32_t v1 = nib[c >> 24] ^ msk[(c >> 16) & 255u];
-                        acc_v0 = sdot8(v0, 0x11111111u, acc_v0);
-                        acc_v1 = sdot8(v1, 0x11111111u, acc_v1);
+                for (int r = 0; r < MR; ++r) {
+                    const uint32_t h = reinterpret_cast<const uint32_t*>(&ph[r])[i];
+                    const uint32_t l = reinterpret_cast<const uint32_t*>(&pl[r])[i];
+                    acc_h0[r] = sdot8(v0, h, acc_h0[r]);
+                    acc_l0[r] = sdot8(v0, l, acc_l0[r]);
+                    acc_h1[r] = sdot8(v1, h, acc_h1[r]);
+                    acc_l1[r] = sdot8(v1, l, acc_l1[r]);
+                }
+            }
+        } else if (CODEC == kQ2) {
+            const uint32_t pair[4] = {cur.x, cur.y, cur.z, cur.w};
 #pragma unroll
-                        for (int r = 0; r < MR; ++r) {
-                            const uint32_t h = reinterpret_cast<const uint32_t*>(&ph[r])[i];
-                            const uint32_t l = reinterpret_cast<const uint32_t*>(&pl[r])[i];
-                            acc_h0[r] = sdot8(v0, h, acc_h0[r]);
-                            acc_l0[r] = sdot8(v0, l, acc_l0[r]);
-                            acc_h1[r] = sdot8(v1, h, acc_h1[r]);
-                            acc_l1[r] = sdot8(v1, l, acc_l1[r]);
-                        }
-                    }
-                } else if (CODEC == kQ2) {
-                    const uint32_t pair[4] = {cur.x, cur.y, cur.z, cur.w};
+            for (int half = 0; half < 2; ++half) {
+                uint4 ph[MR], pl[MR];
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        uint4 ph[MR], pl[MR];
+                for (int r = 0; r < MR; ++r) {
+                    ph[r] = *reinterpret_cast<const uint4*>(planes + r * groups + 8 * j + 4 * half);
+                    pl[r] = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 8 * j + 4 * half);
+                }
 #pragma unroll
-                        for (int r = 0; r < MR; ++r) {
-                            ph[r] = *reinterpret_cast<const uint4*>(planes + r * groups + 8 * j + 4 * half);
-                            pl[r] = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 8 * j + 4 * half);
-                        }
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const uint32_t c = (pair[2 * half + (i >> 1)] >> (16 * (i & 1))) & 0xFFFFu;
-                            const uint32_t v0 = nib[c >> 8] ^ msk[c & 255u];
-                            acc_v0 = sdot8(v0, 0x11111111u, acc_v0);
-#pragma unroll
-                            for (int r = 0; r < MR; ++r) {
-                                acc_h0[r] = sdot8(v0, reinterpret_cast<const uint32_t*>(&ph[r])[i], acc_h0[r]);
-                                acc_l0[r] = sdot8(v0, reinterpret_cast<const uint32_t*>(&pl[r])[i], acc_l0[r]);
-                            }
-                        }
-                    }
-                } else {
-                    const uint32_t word[4] = {cur.x, cur.y, cur.z, cur.w};
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t c = (pair[2 * half + (i >> 1)] >> (16 * (i & 1))) & 0xFFFFu;
+                    const uint32_t v0 = nib[c >> 8] ^ msk[c & 255u];
+                    acc_v0 = sdot8(v0, 0x11111111u, acc_v0);
 #pragma unroll
                     for (int r = 0; r < MR; ++r) {
-                        const uint4 act = *reinterpret_cast<const uint4*>(planes + r * (k / 4) + 4 * j);
-                        const uint32_t aw[4] = {act.x, act.y, act.z, act.w};
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) acc_h0[r] = sdot4(word[i], aw[i], acc_h0[r]);
+                        acc_h0[r] = sdot8(v0, reinterpret_cast<const uint32_t*>(&ph[r])[i], acc_h0[r]);
+                        acc_l0[r] = sdot8(v0, reinterpret_cast<const uint32_t*>(&pl[r])[i], acc_l0[r]);
                     }
                 }
+            }
+        } else {
+            const uint32_t word[4] = {cur.x, cur.y, cur.z, cur.w};
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                const uint4 act = *reinterpret_cast<const uint4*>(planes + r * (k / 4) + 4 * j);
+                const uint32_t aw[4] = {act.x, act.y, act.z, act.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc_h0[r] = sdot4(word[i], aw[i], acc_h0[r]);
+            }
+        }
+    };
+
+    for (int pass = 0; pass < passes; ++pass) {
+        const int row = row_of(pass);
+        const bool live = row < n;
+        const uint4* src = w + (int64_t)(live ? row : 0) * chunks;
+        acc_v0 = acc_v1 = 0;
+#pragma unroll
+        for (int r = 0; r < MR; ++r) acc_h0[r] = acc_l0[r] = acc_h1[r] = acc_l1[r] = 0;
+        if (pass > 0) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) ring[d] = fetch(src, d);
+        }
+        for (int base = 0; base < steps; base += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const uint4 cur = ring[d];
+                ring[d] = fetch(src, base + D + d);
+                if (base + d < per_lane) consume(cur, sub + (base + d) * kLanesPerRow);
             }
         }
 
@@ -178,7 +239,9 @@ __global__ __launch_bounds__(kThreads) void gemv_rowmajor_kernel(
             if (live && sub == 0 && r < m) {
                 if (CODEC == kQ4) total += 5 * sums[r];
                 if (CODEC == kQ2) total += sums[r];
-                const float value = rescale(total, __half2float(ws[row]), __half2float(as[r]));
+                const unsigned short ws_bits = pass == 0 ? ws_first : reinterpret_cast<const unsigned short*>(ws)[row];
+                const float value = rescale(total, __half2float(__ushort_as_half(ws_bits)),
+                                            __half2float(__ushort_as_half(as_bits[r])));
                 if (out_f32)
                     reinterpret_cast<float*>(out)[(int64_t)r * stride + row] = value;
                 else
@@ -204,7 +267,7 @@ int device_cus() {
 
 uint32_t gemv_lds_bytes(const orx_function& f, int mr) {
     const uint32_t planes = f.flags == kW8 ? (uint32_t)mr * f.K : (uint32_t)mr * (f.K / 8) * 8;
-    return (512 + 4) * 4 + planes;
+    return planes;
 }
 
 int mr_for(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : 4; }
@@ -270,13 +333,14 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
     f->flags = codec;
     int passes = passes_override;
     if (passes <= 0) {
-        // enough workgroups for ~1.2 per CU, but as few table rebuilds as that allows
-        passes = f->N / (kRowsPerPass * device_cus());
+        // one pass per workgroup keeps the most waves (and HBM requests) in flight; more passes
+        // only pay off when N is so large that table rebuilds dominate
+        passes = f->N / (kRowsPerPass * device_cus() * 16);
         if (passes < 1) passes = 1;
         if (passes > 8) passes = 8;
     }
     f->block_m = passes;
-    if (gemv_lds_bytes(*f, 4) > 160 * 1024) {
+    if (gemv_lds_bytes(*f, 4) > 160 * 1024 - 4096) {
         set_error("%s: K=%d does not fit the gemv activation planes in LDS", f->symbol.c_str(), f->K);
         return ORX_ERR_BAD_VARIANT;
     }
@@ -288,7 +352,7 @@ int gemv_prepare_device() {
     // Dynamic LDS above 64 KiB needs an opt-in per kernel (kernels.rs:171-190 does the same on CUDA).
     static bool done = false;
     if (done) return ORX_OK;
-    const int limit = 160 * 1024;
+    const int limit = 160 * 1024 - 4096;  // the static tables take 2064 bytes of the 160 KiB
 #define ORX_OPT_IN(kernel)                                                                                   \
     {                                                                                                        \
         int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel),                     \

@@ -42,6 +42,12 @@ def library():
             raise FileNotFoundError(
                 f"{LIBRARY_PATH} is missing: build it with `python -m orinfer_amd.build` (hipcc, gfx950)"
             )
+        try:
+            # liborx must bind to the HIP runtime torch has already loaded: two runtimes in one
+            # process do not share devices or streams
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         lib = ctypes.CDLL(str(LIBRARY_PATH))
         u32x3 = ctypes.POINTER(ctypes.c_uint32)
         lib.orx_resolve.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
