@@ -25,6 +25,11 @@ int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t 
 int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
 int gemv_configure(orx_function* f, int codec, int passes_override);
 int gemv_prepare_device();
+// from k_gemm_big.hip
+void gemm_big_geometry(int rows, int n, bool q4, Geometry* g);
+int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                    void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g,
+                    hipStream_t stream);
 
 namespace {
 
@@ -276,8 +281,15 @@ bool use_gemv(const orx_function& f, int rows) {
     return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
 }
 
+// 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
+bool use_big(const orx_function& f, int rows) { return f.tiles == 256 || (f.tiles == 0 && rows > 128); }
+
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
+    if (use_big(f, rows)) {
+        gemm_big_geometry(rows, f.N, f.flags == kQ4, g);
+        return ORX_OK;
+    }
     const int bm = f.tiles ? f.tiles : pick_bm(rows);
     g->grid[0] = ceil_div((uint32_t)f.N, 128u);
     g->grid[1] = ceil_div((uint32_t)rows, (uint32_t)bm);
@@ -297,6 +309,9 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, 5);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_big(f, rows))
+        return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
+                               f.out_f32, g, stream);
     return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
 
@@ -311,6 +326,9 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.book = nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = 0, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_big(f, rows))
+        return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
+                               stream);
     return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
 
@@ -345,8 +363,8 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         set_error("%s: packed_k must be 0 or 128 (codes only)", name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->tiles != 0 && f->tiles != 32 && f->tiles != 64 && f->tiles != 128) {
-        set_error("%s: block_m must be 32, 64 or 128", name);
+    if (f->tiles != 0 && f->tiles != 32 && f->tiles != 64 && f->tiles != 128 && f->tiles != 256) {
+        set_error("%s: block_m must be 32, 64, 128 or 256", name);
         return ORX_ERR_BAD_VARIANT;
     }
     f->out_f32 = dtype == "float32";
@@ -510,11 +528,11 @@ const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, packed_k=0|128, output_dtype=float16|float32, "
-     "output_stride=N, block_m=0|32|64|128, gemv_passes=0",
+     "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0",
      "A,AS,Book,Out,S,W[,m]"},
     {"int8_projection", make_w8_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, output_dtype=float16|float32, output_stride=N, "
-     "block_m=0|32|64|128",
+     "block_m=0|32|64|128|256",
      "A,Output,TokenScale,Weight,WeightScale[,m]"},
     {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},

@@ -170,10 +170,10 @@ def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
-@pytest.mark.parametrize("block_m", [32, 64, 128])
+@pytest.mark.parametrize("block_m", [32, 64, 128, 256])
 def test_q4_mfma_tiles_and_accumulators(block_m):
     rng = np.random.default_rng(orc.SEED + block_m)
-    m, n, k = 200, 384, 1024
+    m, n, k = 300, 384 + 65, 1024
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     acc = orc.int_dot(a_q, orc.q4_integers(packed, TABLE))
     got = gu.q4_project(gu.dev(a_q), gu.dev(np.ones(m, np.float16)), gu.dev(packed), gu.dev(np.ones(n, np.float16)),
@@ -236,9 +236,24 @@ def test_w8_dynamic_capacity_stride_extremes(m):
     assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
 
 
-def test_w8_mid_size_accumulators():
+@pytest.mark.parametrize("packed_k", [0, 128])
+def test_q4_big_tile_tails_stride_sentinels(packed_k):
+    rng = np.random.default_rng(orc.SEED + 9)
+    m, n, k = 257 + 130, 300, 384
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    storage = torch.full((m + 2, n + 5), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 5,
+                  dtype=torch.float32, algorithm="mfma", packed_k=packed_k, block_m=256)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, orc.q4_integers(packed, TABLE), scales, np.float32))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+
+
+@pytest.mark.parametrize("m,n,k", [(384, 512, 4096), (1000, 777, 640)])
+def test_w8_mid_size_accumulators(m, n, k):
     rng = np.random.default_rng(orc.SEED)
-    m, n, k = 384, 512, 4096
     x = rng.integers(-127, 128, (m, k), dtype=np.int8)
     w = rng.integers(-127, 128, (n, k), dtype=np.int8)
     got = gu.w8_project(gu.dev(x), gu.dev(np.ones(m, np.float16)), gu.dev(w), gu.dev(np.ones(n, np.float16)),
