@@ -13,6 +13,9 @@ SOURCES = ["orx_api.cpp", "k_quant.hip", "k_gemv.hip", "k_gemm.hip", "k_gemm_big
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no contraction: the epilogue's two fp32 multiplies and the fp16 cast must each round on their
+    # own (a fused multiply+convert rounds once and differs from the reference in the last bit)
+    "-ffp-contract=off",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes", "-Wno-unused-command-line-argument",
 ]
 FIXTURE_RUNNER = HERE / "orx_run_fixture"

@@ -141,6 +141,26 @@ __device__ __forceinline__ void build_tables(Q2ByteTables& t, const uint32_t* __
     }
 }
 
+// The four table entries one two-stage code needs; split from the arithmetic so that a kernel can
+// issue the LDS reads early and combine them later (software pipelining around MFMAs).
+struct Q4Lookups {
+    uint2 b0, m0, b1, m1;
+};
+__device__ __forceinline__ Q4Lookups lookup_q4(const Q4ByteTables& t, uint32_t code) {
+    Q4Lookups l;
+    l.b0 = t.basis0[(code >> 8) & 255u];
+    l.m0 = t.mask0[code & 255u];
+    l.b1 = t.basis1[code >> 24];
+    l.m1 = t.mask1[(code >> 16) & 255u];
+    return l;
+}
+__device__ __forceinline__ uint2 combine_q4(const Q4Lookups& l) {
+    uint2 w;
+    w.x = ((l.b0.x ^ l.m0.x) + (l.b1.x ^ l.m1.x) + 0x35353535u) ^ 0x80808080u;
+    w.y = ((l.b0.y ^ l.m0.y) + (l.b1.y ^ l.m1.y) + 0x35353535u) ^ 0x80808080u;
+    return w;
+}
+
 // One u32 two-stage code -> 8 int8 weights (two words: coordinates 0..3 and 4..7).
 // (x0 + x1 + 53) is w+128 in every byte, in [73,183]: no carry between bytes; the XOR
 // turns offset binary into two's complement.
@@ -163,10 +183,13 @@ __device__ __forceinline__ uint2 decode_q2(const Q2ByteTables& t, uint32_t code)
 }
 
 // fp32 epilogue shared by every projection: (float(acc) * ws) * as, two separate roundings
-// (kernels/cuda/model/integer_core.py:19-22).  The volatile-free form below relies on the
-// build flags forbidding reassociation; there is no add, so contraction cannot apply.
+// (kernels/cuda/model/integer_core.py:19-22).
 __device__ __forceinline__ float rescale(int acc, float weight_scale, float token_scale) {
-    return ((float)acc * weight_scale) * token_scale;
+    float value = ((float)acc * weight_scale) * token_scale;
+    // Opaque to the optimiser: a following fp16 cast must not be merged with the multiply into a
+    // mixed-precision fused op, which rounds once instead of fp32-then-fp16.
+    asm volatile("" : "+v"(value));
+    return value;
 }
 
 }  // namespace orx

@@ -22,6 +22,11 @@
 #include "e8p_device.h"
 #include "orx_internal.h"
 
+#ifndef ORX_BIG_TM
+#define ORX_BIG_TM 4
+#define ORX_BIG_TN 2
+#endif
+
 namespace orx {
 namespace {
 
@@ -30,8 +35,10 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTile = 256;     // output tile edge
 constexpr int kStep = 128;     // K bytes per step
-constexpr int kThreads = 512;  // 8 waves
+constexpr int kMaxThreads = 512;
 constexpr int kTileBytes = kTile * kStep;  // 32 KiB per operand per stage
+constexpr int kImagePitch = kTile + 8;     // halves per row of the fp16 output image (bank skew)
+constexpr int kEpilogueTile = kTile * kImagePitch * 2;  // bytes of the output image in LDS
 
 struct BigParams {
     const int8_t* a;
@@ -54,6 +61,16 @@ __device__ __forceinline__ void direct_load_16(const void* global, void* lds_wav
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+// The compiler does not count direct-to-LDS loads as pending at a barrier (they have no register
+// destination), so every barrier that publishes them is preceded by this explicit wait.
+__device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Same, but lets the N youngest vector-memory requests stay in flight (requests retire in order):
+// used when N ordinary loads (weight codes for a later step) were issued after the direct loads.
+template <int N>
+__device__ __forceinline__ void wait_direct_loads_except() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 // XCD-aware tile order: hardware hands consecutive workgroup ids to the 8 XCDs in turn.  Logical
 // id = (id % 8) * per_xcd + id / 8 gives each XCD one contiguous run of logical tiles; inside a
 // run, tiles advance down M in groups of 8 for each N, so concurrent workgroups of one XCD share
@@ -71,12 +88,19 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int* t
     *tn = within / rows_in_group;
 }
 
-template <bool Q4>
-__global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
+// TM x TN blocks of 32x32 per wave: <4,2> = eight waves of 128x64 (two per SIMD),
+// <4,4> = four waves of 128x128 (one per SIMD, accumulators spill over into AGPRs).
+template <bool Q4, int TM, int TN>
+__global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigParams p) {
+    constexpr int WAVES_N = 8 / TN;
+    constexpr int WAVES = (8 / TM) * WAVES_N;
+    constexpr int kThreads = WAVES * 64;
+    constexpr int BLOCKS_PER_WAVE = 32 / WAVES;  // 1 KiB blocks of each operand tile per wave
+    constexpr int CODE_CHUNKS = 1024 / kThreads; // 16-byte code chunks per thread per K step
     extern __shared__ __align__(16) int8_t lds[];  // [2 stages][A 32 KiB | W 32 KiB] (+ Q4 tables)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_m = wave >> 2, wave_n = wave & 3;  // 2 x 4 waves, wave tile 128 x 64
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
     int tile_m, tile_n;
     tile_of(blockIdx.x, p.tiles_m, p.tiles_n, &tile_m, &tile_n);
@@ -84,16 +108,27 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
     const int rows_here = min(kTile, p.m - row0);
     const int cols_here = min(kTile, p.n - col0);
 
+    // Scales of this tile, one or two per thread, fetched now as raw bits so that the epilogue
+    // does not pay a memory round trip: entries 0..255 token scales, 256..511 weight scales.
+    constexpr int SCALES_PER_THREAD = 2 * kTile / kThreads;
+    unsigned short scale_bits[SCALES_PER_THREAD];
+#pragma unroll
+    for (int e = 0; e < SCALES_PER_THREAD; ++e) {
+        const int i = tid + e * kThreads;
+        scale_bits[e] = i < kTile ? reinterpret_cast<const unsigned short*>(p.as)[row0 + min(i, rows_here - 1)]
+                                  : reinterpret_cast<const unsigned short*>(p.ws)[col0 + min(i - kTile, cols_here - 1)];
+    }
+
     Q4ByteTables* tables = reinterpret_cast<Q4ByteTables*>(lds + 4 * kTileBytes);
     if (Q4) build_tables(*tables, p.book, tid, kThreads);
 
     // ---- global -> LDS: one wave instruction = 8 rows x 128 bytes (1 KiB block) ----
-    // wave w owns blocks w*4 .. w*4+3 of each operand tile (32 blocks of 8 rows)
+    // wave w owns BLOCKS_PER_WAVE consecutive blocks of each operand tile (32 blocks of 8 rows)
     const int load_r8 = lane >> 3, load_slot = lane & 7;
     auto issue_direct = [&](const int8_t* base, int limit, int origin, int kt, int8_t* stage) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int block = wave * 4 + b;
+        for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
+            const int block = wave * BLOCKS_PER_WAVE + b;
             const int row = block * 8 + load_r8;
             const int chunk = load_slot ^ swizzle(row);
             const int source_row = origin + min(row, limit - 1);
@@ -101,11 +136,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
         }
     };
     // Q4: one K step of the weight tile is 256 rows x 64 bytes of codes = 1024 chunks of 16 bytes
-    // (4 codes = 32 weights each): two chunks per thread.
-    uint4 code_regs[2];
-    auto load_codes = [&](int kt) {
+    // (4 codes = 32 weights each): CODE_CHUNKS chunks per thread.
+    // Two register sets so that the codes of step t+1 can be in flight while step t is decoded.
+    uint4 code_regs[2][CODE_CHUNKS];
+    auto load_codes = [&](int kt, int set) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < CODE_CHUNKS; ++i) {
             const int c = tid + kThreads * i;      // chunk id: row = c / 4, quarter = c % 4
             const int row = min(c >> 2, cols_here - 1), q = c & 3;
             int64_t byte;
@@ -113,17 +149,18 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
                 byte = ((int64_t)kt * p.n + col0 + row) * 64 + q * 16;
             else
                 byte = ((int64_t)(col0 + row) * (p.k / kStep) + kt) * 64 + q * 16;
-            code_regs[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(p.w) + byte);
+            code_regs[set][i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(p.w) + byte);
         }
     };
-    auto store_decoded = [&](int8_t* stage) {
+    // Decode the codes of one K step (4 codes -> 32 weights -> two 16-byte LDS stores per chunk).
+    auto decode_step = [&](int8_t* stage, int set) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < CODE_CHUNKS; ++i) {
             const int c = tid + kThreads * i;
             const int row = c >> 2, q = c & 3;
-            const uint2 d0 = decode_q4(*tables, code_regs[i].x), d1 = decode_q4(*tables, code_regs[i].y);
-            const uint2 d2 = decode_q4(*tables, code_regs[i].z), d3 = decode_q4(*tables, code_regs[i].w);
-            // 32 weights = chunks 2q and 2q+1 of the row
+            const uint4 codes = code_regs[set][i];
+            const uint2 d0 = decode_q4(*tables, codes.x), d1 = decode_q4(*tables, codes.y);
+            const uint2 d2 = decode_q4(*tables, codes.z), d3 = decode_q4(*tables, codes.w);
             int8_t* row_base = stage + row * kStep;
             const int s = swizzle(row);
             *reinterpret_cast<uint4*>(row_base + (((2 * q) ^ s) * 16)) = make_uint4(d0.x, d0.y, d1.x, d1.y);
@@ -137,14 +174,14 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
     int frag_offset[4];                 // byte offset inside a row for K sub-step ks
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) frag_offset[ks] = ((2 * ks + frag_half) ^ swz) * 16;
-    const int a_lane = (wave_m * 128 + frag_row) * kStep;
-    const int w_lane = (wave_n * 64 + frag_row) * kStep;
+    const int a_lane = (wave_m * TM * 32 + frag_row) * kStep;
+    const int w_lane = (wave_n * TN * 32 + frag_row) * kStep;
 
-    v16i acc[4][2];
+    v16i acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
@@ -152,80 +189,196 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_big_kernel(BigParams p) {
     auto stage_a = [&](int stage) { return lds + stage * 2 * kTileBytes; };
     auto stage_w = [&](int stage) { return lds + kTileBytes + stage * 2 * kTileBytes; };
 
+    // Software pipeline over K steps (two LDS stages, two fragment register slots):
+    //   prologue   steps 0 and 1 requested, step 0 published, its first fragments read
+    //   step kt    sub-steps 0..2: read fragments ks+1, issue MFMAs ks
+    //              barrier: step kt+1 is complete in LDS and nobody reads stage `cur` any more
+    //              read fragments 0 of step kt+1, issue MFMAs of sub-step 3 (their operands are
+    //              already in registers), request step kt+2 into stage `cur`
+    // so the matrix pipe always holds queued work while waves meet at the barrier.
+    const int8_t* w8 = reinterpret_cast<const int8_t*>(p.w);
     issue_direct(p.a, rows_here, row0, 0, stage_a(0));
-    if (Q4) {
-        load_codes(0);
-        __syncthreads();  // tables
-        store_decoded(stage_w(0));
-        if (k_tiles > 1) load_codes(1);
-    } else {
-        issue_direct(reinterpret_cast<const int8_t*>(p.w), cols_here, col0, 0, stage_w(0));
+    if (!Q4) issue_direct(w8, cols_here, col0, 0, stage_w(0));
+    if (k_tiles > 1) {
+        issue_direct(p.a, rows_here, row0, 1, stage_a(1));
+        if (!Q4) issue_direct(w8, cols_here, col0, 1, stage_w(1));
     }
+    if (Q4) {
+        load_codes(0, 0);
+        if (k_tiles > 1) load_codes(1, 1);
+        __syncthreads();  // tables
+        decode_step(stage_w(0), 0);
+        if (k_tiles > 2) load_codes(2, 0);
+        if (k_tiles > 1) decode_step(stage_w(1), 1);
+        if (k_tiles > 3) load_codes(3, 1);
+    }
+    wait_direct_loads();
+    __syncthreads();
 
+    v4i fa[2][TM], fb[2][TN];
+    auto read_fragments = [&](int stage, int ks, int slot) {
+        const int8_t* la = stage_a(stage) + a_lane;
+        const int8_t* lw = stage_w(stage) + w_lane;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const v4i*>(la + i * 32 * kStep + frag_offset[ks]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb[slot][j] = *reinterpret_cast<const v4i*>(lw + j * 32 * kStep + frag_offset[ks]);
+    };
+    auto multiply = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+    };
+    // Q4: the whole weight tile of step kt+2 is decoded in one piece right after MFMA group 3 of
+    // step kt, into the stage the barrier of step kt has just released.  (Threading the decode
+    // between the MFMAs of a group, with or without pipelined table reads, measured 20 % slower:
+    // the LDS waits of the decode then sit in the MFMA issue stream.)
+    read_fragments(0, 0, 0);
     for (int kt = 0; kt < k_tiles; ++kt) {
         const int cur = kt & 1, nxt = cur ^ 1;
-        __syncthreads();  // step kt is in LDS for everybody; everybody is done reading stage nxt
-        if (kt + 1 < k_tiles) {
-            issue_direct(p.a, rows_here, row0, kt + 1, stage_a(nxt));
-            if (!Q4) issue_direct(reinterpret_cast<const int8_t*>(p.w), cols_here, col0, kt + 1, stage_w(nxt));
+#pragma unroll
+        for (int ks = 0; ks < 3; ++ks) {
+            read_fragments(cur, ks + 1, (ks + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);  // reads above stay ahead of the MFMAs below
+            multiply(ks & 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        const int8_t* la = stage_a(cur) + a_lane;
-        const int8_t* lw = stage_w(cur) + w_lane;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            v4i fa[4], fb[2];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const v4i*>(la + i * 32 * kStep + frag_offset[ks]);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) fb[j] = *reinterpret_cast<const v4i*>(lw + j * 32 * kStep + frag_offset[ks]);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        // this wave's part of step kt+1, requested one step ago; the code loads issued after it
+        // (Q4, step kt+3) may stay in flight: a barrier should not wait for HBM
+        if (Q4 && kt + 3 < k_tiles)
+            wait_direct_loads_except<CODE_CHUNKS>();
+        else
+            wait_direct_loads();
+        __syncthreads();
+        if (Q4 && kt + 2 < k_tiles) issue_direct(p.a, rows_here, row0, kt + 2, stage_a(cur));
+        if (kt + 1 < k_tiles) read_fragments(nxt, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!Q4 && kt + 2 < k_tiles) {
+            // W8: requested behind the fragment reads so the 64 KiB burst into LDS does not delay them
+            issue_direct(p.a, rows_here, row0, kt + 2, stage_a(cur));
+            issue_direct(w8, cols_here, col0, kt + 2, stage_w(cur));
         }
-        if (Q4 && kt + 1 < k_tiles) {
-            store_decoded(stage_w(nxt));  // stage nxt was released by the barrier above
-            if (kt + 2 < k_tiles) load_codes(kt + 2);
+        if (Q4 && kt + 2 < k_tiles) {
+            decode_step(stage_w(cur), cur);
+            if (kt + 4 < k_tiles) load_codes(kt + 4, cur);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- epilogue ----
+    // Weights are the MFMA row operand, so a lane holds token row (lane & 31) of each 32x32 block
+    // and, per group of four accumulator registers, four CONSECUTIVE output channels
+    // 8*q + 4*(lane >> 5) + {0..3}.
+    const int half = lane >> 5;
+    if (p.out_f32) {
+        // fp32 heads are rare: 16-byte stores straight from the accumulators
+        const bool vector_ok = p.stride % 4 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int local_col = wave_n * 64 + j * 32 + (lane & 31);
-        if (local_col >= cols_here) continue;
-        const int col = col0 + local_col;
-        const float wscale = __half2float(p.ws[col]);
+        for (int i = 0; i < TM; ++i) {
+            const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
+            if (local_row >= rows_here) continue;
+            const int64_t row = row0 + local_row;
+            const float token_scale = __half2float(p.as[row]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+            for (int j = 0; j < TN; ++j) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int local = wave_m * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (local < rows_here) {
-                    const int64_t row = row0 + local;
-                    const float value = rescale(acc[i][j][r], wscale, __half2float(p.as[row]));
-                    if (p.out_f32)
-                        reinterpret_cast<float*>(p.out)[row * p.stride + col] = value;
-                    else
-                        reinterpret_cast<__half*>(p.out)[row * p.stride + col] = __float2half_rn(value);
+                for (int q = 0; q < 4; ++q) {
+                    const int local_col = (wave_n * TN + j) * 32 + 8 * q + 4 * half;
+                    if (local_col >= cols_here) continue;
+                    const int col = col0 + local_col;
+                    float value[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        value[r] = rescale(acc[i][j][4 * q + r], __half2float(p.ws[min(col + r, p.n - 1)]), token_scale);
+                    float* dst = reinterpret_cast<float*>(p.out) + row * p.stride + col;
+                    if (local_col + 4 <= cols_here && vector_ok && (col & 3) == 0) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(value[0], value[1], value[2], value[3]);
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (local_col + r < cols_here) dst[r] = value[r];
+                    }
                 }
             }
+        }
+        return;
+    }
+    // fp16: rescale into an LDS image of the tile (8-byte writes), then store whole 16-byte pieces
+    // of output rows.  The operand stages are dead after the last K step, so their LDS is reused.
+    __syncthreads();
+    float* lds_as = reinterpret_cast<float*>(lds + kEpilogueTile);  // 256 token scales
+    float* lds_ws = lds_as + kTile;                                  // 256 weight scales
+#pragma unroll
+    for (int e = 0; e < SCALES_PER_THREAD; ++e)
+        lds_as[tid + e * kThreads] = __half2float(__ushort_as_half(scale_bits[e]));  // lds_ws follows lds_as
+    __syncthreads();
+    __half* image = reinterpret_cast<__half*>(lds);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
+        const float token_scale = lds_as[local_row];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int local_col = (wave_n * TN + j) * 32 + 8 * q + 4 * half;
+                const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
+                const __half2 lo = __halves2half2(__float2half_rn(rescale(acc[i][j][4 * q + 0], wscale.x, token_scale)),
+                                                  __float2half_rn(rescale(acc[i][j][4 * q + 1], wscale.y, token_scale)));
+                const __half2 hi = __halves2half2(__float2half_rn(rescale(acc[i][j][4 * q + 2], wscale.z, token_scale)),
+                                                  __float2half_rn(rescale(acc[i][j][4 * q + 3], wscale.w, token_scale)));
+                uint2 packed;
+                packed.x = *reinterpret_cast<const uint32_t*>(&lo);
+                packed.y = *reinterpret_cast<const uint32_t*>(&hi);
+                *reinterpret_cast<uint2*>(image + local_row * kImagePitch + local_col) = packed;
+            }
+        }
+    }
+    __syncthreads();
+    // each thread moves 16 bytes: kThreads/32 rows x 512 bytes per pass
+    const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0) && (col0 % 8 == 0);
+    const int piece = tid & 31, piece_row = tid >> 5;
+    constexpr int ROWS_PER_PASS = kThreads / 32;
+#pragma unroll 4
+    for (int pass = 0; pass < kTile / ROWS_PER_PASS; ++pass) {
+        const int local = pass * ROWS_PER_PASS + piece_row;
+        if (local >= rows_here) break;
+        const uint4 value = *reinterpret_cast<const uint4*>(image + local * kImagePitch + piece * 8);
+        __half* dst = reinterpret_cast<__half*>(p.out) + (int64_t)(row0 + local) * p.stride + col0 + piece * 8;
+        if (aligned && piece * 8 + 8 <= cols_here) {
+            *reinterpret_cast<uint4*>(dst) = value;
+        } else {
+            const __half* h = reinterpret_cast<const __half*>(&value);
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (piece * 8 + e < cols_here) dst[e] = h[e];
         }
     }
 }
 
-constexpr uint32_t kBigLds = 4 * kTileBytes;                       // 128 KiB
-constexpr uint32_t kBigLdsQ4 = 4 * kTileBytes + sizeof(Q4ByteTables);  // + 8 KiB
+// operand stages (128 KiB, + 8 KiB of decode tables for Q4) or the epilogue's output image + scales
+constexpr uint32_t kBigLdsEpilogue = kEpilogueTile + 2 * kTile * 4;
+constexpr uint32_t kBigLds = 4 * kTileBytes > kBigLdsEpilogue ? 4 * kTileBytes : kBigLdsEpilogue;
+constexpr uint32_t kBigLdsQ4 = 4 * kTileBytes + sizeof(Q4ByteTables) > kBigLdsEpilogue
+                                   ? 4 * kTileBytes + sizeof(Q4ByteTables)
+                                   : kBigLdsEpilogue;
+
+// wave shape of the shipped kernels
+constexpr int kTM = ORX_BIG_TM, kTN = ORX_BIG_TN;
+constexpr int kBigThreads = (8 / kTM) * (8 / kTN) * 64;
 
 int prepare() {
     static bool done = false;
     if (done) return ORX_OK;
-    int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<false>),
+    int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<false, kTM, kTN>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds),
                          "hipFuncSetAttribute");
     if (code != ORX_OK) return code;
-    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<true>),
+    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<true, kTM, kTN>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsQ4),
                      "hipFuncSetAttribute");
     if (code != ORX_OK) return code;
@@ -238,7 +391,7 @@ int prepare() {
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTile) * ceil_div((uint32_t)n, (uint32_t)kTile);
     g->grid[1] = g->grid[2] = 1;
-    g->block[0] = kThreads;
+    g->block[0] = kBigThreads;
     g->shared = q4 ? kBigLdsQ4 : kBigLds;
 }
 
@@ -252,9 +405,9 @@ int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* boo
     p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = packed_k, p.out_f32 = out_f32;
     p.tiles_m = (rows + kTile - 1) / kTile, p.tiles_n = (n + kTile - 1) / kTile;
     if (q4)
-        hipLaunchKernelGGL((gemm_big_kernel<true>), dim3(g.grid[0]), dim3(kThreads), g.shared, stream, p);
+        hipLaunchKernelGGL((gemm_big_kernel<true, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
     else
-        hipLaunchKernelGGL((gemm_big_kernel<false>), dim3(g.grid[0]), dim3(kThreads), g.shared, stream, p);
+        hipLaunchKernelGGL((gemm_big_kernel<false, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
     return hip_check(hipGetLastError(), "launch projection (mfma 256x256)");
 }
 
