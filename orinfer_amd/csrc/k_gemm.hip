@@ -25,6 +25,15 @@ int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t 
 int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
 int gemv_configure(orx_function* f, int codec, int passes_override);
 int gemv_prepare_device();
+// from k_stream.hip
+void stream_geometry(int n, Geometry* g);
+int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                  void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
+void stream_grouped_geometry(int n, int tiles, Geometry* g);
+int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                          void* out, const int* counts, const int* offsets, const int* tile_expert, const int* tile_row,
+                          const int* tile_count, int n, int k, int tiles, int block_m, int packed_k,
+                          hipStream_t stream);
 // from k_gemm_big.hip
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g);
 int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
@@ -37,7 +46,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
-enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2 };
+enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3 };
 
 constexpr int kBK = 128;        // K bytes per tile step
 constexpr int kPitch = kBK + 16;  // LDS row pitch in bytes
@@ -281,11 +290,20 @@ bool use_gemv(const orx_function& f, int rows) {
     return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
 }
 
+// weight-streaming kernel for up to 64 rows (auto), or when asked for by name
+bool use_stream(const orx_function& f, int rows) {
+    return rows <= 64 && (f.algorithm == kStream || (f.algorithm == kAuto && f.tiles == 0));
+}
+
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
 bool use_big(const orx_function& f, int rows) { return f.tiles == 256 || (f.tiles == 0 && rows > 128); }
 
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
+    if (use_stream(f, rows)) {
+        stream_geometry(f.N, g);
+        return ORX_OK;
+    }
     if (use_big(f, rows)) {
         gemm_big_geometry(rows, f.N, f.flags == kQ4, g);
         return ORX_OK;
@@ -309,6 +327,9 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, 5);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_stream(f, rows))
+        return stream_launch(kQ4, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32,
+                             stream);
     if (use_big(f, rows))
         return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
                                f.out_f32, g, stream);
@@ -326,6 +347,8 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.book = nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = 0, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_stream(f, rows))
+        return stream_launch(kW8, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, stream);
     if (use_big(f, rows))
         return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
                                stream);
@@ -370,9 +393,17 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     f->out_f32 = dtype == "float32";
     f->capacity = f->M;
     f->flags = codec;
-    f->algorithm = algorithm == "gemv" ? kGemv : algorithm == "mfma" ? kMfma : algorithm == "auto" ? kAuto : -1;
+    f->algorithm = algorithm == "gemv"     ? kGemv
+                   : algorithm == "mfma"   ? kMfma
+                   : algorithm == "stream" ? kStream
+                   : algorithm == "auto"   ? kAuto
+                                           : -1;
     if (f->algorithm < 0) {
-        set_error("%s: algorithm must be auto, gemv or mfma", name);
+        set_error("%s: algorithm must be auto, gemv, stream or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kStream && f->capacity > 64) {
+        set_error("%s: the stream algorithm serves up to 64 rows, variant asks for %d", name, f->capacity);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->algorithm == kGemv && f->packed_k != 0) {
@@ -421,6 +452,10 @@ int make_w8_projection(const Variant& v, orx_function* f) {
 // (tests/cuda/operators/e8p_decode.py:72-84; kernels/cuda/model/e8p_decode.py:60-73 without Patch)
 int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
     (void)rows;
+    if (f.block_m <= 64 && f.algorithm != kMfma) {
+        stream_grouped_geometry(f.N, f.tiles, g);
+        return ORX_OK;
+    }
     g->grid[0] = ceil_div((uint32_t)f.N, 128u);
     g->grid[1] = (uint32_t)f.tiles;
     g->block[0] = 256;
@@ -443,6 +478,9 @@ int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     p.ws = pointer_arg<const __half>(args, 10);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
+    if (f.block_m <= 64 && f.algorithm != kMfma)
+        return stream_grouped_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
+                                     p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.block_m, f.packed_k, stream);
     return launch_mfma<kQ2, true>(f.block_m, p, g, stream);
 }
 
@@ -455,8 +493,14 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     f->K = (int)v.integer("K", 0, &bad);
     f->block_m = (int)v.integer("block_m", 32, &bad);
     f->packed_k = (int)v.integer("packed_k", 128, &bad);
+    const std::string grouped_algorithm = v.string("algorithm", "auto", &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
+    if (grouped_algorithm != "auto" && grouped_algorithm != "mfma" && grouped_algorithm != "stream") {
+        set_error("%s: algorithm must be auto, stream or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->algorithm = grouped_algorithm == "mfma" ? kMfma : kAuto;
     if (f->M <= 0 || f->E <= 0 || f->tiles <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 ||
         (int64_t)f->K * 128 * 128 > 2147483647LL) {
         set_error("%s: invalid E8P decode geometry", name);  // e8p_decode.py:52
@@ -527,16 +571,16 @@ int make_q2_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f,
 const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
-     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, packed_k=0|128, output_dtype=float16|float32, "
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, packed_k=0|128, output_dtype=float16|float32, "
      "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0",
      "A,AS,Book,Out,S,W[,m]"},
     {"int8_projection", make_w8_projection,
-     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|mfma, output_dtype=float16|float32, output_stride=N, "
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "
      "block_m=0|32|64|128|256",
      "A,Output,TokenScale,Weight,WeightScale[,m]"},
-    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0",
+    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
-    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0",
+    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},

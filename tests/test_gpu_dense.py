@@ -170,6 +170,45 @@ def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
+@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("m", [5, 8, 31, 32, 33, 64])
+def test_q4_stream_rows_tails_stride_and_sentinels(m, packed_k):
+    # same construction as the MFMA tail test, through the weight-streaming kernel; K=640 gives the
+    # eight K slices of a workgroup uneven shares (5 blocks over 8 waves, three of them empty)
+    rng = np.random.default_rng(orc.SEED + 100 + m)
+    n, k = 97, 640
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    w = orc.q4_integers(packed, TABLE)
+    storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
+                  dtype=torch.float32, algorithm="stream", packed_k=packed_k)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, w, scales, np.float32))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+    ones_n, ones_m = np.ones(n, np.float16), np.ones(m, np.float16)
+    acc = gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), dtype=torch.float32,
+                        algorithm="stream", packed_k=packed_k)
+    np.testing.assert_array_equal(gu.host(acc).astype(np.int64), orc.int_dot(a_q, w).astype(np.int64))
+    half = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), algorithm="stream", packed_k=packed_k)
+    np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
+
+
+@pytest.mark.parametrize("m,n,k", [(7, 48, 2560), (40, 65, 128), (64, 129, 640)])
+def test_w8_stream_matches_oracle(m, n, k):
+    rng = np.random.default_rng(orc.SEED + m)
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    ws = rng.uniform(0.001, 0.01, n).astype(np.float16)
+    ts = rng.uniform(0.001, 0.01, m).astype(np.float16)
+    out = torch.full((m + 1, n), 99.0, dtype=torch.float16, device=gu.DEV)
+    gu.w8_project(gu.dev(x), gu.dev(ts), gu.dev(w), gu.dev(ws), out=out, algorithm="stream")
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:m], orc.project(x, ts, w, ws))
+    assert (got[m] == 99).all()
+
+
 @pytest.mark.parametrize("block_m", [32, 64, 128, 256])
 def test_q4_mfma_tiles_and_accumulators(block_m):
     rng = np.random.default_rng(orc.SEED + block_m)

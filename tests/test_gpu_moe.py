@@ -78,9 +78,10 @@ def test_routing_metadata_and_dispatch(m, e, k, bm):
     np.testing.assert_array_equal(gu.host(ds), want_ds)
 
 
+@pytest.mark.parametrize("algorithm", ["auto", "mfma"])
 @pytest.mark.parametrize("packed_k", [128, 0])
 @pytest.mark.parametrize("bm", [32, 64, 128])
-def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k):
+def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k, algorithm):
     # count mixes in the spirit of tests/cuda/operators/e8p_exact.py:141-198: empty experts,
     # single rows, exact tile multiples, tails, one hot expert
     rng = np.random.default_rng(orc.SEED + bm)
@@ -97,7 +98,8 @@ def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k):
     te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
     stored = codes if packed_k == 0 else np.stack([orc.q2_pack_k128(c) for c in codes])
     out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
-    kern = gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k)
+    kern = gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
+                     algorithm=algorithm)
     counts, offsets = gu.dev(counts_np), gu.dev(offsets_np)
     tile_count = gu.dev(total)
     args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=counts, Offsets=offsets, P=gu.dev(stored),
