@@ -22,9 +22,12 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA (5.0 POP/s)
 CACHE_BYTES = 256 << 20        # Infinity Cache
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of the contract kernel from two `rocprofv3 --pmc` runs of
+# `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
+# same counter reads for a device copy of 44 564 480 bytes in the same run: FETCH_SIZE reads
+# 21 774.8 for 43 520 KiB (factor 1.9986), WRITE_SIZE reads 43 520.0 (factor 1.0).
+# Projection: fetch 21 873.8 -> 44 767 114 B, write 34.0 -> 34 816 B.
+MEASURED_TRAFFIC_BYTES = 44_801_930
 
 
 def parse():
@@ -34,6 +37,9 @@ def parse():
     p.add_argument("--warmup", type=int, default=24)
     p.add_argument("--no-extra", action="store_true", help="only the contract workload")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--traffic-probe", action="store_true",
+                   help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a plain copy of known size, then the "
+                        "contract kernel once per weight copy, eagerly; no timing")
     return p.parse_args()
 
 
@@ -58,7 +64,8 @@ def main():
         return torch.from_numpy(a.view(view) if view else a).cuda()
 
     def timed_graph(enqueue, launches, replays=3):
-        """Captures `launches` calls of enqueue(i) in one graph; returns best seconds per launch."""
+        """Captures `launches` calls of enqueue(i) in one graph; returns mean seconds per launch over
+        `replays` replays (the first replay uploads the graph and is not counted)."""
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
@@ -67,16 +74,17 @@ def main():
             with torch.cuda.graph(graph, stream=side):
                 for i in range(launches):
                     enqueue(i, side.cuda_stream)
-        best = float("inf")
-        for _ in range(replays + 1):
+        total = 0.0
+        for replay in range(replays + 1):
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             start.record()
             graph.replay()
             stop.record()
             torch.cuda.synchronize()
-            best = min(best, start.elapsed_time(stop) * 1e-3 / launches)
-        return best
+            if replay:
+                total += start.elapsed_time(stop) * 1e-3 / launches
+        return total / replays
 
     book = dev(codebook.book())
 
@@ -113,6 +121,19 @@ def main():
     bytes_c1 = workloads.algorithmic_bytes_q4(1, c1["n"], c1["k"])
     copies = -(-2 * CACHE_BYTES // (c1["n"] * c1["k"] // 2))  # aggregate footprint >= 2x the cache
     main_case = Q4Case(c1, copies)
+    if args.traffic_probe:
+        # counter calibration: a device copy reads and writes exactly `probe.numel()` bytes
+        probe = torch.empty(c1["n"] * c1["k"] // 2, dtype=torch.uint8, device="cuda").random_(0, 256)
+        target = torch.empty_like(probe)
+        main_case.quantize(stream.cuda_stream)
+        for _ in range(4):
+            target.copy_(probe)
+        for i in range(copies):
+            main_case.project(i, stream.cuda_stream)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": {"copy_bytes_read": probe.numel(), "copy_bytes_written": probe.numel(),
+                                            "projection_launches": copies, "algorithmic_bytes": bytes_c1}}))
+        return
     for i in range(args.warmup):
         main_case.step(i, stream.cuda_stream)
     torch.cuda.synchronize()
@@ -256,16 +277,21 @@ def main():
             return orc.project(a_q, a_s[:, 0], w, c1["scales"])
 
         ctx = threadpool_limits(limits=1) if threadpool_limits else None
-        t0 = time.perf_counter()
-        cpu_once()
-        cpu_seconds = time.perf_counter() - t0
+        calls, spent = 0, 0.0
+        while spent < 10.0 and calls < 16:          # bounded sample: about 10 s of host work
+            t0 = time.perf_counter()
+            cpu_once()
+            spent += time.perf_counter() - t0
+            calls += 1
+        cpu_seconds = spent / calls
         if ctx is not None:
             ctx.unregister() if hasattr(ctx, "unregister") else None
         result["cpu_baseline"] = {
             "value": round(bytes_c1 / cpu_seconds / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
             "seconds_per_call": round(cpu_seconds, 3), "host_cpus": os.cpu_count(),
-            "sample": "one full call of the numpy oracle on config 1, M=1 (decode 11.1M two-stage codes, "
-                      "fp64 dot, rescale), single thread",
+            "calls": calls,
+            "sample": "mean of `calls` full calls of the numpy oracle on config 1, M=1 (A8, decode of 11.1M "
+                      "two-stage codes, exact dot, rescale), single thread, about 10 s in total",
         }
     print(json.dumps(result))
 

@@ -13,7 +13,9 @@
 //     sum q*a = 2*(16*sum v*hi + sum v*lo + 8*sum v) + sum a.
 // Two-stage Q4 (w = 4*q0 + q1 = 8*v0 + 2*v1 + 5) keeps one accumulator set per stage.
 // Lanes of a row group own fixed k-chunks; LPR lanes share one output row and are
-// reduced with cross-lane shuffles at the end.  No atomics, no scratch, no host reads.
+// reduced with cross-lane shuffles at the end.  The only atomics are integer adds into LDS for the
+// per-row activation sums (order-independent, so results stay bit-exact); no global atomics, no
+// scratch memory, no host reads.
 #include <hip/hip_fp16.h>
 
 #include "e8p_device.h"

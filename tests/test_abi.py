@@ -1,0 +1,173 @@
+"""CPU checks of the C-ABI library and of the host-side helpers: every symbol declared in
+include/orx.h is exported, resolve / geometry / argument order / error codes behave like the
+engine's catalog (crates/orinfer-engine/src/backend/cuda/kernels.rs:47-61,114-192), and the
+package-side codebook and workload generators agree with the oracle.  Nothing here computes on a
+device."""
+import ctypes
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from oracle import reference as ref
+from orinfer_amd import codebook, lib, workloads
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def declared_symbols():
+    text = (ROOT / "include" / "orx.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(orx_[a-z_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = declared_symbols()
+    assert len(names) == 10 and set(names) == set(lib.EXPORTS)
+    raw = ctypes.CDLL(str(lib.LIBRARY_PATH))
+    for name in names:
+        assert getattr(raw, name) is not None, name
+
+
+def test_catalog_lists_every_symbol_and_resolves():
+    catalog = lib.catalog()["kernels"]
+    symbols = [entry["symbol"] for entry in catalog]
+    assert len(symbols) == len(set(symbols))
+    for needed in ("activation_quantization", "swiglu", "e8p_q4_projection", "int8_projection",
+                   "e8p_decode_grouped", "integer_vq_grouped", "e8p_q4_unpack", "e8p_q2_unpack", "router_topk",
+                   "expert_histogram", "expert_offsets", "expert_tiles", "expert_dispatch", "moe_combine"):
+        assert needed in symbols
+
+
+ABI = {
+    # symbol, variant -> expected argument order (buffers in ASCII order, scalars, m last)
+    ("activation_quantization", (("K", 2560),)): ["Mask", "Q", "S", "X", "rows"],
+    ("swiglu", (("I", 512),)): ["X", "Y", "rows"],
+    ("e8p_q4_projection", (("M", 1), ("N", 9728), ("K", 2560))): ["A", "AS", "Book", "Out", "S", "W"],
+    ("e8p_q4_projection", (("M", 64), ("N", 256), ("K", 256), ("dynamic_rows", True))):
+        ["A", "AS", "Book", "Out", "S", "W", "m"],
+    ("int8_projection", (("M", 8192), ("N", 4096), ("K", 4096))):
+        ["A", "Output", "TokenScale", "Weight", "WeightScale"],
+    ("e8p_decode_grouped", (("rows", 640), ("E", 512), ("tiles", 552), ("N", 1024), ("K", 2048))):
+        ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "TileCount", "TileExpert", "TileRow", "WS"],
+    ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
+    ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
+    ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],
+    ("expert_tiles", (("M", 64),)): ["Counts", "TileExpert", "TileOffsets", "TileRow"],
+    ("expert_dispatch", (("M", 64), ("H", 2048))):
+        ["A", "D", "DS", "IDs", "RelativeSlot", "RowOffsets", "Scale", "SlotMap"],
+    ("moe_combine", (("M", 64), ("H", 2048), ("dynamic_rows", True))):
+        ["Expert", "Output", "Prob", "Shared", "SharedGate", "SlotMap", "m"],
+}
+
+
+@pytest.mark.parametrize("key", list(ABI), ids=lambda k: k[0])
+def test_argument_order_is_the_reference_host_abi(key):
+    symbol, variant = key
+    kernel = lib.Kernel(symbol, **dict(variant))
+    assert kernel.arg_names == ABI[key]
+    buffers = [n for n, kind in zip(kernel.arg_names, kernel.arg_kinds) if kind == 0]
+    assert buffers == sorted(buffers)
+    assert all(kind == 1 for n, kind in zip(kernel.arg_names, kernel.arg_kinds) if n in ("m", "rows"))
+    grid, block, shared = kernel.geometry()
+    assert block[0] * block[1] * block[2] <= 1024
+    assert all(g >= 1 for g in grid) and shared <= 160 * 1024
+
+
+def test_resolve_errors():
+    with pytest.raises(lib.OrxError) as err:
+        lib.Kernel("no_such_kernel", M=1)
+    assert err.value.code == lib.ORX_ERR_UNKNOWN_SYMBOL
+    for variant in (dict(M=1, N=9728), dict(M=1, N=9728, K=2500), dict(M=0, N=128, K=128),
+                    dict(M=1, N=128, K=128, algorithm="cublas"), dict(M=1, N=128, K=128, output_dtype="bfloat16"),
+                    dict(M=8, N=128, K=128, packed_k=96), dict(M=1, N="x", K=128)):
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel("e8p_q4_projection", **variant)
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT, variant
+        assert "e8p_q4_projection" in str(err.value) or "variant" in str(err.value)
+    handle = ctypes.c_void_p()
+    code = lib.library().orx_resolve(b"swiglu", b"{not json", ctypes.byref(handle))
+    assert code == lib.ORX_ERR_BAD_VARIANT and not handle.value
+    assert lib.library().orx_resolve(None, b"{}", ctypes.byref(handle)) == lib.ORX_ERR_BAD_ARGUMENT
+    assert lib.last_error()
+
+
+def test_dynamic_geometry_follows_live_rows():
+    kernel = lib.Kernel("e8p_q4_projection", M=64, N=9728, K=2560, dynamic_rows=True)
+    one, many, big = kernel.geometry(1), kernel.geometry(64), lib.Kernel(
+        "e8p_q4_projection", M=512, N=9728, K=2560, dynamic_rows=True).geometry(512)
+    assert one != many                        # batch-1 and batch-64 take different kernels
+    assert big[0][0] * big[0][1] * big[0][2] == 2 * 38
+    with pytest.raises(lib.OrxError) as err:
+        kernel.geometry(65)
+    assert err.value.code == lib.ORX_ERR_ROWS
+    fixed = lib.Kernel("int8_projection", M=8192, N=4096, K=4096)
+    grid, block, shared = fixed.geometry()
+    assert grid[0] * grid[1] * grid[2] == (8192 // 256) * (4096 // 256) and block == (512, 1, 1)
+    assert shared > 64 * 1024                 # two LDS stages of the 256x256 tile
+
+
+def test_launch_record_is_validated_before_anything_is_enqueued():
+    kernel = lib.Kernel("e8p_q4_projection", M=2, N=256, K=256)
+    grid, block, shared = kernel.geometry()
+    fake = [256] * 6                           # aligned, never dereferenced: every call below is rejected
+    for bad in ((grid[0] + 1, 1, 1), (0, 1, 1)):
+        with pytest.raises(lib.OrxError) as err:
+            kernel.launch_raw(bad, block, shared, 0, fake)
+        assert err.value.code == lib.ORX_ERR_BAD_GEOMETRY
+    with pytest.raises(lib.OrxError) as err:
+        kernel.launch_raw(grid, (block[0] // 2, 1, 1), shared, 0, fake)
+    assert err.value.code == lib.ORX_ERR_BAD_GEOMETRY
+    with pytest.raises(lib.OrxError) as err:
+        kernel.launch_raw(grid, block, shared + 16, 0, fake)
+    assert err.value.code == lib.ORX_ERR_BAD_GEOMETRY
+    for position in range(6):
+        for pointer in (0, 257):                # null, misaligned
+            values = list(fake)
+            values[position] = pointer
+            with pytest.raises(lib.OrxError) as err:
+                kernel.launch_raw(grid, block, shared, 0, values)
+            assert err.value.code == lib.ORX_ERR_BAD_ARGUMENT, (position, pointer)
+    assert lib.library().orx_launch(None, None, None, 0, None, None) == lib.ORX_ERR_BAD_ARGUMENT
+    dynamic = lib.Kernel("e8p_q4_projection", M=4, N=256, K=256, dynamic_rows=True)
+    grid, block, shared = dynamic.geometry(4)
+    for rows in (0, 5, -1):
+        with pytest.raises(lib.OrxError) as err:
+            dynamic.launch_raw(grid, block, shared, 0, fake + [rows])
+        assert err.value.code == lib.ORX_ERR_ROWS
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(lib, "_lib", None)
+    monkeypatch.setattr(lib, "LIBRARY_PATH", tmp_path / "liborx.so")
+    with pytest.raises(FileNotFoundError):
+        lib.Kernel("swiglu", I=128)
+
+
+def test_package_codebook_matches_oracle(golden_basis):
+    assert np.array_equal(codebook.basis(), golden_basis)
+    assert np.array_equal(codebook.selector_table(codebook.basis()), ref.selector_table(ref.basis()))
+    book = codebook.book()
+    assert book.shape == (256, 1) and book.dtype == np.uint32
+    rng = np.random.default_rng(5)
+    q4 = rng.integers(0, 2**32, size=(48, 32), dtype=np.uint32)            # N=48, K=256
+    assert np.array_equal(codebook.q4_to_k_major(q4), ref.q4_pack_k(q4, 128))
+    q2 = rng.integers(0, 2**16, size=(3, 32, 32), dtype=np.uint16)          # E=3, N=32, K=256
+    assert np.array_equal(codebook.q2_to_k_major(q2), np.stack([ref.q2_pack_k128(e) for e in q2]))
+
+
+def test_workload_sizes_and_algorithmic_bytes():
+    # N*K/2 + 2N + M*K + 2M + 2*M*N + 1024 (Q4) and N*K + 2N + M*K + 2M + 2*M*N (W8)
+    assert workloads.algorithmic_bytes_q4(1, 9728, 2560) == 12_494_338
+    assert workloads.algorithmic_bytes_q4(1, 17408, 5120) == 44_640_258
+    assert workloads.algorithmic_bytes_w8(8192, 4096, 4096) == 117_465_088
+    assert workloads.algorithmic_ops(8192, 4096, 4096) == 2 * 8192 * 4096 * 4096
+    case = workloads.config0()
+    assert case["packed"].shape == (9728, 320) and case["packed"].dtype == np.uint32
+    assert case["x"].shape == (1, 2560) and case["x"].dtype == np.float16 and case["scales"].shape == (9728,)
+    again = workloads.config0()
+    assert np.array_equal(case["packed"], again["packed"]) and np.array_equal(case["x"], again["x"])
+    small = workloads.config1(8, n=256, k=256)
+    assert small["x"].shape == (8, 256) and np.array_equal(small["packed"], workloads.config1(1, n=256, k=256)["packed"])
