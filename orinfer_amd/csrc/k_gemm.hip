@@ -420,6 +420,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         } else {
             if (f->algorithm == kGemv && f->capacity > 4) return gemv_configure(f, codec, passes);  // reports the error
             f->block_m = probe.block_m;
+            f->slots = probe.slots;  // ring depth of the replicated-table gemv, 0 = compact tables
         }
     }
     f->geometry = projection_geometry;

@@ -253,6 +253,258 @@ __global__ __launch_bounds__(kThreads) void gemv_rowmajor_kernel(
     }
 }
 
+// ---- bank-replicated tables -----------------------------------------------------------------
+// The two lookups per code are random reads of 1 KiB tables: 64 lanes collide in the LDS banks
+// and the lookups, not HBM, bound the kernel above.  This variant stores every table entry once
+// per lane column (entry i of lane l at byte i*256 + l*4), so lane l only ever touches bank l and
+// every lookup is conflict-free.  Two tables take 128 KiB; a 16-wave workgroup owns a whole CU,
+// stays resident and walks its rows wave by wave (wave g takes row tasks g, g + waves, ...), which
+// spreads a ragged tail evenly over the CUs.  The lookup address is one v_perm_b32: byte 0 and
+// byte 2 come from the lane's column address, byte 1 is the code byte.  That needs the tables at
+// LDS byte 0 and 65536, so the kernel uses dynamic LDS only (no static LDS ahead of it).
+constexpr uint32_t kMskBase = 65536u, kBankedPlanes = 131072u;
+constexpr int kBankedThreads = 1024;
+typedef __attribute__((address_space(3))) const uint32_t lds_word;
+
+// Sum over the 64 lanes with data-parallel-primitive moves only (no LDS traffic); the total lands
+// in lane 63.  Quad swaps, half-row and row mirrors give every lane its row's sum, the two
+// broadcasts carry row sums across rows.
+__device__ __forceinline__ int wave_sum_to_last_lane(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);  // row_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false); // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ uint32_t banked_lookup(uint32_t code, uint32_t column, uint32_t selector) {
+    const uint32_t address = __builtin_amdgcn_perm(code, column, selector);
+    return *reinterpret_cast<lds_word*>(address);
+}
+// selectors: result byte 0 = column byte 0, byte 1 = code byte k, byte 2 = column byte 2 (mask
+// table, base 65536) or zero (basis table, base 0), byte 3 = zero
+constexpr uint32_t kSelNib1 = 0x0C0C0500u, kSelNib3 = 0x0C0C0700u, kSelMsk0 = 0x0C020400u, kSelMsk2 = 0x0C020600u;
+
+// Activations are split differently from the kernel above: a = 16*hi + lo with both nibbles
+// signed, hi = (a + 8) >> 4 and lo = the two's complement low nibble.  That needs no bias term
+// (no third dot product per code), but hi reaches +8 for a >= 120, which a signed nibble reads
+// as -8.  Those few positions (the row maximum and values within 6 % of it) are marked in a
+// third plane, ov = 1, worth 256 each; a chunk whose 32 activations hold such a value is flagged
+// per lane and step, and only flagged chunks pay for the extra dot products.
+//
+// LDS (dynamic only): [0,64K) basis words, [64K,128K) mask words, then the activation planes
+// (hi, lo, ov; MR x K/8 words each), the compact 256-entry tables used to fill the big ones,
+// sums[4] and the per-lane-column overflow flags (one bit per step, 64 steps at most).
+// LPR lanes share one output row (64/LPR rows per wave task); D is the depth of the per-lane
+// ring of 16-byte chunks.  Two-stage Q4 only.
+template <int CODEC, int MR, int D, int LPR>
+__global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
+    const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
+    const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
+    int m, int out_f32) {
+    extern __shared__ __align__(16) uint32_t lds[];
+    constexpr int kRows = 64 / LPR;  // rows per wave task
+    const int groups = k / 8;
+    uint32_t* planes = lds + kBankedPlanes / 4;
+    static_assert(CODEC == kQ4, "the replicated-table kernel decodes two-stage codes");
+    uint32_t* compact = planes + 3 * MR * groups;  // nib[256], msk[256]
+    int* sums = reinterpret_cast<int*>(compact + 512);
+    uint32_t* flags = compact + 512 + 4;  // [LPR][2]: bit s of a column = its chunk of step s holds an overflow
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int sub = lane & (LPR - 1);
+    const int row_in_wave = lane / LPR;
+    const int row_bytes = CODEC == kQ4 ? k / 2 : k / 4;
+    const int chunks = row_bytes / 16;
+    const int steps = chunks / LPR;              // the host guarantees chunks % LPR == 0
+    const int padded = (steps + D - 1) / D * D;  // ring refills happen in whole groups of D
+    const int tasks = (n + kRows - 1) / kRows;
+    const int task_stride = gridDim.x * (kBankedThreads / 64);
+    // Wave-uniform values are kept in scalar registers so that a stream address is a scalar base
+    // plus one 32-bit lane offset: no vector arithmetic per load.
+    const int first_task = __builtin_amdgcn_readfirstlane(wave) * gridDim.x + blockIdx.x;
+    const char* stream = reinterpret_cast<const char*>(w);
+    auto base_of = [&](int task) { return stream + (size_t)min(task, tasks - 1) * kRows * row_bytes; };
+    auto lane_offset = [&](int task) {  // rows past the end re-read the task's first row and are not stored
+        const int row = min(task, tasks - 1) * kRows + row_in_wave;
+        return (uint32_t)((row < n ? row_in_wave : 0) * row_bytes + sub * 16);
+    };
+    auto fetch = [&](const char* base, uint32_t offset, int step) {
+        return *reinterpret_cast<const uint4*>(base + (size_t)min(step, steps - 1) * (LPR * 16) + offset);
+    };
+    uint4 ring[D];
+
+    // ---- setup ----
+    // Every global read is issued before anything waits: scales, selector word, this thread's
+    // activation groups, then the first chunks of the bulk stream.  The memory counter retires in
+    // order, so the small reads can be waited for without waiting for the stream behind them.
+    uint32_t* hi = planes;
+    uint32_t* lo = planes + MR * groups;
+    uint32_t* ov = planes + 2 * MR * groups;
+    unsigned short as_bits[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r) as_bits[r] = reinterpret_cast<const unsigned short*>(as)[min(r, m - 1)];
+    uint32_t selector = book[tid & 255];
+    uint2 raw[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
+        raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
+    {
+        const char* base = base_of(first_task);
+        const uint32_t offset = lane_offset(first_task);
+#pragma unroll
+        for (int d = 0; d < D; ++d) ring[d] = fetch(base, offset, d);
+    }
+    // The mask table needs no load: it is built and replicated while the reads are in flight.
+    if (tid < 4) sums[tid] = 0;
+    if (tid < 2 * LPR + 2) flags[tid] = 0;  // per column, then the union over columns
+    if (tid < 256) compact[256 + tid] = nibble_mask_word((uint32_t)tid);
+    __syncthreads();
+    // replicate: consecutive lanes write consecutive 16-byte pieces (conflict-free); 64 words per
+    // entry, so a piece never straddles two entries
+    for (int piece = tid; piece < 4096; piece += kBankedThreads) {
+        const uint32_t value = compact[256 + (piece >> 4)];
+        reinterpret_cast<uint4*>(lds)[4096 + piece] = make_uint4(value, value, value, value);
+    }
+    // First use of a loaded value.  The empty statements pin that use here: without them the
+    // compiler computes the basis words ahead of the mask table and waits for the read at once.
+    asm volatile("" : "+v"(selector));
+#pragma unroll
+    for (int r = 0; r < MR; ++r) asm volatile("" : "+v"(raw[r].x), "+v"(raw[r].y));
+    if (tid < 256) compact[tid] = nibble_basis_word(selector, 0u);
+    auto add_groups = [&](const uint2 (&v)[MR], int g) {
+        uint32_t any_overflow = 0;
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            const bool live = r < m && g < groups;
+            const uint32_t x = live ? v[r].x : 0u, y = live ? v[r].y : 0u;
+            // bytewise a + 8 (no carry between bytes); its high nibble is hi
+            const uint32_t x8 = ((x & 0x7F7F7F7Fu) + 0x08080808u) ^ (x & 0x80808080u);
+            const uint32_t y8 = ((y & 0x7F7F7F7Fu) + 0x08080808u) ^ (y & 0x80808080u);
+            // bit 7 of a byte set iff 120 <= a <= 127, i.e. (a & 0xF8) == 0x78
+            const uint32_t xd = (x ^ 0x78787878u) & 0xF8F8F8F8u, yd = (y ^ 0x78787878u) & 0xF8F8F8F8u;
+            const uint32_t xo = ~(((xd & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | xd) & 0x80808080u;
+            const uint32_t yo = ~(((yd & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | yd) & 0x80808080u;
+            const uint32_t over = (xo >> 7) | (yo >> 3);
+            if (live) {
+                // coordinates 0..3 to even nibble slots, 4..7 to odd slots
+                hi[r * groups + g] = ((x8 >> 4) & 0x0F0F0F0Fu) | (y8 & 0xF0F0F0F0u);
+                lo[r * groups + g] = (x & 0x0F0F0F0Fu) | ((y << 4) & 0xF0F0F0F0u);
+                ov[r * groups + g] = over;
+            }
+            any_overflow |= over;
+            const int total = wave_sum_to_last_lane(sdot4(x, 0x01010101u, sdot4(y, 0x01010101u, 0)));
+            if (lane == 63 && total != 0) atomicAdd(&sums[r], total);
+        }
+        if (any_overflow) {  // rare: a handful of groups per activation row
+            const int chunk = g >> 2, step = chunk / LPR;
+            atomicOr(&flags[2 * (chunk % LPR) + (step >> 5)], 1u << (step & 31));
+            atomicOr(&flags[2 * LPR + (step >> 5)], 1u << (step & 31));
+        }
+    };
+    if (__builtin_amdgcn_readfirstlane(wave) * 64 < groups) add_groups(raw, tid);  // waves past the row have nothing to add
+    __syncthreads();
+    for (int piece = tid; piece < 4096; piece += kBankedThreads) {
+        const uint32_t value = compact[piece >> 4];
+        reinterpret_cast<uint4*>(lds)[piece] = make_uint4(value, value, value, value);
+    }
+    for (int g = kBankedThreads + tid; g - lane < groups; g += kBankedThreads) {  // K > 8192 only; wave-uniform trip count
+        uint2 more[MR];
+#pragma unroll
+        for (int r = 0; r < MR; ++r)
+            more[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(g, groups - 1));
+        add_groups(more, g);
+    }
+    __syncthreads();
+
+    const uint32_t column = kMskBase + 4u * (uint32_t)lane;
+    const uint64_t flagged = (uint64_t)flags[2 * sub] | (uint64_t)flags[2 * sub + 1] << 32;
+    const uint64_t any_flagged = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)flags[2 * LPR]) |
+                                 (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)flags[2 * LPR + 1]) << 32;
+    int acc_h0[MR], acc_l0[MR], acc_h1[MR], acc_l1[MR], acc_o0[MR], acc_o1[MR];
+    // One 16-byte chunk = 4 codes (coarse code in the low half, residual code in the high half) of
+    // 8 weights each, against every activation row.
+    auto consume = [&](const uint4& cur, int j, int step) {
+        const uint32_t word[4] = {cur.x, cur.y, cur.z, cur.w};
+        uint32_t v0[4], v1[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v0[i] = banked_lookup(word[i], column, kSelNib1) ^ banked_lookup(word[i], column, kSelMsk0);
+            v1[i] = banked_lookup(word[i], column, kSelNib3) ^ banked_lookup(word[i], column, kSelMsk2);
+        }
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            const uint4 ph = *reinterpret_cast<const uint4*>(planes + r * groups + 4 * j);
+            const uint4 pl = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 4 * j);
+            const uint32_t h[4] = {ph.x, ph.y, ph.z, ph.w}, l[4] = {pl.x, pl.y, pl.z, pl.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc_h0[r] = sdot8(v0[i], h[i], acc_h0[r]);
+                acc_l0[r] = sdot8(v0[i], l[i], acc_l0[r]);
+                acc_h1[r] = sdot8(v1[i], h[i], acc_h1[r]);
+                acc_l1[r] = sdot8(v1[i], l[i], acc_l1[r]);
+            }
+        }
+        if ((any_flagged >> step) & 1)  // scalar test first: almost every step skips the vector one
+            if ((flagged >> step) & 1) {
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                const uint4 po = *reinterpret_cast<const uint4*>(planes + (2 * MR + r) * groups + 4 * j);
+                const uint32_t o[4] = {po.x, po.y, po.z, po.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc_o0[r] = sdot8(v0[i], o[i], acc_o0[r]);
+                    acc_o1[r] = sdot8(v1[i], o[i], acc_o1[r]);
+                }
+            }
+        }
+    };
+
+    for (int task = first_task; task < tasks; task += task_stride) {
+        const int row = task * kRows + row_in_wave;
+        const bool live = row < n;
+        const char* base = base_of(task);
+        const char* next_base = base_of(task + task_stride);
+        const uint32_t offset = lane_offset(task), next_offset = lane_offset(task + task_stride);
+        // older than this row's refills, so it has landed long before the epilogue reads it
+        const unsigned short ws_bits = reinterpret_cast<const unsigned short*>(ws)[min(row, n - 1)];
+#pragma unroll
+        for (int r = 0; r < MR; ++r) acc_h0[r] = acc_l0[r] = acc_h1[r] = acc_l1[r] = acc_o0[r] = acc_o1[r] = 0;
+        for (int group = 0; group < padded; group += D) {
+            // the last group of a row refills the ring with the first chunks of the wave's next row
+            const bool last = group + D >= padded;
+            const char* refill = last ? next_base : base;
+            const uint32_t refill_offset = last ? next_offset : offset;
+            const int refill_step = last ? 0 : group + D;
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                // consume, then refill the same registers: a refill issued first would need a
+                // second set of registers and a copy per group
+                if (group + d < steps) consume(ring[d], sub + (group + d) * LPR, group + d);
+                ring[d] = fetch(refill, refill_offset, refill_step + d);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+            // w = 4*q0 + q1 = 8*v0 + 2*v1 + 5 and a = 16*hi + lo + 256*ov
+            int total = 8 * (16 * acc_h0[r] + acc_l0[r] + 256 * acc_o0[r]) + 2 * (16 * acc_h1[r] + acc_l1[r] + 256 * acc_o1[r]);
+#pragma unroll
+            for (int offset = LPR / 2; offset > 0; offset >>= 1) total += __shfl_xor(total, offset, 64);
+            if (live && sub == 0 && r < m) {
+                total += 5 * sums[r];
+                const float value = rescale(total, __half2float(__ushort_as_half(ws_bits)),
+                                            __half2float(__ushort_as_half(as_bits[r])));
+                if (out_f32)
+                    reinterpret_cast<float*>(out)[(int64_t)r * stride + row] = value;
+                else
+                    reinterpret_cast<__half*>(out)[(int64_t)r * stride + row] = __float2half_rn(value);
+            }
+        }
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------
 // slots: N, K, stride, capacity, block_m (= passes), flags (= codec), out_f32
 int device_cus() {
@@ -274,11 +526,65 @@ uint32_t gemv_lds_bytes(const orx_function& f, int mr) {
 
 int mr_for(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : 4; }
 
+// The bank-replicated variant is chosen per launch: it needs its planes to fit beside the 128 KiB
+// of tables, so a variant can run it for 1 row and the compact kernel for 4.  f.slots packs its
+// shape: ring depth | lanes per row << 8 (0 = compact-table kernel only).
+constexpr uint32_t kLdsLimit = 160 * 1024 - 4096;
+uint32_t banked_lds_bytes(const orx_function& f, int mr) {
+    return kBankedPlanes + (uint32_t)mr * (f.K / 8) * 12 + 2048 + 16 + 2 * 32 * 4;  // tables, 3 planes, compact, sums, flags
+}
+bool use_banked(const orx_function& f, int mr) {
+    return f.slots > 0 && f.flags == kQ4 && banked_lds_bytes(f, mr) <= kLdsLimit;
+}
+
 int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
+    const int mr = mr_for(rows);
+    if (use_banked(f, mr)) {
+        const uint32_t lanes_per_row = (uint32_t)f.slots >> 8;
+        const uint32_t tasks = ceil_div((uint32_t)f.N, 64u / lanes_per_row);
+        g->grid[0] = std::min<uint32_t>((uint32_t)device_cus(), ceil_div(tasks, (uint32_t)(kBankedThreads / 64)));
+        g->block[0] = kBankedThreads;
+        g->shared = banked_lds_bytes(f, mr);
+        return ORX_OK;
+    }
     g->grid[0] = ceil_div((uint32_t)f.N, (uint32_t)(kRowsPerPass * f.block_m));
     g->block[0] = kThreads;
-    g->shared = gemv_lds_bytes(f, mr_for(rows));
+    g->shared = gemv_lds_bytes(f, mr);
     return ORX_OK;
+}
+
+template <int D, int LPR>
+int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
+                       const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
+    const dim3 grid(g.grid[0]), block(kBankedThreads);
+    switch (mr_for(rows)) {
+        case 1:
+            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
+                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            break;
+        case 2:
+            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 2, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
+                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            break;
+        default:
+            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 4, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
+                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            break;
+    }
+    return hip_check(hipGetLastError(), "launch projection (gemv, replicated tables)");
+}
+
+template <int LPR>
+int gemv_launch_banked_depth(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
+                             const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
+    switch (f.slots & 255) {
+        case 2: return gemv_launch_banked<2, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+        case 3: return gemv_launch_banked<3, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+        case 4: return gemv_launch_banked<4, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+        case 5: return gemv_launch_banked<5, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+        case 10: return gemv_launch_banked<10, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+        default: return gemv_launch_banked<6, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
+    }
 }
 
 template <int CODEC>
@@ -286,6 +592,12 @@ int gemv_launch_codec(const orx_function& f, int rows, const Geometry& g, hipStr
                       const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
     const dim3 grid(g.grid[0]), block(kThreads);
     const uint4* wp = reinterpret_cast<const uint4*>(w);
+    if constexpr (CODEC == kQ4) {
+        if (use_banked(f, mr_for(rows))) {
+            if ((f.slots >> 8) == 32) return gemv_launch_banked_depth<32>(f, rows, g, stream, a, wp, book, ws, as, out);
+            return gemv_launch_banked_depth<16>(f, rows, g, stream, a, wp, book, ws, as, out);
+        }
+    }
     switch (mr_for(rows)) {
         case 1:
             hipLaunchKernelGGL((gemv_rowmajor_kernel<CODEC, 1>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
@@ -342,7 +654,26 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
         if (passes > 8) passes = 8;
     }
     f->block_m = passes;
-    if (gemv_lds_bytes(*f, 4) > 160 * 1024 - 4096) {
+    // Shape of the replicated-table kernel (0 = compact-table kernel only, which an explicit
+    // gemv_passes asks for): 32 or 16 lanes per row, whichever divides the row's chunk count (the
+    // kernel keeps its step arithmetic scalar by assuming every lane owns the same number of
+    // chunks), and the ring depth in {6,5,4} that pads a row's step count the least.
+    f->slots = 0;
+    if (passes_override <= 0 && codec == kQ4) {
+        const int chunks = f->K / 2 / 16;
+        const int lanes_per_row = chunks % 32 == 0 ? 32 : chunks % 16 == 0 ? 16 : 0;
+        if (lanes_per_row) {
+            const int steps = chunks / lanes_per_row;
+            int best_pad = 1 << 30, depth = 4;
+            for (int candidate : {6, 5, 4}) {
+                const int pad = ceil_div(steps, candidate) * candidate - steps;
+                if (pad < best_pad) best_pad = pad, depth = candidate;
+            }
+            // the overflow flags hold one bit per step in a 64-bit word per lane column
+            if (steps <= 64) f->slots = depth | lanes_per_row << 8;
+        }
+    }
+    if (gemv_lds_bytes(*f, 4) > kLdsLimit) {
         set_error("%s: K=%d does not fit the gemv activation planes in LDS", f->symbol.c_str(), f->K);
         return ORX_ERR_BAD_VARIANT;
     }
@@ -354,7 +685,7 @@ int gemv_prepare_device() {
     // Dynamic LDS above 64 KiB needs an opt-in per kernel (kernels.rs:171-190 does the same on CUDA).
     static bool done = false;
     if (done) return ORX_OK;
-    const int limit = 160 * 1024 - 4096;  // the static tables take 2064 bytes of the 160 KiB
+    const int limit = (int)kLdsLimit;  // the static tables take 2064 bytes of the 160 KiB
 #define ORX_OPT_IN(kernel)                                                                                   \
     {                                                                                                        \
         int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel),                     \
@@ -371,6 +702,15 @@ int gemv_prepare_device() {
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 1>))
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 2>))
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 4>))
+#define ORX_OPT_IN_BANKED(depth, lanes)                       \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes>))    \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 2, depth, lanes>))    \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 4, depth, lanes>))
+    ORX_OPT_IN_BANKED(4, 16) ORX_OPT_IN_BANKED(5, 16) ORX_OPT_IN_BANKED(6, 16)
+    ORX_OPT_IN_BANKED(4, 32) ORX_OPT_IN_BANKED(5, 32) ORX_OPT_IN_BANKED(6, 32)
+    ORX_OPT_IN_BANKED(10, 16) ORX_OPT_IN_BANKED(10, 32)
+    ORX_OPT_IN_BANKED(2, 16) ORX_OPT_IN_BANKED(2, 32) ORX_OPT_IN_BANKED(3, 16) ORX_OPT_IN_BANKED(3, 32)
+#undef ORX_OPT_IN_BANKED
 #undef ORX_OPT_IN
     done = true;
     return ORX_OK;

@@ -152,6 +152,33 @@ def test_q4_gemv_matches_oracle(m, n, k):
     np.testing.assert_array_equal(gu.host(got), want)
 
 
+@pytest.mark.parametrize("variant", [{}, {"gemv_passes": 1}], ids=["replicated-tables", "compact-tables"])
+@pytest.mark.parametrize("m", [1, 2, 4])
+@pytest.mark.parametrize("pattern", ["all_max", "band", "sparse", "negative"])
+def test_q4_gemv_activation_extremes(m, pattern, variant):
+    """Activations at and around the top of the int8 range: the GEMV splits them into signed
+    nibbles, and values of 120..127 take a separate path that random data visits rarely."""
+    n, k = 193, 5120
+    rng = np.random.default_rng(orc.SEED + 77 + m)
+    if pattern == "all_max":
+        a_q = np.full((m, k), 127, np.int8)
+    elif pattern == "band":                       # every boundary value, many times
+        a_q = rng.choice(np.array([111, 112, 119, 120, 121, 126, 127, -120, -121, -127, -128, 7, 8, -8, -9, 0], np.int8),
+                         size=(m, k))
+    elif pattern == "sparse":                     # one overflow in the last chunk of the last row only
+        a_q = rng.integers(-119, 120, (m, k)).astype(np.int8)
+        a_q[m - 1, k - 1] = 124
+    else:
+        a_q = rng.integers(-128, -119, (m, k)).astype(np.int8)
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    acc = orc.int_dot(a_q, orc.q4_integers(packed, TABLE))
+    np.testing.assert_array_equal(acc, orc.int_dot_bruteforce(a_q[:, :256], orc.q4_integers(packed[:, :32], TABLE))
+                                  + orc.int_dot(a_q[:, 256:], orc.q4_integers(packed[:, 32:], TABLE)))
+    got = gu.q4_project(gu.dev(a_q), gu.dev(np.ones(m, np.float16)), gu.dev(packed), gu.dev(np.ones(n, np.float16)),
+                        dtype=torch.float32, algorithm="gemv", **variant)
+    np.testing.assert_array_equal(gu.host(got).astype(np.int64), acc.astype(np.int64))
+
+
 @pytest.mark.parametrize("packed_k", [0, 128])
 @pytest.mark.parametrize("m", [1, 7, 32, 33, 64, 65, 128, 129, 300])
 def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
