@@ -279,6 +279,17 @@ __device__ __forceinline__ int wave_sum_to_last_lane(int v) {
     return v;
 }
 
+__device__ __forceinline__ uint32_t wave_or_to_last_lane(uint32_t bits) {
+    int v = (int)bits;
+    v |= __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
+    v |= __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
+    v |= __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);
+    v |= __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);
+    v |= __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);
+    v |= __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);
+    return (uint32_t)v;
+}
+
 __device__ __forceinline__ uint32_t banked_lookup(uint32_t code, uint32_t column, uint32_t selector) {
     const uint32_t address = __builtin_amdgcn_perm(code, column, selector);
     return *reinterpret_cast<lds_word*>(address);
@@ -295,11 +306,13 @@ constexpr uint32_t kSelNib1 = 0x0C0C0500u, kSelNib3 = 0x0C0C0700u, kSelMsk0 = 0x
 // per lane and step, and only flagged chunks pay for the extra dot products.
 //
 // LDS (dynamic only): [0,64K) basis words, [64K,128K) mask words, then the activation planes
-// (hi, lo, ov; MR x K/8 words each), the compact 256-entry tables used to fill the big ones,
-// sums[4] and the per-lane-column overflow flags (one bit per step, 64 steps at most).
+// (hi, lo, ov; MR x K/8 words each), one partial activation sum per wave and row, and one flag
+// byte per chunk of a row (does it hold an overflow; 64 steps per lane at most).
 // LPR lanes share one output row (64/LPR rows per wave task); D is the depth of the per-lane
-// ring of 16-byte chunks.  Two-stage Q4 only.
-template <int CODEC, int MR, int D, int LPR>
+// ring of 16-byte chunks.  Two-stage Q4 only.  HOLD (one activation row, a row's steps equal to D):
+// a lane meets the same chunk positions in every output row, so it keeps their hi and lo words in
+// registers for the whole kernel and the main loop reads LDS for table lookups only.
+template <int CODEC, int MR, int D, int LPR, bool HOLD>
 __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
@@ -309,9 +322,8 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int groups = k / 8;
     uint32_t* planes = lds + kBankedPlanes / 4;
     static_assert(CODEC == kQ4, "the replicated-table kernel decodes two-stage codes");
-    uint32_t* compact = planes + 3 * MR * groups;  // nib[256], msk[256]
-    int* sums = reinterpret_cast<int*>(compact + 512);
-    uint32_t* flags = compact + 512 + 4;  // [LPR][2]: bit s of a column = its chunk of step s holds an overflow
+    int* wave_sums = reinterpret_cast<int*>(planes + 3 * MR * groups);          // [MR][16 waves]
+    uint8_t* chunk_flags = reinterpret_cast<uint8_t*>(wave_sums + 4 * 16);      // [chunks]: chunk holds an overflow
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int sub = lane & (LPR - 1);
@@ -336,44 +348,74 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     };
     uint4 ring[D];
 
-    // ---- setup ----
+    // ---- setup: one barrier ----
     // Every global read is issued before anything waits: scales, selector word, this thread's
     // activation groups, then the first chunks of the bulk stream.  The memory counter retires in
     // order, so the small reads can be waited for without waiting for the stream behind them.
+    // Each wave then builds its own 16 entries of both tables and its own slice of the planes;
+    // nothing is accumulated across waves with atomics, so nothing has to be cleared first and
+    // the only barrier is the one that publishes the finished tables and planes.  Waves launched
+    // early do this work while the dispatcher is still launching the rest of the workgroup.
     uint32_t* hi = planes;
     uint32_t* lo = planes + MR * groups;
     uint32_t* ov = planes + 2 * MR * groups;
     unsigned short as_bits[MR];
 #pragma unroll
     for (int r = 0; r < MR; ++r) as_bits[r] = reinterpret_cast<const unsigned short*>(as)[min(r, m - 1)];
-    uint32_t selector = book[tid & 255];
+    const int entry_in_wave = lane >> 2, quarter = lane & 3;
+    const int entry = wave * 16 + entry_in_wave;  // 16 waves x 16 entries
+    uint32_t selector = book[entry];
     uint2 raw[MR];
 #pragma unroll
     for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
         raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
-    {
-        const char* base = base_of(first_task);
-        const uint32_t offset = lane_offset(first_task);
+    // The first chunks of the stream are requested in three instalments between the setup steps
+    // rather than all at once: a workgroup's full ring is 80 KiB, and the small reads of waves
+    // that start later would queue behind it in the CU's memory pipeline.
+    const char* first_base = base_of(first_task);
+    const uint32_t first_offset = lane_offset(first_task);
+    auto prefetch = [&](int from, int to) {
 #pragma unroll
-        for (int d = 0; d < D; ++d) ring[d] = fetch(base, offset, d);
-    }
-    // The mask table needs no load: it is built and replicated while the reads are in flight.
-    if (tid < 4) sums[tid] = 0;
-    if (tid < 2 * LPR + 2) flags[tid] = 0;  // per column, then the union over columns
-    if (tid < 256) compact[256 + tid] = nibble_mask_word((uint32_t)tid);
-    __syncthreads();
-    // replicate: consecutive lanes write consecutive 16-byte pieces (conflict-free); 64 words per
-    // entry, so a piece never straddles two entries
-    for (int piece = tid; piece < 4096; piece += kBankedThreads) {
-        const uint32_t value = compact[256 + (piece >> 4)];
-        reinterpret_cast<uint4*>(lds)[4096 + piece] = make_uint4(value, value, value, value);
+        for (int d = 0; d < D; ++d)
+            if (d >= from && d < to) ring[d] = fetch(first_base, first_offset, d);
+    };
+    // Lane `quarter` of a quad makes byte `quarter` of the entry's word (coordinates quarter and
+    // quarter + 4 share that byte); two quad swaps OR the four bytes together.  Every lane then
+    // writes four of the entry's sixteen 16-byte pieces, rotated by the entry so that the 64
+    // lanes of one write spread over all banks.
+    auto quad_or = [](uint32_t v) {
+        v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);
+        v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);
+        return v;
+    };
+    auto replicate = [&](uint32_t table_byte_base, uint32_t value) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t piece = (uint32_t)(entry_in_wave + 4 * quarter + i) & 15u;
+            *reinterpret_cast<uint4*>(reinterpret_cast<char*>(lds) + table_byte_base + entry * 256 + piece * 16) =
+                make_uint4(value, value, value, value);
+        }
+    };
+    {   // mask table: needs no load, built while the reads are in flight
+        const uint32_t u = (uint32_t)entry;
+        const uint32_t parity = __popc(u) & 1u, flips = u ^ parity;
+        const uint32_t low = (sign_bit(flips, quarter) ? 0xEu : 0u) ^ parity;
+        const uint32_t high = (sign_bit(flips, quarter + 4) ? 0xEu : 0u) ^ parity;
+        replicate(kMskBase, quad_or((low | high << 4) << (8 * quarter)));
     }
     // First use of a loaded value.  The empty statements pin that use here: without them the
-    // compiler computes the basis words ahead of the mask table and waits for the read at once.
+    // compiler schedules the basis words ahead of the mask table and waits for the read at once.
     asm volatile("" : "+v"(selector));
 #pragma unroll
     for (int r = 0; r < MR; ++r) asm volatile("" : "+v"(raw[r].x), "+v"(raw[r].y));
-    if (tid < 256) compact[tid] = nibble_basis_word(selector, 0u);
+    {
+        const uint32_t low = (uint32_t)selector_half(selector, quarter) & 15u;
+        const uint32_t high = (uint32_t)selector_half(selector, quarter + 4) & 15u;
+        replicate(0u, quad_or((low | high << 4) << (8 * quarter)));
+    }
+    int wave_total[MR];  // sum of this wave's activations, valid in lane 63
+#pragma unroll
+    for (int r = 0; r < MR; ++r) wave_total[r] = 0;
     auto add_groups = [&](const uint2 (&v)[MR], int g) {
         uint32_t any_overflow = 0;
 #pragma unroll
@@ -395,38 +437,57 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
                 ov[r * groups + g] = over;
             }
             any_overflow |= over;
-            const int total = wave_sum_to_last_lane(sdot4(x, 0x01010101u, sdot4(y, 0x01010101u, 0)));
-            if (lane == 63 && total != 0) atomicAdd(&sums[r], total);
+            wave_total[r] += wave_sum_to_last_lane(sdot4(x, 0x01010101u, sdot4(y, 0x01010101u, 0)));
         }
-        if (any_overflow) {  // rare: a handful of groups per activation row
-            const int chunk = g >> 2, step = chunk / LPR;
-            atomicOr(&flags[2 * (chunk % LPR) + (step >> 5)], 1u << (step & 31));
-            atomicOr(&flags[2 * LPR + (step >> 5)], 1u << (step & 31));
-        }
+        // one byte per chunk (4 groups = one quad of threads): does it hold an overflow?
+        any_overflow = quad_or(any_overflow);
+        if (quarter == 0 && g < groups) chunk_flags[g >> 2] = any_overflow ? 1 : 0;
     };
-    if (__builtin_amdgcn_readfirstlane(wave) * 64 < groups) add_groups(raw, tid);  // waves past the row have nothing to add
-    __syncthreads();
-    for (int piece = tid; piece < 4096; piece += kBankedThreads) {
-        const uint32_t value = compact[piece >> 4];
-        reinterpret_cast<uint4*>(lds)[piece] = make_uint4(value, value, value, value);
-    }
-    for (int g = kBankedThreads + tid; g - lane < groups; g += kBankedThreads) {  // K > 8192 only; wave-uniform trip count
+    // wave-uniform trip count; the first pass uses the groups read above, longer rows (K > 8192) loop
+    if (__builtin_amdgcn_readfirstlane(wave) * 64 < groups) add_groups(raw, tid);
+    for (int g = kBankedThreads + tid; g - lane < groups; g += kBankedThreads) {
         uint2 more[MR];
 #pragma unroll
         for (int r = 0; r < MR; ++r)
             more[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(g, groups - 1));
         add_groups(more, g);
     }
+    if (lane == 63) {
+#pragma unroll
+        for (int r = 0; r < MR; ++r) wave_sums[r * 16 + wave] = wave_total[r];
+    }
+    prefetch(0, 1);
     __syncthreads();
+    prefetch(1, D);
 
     const uint32_t column = kMskBase + 4u * (uint32_t)lane;
-    const uint64_t flagged = (uint64_t)flags[2 * sub] | (uint64_t)flags[2 * sub + 1] << 32;
-    const uint64_t any_flagged = (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)flags[2 * LPR]) |
-                                 (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)flags[2 * LPR + 1]) << 32;
+    // sum of each activation row (scalar), the steps at which this lane's column holds an
+    // overflow, and (scalar) the steps at which any column of the wave does
+    int row_sum[MR];
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+        row_sum[r] = __builtin_amdgcn_readlane(wave_sum_to_last_lane(lane < 16 ? wave_sums[r * 16 + lane] : 0), 63);
+    uint32_t flag_lo = 0, flag_hi = 0;
+    for (int step = 0; step < steps; ++step) {
+        const uint32_t bit = chunk_flags[sub + step * LPR];
+        if (step < 32) flag_lo |= bit << step; else flag_hi |= bit << (step - 32);
+    }
+    const uint64_t flagged = (uint64_t)flag_lo | (uint64_t)flag_hi << 32;
+    const uint64_t any_flagged = (uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)wave_or_to_last_lane(flag_lo), 63) |
+                                 (uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)wave_or_to_last_lane(flag_hi), 63) << 32;
     int acc_h0[MR], acc_l0[MR], acc_h1[MR], acc_l1[MR], acc_o0[MR], acc_o1[MR];
+    static_assert(!HOLD || MR == 1, "held planes are for a single activation row");
+    uint4 held_h[HOLD ? D : 1], held_l[HOLD ? D : 1];
+    if (HOLD) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            held_h[d] = *reinterpret_cast<const uint4*>(planes + 4 * (sub + d * LPR));
+            held_l[d] = *reinterpret_cast<const uint4*>(planes + groups + 4 * (sub + d * LPR));
+        }
+    }
     // One 16-byte chunk = 4 codes (coarse code in the low half, residual code in the high half) of
-    // 8 weights each, against every activation row.
-    auto consume = [&](const uint4& cur, int j, int step) {
+    // 8 weights each, against every activation row.  `slot` is the chunk's ring slot.
+    auto consume = [&](const uint4& cur, int j, int step, int slot) {
         const uint32_t word[4] = {cur.x, cur.y, cur.z, cur.w};
         uint32_t v0[4], v1[4];
 #pragma unroll
@@ -436,8 +497,8 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
         }
 #pragma unroll
         for (int r = 0; r < MR; ++r) {
-            const uint4 ph = *reinterpret_cast<const uint4*>(planes + r * groups + 4 * j);
-            const uint4 pl = *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 4 * j);
+            const uint4 ph = HOLD ? held_h[slot] : *reinterpret_cast<const uint4*>(planes + r * groups + 4 * j);
+            const uint4 pl = HOLD ? held_l[slot] : *reinterpret_cast<const uint4*>(planes + (MR + r) * groups + 4 * j);
             const uint32_t h[4] = {ph.x, ph.y, ph.z, ph.w}, l[4] = {pl.x, pl.y, pl.z, pl.w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -482,7 +543,7 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
             for (int d = 0; d < D; ++d) {
                 // consume, then refill the same registers: a refill issued first would need a
                 // second set of registers and a copy per group
-                if (group + d < steps) consume(ring[d], sub + (group + d) * LPR, group + d);
+                if (group + d < steps) consume(ring[d], sub + (group + d) * LPR, group + d, d);
                 ring[d] = fetch(refill, refill_offset, refill_step + d);
             }
         }
@@ -493,7 +554,7 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
             for (int offset = LPR / 2; offset > 0; offset >>= 1) total += __shfl_xor(total, offset, 64);
             if (live && sub == 0 && r < m) {
-                total += 5 * sums[r];
+                total += 5 * row_sum[r];
                 const float value = rescale(total, __half2float(__ushort_as_half(ws_bits)),
                                             __half2float(__ushort_as_half(as_bits[r])));
                 if (out_f32)
@@ -529,12 +590,14 @@ int mr_for(int rows) { return rows <= 1 ? 1 : rows <= 2 ? 2 : 4; }
 // The bank-replicated variant is chosen per launch: it needs its planes to fit beside the 128 KiB
 // of tables, so a variant can run it for 1 row and the compact kernel for 4.  f.slots packs its
 // shape: ring depth | lanes per row << 8 (0 = compact-table kernel only).
-constexpr uint32_t kLdsLimit = 160 * 1024 - 4096;
+constexpr uint32_t kLdsLimit = 160 * 1024 - 4096;   // compact-table kernel: its static tables take part of the 160 KiB
+constexpr uint32_t kBankedLdsLimit = 160 * 1024;    // replicated-table kernel: dynamic LDS only
 uint32_t banked_lds_bytes(const orx_function& f, int mr) {
-    return kBankedPlanes + (uint32_t)mr * (f.K / 8) * 12 + 2048 + 16 + 2 * 32 * 4;  // tables, 3 planes, compact, sums, flags
+    // tables, 3 planes, wave sums, one flag byte per chunk (rounded up to 16)
+    return kBankedPlanes + (uint32_t)mr * (f.K / 8) * 12 + 4 * 16 * 4 + (((uint32_t)f.K / 32 + 15) & ~15u);
 }
 bool use_banked(const orx_function& f, int mr) {
-    return f.slots > 0 && f.flags == kQ4 && banked_lds_bytes(f, mr) <= kLdsLimit;
+    return f.slots > 0 && f.flags == kQ4 && banked_lds_bytes(f, mr) <= kBankedLdsLimit;
 }
 
 int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
@@ -557,18 +620,23 @@ template <int D, int LPR>
 int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
                        const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
     const dim3 grid(g.grid[0]), block(kBankedThreads);
+    const bool hold = f.K / 32 / LPR == D;  // a row's steps fill the ring exactly
     switch (mr_for(rows)) {
         case 1:
-            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
-                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            if (hold)
+                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            else
+                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false>), grid, block, g.shared, stream, a, w, book,
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
             break;
         case 2:
-            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 2, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
-                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 2, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
             break;
         default:
-            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 4, D, LPR>), grid, block, g.shared, stream, a, w, book, ws, as,
-                               out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 4, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
             break;
     }
     return hip_check(hipGetLastError(), "launch projection (gemv, replicated tables)");
@@ -578,11 +646,8 @@ template <int LPR>
 int gemv_launch_banked_depth(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
                              const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
     switch (f.slots & 255) {
-        case 2: return gemv_launch_banked<2, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
-        case 3: return gemv_launch_banked<3, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
         case 4: return gemv_launch_banked<4, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
         case 5: return gemv_launch_banked<5, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
-        case 10: return gemv_launch_banked<10, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
         default: return gemv_launch_banked<6, LPR>(f, rows, g, stream, a, w, book, ws, as, out);
     }
 }
@@ -685,7 +750,7 @@ int gemv_prepare_device() {
     // Dynamic LDS above 64 KiB needs an opt-in per kernel (kernels.rs:171-190 does the same on CUDA).
     static bool done = false;
     if (done) return ORX_OK;
-    const int limit = (int)kLdsLimit;  // the static tables take 2064 bytes of the 160 KiB
+    int limit = (int)kLdsLimit;  // the static tables take 2064 bytes of the 160 KiB
 #define ORX_OPT_IN(kernel)                                                                                   \
     {                                                                                                        \
         int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel),                     \
@@ -702,14 +767,14 @@ int gemv_prepare_device() {
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 1>))
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 2>))
     ORX_OPT_IN((gemv_rowmajor_kernel<kW8, 4>))
+    limit = (int)kBankedLdsLimit;
 #define ORX_OPT_IN_BANKED(depth, lanes)                       \
-    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes>))    \
-    ORX_OPT_IN((gemv_banked_kernel<kQ4, 2, depth, lanes>))    \
-    ORX_OPT_IN((gemv_banked_kernel<kQ4, 4, depth, lanes>))
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, true>))     \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, false>))    \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 2, depth, lanes, false>))    \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 4, depth, lanes, false>))
     ORX_OPT_IN_BANKED(4, 16) ORX_OPT_IN_BANKED(5, 16) ORX_OPT_IN_BANKED(6, 16)
     ORX_OPT_IN_BANKED(4, 32) ORX_OPT_IN_BANKED(5, 32) ORX_OPT_IN_BANKED(6, 32)
-    ORX_OPT_IN_BANKED(10, 16) ORX_OPT_IN_BANKED(10, 32)
-    ORX_OPT_IN_BANKED(2, 16) ORX_OPT_IN_BANKED(2, 32) ORX_OPT_IN_BANKED(3, 16) ORX_OPT_IN_BANKED(3, 32)
 #undef ORX_OPT_IN_BANKED
 #undef ORX_OPT_IN
     done = true;
