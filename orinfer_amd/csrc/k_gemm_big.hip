@@ -231,6 +231,41 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
     };
+    // W8: a wave's 2*BLOCKS_PER_WAVE load instructions per K step are threaded one by one between
+    // MFMAs and spread over three MFMA groups.  A wave cannot issue anything while a vector-memory
+    // instruction waits for a slot in the CU's memory pipeline, and eight waves that all request
+    // their 8 KiB right after the barrier queue up there for most of an MFMA group; a single
+    // request at a time leaves the wave's next MFMAs issuable almost at once.
+    constexpr int LOADS = 2 * BLOCKS_PER_WAVE;
+    constexpr int PART0 = (LOADS + 2) / 3, PART1 = (LOADS - PART0 + 1) / 2, PART2 = LOADS - PART0 - PART1;
+    static_assert(PART0 <= TM * TN / 2 && PART1 <= TM * TN / 2, "one request after every second MFMA of a group");
+    auto issue_one = [&](int id, int kt_target, int stage) {  // id < BLOCKS_PER_WAVE: activations, else weights
+        const bool weights = id >= BLOCKS_PER_WAVE;
+        const int block = wave * BLOCKS_PER_WAVE + (weights ? id - BLOCKS_PER_WAVE : id);
+        const int row = block * 8 + load_r8;
+        const int chunk = load_slot ^ swizzle(row);
+        const int source_row = weights ? col0 + min(row, cols_here - 1) : row0 + min(row, rows_here - 1);
+        direct_load_16((weights ? w8 : p.a) + (int64_t)source_row * p.k + kt_target * kStep + chunk * 16,
+                       (weights ? stage_w(stage) : stage_a(stage)) + block * 1024);
+    };
+    // Requests are unconditional: a step past the end is clamped to the last one and lands in a
+    // stage that is not read again (the epilogue waits for it before it reuses LDS), which keeps
+    // branches out of the MFMA stream.
+    auto multiply_loading = [&](int slot, int first, int count, int kt_target, int stage) {
+        kt_target = min(kt_target, k_tiles - 1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+                const int index = i * TN + j;
+                if ((index & 1) == 1 && index / 2 < count) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (!Q4) issue_one(first + index / 2, kt_target, stage);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+    };
     // Q4: the whole weight tile of step kt+2 is decoded in one piece right after MFMA group 3 of
     // step kt, into the stage the barrier of step kt has just released.  (Threading the decode
     // between the MFMAs of a group, with or without pipelined table reads, measured 20 % slower:
@@ -238,15 +273,22 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
     read_fragments(0, 0, 0);
     for (int kt = 0; kt < k_tiles; ++kt) {
         const int cur = kt & 1, nxt = cur ^ 1;
-#pragma unroll
-        for (int ks = 0; ks < 3; ++ks) {
-            read_fragments(cur, ks + 1, (ks + 1) & 1);
-            __builtin_amdgcn_sched_barrier(0);  // reads above stay ahead of the MFMAs below
-            multiply(ks & 1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // this wave's part of step kt+1, requested one step ago; the code loads issued after it
-        // (Q4, step kt+3) may stay in flight: a barrier should not wait for HBM
+        // the rest of step kt+1 (its first part went out behind the previous barrier; in step 0 this
+        // repeats part of the prologue's request for step 1, byte for byte)
+        read_fragments(cur, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);  // reads above stay ahead of the MFMAs below
+        multiply_loading(0, PART0, PART1, kt + 1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        read_fragments(cur, 2, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply_loading(1, PART0 + PART1, PART2, kt + 1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        read_fragments(cur, 3, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0);
+        __builtin_amdgcn_sched_barrier(0);
+        // this wave's part of step kt+1; the code loads issued after it (Q4, step kt+3) may stay
+        // in flight: a barrier should not wait for HBM
         if (Q4 && kt + 3 < k_tiles)
             wait_direct_loads_except<CODE_CHUNKS>();
         else
@@ -255,13 +297,8 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
         if (Q4 && kt + 2 < k_tiles) issue_direct(p.a, rows_here, row0, kt + 2, stage_a(cur));
         if (kt + 1 < k_tiles) read_fragments(nxt, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(1);
+        multiply_loading(1, 0, PART0, kt + 2, cur);
         __builtin_amdgcn_sched_barrier(0);
-        if (!Q4 && kt + 2 < k_tiles) {
-            // W8: requested behind the fragment reads so the 64 KiB burst into LDS does not delay them
-            issue_direct(p.a, rows_here, row0, kt + 2, stage_a(cur));
-            issue_direct(w8, cols_here, col0, kt + 2, stage_w(cur));
-        }
         if (Q4 && kt + 2 < k_tiles) {
             decode_step(stage_w(cur), cur);
             if (kt + 4 < k_tiles) load_codes(kt + 4, cur);
@@ -270,6 +307,9 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
     }
 
     // ---- epilogue ----
+    // the clamped requests of the last two steps may still be writing LDS (and a workgroup must
+    // not end with direct-to-LDS loads in flight)
+    if (!Q4) wait_direct_loads();
     // Weights are the MFMA row operand, so a lane holds token row (lane & 31) of each 32x32 block
     // and, per group of four accumulator registers, four CONSECUTIVE output channels
     // 8*q + 4*(lane >> 5) + {0..3}.
