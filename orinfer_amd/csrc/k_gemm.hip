@@ -36,6 +36,8 @@ int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, 
                           hipStream_t stream);
 // from k_gemm_big.hip
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g);
+int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int n, int k, int packed_k,
+                     hipStream_t stream);
 int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                     void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g,
                     hipStream_t stream);
@@ -298,6 +300,13 @@ bool use_stream(const orx_function& f, int rows) {
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
 bool use_big(const orx_function& f, int rows) { return f.tiles == 256 || (f.tiles == 0 && rows > 128); }
 
+// Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel
+// when the rows span several 256-row tiles (each tile would otherwise decode every weight again).
+constexpr int kExpandRows = 512;
+bool use_expand(const orx_function& f, int rows) {
+    return f.flags == kQ4 && f.workspace != nullptr && use_big(f, rows) && rows >= kExpandRows;
+}
+
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_stream(f, rows)) {
@@ -305,7 +314,7 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (use_big(f, rows)) {
-        gemm_big_geometry(rows, f.N, f.flags == kQ4, g);
+        gemm_big_geometry(rows, f.N, f.flags == kQ4 && !use_expand(f, rows), g);
         return ORX_OK;
     }
     const int bm = f.tiles ? f.tiles : pick_bm(rows);
@@ -330,6 +339,12 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     if (use_stream(f, rows))
         return stream_launch(kQ4, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32,
                              stream);
+    if (use_expand(f, rows)) {
+        const int code = q4_expand_launch(p.w, p.book, f.workspace, f.N, f.K, f.packed_k, stream);
+        if (code != ORX_OK) return code;
+        return gemm_big_launch(false, p.a, f.workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0,
+                               f.out_f32, g, stream);
+    }
     if (use_big(f, rows))
         return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
                                f.out_f32, g, stream);
@@ -431,6 +446,22 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
 int make_q4_projection(const Variant& v, orx_function* f) {
     int code = make_projection(v, f, kQ4);
     if (code != ORX_OK) return code;
+    // Scratch for the decoded weights of large-row launches: allocated here, never at launch
+    // (a launch may be under graph capture).  Without a device (a build machine) or without
+    // memory the handle simply keeps decoding inside the GEMM.
+    int devices = 0;
+    const bool wants_scratch = f->capacity >= kExpandRows && (f->algorithm == kAuto || f->algorithm == kMfma) &&
+                               (f->tiles == 0 || f->tiles == 256);
+    bool bad = false;
+    const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);  // diagnostic: keep the decode inside the GEMM
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (wants_scratch && !in_gemm && hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
+        const size_t bytes = (size_t)f->N * f->K;
+        if (hipMalloc(&f->workspace, bytes) == hipSuccess)
+            f->workspace_bytes = bytes;
+        else
+            f->workspace = nullptr, (void)hipGetLastError();
+    }
     f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4},
                {"Out", ArgPointer, 2}, {"S", ArgPointer, 2},  {"W", ArgPointer, 16}};
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
@@ -573,7 +604,7 @@ const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, packed_k=0|128, output_dtype=float16|float32, "
-     "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0",
+     "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0, decode_in_gemm=false",
      "A,AS,Book,Out,S,W[,m]"},
     {"int8_projection", make_w8_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "

@@ -428,6 +428,46 @@ int prepare() {
 
 }  // namespace
 
+// ---- two-stage codes -> int8 weights, once per launch ------------------------------------------
+// A prefill GEMM decodes every weight tile once per 256-row tile of activations; with many row
+// tiles it is cheaper to decode the whole matrix once into scratch (1.5 bytes of HBM traffic per
+// weight) and run the plain int8 kernel on it.  One thread turns 16 bytes of codes (4 codes, 32
+// weights) into 32 consecutive bytes of a row-major (N, K) int8 matrix.
+namespace {
+__global__ __launch_bounds__(512) void q4_expand_kernel(const uint4* __restrict__ codes, const uint32_t* __restrict__ book,
+                                                        int8_t* __restrict__ out, int n, int k, int packed_k) {
+    __shared__ Q4ByteTables tables;
+    build_tables(tables, book, threadIdx.x, 512);
+    __syncthreads();
+    const int64_t total = (int64_t)n * (k / 32);
+    const int per_row = k / 32;
+    for (int64_t c = (int64_t)blockIdx.x * 512 + threadIdx.x; c < total; c += (int64_t)gridDim.x * 512) {
+        int64_t row, k0;
+        if (packed_k == 128) {  // (K/128, N, 16) u32: four chunks per row and K block
+            const int64_t kt = c / ((int64_t)n * 4), rest = c % ((int64_t)n * 4);
+            row = rest >> 2, k0 = kt * 128 + (rest & 3) * 32;
+        } else {
+            row = c / per_row, k0 = (c % per_row) * 32;
+        }
+        const uint4 four = codes[c];
+        const uint2 w0 = decode_q4(tables, four.x), w1 = decode_q4(tables, four.y);
+        const uint2 w2 = decode_q4(tables, four.z), w3 = decode_q4(tables, four.w);
+        uint4* dst = reinterpret_cast<uint4*>(out + row * k + k0);
+        dst[0] = make_uint4(w0.x, w0.y, w1.x, w1.y);
+        dst[1] = make_uint4(w2.x, w2.y, w3.x, w3.y);
+    }
+}
+}  // namespace
+
+int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int n, int k, int packed_k,
+                     hipStream_t stream) {
+    const int64_t chunks = (int64_t)n * (k / 32);
+    const int blocks = (int)std::min<int64_t>((chunks + 511) / 512, 2048);
+    hipLaunchKernelGGL(q4_expand_kernel, dim3(blocks), dim3(512), 0, stream, reinterpret_cast<const uint4*>(codes), book,
+                       reinterpret_cast<int8_t*>(weights), n, k, packed_k);
+    return hip_check(hipGetLastError(), "launch two-stage weight expansion");
+}
+
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTile) * ceil_div((uint32_t)n, (uint32_t)kTile);
     g->grid[1] = g->grid[2] = 1;

@@ -227,6 +227,7 @@ int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
 }
 
 int orx_release(orx_fn f) {
+    if (f != nullptr && f->workspace != nullptr) (void)hipFree(f->workspace);
     delete f;
     return ORX_OK;
 }

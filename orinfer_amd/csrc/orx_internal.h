@@ -57,6 +57,11 @@ struct orx_function {
     int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0;
     bool out_f32 = false;
     const void* device_function = nullptr;  // for hipFuncGetAttributes
+    // Device scratch owned by the handle (allocated when it is resolved on a machine with a
+    // device, freed by orx_release): decoded int8 weights of a two-stage projection that serves
+    // many rows.  Launches of one handle share it, so they must not overlap on different streams.
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
     // rows -> geometry; returns ORX_OK or an error code
     int (*geometry)(const orx_function&, int rows, orx::Geometry*) = nullptr;
     // enqueue on stream; args already validated for count/alignment

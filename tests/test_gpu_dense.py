@@ -317,6 +317,49 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
+@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("decode_in_gemm", [False, True], ids=["decode-once", "decode-in-gemm"])
+def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
+    """From 512 rows on the two-stage weights are decoded once into the handle's scratch and the
+    int8 kernel runs on them; `decode_in_gemm` keeps the decode inside the GEMM.  Same bits either
+    way, also when the weights change between launches of one handle and under graph replay."""
+    rng = np.random.default_rng(orc.SEED + 31 + packed_k)
+    m, n, k = 700, 333, 640
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    other = rng.integers(0, 2**32, packed.shape, dtype=np.uint32)
+    store = (lambda p: p) if packed_k == 0 else (lambda p: orc.q4_pack_k(p, 128))
+    variant = dict(M=1024, N=n, K=k, dynamic_rows=True, output_stride=n + 3)
+    if packed_k:
+        variant["packed_k"] = packed_k
+    if decode_in_gemm:
+        variant["decode_in_gemm"] = True
+    kern = gu.lib.Kernel("e8p_q4_projection", **variant)
+    d_a, d_as, d_s, d_book = gu.dev(a_q), gu.dev(a_s), gu.dev(scales), gu.book()
+    d_w = gu.dev(store(packed))
+    out = torch.full((1024, n + 3), 7.0, dtype=torch.float16, device=gu.DEV)
+    for rows in (700, 512, 511, 3):        # 511 and 3 take the other kernels of the same handle
+        out.fill_(7.0)
+        kern(A=d_a, AS=d_as, Book=d_book, Out=out, S=d_s, W=d_w, m=rows)
+        got = gu.host(out)
+        want = orc.project(a_q[:rows], a_s[:rows], orc.q4_integers(packed, TABLE), scales)
+        np.testing.assert_array_equal(got[:rows, :n], want)
+        assert (got[rows:] == 7).all() and (got[:rows, n:] == 7).all()
+    # same handle, new weight bits in the same buffer, replayed from a graph
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            kern(stream=side.cuda_stream, A=d_a, AS=d_as, Book=d_book, Out=out, S=d_s, W=d_w, m=700)
+    for bits in (other, packed, other):
+        d_w.copy_(gu.dev(store(bits)))
+        out.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = orc.project(a_q, a_s, orc.q4_integers(bits, TABLE), scales)
+        np.testing.assert_array_equal(gu.host(out)[:700, :n], want)
+
+
 @pytest.mark.parametrize("m,n,k", [(384, 512, 4096), (1000, 777, 640)])
 def test_w8_mid_size_accumulators(m, n, k):
     rng = np.random.default_rng(orc.SEED)
