@@ -25,9 +25,9 @@ CACHE_BYTES = 256 << 20        # Infinity Cache
 # HBM bytes per launch of the contract kernel from two `rocprofv3 --pmc` runs of
 # `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
 # same counter reads for a device copy of 44 564 480 bytes in the same run: FETCH_SIZE reads
-# 21 774.8 for 43 520 KiB (factor 1.9986), WRITE_SIZE reads 43 520.0 (factor 1.0).
-# Projection: fetch 21 873.8 -> 44 767 114 B, write 34.0 -> 34 816 B.
-MEASURED_TRAFFIC_BYTES = 44_801_930
+# 21 774.9 for 43 520 KiB (factor 1.9986), WRITE_SIZE reads 43 520.0 (factor 1.0).
+# Projection: fetch 22 002.1 -> 45 029 441 B, write 272.0 -> 278 528 B.
+MEASURED_TRAFFIC_BYTES = 45_307_969
 
 
 def parse():
@@ -168,7 +168,7 @@ def main():
         "data": "synthetic (seeded uniform codes, N(0,1) activations, random-init scales)",
         "config": {"workload": "BASELINE config 1: Q4A8 linear K=5120 N=17408, M=1 decode GEMV, step = A8 + projection",
                    "weight_copies_rotated": copies, "algorithmic_bytes_per_step": bytes_c1},
-        "roofline": {"bound": "hbm", "kernel": "gemv_rowmajor_kernel<Q4,1>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": "gemv_banked_kernel<Q4, 1 row>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": MEASURED_TRAFFIC_BYTES},
     }

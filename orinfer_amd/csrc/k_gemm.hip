@@ -292,17 +292,21 @@ bool use_gemv(const orx_function& f, int rows) {
     return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
 }
 
-// weight-streaming kernel for up to 64 rows (auto), or when asked for by name
+// weight-streaming kernel for up to 64 rows when asked for by name; `auto` also serves 65..128
+// rows with it, as two launches of 64 rows (the second pass finds the weights in the last-level
+// cache and still beats a 128-row MFMA tile that stages both operands through LDS)
 bool use_stream(const orx_function& f, int rows) {
-    return rows <= 64 && (f.algorithm == kStream || (f.algorithm == kAuto && f.tiles == 0));
+    if (f.algorithm == kStream) return rows <= 64;
+    return f.algorithm == kAuto && f.tiles == 0 && rows <= 128;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
 bool use_big(const orx_function& f, int rows) { return f.tiles == 256 || (f.tiles == 0 && rows > 128); }
 
 // Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel
-// when the rows span several 256-row tiles (each tile would otherwise decode every weight again).
-constexpr int kExpandRows = 512;
+// when the rows need the 256-row MFMA tiles (every row tile would otherwise decode every weight
+// again, and even a single tile row gains: the decode leaves the MFMA loop).
+constexpr int kExpandRows = 129;
 bool use_expand(const orx_function& f, int rows) {
     return f.flags == kQ4 && f.workspace != nullptr && use_big(f, rows) && rows >= kExpandRows;
 }
@@ -336,9 +340,16 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, 5);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
-    if (use_stream(f, rows))
-        return stream_launch(kQ4, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32,
-                             stream);
+    if (use_stream(f, rows)) {
+        for (int first = 0; first < rows; first += 64) {
+            const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
+            const int code = stream_launch(kQ4, p.a + (size_t)first * f.K, p.w, p.book, p.ws, p.as + first,
+                                           static_cast<char*>(p.out) + out_offset, std::min(64, rows - first), f.N, f.K,
+                                           f.stride, f.packed_k, f.out_f32, stream);
+            if (code != ORX_OK) return code;
+        }
+        return ORX_OK;
+    }
     if (use_expand(f, rows)) {
         const int code = q4_expand_launch(p.w, p.book, f.workspace, f.N, f.K, f.packed_k, stream);
         if (code != ORX_OK) return code;
@@ -362,8 +373,16 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.book = nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = 0, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
-    if (use_stream(f, rows))
-        return stream_launch(kW8, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, stream);
+    if (use_stream(f, rows)) {
+        for (int first = 0; first < rows; first += 64) {
+            const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
+            const int code = stream_launch(kW8, p.a + (size_t)first * f.K, p.w, p.book, p.ws, p.as + first,
+                                           static_cast<char*>(p.out) + out_offset, std::min(64, rows - first), f.N, f.K,
+                                           f.stride, 0, f.out_f32, stream);
+            if (code != ORX_OK) return code;
+        }
+        return ORX_OK;
+    }
     if (use_big(f, rows))
         return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
                                stream);
