@@ -458,7 +458,10 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         }
     }
     f->geometry = projection_geometry;
-    f->device_function = reinterpret_cast<const void*>(&gemm_kernel<kW8, 128, 128, 2, false>);
+    // a projection handle launches one of several kernels depending on the live rows (1024-thread
+    // GEMV, 512-thread streaming and 256x256 kernels, 256-thread tiles): no single function's
+    // attributes describe it, so orx_query reports the device-wide limits
+    f->device_function = nullptr;
     return ORX_OK;
 }
 

@@ -35,7 +35,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTile = 256;     // output tile edge
 constexpr int kStep = 128;     // K bytes per step
-constexpr int kMaxThreads = 512;
 constexpr int kTileBytes = kTile * kStep;  // 32 KiB per operand per stage
 constexpr int kImagePitch = kTile + 8;     // halves per row of the fp16 output image (bank skew)
 constexpr int kEpilogueTile = kTile * kImagePitch * 2;  // bytes of the output image in LDS
