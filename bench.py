@@ -259,6 +259,19 @@ def main():
             del x, a, o, w
             torch.cuda.empty_cache()
         extra["config4_layer_linears_m8192"] = {"layer_us": round(layer_us, 1), "per_gemm": per}
+
+        # signed block-128 rotation fused with A8: the real producer of the int8 activations
+        rows, width = 8192, 5120
+        x = torch.randn((rows, width), dtype=torch.float16, device="cuda")
+        signs = (torch.randint(0, 2, (width,), device="cuda", dtype=torch.int8) * 2 - 1)
+        q = torch.empty((rows, width), dtype=torch.int8, device="cuda")
+        sc = torch.empty((rows,), dtype=torch.float16, device="cuda")
+        rot = Kernel("rotate_activation_a8", M=rows, K=width)
+        tr = timed_graph(lambda i, st: rot(stream=st, Q=q, S=sc, Signs=signs, X=x), 20)
+        moved = rows * width * 3 + rows * 2 + width
+        extra["rotate_a8_m8192_k5120"] = {"us": round(tr * 1e6, 2), "GBps": round(moved / tr / 1e9, 1),
+                                          "frac_hbm": round(moved / tr / 1e9 / HBM_PEAK_GBS, 4), "bytes": moved}
+        del x, q
     result["extra"] = extra
 
     # ---- CPU baseline: the numpy oracle on the contract workload (one full call) ----

@@ -17,6 +17,9 @@ Every function cites the reference file:line it follows.  Pinning status:
 * project()/rescale()    pinned by brute-force int64 dots and power-of-two KATs
 * router_topk()/metadata pinned by stable argsort / enumeration
 * swiglu(), combine()    pinned by direct formula on tiny inputs
+* rotate(), rotate_a8()  pinned by the Sylvester Hadamard matrix (exact on small
+                         integers), dot preservation and the involution of the
+                         reference's test_vq.py:123-130
 """
 
 import itertools
@@ -191,6 +194,40 @@ def swiglu_fp16(gu):
     one = np.float32(1.0)
     sig = np.where(g >= 0, one / (one + e), e / (one + e)).astype(np.float32)
     return ((g * sig) * u).astype(np.float16)
+
+
+def rotate(x, signs):
+    """Signed block-128 Hadamard rotation in fp32 (python/orinfer_build/quantization/vq.py:20-31).
+
+    y = x * signs, then seven butterfly stages h = 1, 2, .. 64 inside every block of 128
+    (left + right, left - right), then one multiply by fp32(128 ** -0.5).  Every step is a
+    single fp32 operation, so a kernel that runs the stages in the same order is bit-exact.
+    """
+    x = np.asarray(x, dtype=np.float32)
+    signs = np.asarray(signs)
+    if x.shape[-1] % 128 or signs.shape != (x.shape[-1],) or not np.isin(signs, [-1, 1]).all():
+        raise ValueError("block-128 rotation needs one +-1 sign per input channel")
+    y = (x * signs.astype(np.float32)).astype(np.float32)
+    for stage in range(7):
+        h = 1 << stage
+        block = y.reshape(*y.shape[:-1], -1, 2 * h)
+        left, right = block[..., :h].copy(), block[..., h:].copy()
+        block[..., :h], block[..., h:] = left + right, left - right
+    return (y * np.float32(128**-0.5)).astype(np.float32)
+
+
+def rotate_a8(x, signs, swiglu=False):
+    """fp16 activations -> rotated int8 codes + one fp16 scale per row.
+
+    kernels/cuda/model/rotation_a8.py:188-224 (load, optional fp16 SwiGLU boundary, signs,
+    butterflies, fp16 materialisation of the scaled result), :144-164 and :369-383 (row scale
+    and codes: the A8 rule on the materialised fp16 values; the reciprocal form there falls
+    back to the exact divide near ties, so it produces the same codes).
+    """
+    x = np.asarray(x).astype(np.float16)
+    values = swiglu_fp16(x) if swiglu else x
+    rotated = rotate(values.astype(np.float32), signs).astype(np.float16)
+    return a8(rotated)
 
 
 # --------------------------------------------------------------------------

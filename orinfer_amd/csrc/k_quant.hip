@@ -6,6 +6,11 @@
 // ties-to-even (:14-18, :49-65, contract text :71-78).  `fused` quantises
 // fp16(silu(gate)*up) read from X[rows, 2K] (:43-46, op04_swiglu.py:6-17).
 // The kernel is memory-bound: one fp16 read (twice, second pass from L2) and one int8 write.
+//
+// rotate_activation_a8 follows kernels/cuda/model/rotation_a8.py:188-224,369-383: x * sign, seven
+// butterfly stages inside every block of 128 channels in fp32, one multiply by fp32(128^-1/2), an
+// fp16 materialisation, then the same row-wise A8 rule.  Every stage is one fp32 add or subtract
+// in the order of the numpy oracle (quantization/vq.py:20-31), so codes and scales are bit-exact.
 #include <hip/hip_fp16.h>
 
 #include "orx_internal.h"
@@ -105,6 +110,79 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
     }
 }
 
+// One workgroup per row, 4 waves; a wave takes two blocks of 128 channels per step (one per half
+// wave), a lane holds 4 consecutive channels: stages 1 and 2 are local, stages 4..64 are lane
+// exchanges at distance 1..16.  The rotated fp16 row is kept in LDS for the second pass.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void rotate_a8_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                        int8_t* __restrict__ q, __half* __restrict__ s, int k) {
+    extern __shared__ __align__(16) __half rotated[];  // k halves
+    __shared__ float scratch[4];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int half_wave = lane >> 5, l32 = lane & 31;
+    const int blocks = k / 128;
+    const int64_t in_base = (int64_t)row * (SWIGLU ? 2 * k : k);
+    float amax = 0.f;
+    for (int pair = wave; 2 * pair < blocks; pair += 4) {  // wave-uniform trip count
+        const int block = 2 * pair + half_wave;
+        const bool live = block < blocks;
+        const int first = (live ? block : 0) * 128 + 4 * l32;
+        float v[4];
+        {
+            const uint2 raw = *reinterpret_cast<const uint2*>(x + in_base + first);
+            const __half* h = reinterpret_cast<const __half*>(&raw);
+            const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+            uint2 raw_up = make_uint2(0u, 0u);
+            if (SWIGLU) raw_up = *reinterpret_cast<const uint2*>(x + in_base + k + first);
+            const __half* up = reinterpret_cast<const __half*>(&raw_up);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float value = SWIGLU ? swiglu_value(h[j], up[j]) : __half2float(h[j]);
+                const float sign = (float)(int8_t)(sign_word >> (8 * j));
+                v[j] = live ? value * sign : 0.f;
+            }
+        }
+        // distance 1 and 2: inside the lane
+        {
+            const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
+            v[0] = a + c, v[2] = a - c, v[1] = b + d, v[3] = b - d;
+        }
+        // distance 4 .. 64: lanes at distance 1 .. 16; the upper element of a pair keeps left - right
+#pragma unroll
+        for (int bit = 0; bit < 5; ++bit) {
+            const bool upper = (l32 >> bit) & 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float other = __shfl_xor(v[j], 1 << bit, 64);
+                v[j] = upper ? other - v[j] : other + v[j];
+            }
+        }
+        __half out[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float scaled = v[j] * 0.08838834764831845f;
+            // opaque: the fp16 cast below must round the fp32 product, not a fused multiply-convert
+            asm volatile("" : "+v"(scaled));
+            out[j] = __float2half_rn(scaled);
+            amax = fmaxf(amax, fabsf(__half2float(out[j])));
+        }
+        if (live) *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
+    }
+    amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
+    const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
+    const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
+    if (tid == 0) s[row] = stored;
+    const float scale = __half2float(stored);
+    for (int i = tid; i < k / 4; i += 256) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
+        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = packed;
+    }
+}
+
 // fp16 [rows, 2I] -> fp16 [rows, I].  grid (rows, ceil(I/256)).
 __global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ x, __half* __restrict__ y, int width) {
     const int row = blockIdx.x;
@@ -167,6 +245,50 @@ int make_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// slots used: K, flags (bit1 swiglu), capacity
+int rotate_a8_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->block[0] = 256;
+    g->shared = (uint32_t)f.K * 2;
+    return ORX_OK;
+}
+
+// Q, S, Signs, X[, m]   (crates/orinfer-models/src/flash_next/q4.rs:176-196 binds rotation as Q, S, Signs, X)
+int rotate_a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    int8_t* q = pointer_arg<int8_t>(args, 0);
+    __half* s = pointer_arg<__half>(args, 1);
+    const int8_t* signs = pointer_arg<const int8_t>(args, 2);
+    const __half* x = pointer_arg<const __half>(args, 3);
+    if (f.flags & 2)
+        hipLaunchKernelGGL((rotate_a8_kernel<true>), dim3(g.grid[0]), dim3(256), g.shared, stream, x, signs, q, s, f.K);
+    else
+        hipLaunchKernelGGL((rotate_a8_kernel<false>), dim3(g.grid[0]), dim3(256), g.shared, stream, x, signs, q, s, f.K);
+    return hip_check(hipGetLastError(), "launch rotate_activation_a8");
+}
+
+int make_rotate_a8(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("K", 0, &bad);
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const bool swiglu = v.boolean("swiglu", false, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // rotation_a8.py:425-427: K a positive multiple of 128; the row has to fit LDS as fp16
+    if (f->M <= 0 || f->K <= 0 || f->K % 128 || f->K > 32768) {
+        set_error("rotate_activation_a8: need M > 0 and K a multiple of 128 up to 32768");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = swiglu ? 2 : 0;
+    // 8-byte loads of X, 4-byte loads of Signs and stores of Q
+    f->args = {{"Q", ArgPointer, 4}, {"S", ArgPointer, 2}, {"Signs", ArgPointer, 4}, {"X", ArgPointer, 8}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = reinterpret_cast<const void*>(&rotate_a8_kernel<false>);
+    f->geometry = rotate_a8_geometry;
+    f->launch = rotate_a8_launch;
+    return ORX_OK;
+}
+
 int swiglu_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
     g->grid[1] = ceil_div((uint32_t)f.N, 256u);
@@ -205,8 +327,9 @@ const Registration* quant_registrations(int* count) {
     {"activation_quantization", make_a8, "K, group_size=null, masked=false, fused=false, M=capacity",
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
+    {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
     };
-    *count = 2;
+    *count = 3;
     return rows;
 }
 

@@ -125,6 +125,60 @@ def test_swiglu_then_a8_and_fused_form_agree():
     assert torch.equal(q1, q2) and torch.equal(s1, s2)
 
 
+# ---- signed block-128 rotation fused with A8 -------------------------------------------------
+@pytest.mark.parametrize("m,k", [(1, 128), (3, 384), (5, 2560), (2, 5120), (1, 17408)])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_rotate_activation_a8_matches_oracle(m, k, swiglu):
+    rng = np.random.default_rng(orc.SEED + m + k)
+    x = rng.normal(size=(m, 2 * k if swiglu else k)).astype(np.float16)
+    x[0, :3] = [0, 60000, -60000] if not swiglu else [3, -2, 0]
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    want_q, want_s = orc.rotate_a8(x, signs, swiglu=swiglu)
+    variant = dict(M=m, K=k)
+    if swiglu:
+        variant["swiglu"] = True
+    q = torch.full((m + 1, k), 77, dtype=torch.int8, device=gu.DEV)
+    s = torch.full((m + 1,), 5.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("rotate_activation_a8", **variant)(Q=q, S=s, Signs=gu.dev(signs), X=gu.dev(x))
+    if swiglu:
+        # the exponential of the SwiGLU boundary may differ in the last place between libm and the
+        # device: compare the codes on the device's own fp16 SwiGLU values
+        mid = torch.empty((m, k), dtype=torch.float16, device=gu.DEV)
+        gu.kernel("swiglu", I=k)(X=gu.dev(x), Y=mid, rows=m)
+        want_q, want_s = orc.rotate_a8(gu.host(mid), signs)
+    np.testing.assert_array_equal(gu.host(s)[:m], want_s[:, 0])
+    np.testing.assert_array_equal(gu.host(q)[:m], want_q)
+    assert (gu.host(q)[m:] == 77).all() and float(gu.host(s)[m]) == 5.0
+
+
+def test_rotate_activation_a8_dynamic_rows_zero_row_and_graph():
+    rng = np.random.default_rng(orc.SEED + 12)
+    k = 1024
+    x = rng.normal(size=(9, k)).astype(np.float16)
+    x[4] = 0
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    kern = gu.kernel("rotate_activation_a8", M=16, K=k, dynamic_rows=True)
+    d_x, d_signs = gu.dev(x), gu.dev(signs)
+    q = torch.zeros((16, k), dtype=torch.int8, device=gu.DEV)
+    s = torch.zeros((16,), dtype=torch.float16, device=gu.DEV)
+    for rows in (9, 1):
+        q.fill_(9)
+        kern(Q=q, S=s, Signs=d_signs, X=d_x, m=rows)
+        want_q, want_s = orc.rotate_a8(x[:rows], signs)
+        np.testing.assert_array_equal(gu.host(q)[:rows], want_q)
+        np.testing.assert_array_equal(gu.host(s)[:rows], want_s[:, 0])
+        assert (gu.host(q)[rows:] == 9).all()
+    assert float(gu.host(s)[0]) > 0
+    kern(Q=q, S=s, Signs=d_signs, X=d_x, m=9)
+    assert not gu.host(q)[4].any() and float(gu.host(s)[4]) == 1.0
+    # rotated activations against rotated weights reproduce the un-rotated dot products
+    w = rng.normal(size=(6, k)).astype(np.float32)
+    rotated_w = orc.rotate(w, signs)
+    codes, scales = gu.host(q)[:9].astype(np.float32), gu.host(s)[:9].astype(np.float32)
+    approx = (codes * scales[:, None]) @ rotated_w.T
+    np.testing.assert_allclose(approx, x.astype(np.float32) @ w.T, atol=0.6, rtol=0.05)
+
+
 # ---- Q4A8 projections -----------------------------------------------------
 def q4_case(rng, m, n, k):
     x = (rng.normal(size=(m, k))).astype(np.float16)

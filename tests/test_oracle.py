@@ -396,3 +396,62 @@ def test_swiglu_matches_closed_form():
     gf, uf = g.astype(np.float64), u.astype(np.float64)
     np.testing.assert_allclose(got, gf / (1 + np.exp(-gf)) * uf, rtol=2e-3, atol=1e-7)
     assert got[0, 2] == 0 and abs(got[0, 4] - 40) < 0.05
+
+
+# ---- rotation (the producer of A8 activations in the real model) --------------------------------
+def test_rotate_is_the_scaled_sylvester_hadamard_and_exact_on_integers():
+    from scipy.linalg import hadamard
+    rng = np.random.default_rng(orc.SEED)
+    h = hadamard(128).astype(np.int64)
+    x = rng.integers(-64, 65, (3, 256))
+    signs = rng.choice(np.array([-1, 1], np.int8), 256)
+    got = orc.rotate(x.astype(np.float32), signs)
+    # before the final scaling every intermediate is an integer below 2**24: fp32 is exact
+    want = np.concatenate([(x * signs)[:, :128] @ h, (x * signs)[:, 128:] @ h], axis=1)
+    np.testing.assert_array_equal(got, (want.astype(np.float32) * np.float32(128**-0.5)))
+    # a transposed or mis-ordered butterfly fails on a unit vector: column 5 of H, block 1
+    e = np.zeros((1, 256), np.float32)
+    e[0, 128 + 5] = 1
+    np.testing.assert_array_equal(orc.rotate(e, np.ones(256, np.int8))[0, 128:],
+                                  h[:, 5].astype(np.float32) * np.float32(128**-0.5))
+    assert not orc.rotate(e, np.ones(256, np.int8))[0, :128].any()
+
+
+def test_rotate_preserves_dots_and_is_an_involution_up_to_signs():
+    # python/orinfer_build/quantization/test_vq.py:123-130
+    rng = np.random.default_rng(20261002)
+    x = rng.normal(size=(5, 256)).astype(np.float32)
+    w = rng.normal(size=(7, 256)).astype(np.float32)
+    s = rng.choice(np.array([-1, 1], np.int8), 256)
+    np.testing.assert_allclose(orc.rotate(x, s) @ orc.rotate(w, s).T, x @ w.T, atol=2e-5, rtol=2e-5)
+    inverse = orc.rotate(orc.rotate(x, s), np.ones(256, np.int8)) * s
+    np.testing.assert_allclose(inverse, x, atol=1e-6, rtol=1e-5)
+    with pytest.raises(ValueError):
+        orc.rotate(x[:, :100], s[:100])
+    with pytest.raises(ValueError):
+        orc.rotate(x, np.zeros(256, np.int8))
+
+
+def test_rotate_a8_quantises_the_materialised_fp16_values():
+    rng = np.random.default_rng(orc.SEED + 3)
+    x = rng.normal(size=(4, 384)).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), 384)
+    q, s = orc.rotate_a8(x, signs)
+    rotated = orc.rotate(x.astype(np.float32), signs).astype(np.float16)
+    wq, ws = orc.a8(rotated)
+    np.testing.assert_array_equal(q, wq)
+    np.testing.assert_array_equal(s, ws)
+    # a power-of-two row: one non-zero input of 2**-3 gives +-2**-3 * 128**-0.5 everywhere in its block
+    x = np.zeros((1, 128), np.float16)
+    x[0, 7] = 0.125
+    q, s = orc.rotate_a8(x, np.ones(128, np.int8))
+    assert set(np.abs(q[0]).tolist()) == {127} and s.shape == (1, 1)
+    # zero row: scale 1, codes 0
+    q, s = orc.rotate_a8(np.zeros((1, 128), np.float16), np.ones(128, np.int8))
+    assert not q.any() and float(s[0, 0]) == 1.0
+    # the SwiGLU form rotates fp16(silu(gate) * up)
+    gu = rng.normal(size=(2, 256)).astype(np.float16)
+    q, s = orc.rotate_a8(gu, signs[:128], swiglu=True)
+    wq, ws = orc.rotate_a8(orc.swiglu_fp16(gu), signs[:128])
+    np.testing.assert_array_equal(q, wq)
+    np.testing.assert_array_equal(s, ws)
