@@ -230,6 +230,27 @@ def rotate_a8(x, signs, swiglu=False):
     return a8(rotated)
 
 
+def q4_embedding(ids, packed, table, scales, signs):
+    """Token ids -> fp16 rows of the un-rotated embedding (kernels/cuda/model/e8p_q4.py:83-140).
+
+    `packed` is the row-major (vocab, hidden/8) u32 code matrix (the kernel reads its K-major
+    form).  Per row: int8 weights, unsigned block-128 butterflies and * fp32(128**-0.5) (that is
+    rotate() with all signs +1), * fp32(scale[id]), * sign, one fp16 cast; ids outside
+    [0, vocab) give zero rows.
+    """
+    ids = np.asarray(ids)
+    weights = q4_integers(packed, table)
+    vocab, hidden = weights.shape
+    out = np.zeros((ids.shape[0], hidden), np.float16)
+    ones = np.ones(hidden, np.int8)
+    for row, token in enumerate(ids.tolist()):
+        if 0 <= token < vocab:
+            value = rotate(weights[token].astype(np.float32)[None, :], ones)[0]
+            value = (value * np.float32(np.float16(scales[token]))).astype(np.float32)
+            out[row] = (value * np.asarray(signs, np.float32)).astype(np.float16)
+    return out
+
+
 # --------------------------------------------------------------------------
 # Contraction + epilogue
 # --------------------------------------------------------------------------

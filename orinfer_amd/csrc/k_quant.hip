@@ -11,8 +11,13 @@
 // butterfly stages inside every block of 128 channels in fp32, one multiply by fp32(128^-1/2), an
 // fp16 materialisation, then the same row-wise A8 rule.  Every stage is one fp32 add or subtract
 // in the order of the numpy oracle (quantization/vq.py:20-31), so codes and scales are bit-exact.
+//
+// e8p_q4_embedding follows kernels/cuda/model/e8p_q4.py:83-140: gather rows of a K-major two-stage
+// bank by token id, decode to int8, undo the rotation (unsigned butterflies, * fp32(128^-1/2),
+// * row scale, * sign), one fp16 cast; ids outside the vocabulary give zero rows.
 #include <hip/hip_fp16.h>
 
+#include "e8p_device.h"
 #include "orx_internal.h"
 
 namespace orx {
@@ -183,6 +188,61 @@ __global__ __launch_bounds__(256) void rotate_a8_kernel(const __half* __restrict
     }
 }
 
+// One workgroup per token; same lane layout as the rotation above (4 consecutive channels per lane,
+// two blocks of 128 per wave step).  The bank is (hidden/128, vocab, 16) u32: one code holds 8
+// channels, so a lane needs one half of one code.
+__global__ __launch_bounds__(256) void q4_embedding_kernel(const int32_t* __restrict__ ids, const uint32_t* __restrict__ bank,
+                                                           const uint32_t* __restrict__ book, const __half* __restrict__ scale,
+                                                           const int8_t* __restrict__ signs, __half* __restrict__ out,
+                                                           int vocab, int hidden) {
+    __shared__ Q4ByteTables tables;
+    build_tables(tables, book, threadIdx.x, 256);
+    __syncthreads();
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int half_wave = lane >> 5, l32 = lane & 31;
+    const int blocks = hidden / 128;
+    const int id = ids[row];
+    const bool valid = id >= 0 && id < vocab;
+    const float row_scale = valid ? __half2float(scale[id]) : 0.f;
+    for (int pair = wave; 2 * pair < blocks; pair += 4) {
+        const int block = 2 * pair + half_wave;
+        const bool live = block < blocks;
+        const int first = (live ? block : 0) * 128 + 4 * l32;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+        if (valid && live) {
+            const uint32_t code = bank[((int64_t)block * vocab + id) * 16 + (l32 >> 1)];
+            const uint2 weights = decode_q4(tables, code);
+            const uint32_t word = (l32 & 1) ? weights.y : weights.x;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (float)(int8_t)(word >> (8 * j));
+        }
+        {
+            const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
+            v[0] = a + c, v[2] = a - c, v[1] = b + d, v[3] = b - d;
+        }
+#pragma unroll
+        for (int bit = 0; bit < 5; ++bit) {
+            const bool upper = (l32 >> bit) & 1;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float other = __shfl_xor(v[j], 1 << bit, 64);
+                v[j] = upper ? other - v[j] : other + v[j];
+            }
+        }
+        if (live) {
+            const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+            __half result[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float value = ((v[j] * 0.08838834764831845f) * row_scale) * (float)(int8_t)(sign_word >> (8 * j));
+                asm volatile("" : "+v"(value));  // the cast rounds the fp32 value, never a fused multiply-convert
+                result[j] = __float2half_rn(value);
+            }
+            *reinterpret_cast<uint2*>(out + (int64_t)row * hidden + first) = *reinterpret_cast<const uint2*>(result);
+        }
+    }
+}
+
 // fp16 [rows, 2I] -> fp16 [rows, I].  grid (rows, ceil(I/256)).
 __global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ x, __half* __restrict__ y, int width) {
     const int row = blockIdx.x;
@@ -289,6 +349,42 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// slots used: N (vocab), K (hidden), capacity
+int q4_embedding_geometry(const orx_function&, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+// Book, IDs, Output, Scale, Signs, Weight, m   (e8p_q4.py:95-102 in generated-ABI order)
+int q4_embedding_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    hipLaunchKernelGGL(q4_embedding_kernel, dim3(g.grid[0]), dim3(256), 0, stream, pointer_arg<const int32_t>(args, 1),
+                       pointer_arg<const uint32_t>(args, 5), pointer_arg<const uint32_t>(args, 0),
+                       pointer_arg<const __half>(args, 3), pointer_arg<const int8_t>(args, 4), pointer_arg<__half>(args, 2),
+                       f.N, f.K);
+    return hip_check(hipGetLastError(), "launch e8p_q4_embedding");
+}
+
+int make_q4_embedding(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("vocab", 0, &bad);
+    f->K = (int)v.integer("hidden", 0, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128) {
+        set_error("e8p_q4_embedding: need M > 0, vocab > 0 and hidden a multiple of 128");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->dynamic_rows = true;  // the reference kernel always takes the live row count
+    f->args = {{"Book", ArgPointer, 4}, {"IDs", ArgPointer, 4}, {"Output", ArgPointer, 8}, {"Scale", ArgPointer, 2},
+               {"Signs", ArgPointer, 4}, {"Weight", ArgPointer, 4}, {"m", ArgI32, 4}};
+    f->device_function = reinterpret_cast<const void*>(&q4_embedding_kernel);
+    f->geometry = q4_embedding_geometry;
+    f->launch = q4_embedding_launch;
+    return ORX_OK;
+}
+
 int swiglu_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
     g->grid[1] = ceil_div((uint32_t)f.N, 256u);
@@ -328,8 +424,9 @@ const Registration* quant_registrations(int* count) {
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
     {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
+    {"e8p_q4_embedding", make_q4_embedding, "M, vocab, hidden", "Book,IDs,Output,Scale,Signs,Weight,m"},
     };
-    *count = 3;
+    *count = 4;
     return rows;
 }
 

@@ -46,6 +46,7 @@ ABI = {
     ("activation_quantization", (("K", 2560),)): ["Mask", "Q", "S", "X", "rows"],
     ("swiglu", (("I", 512),)): ["X", "Y", "rows"],
     ("rotate_activation_a8", (("M", 8), ("K", 5120))): ["Q", "S", "Signs", "X"],
+    ("e8p_q4_embedding", (("M", 8), ("vocab", 1000), ("hidden", 5120))): ["Book", "IDs", "Output", "Scale", "Signs", "Weight", "m"],
     ("rotate_activation_a8", (("M", 8), ("K", 256), ("swiglu", True), ("dynamic_rows", True))): ["Q", "S", "Signs", "X", "m"],
     ("e8p_q4_projection", (("M", 1), ("N", 9728), ("K", 2560))): ["A", "AS", "Book", "Out", "S", "W"],
     ("e8p_q4_projection", (("M", 64), ("N", 256), ("K", 256), ("dynamic_rows", True))):

@@ -179,6 +179,24 @@ def test_rotate_activation_a8_dynamic_rows_zero_row_and_graph():
     np.testing.assert_allclose(approx, x.astype(np.float32) @ w.T, atol=0.6, rtol=0.05)
 
 
+def test_q4_embedding_gather_matches_oracle():
+    rng = np.random.default_rng(orc.SEED + 40)
+    vocab, hidden, cap = 50, 640, 16
+    packed = rng.integers(0, 2**32, (vocab, hidden // 8), dtype=np.uint32)
+    scales = rng.uniform(0.005, 0.02, vocab).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), hidden)
+    ids = np.array([0, 49, 7, -1, 50, 7, 2**31 - 1, 13, 1], np.int32)
+    kern = gu.kernel("e8p_q4_embedding", M=cap, vocab=vocab, hidden=hidden)
+    out = torch.full((cap, hidden), 3.0, dtype=torch.float16, device=gu.DEV)
+    padded = np.zeros(cap, np.int32)
+    padded[: len(ids)] = ids
+    kern(Book=gu.book(), IDs=gu.dev(padded), Output=out, Scale=gu.dev(scales), Signs=gu.dev(signs),
+         Weight=gu.dev(orc.q4_pack_k(packed, 128)), m=len(ids))
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[: len(ids)], orc.q4_embedding(ids, packed, TABLE, scales, signs))
+    assert not got[3].any() and not got[4].any() and not got[6].any() and (got[len(ids):] == 3).all()
+
+
 # ---- Q4A8 projections -----------------------------------------------------
 def q4_case(rng, m, n, k):
     x = (rng.normal(size=(m, k))).astype(np.float16)

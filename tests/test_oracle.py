@@ -455,3 +455,25 @@ def test_rotate_a8_quantises_the_materialised_fp16_values():
     wq, ws = orc.rotate_a8(orc.swiglu_fp16(gu), signs[:128])
     np.testing.assert_array_equal(q, wq)
     np.testing.assert_array_equal(s, ws)
+
+
+def test_q4_embedding_inverts_the_rotation_of_a_rotated_row():
+    """Weights that are the rotation of a known vector come back as that vector: the embedding
+    kernel's formula is the inverse rotation (H is an involution up to the 1/128 scaling)."""
+    rng = np.random.default_rng(orc.SEED + 21)
+    table = orc.basis()
+    packed = rng.integers(0, 2**32, (6, 32), dtype=np.uint32)          # vocab 6, hidden 256
+    weights = orc.q4_integers(packed, table).astype(np.float32)
+    scales = np.array([0.5, 0.25, 1.0, 0.125, 2.0, 0.0625], np.float16)  # powers of two: exact scaling
+    signs = rng.choice(np.array([-1, 1], np.int8), 256)
+    got = orc.q4_embedding(np.array([3, -1, 0, 6, 5]), packed, table, scales, signs)
+    assert got.shape == (5, 256) and not got[1].any() and not got[3].any()
+    from scipy.linalg import hadamard
+    h = hadamard(128).astype(np.float64)
+    for row, token in ((0, 3), (2, 0), (4, 5)):
+        blocks = weights[token].reshape(2, 128).astype(np.float64) @ h
+        want = blocks.reshape(256) * 128**-0.5 * float(scales[token]) * signs
+        np.testing.assert_allclose(got[row].astype(np.float64), want, rtol=2e-3, atol=1e-3)
+        # rotating the embedding again (with the signs) returns the scaled integer weights
+        again = orc.rotate(got[row].astype(np.float32)[None, :], signs)[0]
+        np.testing.assert_allclose(again, weights[token] * float(scales[token]), atol=0.03 * float(scales[token]) * 8)
