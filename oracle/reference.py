@@ -288,6 +288,17 @@ def project(a_q, a_scale, w_q, w_scale, out_dtype=np.float16):
 # --------------------------------------------------------------------------
 # MoE routing (kernels/cuda/model/moe.py)
 # --------------------------------------------------------------------------
+def int8_swiglu(a_q, token_scale, gate, gate_scale, up, up_scale):
+    """Shared-expert W8 gate/up projections with the SwiGLU boundary
+    (kernels/cuda/model/int8_swiglu.py:10-57, integer_core.py:19-28): both projections are
+    rounded to fp16, then fp16((g / (1 + exp(-g))) * u) evaluated in fp32."""
+    g = project(a_q, token_scale, gate, gate_scale).astype(np.float32)
+    u = project(a_q, token_scale, up, up_scale).astype(np.float32)
+    with np.errstate(over="ignore"):
+        value = (g / (np.float32(1.0) + np.exp(-g).astype(np.float32))).astype(np.float32) * u
+    return value.astype(np.float16)
+
+
 def router_topk(logits, top_k, renormalize=True):
     """fp32 logits [M,E] -> ids int32 [M,k], prob fp32 [M,k] (moe.py:413-494).
 

@@ -501,6 +501,71 @@ int make_w8_projection(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// ---- W8 gate/up projections with the SwiGLU boundary (shared expert) ---------------------------
+// kernels/cuda/model/int8_swiglu.py:10-57 with integer_core.py:19-28: both projections are rounded
+// to fp16, then out = fp16((g / (1 + exp(-g))) * u) in fp32.  Built from the catalog's own int8
+// projection (two launches into the handle's fp16 scratch, row stride 2N) and one elementwise
+// kernel; the scratch is allocated when the handle is resolved.
+__global__ __launch_bounds__(256) void swiglu_pair_kernel(const __half* __restrict__ pair, __half* __restrict__ out, int n) {
+    const int row = blockIdx.x, col = blockIdx.y * 256 + threadIdx.x;
+    if (col >= n) return;
+    const float g = __half2float(pair[(int64_t)row * 2 * n + col]);
+    const float u = __half2float(pair[(int64_t)row * 2 * n + n + col]);
+    float value = __fdiv_rn(g, 1.0f + expf(-g)) * u;
+    asm volatile("" : "+v"(value));  // the cast rounds the fp32 product, never a fused multiply-convert
+    out[(int64_t)row * n + col] = __float2half_rn(value);
+}
+
+// A, Gate, GateScale, Output, TokenScale, Up, UpScale[, m]   (int8_swiglu.py:43-50 in generated-ABI order)
+int int8_swiglu_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    if (f.workspace == nullptr || f.inner == nullptr) {
+        set_error("%s: the handle was resolved without a device, its scratch is missing", f.symbol.c_str());
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    const int8_t* a = pointer_arg<const int8_t>(args, 0);
+    const __half* token_scale = pointer_arg<const __half>(args, 4);
+    __half* pair = static_cast<__half*>(f.workspace);
+    const void* weights[2] = {pointer_arg<const void>(args, 1), pointer_arg<const void>(args, 5)};
+    const __half* scales[2] = {pointer_arg<const __half>(args, 2), pointer_arg<const __half>(args, 6)};
+    for (int side = 0; side < 2; ++side) {
+        void* out = pair + (size_t)side * f.N;
+        void* inner_args[6] = {&a, &out, &token_scale, &weights[side], &scales[side], nullptr};
+        const int code = w8_launch(*f.inner, rows, g, stream, inner_args);
+        if (code != ORX_OK) return code;
+    }
+    hipLaunchKernelGGL(swiglu_pair_kernel, dim3((uint32_t)rows, ceil_div((uint32_t)f.N, 256u)), dim3(256), 0, stream, pair,
+                       pointer_arg<__half>(args, 3), f.N);
+    return hip_check(hipGetLastError(), "launch int8_swiglu (boundary)");
+}
+
+int make_int8_swiglu(const Variant& v, orx_function* f) {
+    int code = make_projection(v, f, kW8);
+    if (code != ORX_OK) return code;
+    if (f->out_f32 || f->stride != f->N) {
+        set_error("int8_swiglu: fp16 output with row stride N only");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"A", ArgPointer, 16},         {"Gate", ArgPointer, 16}, {"GateScale", ArgPointer, 2}, {"Output", ArgPointer, 2},
+               {"TokenScale", ArgPointer, 2}, {"Up", ArgPointer, 16},   {"UpScale", ArgPointer, 2}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    // the projections write fp16 pairs [rows, 2N]: same kernels, row stride 2N
+    f->inner = new orx_function(*f);
+    f->inner->stride = 2 * f->N;
+    f->inner->inner = nullptr;
+    int devices = 0;
+    if (hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
+        const size_t bytes = (size_t)f->capacity * 2 * f->N * sizeof(__half);
+        if (hipMalloc(&f->workspace, bytes) == hipSuccess)
+            f->workspace_bytes = bytes;
+        else
+            f->workspace = nullptr, (void)hipGetLastError();
+    } else {
+        (void)hipGetLastError();
+    }
+    f->launch = int8_swiglu_launch;
+    return ORX_OK;
+}
+
 // ---- routed single-stage experts -----------------------------------------------------------
 // A, AS, Book, C, Counts, Offsets, P, TileCount, TileExpert, TileRow, WS
 // (tests/cuda/operators/e8p_decode.py:72-84; kernels/cuda/model/e8p_decode.py:60-73 without Patch)
@@ -632,6 +697,8 @@ const Registration* gemm_registrations(int* count) {
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "
      "block_m=0|32|64|128|256",
      "A,Output,TokenScale,Weight,WeightScale[,m]"},
+    {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma",
+     "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
     {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
     {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
@@ -639,7 +706,7 @@ const Registration* gemm_registrations(int* count) {
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     };
-    *count = 6;
+    *count = 7;
     return rows;
 }
 

@@ -62,6 +62,8 @@ struct orx_function {
     // many rows.  Launches of one handle share it, so they must not overlap on different streams.
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
+    // A handle composed of other kernels of the catalog keeps them here (owned).
+    orx_function* inner = nullptr;
     // rows -> geometry; returns ORX_OK or an error code
     int (*geometry)(const orx_function&, int rows, orx::Geometry*) = nullptr;
     // enqueue on stream; args already validated for count/alignment

@@ -53,6 +53,8 @@ ABI = {
         ["A", "AS", "Book", "Out", "S", "W", "m"],
     ("int8_projection", (("M", 8192), ("N", 4096), ("K", 4096))):
         ["A", "Output", "TokenScale", "Weight", "WeightScale"],
+    ("int8_swiglu", (("M", 32), ("N", 512), ("K", 2048), ("dynamic_rows", True))):
+        ["A", "Gate", "GateScale", "Output", "TokenScale", "Up", "UpScale", "m"],
     ("e8p_decode_grouped", (("rows", 640), ("E", 512), ("tiles", 552), ("N", 1024), ("K", 2048))):
         ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "TileCount", "TileExpert", "TileRow", "WS"],
     ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],

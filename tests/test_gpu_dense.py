@@ -197,6 +197,23 @@ def test_q4_embedding_gather_matches_oracle():
     assert not got[3].any() and not got[4].any() and not got[6].any() and (got[len(ids):] == 3).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 96, 256), (6, 200, 1024), (70, 130, 384), (300, 260, 256)])
+def test_int8_swiglu_gate_up_boundary(m, n, k):
+    rng = np.random.default_rng(orc.SEED + m + n)
+    a_q = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    a_s = rng.uniform(0.005, 0.02, m).astype(np.float16)
+    gate, up = (rng.integers(-127, 128, (n, k), dtype=np.int8) for _ in range(2))
+    gs, us = (rng.uniform(0.001, 0.004, n).astype(np.float16) for _ in range(2))
+    out = torch.full((m + 1, n), 2.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("int8_swiglu", M=m, N=n, K=k)(A=gu.dev(a_q), Gate=gu.dev(gate), GateScale=gu.dev(gs), Output=out,
+                                            TokenScale=gu.dev(a_s), Up=gu.dev(up), UpScale=gu.dev(us))
+    got = gu.host(out)
+    want = orc.int8_swiglu(a_q, a_s, gate, gs, up, us)
+    # exp() may differ in the last place between the device and libm: one fp16 step at most
+    np.testing.assert_allclose(got[:m].astype(np.float32), want.astype(np.float32), rtol=1e-3, atol=1e-2)
+    assert np.mean(got[:m] == want) > 0.99 and (got[m:] == 2).all()
+
+
 # ---- Q4A8 projections -----------------------------------------------------
 def q4_case(rng, m, n, k):
     x = (rng.normal(size=(m, k))).astype(np.float16)

@@ -477,3 +477,26 @@ def test_q4_embedding_inverts_the_rotation_of_a_rotated_row():
         # rotating the embedding again (with the signs) returns the scaled integer weights
         again = orc.rotate(got[row].astype(np.float32)[None, :], signs)[0]
         np.testing.assert_allclose(again, weights[token] * float(scales[token]), atol=0.03 * float(scales[token]) * 8)
+
+
+def test_int8_swiglu_is_the_fp16_pair_through_the_swiglu_boundary():
+    rng = np.random.default_rng(orc.SEED + 50)
+    a_q = rng.integers(-127, 128, (5, 128), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.02, 5).astype(np.float16)
+    gate, up = (rng.integers(-127, 128, (24, 128), dtype=np.int8) for _ in range(2))
+    gs, us = (rng.uniform(0.001, 0.01, 24).astype(np.float16) for _ in range(2))
+    got = orc.int8_swiglu(a_q, a_s, gate, gs, up, us)
+    pair = np.concatenate([orc.project(a_q, a_s, gate, gs), orc.project(a_q, a_s, up, us)], axis=1)
+    # same boundary as the stand-alone SwiGLU operator, whose sigmoid is written differently:
+    # equal to within one fp16 step
+    stable = orc.swiglu_fp16(pair).astype(np.float32)
+    np.testing.assert_allclose(got.astype(np.float32), stable, rtol=2e-3, atol=1e-6)
+    # hand-computed entry in float64
+    g, u = float(pair[2, 3]), float(pair[2, 24 + 3])
+    assert abs(float(got[2, 3]) - g / (1 + np.exp(-g)) * u) <= 1e-3 * abs(g * u) + 1e-7
+    # a very negative gate gives (signed) zero, not NaN
+    big = orc.int8_swiglu(np.full((1, 128), 127, np.int8), np.array([1.0], np.float16), -np.full((1, 128), 127, np.int8),
+                          np.array([2.0**-6], np.float16), np.ones((1, 128), np.int8), np.array([1.0], np.float16))
+    assert float(orc.project(np.full((1, 128), 127, np.int8), np.array([1.0], np.float16), -np.full((1, 128), 127, np.int8),
+                             np.array([2.0**-6], np.float16))[0, 0]) == -32258.0
+    assert float(big[0, 0]) == 0.0
