@@ -498,5 +498,5 @@ def test_int8_swiglu_is_the_fp16_pair_through_the_swiglu_boundary():
     big = orc.int8_swiglu(np.full((1, 128), 127, np.int8), np.array([1.0], np.float16), -np.full((1, 128), 127, np.int8),
                           np.array([2.0**-6], np.float16), np.ones((1, 128), np.int8), np.array([1.0], np.float16))
     assert float(orc.project(np.full((1, 128), 127, np.int8), np.array([1.0], np.float16), -np.full((1, 128), 127, np.int8),
-                             np.array([2.0**-6], np.float16))[0, 0]) == -32258.0
+                             np.array([2.0**-6], np.float16))[0, 0]) == -32256.0  # fp16(-32258.0)
     assert float(big[0, 0]) == 0.0
