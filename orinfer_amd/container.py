@@ -1,0 +1,180 @@
+"""Weight containers and package records for the quantized linear path (host side, numpy only).
+
+Two things the engine's packaging layer does for this path:
+
+* the E8P two-stage weight container `orinfer-e8p-q4-v1`: a safetensors file with tensors
+  `packed` (N, K/8) u32, `scales` (N) f16, `signs` (K) i8, `basis` (256, 8) i8 and metadata
+  `codec`, `coefficients`, `layout`, `rotation`
+  (python/orinfer_build/quantization/e8p_q4.py:33-58 validation, :80-112 save/load);
+* `Kernel` records: one launch of one symbol with ordered arguments
+  (crates/orinfer-model-sdk/src/artifact.rs:87-110, arguments :176-186, buffers :60-72), named by
+  the row-specialisation rule `slot/rows/MIN-MAX`
+  (crates/orinfer-model-sdk/src/operators/rows.rs:14-58).
+
+A record has no field for a variant, so the symbol carries it
+(`family?M=1&N=9728&K=2560`), which `orx_resolve` accepts.
+"""
+import hashlib
+import json
+from dataclasses import dataclass
+from pathlib import Path
+
+import numpy as np
+
+from . import codebook, lib
+
+CODEC = "orinfer-e8p-q4-v1"
+LAYOUT = "u32-low-coarse-high-residual"
+ROTATION = "signed-block128"
+COEFFICIENTS = (4, 1)
+
+_DTYPES = {np.dtype(np.uint8): "u8", np.dtype(np.int8): "i8", np.dtype(np.uint16): "u16", np.dtype(np.float16): "f16",
+           np.dtype(np.float32): "f32", np.dtype(np.float64): "f64", np.dtype(np.uint32): "u32", np.dtype(np.int32): "i32",
+           np.dtype(np.uint64): "u64", np.dtype(np.int64): "i64"}
+
+
+@dataclass
+class Q4Weights:
+    """One two-stage E8P matrix: row-major codes, one scale per output row, one sign per input."""
+    packed: np.ndarray   # (N, K/8) u32, low half coarse code, high half residual code
+    scales: np.ndarray   # (N,) f16
+    signs: np.ndarray    # (K,) i8, +-1: the rotation the activations must undergo
+
+    def validate(self):
+        p, s, g = self.packed, self.scales, self.signs
+        if p.dtype != np.uint32 or p.ndim != 2 or min(p.shape) <= 0 or (p.shape[1] * 8) % 128:
+            raise ValueError("E8P-Q4 codes must be (N, K/8) uint32 with K a multiple of 128")
+        n, k = p.shape[0], p.shape[1] * 8
+        if s.dtype != np.float16 or s.shape != (n,) or not np.isfinite(s).all() or (s <= 0).any():
+            raise ValueError("E8P-Q4 scales must be N positive finite float16 values")
+        if g.dtype != np.int8 or g.shape != (k,) or not np.isin(g, (-1, 1)).all():
+            raise ValueError("E8P-Q4 signs must be K int8 values of +-1")
+        return n, k
+
+    def k_major(self, packed_k=128):
+        """(K/packed_k, N, packed_k/8) u32, tag e8p-q4-k128-u32 (models/qwen35/storage.py:56-81)."""
+        return codebook.q4_to_k_major(self.packed, packed_k)
+
+
+def save_q4(path, weights):
+    from safetensors.numpy import save_file
+
+    weights.validate()
+    save_file(dict(packed=weights.packed, scales=weights.scales, signs=weights.signs, basis=codebook.basis()), str(path),
+              metadata=dict(codec=CODEC, coefficients=",".join(map(str, COEFFICIENTS)), layout=LAYOUT, rotation=ROTATION))
+
+
+def load_q4(path):
+    """Reads a container; refuses any codec, layout, rotation, coefficient or basis it does not implement."""
+    from safetensors import safe_open
+
+    with safe_open(str(path), framework="numpy") as source:
+        metadata = source.metadata() or {}
+        if (metadata.get("codec") != CODEC or metadata.get("layout") != LAYOUT or metadata.get("rotation") != ROTATION
+                or set(source.keys()) != {"packed", "scales", "signs", "basis"}):
+            raise ValueError("E8P-Q4 codec contract mismatch")
+        if not np.array_equal(source.get_tensor("basis"), codebook.basis()):
+            raise ValueError("E8P-Q4 basis differs from the one the kernels decode")
+        coefficients = tuple(int(v) for v in metadata.get("coefficients", "").split(",") if v)
+        if coefficients != COEFFICIENTS:
+            raise ValueError(f"E8P-Q4 coefficients {coefficients}: the kernels implement {COEFFICIENTS}")
+        weights = Q4Weights(source.get_tensor("packed"), source.get_tensor("scales"), source.get_tensor("signs"))
+    weights.validate()
+    return weights
+
+
+# ---- package records -------------------------------------------------------------------------
+def file_identity(path):
+    data = Path(path).read_bytes()
+    return {"file": Path(path).name, "sha256": hashlib.sha256(data).hexdigest()}
+
+
+def buffer_record(name, array=None, *, dtype=None, shape=None, layout="row-major", access="read", data=None,
+                  alignment=256):
+    """`Buffer` of artifact.rs:60-72.  Either an array (dtype and shape are taken from it) or both."""
+    if array is not None:
+        dtype, shape = _DTYPES[np.asarray(array).dtype], list(np.asarray(array).shape)
+    if access not in ("read", "write", "read_write"):
+        raise ValueError("access must be read, write or read_write")
+    return {"name": name, "dtype": dtype, "shape": list(shape), "layout": layout, "alignment": alignment,
+            "access": access, "data": data}
+
+
+def symbol_with_variant(family, **variant):
+    def text(value):
+        return "true" if value is True else "false" if value is False else str(value)
+    return family + "?" + "&".join(f"{key}={text(value)}" for key, value in variant.items()) if variant else family
+
+
+def kernel_record(name, family, variant, bindings, rows=0):
+    """`Kernel` of artifact.rs:87-110 for one launch of `family` with `variant`.
+
+    bindings: argument name -> buffer name | (buffer name, byte offset) | int (scalar).  The grid,
+    block and LDS bytes are the library's own for `rows` live rows (0 = the variant's M)."""
+    kernel = lib.Kernel(family, **variant)
+    grid, block, shared = kernel.geometry(rows)
+    args = []
+    for arg_name, kind in zip(kernel.arg_names, kernel.arg_kinds):
+        if arg_name not in bindings:
+            raise KeyError(f"{family}: no binding for argument {arg_name}")
+        bound = bindings[arg_name]
+        if kind == 1:
+            args.append({"kind": "i32", "value": int(bound)})
+        elif isinstance(bound, tuple):
+            args.append({"kind": "buffer_slice", "name": bound[0], "offset": int(bound[1])})
+        else:
+            args.append({"kind": "buffer", "name": bound})
+    root = Path(__file__).resolve().parent
+    return {
+        "name": name,
+        "module": file_identity(lib.LIBRARY_PATH),
+        "source": file_identity(root / "csrc" / "orx_api.cpp"),
+        "host_abi": file_identity(root.parent / "include" / "orx.h"),
+        "symbol": symbol_with_variant(family, **variant),
+        "grid": list(grid), "block": list(block), "shared_memory_bytes": shared, "cooperative": False,
+        "args": args,
+    }
+
+
+def projection_records(slot, n, k, capacity, *, family="e8p_q4_projection", bindings=None):
+    """Row-specialised records of one projection slot under the naming rule `slot/rows/MIN-MAX`:
+    the decode kernel for 1..4 rows, the streaming kernel up to 128, the MFMA tiles above, each a
+    separately resolvable symbol whose geometry is recorded for the top of its range."""
+    ranges = [(1, min(4, capacity))]
+    if capacity > 4:
+        ranges.append((5, min(128, capacity)))
+    if capacity > 128:
+        ranges.append((129, capacity))
+    records = []
+    for low, high in ranges:
+        variant = dict(M=high, N=n, K=k, dynamic_rows=True)
+        names = lib.Kernel(family, **variant).arg_names
+        bound = dict(bindings or {a: a for a in names})
+        bound["m"] = high
+        records.append(kernel_record(f"{slot}/rows/{low}-{high}", family, variant, bound, rows=high))
+    return records
+
+
+def fixture_manifest(buffers, records, validation, *, rows=None):
+    """The same records as a manifest of the `orx_run_fixture` runner (buffers: name -> bytes | array file)."""
+    kernels = []
+    for record in records:
+        family, _, query = record["symbol"].partition("?")
+        args = []
+        for arg in record["args"]:
+            if arg["kind"] == "buffer":
+                args.append({"buffer": arg["name"]})
+            elif arg["kind"] == "buffer_slice":
+                args.append({"buffer": arg["name"], "offset": arg["offset"]})
+            else:
+                args.append({"i32": arg["value"]})
+        entry = {"symbol": record["symbol"], "grid": record["grid"], "block": record["block"],
+                 "shared": record["shared_memory_bytes"], "args": args}
+        if rows is not None:
+            entry["rows"] = rows
+        kernels.append(entry)
+    return {"schema_version": 1, "target": "gfx950", "buffers": buffers, "kernels": kernels, "validation": validation}
+
+
+def dumps(record):
+    return json.dumps(record, indent=1, sort_keys=False)

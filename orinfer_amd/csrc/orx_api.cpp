@@ -199,19 +199,54 @@ int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
         return ORX_ERR_BAD_ARGUMENT;
     }
     *out = nullptr;
-    const Registration* r = find(symbol);
+    // A package record has one `symbol` string and no place for a variant (artifact.rs:87-110), so
+    // a symbol may carry it: "family?M=1&N=9728&K=2560&algorithm=gemv".  Values that are not
+    // integers or true/false are taken as strings.
+    std::string family(symbol), inline_variant;
+    const size_t mark = family.find('?');
+    if (mark != std::string::npos) {
+        const std::string query = family.substr(mark + 1);
+        family.resize(mark);
+        inline_variant = "{";
+        size_t at = 0;
+        while (at < query.size()) {
+            size_t end = query.find('&', at);
+            if (end == std::string::npos) end = query.size();
+            const std::string pair = query.substr(at, end - at);
+            const size_t eq = pair.find('=');
+            if (eq == std::string::npos || eq == 0) {
+                set_error("orx_resolve %s: malformed variant in symbol", symbol);
+                return ORX_ERR_BAD_VARIANT;
+            }
+            const std::string key = pair.substr(0, eq), value = pair.substr(eq + 1);
+            bool number = !value.empty();
+            for (size_t c = 0; c < value.size(); ++c)
+                if (!(isdigit((unsigned char)value[c]) || (c == 0 && value[c] == '-' && value.size() > 1))) number = false;
+            if (inline_variant.size() > 1) inline_variant += ",";
+            inline_variant += "\"" + key + "\":";
+            inline_variant += (number || value == "true" || value == "false") ? value : "\"" + value + "\"";
+            at = end + 1;
+        }
+        inline_variant += "}";
+        if (variant_json != nullptr && variant_json[0] != 0 && strcmp(variant_json, "{}") != 0) {
+            set_error("orx_resolve %s: variant given both in the symbol and as JSON", symbol);
+            return ORX_ERR_BAD_VARIANT;
+        }
+        variant_json = inline_variant.c_str();
+    }
+    const Registration* r = find(family.c_str());
     if (r == nullptr) {
-        set_error("orx_resolve: unknown symbol %s", symbol);
+        set_error("orx_resolve: unknown symbol %s", family.c_str());
         return ORX_ERR_UNKNOWN_SYMBOL;
     }
     Variant variant;
     std::string why;
     if (!parse_variant(variant_json, &variant, &why)) {
-        set_error("orx_resolve %s: %s", symbol, why.c_str());
+        set_error("orx_resolve %s: %s", family.c_str(), why.c_str());
         return ORX_ERR_BAD_VARIANT;
     }
     orx_function* f = new orx_function();
-    f->symbol = symbol;
+    f->symbol = family;
     int code = r->factory(variant, f);
     if (code != ORX_OK) {
         delete f;

@@ -1,0 +1,123 @@
+"""Weight container `orinfer-e8p-q4-v1` and package records (host side).  The container round trip
+follows python/orinfer_build/quantization/e8p_q4.py:80-112; records follow the `Kernel` schema of
+crates/orinfer-model-sdk/src/artifact.rs:87-110 and the naming rule of operators/rows.rs:14-58."""
+import json
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import reference as orc
+from orinfer_amd import build, codebook, container, lib
+
+
+def weights(rng, n=48, k=256):
+    return container.Q4Weights(rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32),
+                               rng.uniform(0.005, 0.02, n).astype(np.float16),
+                               rng.choice(np.array([-1, 1], np.int8), k))
+
+
+def test_container_round_trip_and_contract_checks(tmp_path):
+    from safetensors.numpy import save_file
+    rng = np.random.default_rng(orc.SEED)
+    w = weights(rng)
+    container.save_q4(tmp_path / "w.safetensors", w)
+    back = container.load_q4(tmp_path / "w.safetensors")
+    for a, b in ((w.packed, back.packed), (w.scales, back.scales), (w.signs, back.signs)):
+        np.testing.assert_array_equal(a, b)
+    np.testing.assert_array_equal(back.k_major(), orc.q4_pack_k(w.packed, 128))
+    good = dict(codec=container.CODEC, coefficients="4,1", layout=container.LAYOUT, rotation=container.ROTATION)
+    tensors = dict(packed=w.packed, scales=w.scales, signs=w.signs, basis=codebook.basis())
+    for key, value in (("codec", "orinfer-e8p-q4-v2"), ("coefficients", "7,2"), ("layout", "u32"), ("rotation", "none")):
+        save_file(tensors, str(tmp_path / "bad.safetensors"), metadata=dict(good, **{key: value}))
+        with pytest.raises(ValueError):
+            container.load_q4(tmp_path / "bad.safetensors")
+    wrong_basis = codebook.basis().copy()
+    wrong_basis[0, 0] = 6
+    save_file(dict(tensors, basis=wrong_basis), str(tmp_path / "bad.safetensors"), metadata=good)
+    with pytest.raises(ValueError):
+        container.load_q4(tmp_path / "bad.safetensors")
+    save_file(dict(tensors, extra=w.signs), str(tmp_path / "bad.safetensors"), metadata=good)
+    with pytest.raises(ValueError):
+        container.load_q4(tmp_path / "bad.safetensors")
+    for broken in (container.Q4Weights(w.packed.astype(np.int32), w.scales, w.signs),
+                   container.Q4Weights(w.packed, w.scales[:-1], w.signs),
+                   container.Q4Weights(w.packed, w.scales, np.zeros_like(w.signs)),
+                   container.Q4Weights(w.packed[:, :5], w.scales, w.signs[:40])):
+        with pytest.raises(ValueError):
+            broken.validate()
+
+
+def test_symbol_carries_its_variant():
+    plain = lib.Kernel("e8p_q4_projection", M=4, N=9728, K=2560, dynamic_rows=True)
+    packed = lib.Kernel(container.symbol_with_variant("e8p_q4_projection", M=4, N=9728, K=2560, dynamic_rows=True))
+    assert packed.arg_names == plain.arg_names and packed.geometry(1) == plain.geometry(1)
+    assert lib.Kernel("int8_projection?M=8192&N=4096&K=4096&output_dtype=float32").geometry() == \
+        lib.Kernel("int8_projection", M=8192, N=4096, K=4096, output_dtype="float32").geometry()
+    for bad in ("e8p_q4_projection?M=1&N", "e8p_q4_projection?=3", "nothing?M=1"):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel(bad)
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("e8p_q4_projection?M=1&N=128&K=128", M=1)
+
+
+def test_kernel_records_follow_the_package_schema():
+    records = container.projection_records("decoder.0.qkv", 7168, 5120, 8192)
+    assert [r["name"] for r in records] == ["decoder.0.qkv/rows/1-4", "decoder.0.qkv/rows/5-128",
+                                            "decoder.0.qkv/rows/129-8192"]
+    keys = {"name", "module", "source", "host_abi", "symbol", "grid", "block", "shared_memory_bytes", "cooperative", "args"}
+    for record in records:
+        assert set(record) == keys and record["cooperative"] is False
+        assert record["symbol"].startswith("e8p_q4_projection?M=")
+        for identity in (record["module"], record["source"], record["host_abi"]):
+            assert set(identity) == {"file", "sha256"} and len(identity["sha256"]) == 64
+        assert [a.get("name", "m") for a in record["args"]] == ["A", "AS", "Book", "Out", "S", "W", "m"]
+        assert record["args"][-1]["kind"] == "i32" and all(a["kind"] == "buffer" for a in record["args"][:-1])
+        threads = record["block"][0] * record["block"][1] * record["block"][2]
+        assert 0 < threads <= 1024 and all(g > 0 for g in record["grid"])   # artifact.rs validate_geometry
+        # the record resolves and its launch geometry is what the library would use
+        kernel = lib.Kernel(record["symbol"])
+        rows = record["args"][-1]["value"]
+        assert kernel.geometry(rows) == (tuple(record["grid"]), tuple(record["block"]), record["shared_memory_bytes"])
+    json.loads(container.dumps(records[0]))
+    sliced = container.kernel_record("embed", "e8p_q4_embedding", dict(M=8, vocab=100, hidden=256),
+                                     dict(Book="Book", IDs=("Tokens", 64), Output="Hidden", Scale="Scale", Signs="Signs",
+                                          Weight="Bank", m=3), rows=3)
+    assert sliced["args"][1] == {"kind": "buffer_slice", "name": "Tokens", "offset": 64}
+    buffer = container.buffer_record("W", np.zeros((4, 8), np.uint32), layout="e8p-q4-k128-u32")
+    assert buffer["dtype"] == "u32" and buffer["shape"] == [4, 8] and buffer["access"] == "read"
+
+
+@pytest.mark.gpu
+def test_container_to_records_to_fixture_run(tmp_path):
+    """File -> container -> records -> launch through the fixture runner, checked against the oracle."""
+    rng = np.random.default_rng(orc.SEED + 8)
+    n, k, rows = 320, 640, 3
+    w = weights(rng, n, k)
+    container.save_q4(tmp_path / "layer.safetensors", w)
+    loaded = container.load_q4(tmp_path / "layer.safetensors")
+    x = rng.normal(size=(rows, k)).astype(np.float16)
+    # the model rotates activations with the container's signs before A8
+    a_q, a_s = orc.rotate_a8(x, loaded.signs)
+    want = orc.project(a_q, a_s[:, 0], orc.q4_integers(loaded.packed, orc.basis()), loaded.scales, np.float32)
+    want.tofile(tmp_path / "Out.f32")
+    arrays = {"X": x, "Signs": loaded.signs, "Book": codebook.book(), "S": loaded.scales, "W": loaded.packed}
+    buffers = []
+    for name, array in arrays.items():
+        np.ascontiguousarray(array).tofile(tmp_path / f"{name}.bin")
+        buffers.append({"name": name, "file": f"{name}.bin", "bytes": int(np.asarray(array).nbytes)})
+    buffers += [{"name": "A", "bytes": 4 * k, "fill": 0}, {"name": "AS", "bytes": 8, "fill": 0},
+                {"name": "Out", "bytes": 4 * n * 2, "fill": 0}]
+    rotate = container.kernel_record("layer.rotate/rows/1-4", "rotate_activation_a8", dict(M=4, K=k, dynamic_rows=True),
+                                     dict(Q="A", S="AS", Signs="Signs", X="X", m=rows), rows=rows)
+    project = container.projection_records("layer.proj", n, k, 4, bindings=dict(A="A", AS="AS", Book="Book", Out="Out",
+                                                                                  S="S", W="W"))[0]
+    project["args"][-1]["value"] = rows
+    manifest = container.fixture_manifest(buffers, [rotate, project],
+                                          dict(output="Out", output_dtype="f16", reference="Out.f32",
+                                               relative_l2_tolerance=1e-3, zero_input="X", repetitions=5), rows=rows)
+    (tmp_path / "manifest.json").write_text(json.dumps(manifest))
+    done = subprocess.run([str(build.FIXTURE_RUNNER), str(tmp_path / "manifest.json")], capture_output=True, text=True,
+                          timeout=120)
+    report = json.loads(done.stdout.strip().splitlines()[-1])
+    assert done.returncode == 0 and report["ok"] and report["relative_l2"] < 1e-3, (report, done.stderr)
