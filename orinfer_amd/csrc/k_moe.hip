@@ -22,13 +22,30 @@ __device__ __forceinline__ float key_value(uint32_t ordered) {
     return __uint_as_float((ordered & 0x80000000u) ? ordered ^ 0x80000000u : ~ordered);
 }
 
+// Maximum of a 64-bit key over the wave with data-parallel-primitive moves only (no LDS round
+// trips: the selection loop below is a chain of top_k dependent reductions).  Quad swaps, half-row
+// and row mirrors give every lane its row's maximum; two broadcasts carry it across rows into
+// lane 63, which is then read back as a scalar.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void dpp_max_step(uint32_t& hi, uint32_t& lo) {
+    // lanes outside ROW_MASK receive their own value back
+    const uint32_t other_hi = (uint32_t)__builtin_amdgcn_update_dpp((int)hi, (int)hi, CTRL, ROW_MASK, 0xF, false);
+    const uint32_t other_lo = (uint32_t)__builtin_amdgcn_update_dpp((int)lo, (int)lo, CTRL, ROW_MASK, 0xF, false);
+    const bool take = other_hi > hi || (other_hi == hi && other_lo > lo);
+    hi = take ? other_hi : hi;
+    lo = take ? other_lo : lo;
+}
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-#pragma unroll
-    for (int offset = 32; offset > 0; offset >>= 1) {
-        const unsigned long long other = __shfl_xor(v, offset, 64);
-        v = other > v ? other : v;
-    }
-    return v;
+    uint32_t hi = (uint32_t)(v >> 32), lo = (uint32_t)v;
+    dpp_max_step<0xB1, 0xF>(hi, lo);   // quad_perm [1,0,3,2]
+    dpp_max_step<0x4E, 0xF>(hi, lo);   // quad_perm [2,3,0,1]
+    dpp_max_step<0x141, 0xF>(hi, lo);  // row_half_mirror
+    dpp_max_step<0x140, 0xF>(hi, lo);  // row_mirror
+    dpp_max_step<0x142, 0xA>(hi, lo);  // row_bcast:15 into rows 1 and 3
+    dpp_max_step<0x143, 0xC>(hi, lo);  // row_bcast:31 into rows 2 and 3
+    const uint32_t top_hi = (uint32_t)__builtin_amdgcn_readlane((int)hi, 63);
+    const uint32_t top_lo = (uint32_t)__builtin_amdgcn_readlane((int)lo, 63);
+    return ((unsigned long long)top_hi << 32) | top_lo;
 }
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -39,17 +56,18 @@ __device__ __forceinline__ float wave_sum(float v) {
 // One wave per row; each lane keeps ceil(E/64) keys in registers.  Key = ordered score in the
 // high word, (E - id) in the low word, so one max picks the score and the lowest id on ties.
 constexpr int kMaxLocal = 16;  // E <= 1024
+template <int LOCAL>  // keys per lane: ceil(E / 64) rounded up to a power of two
 __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids,
                                                           float* __restrict__ prob, int m, int e, int top_k,
                                                           int renormalize) {
     const int lane = threadIdx.x & 63;
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= m) return;
-    unsigned long long keys[kMaxLocal];
+    unsigned long long keys[LOCAL];
     float all_exp = 0.f;
     float local_max = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < kMaxLocal; ++j) {
+    for (int j = 0; j < LOCAL; ++j) {
         const int id = j * 64 + lane;
         keys[j] = 0ull;
         if (id < e) {
@@ -63,7 +81,7 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
     for (int offset = 32; offset > 0; offset >>= 1) global_max = fmaxf(global_max, __shfl_xor(global_max, offset, 64));
     if (!renormalize) {
 #pragma unroll
-        for (int j = 0; j < kMaxLocal; ++j) {
+        for (int j = 0; j < LOCAL; ++j) {
             const int id = j * 64 + lane;
             if (id < e) all_exp += expf(logits[(int64_t)row * e + id] - global_max);
         }
@@ -73,12 +91,12 @@ __global__ __launch_bounds__(256) void router_topk_kernel(const float* __restric
     for (int rank = 0; rank < top_k; ++rank) {
         unsigned long long best = 0ull;
 #pragma unroll
-        for (int j = 0; j < kMaxLocal; ++j) best = keys[j] > best ? keys[j] : best;
+        for (int j = 0; j < LOCAL; ++j) best = keys[j] > best ? keys[j] : best;
         best = wave_max_u64(best);
         const int id = e - (int)(uint32_t)(best & 0xFFFFFFFFull);
         const float score = key_value((uint32_t)(best >> 32));
 #pragma unroll
-        for (int j = 0; j < kMaxLocal; ++j)
+        for (int j = 0; j < LOCAL; ++j)
             if (j * 64 + lane == id) keys[j] = 0ull;
         if (lane == rank) {
             ids[(int64_t)row * top_k + rank] = id;
@@ -168,6 +186,100 @@ __global__ __launch_bounds__(256) void expert_tiles_kernel(const int* __restrict
     }
 }
 
+// ---- all routing metadata in one launch ---------------------------------------------------------
+// kernels/cuda/model/moe.py:713-764: counts, stable relative slots, row and tile prefixes and the
+// tile list from one workgroup, instead of three dependent launches.  16 waves; wave w owns a
+// contiguous run of assignments (token-major) and walks it 64 at a time: lanes that name the same
+// expert are ranked by lane order with one ballot per distinct expert (scalar loop, no memory
+// traffic), on top of the expert's running count in the wave's own counter row.  A prefix over the
+// 16 rows per expert then turns wave-local slots into global ones.  No atomics, one writer per
+// element, token-major stable order; a token may name an expert more than once.
+// LDS (dynamic): counters[16][E], wave-local slots[capacity assignments], scan totals.
+constexpr int kMetaWaves = 16, kMetaThreads = kMetaWaves * 64;
+__global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
+    const int* __restrict__ ids, int* __restrict__ counts, int* __restrict__ relative, int* __restrict__ row_offsets,
+    int* __restrict__ tile_count, int* __restrict__ tile_expert, int* __restrict__ tile_offsets, int* __restrict__ tile_row,
+    int m, int experts, int top_k, int block_m) {
+    extern __shared__ int meta_lds[];
+    int* counters = meta_lds;                          // [kMetaWaves][experts]
+    int* wave_rows = counters + kMetaWaves * experts;  // [kMetaWaves]
+    int* wave_tiles = wave_rows + kMetaWaves;          // [kMetaWaves]
+    int* local = wave_tiles + kMetaWaves;              // [assignments]: id << 16 | wave-local slot... two arrays below
+    const int assignments = m * top_k;
+    int* local_id = local + assignments;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int i = tid; i < kMetaWaves * experts; i += kMetaThreads) counters[i] = 0;
+    __syncthreads();
+    // this wave's run of assignments, a multiple of 64 long
+    const int per_wave = ((assignments + kMetaWaves - 1) / kMetaWaves + 63) & ~63;
+    const int first = wave * per_wave, last = min(assignments, first + per_wave);
+    int* mine = counters + wave * experts;
+    for (int base = first; base < last; base += 64) {
+        const int at = base + lane;
+        const bool valid = at < last;
+        const int id = valid ? ids[at] : -1;
+        const int running = valid ? mine[id] : 0;  // nobody has written this expert in this step yet
+        int rank = 0, group = 0;
+        unsigned long long remaining = __ballot(valid);
+        while (remaining != 0ull) {  // wave-uniform: one round per distinct expert among the 64 lanes
+            const int leader = __ffsll((long long)remaining) - 1;
+            const int expert = __builtin_amdgcn_readlane(id, leader);
+            const unsigned long long same = __ballot(valid && id == expert);
+            if (valid && id == expert) {
+                rank = __popcll(same & ((1ull << lane) - 1ull));
+                group = __popcll(same);
+            }
+            remaining &= ~same;
+        }
+        if (valid) {
+            local[at] = running + rank;
+            local_id[at] = id;
+            if (rank == group - 1) mine[id] = running + group;
+        }
+    }
+    __syncthreads();
+    // per expert: exclusive prefix over the 16 wave rows, total count
+    int count = 0;
+    if (tid < experts) {
+        for (int w = 0; w < kMetaWaves; ++w) {
+            const int t = counters[w * experts + tid];
+            counters[w * experts + tid] = count;
+            count += t;
+        }
+        counts[tid] = count;
+    }
+    __syncthreads();
+    // global relative slots, written once and coalesced
+    for (int at = tid; at < assignments; at += kMetaThreads)
+        relative[at] = local[at] + counters[(at / per_wave) * experts + local_id[at]];
+    // exclusive scans of count and ceil(count / block_m) over the experts (one per thread)
+    const int tiles = (count + block_m - 1) / block_m;
+    int row_scan = count, tile_scan = tiles;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const int r = __shfl_up(row_scan, offset, 64), t = __shfl_up(tile_scan, offset, 64);
+        if (lane >= offset) row_scan += r, tile_scan += t;
+    }
+    if (lane == 63) wave_rows[wave] = row_scan, wave_tiles[wave] = tile_scan;
+    __syncthreads();
+    int row_base = 0, tile_base = 0, tile_total = 0;
+    for (int w = 0; w < kMetaWaves; ++w) {
+        if (w < wave) row_base += wave_rows[w], tile_base += wave_tiles[w];
+        tile_total += wave_tiles[w];
+    }
+    if (tid == 0) tile_count[0] = tile_total;
+    if (tid < experts) {
+        const int first_tile = tile_base + tile_scan - tiles;
+        row_offsets[tid] = row_base + row_scan - count;
+        tile_offsets[tid] = first_tile;
+        for (int t = 0; t < tiles; ++t) {
+            tile_expert[first_tile + t] = tid;
+            tile_row[first_tile + t] = t * block_m;
+        }
+    }
+}
+
 // grid M*top_k: copy one int8 row and its scales to the expert-sorted slot.
 __global__ __launch_bounds__(256) void expert_dispatch_kernel(const int8_t* __restrict__ a, int8_t* __restrict__ d,
                                                               __half* __restrict__ ds, const int* __restrict__ ids,
@@ -228,8 +340,20 @@ int rows_geometry_router(const orx_function&, int rows, Geometry* g) {
     return ORX_OK;
 }
 int router_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(router_topk_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const float>(args, 1),
-                       pointer_arg<int>(args, 0), pointer_arg<float>(args, 2), rows, f.E, f.top_k, f.flags);
+    const float* logits = pointer_arg<const float>(args, 1);
+    int* ids = pointer_arg<int>(args, 0);
+    float* prob = pointer_arg<float>(args, 2);
+    const dim3 grid(g.grid[0]), block(256);
+    if (f.E <= 64)
+        hipLaunchKernelGGL(router_topk_kernel<1>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
+    else if (f.E <= 128)
+        hipLaunchKernelGGL(router_topk_kernel<2>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
+    else if (f.E <= 256)
+        hipLaunchKernelGGL(router_topk_kernel<4>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
+    else if (f.E <= 512)
+        hipLaunchKernelGGL(router_topk_kernel<8>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
+    else
+        hipLaunchKernelGGL(router_topk_kernel<16>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
     return hip_check(hipGetLastError(), "launch router_topk");
 }
 int make_router(const Variant& v, orx_function* f) {
@@ -245,7 +369,7 @@ int make_router(const Variant& v, orx_function* f) {
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = rows_geometry_router;
     f->launch = router_launch;
-    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel);
+    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel<16>);
     return ORX_OK;
 }
 
@@ -324,6 +448,51 @@ int make_tiles(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+int metadata_geometry(const orx_function& f, int, Geometry* g) {
+    g->grid[0] = 1;
+    g->block[0] = kMetaThreads;
+    // counters, scan totals, wave-local slot and expert of every assignment the variant can hold
+    g->shared = (uint32_t)((kMetaWaves * f.E + 2 * kMetaWaves + 2 * f.M * f.top_k) * sizeof(int));
+    return ORX_OK;
+}
+// Counts, IDs, RelativeSlot, RowOffsets, TileCount, TileExpert, TileOffsets, TileRow[, m]
+// (moe.py:726-735 in generated-ABI order)
+int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    static bool opted_in = false;  // 64 KiB of counters at E = 1024 needs the LDS opt-in
+    if (!opted_in) {
+        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&route_metadata_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                                   "hipFuncSetAttribute");
+        if (code != ORX_OK) return code;
+        opted_in = true;
+    }
+    hipLaunchKernelGGL(route_metadata_kernel, dim3(1), dim3(kMetaThreads), g.shared, s, pointer_arg<const int>(args, 1),
+                       pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), pointer_arg<int>(args, 3),
+                       pointer_arg<int>(args, 4), pointer_arg<int>(args, 5), pointer_arg<int>(args, 6),
+                       pointer_arg<int>(args, 7), rows, f.E, f.top_k, f.block_m);
+    return hip_check(hipGetLastError(), "launch route_metadata");
+}
+int make_metadata(const Variant& v, orx_function* f) {
+    if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->block_m = (int)v.integer("block_m", 16, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // one expert per thread, one route per lane; the reference's own form is decode-only (M <= 1024)
+    if (f->M <= 0 || f->E <= 0 || f->E > kMetaThreads || f->top_k <= 0 || f->top_k > f->E || !valid_block_m(f->block_m) ||
+        (size_t)(kMetaWaves * f->E + 2 * kMetaWaves + 2 * (size_t)f->M * f->top_k) * sizeof(int) > 160 * 1024) {
+        set_error("route_metadata: need E <= 1024, top_k <= E, a valid block_m and M*top_k small enough for LDS");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"Counts", ArgPointer, 4},     {"IDs", ArgPointer, 4},        {"RelativeSlot", ArgPointer, 4},
+               {"RowOffsets", ArgPointer, 4}, {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
+               {"TileOffsets", ArgPointer, 4}, {"TileRow", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = metadata_geometry;
+    f->launch = metadata_launch;
+    f->device_function = reinterpret_cast<const void*>(&route_metadata_kernel);
+    return ORX_OK;
+}
+
 int dispatch_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)(rows * f.top_k);
     g->block[0] = 256;
@@ -399,12 +568,14 @@ const Registration* moe_registrations(int* count) {
     {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
     {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
+    {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false",
+     "Counts,IDs,RelativeSlot,RowOffsets,TileCount,TileExpert,TileOffsets,TileRow[,m]"},
     {"expert_dispatch", make_dispatch, "M, H, E=512, top_k=10, scale_group=H, dynamic_rows=false",
      "A,D,DS,IDs,RelativeSlot,RowOffsets,Scale,SlotMap[,m]"},
     {"moe_combine", make_combine, "M, H, slots=M*top_k, top_k=10, dynamic_rows=false",
      "Expert,Output,Prob,Shared,SharedGate,SlotMap[,m]"},
     };
-    *count = 6;
+    *count = 7;
     return rows;
 }
 

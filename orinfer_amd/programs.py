@@ -75,7 +75,7 @@ class MoeLayer:
     """Q2A8 expert layer: token-sort, grouped gate_up, SwiGLU->A8, grouped down, weighted combine."""
 
     def __init__(self, tokens, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales,
-                 block_m=32, packed_k=128):
+                 block_m=32, packed_k=128, fused_metadata=None):
         self.tokens, self.experts, self.top_k = tokens, experts, top_k
         self.hidden, self.inter, self.block_m = hidden, intermediate, block_m
         assignments = tokens * top_k
@@ -111,6 +111,11 @@ class MoeLayer:
         self.down_out = torch.empty((assignments, hidden), **f16)
         self.out = torch.empty((tokens, hidden), **f16)
         common = dict(M=tokens, E=experts, top_k=top_k)
+        # one launch for all routing metadata where the fused kernel applies (kernels/cuda/model/moe.py:713-764),
+        # the three-kernel form otherwise
+        if fused_metadata is None:
+            fused_metadata = experts <= 1024 and (16 * experts + 32 + 2 * tokens * top_k) * 4 <= 160 * 1024
+        self.k_metadata = Kernel("route_metadata", block_m=block_m, **common) if fused_metadata else None
         self.k_router = Kernel("router_topk", renormalize=True, **common)
         self.k_histogram = Kernel("expert_histogram", **common)
         self.k_offsets = Kernel("expert_offsets", E=experts, block_m=block_m)
@@ -126,11 +131,16 @@ class MoeLayer:
     def run(self, x16, logits, stream=None):
         s = stream
         self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
-        self.k_histogram(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative)
-        self.k_offsets(stream=s, Counts=self.counts, RowOffsets=self.row_offsets, TileCount=self.tile_count,
-                       TileOffsets=self.tile_offsets)
-        self.k_tiles(stream=s, Counts=self.counts, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
-                     TileRow=self.tile_row)
+        if self.k_metadata is not None:
+            self.k_metadata(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative,
+                            RowOffsets=self.row_offsets, TileCount=self.tile_count, TileExpert=self.tile_expert,
+                            TileOffsets=self.tile_offsets, TileRow=self.tile_row)
+        else:
+            self.k_histogram(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative)
+            self.k_offsets(stream=s, Counts=self.counts, RowOffsets=self.row_offsets, TileCount=self.tile_count,
+                           TileOffsets=self.tile_offsets)
+            self.k_tiles(stream=s, Counts=self.counts, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
+                         TileRow=self.tile_row)
         self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=self.tokens)
         self.k_dispatch(stream=s, A=self.a_q, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
                         RowOffsets=self.row_offsets, Scale=self.a_s, SlotMap=self.slot_map)

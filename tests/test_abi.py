@@ -61,6 +61,8 @@ ABI = {
     ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
     ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],
     ("expert_tiles", (("M", 64),)): ["Counts", "TileExpert", "TileOffsets", "TileRow"],
+    ("route_metadata", (("M", 64), ("E", 128), ("top_k", 8), ("block_m", 32), ("dynamic_rows", True))):
+        ["Counts", "IDs", "RelativeSlot", "RowOffsets", "TileCount", "TileExpert", "TileOffsets", "TileRow", "m"],
     ("expert_dispatch", (("M", 64), ("H", 2048))):
         ["A", "D", "DS", "IDs", "RelativeSlot", "RowOffsets", "Scale", "SlotMap"],
     ("moe_combine", (("M", 64), ("H", 2048), ("dynamic_rows", True))):

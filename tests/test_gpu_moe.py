@@ -78,6 +78,39 @@ def test_routing_metadata_and_dispatch(m, e, k, bm):
     np.testing.assert_array_equal(gu.host(ds), want_ds)
 
 
+@pytest.mark.parametrize("m,e,k,bm", [(256, 128, 8, 32), (37, 16, 4, 8), (1, 512, 10, 16), (300, 7, 3, 64), (5, 3, 3, 128),
+                                      (1024, 1024, 10, 16), (17, 64, 64, 8), (40, 100, 100, 16)])
+@pytest.mark.parametrize("repeats", [False, True], ids=["unique-routes", "repeated-routes"])
+def test_route_metadata_one_launch(m, e, k, bm, repeats):
+    """The fused form must write exactly what histogram + offsets + tiles write, also for dynamic
+    rows and when a token names one expert twice (ranked by route order)."""
+    rng = np.random.default_rng(orc.SEED + m + e)
+    ids_np = np.stack([rng.choice(e, k, replace=False) for _ in range(m)]).astype(np.int32)
+    if repeats and k > 1:
+        ids_np[:, -1] = ids_np[:, 0]
+        ids_np[0, :] = ids_np[0, 0]
+    cap_rows = m + 3
+    kern = gu.kernel("route_metadata", M=cap_rows, E=e, top_k=k, block_m=bm, dynamic_rows=True)
+    padded = np.full((cap_rows, k), 0, np.int32)
+    padded[:m] = ids_np
+    cap = orc.tile_capacity(cap_rows * k, e, bm)
+    out = {name: torch.full(shape, -1, **I32) for name, shape in
+           (("Counts", (e,)), ("RelativeSlot", (cap_rows, k)), ("RowOffsets", (e,)), ("TileCount", (1,)),
+            ("TileExpert", (cap,)), ("TileOffsets", (e,)), ("TileRow", (cap,)))}
+    kern(IDs=gu.dev(padded), m=m, **out)
+    want_counts, want_rel = orc.expert_histogram(ids_np, e)
+    want_rows, want_tiles, want_total = orc.expert_offsets(want_counts, bm)
+    want_te, want_tr = orc.expert_tiles(want_counts, want_tiles, bm, cap)
+    np.testing.assert_array_equal(gu.host(out["Counts"]), want_counts)
+    np.testing.assert_array_equal(gu.host(out["RelativeSlot"])[:m], want_rel)
+    assert (gu.host(out["RelativeSlot"])[m:] == -1).all()
+    np.testing.assert_array_equal(gu.host(out["RowOffsets"]), want_rows)
+    np.testing.assert_array_equal(gu.host(out["TileOffsets"]), want_tiles)
+    np.testing.assert_array_equal(gu.host(out["TileCount"]), want_total)
+    np.testing.assert_array_equal(gu.host(out["TileExpert"]), want_te)
+    np.testing.assert_array_equal(gu.host(out["TileRow"]), want_tr)
+
+
 @pytest.mark.parametrize("algorithm", ["auto", "mfma"])
 @pytest.mark.parametrize("packed_k", [128, 0])
 @pytest.mark.parametrize("bm", [32, 64, 128])
