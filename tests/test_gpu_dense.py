@@ -224,7 +224,7 @@ def q4_case(rng, m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
-@pytest.mark.parametrize("n,k", [(65, 256), (257, 2560), (1024, 5120)])
+@pytest.mark.parametrize("n,k", [(65, 256), (257, 2560), (1024, 5120), (130, 17408), (33, 8192 + 512), (70, 1536)])
 def test_q4_gemv_matches_oracle(m, n, k):
     rng = np.random.default_rng(orc.SEED + m + n)
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
