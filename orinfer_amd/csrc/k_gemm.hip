@@ -30,6 +30,13 @@ void stream_geometry(int n, Geometry* g);
 int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
+bool grouped_resident_eligible(int n, int k, int block_m, int tiles);
+bool grouped_resident_preferred(int rows, int experts, int n);
+void grouped_resident_geometry(int k, Geometry* g);
+int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                            void* out, const int* counts, const int* offsets, const int* tile_expert,
+                            const int* tile_row, const int* tile_count, int n, int k, int tiles, int packed_k,
+                            hipStream_t stream);
 int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, const int* counts, const int* offsets, const int* tile_expert, const int* tile_row,
                           const int* tile_count, int n, int k, int tiles, int block_m, int packed_k,
@@ -48,7 +55,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
-enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3 };
+enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4 };
 
 constexpr int kBK = 128;        // K bytes per tile step
 constexpr int kPitch = kBK + 16;  // LDS row pitch in bytes
@@ -569,8 +576,20 @@ int make_int8_swiglu(const Variant& v, orx_function* f) {
 // ---- routed single-stage experts -----------------------------------------------------------
 // A, AS, Book, C, Counts, Offsets, P, TileCount, TileExpert, TileRow, WS
 // (tests/cuda/operators/e8p_decode.py:72-84; kernels/cuda/model/e8p_decode.py:60-73 without Patch)
+// Resident kernel: forced by `algorithm=resident`, chosen by `auto` once the routed rows give every
+// CU a unit of its own.
+bool grouped_uses_resident(const orx_function& f) {
+    if (f.algorithm == kResident) return true;
+    return f.algorithm == kAuto && grouped_resident_eligible(f.N, f.K, f.block_m, f.tiles) &&
+           grouped_resident_preferred(f.capacity, f.E, f.N);
+}
+
 int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
     (void)rows;
+    if (grouped_uses_resident(f)) {
+        grouped_resident_geometry(f.K, g);
+        return ORX_OK;
+    }
     if (f.block_m <= 64 && f.algorithm != kMfma) {
         stream_grouped_geometry(f.N, f.tiles, g);
         return ORX_OK;
@@ -597,6 +616,9 @@ int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     p.ws = pointer_arg<const __half>(args, 10);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
+    if (grouped_uses_resident(f))
+        return grouped_resident_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
+                                       p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.packed_k, stream);
     if (f.block_m <= 64 && f.algorithm != kMfma)
         return stream_grouped_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
                                      p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.block_m, f.packed_k, stream);
@@ -615,11 +637,15 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     const std::string grouped_algorithm = v.string("algorithm", "auto", &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
-    if (grouped_algorithm != "auto" && grouped_algorithm != "mfma" && grouped_algorithm != "stream") {
-        set_error("%s: algorithm must be auto, stream or mfma", name);
+    if (grouped_algorithm != "auto" && grouped_algorithm != "mfma" && grouped_algorithm != "stream" &&
+        grouped_algorithm != "resident") {
+        set_error("%s: algorithm must be auto, stream, resident or mfma", name);
         return ORX_ERR_BAD_VARIANT;
     }
-    f->algorithm = grouped_algorithm == "mfma" ? kMfma : kAuto;
+    f->algorithm = grouped_algorithm == "mfma"       ? kMfma
+                   : grouped_algorithm == "stream"   ? kStream
+                   : grouped_algorithm == "resident" ? kResident
+                                                     : kAuto;
     if (f->M <= 0 || f->E <= 0 || f->tiles <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 ||
         (int64_t)f->K * 128 * 128 > 2147483647LL) {
         set_error("%s: invalid E8P decode geometry", name);  // e8p_decode.py:52
@@ -633,13 +659,19 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
         set_error("%s: packed_k must be 128 (K-major) or 0 (row-major per expert)", name);
         return ORX_ERR_BAD_VARIANT;
     }
+    if (f->algorithm == kResident && !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles)) {
+        set_error("%s: algorithm=resident needs block_m=32, at most 1024 tiles, N a multiple of 32 and K/128 even or a multiple of 3, K <= 2304",
+                  name);
+        return ORX_ERR_BAD_VARIANT;
+    }
     f->args = {{"A", ArgPointer, 16},         {"AS", ArgPointer, 2},         {"Book", ArgPointer, 4},
                {"C", ArgPointer, 2},          {"Counts", ArgPointer, 4},     {"Offsets", ArgPointer, 4},
                {"P", ArgPointer, 16},         {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
                {"TileRow", ArgPointer, 4},    {"WS", ArgPointer, 2}};
     f->geometry = grouped_geometry;
     f->launch = grouped_launch;
-    f->device_function = reinterpret_cast<const void*>(&gemm_kernel<kQ2, 32, 128, 1, true>);
+    // several kernels with different block sizes serve this symbol: report the device-wide limits
+    f->device_function = nullptr;
     return ORX_OK;
 }
 
@@ -699,9 +731,9 @@ const Registration* gemm_registrations(int* count) {
      "A,Output,TokenScale,Weight,WeightScale[,m]"},
     {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
-    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
+    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
-    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|mfma",
+    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},

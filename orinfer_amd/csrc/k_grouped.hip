@@ -1,0 +1,484 @@
+// Routed single-stage (Q2) expert projections when the routed tiles are many enough to occupy the
+// whole chip: one resident workgroup of 16 waves per CU.
+//
+// Reference counterpart: the warp-owned routed decode kernels/cuda/model/e8p_decode.py:36-245 (codes
+// go from global memory through a lookup table straight into MMA operand registers) behind the tile
+// metadata of kernels/cuda/model/routing.py.  Arithmetic: exact int32 over the full K,
+// (float(acc) * ws) * as, rounded to fp16 once.
+//
+// MI355X design.  The work is a weight stream (2 bits per weight, every expert's matrix read once
+// per routed tile) against at most 32 token rows per tile, so it is bound by HBM and by the decode.
+//  * A unit is (tile, 512 output channels): each of the 16 waves owns 32 channels over the full K,
+//    so there is no split-K reduction and no barrier inside a unit.  A wave streams its codes with
+//    one 16-byte load per lane and 128-wide K block through a register ring that is refilled right
+//    after use, also across the end of a unit into the first blocks of the next one.
+//  * The tile's activations are staged once per workgroup into LDS with coalesced 16-byte loads
+//    (rows padded by 16 bytes, so the per-lane 16-byte fragment reads do not collide); fetching
+//    them per lane from L1 costs one cache access per lane and instruction and was the limit of the
+//    streaming kernel this one replaces for large routed batches.
+//  * The two 8-byte table lookups per code are random; each table entry is stored 16 times (entry i
+//    for lane l at byte i*128 + (l%16)*8) so the lanes of one access group never share a bank.
+//  * Units are dealt to workgroups in contiguous runs (a run mostly stays inside one tile, so the
+//    staged rows are reused).  What does not divide evenly is finished in a second phase where a
+//    32-channel block is split over K between the waves and summed with LDS integer atomics
+//    (integer addition is exact in any order), so no CU has to run a whole extra unit.
+#include <hip/hip_fp16.h>
+
+#include "e8p_device.h"
+#include "orx_internal.h"
+
+namespace orx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kWaves = 16;
+constexpr int kThreads = kWaves * 64;
+constexpr int kSpan = kWaves * 32;             // output channels of one unit
+constexpr uint32_t kBasisBase = 0;             // 256 entries x 16 copies x 8 bytes
+constexpr uint32_t kMaskBase = 32768;
+constexpr uint32_t kInfoBase = 65536;          // (expert, first row, rows) of every routed tile
+constexpr int kMaxTiles = 1024;
+constexpr uint32_t kSumBase = kInfoBase + kMaxTiles * 12;  // phase-two sums, then the staged token rows
+constexpr int kRowPad = 16;
+constexpr int kSumStride = 33;                 // ints per token row of a phase-two sum block
+constexpr int kSumBlock = 32 * kSumStride;     // ints
+constexpr int kMaxPieces = 5;                  // 16-byte pieces a thread stages per tile (K <= 2560)
+
+struct GroupedParams {
+    const int8_t* a;
+    const uint8_t* w;
+    const uint32_t* book;
+    const __half* ws;
+    const __half* as;
+    __half* out;
+    const int* counts;
+    const int* offsets;
+    const int* tile_expert;
+    const int* tile_row;
+    const int* tile_count;
+    int n, k, k_major, tile_capacity;
+    int64_t expert_weight_stride;  // bytes
+};
+
+struct Tile {
+    int expert, row0, rows;
+};
+
+// The split of K between waves in phase two: K blocks per wave, waves per 32-channel block, blocks
+// a workgroup sums at once.
+struct Split {
+    int slice, ways, per_pass;
+};
+__host__ __device__ inline Split phase_two_split(int kb_count) {
+    Split s;
+    s.slice = (kb_count + kWaves - 1) / kWaves;
+    s.ways = (kb_count + s.slice - 1) / s.slice;
+    s.per_pass = kWaves / s.ways;
+    return s;
+}
+
+// D: K blocks per ring group (the ring depth); K/128 is a multiple of it.
+template <int D>
+__global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5, frag = lane & 31;
+    const int kb_count = p.k / 128;
+    const int spans = (p.n + kSpan - 1) / kSpan;
+    const int groups = (int)gridDim.x, group = (int)blockIdx.x;
+    const Split split = phase_two_split(kb_count);
+    const uint32_t tile_base = kSumBase + (uint32_t)split.per_pass * kSumBlock * 4;
+    const int tile_stride = p.k + kRowPad;
+    int* sums = reinterpret_cast<int*>(lds + kSumBase);
+
+    // ---- set-up: two round trips to memory, then one barrier ------------------------------------
+    // First trip: the selector table (waves 0-3 build the basis table from it, waves 4-7 the mask
+    // table, which needs no load), the tile count and, one tile per thread, every tile's expert and
+    // first row.  Second trip: that expert's row count and offset.  The tile list then sits in LDS,
+    // so nothing later in the kernel waits for a chain of dependent loads.
+    uint32_t selector = 0;
+    if (wave < 4) selector = p.book[tid];
+    const int listed = min(p.tile_capacity, kMaxTiles);
+    const int my_tile = min(tid, listed - 1);
+    const int my_expert = p.tile_expert[my_tile], my_first = p.tile_row[my_tile];
+    const int tile_count = min(p.tile_count[0], listed);
+    const bool listed_here = tid < tile_count;
+    const int safe_expert = listed_here ? my_expert : 0;  // entries beyond the count are not initialised
+    const int my_count = p.counts[safe_expert], my_offset = p.offsets[safe_expert];
+    if (wave < 8) {
+        const int entry = tid & 255;
+        const uint2 value = wave < 4 ? byte_basis_signed(selector) : byte_mask_signed((uint32_t)entry);
+        const uint4 pair = make_uint4(value.x, value.y, value.x, value.y);
+        uint8_t* dst = lds + (wave < 4 ? kBasisBase : kMaskBase) + entry * 128;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
+    }
+    for (int i = tid; i < split.per_pass * kSumBlock; i += kThreads) sums[i] = 0;
+    if (listed_here) {
+        int* info = reinterpret_cast<int*>(lds + kInfoBase) + 3 * tid;
+        info[0] = my_expert, info[1] = my_offset + my_first, info[2] = min(32, my_count - my_first);
+    }
+    __syncthreads();
+    auto tile_info = [&](int tile) {
+        const int* info = reinterpret_cast<const int*>(lds + kInfoBase) + 3 * tile;
+        Tile t;
+        t.expert = __builtin_amdgcn_readfirstlane(info[0]);
+        t.row0 = __builtin_amdgcn_readfirstlane(info[1]);
+        t.rows = __builtin_amdgcn_readfirstlane(info[2]);
+        return t;
+    };
+
+    // ---- how the units are dealt -----------------------------------------------------------
+    // Every workgroup runs `full` units; the rest is either one more unit for the first
+    // workgroups or, when that rest is small, split over K in phase two.  Runs are contiguous, so
+    // a run mostly stays inside one tile and its staged rows are reused.
+    const int units = tile_count * spans;
+    const int full = units / groups;
+    int leftover = units - full * groups;
+    const int passes = (leftover * kWaves + groups * split.per_pass - 1) / (groups * split.per_pass);
+    int my_units = full, first_unit = group * full;
+    if (passes > max(1, kb_count / 8)) {
+        first_unit += min(group, leftover);
+        if (group < leftover) ++my_units;
+        leftover = 0;
+    }
+
+    // ---- weight stream of this lane ----------------------------------------------------------
+    const int64_t kb_step = p.k_major ? (int64_t)p.n * 32 : 32;
+    auto lane_weights = [&](int expert, int n0) -> const uint8_t* {
+        const int64_t row = n0 + frag;
+        const int64_t offset = p.k_major ? row * 32 : row * kb_count * 32;
+        return p.w + (int64_t)expert * p.expert_weight_stride + offset + half * 16;
+    };
+    auto fetch = [&](const uint8_t* base, int kb) { return *reinterpret_cast<const uint4*>(base + kb * kb_step); };
+
+    // ---- decode ------------------------------------------------------------------------------
+    const uint32_t copy = (uint32_t)(lane & 15) * 8;
+    auto lookup = [&](uint32_t byte) { return *reinterpret_cast<const uint2*>(lds + byte); };
+    auto decode_pair = [&](uint32_t word) -> v4i {  // two codes -> the 16 weights of one MFMA sub-step
+        const uint2 b0 = lookup(kBasisBase + (((word & 0xFF00u) >> 1) | copy));
+        const uint2 m0 = lookup(kMaskBase + (((word & 0xFFu) << 7) | copy));
+        const uint2 b1 = lookup(kBasisBase + (((word >> 17) & 0x7F80u) | copy));
+        const uint2 m1 = lookup(kMaskBase + (((word >> 9) & 0x7F80u) | copy));
+        return v4i{(int)(b0.x ^ m0.x), (int)(b0.y ^ m0.y), (int)(b1.x ^ m1.x), (int)(b1.y ^ m1.y)};
+    };
+
+    // ---- staging of a tile's token rows ------------------------------------------------------
+    const int row_pieces = p.k / 16;
+    auto stage_store_piece = [&](int pieces, int piece, const uint4& value) {
+        if (piece < pieces) {
+            const int row = piece / row_pieces, col = piece - row * row_pieces;
+            *reinterpret_cast<uint4*>(lds + tile_base + row * tile_stride + col * 16) = value;
+        }
+    };
+
+    // accumulator register r of a lane: channel 8*(r/4) + 4*half + r%4 of the block, token `frag`
+    struct Scales {
+        uint2 weight[4];  // four fp16 channel scales per 8-channel step
+        __half token;
+    };
+    auto load_scales = [&](int expert, int64_t row, int n0) {
+        Scales s;
+        const __half* scales = p.ws + (int64_t)expert * p.n + n0 + 4 * half;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s.weight[j] = *reinterpret_cast<const uint2*>(scales + 8 * j);
+        s.token = p.as[row];
+        return s;
+    };
+    auto store_block = [&](const v16i& acc, const Scales& scales, int64_t row, int n0) {
+        const float token_scale = __half2float(scales.token);
+        __half* dst = p.out + row * p.n + n0 + 4 * half;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint2 bits = scales.weight[j];
+            const __half2 s01 = *reinterpret_cast<const __half2*>(&bits.x), s23 = *reinterpret_cast<const __half2*>(&bits.y);
+            const float s[4] = {__low2float(s01), __high2float(s01), __low2float(s23), __high2float(s23)};
+            __half h[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[i] = __float2half_rn(rescale(acc[4 * j + i], s[i], token_scale));
+            uint2 packed;
+            packed.x = (uint32_t)__half_as_ushort(h[0]) | (uint32_t)__half_as_ushort(h[1]) << 16;
+            packed.y = (uint32_t)__half_as_ushort(h[2]) | (uint32_t)__half_as_ushort(h[3]) << 16;
+            *reinterpret_cast<uint2*>(dst + 8 * j) = packed;
+        }
+    };
+
+    struct Unit {
+        int tile, n0, expert, row0, rows;  // n0: first channel of this wave; rows <= 0: nothing to do
+    };
+    auto unit_at = [&](int u) {
+        Unit unit = {-1, 0, 0, 0, 0};
+        if (u < my_units) {
+            const int index = first_unit + u;
+            unit.tile = index / spans;
+            unit.n0 = (index - unit.tile * spans) * kSpan + wave * 32;
+            const Tile t = tile_info(unit.tile);
+            unit.expert = t.expert, unit.row0 = t.row0, unit.rows = unit.n0 < p.n ? t.rows : 0;
+        }
+        return unit;
+    };
+
+    // ---- phase two's work of this wave (first pass), requested now and used at the very end --------
+    const int blocks = leftover * kWaves, first_leftover = full * groups;
+    const int local = wave / split.ways, part = wave - local * split.ways;
+    struct Piece {
+        int n0, kb_first, kb_last;
+        Tile tile;
+        bool active;
+    };
+    auto piece_of = [&](int pass) {
+        Piece piece = {0, 0, 0, {0, 0, 0}, false};
+        const int block = (pass * groups + group) * split.per_pass + local;
+        if (local < split.per_pass && block < blocks) {
+            const int unit = first_leftover + block / kWaves;
+            const int tile = unit / spans;
+            piece.n0 = (unit - tile * spans) * kSpan + (block % kWaves) * 32;
+            piece.tile = tile_info(tile);
+            piece.kb_first = part * split.slice;
+            piece.kb_last = min(kb_count, piece.kb_first + split.slice);
+            piece.active = piece.n0 < p.n && piece.tile.rows > 0 && piece.kb_first < piece.kb_last;
+        }
+        return piece;
+    };
+    auto piece_rows = [&](const Piece& piece) {
+        return p.a + (int64_t)(piece.tile.row0 + min(frag, piece.tile.rows - 1)) * p.k + half * 64;
+    };
+    const Piece early = piece_of(0);
+    uint4 early_codes = make_uint4(0, 0, 0, 0), early_tokens[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) early_tokens[s] = make_uint4(0, 0, 0, 0);
+
+    // ---- phase one: whole units ------------------------------------------------------------------
+    Tile staged_tile = {0, 0, 0};
+    int staged = -1;
+    uint4 ring[D];
+    bool ring_ready = false;
+    for (int u = 0; u < my_units; ++u) {
+        const Unit cur = unit_at(u), nxt = unit_at(u + 1);
+        if (cur.tile != staged) {
+            staged_tile = tile_info(cur.tile);
+            // unconditional loads of clamped pieces (named registers, not an array: an array would be
+            // kept in scratch memory), so that all of them are in flight together
+            const uint4* src =
+                reinterpret_cast<const uint4*>(p.a + (int64_t)(staged_tile.rows > 0 ? staged_tile.row0 : 0) * p.k);
+            const int pieces = staged_tile.rows * row_pieces, last_piece = max(pieces, 1) - 1;
+            const uint4 held0 = src[min(tid, last_piece)], held1 = src[min(tid + kThreads, last_piece)],
+                        held2 = src[min(tid + 2 * kThreads, last_piece)], held3 = src[min(tid + 3 * kThreads, last_piece)],
+                        held4 = src[min(tid + 4 * kThreads, last_piece)];
+            static_assert(kMaxPieces == 5, "one named register per piece");
+            if (u == 0) {
+                // the first codes and phase two's operands travel together with the first tile's rows
+                if (cur.rows > 0) {
+                    const uint8_t* weights = lane_weights(cur.expert, cur.n0);
+#pragma unroll
+                    for (int d = 0; d < D; ++d) ring[d] = fetch(weights, d);
+                    ring_ready = true;
+                }
+            } else {
+                __syncthreads();  // every wave has finished with the rows staged before
+            }
+            stage_store_piece(pieces, tid, held0);
+            stage_store_piece(pieces, tid + kThreads, held1);
+            stage_store_piece(pieces, tid + 2 * kThreads, held2);
+            stage_store_piece(pieces, tid + 3 * kThreads, held3);
+            stage_store_piece(pieces, tid + 4 * kThreads, held4);
+            staged = cur.tile;
+            __syncthreads();
+        }
+        // the same wave's block in the next unit, for the refill that crosses the unit's end
+        const bool have_next = nxt.rows > 0;
+        const uint8_t* next_weights = lane_weights(have_next ? nxt.expert : 0, have_next ? nxt.n0 : 0);
+        if (cur.rows <= 0) {
+            ring_ready = false;
+            if (have_next) {
+#pragma unroll
+                for (int d = 0; d < D; ++d) ring[d] = fetch(next_weights, d);
+                ring_ready = true;
+            }
+        } else {
+            const uint8_t* weights = lane_weights(cur.expert, cur.n0);
+            if (!ring_ready) {
+#pragma unroll
+                for (int d = 0; d < D; ++d) ring[d] = fetch(weights, d);
+            }
+            const int64_t row = cur.row0 + min(frag, cur.rows - 1);
+            const Scales scales = load_scales(cur.expert, row, cur.n0);
+            const uint8_t* rows = lds + tile_base + min(frag, cur.rows - 1) * tile_stride + half * 64;
+            v16i acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0;
+            for (int g = 0; g < kb_count; g += D) {
+                const bool last = g + D >= kb_count;
+#pragma unroll
+                for (int d = 0; d < D; ++d) {
+                    const uint4 codes = ring[d];
+                    const uint8_t* refill = last ? next_weights : weights + (g + D) * kb_step;
+                    if (!last || have_next) ring[d] = fetch(refill, d);
+                    const uint32_t word[4] = {codes.x, codes.y, codes.z, codes.w};
+                    const uint8_t* fragment = rows + (g + d) * 128;
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        const v4i weight_operand = decode_pair(word[s]);
+                        const v4i token_operand = *reinterpret_cast<const v4i*>(fragment + 16 * s);
+                        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(weight_operand, token_operand, acc, 0, 0, 0);
+                    }
+                }
+            }
+            ring_ready = have_next;
+            if (u + 1 == my_units && early.active) {
+                // last unit: phase two's first operands are requested before the stores are waited for
+                early_codes = fetch(lane_weights(early.tile.expert, early.n0), early.kb_first);
+                const uint4* fragment = reinterpret_cast<const uint4*>(piece_rows(early) + early.kb_first * 128);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) early_tokens[s] = fragment[s];
+            }
+            if (frag < cur.rows) store_block(acc, scales, row, cur.n0);
+        }
+    }
+
+    // ---- phase two: the rest, 32-channel blocks split over K between waves ----------------------
+    if (leftover == 0) return;
+    const bool early_loaded = my_units > 0 && unit_at(my_units - 1).rows > 0;
+    for (int pass = 0; (pass * groups + group) * split.per_pass < blocks; ++pass) {
+        const int first_block = (pass * groups + group) * split.per_pass;
+        if (pass > 0) {
+            __syncthreads();  // the previous pass's sums have been read
+            for (int i = tid; i < split.per_pass * kSumBlock; i += kThreads) sums[i] = 0;
+            __syncthreads();
+        }
+        const Piece piece = pass == 0 ? early : piece_of(pass);
+        if (piece.active) {
+            const uint8_t* weights = lane_weights(piece.tile.expert, piece.n0);
+            const int8_t* rows = piece_rows(piece);
+            v16i acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0;
+            auto multiply = [&](const uint4& codes, const uint4 (&tokens)[4]) {
+                const uint32_t word[4] = {codes.x, codes.y, codes.z, codes.w};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const v4i weight_operand = decode_pair(word[s]);
+                    const v4i token_operand = {(int)tokens[s].x, (int)tokens[s].y, (int)tokens[s].z, (int)tokens[s].w};
+                    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(weight_operand, token_operand, acc, 0, 0, 0);
+                }
+            };
+            int kb = piece.kb_first;
+            if (pass == 0 && early_loaded) {
+                multiply(early_codes, early_tokens);
+                ++kb;
+            }
+            for (; kb < piece.kb_last; ++kb) {
+                const uint4 codes = fetch(weights, kb);
+                const uint4* fragment = reinterpret_cast<const uint4*>(rows + kb * 128);
+                const uint4 tokens[4] = {fragment[0], fragment[1], fragment[2], fragment[3]};
+                multiply(codes, tokens);
+            }
+            int* mine = sums + local * kSumBlock + frag * kSumStride + 4 * half;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) atomicAdd(mine + 8 * (r >> 2) + (r & 3), acc[r]);
+        }
+        __syncthreads();
+        for (int e = 0; e < split.per_pass; ++e) {
+            const int done = first_block + e;
+            if (done >= blocks) break;
+            const int unit = first_leftover + done / kWaves;
+            const int tile = unit / spans;
+            const int n0 = (unit - tile * spans) * kSpan + (done % kWaves) * 32;
+            const Tile t = tile_info(tile);
+            const int token = tid >> 5, channel = tid & 31;
+            if (n0 >= p.n || token >= t.rows) continue;
+            const int64_t row = t.row0 + token;
+            const int total = sums[e * kSumBlock + token * kSumStride + channel];
+            const float value = rescale(total, __half2float(p.ws[(int64_t)t.expert * p.n + n0 + channel]),
+                                        __half2float(p.as[row]));
+            p.out[row * p.n + n0 + channel] = __float2half_rn(value);
+        }
+    }
+}
+
+int device_compute_units() {
+    static int units = 0;
+    if (units == 0) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess)
+            units = prop.multiProcessorCount;
+        else
+            (void)hipGetLastError();
+        if (units <= 0) units = 256;
+    }
+    return units;
+}
+
+int ring_depth(int k) {
+    const int kb = k / 128;
+    return kb % 2 == 0 ? 2 : kb % 3 == 0 ? 3 : 0;
+}
+
+uint32_t resident_lds_bytes(int k) {
+    const Split split = phase_two_split(k / 128);
+    return kSumBase + (uint32_t)split.per_pass * kSumBlock * 4u + 32u * (uint32_t)(k + kRowPad);
+}
+
+constexpr uint32_t kLdsLimit = 160 * 1024;
+
+}  // namespace
+
+// Shapes the resident kernel takes: tiles of at most 32 rows, whole 32-channel blocks, a K whose
+// blocks divide into ring groups and whose staged rows fit beside the tables.
+bool grouped_resident_eligible(int n, int k, int block_m, int tiles) {
+    return block_m == 32 && n % 32 == 0 && k % 128 == 0 && ring_depth(k) > 0 && tiles <= kMaxTiles &&
+           k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k) <= kLdsLimit;
+}
+
+// Worth it once the routed tiles give every CU at least one unit; below that the streaming kernel's
+// many small workgroups spread better.
+bool grouped_resident_preferred(int rows, int experts, int n) {
+    const int tiles = max((rows + 31) / 32, min(experts, rows));
+    return (int64_t)tiles * ((n + kSpan - 1) / kSpan) >= device_compute_units();
+}
+
+void grouped_resident_geometry(int k, Geometry* g) {
+    g->grid[0] = (uint32_t)device_compute_units();
+    g->grid[1] = g->grid[2] = 1;
+    g->block[0] = kThreads;
+    g->shared = resident_lds_bytes(k);
+}
+
+int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                            void* out, const int* counts, const int* offsets, const int* tile_expert,
+                            const int* tile_row, const int* tile_count, int n, int k, int tiles, int packed_k,
+                            hipStream_t stream) {
+    static bool opted_in = false;
+    if (!opted_in) {
+        // Dynamic LDS above 64 KiB needs an opt-in per kernel.
+        const void* kernels[] = {reinterpret_cast<const void*>(&grouped_resident_kernel<3>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2>)};
+        for (const void* kernel : kernels) {
+            const int code = hip_check(
+                hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit), "hipFuncSetAttribute");
+            if (code != ORX_OK) return code;
+        }
+        opted_in = true;
+    }
+    GroupedParams p = {};
+    p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as;
+    p.out = reinterpret_cast<__half*>(out);
+    p.counts = counts, p.offsets = offsets, p.tile_expert = tile_expert, p.tile_row = tile_row, p.tile_count = tile_count;
+    p.n = n, p.k = k, p.k_major = packed_k != 0, p.tile_capacity = tiles;
+    p.expert_weight_stride = (int64_t)n * (k / 8) * 2;
+    Geometry g;
+    grouped_resident_geometry(k, &g);
+    const dim3 grid(g.grid[0]), block(kThreads);
+    switch (ring_depth(k)) {
+        case 3: hipLaunchKernelGGL(grouped_resident_kernel<3>, grid, block, g.shared, stream, p); break;
+        case 2: hipLaunchKernelGGL(grouped_resident_kernel<2>, grid, block, g.shared, stream, p); break;
+        default: set_error("routed projection: K=%d does not divide into ring groups", k); return ORX_ERR_BAD_VARIANT;
+    }
+    return hip_check(hipGetLastError(), "launch routed projection (resident)");
+}
+
+}  // namespace orx

@@ -160,6 +160,83 @@ def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k, algorithm):
     np.testing.assert_array_equal(got[hi:rows], want[hi:])
 
 
+# Cases of the resident routed kernel (one 16-wave workgroup per CU, units of one tile x 512
+# channels).  With 256 CUs: whole units plus a K-split rest for three ring depths and both split
+# widths, a launch that is K-split only, one extra unit for some workgroups, and runs of three
+# units that change tile in the middle.
+RESIDENT_CASES = {
+    "units-and-rest-k512": dict(e=64, n=1536, k=512, high=70),
+    "units-and-rest-k384": dict(e=9, n=14848, k=384, counts=[0, 1, 32, 33, 0, 95, 7, 0, 2]),
+    "rest-only-k256": dict(e=40, n=512, k=256, high=40),
+    "extra-unit-k2048": dict(e=50, n=1024, k=2048, high=20),
+    "tile-change-k512": dict(e=128, n=1536, k=512, high=80),
+}
+
+
+@pytest.mark.parametrize("packed_k", [128, 0])
+@pytest.mark.parametrize("case", list(RESIDENT_CASES))
+def test_grouped_q2_resident_kernel(case, packed_k):
+    spec = RESIDENT_CASES[case]
+    e, n, k, bm = spec["e"], spec["n"], spec["k"], 32
+    rng = np.random.default_rng(orc.SEED + e + k)
+    if "counts" in spec:
+        counts_np = np.array(spec["counts"], np.int32)
+    else:
+        counts_np = rng.integers(0, spec["high"] + 1, e).astype(np.int32)
+        counts_np[rng.integers(0, e, max(1, e // 10))] = 0
+    rows = int(counts_np.sum())
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_q[0, :2] = [-128, 127]
+    a_s = rng.uniform(0.01, 0.03, rows).astype(np.float16)
+    offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+    cap = orc.tile_capacity(rows, e, bm)
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+    stored = codes if packed_k == 0 else np.stack([orc.q2_pack_k128(c) for c in codes])
+    out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
+    kern = gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
+                     algorithm="resident")
+    assert tuple(kern.geometry()[1])[0] == 1024
+    counts = gu.dev(counts_np)
+    tile_count = gu.dev(total)
+    args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=counts, Offsets=gu.dev(offsets_np),
+                P=gu.dev(stored), TileCount=tile_count, TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
+    kern(**args)
+    w = np.stack([orc.q2_integers(c, TABLE) for c in codes])
+    want = orc.grouped_project(a_q, a_s[:, None], w, ws, counts_np, offsets_np)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows] == 55).all()
+    # the streaming kernel gives the same bytes
+    other = torch.full_like(out, 55.0)
+    gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
+              algorithm="stream")(**{**args, "C": other})
+    assert torch.equal(out, other)
+    # a zero tile count leaves C untouched; a zeroed expert count skips exactly its rows
+    out.fill_(55)
+    tile_count.zero_()
+    kern(**args)
+    assert bool((out == 55).all())
+    tile_count.copy_(gu.dev(total))
+    hot = int(np.argmax(counts_np))
+    counts[hot] = 0
+    kern(**args)
+    got = gu.host(out)
+    lo, hi = offsets_np[hot], offsets_np[hot] + counts_np[hot]
+    assert (got[lo:hi] == 55).all()
+    np.testing.assert_array_equal(got[:lo], want[:lo])
+    np.testing.assert_array_equal(got[hi:rows], want[hi:])
+
+
+def test_grouped_resident_rejects_shapes_it_cannot_take():
+    for bad in (dict(N=200, K=384), dict(N=256, K=128), dict(N=256, K=3072), dict(N=256, K=512, block_m=64)):
+        variant = dict(rows=64, E=4, tiles=6, block_m=32, packed_k=128, algorithm="resident")
+        variant.update(bad)
+        with pytest.raises(Exception, match="resident"):
+            gu.kernel("e8p_decode_grouped", **variant)
+
+
 @pytest.mark.parametrize("m,h,slots", [(1, 2560, 10), (8, 2560, 80), (17, 257, 37), (512, 2560, 5120)])
 def test_combine_invalid_slots_and_shared_expert(m, h, slots):
     # tests/cuda/operators/moe.py:98-118
