@@ -52,6 +52,9 @@ int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* boo
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+// Register arrays hold the native vector type: an array of HIP's uint4 struct that is filled in
+// one lambda and read in another is kept in scratch memory by the compiler.
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
@@ -135,14 +138,14 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, 256);
 
     const int k_tiles = p.k / kBK;
-    uint4 reg_a[A_CHUNKS], reg_w[W_CHUNKS];
+    v4u held_a[A_CHUNKS], held_w[W_CHUNKS];
 
-    auto load_tile = [&](int kt) {
+    auto load_tile = [&](int kt, v4u (&reg_a)[A_CHUNKS], v4u (&reg_w)[W_CHUNKS]) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + 256 * i;
             const int r = min(c >> 3, rows_here - 1), kc = c & 7;
-            reg_a[i] = *reinterpret_cast<const uint4*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
+            reg_a[i] = *reinterpret_cast<const v4u*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
@@ -156,15 +159,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
                 byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
             else  // (N, K/8 codes)
                 byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
-            reg_w[i] = *reinterpret_cast<const uint4*>(w_base + byte);
+            reg_w[i] = *reinterpret_cast<const v4u*>(w_base + byte);
         }
     };
 
-    auto store_tile = [&]() {
+    auto store_tile = [&](const v4u (&reg_a)[A_CHUNKS], const v4u (&reg_w)[W_CHUNKS]) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + 256 * i;
-            *reinterpret_cast<uint4*>(lds_a + (c >> 3) * kPitch + (c & 7) * 16) = reg_a[i];
+            *reinterpret_cast<v4u*>(lds_a + (c >> 3) * kPitch + (c & 7) * 16) = reg_a[i];
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             constexpr int PER_ROW = weight_chunks<CODEC>();
             const int nn = c / PER_ROW, q = c % PER_ROW;
             if constexpr (CODEC == kW8) {
-                *reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
+                *reinterpret_cast<v4u*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
             } else if constexpr (CODEC == kQ4) {
                 // 4 u32 codes -> 32 weights at k offset q*32
                 const uint2 d0 = decode_q4(tables, reg_w[i].x), d1 = decode_q4(tables, reg_w[i].y);
@@ -201,12 +204,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    load_tile(0);
+    load_tile(0, held_a, held_w);
     __syncthreads();  // tables ready
     for (int kt = 0; kt < k_tiles; ++kt) {
-        store_tile();
+        store_tile(held_a, held_w);
         __syncthreads();
-        if (kt + 1 < k_tiles) load_tile(kt + 1);
+        if (kt + 1 < k_tiles) load_tile(kt + 1, held_a, held_w);
         const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
 #pragma unroll
         for (int ks = 0; ks < kBK / 32; ++ks) {

@@ -31,6 +31,7 @@ namespace orx {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTile = 256;     // output tile edge
@@ -137,7 +138,7 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
     // Q4: one K step of the weight tile is 256 rows x 64 bytes of codes = 1024 chunks of 16 bytes
     // (4 codes = 32 weights each): CODE_CHUNKS chunks per thread.
     // Two register sets so that the codes of step t+1 can be in flight while step t is decoded.
-    uint4 code_regs[2][CODE_CHUNKS];
+    v4u code_regs[2][CODE_CHUNKS];  // native vectors: an array of HIP's uint4 struct would live in scratch memory
     auto load_codes = [&](int kt, int set) {
 #pragma unroll
         for (int i = 0; i < CODE_CHUNKS; ++i) {
@@ -148,7 +149,7 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
                 byte = ((int64_t)kt * p.n + col0 + row) * 64 + q * 16;
             else
                 byte = ((int64_t)(col0 + row) * (p.k / kStep) + kt) * 64 + q * 16;
-            code_regs[set][i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(p.w) + byte);
+            code_regs[set][i] = *reinterpret_cast<const v4u*>(reinterpret_cast<const int8_t*>(p.w) + byte);
         }
     };
     // Decode the codes of one K step (4 codes -> 32 weights -> two 16-byte LDS stores per chunk).
@@ -157,7 +158,7 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
         for (int i = 0; i < CODE_CHUNKS; ++i) {
             const int c = tid + kThreads * i;
             const int row = c >> 2, q = c & 3;
-            const uint4 codes = code_regs[set][i];
+            const v4u codes = code_regs[set][i];
             const uint2 d0 = decode_q4(*tables, codes.x), d1 = decode_q4(*tables, codes.y);
             const uint2 d2 = decode_q4(*tables, codes.z), d3 = decode_q4(*tables, codes.w);
             int8_t* row_base = stage + row * kStep;

@@ -32,6 +32,7 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 16;
 constexpr int kThreads = kWaves * 64;
@@ -167,11 +168,26 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     };
 
     // ---- staging of a tile's token rows ------------------------------------------------------
+    // Register arrays hold the native vector type: an array of HIP's uint4 struct that is filled in
+    // one lambda and read in another is kept in scratch memory by the compiler.
+    v4u held[kMaxPieces];
     const int row_pieces = p.k / 16;
-    auto stage_store_piece = [&](int pieces, int piece, const uint4& value) {
-        if (piece < pieces) {
-            const int row = piece / row_pieces, col = piece - row * row_pieces;
-            *reinterpret_cast<uint4*>(lds + tile_base + row * tile_stride + col * 16) = value;
+    auto stage_load = [&](const Tile& t) {
+        // unconditional loads of clamped pieces, so that all of them are in flight together
+        const v4u* src = reinterpret_cast<const v4u*>(p.a + (int64_t)(t.rows > 0 ? t.row0 : 0) * p.k);
+        const int last_piece = max(t.rows * row_pieces, 1) - 1;
+#pragma unroll
+        for (int i = 0; i < kMaxPieces; ++i) held[i] = src[min(tid + i * kThreads, last_piece)];
+    };
+    auto stage_store = [&](const Tile& t) {
+        const int pieces = t.rows * row_pieces;
+#pragma unroll
+        for (int i = 0; i < kMaxPieces; ++i) {
+            const int piece = tid + i * kThreads;
+            if (piece < pieces) {
+                const int row = piece / row_pieces, col = piece - row * row_pieces;
+                *reinterpret_cast<v4u*>(lds + tile_base + row * tile_stride + col * 16) = held[i];
+            }
         }
     };
 
@@ -260,15 +276,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
         const Unit cur = unit_at(u), nxt = unit_at(u + 1);
         if (cur.tile != staged) {
             staged_tile = tile_info(cur.tile);
-            // unconditional loads of clamped pieces (named registers, not an array: an array would be
-            // kept in scratch memory), so that all of them are in flight together
-            const uint4* src =
-                reinterpret_cast<const uint4*>(p.a + (int64_t)(staged_tile.rows > 0 ? staged_tile.row0 : 0) * p.k);
-            const int pieces = staged_tile.rows * row_pieces, last_piece = max(pieces, 1) - 1;
-            const uint4 held0 = src[min(tid, last_piece)], held1 = src[min(tid + kThreads, last_piece)],
-                        held2 = src[min(tid + 2 * kThreads, last_piece)], held3 = src[min(tid + 3 * kThreads, last_piece)],
-                        held4 = src[min(tid + 4 * kThreads, last_piece)];
-            static_assert(kMaxPieces == 5, "one named register per piece");
+            stage_load(staged_tile);
             if (u == 0) {
                 // the first codes and phase two's operands travel together with the first tile's rows
                 if (cur.rows > 0) {
@@ -280,11 +288,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
             } else {
                 __syncthreads();  // every wave has finished with the rows staged before
             }
-            stage_store_piece(pieces, tid, held0);
-            stage_store_piece(pieces, tid + kThreads, held1);
-            stage_store_piece(pieces, tid + 2 * kThreads, held2);
-            stage_store_piece(pieces, tid + 3 * kThreads, held3);
-            stage_store_piece(pieces, tid + 4 * kThreads, held4);
+            stage_store(staged_tile);
             staged = cur.tile;
             __syncthreads();
         }
