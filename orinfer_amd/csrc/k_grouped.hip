@@ -24,6 +24,9 @@
 //    (integer addition is exact in any order), so no CU has to run a whole extra unit.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
+#include <cmath>
+
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -438,11 +441,14 @@ bool grouped_resident_eligible(int n, int k, int block_m, int tiles) {
            k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k) <= kLdsLimit;
 }
 
-// Worth it once the routed tiles give every CU at least one unit; below that the streaming kernel's
-// many small workgroups spread better.
+// Worth it once the routed tiles give most CUs a unit of their own; below that the streaming
+// kernel's many small workgroups spread better (measured crossover: about 32 tokens x top-8 over 128
+// experts).  The tile count is only known on the device; with uniform routing `rows` assignments hit
+// about E (1 - exp(-rows / E)) experts.
 bool grouped_resident_preferred(int rows, int experts, int n) {
-    const int tiles = max((rows + 31) / 32, min(experts, rows));
-    return (int64_t)tiles * ((n + kSpan - 1) / kSpan) >= device_compute_units();
+    const double hit = experts * (1.0 - std::exp(-(double)rows / experts));
+    const double tiles = std::max((double)((rows + 31) / 32), hit);
+    return tiles * ((n + kSpan - 1) / kSpan) >= 0.8 * device_compute_units();
 }
 
 void grouped_resident_geometry(int k, Geometry* g) {
