@@ -1,0 +1,289 @@
+// Two-stage (Q4) projections for 5..32 token rows (batched decode): one resident workgroup of 16
+// waves per CU, the whole weight stream of a wave requested up front.
+//
+// Reference counterparts: the small-row Tensor Core schedules of kernels/cuda/model/integer_core.py
+// (block_m 8..32) behind kernels/cuda/model/e8p_q4.py:143-264.  Arithmetic: exact int32 over the full
+// K, (float(acc) * ws) * as.
+//
+// MI355X design.  With so few rows the projection is a weight stream (0.5 byte per weight) and the
+// kernel is shaped so that nothing but that stream touches memory inside the loop:
+//  * Output channels are dealt to CUs in equal contiguous runs (N / CUs each, 68 at N = 17408), cut
+//    into blocks of 16 channels for v_mfma_i32_16x16x64_i8, so every CU has the same work.
+//  * K is split over the 16 waves.  A wave keeps the token fragments of its K slice in registers for
+//    the whole kernel (they are the same for every channel block), so activations are read once
+//    per CU; its codes stream through a ring of P channel blocks that is refilled right after use.
+//  * Codes are decoded with two 8-byte lookups per stage in tables stored 16 times (entry i for
+//    lane l at byte i*128 + (l%16)*8), so the lanes of one access group never share a bank; the two
+//    stages share one pair of tables (values v+8, shifted by the stage's weight when combined).
+//  * The 16 K-slice partial sums of a block are added with LDS integer atomics (exact in any order)
+//    into a buffer per block; one barrier per group of P blocks, then 16 x M threads rescale and
+//    store the group while the other waves already decode the next one.
+#include <hip/hip_fp16.h>
+
+#include "e8p_device.h"
+#include "orx_internal.h"
+
+namespace orx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 16;
+constexpr int kThreads = kWaves * 64;
+constexpr uint32_t kBasisBase = 0;        // 256 entries x 16 copies x 8 bytes: (h ^ 8) per coordinate
+constexpr uint32_t kMaskBase = 32768;     // the same for the sign/parity masks
+constexpr uint32_t kSumBase = 65536;      // two sets of kMaxHeld buffers of 16 channels x 33 ints
+constexpr int kSumStride = 33;
+constexpr int kSumBuffer = 16 * kSumStride;
+constexpr int kMaxHeld = 3;               // channel blocks between two barriers (= ring depth)
+constexpr uint32_t kScaleBase = kSumBase + 2 * kMaxHeld * kSumBuffer * 4;  // fp16 weight scales of this CU's channels
+
+struct DenseParams {
+    const int8_t* a;
+    const uint8_t* w;
+    const uint32_t* book;
+    const __half* ws;
+    const __half* as;
+    void* out;
+    int n, k, stride, m, out_f32;
+};
+
+// S: 64-wide K steps per wave (K = 1024 S); CB: token tiles of 16; P: channel blocks whose codes a
+// lane holds at once.
+template <int S, int CB, int P>
+__global__ __launch_bounds__(kThreads) void dense_resident_kernel(DenseParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int column = lane & 15, quarter = lane >> 4;  // MFMA operand row/column and 16-byte K group
+    const int groups = (int)gridDim.x, group = (int)blockIdx.x;
+    const int run = (p.n + groups - 1) / groups;        // channels per CU
+    const int first_row = group * run;
+    const int rows_here = min(run, p.n - first_row);
+    if (rows_here <= 0) return;                         // same for the whole workgroup
+    const int blocks = (rows_here + 15) / 16;
+    int* sums = reinterpret_cast<int*>(lds + kSumBase);
+    __half* scales = reinterpret_cast<__half*>(lds + kScaleBase);
+
+    // ---- set-up reads ------------------------------------------------------------------------------
+    // A lane's K positions inside its wave's slice: steps come in pairs, and in a pair the lane owns 32
+    // consecutive weights (first 16 for the even step, next 16 for the odd one), so that its codes
+    // of a pair are one 16-byte load; an odd last step is an 8-byte load.  Both operands follow the
+    // same map, which is all the MFMA needs.
+    uint32_t selector = 0;
+    if (wave < 4) selector = p.book[tid];
+    constexpr int kPairs = S / 2;
+    constexpr bool kOdd = S % 2 != 0;
+    const int k_slice = p.k / kWaves;
+    auto step_offset = [&](int s) {  // first weight of step s for this lane, inside the slice
+        return s < 2 * kPairs ? 128 * (s >> 1) + 32 * quarter + 16 * (s & 1) : 64 * s + 16 * quarter;
+    };
+    v4u tokens[CB][S];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+        const int8_t* row = p.a + (int64_t)min(16 * c + column, p.m - 1) * p.k + wave * k_slice;
+#pragma unroll
+        for (int s = 0; s < S; ++s) tokens[c][s] = *reinterpret_cast<const v4u*>(row + step_offset(s));
+    }
+    // codes of this lane: channel row `column` of a block (8 weights per 4-byte code)
+    const int64_t row_bytes = p.k / 2;
+    struct Codes {
+        v4u pair[kPairs > 0 ? kPairs : 1];
+        v2u last;
+    };
+    auto load_codes = [&](Codes& codes, int block) {
+        const int row = first_row + min(16 * block + column, rows_here - 1);
+        const uint8_t* src = p.w + row * row_bytes + wave * (k_slice / 2);
+#pragma unroll
+        for (int d = 0; d < kPairs; ++d) codes.pair[d] = *reinterpret_cast<const v4u*>(src + 64 * d + 16 * quarter);
+        if (kOdd) codes.last = *reinterpret_cast<const v2u*>(src + 32 * (S - 1) + 8 * quarter);
+    };
+    // Only the first block's codes travel with the set-up reads; the rest of the ring is requested
+    // after the barrier.  A wave cannot issue anything while one of its loads waits for a slot in
+    // the CU's memory pipeline, so a whole stream requested up front would hold back the table
+    // build and with it every wave's first MFMA.
+    Codes ring[P];
+    load_codes(ring[0], 0);
+    // finalising threads: token tid/16, channel tid%16 of a block
+    const int out_channel = tid & 15, out_token = tid >> 4;
+    const bool finalises = out_token < p.m && out_token < 16 * CB;
+    const float token_scale = __half2float(p.as[min(out_token, p.m - 1)]);
+    for (int i = tid; i < rows_here; i += kThreads) scales[i] = p.ws[first_row + i];
+
+    if (wave < 8) {
+        const int entry = tid & 255;
+        const uint2 value = wave < 4 ? byte_basis_biased(selector, 0) : byte_mask_biased((uint32_t)entry, 0);
+        const uint4 pair = make_uint4(value.x, value.y, value.x, value.y);
+        uint8_t* dst = lds + (wave < 4 ? kBasisBase : kMaskBase) + entry * 128;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
+    }
+    for (int i = tid; i < 2 * kMaxHeld * kSumBuffer; i += kThreads) sums[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int slot = 1; slot < P; ++slot) load_codes(ring[slot], min(slot, blocks - 1));
+
+    const uint32_t copy = (uint32_t)(lane & 15) * 8;
+    auto lookup = [&](uint32_t byte) { return *reinterpret_cast<const uint2*>(lds + byte); };
+    // one u32 two-stage code -> 8 int8 weights: w + 128 = 8 (v0 + 8) + 2 (v1 + 8) + 53 in every byte
+    auto decode = [&](uint32_t code) {
+        const uint2 b0 = lookup(kBasisBase + (((code & 0xFF00u) >> 1) | copy));
+        const uint2 m0 = lookup(kMaskBase + (((code & 0xFFu) << 7) | copy));
+        const uint2 b1 = lookup(kBasisBase + (((code >> 17) & 0x7F80u) | copy));
+        const uint2 m1 = lookup(kMaskBase + (((code >> 9) & 0x7F80u) | copy));
+        uint2 w;
+        w.x = ((((b0.x ^ m0.x) << 3) + ((b1.x ^ m1.x) << 1)) + 0x35353535u) ^ 0x80808080u;
+        w.y = ((((b0.y ^ m0.y) << 3) + ((b1.y ^ m1.y) << 1)) + 0x35353535u) ^ 0x80808080u;
+        return w;
+    };
+
+    // One barrier per group of P blocks: the waves decode P blocks back to back, each into its own
+    // sum buffer, meet once, and the finalising threads store the group while the others go on.
+    // (Tried: no barrier at all, with an arrival counter per block and the last wave storing it.  The
+    // waves then drift apart by up to 8 us, because a wave whose loads are accepted late by the CU's
+    // memory pipeline never catches up, and the kernel gets slower.)
+    static_assert(P <= kMaxHeld, "one sum buffer per held block");
+    for (int first = 0, set = 0; first < blocks; first += P, set ^= 1) {
+        int* group_sums = sums + set * (kMaxHeld * kSumBuffer);
+#pragma unroll
+        for (int slot = 0; slot < P; ++slot) {
+            const int block = first + slot;
+            if (block < blocks) {  // same for the whole workgroup
+                v4i acc[CB];
+#pragma unroll
+                for (int c = 0; c < CB; ++c) acc[c] = v4i{0, 0, 0, 0};
+#pragma unroll
+                for (int s = 0; s < S; ++s) {
+                    uint32_t first_code, second_code;  // the 16 weights of this step
+                    if (s < 2 * kPairs) {
+                        const v4u pair = ring[slot].pair[s >> 1];
+                        first_code = (s & 1) ? pair.z : pair.x, second_code = (s & 1) ? pair.w : pair.y;
+                    } else {
+                        first_code = ring[slot].last.x, second_code = ring[slot].last.y;
+                    }
+                    const uint2 lo = decode(first_code), hi = decode(second_code);
+                    const v4i weights = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+#pragma unroll
+                    for (int c = 0; c < CB; ++c) {
+                        const v4i token = {(int)tokens[c][s].x, (int)tokens[c][s].y, (int)tokens[c][s].z, (int)tokens[c][s].w};
+                        acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights, token, acc[c], 0, 0, 0);
+                    }
+                }
+                if (block + P < blocks) load_codes(ring[slot], block + P);
+                // accumulator i of a lane: channel 4*quarter + i, token 16*c + column
+                int* mine = group_sums + slot * kSumBuffer + 4 * quarter * kSumStride + column;
+#pragma unroll
+                for (int c = 0; c < CB; ++c)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) atomicAdd(mine + i * kSumStride + 16 * c, acc[c][i]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int slot = 0; slot < P; ++slot) {
+            const int channel = 16 * (first + slot) + out_channel;
+            if (finalises && channel < rows_here) {
+                int* cell = group_sums + slot * kSumBuffer + out_channel * kSumStride + out_token;
+                const float value = rescale(*cell, __half2float(scales[channel]), token_scale);
+                *cell = 0;
+                const int64_t index = (int64_t)out_token * p.stride + first_row + channel;
+                if (p.out_f32)
+                    reinterpret_cast<float*>(p.out)[index] = value;
+                else
+                    reinterpret_cast<__half*>(p.out)[index] = __float2half_rn(value);
+            }
+        }
+    }
+}
+
+int device_compute_units() {
+    static int units = 0;
+    if (units == 0) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess)
+            units = prop.multiProcessorCount;
+        else
+            (void)hipGetLastError();
+        if (units <= 0) units = 256;
+    }
+    return units;
+}
+
+// Channel blocks whose codes a lane holds at once: 3 (2 where the token fragments of a long K leave
+// less room); ring depths beyond that only delay the first MFMA.
+constexpr int held_blocks(int steps, int tiles) { return 4 * steps * tiles + 6 * steps > 84 ? 2 : 3; }
+
+uint32_t lds_bytes(int n) {
+    const int run = (n + device_compute_units() - 1) / device_compute_units();
+    return kScaleBase + (((uint32_t)run * 2 + 15) & ~15u);
+}
+constexpr uint32_t kLdsLimit = 160 * 1024;
+
+template <int S, int CB>
+int launch_shape(const DenseParams& p, hipStream_t stream) {
+    constexpr int P = held_blocks(S, CB);
+    hipLaunchKernelGGL((dense_resident_kernel<S, CB, P>), dim3(device_compute_units()), dim3(kThreads), lds_bytes(p.n), stream, p);
+    return hip_check(hipGetLastError(), "launch projection (resident)");
+}
+
+template <int S>
+int launch_steps(const DenseParams& p, hipStream_t stream) {
+    return p.m <= 16 ? launch_shape<S, 1>(p, stream) : launch_shape<S, 2>(p, stream);
+}
+
+template <int S, int CB>
+int opt_in() {
+    return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_resident_kernel<S, CB, held_blocks(S, CB)>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
+                     "hipFuncSetAttribute");
+}
+
+}  // namespace
+
+// Row-major two-stage codes, K a multiple of 1024 up to 8192 (a wave's K slice is whole 64-wide
+// steps and its token fragments fit in registers), at most 32 rows per launch.
+bool dense_resident_eligible(int n, int k, int packed_k) {
+    return packed_k == 0 && k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n) <= kLdsLimit;
+}
+
+void dense_resident_geometry(int n, Geometry* g) {
+    g->grid[0] = (uint32_t)device_compute_units();
+    g->grid[1] = g->grid[2] = 1;
+    g->block[0] = kThreads;
+    g->shared = lds_bytes(n);
+}
+
+int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                          void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream) {
+    static bool opted_in = false;
+    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
+        const int codes[] = {opt_in<1, 1>(), opt_in<1, 2>(), opt_in<2, 1>(), opt_in<2, 2>(), opt_in<3, 1>(), opt_in<3, 2>(),
+                             opt_in<4, 1>(), opt_in<4, 2>(), opt_in<5, 1>(), opt_in<5, 2>(), opt_in<6, 1>(), opt_in<6, 2>(),
+                             opt_in<7, 1>(), opt_in<7, 2>(), opt_in<8, 1>(), opt_in<8, 2>()};
+        for (int code : codes)
+            if (code != ORX_OK) return code;
+        opted_in = true;
+    }
+    if (rows < 1 || rows > 32 || !dense_resident_eligible(n, k, 0)) {
+        set_error("projection (resident): needs 1..32 rows and K a multiple of 1024 up to 8192");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    DenseParams p = {};
+    p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32;
+    switch (k / 1024) {
+        case 1: return launch_steps<1>(p, stream);
+        case 2: return launch_steps<2>(p, stream);
+        case 3: return launch_steps<3>(p, stream);
+        case 4: return launch_steps<4>(p, stream);
+        case 5: return launch_steps<5>(p, stream);
+        case 6: return launch_steps<6>(p, stream);
+        case 7: return launch_steps<7>(p, stream);
+        default: return launch_steps<8>(p, stream);
+    }
+}
+
+}  // namespace orx

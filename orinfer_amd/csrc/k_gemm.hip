@@ -30,6 +30,10 @@ void stream_geometry(int n, Geometry* g);
 int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
+bool dense_resident_eligible(int n, int k, int packed_k);
+void dense_resident_geometry(int n, Geometry* g);
+int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
+                          void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream);
 bool grouped_resident_eligible(int n, int k, int block_m, int tiles);
 bool grouped_resident_preferred(int rows, int experts, int n);
 void grouped_resident_geometry(int k, Geometry* g);
@@ -302,16 +306,30 @@ bool use_gemv(const orx_function& f, int rows) {
     return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
 }
 
-// weight-streaming kernel for up to 64 rows when asked for by name; `auto` also serves 65..128
-// rows with it, as two launches of 64 rows (the second pass finds the weights in the last-level
-// cache and still beats a 128-row MFMA tile that stages both operands through LDS)
+// weight-streaming kernel for up to 64 rows.  Two-stage codes of 65..128 rows go to the 128x128
+// MFMA tiles with the decode inside (measured at N=17408, K=5120, 128 rows: 59 us against 91 us for
+// two streaming launches and 118 us for the 256x256 kernel).  W8 leaves the streaming kernel above
+// 16 rows: the 32/64/128-row tiles measure 27 / 31 / 40 us at 32 / 48 / 128 rows against 29 / 43 / 94.
 bool use_stream(const orx_function& f, int rows) {
     if (f.algorithm == kStream) return rows <= 64;
-    return f.algorithm == kAuto && f.tiles == 0 && rows <= 128;
+    return f.algorithm == kAuto && f.tiles == 0 && rows <= (f.flags == kQ4 ? 64 : 16);
+}
+
+// Resident two-stage kernel (32 rows per launch) where the streaming kernel would run and the shape
+// fits; `algorithm=resident` asks for it by name.
+bool use_resident(const orx_function& f, int rows) {
+    if (f.flags != kQ4 || !dense_resident_eligible(f.N, f.K, f.packed_k)) return false;
+    if (f.algorithm == kResident) return rows <= 128;
+    return f.algorithm == kAuto && f.tiles == 0 && rows > 4 && rows <= 32;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
-bool use_big(const orx_function& f, int rows) { return f.tiles == 256 || (f.tiles == 0 && rows > 128); }
+// (from 385 rows: up to 384 the 128x128 tiles measure 73..77 us for two-stage codes at N=17408,
+// K=5120 against 86..93 us for decode-once + 256x256, and 54..60 us against 58..62 us for W8; at 512
+// rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
+bool use_big(const orx_function& f, int rows) {
+    return f.tiles == 256 || (f.tiles == 0 && rows > 384);
+}
 
 // Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel
 // when the rows need the 256-row MFMA tiles (every row tile would otherwise decode every weight
@@ -323,6 +341,10 @@ bool use_expand(const orx_function& f, int rows) {
 
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
+    if (use_resident(f, rows)) {
+        dense_resident_geometry(f.N, g);
+        return ORX_OK;
+    }
     if (use_stream(f, rows)) {
         stream_geometry(f.N, g);
         return ORX_OK;
@@ -350,6 +372,16 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, 5);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_resident(f, rows)) {
+        for (int first = 0; first < rows; first += 32) {
+            const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
+            const int code = dense_resident_launch(p.a + (size_t)first * f.K, p.w, p.book, p.ws, p.as + first,
+                                                   static_cast<char*>(p.out) + out_offset, std::min(32, rows - first),
+                                                   f.N, f.K, f.stride, f.out_f32, stream);
+            if (code != ORX_OK) return code;
+        }
+        return ORX_OK;
+    }
     if (use_stream(f, rows)) {
         for (int first = 0; first < rows; first += 64) {
             const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
@@ -439,11 +471,18 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     f->flags = codec;
     f->algorithm = algorithm == "gemv"     ? kGemv
                    : algorithm == "mfma"   ? kMfma
-                   : algorithm == "stream" ? kStream
-                   : algorithm == "auto"   ? kAuto
-                                           : -1;
+                   : algorithm == "stream"   ? kStream
+                   : algorithm == "resident" ? kResident
+                   : algorithm == "auto"     ? kAuto
+                                             : -1;
     if (f->algorithm < 0) {
-        set_error("%s: algorithm must be auto, gemv, stream or mfma", name);
+        set_error("%s: algorithm must be auto, gemv, stream, resident or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kResident &&
+        (codec != kQ4 || f->capacity > 128 || !dense_resident_eligible(f->N, f->K, f->packed_k))) {
+        set_error("%s: algorithm=resident serves two-stage row-major codes, at most 128 rows, K a multiple of 1024 up to 8192",
+                  name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->algorithm == kStream && f->capacity > 64) {

@@ -311,6 +311,53 @@ def test_q4_stream_rows_tails_stride_and_sentinels(m, packed_k):
     np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
 
 
+# The resident two-stage kernel (16 waves per CU, K split over the waves, channel blocks of 16):
+# every K it takes (1..8 steps per wave), one and two token tiles, channel counts that leave CUs
+# without work, with a part block or with several rounds of held blocks, more than 32 rows (several
+# launches), the contract shape, fp32 and fp16 outputs with a stride and sentinels around them.
+@pytest.mark.parametrize("m,n,k", [(5, 97, 1024), (16, 300, 2048), (17, 1000, 3072), (8, 5000, 4096), (32, 17408, 5120),
+                                   (9, 4100, 6144), (31, 600, 7168), (32, 9000, 8192), (33, 513, 1024), (128, 2050, 5120),
+                                   (1, 40, 2048)])
+def test_q4_resident_rows_blocks_and_tails(m, n, k):
+    rng = np.random.default_rng(orc.SEED + 300 + m + n)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    w = orc.q4_integers(packed, TABLE)
+    storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), out=storage, stride=n + 3,
+                  dtype=torch.float32, algorithm="resident")
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, w, scales, np.float32))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+    ones_n, ones_m = np.ones(n, np.float16), np.ones(m, np.float16)
+    acc = gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(packed), gu.dev(ones_n), dtype=torch.float32,
+                        algorithm="resident")
+    np.testing.assert_array_equal(gu.host(acc).astype(np.int64), orc.int_dot(a_q, w).astype(np.int64))
+    half = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), algorithm="resident")
+    np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
+    # launched again into the same buffers (the sums in LDS start from zero every time)
+    again = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), algorithm="resident")
+    assert torch.equal(half, again)
+
+
+def test_q4_resident_dynamic_rows_and_refusals():
+    rng = np.random.default_rng(orc.SEED + 77)
+    n, k = 777, 2048
+    a_q, a_s, packed, scales = q4_case(rng, 100, n, k)
+    w = orc.q4_integers(packed, TABLE)
+    for rows in (5, 32, 33, 64, 100):
+        got = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), rows=rows, dynamic=True,
+                            capacity=100, algorithm="resident")
+        np.testing.assert_array_equal(gu.host(got)[:rows], orc.project(a_q[:rows], a_s[:rows], w, scales))
+    for bad in (dict(K=2560), dict(K=9216), dict(packed_k=128), dict(M=129)):
+        variant = dict(M=8, N=256, K=1024, algorithm="resident")
+        variant.update(bad)
+        with pytest.raises(Exception, match="resident"):
+            gu.kernel("e8p_q4_projection", **variant)
+    with pytest.raises(Exception, match="resident"):
+        gu.kernel("int8_projection", M=8, N=256, K=1024, algorithm="resident")
+
+
 @pytest.mark.parametrize("m,n,k", [(7, 48, 2560), (40, 65, 128), (64, 129, 640)])
 def test_w8_stream_matches_oracle(m, n, k):
     rng = np.random.default_rng(orc.SEED + m)
