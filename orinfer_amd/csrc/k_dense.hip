@@ -12,8 +12,8 @@
 //  * K is split over the 16 waves.  A wave keeps the token fragments of its K slice in registers for
 //    the whole kernel (they are the same for every channel block), so activations are read once
 //    per CU; its codes stream through a ring of P channel blocks that is refilled right after use.
-//  * Codes are decoded with two 8-byte lookups per stage in tables stored 16 times (entry i for
-//    lane l at byte i*128 + (l%16)*8), so the lanes of one access group never share a bank; the two
+//  * Codes are decoded with two 8-byte lookups per stage in tables stored 16 times (one copy per
+//    lane of an access group, so lanes never share a bank; the address is one v_perm_b32); the two
 //    stages share one pair of tables (values v+8, shifted by the stage's weight when combined).
 //  * The 16 K-slice partial sums of a block are added with LDS integer atomics (exact in any order)
 //    into a buffer per block; one barrier per group of P blocks, then 16 x M threads rescale and
@@ -30,10 +30,11 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 16;
-constexpr int kThreads = kWaves * 64;
-constexpr uint32_t kBasisBase = 0;        // 256 entries x 16 copies x 8 bytes: (h ^ 8) per coordinate
-constexpr uint32_t kMaskBase = 32768;     // the same for the sign/parity masks
+constexpr int kMaxThreads = 1024;
+// Tables: entry i of the basis table ((h ^ 8) per coordinate) at byte i*256 + copy*8, entry u of the
+// sign/parity mask table at u*256 + 128 + copy*8, 16 copies each.  With the entry index in the
+// address's second byte, one v_perm_b32 builds a lookup address from a byte of the code.
+constexpr uint32_t kMaskOffset = 128;
 constexpr uint32_t kSumBase = 65536;      // two sets of kMaxHeld buffers of 16 channels x 33 ints
 constexpr int kSumStride = 33;
 constexpr int kSumBuffer = 16 * kSumStride;
@@ -50,10 +51,11 @@ struct DenseParams {
     int n, k, stride, m, out_f32;
 };
 
-// S: 64-wide K steps per wave (K = 1024 S); CB: token tiles of 16; P: channel blocks whose codes a
-// lane holds at once.
-template <int S, int CB, int P>
-__global__ __launch_bounds__(kThreads) void dense_resident_kernel(DenseParams p) {
+// W: waves per workgroup (K is split over them); S: 64-wide K steps per wave (K = 64 W S); CB: token
+// tiles of 16; P: channel blocks whose codes a lane holds at once.
+template <int W, int S, int CB, int P>
+__global__ __launch_bounds__(W * 64) void dense_resident_kernel(DenseParams p) {
+    constexpr int kWaves = W, kThreads = W * 64;
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,11 +114,12 @@ __global__ __launch_bounds__(kThreads) void dense_resident_kernel(DenseParams p)
     const float token_scale = __half2float(p.as[min(out_token, p.m - 1)]);
     for (int i = tid; i < rows_here; i += kThreads) scales[i] = p.ws[first_row + i];
 
+    static_assert(W >= 8, "waves 0-3 build the basis table, waves 4-7 the mask table");
     if (wave < 8) {
         const int entry = tid & 255;
         const uint2 value = wave < 4 ? byte_basis_biased(selector, 0) : byte_mask_biased((uint32_t)entry, 0);
         const uint4 pair = make_uint4(value.x, value.y, value.x, value.y);
-        uint8_t* dst = lds + (wave < 4 ? kBasisBase : kMaskBase) + entry * 128;
+        uint8_t* dst = lds + entry * 256 + (wave < 4 ? 0 : kMaskOffset);
 #pragma unroll
         for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
     }
@@ -125,14 +128,18 @@ __global__ __launch_bounds__(kThreads) void dense_resident_kernel(DenseParams p)
 #pragma unroll
     for (int slot = 1; slot < P; ++slot) load_codes(ring[slot], min(slot, blocks - 1));
 
+    // byte 0: this lane's copy in the basis half of an entry, byte 1: in the mask half
     const uint32_t copy = (uint32_t)(lane & 15) * 8;
-    auto lookup = [&](uint32_t byte) { return *reinterpret_cast<const uint2*>(lds + byte); };
+    const uint32_t columns = copy | (kMaskOffset | copy) << 8;
+    // selectors of v_perm_b32(code, columns): address byte 0 = a byte of `columns`, byte 1 = a byte of the code
+    constexpr uint32_t kBasisLow = 0x0C0C0500u, kMaskLow = 0x0C0C0401u, kBasisHigh = 0x0C0C0700u, kMaskHigh = 0x0C0C0601u;
+    auto lookup = [&](uint32_t code, uint32_t selector) {
+        return *reinterpret_cast<const uint2*>(lds + __builtin_amdgcn_perm(code, columns, selector));
+    };
     // one u32 two-stage code -> 8 int8 weights: w + 128 = 8 (v0 + 8) + 2 (v1 + 8) + 53 in every byte
     auto decode = [&](uint32_t code) {
-        const uint2 b0 = lookup(kBasisBase + (((code & 0xFF00u) >> 1) | copy));
-        const uint2 m0 = lookup(kMaskBase + (((code & 0xFFu) << 7) | copy));
-        const uint2 b1 = lookup(kBasisBase + (((code >> 17) & 0x7F80u) | copy));
-        const uint2 m1 = lookup(kMaskBase + (((code >> 9) & 0x7F80u) | copy));
+        const uint2 b0 = lookup(code, kBasisLow), m0 = lookup(code, kMaskLow);
+        const uint2 b1 = lookup(code, kBasisHigh), m1 = lookup(code, kMaskHigh);
         uint2 w;
         w.x = ((((b0.x ^ m0.x) << 3) + ((b1.x ^ m1.x) << 1)) + 0x35353535u) ^ 0x80808080u;
         w.y = ((((b0.y ^ m0.y) << 3) + ((b1.y ^ m1.y) << 1)) + 0x35353535u) ^ 0x80808080u;
@@ -216,29 +223,41 @@ int device_compute_units() {
 // less room); ring depths beyond that only delay the first MFMA.
 constexpr int held_blocks(int steps, int tiles) { return 4 * steps * tiles + 6 * steps > 84 ? 2 : 3; }
 
-uint32_t lds_bytes(int n) {
-    const int run = (n + device_compute_units() - 1) / device_compute_units();
+// One workgroup of 16 waves per CU.  (Tried for up to 16 rows: two workgroups of 8 waves per CU, each
+// wave owning K/8, so that one workgroup decodes while the other waits for memory: 20.6 against
+// 19.2 us.)
+int waves_for(int rows, int k) {
+    (void)rows, (void)k;
+    return 16;
+}
+int workgroups_for(int rows, int k) { return device_compute_units() * (waves_for(rows, k) == 8 ? 2 : 1); }
+
+uint32_t lds_bytes(int n, int workgroups) {
+    const int run = (n + workgroups - 1) / workgroups;
     return kScaleBase + (((uint32_t)run * 2 + 15) & ~15u);
 }
 constexpr uint32_t kLdsLimit = 160 * 1024;
 
-template <int S, int CB>
+template <int W, int S, int CB>
 int launch_shape(const DenseParams& p, hipStream_t stream) {
     constexpr int P = held_blocks(S, CB);
-    hipLaunchKernelGGL((dense_resident_kernel<S, CB, P>), dim3(device_compute_units()), dim3(kThreads), lds_bytes(p.n), stream, p);
+    static bool opted_in = false;
+    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
+        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_resident_kernel<W, S, CB, P>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
+                                   "hipFuncSetAttribute");
+        if (code != ORX_OK) return code;
+        opted_in = true;
+    }
+    const int workgroups = workgroups_for(p.m, p.k);
+    hipLaunchKernelGGL((dense_resident_kernel<W, S, CB, P>), dim3(workgroups), dim3(W * 64), lds_bytes(p.n, workgroups),
+                       stream, p);
     return hip_check(hipGetLastError(), "launch projection (resident)");
 }
 
-template <int S>
+template <int S16>  // S16: steps per wave with 16 waves
 int launch_steps(const DenseParams& p, hipStream_t stream) {
-    return p.m <= 16 ? launch_shape<S, 1>(p, stream) : launch_shape<S, 2>(p, stream);
-}
-
-template <int S, int CB>
-int opt_in() {
-    return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_resident_kernel<S, CB, held_blocks(S, CB)>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
-                     "hipFuncSetAttribute");
+    return p.m <= 16 ? launch_shape<16, S16, 1>(p, stream) : launch_shape<16, S16, 2>(p, stream);
 }
 
 }  // namespace
@@ -246,27 +265,19 @@ int opt_in() {
 // Row-major two-stage codes, K a multiple of 1024 up to 8192 (a wave's K slice is whole 64-wide
 // steps and its token fragments fit in registers), at most 32 rows per launch.
 bool dense_resident_eligible(int n, int k, int packed_k) {
-    return packed_k == 0 && k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n) <= kLdsLimit;
+    return packed_k == 0 && k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n, device_compute_units()) <= kLdsLimit;
 }
 
-void dense_resident_geometry(int n, Geometry* g) {
-    g->grid[0] = (uint32_t)device_compute_units();
+void dense_resident_geometry(int rows, int n, int k, Geometry* g) {
+    const int chunk = rows < 32 ? rows : 32;  // rows per launch
+    g->grid[0] = (uint32_t)workgroups_for(chunk, k);
     g->grid[1] = g->grid[2] = 1;
-    g->block[0] = kThreads;
-    g->shared = lds_bytes(n);
+    g->block[0] = (uint32_t)waves_for(chunk, k) * 64;
+    g->shared = lds_bytes(n, (int)g->grid[0]);
 }
 
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream) {
-    static bool opted_in = false;
-    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
-        const int codes[] = {opt_in<1, 1>(), opt_in<1, 2>(), opt_in<2, 1>(), opt_in<2, 2>(), opt_in<3, 1>(), opt_in<3, 2>(),
-                             opt_in<4, 1>(), opt_in<4, 2>(), opt_in<5, 1>(), opt_in<5, 2>(), opt_in<6, 1>(), opt_in<6, 2>(),
-                             opt_in<7, 1>(), opt_in<7, 2>(), opt_in<8, 1>(), opt_in<8, 2>()};
-        for (int code : codes)
-            if (code != ORX_OK) return code;
-        opted_in = true;
-    }
     if (rows < 1 || rows > 32 || !dense_resident_eligible(n, k, 0)) {
         set_error("projection (resident): needs 1..32 rows and K a multiple of 1024 up to 8192");
         return ORX_ERR_BAD_VARIANT;

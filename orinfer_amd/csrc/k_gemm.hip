@@ -31,7 +31,7 @@ int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* boo
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
 bool dense_resident_eligible(int n, int k, int packed_k);
-void dense_resident_geometry(int n, Geometry* g);
+void dense_resident_geometry(int rows, int n, int k, Geometry* g);
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream);
 bool grouped_resident_eligible(int n, int k, int block_m, int tiles);
@@ -302,8 +302,10 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
     return hip_check(hipGetLastError(), "launch projection (mfma)");
 }
 
+bool use_resident(const orx_function& f, int rows);
 bool use_gemv(const orx_function& f, int rows) {
-    return f.algorithm == kGemv || (f.algorithm == kAuto && rows <= 4 && f.packed_k == 0);
+    if (f.algorithm == kGemv) return true;
+    return f.algorithm == kAuto && rows <= 4 && f.packed_k == 0 && !use_resident(f, rows);
 }
 
 // weight-streaming kernel for up to 64 rows.  Two-stage codes of 65..128 rows go to the 128x128
@@ -320,7 +322,9 @@ bool use_stream(const orx_function& f, int rows) {
 bool use_resident(const orx_function& f, int rows) {
     if (f.flags != kQ4 || !dense_resident_eligible(f.N, f.K, f.packed_k)) return false;
     if (f.algorithm == kResident) return rows <= 128;
-    return f.algorithm == kAuto && f.tiles == 0 && rows > 4 && rows <= 32;
+    // from 3 rows: the GEMV's dot products grow with the row count (23 us at 3 and 4 rows of
+    // N=17408, K=5120), this kernel's MFMAs do not (19 us from 3 to 8 rows)
+    return f.algorithm == kAuto && f.tiles == 0 && rows > 2 && rows <= 32;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
@@ -342,7 +346,7 @@ bool use_expand(const orx_function& f, int rows) {
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_resident(f, rows)) {
-        dense_resident_geometry(f.N, g);
+        dense_resident_geometry(rows, f.N, f.K, g);
         return ORX_OK;
     }
     if (use_stream(f, rows)) {

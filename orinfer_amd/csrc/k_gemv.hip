@@ -605,7 +605,9 @@ int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_banked(f, mr)) {
         const uint32_t lanes_per_row = (uint32_t)f.slots >> 8;
         const uint32_t tasks = ceil_div((uint32_t)f.N, 64u / lanes_per_row);
-        g->grid[0] = std::min<uint32_t>((uint32_t)device_cus(), ceil_div(tasks, (uint32_t)(kBankedThreads / 64)));
+        // every CU gets a workgroup as soon as there is a task for each: a small matrix then runs with
+        // some idle waves per CU rather than with idle CUs
+        g->grid[0] = std::min<uint32_t>((uint32_t)device_cus(), tasks);
         g->block[0] = kBankedThreads;
         g->shared = banked_lds_bytes(f, mr);
         return ORX_OK;
