@@ -1,23 +1,23 @@
-// Two-stage (Q4) projections for 5..32 token rows (batched decode): one resident workgroup of 16
-// waves per CU, the whole weight stream of a wave requested up front.
+// Two-stage (Q4) projections for 3..32 token rows (batched decode): one resident workgroup per CU.
 //
 // Reference counterparts: the small-row Tensor Core schedules of kernels/cuda/model/integer_core.py
 // (block_m 8..32) behind kernels/cuda/model/e8p_q4.py:143-264.  Arithmetic: exact int32 over the full
 // K, (float(acc) * ws) * as.
 //
-// MI355X design.  With so few rows the projection is a weight stream (0.5 byte per weight) and the
-// kernel is shaped so that nothing but that stream touches memory inside the loop:
+// MI355X design.  With so few rows the projection is a weight stream (0.5 byte per weight):
 //  * Output channels are dealt to CUs in equal contiguous runs (N / CUs each, 68 at N = 17408), cut
 //    into blocks of 16 channels for v_mfma_i32_16x16x64_i8, so every CU has the same work.
-//  * K is split over the 16 waves.  A wave keeps the token fragments of its K slice in registers for
-//    the whole kernel (they are the same for every channel block), so activations are read once
-//    per CU; its codes stream through a ring of P channel blocks that is refilled right after use.
+//  * K is split over the decoding waves.  A wave keeps the token fragments of its K slice in
+//    registers for the whole kernel (they are the same for every channel block), so activations are
+//    read once per CU.
 //  * Codes are decoded with two 8-byte lookups per stage in tables stored 16 times (one copy per
 //    lane of an access group, so lanes never share a bank; the address is one v_perm_b32); the two
 //    stages share one pair of tables (values v+8, shifted by the stage's weight when combined).
-//  * The 16 K-slice partial sums of a block are added with LDS integer atomics (exact in any order)
-//    into a buffer per block; one barrier per group of P blocks, then 16 x M threads rescale and
-//    store the group while the other waves already decode the next one.
+//  * The K-slice partial sums of a block are added with LDS integer atomics (exact in any order);
+//    after a barrier 16 x M threads rescale and store the block while the others decode the next.
+// Two kernels share this: dense_specialized_kernel (K up to 5120 in steps of 512: four loader waves
+// stream the codes into LDS, eight decoder waves never touch memory) and dense_resident_kernel (K up
+// to 8192 in steps of 1024: sixteen waves, each loading its own codes through a register ring).
 #include <hip/hip_fp16.h>
 
 #include "e8p_device.h"
@@ -205,6 +205,180 @@ __global__ __launch_bounds__(W * 64) void dense_resident_kernel(DenseParams p) {
     }
 }
 
+// ---- the same projection with loader waves -------------------------------------------------------------
+// A wave cannot issue anything while one of its vector loads waits for a slot in the CU's memory
+// pipeline, and in a bandwidth-bound kernel that is most of the time: in the kernel above the decode
+// of a wave is serialised behind its own code loads (decode alone 12.9 us, loads alone 13.4 us,
+// together 19.5 us at N=17408, K=5120, 8 rows).  Here four loader waves do nothing but request the
+// CU's codes, whole rows at a time and straight into LDS (no registers, fully contiguous requests),
+// while eight decoder waves (two per SIMD, K split eight ways) never touch memory after set-up: they
+// read their codes from LDS.  Two code buffers of 16 channel rows each; one barrier per block.
+constexpr int kDecoders = 8, kLoaders = 4;
+constexpr int kSpecThreads = (kDecoders + kLoaders) * 64;
+constexpr int kRowPad = 16;  // bytes between staged code rows: 16 rows read at the same K then hit 16 different bank groups
+
+__device__ __forceinline__ void direct_load_16(const void* global, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+// S: 64-wide K steps per decoder wave (K = 512 S); CB: token tiles of 16.
+template <int S, int CB>
+__global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DenseParams p) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int column = lane & 15, quarter = lane >> 4;
+    const int groups = (int)gridDim.x, group = (int)blockIdx.x;
+    const int run = (p.n + groups - 1) / groups;
+    const int first_row = group * run;
+    const int rows_here = min(run, p.n - first_row);
+    if (rows_here <= 0) return;  // same for the whole workgroup
+    const int blocks = (rows_here + 15) / 16;
+    constexpr int kRowBytes = 256 * S;                       // codes of one channel row
+    constexpr int kPitch = kRowBytes + kRowPad;
+    constexpr int kPieces = (kRowBytes + 1023) / 1024;       // 1 KiB requests per row
+    constexpr int kPerLoader = 16 * kPieces / kLoaders;      // requests of one loader wave per block
+    static_assert(16 * kPieces % kLoaders == 0, "every loader wave issues the same number of requests");
+    int* sums = reinterpret_cast<int*>(lds + kSumBase);
+    __half* scales = reinterpret_cast<__half*>(lds + kScaleBase);
+    const uint32_t code_base = kScaleBase + (((uint32_t)run * 2 + 15) & ~15u);
+    auto buffer = [&](int block) { return lds + code_base + (block & 1) * (16 * kPitch); };
+
+    if (wave >= kDecoders) {
+        // ---- loader waves ----
+        // One block is in flight at a time, requested the moment its buffer is released.  One block
+        // per CU (10 MB over the chip) already keeps HBM busy: it lands 2 us after the request,
+        // which is the CU's share of the bandwidth.  Requesting more at once only delays the first
+        // block, because everything in flight shares that bandwidth (two blocks at the start: first
+        // MFMA at 5.2 us; a third block parked in the loaders' registers: 0.7 us slower overall).
+        const int loader = wave - kDecoders;
+        auto request = [&](int block) {
+            const int rows_in_block = min(16, rows_here - 16 * block);
+            const uint8_t* src = p.w + (int64_t)(first_row + 16 * block) * kRowBytes;
+            uint8_t* dst = buffer(block);
+#pragma unroll
+            for (int i = 0; i < kPerLoader; ++i) {
+                const int piece = loader + kLoaders * i, row = piece / kPieces, part = piece - row * kPieces;
+                const int offset = part * 1024 + lane * 16;
+                if (row < rows_in_block && offset < kRowBytes)
+                    direct_load_16(src + (int64_t)row * kRowBytes + offset, dst + row * kPitch + part * 1024);
+            }
+        };
+        request(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // direct-to-LDS requests are not waited for by a barrier
+        __syncthreads();
+        for (int block = 0; block < blocks; ++block) {
+            if (block + 1 < blocks) request(block + 1);       // its buffer was released at the last barrier
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();                                   // block + 1 has landed, the decoders are done with `block`
+        }
+        return;
+    }
+
+    // ---- decoder waves ----
+    uint32_t selector = 0;
+    if (wave < 4) selector = p.book[tid];
+    constexpr int kPairs = S / 2;
+    constexpr bool kOdd = S % 2 != 0;
+    constexpr int kSlice = 64 * S;  // K positions of one decoder wave
+    auto step_offset = [&](int s) {  // same K map as above: pairs of steps share 32 consecutive weights per lane
+        return s < 2 * kPairs ? 128 * (s >> 1) + 32 * quarter + 16 * (s & 1) : 64 * s + 16 * quarter;
+    };
+    v4u tokens[CB][S];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+        const int8_t* row = p.a + (int64_t)min(16 * c + column, p.m - 1) * p.k + wave * kSlice;
+#pragma unroll
+        for (int s = 0; s < S; ++s) tokens[c][s] = *reinterpret_cast<const v4u*>(row + step_offset(s));
+    }
+    const int out_channel = tid & 15, out_token = tid >> 4;  // 512 decoder threads: 32 tokens x 16 channels
+    const bool finalises = out_token < p.m && out_token < 16 * CB;
+    const float token_scale = __half2float(p.as[min(out_token, p.m - 1)]);
+    for (int i = tid; i < rows_here; i += kDecoders * 64) scales[i] = p.ws[first_row + i];
+    {
+        const int entry = tid & 255;
+        const uint2 value = wave < 4 ? byte_basis_biased(selector, 0) : byte_mask_biased((uint32_t)entry, 0);
+        const uint4 pair = make_uint4(value.x, value.y, value.x, value.y);
+        uint8_t* dst = lds + entry * 256 + (wave < 4 ? 0 : kMaskOffset);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
+    }
+    for (int i = tid; i < 2 * kSumBuffer; i += kDecoders * 64) sums[i] = 0;
+    __syncthreads();
+
+    const uint32_t copy = (uint32_t)(lane & 15) * 8;
+    const uint32_t columns = copy | (kMaskOffset | copy) << 8;
+    constexpr uint32_t kBasisLow = 0x0C0C0500u, kMaskLow = 0x0C0C0401u, kBasisHigh = 0x0C0C0700u, kMaskHigh = 0x0C0C0601u;
+    // The tables start at LDS address 0 (the kernel has no static LDS), so the permuted bytes are the
+    // address itself.
+    typedef const __attribute__((address_space(3))) v2u* TableEntry;
+    auto lookup = [&](uint32_t code, uint32_t selector_bytes) {
+        return *reinterpret_cast<TableEntry>((uintptr_t)__builtin_amdgcn_perm(code, columns, selector_bytes));
+    };
+    // All lookups of a group of codes are requested before the first is used: with two decoder waves
+    // per SIMD there is little else to hide the LDS latency behind.
+    struct Looked {
+        v2u b0, m0, b1, m1;
+    };
+    auto request = [&](uint32_t code) {
+        return Looked{lookup(code, kBasisLow), lookup(code, kMaskLow), lookup(code, kBasisHigh), lookup(code, kMaskHigh)};
+    };
+    // one u32 two-stage code -> 8 int8 weights: w + 128 = 8 (v0 + 8) + 2 (v1 + 8) + 53 in every byte
+    auto combine = [&](const Looked& l) {
+        v2u w;
+        w.x = ((((l.b0.x ^ l.m0.x) << 3) + ((l.b1.x ^ l.m1.x) << 1)) + 0x35353535u) ^ 0x80808080u;
+        w.y = ((((l.b0.y ^ l.m0.y) << 3) + ((l.b1.y ^ l.m1.y) << 1)) + 0x35353535u) ^ 0x80808080u;
+        return w;
+    };
+    auto multiply = [&](v4i (&acc)[CB], const v2u& lo, const v2u& hi, int s) {
+        const v4i weights = {(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
+#pragma unroll
+        for (int c = 0; c < CB; ++c) {
+            const v4i token = {(int)tokens[c][s].x, (int)tokens[c][s].y, (int)tokens[c][s].z, (int)tokens[c][s].w};
+            acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights, token, acc[c], 0, 0, 0);
+        }
+    };
+    const int lane_codes = column * kPitch + wave * (kSlice / 2);  // this lane's row and this wave's K slice in a buffer
+
+    for (int block = 0; block < blocks; ++block) {
+        const uint8_t* src = buffer(block) + lane_codes;
+        v4i acc[CB];
+#pragma unroll
+        for (int c = 0; c < CB; ++c) acc[c] = v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int d = 0; d < kPairs; ++d) {
+            const v4u pair = *reinterpret_cast<const v4u*>(src + 64 * d + 16 * quarter);
+            const Looked l0 = request(pair.x), l1 = request(pair.y), l2 = request(pair.z), l3 = request(pair.w);
+            multiply(acc, combine(l0), combine(l1), 2 * d);
+            multiply(acc, combine(l2), combine(l3), 2 * d + 1);
+        }
+        if (kOdd) {
+            const v2u last = *reinterpret_cast<const v2u*>(src + 32 * (S - 1) + 8 * quarter);
+            const Looked l0 = request(last.x), l1 = request(last.y);
+            multiply(acc, combine(l0), combine(l1), S - 1);
+        }
+        int* block_sums = sums + (block & 1) * kSumBuffer;
+        int* mine = block_sums + 4 * quarter * kSumStride + column;
+#pragma unroll
+        for (int c = 0; c < CB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) atomicAdd(mine + i * kSumStride + 16 * c, acc[c][i]);
+        __syncthreads();
+        const int channel = 16 * block + out_channel;
+        if (finalises && channel < rows_here) {
+            int* cell = block_sums + out_channel * kSumStride + out_token;
+            const float value = rescale(*cell, __half2float(scales[channel]), token_scale);
+            *cell = 0;
+            const int64_t index = (int64_t)out_token * p.stride + first_row + channel;
+            if (p.out_f32)
+                reinterpret_cast<float*>(p.out)[index] = value;
+            else
+                reinterpret_cast<__half*>(p.out)[index] = __float2half_rn(value);
+        }
+    }
+}
+
 int device_compute_units() {
     static int units = 0;
     if (units == 0) {
@@ -255,6 +429,34 @@ int launch_shape(const DenseParams& p, hipStream_t stream) {
     return hip_check(hipGetLastError(), "launch projection (resident)");
 }
 
+uint32_t specialized_lds_bytes(int n, int k) {
+    const int run = (n + device_compute_units() - 1) / device_compute_units();
+    return kScaleBase + (((uint32_t)run * 2 + 15) & ~15u) + 2u * 16u * (uint32_t)(k / 2 + kRowPad);
+}
+
+// Loader-wave kernel: K a multiple of 512 up to 5120 (a decoder wave holds the token fragments of K/8).
+bool specialized_fits(int n, int k) { return k % 512 == 0 && k / 512 <= 10 && specialized_lds_bytes(n, k) <= kLdsLimit; }
+
+template <int S, int CB>
+int launch_specialized_shape(const DenseParams& p, hipStream_t stream) {
+    static bool opted_in = false;
+    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
+        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_specialized_kernel<S, CB>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
+                                   "hipFuncSetAttribute");
+        if (code != ORX_OK) return code;
+        opted_in = true;
+    }
+    hipLaunchKernelGGL((dense_specialized_kernel<S, CB>), dim3(device_compute_units()), dim3(kSpecThreads),
+                       specialized_lds_bytes(p.n, p.k), stream, p);
+    return hip_check(hipGetLastError(), "launch projection (resident, loader waves)");
+}
+
+template <int S>
+int launch_specialized(const DenseParams& p, hipStream_t stream) {
+    return p.m <= 16 ? launch_specialized_shape<S, 1>(p, stream) : launch_specialized_shape<S, 2>(p, stream);
+}
+
 template <int S16>  // S16: steps per wave with 16 waves
 int launch_steps(const DenseParams& p, hipStream_t stream) {
     return p.m <= 16 ? launch_shape<16, S16, 1>(p, stream) : launch_shape<16, S16, 2>(p, stream);
@@ -265,13 +467,21 @@ int launch_steps(const DenseParams& p, hipStream_t stream) {
 // Row-major two-stage codes, K a multiple of 1024 up to 8192 (a wave's K slice is whole 64-wide
 // steps and its token fragments fit in registers), at most 32 rows per launch.
 bool dense_resident_eligible(int n, int k, int packed_k) {
-    return packed_k == 0 && k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n, device_compute_units()) <= kLdsLimit;
+    if (packed_k != 0) return false;
+    if (specialized_fits(n, k)) return true;
+    return k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n, device_compute_units()) <= kLdsLimit;
 }
 
 void dense_resident_geometry(int rows, int n, int k, Geometry* g) {
     const int chunk = rows < 32 ? rows : 32;  // rows per launch
-    g->grid[0] = (uint32_t)workgroups_for(chunk, k);
     g->grid[1] = g->grid[2] = 1;
+    if (specialized_fits(n, k)) {
+        g->grid[0] = (uint32_t)device_compute_units();
+        g->block[0] = kSpecThreads;
+        g->shared = specialized_lds_bytes(n, k);
+        return;
+    }
+    g->grid[0] = (uint32_t)workgroups_for(chunk, k);
     g->block[0] = (uint32_t)waves_for(chunk, k) * 64;
     g->shared = lds_bytes(n, (int)g->grid[0]);
 }
@@ -279,12 +489,26 @@ void dense_resident_geometry(int rows, int n, int k, Geometry* g) {
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream) {
     if (rows < 1 || rows > 32 || !dense_resident_eligible(n, k, 0)) {
-        set_error("projection (resident): needs 1..32 rows and K a multiple of 1024 up to 8192");
+        set_error("projection (resident): needs 1..32 rows and K a multiple of 512 up to 5120 or of 1024 up to 8192");
         return ORX_ERR_BAD_VARIANT;
     }
     DenseParams p = {};
     p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
     p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32;
+    if (specialized_fits(n, k)) {
+        switch (k / 512) {
+            case 1: return launch_specialized<1>(p, stream);
+            case 2: return launch_specialized<2>(p, stream);
+            case 3: return launch_specialized<3>(p, stream);
+            case 4: return launch_specialized<4>(p, stream);
+            case 5: return launch_specialized<5>(p, stream);
+            case 6: return launch_specialized<6>(p, stream);
+            case 7: return launch_specialized<7>(p, stream);
+            case 8: return launch_specialized<8>(p, stream);
+            case 9: return launch_specialized<9>(p, stream);
+            default: return launch_specialized<10>(p, stream);
+        }
+    }
     switch (k / 1024) {
         case 1: return launch_steps<1>(p, stream);
         case 2: return launch_steps<2>(p, stream);

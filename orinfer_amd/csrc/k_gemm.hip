@@ -485,7 +485,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     }
     if (f->algorithm == kResident &&
         (codec != kQ4 || f->capacity > 128 || !dense_resident_eligible(f->N, f->K, f->packed_k))) {
-        set_error("%s: algorithm=resident serves two-stage row-major codes, at most 128 rows, K a multiple of 1024 up to 8192",
+        set_error("%s: algorithm=resident serves two-stage row-major codes, at most 128 rows, K a multiple of 512 up to 5120 or of 1024 up to 8192",
                   name);
         return ORX_ERR_BAD_VARIANT;
     }

@@ -311,13 +311,15 @@ def test_q4_stream_rows_tails_stride_and_sentinels(m, packed_k):
     np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
 
 
-# The resident two-stage kernel (16 waves per CU, K split over the waves, channel blocks of 16):
-# every K it takes (1..8 steps per wave), one and two token tiles, channel counts that leave CUs
+# The resident two-stage kernels (K split over the waves of one workgroup per CU, channel blocks of
+# 16; K up to 5120 in steps of 512 with loader waves, up to 8192 in steps of 1024 without): every K
+# they take, one and two token tiles, channel counts that leave CUs
 # without work, with a part block or with several rounds of held blocks, more than 32 rows (several
 # launches), the contract shape, fp32 and fp16 outputs with a stride and sentinels around them.
 @pytest.mark.parametrize("m,n,k", [(5, 97, 1024), (16, 300, 2048), (17, 1000, 3072), (8, 5000, 4096), (32, 17408, 5120),
                                    (9, 4100, 6144), (31, 600, 7168), (32, 9000, 8192), (33, 513, 1024), (128, 2050, 5120),
-                                   (1, 40, 2048)])
+                                   (1, 40, 2048), (3, 9728, 2560), (20, 70, 512), (7, 1111, 1536), (32, 4099, 3584),
+                                   (16, 257, 4608)])
 def test_q4_resident_rows_blocks_and_tails(m, n, k):
     rng = np.random.default_rng(orc.SEED + 300 + m + n)
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
@@ -349,7 +351,7 @@ def test_q4_resident_dynamic_rows_and_refusals():
         got = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), rows=rows, dynamic=True,
                             capacity=100, algorithm="resident")
         np.testing.assert_array_equal(gu.host(got)[:rows], orc.project(a_q[:rows], a_s[:rows], w, scales))
-    for bad in (dict(K=2560), dict(K=9216), dict(packed_k=128), dict(M=129)):
+    for bad in (dict(K=1280), dict(K=9216), dict(packed_k=128), dict(M=129)):
         variant = dict(M=8, N=256, K=1024, algorithm="resident")
         variant.update(bad)
         with pytest.raises(Exception, match="resident"):
