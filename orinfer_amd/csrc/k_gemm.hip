@@ -324,7 +324,9 @@ bool use_resident(const orx_function& f, int rows) {
     if (f.algorithm == kResident) return rows <= 128;
     // from 3 rows: the GEMV's dot products grow with the row count (23 us at 3 and 4 rows of
     // N=17408, K=5120), this kernel's MFMAs do not (19 us from 3 to 8 rows)
-    return f.algorithm == kAuto && f.tiles == 0 && rows > 2 && rows <= 32;
+    // up to 64 rows as two launches of 32 (36 and 39 us at 48 and 64 rows against 42 and 48 us for
+    // the streaming kernel)
+    return f.algorithm == kAuto && f.tiles == 0 && rows > 2 && rows <= 64;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
