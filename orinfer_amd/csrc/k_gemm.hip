@@ -25,6 +25,7 @@ int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t 
 int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
 int gemv_configure(orx_function* f, int codec, int passes_override);
 int gemv_prepare_device();
+bool gemv_serves_k_major(const orx_function& f, int rows);
 // from k_stream.hip
 void stream_geometry(int n, Geometry* g);
 int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
@@ -305,7 +306,10 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
 bool use_resident(const orx_function& f, int rows);
 bool use_gemv(const orx_function& f, int rows) {
     if (f.algorithm == kGemv) return true;
-    return f.algorithm == kAuto && rows <= 4 && f.packed_k == 0 && !use_resident(f, rows);
+    if (f.algorithm != kAuto) return false;
+    // K-major codes: 1 and 2 rows (13.4 and 16.5 us at N=17408, K=5120; the streaming kernel takes 17.2)
+    if (f.packed_k != 0) return rows <= 2 && gemv_serves_k_major(f, rows);
+    return rows <= 4 && !use_resident(f, rows);
 }
 
 // weight-streaming kernel for up to 64 rows.  Two-stage codes of 65..128 rows go to the 128x128
@@ -495,11 +499,12 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         set_error("%s: the stream algorithm serves up to 64 rows, variant asks for %d", name, f->capacity);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv && f->packed_k != 0) {
-        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0)", name);
+    if (f->algorithm == kGemv && f->packed_k != 0 && (codec != kQ4 || f->K % 256 != 0)) {
+        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0), or K-major two-stage codes with K a multiple of 256",
+                  name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv || (f->algorithm == kAuto && f->packed_k == 0)) {
+    if (f->algorithm == kGemv || (f->algorithm == kAuto && (f->packed_k == 0 || (codec == kQ4 && f->K % 256 == 0)))) {
         orx_function probe = *f;
         if (probe.capacity > 4) probe.capacity = 4;
         int code = gemv_configure(&probe, codec, passes);

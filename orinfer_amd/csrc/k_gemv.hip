@@ -312,12 +312,16 @@ constexpr uint32_t kSelNib1 = 0x0C0C0500u, kSelNib3 = 0x0C0C0700u, kSelMsk0 = 0x
 // ring of 16-byte chunks.  Two-stage Q4 only.  HOLD (one activation row, a row's steps equal to D):
 // a lane meets the same chunk positions in every output row, so it keeps their hi and lo words in
 // registers for the whole kernel and the main loop reads LDS for table lookups only.
-template <int CODEC, int MR, int D, int LPR, bool HOLD>
+// LAYOUT: lanes per row, + 64 for K-major codes.
+constexpr int kKMajorLayout = 64;
+template <int CODEC, int MR, int D, int LAYOUT, bool HOLD>
 __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
     int m, int out_f32) {
     extern __shared__ __align__(16) uint32_t lds[];
+    constexpr int LPR = LAYOUT & (kKMajorLayout - 1);
+    constexpr bool kKMajor = LAYOUT >= kKMajorLayout;
     constexpr int kRows = 64 / LPR;  // rows per wave task
     const int groups = k / 8;
     uint32_t* planes = lds + kBankedPlanes / 4;
@@ -338,13 +342,21 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     // plus one 32-bit lane offset: no vector arithmetic per load.
     const int first_task = __builtin_amdgcn_readfirstlane(wave) * gridDim.x + blockIdx.x;
     const char* stream = reinterpret_cast<const char*>(w);
-    auto base_of = [&](int task) { return stream + (size_t)min(task, tasks - 1) * kRows * row_bytes; };
+    // K-major codes (K/128 blocks of N rows x 64 bytes): a task is still 64/LPR adjacent rows, a step
+    // is LPR/4 K blocks, and the lanes of one K block read the task's rows as one contiguous run of
+    // 64 bytes per row.  A lane still owns chunk sub + step * LPR of its row, so everything below the
+    // addressing is shared with the row-major form.
+    const size_t task_bytes = kKMajor ? (size_t)kRows * 64 : (size_t)kRows * row_bytes;
+    const size_t step_bytes = kKMajor ? (size_t)n * 64 * (LPR / 4) : (size_t)LPR * 16;
+    auto base_of = [&](int task) { return stream + (size_t)min(task, tasks - 1) * task_bytes; };
     auto lane_offset = [&](int task) {  // rows past the end re-read the task's first row and are not stored
         const int row = min(task, tasks - 1) * kRows + row_in_wave;
-        return (uint32_t)((row < n ? row_in_wave : 0) * row_bytes + sub * 16);
+        const int local_row = row < n ? row_in_wave : 0;
+        if (kKMajor) return (uint32_t)((sub >> 2) * n * 64 + local_row * 64 + (sub & 3) * 16);
+        return (uint32_t)(local_row * row_bytes + sub * 16);
     };
     auto fetch = [&](const char* base, uint32_t offset, int step) {
-        return *reinterpret_cast<const uint4*>(base + (size_t)min(step, steps - 1) * (LPR * 16) + offset);
+        return *reinterpret_cast<const uint4*>(base + (size_t)min(step, steps - 1) * step_bytes + offset);
     };
     uint4 ring[D];
 
@@ -603,7 +615,7 @@ bool use_banked(const orx_function& f, int mr) {
 int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
     const int mr = mr_for(rows);
     if (use_banked(f, mr)) {
-        const uint32_t lanes_per_row = (uint32_t)f.slots >> 8;
+        const uint32_t lanes_per_row = ((uint32_t)f.slots >> 8) & (uint32_t)(kKMajorLayout - 1);
         const uint32_t tasks = ceil_div((uint32_t)f.N, 64u / lanes_per_row);
         // every CU gets a workgroup as soon as there is a task for each: a small matrix then runs with
         // some idle waves per CU rather than with idle CUs
@@ -618,11 +630,11 @@ int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
     return ORX_OK;
 }
 
-template <int D, int LPR>
+template <int D, int LPR>  // LPR: the kernel's LAYOUT (lanes per row, + 64 for K-major codes)
 int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
                        const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
     const dim3 grid(g.grid[0]), block(kBankedThreads);
-    const bool hold = f.K / 32 / LPR == D;  // a row's steps fill the ring exactly
+    const bool hold = f.K / 32 / (LPR & (kKMajorLayout - 1)) == D;  // a row's steps fill the ring exactly
     switch (mr_for(rows)) {
         case 1:
             if (hold)
@@ -661,8 +673,12 @@ int gemv_launch_codec(const orx_function& f, int rows, const Geometry& g, hipStr
     const uint4* wp = reinterpret_cast<const uint4*>(w);
     if constexpr (CODEC == kQ4) {
         if (use_banked(f, mr_for(rows))) {
-            if ((f.slots >> 8) == 32) return gemv_launch_banked_depth<32>(f, rows, g, stream, a, wp, book, ws, as, out);
-            return gemv_launch_banked_depth<16>(f, rows, g, stream, a, wp, book, ws, as, out);
+            switch (f.slots >> 8) {
+                case 32: return gemv_launch_banked_depth<32>(f, rows, g, stream, a, wp, book, ws, as, out);
+                case kKMajorLayout + 16: return gemv_launch_banked_depth<kKMajorLayout + 16>(f, rows, g, stream, a, wp, book, ws, as, out);
+                case kKMajorLayout + 8: return gemv_launch_banked_depth<kKMajorLayout + 8>(f, rows, g, stream, a, wp, book, ws, as, out);
+                default: return gemv_launch_banked_depth<16>(f, rows, g, stream, a, wp, book, ws, as, out);
+            }
         }
     }
     switch (mr_for(rows)) {
@@ -686,6 +702,11 @@ int gemv_launch_codec(const orx_function& f, int rows, const Geometry& g, hipStr
 
 int gemv_prepare_device();
 
+// K-major two-stage codes are only served by the replicated-table kernel.
+bool gemv_serves_k_major(const orx_function& f, int rows) {
+    return f.flags == kQ4 && f.packed_k == 128 && ((uint32_t)f.slots >> 8) >= (uint32_t)kKMajorLayout && use_banked(f, mr_for(rows));
+}
+
 // Launchers used by the projection factories.  Argument order is the caller's business:
 // they pass already-unmarshalled pointers.
 int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
@@ -693,6 +714,10 @@ int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t 
     // LDS opt-in needs a device, so it happens at the first launch rather than at resolve time
     const int ready = gemv_prepare_device();
     if (ready != ORX_OK) return ready;
+    if (f.packed_k != 0 && !gemv_serves_k_major(f, rows)) {
+        set_error("%s: the gemv algorithm does not serve this K-major shape for %d rows", f.symbol.c_str(), rows);
+        return ORX_ERR_BAD_VARIANT;
+    }
     if (f.flags == kQ4) return gemv_launch_codec<kQ4>(f, rows, g, stream, a, w, book, ws, as, out);
     if (f.flags == kQ2) return gemv_launch_codec<kQ2>(f, rows, g, stream, a, w, book, ws, as, out);
     return gemv_launch_codec<kW8>(f, rows, g, stream, a, w, book, ws, as, out);
@@ -728,7 +753,10 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
     f->slots = 0;
     if (passes_override <= 0 && codec == kQ4) {
         const int chunks = f->K / 2 / 16;
-        const int lanes_per_row = chunks % 32 == 0 ? 32 : chunks % 16 == 0 ? 16 : 0;
+        int lanes_per_row = chunks % 32 == 0 ? 32 : chunks % 16 == 0 ? 16 : 0;
+        // K-major codes: 16 lanes per row measure best (13.4 us at N=17408, K=5120 against 15.1 with 8
+        // and 15.0 with 32), 8 for a K that is a multiple of 256 only
+        if (f->packed_k == 128) lanes_per_row = chunks % 16 == 0 ? 16 : chunks % 8 == 0 ? 8 : 0;
         if (lanes_per_row) {
             const int steps = chunks / lanes_per_row;
             int best_pad = 1 << 30, depth = 4;
@@ -737,7 +765,7 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
                 if (pad < best_pad) best_pad = pad, depth = candidate;
             }
             // the overflow flags hold one bit per step in a 64-bit word per lane column
-            if (steps <= 64) f->slots = depth | lanes_per_row << 8;
+            if (steps <= 64) f->slots = depth | (lanes_per_row + (f->packed_k == 128 ? kKMajorLayout : 0)) << 8;
         }
     }
     if (gemv_lds_bytes(*f, 4) > kLdsLimit) {
@@ -777,6 +805,8 @@ int gemv_prepare_device() {
     ORX_OPT_IN((gemv_banked_kernel<kQ4, 4, depth, lanes, false>))
     ORX_OPT_IN_BANKED(4, 16) ORX_OPT_IN_BANKED(5, 16) ORX_OPT_IN_BANKED(6, 16)
     ORX_OPT_IN_BANKED(4, 32) ORX_OPT_IN_BANKED(5, 32) ORX_OPT_IN_BANKED(6, 32)
+    ORX_OPT_IN_BANKED(4, kKMajorLayout + 8) ORX_OPT_IN_BANKED(5, kKMajorLayout + 8) ORX_OPT_IN_BANKED(6, kKMajorLayout + 8)
+    ORX_OPT_IN_BANKED(4, kKMajorLayout + 16) ORX_OPT_IN_BANKED(5, kKMajorLayout + 16) ORX_OPT_IN_BANKED(6, kKMajorLayout + 16)
 #undef ORX_OPT_IN_BANKED
 #undef ORX_OPT_IN
     done = true;

@@ -241,6 +241,43 @@ def test_q4_gemv_matches_oracle(m, n, k):
     np.testing.assert_array_equal(gu.host(got), want)
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("n,k", [(65, 256), (257, 2560), (1024, 5120), (130, 16384), (33, 8192 + 512), (7, 1536), (17408, 5120),
+                                 (40, 17408), (9, 768)])
+def test_q4_gemv_k_major_codes_match_oracle(m, n, k):
+    """The reference's storage layout (K/128 blocks of N rows): 16 lanes per row and tasks of 4 adjacent rows, or 8 lanes
+    and 8 rows when K is a multiple of 256 only."""
+    rng = np.random.default_rng(orc.SEED + 500 + m + n)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :4] = [-128, -1, 0, 127]
+    stored = orc.q4_pack_k(packed, 128)
+    w = orc.q4_integers(packed, TABLE)
+    acc = orc.int_dot(a_q, w)
+    ones_n, ones_m = np.ones(n, np.float16), np.ones(m, np.float16)
+    planes_fit = 131072 + (1 if m == 1 else 2 if m == 2 else 4) * (k // 8) * 12 + 256 + k // 32 + 16 <= 160 * 1024
+    if not planes_fit:  # the activation planes of so many rows do not fit beside the tables: refused at launch
+        with pytest.raises(Exception, match="K-major"):
+            gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), algorithm="gemv", packed_k=128)
+        return
+    got_acc = gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), dtype=torch.float32,
+                            algorithm="gemv", packed_k=128)
+    np.testing.assert_array_equal(gu.host(got_acc).astype(np.int64), acc.astype(np.int64))
+    storage = torch.full((m + 1, n + 5), 91.0, dtype=torch.float16, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 5,
+                  algorithm="gemv", packed_k=128)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.rescale(acc, scales, a_s))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+    if m <= 2:  # what `auto` picks for K-major codes at 1 and 2 rows
+        auto = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=128)
+        np.testing.assert_array_equal(gu.host(auto), orc.rescale(acc, scales, a_s))
+
+
+def test_q4_gemv_k_major_refuses_what_it_cannot_read():
+    with pytest.raises(Exception, match="gemv"):
+        gu.kernel("e8p_q4_projection", M=1, N=64, K=384, packed_k=128, algorithm="gemv")
+
+
 @pytest.mark.parametrize("variant", [{}, {"gemv_passes": 1}], ids=["replicated-tables", "compact-tables"])
 @pytest.mark.parametrize("m", [1, 2, 4])
 @pytest.mark.parametrize("pattern", ["all_max", "band", "sparse", "negative"])
