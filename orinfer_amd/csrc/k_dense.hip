@@ -48,7 +48,7 @@ struct DenseParams {
     const __half* ws;
     const __half* as;
     void* out;
-    int n, k, stride, m, out_f32;
+    int n, k, stride, m, out_f32, k_major;
 };
 
 // W: waves per workgroup (K is split over them); S: 64-wide K steps per wave (K = 64 W S); CB: token
@@ -222,8 +222,9 @@ __device__ __forceinline__ void direct_load_16(const void* global, void* lds_wav
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-// S: 64-wide K steps per decoder wave (K = 512 S); CB: token tiles of 16.
-template <int S, int CB>
+// S: 64-wide K steps per decoder wave (K = 512 S); CB: token tiles of 16; KM: K-major codes (K/128
+// blocks of N rows x 64 bytes; S is even then, so a decoder wave owns whole K blocks).
+template <int S, int CB, bool KM>
 __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DenseParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -238,8 +239,10 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
     constexpr int kRowBytes = 256 * S;                       // codes of one channel row
     constexpr int kPitch = kRowBytes + kRowPad;
     constexpr int kPieces = (kRowBytes + 1023) / 1024;       // 1 KiB requests per row
-    constexpr int kPerLoader = 16 * kPieces / kLoaders;      // requests of one loader wave per block
+    constexpr int kKBlocks = kDecoders * S / 2;              // K-major: one 1 KiB request per K block and channel block
+    constexpr int kPerLoader = (KM ? kKBlocks : 16 * kPieces) / kLoaders;  // requests of one loader wave per block
     static_assert(16 * kPieces % kLoaders == 0, "every loader wave issues the same number of requests");
+    static_assert(!KM || S % 2 == 0, "K-major: a decoder wave owns whole K blocks");
     int* sums = reinterpret_cast<int*>(lds + kSumBase);
     __half* scales = reinterpret_cast<__half*>(lds + kScaleBase);
     const uint32_t code_base = kScaleBase + (((uint32_t)run * 2 + 15) & ~15u);
@@ -255,14 +258,27 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
         const int loader = wave - kDecoders;
         auto request = [&](int block) {
             const int rows_in_block = min(16, rows_here - 16 * block);
-            const uint8_t* src = p.w + (int64_t)(first_row + 16 * block) * kRowBytes;
             uint8_t* dst = buffer(block);
+            if constexpr (KM) {
+                // One request is one K block of the 16 rows: 1 KiB contiguous in memory.  LDS position
+                // i (16 bytes each) holds row i/4, piece (i%4) ^ ((i/8)&3): with that swizzle the
+                // decoders' reads of one piece of 16 different rows fall into different bank groups.
+                const int row = lane >> 2, piece = (lane & 3) ^ ((lane >> 3) & 3);
+                const uint8_t* src = p.w + ((int64_t)first_row + 16 * block + row) * 64 + piece * 16;
 #pragma unroll
-            for (int i = 0; i < kPerLoader; ++i) {
-                const int piece = loader + kLoaders * i, row = piece / kPieces, part = piece - row * kPieces;
-                const int offset = part * 1024 + lane * 16;
-                if (row < rows_in_block && offset < kRowBytes)
-                    direct_load_16(src + (int64_t)row * kRowBytes + offset, dst + row * kPitch + part * 1024);
+                for (int i = 0; i < kPerLoader; ++i) {
+                    const int kb = loader + kLoaders * i;
+                    if (row < rows_in_block) direct_load_16(src + (int64_t)kb * p.n * 64, dst + kb * 1024);
+                }
+            } else {
+                const uint8_t* src = p.w + (int64_t)(first_row + 16 * block) * kRowBytes;
+#pragma unroll
+                for (int i = 0; i < kPerLoader; ++i) {
+                    const int piece = loader + kLoaders * i, row = piece / kPieces, part = piece - row * kPieces;
+                    const int offset = part * 1024 + lane * 16;
+                    if (row < rows_in_block && offset < kRowBytes)
+                        direct_load_16(src + (int64_t)row * kRowBytes + offset, dst + row * kPitch + part * 1024);
+                }
             }
         };
         request(0);
@@ -339,7 +355,10 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
             acc[c] = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights, token, acc[c], 0, 0, 0);
         }
     };
-    const int lane_codes = column * kPitch + wave * (kSlice / 2);  // this lane's row and this wave's K slice in a buffer
+    // this lane's codes in a buffer: row `column`, this wave's K slice, then 64 bytes per pair of steps
+    const int lane_codes = KM ? wave * (S / 2) * 1024 + (column * 4 + (quarter ^ ((column >> 1) & 3))) * 16
+                              : column * kPitch + wave * (kSlice / 2) + 16 * quarter;
+    constexpr int kPairBytes = KM ? 1024 : 64;
 
     for (int block = 0; block < blocks; ++block) {
         const uint8_t* src = buffer(block) + lane_codes;
@@ -348,13 +367,13 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
         for (int c = 0; c < CB; ++c) acc[c] = v4i{0, 0, 0, 0};
 #pragma unroll
         for (int d = 0; d < kPairs; ++d) {
-            const v4u pair = *reinterpret_cast<const v4u*>(src + 64 * d + 16 * quarter);
+            const v4u pair = *reinterpret_cast<const v4u*>(src + kPairBytes * d);
             const Looked l0 = request(pair.x), l1 = request(pair.y), l2 = request(pair.z), l3 = request(pair.w);
             multiply(acc, combine(l0), combine(l1), 2 * d);
             multiply(acc, combine(l2), combine(l3), 2 * d + 1);
         }
         if (kOdd) {
-            const v2u last = *reinterpret_cast<const v2u*>(src + 32 * (S - 1) + 8 * quarter);
+            const v2u last = *reinterpret_cast<const v2u*>(src + 32 * (S - 1) - 8 * quarter);  // lane_codes holds 16 * quarter
             const Looked l0 = request(last.x), l1 = request(last.y);
             multiply(acc, combine(l0), combine(l1), S - 1);
         }
@@ -435,26 +454,33 @@ uint32_t specialized_lds_bytes(int n, int k) {
 }
 
 // Loader-wave kernel: K a multiple of 512 up to 5120 (a decoder wave holds the token fragments of K/8).
-bool specialized_fits(int n, int k) { return k % 512 == 0 && k / 512 <= 10 && specialized_lds_bytes(n, k) <= kLdsLimit; }
+bool specialized_fits(int n, int k, int packed_k) {
+    if (k % 512 != 0 || k / 512 > 10 || specialized_lds_bytes(n, k) > kLdsLimit) return false;
+    return packed_k == 0 || (packed_k == 128 && k % 1024 == 0);
+}
 
-template <int S, int CB>
+template <int S, int CB, bool KM>
 int launch_specialized_shape(const DenseParams& p, hipStream_t stream) {
     static bool opted_in = false;
     if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
-        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_specialized_kernel<S, CB>),
+        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_specialized_kernel<S, CB, KM>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
                                    "hipFuncSetAttribute");
         if (code != ORX_OK) return code;
         opted_in = true;
     }
-    hipLaunchKernelGGL((dense_specialized_kernel<S, CB>), dim3(device_compute_units()), dim3(kSpecThreads),
+    hipLaunchKernelGGL((dense_specialized_kernel<S, CB, KM>), dim3(device_compute_units()), dim3(kSpecThreads),
                        specialized_lds_bytes(p.n, p.k), stream, p);
     return hip_check(hipGetLastError(), "launch projection (resident, loader waves)");
 }
 
 template <int S>
 int launch_specialized(const DenseParams& p, hipStream_t stream) {
-    return p.m <= 16 ? launch_specialized_shape<S, 1>(p, stream) : launch_specialized_shape<S, 2>(p, stream);
+    if constexpr (S % 2 == 0) {
+        if (p.k_major)
+            return p.m <= 16 ? launch_specialized_shape<S, 1, true>(p, stream) : launch_specialized_shape<S, 2, true>(p, stream);
+    }
+    return p.m <= 16 ? launch_specialized_shape<S, 1, false>(p, stream) : launch_specialized_shape<S, 2, false>(p, stream);
 }
 
 template <int S16>  // S16: steps per wave with 16 waves
@@ -467,15 +493,14 @@ int launch_steps(const DenseParams& p, hipStream_t stream) {
 // Row-major two-stage codes, K a multiple of 1024 up to 8192 (a wave's K slice is whole 64-wide
 // steps and its token fragments fit in registers), at most 32 rows per launch.
 bool dense_resident_eligible(int n, int k, int packed_k) {
-    if (packed_k != 0) return false;
-    if (specialized_fits(n, k)) return true;
-    return k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n, device_compute_units()) <= kLdsLimit;
+    if (specialized_fits(n, k, packed_k)) return true;
+    return packed_k == 0 && k % 1024 == 0 && k / 1024 <= 8 && lds_bytes(n, device_compute_units()) <= kLdsLimit;
 }
 
-void dense_resident_geometry(int rows, int n, int k, Geometry* g) {
+void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g) {
     const int chunk = rows < 32 ? rows : 32;  // rows per launch
     g->grid[1] = g->grid[2] = 1;
-    if (specialized_fits(n, k)) {
+    if (specialized_fits(n, k, packed_k)) {
         g->grid[0] = (uint32_t)device_compute_units();
         g->block[0] = kSpecThreads;
         g->shared = specialized_lds_bytes(n, k);
@@ -487,15 +512,15 @@ void dense_resident_geometry(int rows, int n, int k, Geometry* g) {
 }
 
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                          void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream) {
-    if (rows < 1 || rows > 32 || !dense_resident_eligible(n, k, 0)) {
+                          void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream) {
+    if (rows < 1 || rows > 32 || !dense_resident_eligible(n, k, packed_k)) {
         set_error("projection (resident): needs 1..32 rows and K a multiple of 512 up to 5120 or of 1024 up to 8192");
         return ORX_ERR_BAD_VARIANT;
     }
     DenseParams p = {};
     p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
-    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32;
-    if (specialized_fits(n, k)) {
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k != 0;
+    if (specialized_fits(n, k, packed_k)) {
         switch (k / 512) {
             case 1: return launch_specialized<1>(p, stream);
             case 2: return launch_specialized<2>(p, stream);

@@ -32,9 +32,9 @@ int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* boo
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
 bool dense_resident_eligible(int n, int k, int packed_k);
-void dense_resident_geometry(int rows, int n, int k, Geometry* g);
+void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g);
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                          void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream);
+                          void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 bool grouped_resident_eligible(int n, int k, int block_m, int tiles);
 bool grouped_resident_preferred(int rows, int experts, int n);
 void grouped_resident_geometry(int k, Geometry* g);
@@ -307,8 +307,9 @@ bool use_resident(const orx_function& f, int rows);
 bool use_gemv(const orx_function& f, int rows) {
     if (f.algorithm == kGemv) return true;
     if (f.algorithm != kAuto) return false;
-    // K-major codes: 1 and 2 rows (13.4 and 16.5 us at N=17408, K=5120; the streaming kernel takes 17.2)
-    if (f.packed_k != 0) return rows <= 2 && gemv_serves_k_major(f, rows);
+    // K-major codes: 1 row (13.4 us at N=17408, K=5120; the streaming kernel takes 17.2), and 2 rows
+    // (16.4 us) where the batched-decode kernel (15.4 us) does not take the shape
+    if (f.packed_k != 0) return rows <= 2 && gemv_serves_k_major(f, rows) && !use_resident(f, rows);
     return rows <= 4 && !use_resident(f, rows);
 }
 
@@ -330,7 +331,7 @@ bool use_resident(const orx_function& f, int rows) {
     // N=17408, K=5120), this kernel's MFMAs do not (19 us from 3 to 8 rows)
     // up to 64 rows as two launches of 32 (36 and 39 us at 48 and 64 rows against 42 and 48 us for
     // the streaming kernel)
-    return f.algorithm == kAuto && f.tiles == 0 && rows > 2 && rows <= 64;
+    return f.algorithm == kAuto && f.tiles == 0 && rows > (f.packed_k != 0 ? 1 : 2) && rows <= 64;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
@@ -352,7 +353,7 @@ bool use_expand(const orx_function& f, int rows) {
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_resident(f, rows)) {
-        dense_resident_geometry(rows, f.N, f.K, g);
+        dense_resident_geometry(rows, f.N, f.K, f.packed_k, g);
         return ORX_OK;
     }
     if (use_stream(f, rows)) {
@@ -387,7 +388,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
             const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
             const int code = dense_resident_launch(p.a + (size_t)first * f.K, p.w, p.book, p.ws, p.as + first,
                                                    static_cast<char*>(p.out) + out_offset, std::min(32, rows - first),
-                                                   f.N, f.K, f.stride, f.out_f32, stream);
+                                                   f.N, f.K, f.stride, f.packed_k, f.out_f32, stream);
             if (code != ORX_OK) return code;
         }
         return ORX_OK;

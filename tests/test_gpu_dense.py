@@ -379,6 +379,25 @@ def test_q4_resident_rows_blocks_and_tails(m, n, k):
     assert torch.equal(half, again)
 
 
+@pytest.mark.parametrize("m,n,k", [(3, 97, 1024), (16, 300, 2048), (17, 1000, 3072), (8, 5000, 4096), (32, 17408, 5120),
+                                   (64, 2050, 5120), (5, 40, 2048)])
+def test_q4_resident_k_major_codes(m, n, k):
+    """The loader/decoder kernel on the reference's storage layout (K/128 blocks of N rows x 64 bytes)."""
+    rng = np.random.default_rng(orc.SEED + 400 + m + n)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    stored = orc.q4_pack_k(packed, 128)
+    w = orc.q4_integers(packed, TABLE)
+    storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
+                  dtype=torch.float32, algorithm="resident", packed_k=128)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, w, scales, np.float32))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+    half = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=128)  # what `auto` picks
+    np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
+
+
 def test_q4_resident_dynamic_rows_and_refusals():
     rng = np.random.default_rng(orc.SEED + 77)
     n, k = 777, 2048
@@ -388,7 +407,7 @@ def test_q4_resident_dynamic_rows_and_refusals():
         got = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), rows=rows, dynamic=True,
                             capacity=100, algorithm="resident")
         np.testing.assert_array_equal(gu.host(got)[:rows], orc.project(a_q[:rows], a_s[:rows], w, scales))
-    for bad in (dict(K=1280), dict(K=9216), dict(packed_k=128), dict(M=129)):
+    for bad in (dict(K=1280), dict(K=9216), dict(packed_k=128, K=1536), dict(M=129)):
         variant = dict(M=8, N=256, K=1024, algorithm="resident")
         variant.update(bad)
         with pytest.raises(Exception, match="resident"):
