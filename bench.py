@@ -91,19 +91,21 @@ def main():
     class Q4Case:
         """One Q4A8 linear at (rows, n, k) with `copies` distinct weight tensors."""
 
-        def __init__(self, case, copies, algorithm="auto"):
+        def __init__(self, case, copies, algorithm="auto", packed_k=0):
             self.rows, self.n, self.k = case["rows"], case["n"], case["k"]
             rng = np.random.default_rng(7)
-            self.weights = [dev(case["packed"])]
+            first = case["packed"] if packed_k == 0 else codebook.q4_to_k_major(case["packed"], packed_k)
+            self.weights = [dev(first)]
             for _ in range(copies - 1):  # same shape and statistics, different bits
-                self.weights.append(dev(rng.integers(0, 2**32, case["packed"].shape, dtype=np.uint32)))
+                self.weights.append(dev(rng.integers(0, 2**32, first.shape, dtype=np.uint32)))
             self.scales = dev(case["scales"])
             self.x = dev(case["x"])
             self.a_q = torch.empty((self.rows, self.k), dtype=torch.int8, device="cuda")
             self.a_s = torch.empty((self.rows, 1), dtype=torch.float16, device="cuda")
             self.out = torch.empty((self.rows, self.n), dtype=torch.float16, device="cuda")
             self.quant = Kernel("activation_quantization", K=self.k)
-            self.proj = Kernel("e8p_q4_projection", M=self.rows, N=self.n, K=self.k, algorithm=algorithm)
+            self.proj = Kernel("e8p_q4_projection", M=self.rows, N=self.n, K=self.k, algorithm=algorithm,
+                               **({"packed_k": packed_k} if packed_k else {}))
 
         def quantize(self, s):
             self.quant(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=self.x, rows=self.rows)
@@ -195,6 +197,16 @@ def main():
                                 "frac_int8": round(ops / t / 1e12 / INT8_PEAK_TOPS, 4)}
             del case
         extra["config1_q4a8_sweep"] = sweep
+        # the same projection on the reference's storage layout (K-major blocks of 128)
+        k_major = {}
+        for rows in (1, 8, 32):
+            case = Q4Case(workloads.config1(rows), copies, packed_k=128)
+            t = timed_graph(lambda i, s: case.project(i, s), 2 * copies)
+            b = workloads.algorithmic_bytes_q4(rows, case.n, case.k)
+            k_major[str(rows)] = {"us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
+                                  "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4)}
+            del case
+        extra["config1_q4a8_k_major_codes"] = k_major
         del main_case
         torch.cuda.empty_cache()
         # config 2 W8A8
