@@ -247,6 +247,11 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
     __half* scales = reinterpret_cast<__half*>(lds + kScaleBase);
     const uint32_t code_base = kScaleBase + (((uint32_t)run * 2 + 15) & ~15u);
     auto buffer = [&](int block) { return lds + code_base + (block & 1) * (16 * kPitch); };
+    // The block that is not full (this CU's last rows) goes first: it lands quickly, while the tables
+    // are still being built, and the kernel does not end with a block that is mostly padding.
+    const int odd_rows = rows_here & 15;
+    auto block_start = [&](int block) { return odd_rows == 0 ? 16 * block : block == 0 ? rows_here - odd_rows : 16 * (block - 1); };
+    auto block_rows = [&](int block) { return odd_rows != 0 && block == 0 ? odd_rows : 16; };
 
     if (wave >= kDecoders) {
         // ---- loader waves ----
@@ -257,21 +262,21 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
         // MFMA at 5.2 us; a third block parked in the loaders' registers: 0.7 us slower overall).
         const int loader = wave - kDecoders;
         auto request = [&](int block) {
-            const int rows_in_block = min(16, rows_here - 16 * block);
+            const int rows_in_block = block_rows(block), start = block_start(block);
             uint8_t* dst = buffer(block);
             if constexpr (KM) {
                 // One request is one K block of the 16 rows: 1 KiB contiguous in memory.  LDS position
                 // i (16 bytes each) holds row i/4, piece (i%4) ^ ((i/8)&3): with that swizzle the
                 // decoders' reads of one piece of 16 different rows fall into different bank groups.
                 const int row = lane >> 2, piece = (lane & 3) ^ ((lane >> 3) & 3);
-                const uint8_t* src = p.w + ((int64_t)first_row + 16 * block + row) * 64 + piece * 16;
+                const uint8_t* src = p.w + ((int64_t)first_row + start + row) * 64 + piece * 16;
 #pragma unroll
                 for (int i = 0; i < kPerLoader; ++i) {
                     const int kb = loader + kLoaders * i;
                     if (row < rows_in_block) direct_load_16(src + (int64_t)kb * p.n * 64, dst + kb * 1024);
                 }
             } else {
-                const uint8_t* src = p.w + (int64_t)(first_row + 16 * block) * kRowBytes;
+                const uint8_t* src = p.w + (int64_t)(first_row + start) * kRowBytes;
 #pragma unroll
                 for (int i = 0; i < kPerLoader; ++i) {
                     const int piece = loader + kLoaders * i, row = piece / kPieces, part = piece - row * kPieces;
@@ -384,11 +389,13 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
 #pragma unroll
             for (int i = 0; i < 4; ++i) atomicAdd(mine + i * kSumStride + 16 * c, acc[c][i]);
         __syncthreads();
-        const int channel = 16 * block + out_channel;
-        if (finalises && channel < rows_here) {
-            int* cell = block_sums + out_channel * kSumStride + out_token;
-            const float value = rescale(*cell, __half2float(scales[channel]), token_scale);
-            *cell = 0;
+        const int channel = block_start(block) + out_channel;
+        // every cell is cleared, also those of padding rows: the buffer serves another block next
+        int* cell = block_sums + out_channel * kSumStride + out_token;
+        const int total = out_token < 16 * CB ? *cell : 0;
+        if (out_token < 16 * CB) *cell = 0;
+        if (finalises && out_channel < block_rows(block)) {
+            const float value = rescale(total, __half2float(scales[channel]), token_scale);
             const int64_t index = (int64_t)out_token * p.stride + first_row + channel;
             if (p.out_f32)
                 reinterpret_cast<float*>(p.out)[index] = value;
