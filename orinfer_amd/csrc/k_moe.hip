@@ -215,23 +215,21 @@ __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
     const int per_wave = ((assignments + kMetaWaves - 1) / kMetaWaves + 63) & ~63;
     const int first = wave * per_wave, last = min(assignments, first + per_wave);
     int* mine = counters + wave * experts;
+    const int id_bits = 32 - __builtin_clz(max(experts - 1, 1));
     for (int base = first; base < last; base += 64) {
         const int at = base + lane;
         const bool valid = at < last;
         const int id = valid ? ids[at] : -1;
         const int running = valid ? mine[id] : 0;  // nobody has written this expert in this step yet
-        int rank = 0, group = 0;
-        unsigned long long remaining = __ballot(valid);
-        while (remaining != 0ull) {  // wave-uniform: one round per distinct expert among the 64 lanes
-            const int leader = __ffsll((long long)remaining) - 1;
-            const int expert = __builtin_amdgcn_readlane(id, leader);
-            const unsigned long long same = __ballot(valid && id == expert);
-            if (valid && id == expert) {
-                rank = __popcll(same & ((1ull << lane) - 1ull));
-                group = __popcll(same);
-            }
-            remaining &= ~same;
+        // the lanes that hold the same expert, found one id bit at a time
+        unsigned long long same = __ballot(valid);
+        for (int bit = 0; bit < id_bits; ++bit) {
+            const bool set = (id >> bit) & 1;
+            const unsigned long long with = __ballot(valid && set);
+            same &= set ? with : ~with;
         }
+        const int rank = __popcll(same & ((1ull << lane) - 1ull));
+        const int group = __popcll(same);
         if (valid) {
             local[at] = running + rank;
             local_id[at] = id;
