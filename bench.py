@@ -283,7 +283,18 @@ def main():
         moved = rows * width * 3 + rows * 2 + width
         extra["rotate_a8_m8192_k5120"] = {"us": round(tr * 1e6, 2), "GBps": round(moved / tr / 1e9, 1),
                                           "frac_hbm": round(moved / tr / 1e9 / HBM_PEAK_GBS, 4), "bytes": moved}
-        del x, q
+        # the same with the residual add and RMSNorm in front: fp16 + fp32 in, fp16 + fp32 + int8 out
+        res = torch.randn((rows, width), dtype=torch.float32, device="cuda")
+        res_out = torch.empty_like(res)
+        gain = torch.randn((width,), dtype=torch.float16, device="cuda") * 0.1
+        y = torch.empty_like(x)
+        fused = Kernel("residual_norm_rotate_a8", M=rows, K=width)
+        tf = timed_graph(lambda i, st: fused(stream=st, Q=q, R=res, RO=res_out, S=sc, Signs=signs, W=gain, X=x, Y=y), 20)
+        moved = rows * width * (2 + 4 + 2 + 4 + 1) + rows * 2 + width * 3
+        extra["residual_norm_rotate_a8_m8192_k5120"] = {"us": round(tf * 1e6, 2), "GBps": round(moved / tf / 1e9, 1),
+                                                        "frac_hbm": round(moved / tf / 1e9 / HBM_PEAK_GBS, 4),
+                                                        "bytes": moved}
+        del x, q, res, res_out, y
     result["extra"] = extra
 
     # ---- CPU baseline: the numpy oracle on the contract workload (one full call) ----

@@ -230,6 +230,35 @@ def rotate_a8(x, signs, swiglu=False):
     return a8(rotated)
 
 
+def residual_norm(x, residual, weight, epsilon=1e-6, zero_centered=True):
+    """Residual add and RMSNorm: (fp16 normalised row, fp32 residual sum).
+
+    kernels/cuda/operators/op02_residual_norm.py:13-38: sum = fp32(x) + residual is returned
+    unrounded; the row is normalised as fp16((sum * rsqrt(mean(sum^2) + epsilon)) * (fp32(w) + 1))
+    (+0 when the weights are not stored zero-centred), the two products in fp32 in that order.
+    The mean is taken in float64 here: the order of the fp32 partial sums is the reference
+    kernel's own business, so a kernel is compared to one fp16 unit in the last place.
+    """
+    x = np.asarray(x).astype(np.float16)
+    total = (x.astype(np.float32) + np.asarray(residual, dtype=np.float32)).astype(np.float32)
+    mean = (total.astype(np.float64) ** 2).sum(axis=-1, keepdims=True) / x.shape[-1]
+    inverse = (1.0 / np.sqrt(mean.astype(np.float32).astype(np.float64) + np.float32(epsilon))).astype(np.float32)
+    gain = (np.asarray(weight).astype(np.float16).astype(np.float32) + np.float32(1.0 if zero_centered else 0.0))
+    scaled = (total * inverse).astype(np.float32)
+    return (scaled * gain).astype(np.float32).astype(np.float16), total
+
+
+def residual_norm_rotate_a8(x, residual, weight, signs, epsilon=1e-6, zero_centered=True):
+    """Fused residual RMSNorm + rotation + A8: (Y fp16, RO fp32, codes, row scales).
+
+    kernels/cuda/model/rotation_a8.py:607-659: the rotation reads the fp16 normalised row, so the
+    result equals rotate_a8 of Y (the reference's own check, models/qwen35/check_rows.py:167-172).
+    """
+    y, total = residual_norm(x, residual, weight, epsilon, zero_centered)
+    codes, scales = rotate_a8(y, signs)
+    return y, total, codes, scales
+
+
 def q4_embedding(ids, packed, table, scales, signs):
     """Token ids -> fp16 rows of the un-rotated embedding (kernels/cuda/model/e8p_q4.py:83-140).
 

@@ -115,6 +115,55 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
     }
 }
 
+// Seven butterfly stages over one block of 128 channels held by a half wave (lane l32 holds channels
+// 4*l32 .. 4*l32+3), the multiply by fp32(128^-1/2) and the fp16 materialisation; returns the largest
+// magnitude of the four fp16 results.
+__device__ __forceinline__ float rotate_block(float (&v)[4], int l32, __half (&out)[4]) {
+    // distance 1 and 2: inside the lane
+    {
+        const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
+        v[0] = a + c, v[2] = a - c, v[1] = b + d, v[3] = b - d;
+    }
+    // distance 4 .. 64: lanes at distance 1 .. 16; the upper element of a pair keeps left - right
+#pragma unroll
+    for (int bit = 0; bit < 5; ++bit) {
+        const bool upper = (l32 >> bit) & 1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float other = __shfl_xor(v[j], 1 << bit, 64);
+            v[j] = upper ? other - v[j] : other + v[j];
+        }
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        float scaled = v[j] * 0.08838834764831845f;
+        // opaque: the fp16 cast below must round the fp32 product, not a fused multiply-convert
+        asm volatile("" : "+v"(scaled));
+        out[j] = __float2half_rn(scaled);
+        amax = fmaxf(amax, fabsf(__half2float(out[j])));
+    }
+    return amax;
+}
+
+// Row scale from the largest magnitude, stored once, and the int8 codes of the fp16 row in LDS.
+__device__ __forceinline__ void quantise_row(const __half* rotated, float amax, int8_t* __restrict__ q,
+                                             __half* __restrict__ s, int row, int k) {
+    const int tid = threadIdx.x;
+    const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
+    const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
+    if (tid == 0) s[row] = stored;
+    const float scale = __half2float(stored);
+    for (int i = tid; i < k / 4; i += 256) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
+        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = packed;
+    }
+}
+
 // One workgroup per row, 4 waves; a wave takes two blocks of 128 channels per step (one per half
 // wave), a lane holds 4 consecutive channels: stages 1 and 2 are local, stages 4..64 are lane
 // exchanges at distance 1..16.  The rotated fp16 row is kept in LDS for the second pass.
@@ -147,45 +196,82 @@ __global__ __launch_bounds__(256) void rotate_a8_kernel(const __half* __restrict
                 v[j] = live ? value * sign : 0.f;
             }
         }
-        // distance 1 and 2: inside the lane
-        {
-            const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
-            v[0] = a + c, v[2] = a - c, v[1] = b + d, v[3] = b - d;
-        }
-        // distance 4 .. 64: lanes at distance 1 .. 16; the upper element of a pair keeps left - right
-#pragma unroll
-        for (int bit = 0; bit < 5; ++bit) {
-            const bool upper = (l32 >> bit) & 1;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float other = __shfl_xor(v[j], 1 << bit, 64);
-                v[j] = upper ? other - v[j] : other + v[j];
-            }
-        }
         __half out[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            float scaled = v[j] * 0.08838834764831845f;
-            // opaque: the fp16 cast below must round the fp32 product, not a fused multiply-convert
-            asm volatile("" : "+v"(scaled));
-            out[j] = __float2half_rn(scaled);
-            amax = fmaxf(amax, fabsf(__half2float(out[j])));
-        }
+        amax = fmaxf(amax, rotate_block(v, l32, out));
         if (live) *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
     }
     amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
-    const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
-    const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
-    if (tid == 0) s[row] = stored;
-    const float scale = __half2float(stored);
-    for (int i = tid; i < k / 4; i += 256) {
-        const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
-        const __half* h = reinterpret_cast<const __half*>(&raw);
-        uint32_t packed = 0;
+    quantise_row(rotated, amax, q, s, row, k);
+}
+
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
-        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = packed;
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    return (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+}
+
+// Residual add + RMSNorm in front of the rotation, one workgroup per row, same lane layout as
+// rotate_a8_kernel.  First pass: RO = fp32(X) + R, sum of squares.  Second pass: the fp32 sum is read
+// back by the thread that wrote it, Y = fp16((sum * rsqrt(mean + eps)) * (W + offset)), and that fp16
+// value goes through signs, butterflies and A8 as if rotate_a8_kernel had read Y.
+__global__ __launch_bounds__(256) void residual_norm_rotate_a8_kernel(
+    const __half* __restrict__ x, const float* __restrict__ r, const __half* __restrict__ w, __half* __restrict__ y,
+    float* __restrict__ ro, const int8_t* __restrict__ signs, int8_t* __restrict__ q, __half* __restrict__ s, int k,
+    float epsilon, float weight_offset) {
+    extern __shared__ __align__(16) __half rotated[];  // k halves
+    __shared__ float scratch[4], sum_scratch[4];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int half_wave = lane >> 5, l32 = lane & 31;
+    const int blocks = k / 128;  // even: k is a multiple of 256
+    const int64_t base = (int64_t)row * k;
+    float squares = 0.f;
+    for (int pair = wave; 2 * pair < blocks; pair += 4) {
+        const int first = (2 * pair + half_wave) * 128 + 4 * l32;
+        const uint2 raw = *reinterpret_cast<const uint2*>(x + base + first);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const float4 residual = *reinterpret_cast<const float4*>(r + base + first);
+        float4 sum;
+        sum.x = __half2float(h[0]) + residual.x;
+        sum.y = __half2float(h[1]) + residual.y;
+        sum.z = __half2float(h[2]) + residual.z;
+        sum.w = __half2float(h[3]) + residual.w;
+        *reinterpret_cast<float4*>(ro + base + first) = sum;
+        squares += sum.x * sum.x;
+        squares += sum.y * sum.y;
+        squares += sum.z * sum.z;
+        squares += sum.w * sum.w;
     }
+    const float total = block_sum(squares, sum_scratch);
+    const float inverse = rsqrtf(__fdiv_rn(total, (float)k) + epsilon);
+    float amax = 0.f;
+    for (int pair = wave; 2 * pair < blocks; pair += 4) {
+        const int first = (2 * pair + half_wave) * 128 + 4 * l32;
+        const float4 sum = *reinterpret_cast<const float4*>(ro + base + first);  // written above by this thread
+        const uint2 raw_w = *reinterpret_cast<const uint2*>(w + first);
+        const __half* weight = reinterpret_cast<const __half*>(&raw_w);
+        const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+        const float values[4] = {sum.x, sum.y, sum.z, sum.w};
+        __half normalized[4];
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float scaled = values[j] * inverse;
+            asm volatile("" : "+v"(scaled));  // two roundings, as written: (sum * inverse) * weight
+            float product = scaled * (__half2float(weight[j]) + weight_offset);
+            asm volatile("" : "+v"(product));
+            normalized[j] = __float2half_rn(product);
+            v[j] = __half2float(normalized[j]) * (float)(int8_t)(sign_word >> (8 * j));
+        }
+        *reinterpret_cast<uint2*>(y + base + first) = *reinterpret_cast<const uint2*>(normalized);
+        __half out[4];
+        amax = fmaxf(amax, rotate_block(v, l32, out));
+        *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
+    }
+    amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
+    quantise_row(rotated, amax, q, s, row, k);
 }
 
 // One workgroup per token; same lane layout as the rotation above (4 consecutive channels per lane,
@@ -349,6 +435,53 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// slots used: K, flags (bit0: weights stored zero-centred), capacity
+int residual_rotate_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->block[0] = 256;
+    g->shared = (uint32_t)f.K * 2;
+    return ORX_OK;
+}
+
+// Q, R, RO, S, Signs, W, X, Y[, m]: the buffers of rotation_a8.py:621-630 in generated-ABI order
+int residual_rotate_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    int8_t* q = pointer_arg<int8_t>(args, 0);
+    const float* r = pointer_arg<const float>(args, 1);
+    float* ro = pointer_arg<float>(args, 2);
+    __half* s = pointer_arg<__half>(args, 3);
+    const int8_t* signs = pointer_arg<const int8_t>(args, 4);
+    const __half* w = pointer_arg<const __half>(args, 5);
+    const __half* x = pointer_arg<const __half>(args, 6);
+    __half* y = pointer_arg<__half>(args, 7);
+    hipLaunchKernelGGL(residual_norm_rotate_a8_kernel, dim3(g.grid[0]), dim3(256), g.shared, stream, x, r, w, y, ro, signs,
+                       q, s, f.K, 1e-6f, (f.flags & 1) ? 1.0f : 0.0f);
+    return hip_check(hipGetLastError(), "launch residual_norm_rotate_a8");
+}
+
+int make_residual_rotate(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("K", 5120, &bad);
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const bool zero_centered = v.boolean("zero_centered", true, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // rotation_a8.py:612-613: complete 256-column tiles; the row has to fit LDS as fp16
+    if (f->M <= 0 || f->K <= 0 || f->K % 256 || f->K > 32768) {
+        set_error("residual_norm_rotate_a8: need M > 0 and K a multiple of 256 up to 32768");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = zero_centered ? 1 : 0;
+    // 16-byte accesses of R and RO, 8-byte of X, W and Y, 4-byte of Signs and Q
+    f->args = {{"Q", ArgPointer, 4},     {"R", ArgPointer, 16}, {"RO", ArgPointer, 16}, {"S", ArgPointer, 2},
+               {"Signs", ArgPointer, 4}, {"W", ArgPointer, 8},  {"X", ArgPointer, 8},   {"Y", ArgPointer, 8}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = reinterpret_cast<const void*>(&residual_norm_rotate_a8_kernel);
+    f->geometry = residual_rotate_geometry;
+    f->launch = residual_rotate_launch;
+    return ORX_OK;
+}
+
 // slots used: N (vocab), K (hidden), capacity
 int q4_embedding_geometry(const orx_function&, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
@@ -424,9 +557,11 @@ const Registration* quant_registrations(int* count) {
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
     {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
+    {"residual_norm_rotate_a8", make_residual_rotate, "M, K=5120, dynamic_rows=false, zero_centered=true",
+     "Q,R,RO,S,Signs,W,X,Y[,m]"},
     {"e8p_q4_embedding", make_q4_embedding, "M, vocab, hidden", "Book,IDs,Output,Scale,Signs,Weight,m"},
     };
-    *count = 4;
+    *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;
 }
 

@@ -35,7 +35,8 @@ def test_catalog_lists_every_symbol_and_resolves():
     catalog = lib.catalog()["kernels"]
     symbols = [entry["symbol"] for entry in catalog]
     assert len(symbols) == len(set(symbols))
-    for needed in ("activation_quantization", "swiglu", "rotate_activation_a8", "e8p_q4_projection", "int8_projection",
+    for needed in ("activation_quantization", "swiglu", "rotate_activation_a8", "residual_norm_rotate_a8", "e8p_q4_projection",
+                   "int8_projection",
                    "e8p_decode_grouped", "integer_vq_grouped", "e8p_q4_unpack", "e8p_q2_unpack", "router_topk",
                    "expert_histogram", "expert_offsets", "expert_tiles", "expert_dispatch", "moe_combine"):
         assert needed in symbols
@@ -46,6 +47,9 @@ ABI = {
     ("activation_quantization", (("K", 2560),)): ["Mask", "Q", "S", "X", "rows"],
     ("swiglu", (("I", 512),)): ["X", "Y", "rows"],
     ("rotate_activation_a8", (("M", 8), ("K", 5120))): ["Q", "S", "Signs", "X"],
+    ("residual_norm_rotate_a8", (("M", 8),)): ["Q", "R", "RO", "S", "Signs", "W", "X", "Y"],
+    ("residual_norm_rotate_a8", (("M", 4096), ("K", 2560), ("dynamic_rows", True), ("zero_centered", False))):
+        ["Q", "R", "RO", "S", "Signs", "W", "X", "Y", "m"],
     ("e8p_q4_embedding", (("M", 8), ("vocab", 1000), ("hidden", 5120))): ["Book", "IDs", "Output", "Scale", "Signs", "Weight", "m"],
     ("rotate_activation_a8", (("M", 8), ("K", 256), ("swiglu", True), ("dynamic_rows", True))): ["Q", "S", "Signs", "X", "m"],
     ("e8p_q4_projection", (("M", 1), ("N", 9728), ("K", 2560))): ["A", "AS", "Book", "Out", "S", "W"],

@@ -179,6 +179,89 @@ def test_rotate_activation_a8_dynamic_rows_zero_row_and_graph():
     np.testing.assert_allclose(approx, x.astype(np.float32) @ w.T, atol=0.6, rtol=0.05)
 
 
+def ulps_fp16(a, b):
+    """Distance in fp16 units in the last place (both finite)."""
+    def key(v):
+        bits = np.asarray(v, np.float16).view(np.int16).astype(np.int32)
+        return np.where(bits < 0, -(bits & 0x7FFF), bits)
+    return np.abs(key(a) - key(b))
+
+
+@pytest.mark.parametrize("m,k,zero_centered", [(1, 256, True), (3, 1536, True), (5, 5120, True), (2, 5120, False),
+                                               (1, 17408, True)])
+def test_residual_norm_rotate_a8_matches_oracle(m, k, zero_centered):
+    rng = np.random.default_rng(orc.SEED + 3 * m + k)
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    r = rng.normal(size=(m, k)).astype(np.float32)
+    w = (rng.normal(size=k) * 0.1 + (0.0 if zero_centered else 1.0)).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    variant = dict(M=m, K=k)
+    if not zero_centered:
+        variant["zero_centered"] = False
+    # one spare row behind every output, as in the reference's check (check_rows.py:156-161,172)
+    y = torch.full((m + 1, k), 91, dtype=torch.float16, device=gu.DEV)
+    ro = torch.full((m + 1, k), 91, dtype=torch.float32, device=gu.DEV)
+    q = torch.full((m + 1, k), 91, dtype=torch.int8, device=gu.DEV)
+    s = torch.full((m + 1,), 91, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("residual_norm_rotate_a8", **variant)(Q=q, R=gu.dev(r), RO=ro, S=s, Signs=gu.dev(signs), W=gu.dev(w),
+                                                    X=gu.dev(x), Y=y)
+    want_y, want_ro, _, _ = orc.residual_norm_rotate_a8(x, r, w, signs, zero_centered=zero_centered)
+    np.testing.assert_array_equal(gu.host(ro)[:m], want_ro)  # one fp32 add: exact
+    got_y = gu.host(y)[:m]
+    # fp16((sum * rsqrt(mean + eps)) * gain): the fp32 sum of squares and the reciprocal square root
+    # may differ in the last place from the float64 restatement, which moves an fp16 rounding by
+    # at most one unit in the last place
+    distance = ulps_fp16(got_y, want_y)
+    assert distance.max() <= 1 and (distance > 0).mean() < 0.02
+    # the rotation and the quantiser read the fp16 row the kernel wrote: codes and scales are exact
+    want_q, want_s = orc.rotate_a8(got_y, signs)
+    np.testing.assert_array_equal(gu.host(q)[:m], want_q)
+    np.testing.assert_array_equal(gu.host(s)[:m], want_s[:, 0])
+    for spare in (y, ro, q, s):
+        assert (gu.host(spare)[m:] == 91).all()
+
+
+def test_residual_norm_rotate_a8_dynamic_rows_zero_rows_and_composition():
+    rng = np.random.default_rng(orc.SEED + 77)
+    k, cap = 5120, 32
+    x = rng.normal(size=(17, k)).astype(np.float16)
+    r = rng.normal(size=(17, k)).astype(np.float32)
+    x[6], r[6] = 0, 0
+    w = (rng.normal(size=k) * 0.1).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    kern = gu.kernel("residual_norm_rotate_a8", M=cap, K=k, dynamic_rows=True)
+    rotation = gu.kernel("rotate_activation_a8", M=cap, K=k, dynamic_rows=True)
+    d = dict(R=gu.dev(r), Signs=gu.dev(signs), W=gu.dev(w), X=gu.dev(x))
+    y = torch.zeros((cap, k), dtype=torch.float16, device=gu.DEV)
+    ro = torch.zeros((cap, k), dtype=torch.float32, device=gu.DEV)
+    q = torch.zeros((cap, k), dtype=torch.int8, device=gu.DEV)
+    s = torch.zeros((cap,), dtype=torch.float16, device=gu.DEV)
+    for rows in (17, 1, 8):
+        for out in (y, ro, q, s):
+            out.fill_(91)
+        kern(Q=q, RO=ro, S=s, Y=y, m=rows, **d)
+        # the reference's own check: the fused kernel equals the rotation kernel run on Y
+        q2 = torch.zeros_like(q)
+        s2 = torch.zeros_like(s)
+        rotation(Q=q2, S=s2, Signs=d["Signs"], X=y, m=rows)
+        assert torch.equal(q[:rows], q2[:rows]) and torch.equal(s[:rows], s2[:rows])
+        assert (gu.host(q)[rows:] == 91).all() and (gu.host(y)[rows:] == 91).all()
+        np.testing.assert_array_equal(gu.host(ro)[:rows], x[:rows].astype(np.float32) + r[:rows])
+    kern(Q=q, RO=ro, S=s, Y=y, m=17, **d)
+    # an all-zero row: zero codes, scale one (check_rows.py:186-190)
+    assert not gu.host(q)[6].any() and float(gu.host(s)[6]) == 1.0 and not gu.host(y)[6].any()
+    # unit RMS before the gain: mean(Y / (1 + w))^2 is 1 to fp16 accuracy
+    unit = gu.host(y)[:17].astype(np.float64) / (1.0 + w.astype(np.float64))
+    live = [i for i in range(17) if i != 6]
+    np.testing.assert_allclose((unit[live] ** 2).mean(axis=1), 1.0, rtol=2e-3)
+
+
+def test_residual_norm_rotate_a8_refuses_incomplete_tiles():
+    for k in (128, 5120 + 128, 0, 32768 + 256):
+        with pytest.raises(Exception):
+            gu.kernel("residual_norm_rotate_a8", M=4, K=k)
+
+
 def test_q4_embedding_gather_matches_oracle():
     rng = np.random.default_rng(orc.SEED + 40)
     vocab, hidden, cap = 50, 640, 16

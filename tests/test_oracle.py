@@ -457,6 +457,58 @@ def test_rotate_a8_quantises_the_materialised_fp16_values():
     np.testing.assert_array_equal(s, ws)
 
 
+def test_residual_norm_closed_forms():
+    """Cases the mathematics fixes (kernels/cuda/operators/op02_residual_norm.py:13-38)."""
+    k = 256
+    # a constant row c with zero weights normalises to c / sqrt(c^2 + eps): +-1 to fp16 accuracy,
+    # and the residual sum comes back unrounded in fp32
+    x = np.full((1, k), 0.5, np.float16)
+    r = np.full((1, k), 2.0 ** -20, np.float32)
+    y, total = orc.residual_norm(x, r, np.zeros(k, np.float16))
+    assert total.dtype == np.float32 and (total == np.float32(0.5) + np.float32(2.0 ** -20)).all()
+    assert (y == np.float16(1.0)).all()
+    y, _ = orc.residual_norm(-x, -r, np.zeros(k, np.float16))
+    assert (y == np.float16(-1.0)).all()
+    # zero-centred weights add one to the gain; plain weights do not
+    w = np.full(k, 0.5, np.float16)
+    y, _ = orc.residual_norm(x, r, w)
+    assert (y == np.float16(1.5)).all()
+    y, _ = orc.residual_norm(x, r, w, zero_centered=False)
+    assert (y == np.float16(0.5)).all()
+    # scale invariance: doubling x and r leaves the normalised row unchanged up to the last place
+    # (epsilon and the rounding of the reciprocal root do not scale)
+    rng = np.random.default_rng(orc.SEED + 21)
+    x = rng.normal(size=(3, 512)).astype(np.float16)
+    r = rng.normal(size=(3, 512)).astype(np.float32)
+    w = (rng.normal(size=512) * 0.1).astype(np.float16)
+    y1, t1 = orc.residual_norm(x, r, w)
+    y2, t2 = orc.residual_norm(x * np.float16(2), r * 2, w)
+    np.testing.assert_array_equal(t2, 2 * t1)
+    np.testing.assert_allclose(y1.astype(np.float64), y2.astype(np.float64), rtol=2 ** -10, atol=2 ** -24)
+    # against a float64 evaluation of the formula; unit mean square before the gain
+    t64 = x.astype(np.float64) + r.astype(np.float64)
+    want = t64 / np.sqrt((t64 ** 2).mean(axis=1, keepdims=True) + 1e-6) * (1.0 + w.astype(np.float64))
+    np.testing.assert_allclose(y1.astype(np.float64), want, rtol=2 ** -10, atol=2 ** -24)
+    # the zero row: epsilon keeps the reciprocal finite, the row stays zero
+    y, t = orc.residual_norm(np.zeros((1, k), np.float16), np.zeros((1, k), np.float32), w[:k])
+    assert not y.any() and not t.any()
+
+
+def test_residual_norm_rotate_a8_is_the_rotation_of_the_normalised_row():
+    rng = np.random.default_rng(orc.SEED + 22)
+    x = rng.normal(size=(4, 512)).astype(np.float16)
+    r = rng.normal(size=(4, 512)).astype(np.float32)
+    x[2], r[2] = 0, 0
+    w = (rng.normal(size=512) * 0.1).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), 512)
+    y, total, q, s = orc.residual_norm_rotate_a8(x, r, w, signs)
+    wy, wt = orc.residual_norm(x, r, w)
+    wq, ws = orc.rotate_a8(wy, signs)
+    for got, want in ((y, wy), (total, wt), (q, wq), (s, ws)):
+        np.testing.assert_array_equal(got, want)
+    assert not q[2].any() and float(s[2, 0]) == 1.0  # models/qwen35/check_rows.py:186-190
+
+
 def test_q4_embedding_inverts_the_rotation_of_a_rotated_row():
     """Weights that are the rotation of a known vector come back as that vector: the embedding
     kernel's formula is the inverse rotation (H is an involution up to the 1/128 scaling)."""
