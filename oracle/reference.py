@@ -433,6 +433,28 @@ def grouped_project(d, ds, weights_int8, weight_scales, counts, row_offsets):
     return out
 
 
+def route_project(a_q, a_scale, weights_int8, weight_scales, ids, shared_input):
+    """Single-token expert routes: C[route] = project(A[row], W[ids[route]]) (integer_vq.py:380-444).
+
+    Every route indexes its expert's bank directly; row = 0 when all routes share one token row,
+    else row = route.  Same int32 dot and rescale as every other projection here.
+    """
+    ids = np.asarray(ids).reshape(-1)
+    a_q = np.asarray(a_q)
+    scale = np.asarray(a_scale).reshape(-1)
+    out = np.zeros((len(ids), weights_int8.shape[1]), np.float16)
+    for route, expert in enumerate(ids):
+        row = 0 if shared_input else route
+        acc = int_dot(a_q[row : row + 1], weights_int8[expert])
+        out[route] = rescale(acc, weight_scales[expert], scale[row : row + 1])[0]
+    return out
+
+
+def raw_table_words(table):
+    """The 256x8 int8 table as (256, 2) u32, the Book of the raw-basis kernels (vq.py:203)."""
+    return np.ascontiguousarray(np.asarray(table, np.int8)).view("<u4").reshape(256, 2)
+
+
 def moe_layer(x, logits, gate_up_codes, gate_up_scales, down_codes, down_scales, table, top_k, block_m=16):
     """Whole Q2A8 expert layer in the reference's program order
     (tests/cuda/operators/flash_next_quantized.py:117-135; kernels/cuda/model/moe.py):

@@ -698,6 +698,184 @@ int gemv_launch_codec(const orx_function& f, int rows, const Geometry& g, hipStr
     return hip_check(hipGetLastError(), "launch projection (gemv)");
 }
 
+
+// ---- single-token expert routes (kernels/cuda/model/integer_vq.py:380-444) ---------------------
+//
+// Every route indexes its expert's bank directly: no sorting, no tile list.  Book is the raw table
+// as (256, 2) u32 (vq.py:199-204): eight signed even bytes per entry, any values (the reference's
+// test draws random tables, tests/cuda/operators/flash_mtp_optimization.py:133), so the decode is
+// the general one: byte j of the quad is +-table[b][j] by sign bit j of (u ^ parity), plus one for
+// even parity, minus one for odd (vq.py:34-43).  The table is only assumed to hold bytes whose
+// negation fits int8 (the reference's tables are even, within +-126).
+//
+// One workgroup per (route, 32 output channels).  P is (E, K/128, N, 16) u16, so the 32 channels of
+// one K block are 1 KiB of consecutive codes: a wave reads them with one 16-byte load per lane
+// (lane = channel * 2 + half of the block), the eight waves take K blocks round robin.  The token row
+// is staged in LDS once; lanes of one half read the same 64 bytes from it (broadcast).
+
+constexpr uint32_t kHighBits = 0x80808080u, kLowBits = 0x7f7f7f7fu;
+
+// per byte: 0 - b, without carries between bytes
+__device__ __forceinline__ uint32_t negate_bytes(uint32_t b) { return (kHighBits - (b & kLowBits)) ^ (~b & kHighBits); }
+
+// byte masks of the coordinates whose sign bit is set: bits 0, 4, 1, 5 of `signs` (vq.py:17)
+__device__ __forceinline__ uint32_t sign_mask(uint32_t signs) {
+    const uint32_t flags = (signs & 1u) | ((signs & 16u) << 4) | ((signs & 2u) << 15) | ((signs & 32u) << 19);
+    return flags * 255u;
+}
+
+constexpr int kRouteChannels = 32, kRouteWaves = 8, kRouteThreads = 64 * kRouteWaves, kRouteDepth = 2;
+constexpr int kRouteTableBytes = 256 * 16, kRouteMaskBytes = 256 * 8, kRoutePartialBytes = kRouteWaves * kRouteChannels * 4;
+
+// The decode is split so that the inner loop is two table reads and two selects per code:
+//   q[j] = +-t[j] + c,  c = 1 - 2 * parity   =>   a . q = a . (+-t) + c * sum(a)
+// with +-t picked per byte between the table entry and its negation (both prepared per entry at
+// set-up), the byte masks of u prepared per u, and the sums of every 8 token bytes prepared once.
+__global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
+    const int8_t* __restrict__ a, const __half* __restrict__ as, const uint32_t* __restrict__ book, __half* __restrict__ c,
+    const int32_t* __restrict__ ids, const uint16_t* __restrict__ p, const __half* __restrict__ ws, int experts, int n,
+    int k, int shared_input) {
+    extern __shared__ __align__(16) uint8_t route_lds[];
+    uint4* table = reinterpret_cast<uint4*>(route_lds);                                    // entry, negated entry
+    uint2* masks = reinterpret_cast<uint2*>(route_lds + kRouteTableBytes);                  // per u
+    int* partial = reinterpret_cast<int*>(route_lds + kRouteTableBytes + kRouteMaskBytes);  // [waves][channels]
+    uint4* token = reinterpret_cast<uint4*>(route_lds + kRouteTableBytes + kRouteMaskBytes + kRoutePartialBytes);
+    int* token_sums = reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(token) + k);        // k / 8 sums
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int route = blockIdx.y;
+    const int expert = ids[route];
+    if ((unsigned)expert >= (unsigned)experts) return;  // nothing to index: the row stays as it was
+    const int row = shared_input ? 0 : route;
+    const int blocks = k / 128;
+    const int channel = blockIdx.x * kRouteChannels + (lane >> 1);
+    const int half = lane & 1;
+    const bool live = channel < n;
+    // codes of this lane: 16 bytes per K block, K blocks wave, wave + 8, ...; the first kRouteDepth
+    // loads leave before anything else
+    const uint4* codes = reinterpret_cast<const uint4*>(p + (((int64_t)expert * blocks) * n + (live ? channel : 0)) * 16) + half;
+    const int64_t block_stride = (int64_t)n * 2;  // uint4 per K block
+    uint4 held[kRouteDepth];
+#pragma unroll
+    for (int d = 0; d < kRouteDepth; ++d) {
+        const int kb = wave + d * kRouteWaves;
+        held[d] = kb < blocks ? codes[kb * block_stride] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    if (tid < 256) {
+        const uint2 entry = reinterpret_cast<const uint2*>(book)[tid];
+        table[tid] = make_uint4(entry.x, entry.y, negate_bytes(entry.x), negate_bytes(entry.y));
+    } else {
+        const uint32_t u = tid - 256;
+        const uint32_t signs = u ^ (__popc(u) & 1u);
+        masks[u] = make_uint2(sign_mask(signs), sign_mask(signs >> 2));
+    }
+    for (int i = tid; i < k / 8; i += kRouteThreads) {
+        const uint2 bytes = reinterpret_cast<const uint2*>(a + (int64_t)row * k)[i];
+        reinterpret_cast<uint2*>(token)[i] = bytes;
+        token_sums[i] = __builtin_amdgcn_sdot4((int)bytes.y, 0x01010101, __builtin_amdgcn_sdot4((int)bytes.x, 0x01010101, 0, false), false);
+    }
+    __syncthreads();
+    int acc = 0;
+    for (int first = wave; first < blocks; first += kRouteDepth * kRouteWaves) {
+#pragma unroll
+        for (int d = 0; d < kRouteDepth; ++d) {
+            const int kb = first + d * kRouteWaves;
+            if (kb >= blocks) break;  // wave-uniform
+            const uint4 now = held[d];
+            const int next = kb + kRouteDepth * kRouteWaves;
+            if (next < blocks) held[d] = codes[next * block_stride];
+            const uint32_t words[4] = {now.x, now.y, now.z, now.w};
+            const uint4* fragment = token + kb * 8 + half * 4;                                  // 64 token bytes
+            const int4* sums = reinterpret_cast<const int4*>(token_sums + kb * 16 + half * 8);  // of 8 codes
+            const int4 sums_low = sums[0], sums_high = sums[1];
+            const int sum_of[8] = {sums_low.x, sums_low.y, sums_low.z, sums_low.w, sums_high.x, sums_high.y, sums_high.z, sums_high.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint4 values = fragment[i];  // 16 token bytes: two codes
+                const uint32_t pair[4] = {values.x, values.y, values.z, values.w};
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const uint32_t code = (words[i] >> (16 * j)) & 0xffffu;
+                    const uint32_t u = code & 255u;
+                    const uint4 entry = table[code >> 8];
+                    const uint2 mask = masks[u];
+                    const uint32_t low = (entry.x & ~mask.x) | (entry.z & mask.x);
+                    const uint32_t high = (entry.y & ~mask.y) | (entry.w & mask.y);
+                    acc = __builtin_amdgcn_sdot4((int)pair[2 * j], (int)low, acc, false);
+                    acc = __builtin_amdgcn_sdot4((int)pair[2 * j + 1], (int)high, acc, false);
+                    acc += (__popc(u) & 1u) ? -sum_of[2 * i + j] : sum_of[2 * i + j];
+                }
+            }
+        }
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    if (half == 0) partial[wave * kRouteChannels + (lane >> 1)] = acc;
+    __syncthreads();
+    if (tid < kRouteChannels) {
+        const int out_channel = blockIdx.x * kRouteChannels + tid;
+        if (out_channel < n) {
+            int total = 0;
+#pragma unroll
+            for (int w = 0; w < kRouteWaves; ++w) total += partial[w * kRouteChannels + tid];
+            const float scaled = ((float)total * __half2float(ws[(int64_t)expert * n + out_channel])) * __half2float(as[row]);
+            c[(int64_t)route * n + out_channel] = __float2half_rn(scaled);
+        }
+    }
+}
+
+// slots used: E, M (routes), N, K, flags (bit0 shared_input)
+int route_gemv_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)f.N, (uint32_t)kRouteChannels);
+    g->grid[1] = (uint32_t)f.M;
+    g->block[0] = kRouteThreads;
+    g->shared = (uint32_t)(kRouteTableBytes + kRouteMaskBytes + kRoutePartialBytes) + (uint32_t)f.K + (uint32_t)f.K / 2;
+    return ORX_OK;
+}
+
+// A, AS, Book, C, IDs, P, WS: the buffers of integer_vq.py:388-395 in generated-ABI order
+int route_gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    const int8_t* a = pointer_arg<const int8_t>(args, 0);
+    const __half* as = pointer_arg<const __half>(args, 1);
+    const uint32_t* book = pointer_arg<const uint32_t>(args, 2);
+    __half* c = pointer_arg<__half>(args, 3);
+    const int32_t* ids = pointer_arg<const int32_t>(args, 4);
+    const uint16_t* p = pointer_arg<const uint16_t>(args, 5);
+    const __half* ws = pointer_arg<const __half>(args, 6);
+    hipLaunchKernelGGL(route_gemv_kernel, dim3(g.grid[0], g.grid[1]), dim3(kRouteThreads), g.shared, stream, a, as, book, c, ids, p,
+                       ws, f.E, f.N, f.K, f.flags & 1);
+    return hip_check(hipGetLastError(), "launch integer_e8p_gemv");
+}
+
+int make_route_gemv(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->E = (int)v.integer("E", 0, &bad);
+    f->capacity = f->M = (int)v.integer("routes", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    const bool shared_input = v.boolean("shared_input", false, &bad);
+    const long long block_n = v.integer("block_n", 8, &bad);  // the reference's tile hint: accepted, not used
+    if (bad || !v.has("shared_input")) {
+        set_error("integer_e8p_gemv: needs E, routes, N, K and shared_input");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    // integer_vq.py:382-383: K in whole 128-blocks, int32-exact dots, block_n in (4, 8, 16)
+    if (f->E <= 0 || f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 || (long long)f->K * 128 * 128 >= (1ll << 31) ||
+        (block_n != 4 && block_n != 8 && block_n != 16) || f->K > 65536) {
+        set_error("integer_e8p_gemv: need E, routes, N > 0, K a multiple of 128 with K*128*128 < 2^31, block_n in 4|8|16");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = shared_input ? 1 : 0;
+    // 16-byte loads of A rows and P, 8-byte loads of Book
+    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 8}, {"C", ArgPointer, 2},
+               {"IDs", ArgPointer, 4}, {"P", ArgPointer, 16}, {"WS", ArgPointer, 2}};
+    f->device_function = reinterpret_cast<const void*>(&route_gemv_kernel);
+    f->geometry = route_gemv_geometry;
+    f->launch = route_gemv_launch;
+    return ORX_OK;
+}
+
 }  // namespace
 
 int gemv_prepare_device();
@@ -814,9 +992,10 @@ int gemv_prepare_device() {
 }
 
 const Registration* gemv_registrations(int* count) {
-    static const Registration rows[] = {{nullptr, nullptr, nullptr, nullptr}
+    static const Registration rows[] = {
+    {"integer_e8p_gemv", make_route_gemv, "E, routes, N, K, shared_input, block_n=8", "A,AS,Book,C,IDs,P,WS"},
     };
-    *count = 0;
+    *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;
 }
 

@@ -37,7 +37,7 @@ def test_catalog_lists_every_symbol_and_resolves():
     assert len(symbols) == len(set(symbols))
     for needed in ("activation_quantization", "swiglu", "rotate_activation_a8", "residual_norm_rotate_a8", "e8p_q4_projection",
                    "int8_projection",
-                   "e8p_decode_grouped", "integer_vq_grouped", "e8p_q4_unpack", "e8p_q2_unpack", "router_topk",
+                   "e8p_decode_grouped", "integer_vq_grouped", "integer_e8p_gemv", "e8p_q4_unpack", "e8p_q2_unpack", "router_topk",
                    "expert_histogram", "expert_offsets", "expert_tiles", "expert_dispatch", "moe_combine"):
         assert needed in symbols
 
@@ -61,6 +61,8 @@ ABI = {
         ["A", "Gate", "GateScale", "Output", "TokenScale", "Up", "UpScale", "m"],
     ("e8p_decode_grouped", (("rows", 640), ("E", 512), ("tiles", 552), ("N", 1024), ("K", 2048))):
         ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "TileCount", "TileExpert", "TileRow", "WS"],
+    ("integer_e8p_gemv", (("E", 128), ("routes", 8), ("N", 1024), ("K", 2048), ("shared_input", True))):
+        ["A", "AS", "Book", "C", "IDs", "P", "WS"],
     ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
     ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
     ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],

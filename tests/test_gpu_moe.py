@@ -345,3 +345,104 @@ def test_moe_layer_graph_replay_with_new_routing():
     gu.sync()
     assert torch.equal(layer.out, replayed)
     assert not torch.equal(replayed, eager)
+
+
+# ---- single-token routes: every route indexes its expert's bank directly -----------------------
+def route_case(rng, e, routes, n, k, table, shared):
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    weights = np.stack([orc.q2_integers(c, table) for c in codes])
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    rows = 1 if shared else routes
+    a_q = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    return codes, weights, stored, a_q
+
+
+@pytest.mark.parametrize("n,k", [(65, 256), (1280, 2560), (2560, 640)])
+@pytest.mark.parametrize("shared", [True, False])
+def test_route_gemv_random_even_tables(n, k, shared):
+    """The reference's own check (tests/cuda/operators/flash_mtp_optimization.py:131-175): a random
+    even table (zeros and negative bytes included), int8 rows down to -128, power-of-two scales, a
+    guard row behind the output, then other ids and negated rows through the same handle."""
+    rng = np.random.default_rng(20261002 + n)
+    e, routes = 12, 3
+    table = (rng.integers(-63, 64, (256, 8)) * 2).astype(np.int8)
+    table[5] = 0
+    _, weights, stored, a_q = route_case(rng, e, routes, n, k, table, shared)
+    rows = a_q.shape[0]
+    ws = np.full((e, n), 0.015625, np.float16)
+    scale = np.full(rows, 0.0078125, np.float16)
+    ids = np.array([[11, 2, 7]], np.int32)
+    out = torch.full((routes + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    kern = gu.kernel("integer_e8p_gemv", E=e, routes=routes, N=n, K=k, shared_input=shared)
+    d_a, d_ids = gu.dev(a_q), gu.dev(ids)
+    args = dict(A=d_a, AS=gu.dev(scale), Book=gu.dev(orc.raw_table_words(table)), C=out, IDs=d_ids, P=gu.dev(stored),
+                WS=gu.dev(ws))
+    kern(**args)
+    np.testing.assert_array_equal(gu.host(out)[:routes], orc.route_project(a_q, scale, weights, ws, ids, shared))
+    assert (gu.host(out)[routes] == 91).all()
+    a_q = np.where(a_q == -128, 127, -a_q).astype(np.int8)
+    ids = np.array([[0, 9, 3]], np.int32)
+    d_a.copy_(gu.dev(a_q))
+    d_ids.copy_(gu.dev(ids))
+    kern(**args)
+    np.testing.assert_array_equal(gu.host(out)[:routes], orc.route_project(a_q, scale, weights, ws, ids, shared))
+    assert (gu.host(out)[routes] == 91).all()
+
+
+@pytest.mark.parametrize("n,k,shared", [(1024, 2048, True), (2048, 512, False)])
+def test_route_gemv_production_table_and_repeated_experts(n, k, shared):
+    # the shapes of one routed token: gate/up from the shared row, down from one row per route
+    rng = np.random.default_rng(orc.SEED + n)
+    e, routes = 128, 8
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    rows = 1 if shared else routes
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.03, rows).astype(np.float16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    ids = np.array([[127, 0, 5, 5, 64, 31, 127, 2]], np.int32)
+    out = torch.full((routes + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    kern = gu.kernel("integer_e8p_gemv", E=e, routes=routes, N=n, K=k, shared_input=shared, block_n=16)
+    d_ids = gu.dev(ids)
+    args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.dev(orc.raw_table_words(TABLE)), C=out, IDs=d_ids,
+                P=gu.dev(stored), WS=gu.dev(ws))
+    kern(**args)
+    used = sorted(set(ids.ravel().tolist()))
+    weights = np.zeros((e, n, k), np.int8)
+    for x in used:
+        weights[x] = orc.q2_integers(codes[x], TABLE)
+    want = orc.route_project(a_q, a_s, weights, ws, ids, shared)
+    np.testing.assert_array_equal(gu.host(out)[:routes], want)
+    # the routed batch of one token through the grouped kernel gives the same bytes
+    if shared:
+        counts = np.bincount(ids.ravel(), minlength=e).astype(np.int32)
+        offsets, tile_offsets, total = orc.expert_offsets(counts, 32)
+        cap = orc.tile_capacity(routes, e, 32)
+        te, tr = orc.expert_tiles(counts, tile_offsets, 32, cap)
+        grouped = torch.zeros((routes, n), dtype=torch.float16, device=gu.DEV)
+        gu.kernel("e8p_decode_grouped", rows=routes, E=e, tiles=cap, N=n, K=k, block_m=32)(
+            A=gu.dev(np.repeat(a_q, routes, 0)), AS=gu.dev(np.repeat(a_s, routes)), Book=gu.book(), C=grouped,
+            Counts=gu.dev(counts), Offsets=gu.dev(offsets), P=gu.dev(stored), TileCount=gu.dev(total),
+            TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
+        order = np.argsort(ids.ravel(), kind="stable")
+        np.testing.assert_array_equal(gu.host(grouped), want[order])
+    # an id outside the bank leaves its row as it was
+    out.fill_(91)
+    bad = ids.copy()
+    bad[0, 3], bad[0, 6] = e, -1
+    d_ids.copy_(gu.dev(bad))
+    kern(**args)
+    got = gu.host(out)
+    assert (got[3] == 91).all() and (got[6] == 91).all() and (got[routes] == 91).all()
+    keep = [0, 1, 2, 4, 5, 7]
+    np.testing.assert_array_equal(got[keep], want[keep])
+
+
+def test_route_gemv_refuses_bad_variants():
+    for variant in (dict(E=4, routes=2, N=64, K=192, shared_input=True),
+                    dict(E=4, routes=2, N=64, K=256),
+                    dict(E=0, routes=2, N=64, K=256, shared_input=False),
+                    dict(E=4, routes=2, N=64, K=256, shared_input=False, block_n=32),
+                    dict(E=4, routes=2, N=64, K=131072, shared_input=False)):
+        with pytest.raises(Exception):
+            gu.kernel("integer_e8p_gemv", **variant)

@@ -509,6 +509,34 @@ def test_residual_norm_rotate_a8_is_the_rotation_of_the_normalised_row():
     assert not q[2].any() and float(s[2, 0]) == 1.0  # models/qwen35/check_rows.py:186-190
 
 
+def test_route_project_indexes_banks_directly():
+    """integer_vq.py:380-444 against a float64 dot (the reference test's oracle, flash_mtp_optimization.py:159-166)."""
+    rng = np.random.default_rng(orc.SEED + 31)
+    e, routes, n, k = 5, 3, 7, 256
+    table = (rng.integers(-63, 64, (256, 8)) * 2).astype(np.int8)
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    weights = np.stack([orc.q2_integers(c, table) for c in codes])
+    assert np.abs(weights.astype(np.int32)).max() <= 127 and (weights.astype(np.int32) % 2 != 0).all()
+    ws = np.full((e, n), 0.015625, np.float16)
+    ids = np.array([[4, 0, 4]], np.int32)
+    for shared in (True, False):
+        rows = 1 if shared else routes
+        a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+        scale = np.full(rows, 0.0078125, np.float16)
+        got = orc.route_project(a, scale, weights, ws, ids, shared)
+        for route in range(routes):
+            row = 0 if shared else route
+            acc = (weights[ids[0, route]].astype(np.float64) * a[row].astype(np.float64)).sum(-1)
+            want = (np.float32(acc) * np.float32(0.015625)) * np.float32(0.0078125)
+            np.testing.assert_array_equal(got[route], want.astype(np.float16))
+        if shared:
+            np.testing.assert_array_equal(got[0], got[2])  # the same expert twice
+    # the raw table words are the table bytes, little endian, coordinates 0-3 then 4-7
+    words = orc.raw_table_words(table)
+    assert words.shape == (256, 2) and words.dtype == np.uint32
+    assert ((words[9, 1] >> 16) & 255) == (int(table[9, 6]) & 255)
+
+
 def test_q4_embedding_inverts_the_rotation_of_a_rotated_row():
     """Weights that are the rotation of a known vector come back as that vector: the embedding
     kernel's formula is the inverse rotation (H is an involution up to the 1/128 scaling)."""
