@@ -382,6 +382,55 @@ def expert_tiles(counts, tile_offsets, block_m, capacity):
     return tile_expert, tile_row
 
 
+def single_route_metadata(ids, experts, capacity):
+    """One token's routes in expert-id order (moe.py:659-709): every selected expert owns one row
+    and one tile.  Returns counts, relative slots (all zero), row offsets, tile offsets (equal to
+    the row offsets), tile experts and tile rows (entries from top_k on stay -1 here: the kernel
+    leaves them as they were) and the tile count (top_k).  ids distinct and inside [0, experts).
+    """
+    ids = np.asarray(ids, np.int32).reshape(-1)
+    experts_axis = np.arange(experts)[:, None]
+    counts = (ids[None, :] == experts_axis).sum(axis=1).astype(np.int32)
+    offsets = (ids[None, :] < experts_axis).sum(axis=1).astype(np.int32)
+    tile_expert = np.full(capacity, -1, np.int32)
+    tile_row = np.full(capacity, -1, np.int32)
+    for expert in ids:
+        position = int((ids < expert).sum())
+        tile_expert[position] = expert
+        tile_row[position] = 0
+    return (counts, np.zeros((1, len(ids)), np.int32), offsets, offsets.copy(), tile_expert, tile_row,
+            np.array([len(ids)], np.int32))
+
+
+def expert_partition(counts, hot_m, cold_m, cold_rows, hot_capacity, cold_capacity):
+    """Hot / cold tile lists over common row offsets (kernels/cuda/model/expert_partition.py:16-89).
+
+    Experts with more than cold_rows rows get tiles of hot_m rows, the others tiles of cold_m rows.
+    Returns a dict of RowOffsets, TileOffsets, TileCount, ColdOffsets, ColdCount and the four tile
+    lists (entries past the counts stay -1 here; the kernel leaves them as they were).
+    """
+    counts = np.asarray(counts, np.int64)
+    is_hot = counts > cold_rows
+    hot = np.where(is_hot, (counts + hot_m - 1) // hot_m, 0)
+    cold = np.where(~is_hot, (counts + cold_m - 1) // cold_m, 0)
+    out = {
+        "RowOffsets": (np.cumsum(counts) - counts).astype(np.int32),
+        "TileOffsets": (np.cumsum(hot) - hot).astype(np.int32),
+        "ColdOffsets": (np.cumsum(cold) - cold).astype(np.int32),
+        "TileCount": np.array([hot.sum()], np.int32),
+        "ColdCount": np.array([cold.sum()], np.int32),
+        "TileExpert": np.full(hot_capacity, -1, np.int32), "TileRow": np.full(hot_capacity, -1, np.int32),
+        "ColdExpert": np.full(cold_capacity, -1, np.int32), "ColdRow": np.full(cold_capacity, -1, np.int32),
+    }
+    for e, c in enumerate(counts):
+        names, height, base = (("TileExpert", "TileRow"), hot_m, out["TileOffsets"][e]) if is_hot[e] else (
+            ("ColdExpert", "ColdRow"), cold_m, out["ColdOffsets"][e])
+        for tile in range((int(c) + height - 1) // height):
+            out[names[0]][base + tile] = e
+            out[names[1]][base + tile] = tile * height
+    return out
+
+
 def tile_capacity(assignments, experts, block_m):
     """ceil(M*k/bm) + min(E, M*k) (moe.py:263-264)."""
     return (assignments + block_m - 1) // block_m + min(experts, assignments)

@@ -792,7 +792,7 @@ const Registration* gemm_registrations(int* count) {
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     };
-    *count = 7;
+    *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;
 }
 

@@ -186,6 +186,64 @@ __global__ __launch_bounds__(256) void expert_tiles_kernel(const int* __restrict
     }
 }
 
+// ---- hot / cold expert partition (kernels/cuda/model/expert_partition.py:16-89) -----------------
+// Experts with more than cold_rows routed rows get tiles of hot_m rows in one list, the others tiles
+// of cold_m rows in a second list; row offsets are the common ones, so two grouped launches (one per
+// list) write disjoint rows of the same output.
+__global__ __launch_bounds__(256) void partition_offsets_kernel(const int* __restrict__ counts, int* __restrict__ row_offsets,
+                                                                int* __restrict__ tile_offsets, int* __restrict__ tile_count,
+                                                                int* __restrict__ cold_offsets, int* __restrict__ cold_count,
+                                                                int experts, int hot_m, int cold_m, int cold_rows) {
+    __shared__ int scan[3][256];
+    int base[3] = {0, 0, 0};
+    for (int first = 0; first < experts; first += 256) {
+        const int e = first + threadIdx.x;
+        const int c = e < experts ? counts[e] : 0;
+        const int own[3] = {c, c > cold_rows ? (c + hot_m - 1) / hot_m : 0, c <= cold_rows ? (c + cold_m - 1) / cold_m : 0};
+#pragma unroll
+        for (int i = 0; i < 3; ++i) scan[i][threadIdx.x] = own[i];
+        __syncthreads();
+        for (int offset = 1; offset < 256; offset <<= 1) {
+            int add[3];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) add[i] = threadIdx.x >= offset ? scan[i][threadIdx.x - offset] : 0;
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 3; ++i) scan[i][threadIdx.x] += add[i];
+            __syncthreads();
+        }
+        if (e < experts) {
+            row_offsets[e] = base[0] + scan[0][threadIdx.x] - own[0];
+            tile_offsets[e] = base[1] + scan[1][threadIdx.x] - own[1];
+            cold_offsets[e] = base[2] + scan[2][threadIdx.x] - own[2];
+        }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) base[i] += scan[i][255];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) tile_count[0] = base[1], cold_count[0] = base[2];
+}
+
+// grid E
+__global__ __launch_bounds__(256) void partition_tiles_kernel(const int* __restrict__ counts,
+                                                              const int* __restrict__ tile_offsets,
+                                                              int* __restrict__ tile_expert, int* __restrict__ tile_row,
+                                                              const int* __restrict__ cold_offsets,
+                                                              int* __restrict__ cold_expert, int* __restrict__ cold_row,
+                                                              int hot_m, int cold_m, int cold_rows) {
+    const int e = blockIdx.x;
+    const int c = counts[e];
+    const bool cold = c <= cold_rows;
+    const int height = cold ? cold_m : hot_m;
+    const int base = cold ? cold_offsets[e] : tile_offsets[e];
+    int* experts_out = cold ? cold_expert : tile_expert;
+    int* rows_out = cold ? cold_row : tile_row;
+    for (int tile = threadIdx.x; tile * height < c; tile += 256) {
+        experts_out[base + tile] = e;
+        rows_out[base + tile] = tile * height;
+    }
+}
+
 // ---- all routing metadata in one launch ---------------------------------------------------------
 // kernels/cuda/model/moe.py:713-764: counts, stable relative slots, row and tile prefixes and the
 // tile list from one workgroup, instead of three dependent launches.  16 waves; wave w owns a
@@ -276,6 +334,39 @@ __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
             tile_row[first_tile + t] = t * block_m;
         }
     }
+}
+
+// One token: every selected expert owns one row and one tile, in expert-id order
+// (moe.py:659-709; ids distinct and inside [0, E), as router_topk leaves them).  One workgroup;
+// thread e counts the ids equal to and below e, thread rank places its id.  Tiles from top_k on
+// are left as they were.
+__global__ __launch_bounds__(256) void single_route_metadata_kernel(const int* __restrict__ ids, int* __restrict__ counts,
+                                                                    int* __restrict__ relative, int* __restrict__ offsets,
+                                                                    int* __restrict__ tile_offsets,
+                                                                    int* __restrict__ tile_expert, int* __restrict__ tile_row,
+                                                                    int* __restrict__ tile_count, int experts, int top_k) {
+    extern __shared__ int route_ids[];  // top_k
+    for (int rank = threadIdx.x; rank < top_k; rank += 256) route_ids[rank] = ids[rank];
+    __syncthreads();
+    for (int expert = threadIdx.x; expert < experts; expert += 256) {
+        int equal = 0, below = 0;
+        for (int rank = 0; rank < top_k; ++rank) {
+            equal += route_ids[rank] == expert;
+            below += route_ids[rank] < expert;
+        }
+        counts[expert] = equal;
+        offsets[expert] = below;
+        tile_offsets[expert] = below;
+    }
+    for (int rank = threadIdx.x; rank < top_k; rank += 256) {
+        const int mine = route_ids[rank];
+        int position = 0;
+        for (int other = 0; other < top_k; ++other) position += route_ids[other] < mine;
+        relative[rank] = 0;
+        tile_expert[position] = mine;
+        tile_row[position] = 0;
+    }
+    if (threadIdx.x == 0) tile_count[0] = top_k;
 }
 
 // grid M*top_k: copy one int8 row and its scales to the expert-sorted slot.
@@ -491,6 +582,100 @@ int make_metadata(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+int single_metadata_geometry(const orx_function& f, int, Geometry* g) {
+    g->grid[0] = 1;
+    g->block[0] = 256;
+    g->shared = (uint32_t)(f.top_k * sizeof(int));
+    return ORX_OK;
+}
+// Counts, IDs, Offsets, Relative, TileCount, TileExpert, TileOffsets, TileRow (moe.py:674-683 in generated-ABI order)
+int single_metadata_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(single_route_metadata_kernel, dim3(1), dim3(256), g.shared, s, pointer_arg<const int>(args, 1),
+                       pointer_arg<int>(args, 0), pointer_arg<int>(args, 3), pointer_arg<int>(args, 2),
+                       pointer_arg<int>(args, 6), pointer_arg<int>(args, 5), pointer_arg<int>(args, 7),
+                       pointer_arg<int>(args, 4), f.E, f.top_k);
+    return hip_check(hipGetLastError(), "launch single_route_metadata");
+}
+int make_single_metadata(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->E = (int)v.integer("E", 512, &bad);
+    f->top_k = (int)v.integer("top_k", 10, &bad);
+    f->tiles = (int)v.integer("capacity", 11, &bad);
+    f->M = f->capacity = 1;
+    // moe.py:665-671
+    if (bad || f->E <= 0 || f->top_k <= 0 || f->tiles <= 0 || f->top_k > f->E || f->tiles < f->top_k || f->top_k > 8192) {
+        set_error("single_route_metadata: need 0 < top_k <= E and capacity >= top_k");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"Counts", ArgPointer, 4},    {"IDs", ArgPointer, 4},        {"Offsets", ArgPointer, 4},
+               {"Relative", ArgPointer, 4},  {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
+               {"TileOffsets", ArgPointer, 4}, {"TileRow", ArgPointer, 4}};
+    f->geometry = single_metadata_geometry;
+    f->launch = single_metadata_launch;
+    f->device_function = reinterpret_cast<const void*>(&single_route_metadata_kernel);
+    return ORX_OK;
+}
+
+// slots used: E, block_m (hot_m), block_n (cold_m), group (cold_rows)
+bool partition_fields(const Variant& v, orx_function* f, const char* who) {
+    bool bad = false;
+    f->E = (int)v.integer("experts", 0, &bad);
+    f->block_m = (int)v.integer("hot_m", 0, &bad);
+    f->block_n = (int)v.integer("cold_m", 0, &bad);
+    f->group = (int)v.integer("cold_rows", 0, &bad);
+    // expert_partition.py:10-13
+    if (bad || f->E <= 0 || f->block_m <= 0 || f->block_n <= 0 || f->group <= 0) {
+        set_error("%s: need experts, hot_m, cold_m and cold_rows, all positive", who);
+        return false;
+    }
+    return true;
+}
+// ColdCount, ColdOffsets, Counts, RowOffsets, TileCount, TileOffsets (expert_partition.py:21-28 in generated-ABI order)
+int partition_offsets_launch(const orx_function& f, int, const Geometry&, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(partition_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 2),
+                       pointer_arg<int>(args, 3), pointer_arg<int>(args, 5), pointer_arg<int>(args, 4),
+                       pointer_arg<int>(args, 1), pointer_arg<int>(args, 0), f.E, f.block_m, f.block_n, f.group);
+    return hip_check(hipGetLastError(), "launch expert_partition_offsets");
+}
+int make_partition_offsets(const Variant& v, orx_function* f) {
+    if (!partition_fields(v, f, "expert_partition_offsets")) return ORX_ERR_BAD_VARIANT;
+    f->capacity = 1;
+    f->args = {{"ColdCount", ArgPointer, 4},  {"ColdOffsets", ArgPointer, 4}, {"Counts", ArgPointer, 4},
+               {"RowOffsets", ArgPointer, 4}, {"TileCount", ArgPointer, 4},   {"TileOffsets", ArgPointer, 4}};
+    f->geometry = one_block_geometry;
+    f->launch = partition_offsets_launch;
+    f->device_function = reinterpret_cast<const void*>(&partition_offsets_kernel);
+    return ORX_OK;
+}
+// ColdExpert, ColdOffsets, ColdRow, Counts, TileExpert, TileOffsets, TileRow[, m] (expert_partition.py:70-78)
+int partition_tiles_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(partition_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 3),
+                       pointer_arg<const int>(args, 5), pointer_arg<int>(args, 4), pointer_arg<int>(args, 6),
+                       pointer_arg<const int>(args, 1), pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), f.block_m,
+                       f.block_n, f.group);
+    return hip_check(hipGetLastError(), "launch expert_partition_tiles");
+}
+int make_partition_tiles(const Variant& v, orx_function* f) {
+    if (!partition_fields(v, f, "expert_partition_tiles")) return ORX_ERR_BAD_VARIANT;
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->top_k = (int)v.integer("top_k", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    // expert_partition.py:64-65
+    if (bad || f->M <= 0 || f->top_k <= 0 || f->top_k > f->E) {
+        set_error("expert_partition_tiles: need M > 0 and 0 < top_k <= experts");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"ColdExpert", ArgPointer, 4}, {"ColdOffsets", ArgPointer, 4}, {"ColdRow", ArgPointer, 4},
+               {"Counts", ArgPointer, 4},     {"TileExpert", ArgPointer, 4},  {"TileOffsets", ArgPointer, 4},
+               {"TileRow", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = histogram_geometry;
+    f->launch = partition_tiles_launch;
+    f->device_function = reinterpret_cast<const void*>(&partition_tiles_kernel);
+    return ORX_OK;
+}
+
 int dispatch_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)(rows * f.top_k);
     g->block[0] = 256;
@@ -568,12 +753,18 @@ const Registration* moe_registrations(int* count) {
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
     {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false",
      "Counts,IDs,RelativeSlot,RowOffsets,TileCount,TileExpert,TileOffsets,TileRow[,m]"},
+    {"single_route_metadata", make_single_metadata, "E=512, top_k=10, capacity=11",
+     "Counts,IDs,Offsets,Relative,TileCount,TileExpert,TileOffsets,TileRow"},
+    {"expert_partition_offsets", make_partition_offsets, "experts, hot_m, cold_m, cold_rows",
+     "ColdCount,ColdOffsets,Counts,RowOffsets,TileCount,TileOffsets"},
+    {"expert_partition_tiles", make_partition_tiles, "M, experts, top_k, hot_m, cold_m, cold_rows, dynamic_rows=false",
+     "ColdExpert,ColdOffsets,ColdRow,Counts,TileExpert,TileOffsets,TileRow[,m]"},
     {"expert_dispatch", make_dispatch, "M, H, E=512, top_k=10, scale_group=H, dynamic_rows=false",
      "A,D,DS,IDs,RelativeSlot,RowOffsets,Scale,SlotMap[,m]"},
     {"moe_combine", make_combine, "M, H, slots=M*top_k, top_k=10, dynamic_rows=false",
      "Expert,Output,Prob,Shared,SharedGate,SlotMap[,m]"},
     };
-    *count = 7;
+    *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;
 }
 

@@ -63,6 +63,12 @@ ABI = {
         ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "TileCount", "TileExpert", "TileRow", "WS"],
     ("integer_e8p_gemv", (("E", 128), ("routes", 8), ("N", 1024), ("K", 2048), ("shared_input", True))):
         ["A", "AS", "Book", "C", "IDs", "P", "WS"],
+    ("single_route_metadata", ()): ["Counts", "IDs", "Offsets", "Relative", "TileCount", "TileExpert", "TileOffsets", "TileRow"],
+    ("expert_partition_offsets", (("experts", 128), ("hot_m", 32), ("cold_m", 8), ("cold_rows", 8))):
+        ["ColdCount", "ColdOffsets", "Counts", "RowOffsets", "TileCount", "TileOffsets"],
+    ("expert_partition_tiles", (("M", 64), ("experts", 128), ("top_k", 8), ("hot_m", 32), ("cold_m", 8), ("cold_rows", 8),
+                                ("dynamic_rows", True))):
+        ["ColdExpert", "ColdOffsets", "ColdRow", "Counts", "TileExpert", "TileOffsets", "TileRow", "m"],
     ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
     ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
     ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],

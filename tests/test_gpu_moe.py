@@ -446,3 +446,62 @@ def test_route_gemv_refuses_bad_variants():
                     dict(E=4, routes=2, N=64, K=131072, shared_input=False)):
         with pytest.raises(Exception):
             gu.kernel("integer_e8p_gemv", **variant)
+
+
+@pytest.mark.parametrize("experts,top_k,capacity", [(512, 10, 11), (128, 8, 8), (16, 16, 20), (300, 1, 4)])
+def test_single_route_metadata_matches_oracle(experts, top_k, capacity):
+    rng = np.random.default_rng(orc.SEED + experts)
+    kern = gu.kernel("single_route_metadata", E=experts, top_k=top_k, capacity=capacity)
+    out = {name: torch.full((size,), 77, dtype=torch.int32, device=gu.DEV)
+           for name, size in (("Counts", experts), ("Relative", top_k), ("Offsets", experts), ("TileOffsets", experts),
+                              ("TileExpert", capacity), ("TileRow", capacity), ("TileCount", 1))}
+    d_ids = torch.zeros((1, top_k), dtype=torch.int32, device=gu.DEV)
+    for _ in range(2):  # the same handle and buffers with other ids
+        ids = rng.permutation(experts)[:top_k].astype(np.int32)[None, :]
+        d_ids.copy_(gu.dev(ids))
+        kern(IDs=d_ids, **out)
+        counts, relative, offsets, tile_offsets, tile_expert, tile_row, tile_count = orc.single_route_metadata(
+            ids, experts, capacity)
+        np.testing.assert_array_equal(gu.host(out["Counts"]), counts)
+        np.testing.assert_array_equal(gu.host(out["Relative"]), relative[0])
+        np.testing.assert_array_equal(gu.host(out["Offsets"]), offsets)
+        np.testing.assert_array_equal(gu.host(out["TileOffsets"]), tile_offsets)
+        np.testing.assert_array_equal(gu.host(out["TileCount"]), tile_count)
+        np.testing.assert_array_equal(gu.host(out["TileExpert"])[:top_k], tile_expert[:top_k])
+        np.testing.assert_array_equal(gu.host(out["TileRow"])[:top_k], tile_row[:top_k])
+        # the unused tile tail is preserved (moe.py:663)
+        assert (gu.host(out["TileExpert"])[top_k:] == 77).all() and (gu.host(out["TileRow"])[top_k:] == 77).all()
+    for variant in (dict(E=4, top_k=5), dict(E=8, top_k=4, capacity=3), dict(E=0)):
+        with pytest.raises(Exception):
+            gu.kernel("single_route_metadata", **variant)
+
+
+@pytest.mark.parametrize("experts,hot_m,cold_m,cold_rows", [(23, 16, 4, 8), (300, 32, 8, 8), (128, 64, 16, 100)])
+def test_expert_partition_matches_oracle(experts, hot_m, cold_m, cold_rows):
+    rng = np.random.default_rng(orc.SEED + experts + hot_m)
+    m, top_k = 96, min(8, experts)
+    ids, _ = orc.router_topk(rng.normal(size=(m, experts)).astype(np.float32), top_k)
+    counts, _ = orc.expert_histogram(ids, experts)
+    counts[0] = cold_rows  # on the threshold: cold
+    hot_cap = orc.tile_capacity(m * top_k, experts, hot_m)
+    cold_cap = orc.tile_capacity(m * top_k, experts, cold_m)
+    want = orc.expert_partition(counts, hot_m, cold_m, cold_rows, hot_cap, cold_cap)
+    sizes = dict(RowOffsets=experts, TileOffsets=experts, ColdOffsets=experts, TileCount=1, ColdCount=1,
+                 TileExpert=hot_cap, TileRow=hot_cap, ColdExpert=cold_cap, ColdRow=cold_cap)
+    out = {name: torch.full((size,), -1, dtype=torch.int32, device=gu.DEV) for name, size in sizes.items()}
+    d_counts = gu.dev(counts)
+    shape = dict(experts=experts, hot_m=hot_m, cold_m=cold_m, cold_rows=cold_rows)
+    gu.kernel("expert_partition_offsets", **shape)(
+        Counts=d_counts, **{name: out[name] for name in ("ColdCount", "ColdOffsets", "RowOffsets", "TileCount", "TileOffsets")})
+    gu.kernel("expert_partition_tiles", M=m, top_k=top_k, dynamic_rows=True, **shape)(
+        Counts=d_counts, m=m,
+        **{name: out[name] for name in ("ColdExpert", "ColdOffsets", "ColdRow", "TileExpert", "TileOffsets", "TileRow")})
+    for name in sizes:
+        np.testing.assert_array_equal(gu.host(out[name]), want[name], err_msg=name)
+    assert int(want["TileCount"][0]) > 0 or cold_rows >= counts.max()
+    for variant in (dict(experts=0, hot_m=8, cold_m=8, cold_rows=1), dict(experts=4, hot_m=8, cold_m=0, cold_rows=1),
+                    dict(experts=4, hot_m=8, cold_m=8)):
+        with pytest.raises(Exception):
+            gu.kernel("expert_partition_offsets", **variant)
+    with pytest.raises(Exception):
+        gu.kernel("expert_partition_tiles", M=4, top_k=9, experts=8, hot_m=8, cold_m=8, cold_rows=2)

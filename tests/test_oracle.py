@@ -537,6 +537,63 @@ def test_route_project_indexes_banks_directly():
     assert ((words[9, 1] >> 16) & 255) == (int(table[9, 6]) & 255)
 
 
+def test_single_route_metadata_is_the_general_metadata_of_one_token():
+    """moe.py:659-709: with distinct ids the one-token form equals histogram + offsets + tiles
+    (moe.py:177-282) at any tile height."""
+    rng = np.random.default_rng(orc.SEED + 41)
+    for experts, top_k in ((512, 10), (128, 8), (16, 16), (7, 1)):
+        ids = rng.permutation(experts)[:top_k].astype(np.int32)[None, :]
+        capacity = top_k + 3
+        counts, relative, offsets, tile_offsets, tile_expert, tile_row, tile_count = orc.single_route_metadata(
+            ids, experts, capacity)
+        want_counts, want_relative = orc.expert_histogram(ids, experts)
+        np.testing.assert_array_equal(counts, want_counts)
+        np.testing.assert_array_equal(relative, want_relative)
+        for block_m in (8, 32):
+            want_offsets, want_tile_offsets, want_total = orc.expert_offsets(want_counts, block_m)
+            want_expert, want_row = orc.expert_tiles(want_counts, want_tile_offsets, block_m, capacity)
+            np.testing.assert_array_equal(offsets, want_offsets)
+            np.testing.assert_array_equal(tile_offsets, want_tile_offsets)
+            np.testing.assert_array_equal(tile_count, want_total)
+            np.testing.assert_array_equal(tile_expert, want_expert)
+            np.testing.assert_array_equal(tile_row, want_row)
+        assert tile_expert[:top_k].tolist() == sorted(ids.ravel().tolist()) and (tile_expert[top_k:] == -1).all()
+
+
+def test_expert_partition_covers_every_row_once():
+    """expert_partition.py:1-5: both lists keep the global row offsets and own disjoint tiles."""
+    rng = np.random.default_rng(orc.SEED + 43)
+    counts = rng.integers(0, 40, 23).astype(np.int32)
+    counts[[0, 5]] = 0
+    counts[7], counts[8] = 8, 9  # on and just above the threshold
+    hot_m, cold_m, cold_rows = 16, 4, 8
+    total = int(counts.sum())
+    part = orc.expert_partition(counts, hot_m, cold_m, cold_rows, orc.tile_capacity(total, 23, hot_m),
+                                orc.tile_capacity(total, 23, cold_m))
+    seen = np.zeros(total, np.int32)
+    for experts, rows, count, height, hot in (("TileExpert", "TileRow", "TileCount", hot_m, True),
+                                              ("ColdExpert", "ColdRow", "ColdCount", cold_m, False)):
+        live = int(part[count][0])
+        assert (part[experts][live:] == -1).all()
+        for e, first in zip(part[experts][:live], part[rows][:live]):
+            assert (counts[e] > cold_rows) == hot
+            rows_in_tile = min(height, counts[e] - first)
+            assert rows_in_tile > 0
+            seen[part["RowOffsets"][e] + first : part["RowOffsets"][e] + first + rows_in_tile] += 1
+        assert list(part[experts][:live]) == sorted(part[experts][:live])
+    assert (seen == 1).all()
+    # a threshold below every count gives the plain tile list of moe.py:214-282 in the hot list
+    plain = orc.expert_partition(np.maximum(counts, 1), hot_m, cold_m, 0, 64, 64)
+    offsets, tile_offsets, tile_total = orc.expert_offsets(np.maximum(counts, 1), hot_m)
+    tile_expert, tile_row = orc.expert_tiles(np.maximum(counts, 1), tile_offsets, hot_m, 64)
+    np.testing.assert_array_equal(plain["RowOffsets"], offsets)
+    np.testing.assert_array_equal(plain["TileOffsets"], tile_offsets)
+    np.testing.assert_array_equal(plain["TileCount"], tile_total)
+    np.testing.assert_array_equal(plain["TileExpert"], tile_expert)
+    np.testing.assert_array_equal(plain["TileRow"], tile_row)
+    assert plain["ColdCount"][0] == 0
+
+
 def test_q4_embedding_inverts_the_rotation_of_a_rotated_row():
     """Weights that are the rotation of a known vector come back as that vector: the embedding
     kernel's formula is the inverse rotation (H is an involution up to the 1/128 scaling)."""
