@@ -85,6 +85,7 @@ struct GemmParams {
     const int* tile_row;
     const int* tile_count;
     int64_t expert_weight_stride;  // bytes between experts in w
+    int tile_rows;                 // rows a routed tile may hold (0: the kernel's own tile height)
 };
 
 template <int CODEC>
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         const int expert = p.tile_expert[tile];
         const int first = p.tile_row[tile];
         row0 = p.offsets[expert] + first;
-        rows_here = min(BM, p.counts[expert] - first);
+        rows_here = min(p.tile_rows > 0 ? min(BM, p.tile_rows) : BM, p.counts[expert] - first);
         if (rows_here <= 0) return;
         w_base += (int64_t)expert * p.expert_weight_stride;
         ws += (int64_t)expert * p.n;
@@ -729,6 +730,83 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// ---- routed Q4 / W8 banks (kernels/cuda/model/moe.py:52-143) ---------------------------------
+// A, AS, Book, Counts, Offsets, Out, TileCount, TileExpert, TileRow, W, WS[, m]: the buffers of
+// moe.py:115-127 in generated-ABI order.  The tile list is the caller's (built with the variant's
+// block_m); a tile runs on the smallest MFMA tile that holds block_m rows.
+int experts_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)f.N, 128u);
+    g->grid[1] = (uint32_t)f.tiles;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int experts_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.as = pointer_arg<const __half>(args, 1);
+    p.book = pointer_arg<const uint32_t>(args, 2);
+    p.counts = pointer_arg<const int>(args, 3);
+    p.offsets = pointer_arg<const int>(args, 4);
+    p.out = pointer_arg<void>(args, 5);
+    p.tile_count = pointer_arg<const int>(args, 6);
+    p.tile_expert = pointer_arg<const int>(args, 7);
+    p.tile_row = pointer_arg<const int>(args, 8);
+    p.w = pointer_arg<const void>(args, 9);
+    p.ws = pointer_arg<const __half>(args, 10);
+    p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity * f.top_k, p.out_f32 = 0;
+    p.tile_rows = f.block_m;
+    const int bm = f.block_m <= 32 ? 32 : f.block_m <= 64 ? 64 : 128;
+    if (f.flags == kQ4) {
+        p.packed_k = 128;
+        p.expert_weight_stride = (int64_t)f.N * (f.K / 2);
+        return launch_mfma<kQ4, true>(bm, p, g, stream);
+    }
+    p.packed_k = 0;
+    p.expert_weight_stride = (int64_t)f.N * f.K;
+    return launch_mfma<kW8, true>(bm, p, g, stream);
+}
+
+int make_integer_experts(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->E = (int)v.integer("E", 0, &bad);
+    f->top_k = (int)v.integer("top_k", 0, &bad);
+    f->block_m = (int)v.integer("block_m", 16, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const std::string codec = v.string("codec", "e8p_q4", &bad);
+    // the reference's tile hints: checked as it checks them (moe.py:72-88), otherwise not used
+    const long long block_n = v.integer("block_n", 64, &bad), block_k = v.integer("block_k", 128, &bad);
+    const long long stages = v.integer("stages", 2, &bad), minimum_blocks = v.integer("minimum_blocks", 1, &bad);
+    (void)v.integer("tail_m", 0, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    const bool w8 = codec == "w8";
+    const bool block_m_ok = f->block_m == 8 || f->block_m == 16 || f->block_m == 32 || f->block_m == 64 || f->block_m == 128;
+    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || f->K % 128 || !block_m_ok ||
+        (block_n != 32 && block_n != 64 && block_n != 128) || (!w8 && codec != "e8p_q4") ||
+        (w8 && (f->block_m == 8 || block_n == 32)) || (block_k != 128 && block_k != 256) || f->K % block_k ||
+        (stages != 1 && stages != 2) || minimum_blocks <= 0 || (int64_t)f->K * 128 * 128 > 2147483647LL) {
+        set_error("integer_experts: invalid grouped integer projection geometry (block_m 8..128 here)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = w8 ? kW8 : kQ4;
+    const int64_t assignments = (int64_t)f->M * f->top_k;
+    f->tiles = (int)((assignments + f->block_m - 1) / f->block_m + std::min<int64_t>(f->E, assignments));  // moe.py:89
+    f->args = {{"A", ArgPointer, 16},        {"AS", ArgPointer, 2},         {"Book", ArgPointer, 4},
+               {"Counts", ArgPointer, 4},    {"Offsets", ArgPointer, 4},    {"Out", ArgPointer, 2},
+               {"TileCount", ArgPointer, 4}, {"TileExpert", ArgPointer, 4}, {"TileRow", ArgPointer, 4},
+               {"W", ArgPointer, 16},        {"WS", ArgPointer, 2}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = experts_geometry;
+    f->launch = experts_launch;
+    f->device_function = nullptr;
+    return ORX_OK;
+}
+
 // ---- unpack ----------------------------------------------------------------------------------
 // Book, Output, W
 int unpack_geometry(const orx_function& f, int rows, Geometry* g) {
@@ -789,6 +867,9 @@ const Registration* gemm_registrations(int* count) {
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
     {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
+    {"integer_experts", make_integer_experts,
+     "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
+     "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     };

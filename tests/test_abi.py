@@ -69,6 +69,10 @@ ABI = {
     ("expert_partition_tiles", (("M", 64), ("experts", 128), ("top_k", 8), ("hot_m", 32), ("cold_m", 8), ("cold_rows", 8),
                                 ("dynamic_rows", True))):
         ["ColdExpert", "ColdOffsets", "ColdRow", "Counts", "TileExpert", "TileOffsets", "TileRow", "m"],
+    ("integer_experts", (("M", 64), ("N", 1024), ("K", 2048), ("E", 128), ("top_k", 8), ("dynamic_rows", True))):
+        ["A", "AS", "Book", "Counts", "Offsets", "Out", "TileCount", "TileExpert", "TileRow", "W", "WS", "m"],
+    ("integer_experts", (("M", 64), ("N", 1024), ("K", 2048), ("E", 128), ("top_k", 8), ("codec", "w8"))):
+        ["A", "AS", "Book", "Counts", "Offsets", "Out", "TileCount", "TileExpert", "TileRow", "W", "WS"],
     ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
     ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
     ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],

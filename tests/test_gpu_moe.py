@@ -505,3 +505,85 @@ def test_expert_partition_matches_oracle(experts, hot_m, cold_m, cold_rows):
             gu.kernel("expert_partition_offsets", **variant)
     with pytest.raises(Exception):
         gu.kernel("expert_partition_tiles", M=4, top_k=9, experts=8, hot_m=8, cold_m=8, cold_rows=2)
+
+
+# ---- routed Q4 / W8 banks (integer_experts) -----------------------------------------------------
+@pytest.mark.parametrize("codec,bm", [("e8p_q4", 8), ("e8p_q4", 16), ("e8p_q4", 64), ("e8p_q4", 128), ("w8", 16),
+                                      ("w8", 32), ("w8", 128)])
+def test_integer_experts_q4_and_w8_banks(codec, bm):
+    rng = np.random.default_rng(orc.SEED + bm + len(codec))
+    e, n, k, m, top_k = 9, 200, 384, 40, 3
+    logits = rng.normal(size=(m, e)).astype(np.float32)
+    logits[:, 4] = -50  # an expert nobody picks
+    logits[:, 2] += 3   # a hot one
+    ids, _ = orc.router_topk(logits, top_k)
+    counts_np, relative = orc.expert_histogram(ids, e)
+    rows = m * top_k
+    offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+    cap = orc.tile_capacity(rows, e, bm)
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+    if codec == "e8p_q4":
+        packed = rng.integers(0, 2**32, (e, n, k // 8), dtype=np.uint32)
+        weights = np.stack([orc.q4_integers(x, TABLE) for x in packed])
+        stored = np.stack([orc.q4_pack_k(x, 128) for x in packed])
+    else:
+        weights = rng.integers(-128, 128, (e, n, k), dtype=np.int8)
+        stored = weights
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_q[0, :2] = [-128, 127]
+    a_s = rng.uniform(0.01, 0.03, rows).astype(np.float16)
+    out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
+    kern = gu.kernel("integer_experts", M=m, N=n, K=k, E=e, top_k=top_k, codec=codec, block_m=bm,
+                     block_n=64 if codec == "w8" else 32)
+    counts, tile_count = gu.dev(counts_np), gu.dev(total)
+    args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), Counts=counts, Offsets=gu.dev(offsets_np), Out=out,
+                TileCount=tile_count, TileExpert=gu.dev(te), TileRow=gu.dev(tr), W=gu.dev(stored), WS=gu.dev(ws))
+    kern(**args)
+    want = orc.grouped_project(a_q, a_s[:, None], weights, ws, counts_np, offsets_np)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows] == 55).all()
+    # a zero tile count leaves the output untouched; zeroing one expert's count skips exactly its rows
+    out.fill_(55)
+    tile_count.zero_()
+    kern(**args)
+    assert bool((out == 55).all())
+    tile_count.copy_(gu.dev(total))
+    counts[2] = 0
+    kern(**args)
+    got = gu.host(out)
+    lo, hi = offsets_np[2], offsets_np[2] + counts_np[2]
+    assert (got[lo:hi] == 55).all()
+    np.testing.assert_array_equal(np.delete(got[:rows], np.s_[lo:hi], 0), np.delete(want, np.s_[lo:hi], 0))
+
+
+def test_integer_experts_dynamic_rows_and_refusals():
+    rng = np.random.default_rng(orc.SEED + 5)
+    e, n, k, cap_m, top_k, bm = 6, 128, 256, 64, 2, 16
+    kern = gu.kernel("integer_experts", M=cap_m, N=n, K=k, E=e, top_k=top_k, block_m=bm, dynamic_rows=True)
+    packed = rng.integers(0, 2**32, (e, n, k // 8), dtype=np.uint32)
+    weights = np.stack([orc.q4_integers(x, TABLE) for x in packed])
+    stored = gu.dev(np.stack([orc.q4_pack_k(x, 128) for x in packed]))
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    cap = orc.tile_capacity(cap_m * top_k, e, bm)
+    for m in (64, 5, 1):
+        ids, _ = orc.router_topk(rng.normal(size=(m, e)).astype(np.float32), top_k)
+        counts_np, _ = orc.expert_histogram(ids, e)
+        rows = m * top_k
+        offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+        te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+        a_q = rng.integers(-127, 128, (cap_m * top_k, k), dtype=np.int8)
+        a_s = rng.uniform(0.01, 0.03, cap_m * top_k).astype(np.float16)
+        out = torch.full((cap_m * top_k, n), 55.0, dtype=torch.float16, device=gu.DEV)
+        kern(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), Counts=gu.dev(counts_np), Offsets=gu.dev(offsets_np), Out=out,
+             TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), W=stored, WS=gu.dev(ws), m=m)
+        want = orc.grouped_project(a_q[:rows], a_s[:rows, None], weights, ws, counts_np, offsets_np)
+        np.testing.assert_array_equal(gu.host(out)[:rows], want)
+        assert (gu.host(out)[rows:] == 55).all()
+    for variant in (dict(block_m=256), dict(block_m=12), dict(codec="w8", block_m=8), dict(codec="w8", block_n=32),
+                    dict(codec="q2"), dict(K=192), dict(top_k=7), dict(block_k=256, K=384), dict(stages=3)):
+        base = dict(M=8, N=64, K=256, E=6, top_k=2)
+        base.update(variant)
+        with pytest.raises(Exception):
+            gu.kernel("integer_experts", **base)
