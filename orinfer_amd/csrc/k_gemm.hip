@@ -563,6 +563,23 @@ int make_w8_projection(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// kernels/cuda/model/int8_projection.py:65-107: the reference's DP4A form for up to 8-row tiles.  Same
+// buffers and arithmetic as int8_projection; here the row count picks the kernel, so the tile hints
+// are checked as the reference checks them and dropped.
+int make_w8_small_projection(const Variant& v, orx_function* f) {
+    bool bad = false;
+    const long long m = v.integer("M", 0, &bad);
+    const long long block_m = v.integer("block_m", m < 4 ? m : 4, &bad), block_n = v.integer("block_n", 4, &bad);
+    if (bad || block_m < 1 || block_m > 8 || (block_n != 4 && block_n != 8 && block_n != 16)) {
+        set_error("int8_small_projection: invalid INT8 DP4A tile (block_m 1..8, block_n 4|8|16)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    Variant plain = v;
+    plain.fields.erase("block_m");
+    plain.fields.erase("block_n");
+    return make_w8_projection(plain, f);
+}
+
 // ---- W8 gate/up projections with the SwiGLU boundary (shared expert) ---------------------------
 // kernels/cuda/model/int8_swiglu.py:10-57 with integer_core.py:19-28: both projections are rounded
 // to fp16, then out = fp16((g / (1 + exp(-g))) * u) in fp32.  Built from the catalog's own int8
@@ -860,6 +877,9 @@ const Registration* gemm_registrations(int* count) {
     {"int8_projection", make_w8_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "
      "block_m=0|32|64|128|256",
+     "A,Output,TokenScale,Weight,WeightScale[,m]"},
+    {"int8_small_projection", make_w8_small_projection,
+     "M, N, K, dynamic_rows=false, output_dtype=float16|float32, output_stride=N, block_m=min(M,4) (1..8), block_n=4|8|16",
      "A,Output,TokenScale,Weight,WeightScale[,m]"},
     {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},

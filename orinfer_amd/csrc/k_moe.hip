@@ -462,6 +462,21 @@ int make_router(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// kernels/cuda/model/moe.py:332-409: the reference's one-warp-per-row form; same ids (descending
+// logit, ties to the lower id, +-0 equal) and probabilities renormalised over the selected routes.
+int make_router_warp(const Variant& v, orx_function* f) {
+    bool bad = false;
+    const long long experts = v.integer("E", 0, &bad), top_k = v.integer("top_k", 0, &bad), warps = v.integer("warps", 4, &bad);
+    if (bad || !v.has("E") || !v.has("top_k") || experts % 32 || top_k > 32 || (warps != 1 && warps != 2 && warps != 4) ||
+        v.has("renormalize")) {
+        set_error("router_topk_warp: invalid warp router geometry (E a multiple of 32, top_k <= 32, warps 1|2|4)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    Variant plain = v;
+    plain.fields.erase("warps");
+    return make_router(plain, f);
+}
+
 int histogram_geometry(const orx_function& f, int, Geometry* g) {
     g->grid[0] = (uint32_t)f.E;
     g->block[0] = 256;
@@ -748,6 +763,7 @@ int make_combine(const Variant& v, orx_function* f) {
 const Registration* moe_registrations(int* count) {
     static const Registration rows[] = {
     {"router_topk", make_router, "M, E=512, top_k=10, renormalize=true, dynamic_rows=false", "IDs,Logits,Prob[,m]"},
+    {"router_topk_warp", make_router_warp, "M, E, top_k, dynamic_rows=false, warps=4", "IDs,Logits,Prob[,m]"},
     {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
     {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},

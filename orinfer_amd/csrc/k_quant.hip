@@ -204,6 +204,37 @@ __global__ __launch_bounds__(256) void rotate_a8_kernel(const __half* __restrict
     quantise_row(rotated, amax, q, s, row, k);
 }
 
+// The rotation alone (kernels/cuda/model/integer_vq.py:447-486): Y = fp16(rotated * 128^-1/2), the
+// values rotate_a8_kernel quantises.  Same lane layout; nothing is kept in LDS.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void rotate_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                     __half* __restrict__ y, int k) {
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int half_wave = lane >> 5, l32 = lane & 31;
+    const int blocks = k / 128;
+    const int64_t in_base = (int64_t)row * (SWIGLU ? 2 * k : k);
+    for (int pair = wave; 2 * pair < blocks; pair += 4) {  // wave-uniform trip count
+        const int block = 2 * pair + half_wave;
+        const bool live = block < blocks;
+        const int first = (live ? block : 0) * 128 + 4 * l32;
+        const uint2 raw = *reinterpret_cast<const uint2*>(x + in_base + first);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+        uint2 raw_up = make_uint2(0u, 0u);
+        if (SWIGLU) raw_up = *reinterpret_cast<const uint2*>(x + in_base + k + first);
+        const __half* up = reinterpret_cast<const __half*>(&raw_up);
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float value = SWIGLU ? swiglu_value(h[j], up[j]) : __half2float(h[j]);
+            v[j] = live ? value * (float)(int8_t)(sign_word >> (8 * j)) : 0.f;
+        }
+        __half out[4];
+        rotate_block(v, l32, out);
+        if (live) *reinterpret_cast<uint2*>(y + (int64_t)row * k + first) = *reinterpret_cast<const uint2*>(out);
+    }
+}
+
 __device__ __forceinline__ float block_sum(float v, float* scratch) {
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
@@ -435,6 +466,41 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// slots used: K, flags (bit1 swiglu)
+int rotate_geometry(const orx_function&, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+// Signs, X, Y (integer_vq.py:454-458 in generated-ABI order)
+int rotate_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    const int8_t* signs = pointer_arg<const int8_t>(args, 0);
+    const __half* x = pointer_arg<const __half>(args, 1);
+    __half* y = pointer_arg<__half>(args, 2);
+    if (f.flags & 2)
+        hipLaunchKernelGGL((rotate_kernel<true>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
+    else
+        hipLaunchKernelGGL((rotate_kernel<false>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
+    return hip_check(hipGetLastError(), "launch rotate_activation");
+}
+int make_rotate(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("K", 0, &bad);
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    const bool swiglu = v.boolean("swiglu", false, &bad);
+    if (bad || f->M <= 0 || f->K <= 0 || f->K % 128) {
+        set_error("rotate_activation: invalid block-128 activation rotation");  // integer_vq.py:449-450
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = swiglu ? 2 : 0;
+    f->args = {{"Signs", ArgPointer, 4}, {"X", ArgPointer, 8}, {"Y", ArgPointer, 8}};
+    f->device_function = reinterpret_cast<const void*>(&rotate_kernel<false>);
+    f->geometry = rotate_geometry;
+    f->launch = rotate_launch;
+    return ORX_OK;
+}
+
 // slots used: K, flags (bit0: weights stored zero-centred), capacity
 int residual_rotate_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
@@ -557,6 +623,7 @@ const Registration* quant_registrations(int* count) {
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
     {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
+    {"rotate_activation", make_rotate, "M, K, swiglu=false", "Signs,X,Y"},
     {"residual_norm_rotate_a8", make_residual_rotate, "M, K=5120, dynamic_rows=false, zero_centered=true",
      "Q,R,RO,S,Signs,W,X,Y[,m]"},
     {"e8p_q4_embedding", make_q4_embedding, "M, vocab, hidden", "Book,IDs,Output,Scale,Signs,Weight,m"},

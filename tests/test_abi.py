@@ -73,6 +73,10 @@ ABI = {
         ["A", "AS", "Book", "Counts", "Offsets", "Out", "TileCount", "TileExpert", "TileRow", "W", "WS", "m"],
     ("integer_experts", (("M", 64), ("N", 1024), ("K", 2048), ("E", 128), ("top_k", 8), ("codec", "w8"))):
         ["A", "AS", "Book", "Counts", "Offsets", "Out", "TileCount", "TileExpert", "TileRow", "W", "WS"],
+    ("router_topk_warp", (("M", 64), ("E", 128), ("top_k", 8), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
+    ("rotate_activation", (("M", 8), ("K", 5120), ("swiglu", True))): ["Signs", "X", "Y"],
+    ("int8_small_projection", (("M", 4), ("N", 4096), ("K", 4096), ("dynamic_rows", True))):
+        ["A", "Output", "TokenScale", "Weight", "WeightScale", "m"],
     ("router_topk", (("M", 64), ("dynamic_rows", True))): ["IDs", "Logits", "Prob", "m"],
     ("expert_histogram", (("M", 64),)): ["Counts", "IDs", "RelativeSlot"],
     ("expert_offsets", ()): ["Counts", "RowOffsets", "TileCount", "TileOffsets"],

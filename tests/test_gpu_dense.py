@@ -262,6 +262,56 @@ def test_residual_norm_rotate_a8_refuses_incomplete_tiles():
             gu.kernel("residual_norm_rotate_a8", M=4, K=k)
 
 
+@pytest.mark.parametrize("m,k,swiglu", [(1, 128, False), (3, 2560, False), (2, 5120, True), (4, 384, True)])
+def test_rotate_activation_gives_the_values_the_fused_kernel_quantises(m, k, swiglu):
+    # kernels/cuda/model/integer_vq.py:447-486
+    rng = np.random.default_rng(orc.SEED + m + k)
+    x = rng.normal(size=(m, 2 * k if swiglu else k)).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    y = torch.full((m + 1, k), 7.0, dtype=torch.float16, device=gu.DEV)
+    variant = dict(M=m, K=k, swiglu=True) if swiglu else dict(M=m, K=k)
+    gu.kernel("rotate_activation", **variant)(Signs=gu.dev(signs), X=gu.dev(x), Y=y)
+    values = x
+    if swiglu:  # the device's own fp16 SwiGLU values (the exponential may differ from libm in the last place)
+        mid = torch.empty((m, k), dtype=torch.float16, device=gu.DEV)
+        gu.kernel("swiglu", I=k)(X=gu.dev(x), Y=mid, rows=m)
+        values = gu.host(mid)
+    want = orc.rotate(values.astype(np.float32), signs).astype(np.float16)
+    np.testing.assert_array_equal(gu.host(y)[:m], want)
+    assert (gu.host(y)[m] == 7).all()
+    # A8 of these values is what rotate_activation_a8 writes
+    q = torch.zeros((m, k), dtype=torch.int8, device=gu.DEV)
+    s = torch.zeros((m,), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("rotate_activation_a8", **variant)(Q=q, S=s, Signs=gu.dev(signs), X=gu.dev(x))
+    want_q, want_s = orc.a8(gu.host(y)[:m])
+    np.testing.assert_array_equal(gu.host(q), want_q)
+    np.testing.assert_array_equal(gu.host(s), want_s[:, 0])
+    with pytest.raises(Exception):
+        gu.kernel("rotate_activation", M=2, K=192)
+
+
+@pytest.mark.parametrize("m,block_m", [(1, None), (3, None), (8, 8), (6, 2)])
+def test_int8_small_projection_symbol(m, block_m):
+    # kernels/cuda/model/int8_projection.py:65-107: same buffers and arithmetic as int8_projection
+    rng = np.random.default_rng(orc.SEED + m)
+    n, k = 136, 384
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    ws = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    ts = rng.uniform(0.01, 0.03, m).astype(np.float16)
+    variant = dict(M=m, N=n, K=k, block_n=8, output_stride=n + 8)
+    if block_m:
+        variant["block_m"] = block_m
+    out = torch.full((m, n + 8), 9.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("int8_small_projection", **variant)(A=gu.dev(a), Output=out, TokenScale=gu.dev(ts), Weight=gu.dev(w),
+                                                  WeightScale=gu.dev(ws))
+    np.testing.assert_array_equal(gu.host(out)[:, :n], orc.project(a, ts, w, ws))
+    assert (gu.host(out)[:, n:] == 9).all()
+    for bad in (dict(block_m=9), dict(block_n=32), dict(block_m=0)):
+        with pytest.raises(Exception):
+            gu.kernel("int8_small_projection", M=4, N=n, K=k, **bad)
+
+
 def test_q4_embedding_gather_matches_oracle():
     rng = np.random.default_rng(orc.SEED + 40)
     vocab, hidden, cap = 50, 640, 16

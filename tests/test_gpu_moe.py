@@ -587,3 +587,21 @@ def test_integer_experts_dynamic_rows_and_refusals():
         base.update(variant)
         with pytest.raises(Exception):
             gu.kernel("integer_experts", **base)
+
+
+@pytest.mark.parametrize("m,e,k,warps", [(5, 128, 8, 4), (64, 512, 10, 2), (1, 32, 32, 1)])
+def test_router_topk_warp_symbol(m, e, k, warps):
+    # kernels/cuda/model/moe.py:332-409: same ranking rule, probabilities over the selected routes
+    rng = np.random.default_rng(orc.SEED + e + k)
+    logits = (rng.normal(size=(m, e)) * 5).astype(np.float32)
+    logits[0, :4] = [0.0, -0.0, 0.0, 3.0]
+    ids = torch.full((m, k), -1, **I32)
+    prob = torch.full((m, k), float("nan"), dtype=torch.float32, device=gu.DEV)
+    gu.kernel("router_topk_warp", M=m, E=e, top_k=k, warps=warps)(IDs=ids, Logits=gu.dev(logits), Prob=prob)
+    want_ids, want_prob = orc.router_topk(logits, k, True)
+    np.testing.assert_array_equal(gu.host(ids), want_ids)
+    np.testing.assert_allclose(gu.host(prob), want_prob, atol=2e-6, rtol=2e-5)
+    np.testing.assert_allclose(gu.host(prob).sum(axis=1), 1.0, rtol=1e-6)
+    for variant in (dict(E=100, top_k=4), dict(E=128, top_k=33), dict(E=128, top_k=4, warps=3)):
+        with pytest.raises(Exception):
+            gu.kernel("router_topk_warp", M=4, **variant)
