@@ -242,6 +242,26 @@ def main():
                                            "code_bytes_touched": code_bytes,
                                            "GBps_codes": round(code_bytes / t / 1e9, 1)}
         del layer
+        # one token of the same layer: its 8 routes index the banks directly (no sorting, no tiles)
+        raw_book = dev(codebook.raw_book())
+        e3, h3, i3, k3 = c3["experts"], c3["hidden"], c3["intermediate"], c3["top_k"]
+        routes = torch.tensor([[3, 77, 12, 100, 64, 31, 127, 2]], dtype=torch.int32, device="cuda")
+        single = {}
+        for name, codes, scales, n, k, shared in (("gate_up", c3["gate_up"], c3["gate_up_scales"], 2 * i3, h3, True),
+                                                  ("down", c3["down"], c3["down_scales"], h3, i3, False)):
+            bank = dev(codes).view(e3, n, k // 128, 16).permute(0, 2, 1, 3).contiguous()
+            rows = 1 if shared else k3
+            a = torch.randint(-127, 128, (rows, k), dtype=torch.int8, device="cuda")
+            a_scale = torch.full((rows,), 0.01, dtype=torch.float16, device="cuda")
+            out = torch.empty((k3, n), dtype=torch.float16, device="cuda")
+            kern = Kernel("integer_e8p_gemv", E=e3, routes=k3, N=n, K=k, shared_input=shared)
+            ws_dev = dev(scales)
+            t = timed_graph(lambda i, st: kern(stream=st, A=a, AS=a_scale, Book=raw_book, C=out, IDs=routes, P=bank,
+                                               WS=ws_dev), 20)
+            moved = k3 * n * k // 4
+            single[name] = {"us": round(t * 1e6, 2), "GBps_codes": round(moved / t / 1e9, 1)}
+            del bank
+        extra["config3_single_token_routes"] = single
         torch.cuda.empty_cache()
         # config 4 layer linears
         c4 = workloads.config4()

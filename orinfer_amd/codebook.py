@@ -48,6 +48,13 @@ def book():
     return selector_table(basis())
 
 
+def raw_book(table=None):
+    """The 256 x 8 int8 table as (256, 2) u32 words: the `Book` of the raw-table kernels
+    (`integer_e8p_gemv`; python/orinfer_build/quantization/vq.py:203)."""
+    table = basis() if table is None else np.asarray(table, np.int8)
+    return np.ascontiguousarray(table).view("<u4").reshape(256, 2)
+
+
 def q4_to_k_major(packed, packed_k=128):
     """(N, K/8) u32 -> (K/packed_k, N, packed_k/8), tag e8p-q4-k128-u32."""
     n, vectors = packed.shape

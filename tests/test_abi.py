@@ -183,6 +183,8 @@ def test_package_codebook_matches_oracle(golden_basis):
     assert np.array_equal(codebook.q4_to_k_major(q4), ref.q4_pack_k(q4, 128))
     q2 = rng.integers(0, 2**16, size=(3, 32, 32), dtype=np.uint16)          # E=3, N=32, K=256
     assert np.array_equal(codebook.q2_to_k_major(q2), np.stack([ref.q2_pack_k128(e) for e in q2]))
+    assert np.array_equal(codebook.raw_book(), ref.raw_table_words(golden_basis))
+    assert np.array_equal(codebook.raw_book(golden_basis[::-1]), ref.raw_table_words(golden_basis[::-1]))
 
 
 def test_workload_sizes_and_algorithmic_bytes():
