@@ -55,8 +55,14 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return r;
 }
 
-__device__ __forceinline__ int8_t quantise(float value, float scale) {
-    const float r = rintf(__fdiv_rn(value, scale));
+// rint(value / scale), clamped: the product with the reciprocal decides, except within 2^-14 of a
+// tie, where the correctly rounded quotient does.  The product is within 4 units in the last place
+// of the quotient (|quotient| < 128.5, so 2^-15 at most), so the two round alike everywhere else;
+// the reference's kernel takes the same shortcut (kernels/cuda/model/rotation_a8.py:153-164).
+__device__ __forceinline__ int8_t quantise(float value, float scale, float inverse) {
+    const float guess = value * inverse;
+    float r = rintf(guess);
+    if (fabsf(fabsf(guess - r) - 0.5f) < 6.103515625e-05f) r = rintf(__fdiv_rn(value, scale));
     return (int8_t)fmaxf(-127.f, fminf(127.f, r));
 }
 
@@ -95,6 +101,7 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
     const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
     if (threadIdx.x == 0) s[(int64_t)row * groups + g] = stored;
     const float scale = __half2float(stored);
+    const float inverse = __frcp_rn(scale);
     if (vector) {
         const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
         uint2* dst = reinterpret_cast<uint2*>(q + out_base + first);
@@ -104,14 +111,14 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
             uint32_t lo = 0, hi = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                lo |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
-                hi |= ((uint32_t)(uint8_t)quantise(__half2float(h[j + 4]), scale)) << (8 * j);
+                lo |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale, inverse)) << (8 * j);
+                hi |= ((uint32_t)(uint8_t)quantise(__half2float(h[j + 4]), scale, inverse)) << (8 * j);
             }
             dst[i] = make_uint2(lo, hi);
         }
     } else {
         for (int i = threadIdx.x; i < width; i += blockDim.x)
-            q[out_base + first + i] = quantise(load_value<FUSED, MASKED>(x, mask, in_base, k, first + i), scale);
+            q[out_base + first + i] = quantise(load_value<FUSED, MASKED>(x, mask, in_base, k, first + i), scale, inverse);
     }
 }
 
@@ -124,14 +131,29 @@ __device__ __forceinline__ float rotate_block(float (&v)[4], int l32, __half (&o
         const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
         v[0] = a + c, v[2] = a - c, v[1] = b + d, v[3] = b - d;
     }
-    // distance 4 .. 64: lanes at distance 1 .. 16; the upper element of a pair keeps left - right
+    // distance 4 .. 64: lanes at distance 1 .. 16.  The upper lane of a pair keeps left - right, the
+    // lower one left + right: both are partner + (own with the sign flipped in the upper lane), one
+    // fp32 add.  The partner comes through the data-parallel lane controls where they can express
+    // the exchange (quad permutes, row rotate by 8, two masked row shifts by 4), else a shuffle.
 #pragma unroll
     for (int bit = 0; bit < 5; ++bit) {
-        const bool upper = (l32 >> bit) & 1;
+        const uint32_t flip = ((uint32_t)(l32 >> bit) & 1u) << 31;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float other = __shfl_xor(v[j], 1 << bit, 64);
-            v[j] = upper ? other - v[j] : other + v[j];
+            const int own = __float_as_int(v[j]);
+            int partner;
+            if (bit == 0)
+                partner = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+            else if (bit == 1)
+                partner = __builtin_amdgcn_update_dpp(0, own, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+            else if (bit == 2) {
+                partner = __builtin_amdgcn_update_dpp(own, own, 0x104, 0xF, 0x5, false);      // row_shl:4 into banks 0, 2
+                partner = __builtin_amdgcn_update_dpp(partner, own, 0x114, 0xF, 0xA, false);  // row_shr:4 into banks 1, 3
+            } else if (bit == 3)
+                partner = __builtin_amdgcn_update_dpp(0, own, 0x128, 0xF, 0xF, true);  // row_ror:8
+            else
+                partner = __float_as_int(__shfl_xor(v[j], 16, 64));
+            v[j] = __int_as_float(partner) + __int_as_float(own ^ (int)flip);
         }
     }
     float amax = 0.f;
@@ -154,51 +176,69 @@ __device__ __forceinline__ void quantise_row(const __half* rotated, float amax, 
     const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
     if (tid == 0) s[row] = stored;
     const float scale = __half2float(stored);
-    for (int i = tid; i < k / 4; i += 256) {
+    const float inverse = __frcp_rn(scale);
+    for (int i = tid; i < k / 4; i += blockDim.x) {
         const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
         const __half* h = reinterpret_cast<const __half*>(&raw);
         uint32_t packed = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale)) << (8 * j);
+        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale, inverse)) << (8 * j);
         *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = packed;
     }
 }
 
-// One workgroup per row, 4 waves; a wave takes two blocks of 128 channels per step (one per half
+constexpr int kRotateBatch = 5;
+constexpr int kRotateWideRows = 256;  // up to one row per CU
+
+// One workgroup per row, 4 waves (16 when rows are few: the latency of one row is what counts then);
+// a wave takes two blocks of 128 channels per step (one per half
 // wave), a lane holds 4 consecutive channels: stages 1 and 2 are local, stages 4..64 are lane
 // exchanges at distance 1..16.  The rotated fp16 row is kept in LDS for the second pass.
-template <bool SWIGLU>
-__global__ __launch_bounds__(256) void rotate_a8_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
-                                                        int8_t* __restrict__ q, __half* __restrict__ s, int k) {
+template <bool SWIGLU, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void rotate_a8_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                            int8_t* __restrict__ q, __half* __restrict__ s, int k) {
     extern __shared__ __align__(16) __half rotated[];  // k halves
-    __shared__ float scratch[4];
+    __shared__ float scratch[THREADS / 64];
+    constexpr int kWaves = THREADS / 64;
+    constexpr int kBatch = THREADS == 256 ? kRotateBatch : 2;  // steps whose loads leave together
     const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int half_wave = lane >> 5, l32 = lane & 31;
     const int blocks = k / 128;
     const int64_t in_base = (int64_t)row * (SWIGLU ? 2 * k : k);
     float amax = 0.f;
-    for (int pair = wave; 2 * pair < blocks; pair += 4) {  // wave-uniform trip count
-        const int block = 2 * pair + half_wave;
-        const bool live = block < blocks;
-        const int first = (live ? block : 0) * 128 + 4 * l32;
-        float v[4];
-        {
-            const uint2 raw = *reinterpret_cast<const uint2*>(x + in_base + first);
-            const __half* h = reinterpret_cast<const __half*>(&raw);
-            const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
-            uint2 raw_up = make_uint2(0u, 0u);
-            if (SWIGLU) raw_up = *reinterpret_cast<const uint2*>(x + in_base + k + first);
-            const __half* up = reinterpret_cast<const __half*>(&raw_up);
+    // kRotateBatch steps at a time, all their loads first: a row is only a few KiB, and one step's
+    // load-to-use latency per step would leave the memory system idle
+    for (int base = wave; 2 * base < blocks; base += kWaves * kBatch) {  // wave-uniform trip counts
+        uint2 raw[kBatch], raw_up[kBatch];
+        uint32_t sign_word[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const int block = 2 * (base + kWaves * u) + half_wave;
+            const int first = (block < blocks ? block : 0) * 128 + 4 * l32;  // clamped, so unconditional
+            raw[u] = *reinterpret_cast<const uint2*>(x + in_base + first);
+            sign_word[u] = *reinterpret_cast<const uint32_t*>(signs + first);
+            raw_up[u] = make_uint2(0u, 0u);
+            if (SWIGLU) raw_up[u] = *reinterpret_cast<const uint2*>(x + in_base + k + first);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            if (2 * (base + kWaves * u) >= blocks) break;
+            const int block = 2 * (base + kWaves * u) + half_wave;
+            const bool live = block < blocks;
+            const int first = (live ? block : 0) * 128 + 4 * l32;
+            const __half* h = reinterpret_cast<const __half*>(&raw[u]);
+            const __half* up = reinterpret_cast<const __half*>(&raw_up[u]);
+            float v[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float value = SWIGLU ? swiglu_value(h[j], up[j]) : __half2float(h[j]);
-                const float sign = (float)(int8_t)(sign_word >> (8 * j));
+                const float sign = (float)(int8_t)(sign_word[u] >> (8 * j));
                 v[j] = live ? value * sign : 0.f;
             }
+            __half out[4];
+            amax = fmaxf(amax, rotate_block(v, l32, out));
+            if (live) *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
         }
-        __half out[4];
-        amax = fmaxf(amax, rotate_block(v, l32, out));
-        if (live) *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
     }
     amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
     quantise_row(rotated, amax, q, s, row, k);
@@ -425,7 +465,8 @@ int make_a8(const Variant& v, orx_function* f) {
 // slots used: K, flags (bit1 swiglu), capacity
 int rotate_a8_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
-    g->block[0] = 256;
+    // few rows (decode): 16 waves share one row, so that a row is one or two steps per wave
+    g->block[0] = rows <= kRotateWideRows && f.K >= 2048 ? 1024 : 256;
     g->shared = (uint32_t)f.K * 2;
     return ORX_OK;
 }
@@ -437,10 +478,17 @@ int rotate_a8_launch(const orx_function& f, int rows, const Geometry& g, hipStre
     __half* s = pointer_arg<__half>(args, 1);
     const int8_t* signs = pointer_arg<const int8_t>(args, 2);
     const __half* x = pointer_arg<const __half>(args, 3);
-    if (f.flags & 2)
-        hipLaunchKernelGGL((rotate_a8_kernel<true>), dim3(g.grid[0]), dim3(256), g.shared, stream, x, signs, q, s, f.K);
-    else
-        hipLaunchKernelGGL((rotate_a8_kernel<false>), dim3(g.grid[0]), dim3(256), g.shared, stream, x, signs, q, s, f.K);
+    const dim3 grid(g.grid[0]), block(g.block[0]);
+    if (g.block[0] == 1024) {
+        if (f.flags & 2)
+            hipLaunchKernelGGL((rotate_a8_kernel<true, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+        else
+            hipLaunchKernelGGL((rotate_a8_kernel<false, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+    } else if (f.flags & 2) {
+        hipLaunchKernelGGL((rotate_a8_kernel<true>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+    } else {
+        hipLaunchKernelGGL((rotate_a8_kernel<false>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+    }
     return hip_check(hipGetLastError(), "launch rotate_activation_a8");
 }
 
@@ -460,7 +508,8 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     // 8-byte loads of X, 4-byte loads of Signs and stores of Q
     f->args = {{"Q", ArgPointer, 4}, {"S", ArgPointer, 2}, {"Signs", ArgPointer, 4}, {"X", ArgPointer, 8}};
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
-    f->device_function = reinterpret_cast<const void*>(&rotate_a8_kernel<false>);
+    // kernels with 256 and 1024 threads serve this symbol: report the device-wide limits
+    f->device_function = nullptr;
     f->geometry = rotate_a8_geometry;
     f->launch = rotate_a8_launch;
     return ORX_OK;
