@@ -66,12 +66,32 @@ __device__ __forceinline__ int8_t quantise(float value, float scale, float inver
     return (int8_t)fmaxf(-127.f, fminf(127.f, r));
 }
 
+// Four codes packed into one word; one test (and, rarely, four exact quotients) for the four.
+__device__ __forceinline__ uint32_t quantise4(const float (&value)[4], float scale, float inverse) {
+    float r[4];
+    float nearest = 1.0f;  // smallest distance of a product from a tie
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float guess = value[j] * inverse;
+        r[j] = rintf(guess);
+        nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
+    }
+    if (nearest < 6.103515625e-05f) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
+    }
+    uint32_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * j);
+    return packed;
+}
+
 // grid (rows, groups), 256 threads.
-template <bool FUSED, bool MASKED>
-__global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
-                                                 int8_t* __restrict__ q, __half* __restrict__ s, int k, int group,
-                                                 int groups) {
-    __shared__ float scratch[4];
+template <bool FUSED, bool MASKED, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
+                                                     int8_t* __restrict__ q, __half* __restrict__ s, int k, int group,
+                                                     int groups) {
+    __shared__ float scratch[THREADS / 64];
     const int row = blockIdx.x, g = blockIdx.y;
     const int first = g * group;
     const int width = min(group, k - first);
@@ -81,10 +101,16 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
     const bool vector = !FUSED && !MASKED && (k % 8 == 0) && (group % 8 == 0) &&
                         ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
     float amax = 0.f;
+    // a group of at most one 16-byte piece per thread stays in registers between the two passes
+    // (only in the 16-wave form: carrying the piece through the loops costs the 4-wave form its
+    // overlap of loads, 28 -> 48 us at 8192 x 5120)
+    const bool held = THREADS == 1024 && vector && width / 8 <= THREADS;
+    uint4 kept = make_uint4(0u, 0u, 0u, 0u);
     if (vector) {
         const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
         for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
             const uint4 raw = src[i];
+            if (THREADS == 1024) kept = raw;
             const __half2* h = reinterpret_cast<const __half2*>(&raw);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -106,15 +132,11 @@ __global__ __launch_bounds__(256) void a8_kernel(const __half* __restrict__ x, c
         const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
         uint2* dst = reinterpret_cast<uint2*>(q + out_base + first);
         for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
-            const uint4 raw = src[i];
+            const uint4 raw = held ? kept : src[i];
             const __half* h = reinterpret_cast<const __half*>(&raw);
-            uint32_t lo = 0, hi = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                lo |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale, inverse)) << (8 * j);
-                hi |= ((uint32_t)(uint8_t)quantise(__half2float(h[j + 4]), scale, inverse)) << (8 * j);
-            }
-            dst[i] = make_uint2(lo, hi);
+            const float low[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+            const float high[4] = {__half2float(h[4]), __half2float(h[5]), __half2float(h[6]), __half2float(h[7])};
+            dst[i] = make_uint2(quantise4(low, scale, inverse), quantise4(high, scale, inverse));
         }
     } else {
         for (int i = threadIdx.x; i < width; i += blockDim.x)
@@ -180,10 +202,8 @@ __device__ __forceinline__ void quantise_row(const __half* rotated, float amax, 
     for (int i = tid; i < k / 4; i += blockDim.x) {
         const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
         const __half* h = reinterpret_cast<const __half*>(&raw);
-        uint32_t packed = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)quantise(__half2float(h[j]), scale, inverse)) << (8 * j);
-        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = packed;
+        const float values[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = quantise4(values, scale, inverse);
     }
 }
 
@@ -412,10 +432,13 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ 
 
 // ---- host side -----------------------------------------------------------------------------
 // slots used: K, group, flags (bit0 masked, bit1 fused), capacity
+// few rows of long groups (decode): 16 waves per group, one 16-byte piece per thread
+bool a8_wide(const orx_function& f, int rows) { return f.flags == 0 && rows <= 256 && f.group >= 2048; }
+
 int a8_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
     g->grid[1] = ceil_div((uint32_t)f.K, (uint32_t)f.group);
-    g->block[0] = 256;
+    g->block[0] = a8_wide(f, rows) ? 1024 : 256;
     return ORX_OK;
 }
 
@@ -428,7 +451,9 @@ int a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     const dim3 grid(g.grid[0], g.grid[1]), block(256);
     const int groups = (int)g.grid[1];
     const bool masked = f.flags & 1, fused = f.flags & 2;
-    if (fused && masked)
+    if (g.block[0] == 1024)
+        hipLaunchKernelGGL((a8_kernel<false, false, 1024>), grid, dim3(1024), 0, stream, x, mask, q, s, f.K, f.group, groups);
+    else if (fused && masked)
         hipLaunchKernelGGL((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused)
         hipLaunchKernelGGL((a8_kernel<true, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
@@ -456,7 +481,7 @@ int make_a8(const Variant& v, orx_function* f) {
     // Mask may be null unless masked (the reference ignores it then, op30:75-76)
     f->args = {{"Mask", ArgPointer, masked ? 1u : 0x80000001u}, {"Q", ArgPointer, 1}, {"S", ArgPointer, 2},
                {"X", ArgPointer, 2}, {"rows", ArgI32, 4}};
-    f->device_function = reinterpret_cast<const void*>(&a8_kernel<false, false>);
+    f->device_function = nullptr;  // kernels with 256 and 1024 threads serve this symbol
     f->geometry = a8_geometry;
     f->launch = a8_launch;
     return ORX_OK;
