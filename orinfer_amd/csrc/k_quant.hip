@@ -207,6 +207,58 @@ __device__ __forceinline__ void quantise_row(const __half* rotated, float amax, 
     }
 }
 
+// Short groups (at most 512 values): one wave per (row, group), four per workgroup, a lane holds one
+// 16-byte piece; the maximum is a wave reduction, so there is no barrier and no second read.
+template <bool FUSED>
+__global__ __launch_bounds__(256) void a8_wave_kernel(const __half* __restrict__ x, int8_t* __restrict__ q,
+                                                      __half* __restrict__ s, int k, int group, int groups, int rows) {
+    const int lane = threadIdx.x & 63;
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);  // wave-uniform
+    if (unit >= rows * groups) return;
+    const int row = unit / groups, g = unit % groups;
+    const int first = g * group;
+    const int width = min(group, k - first);
+    const int64_t in_base = (int64_t)row * (FUSED ? 2 * k : k);
+    const int64_t out_base = (int64_t)row * k;
+    const bool vector = (k % 8 == 0) && (group % 8 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
+                        ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
+    float value[8];
+    float amax = 0.f;
+    if (vector) {
+        const bool live = lane < width / 8;
+        const int piece = live ? lane : 0;
+        const uint4 raw = *reinterpret_cast<const uint4*>(x + in_base + first + 8 * piece);
+        uint4 raw_up = make_uint4(0u, 0u, 0u, 0u);
+        if (FUSED) raw_up = *reinterpret_cast<const uint4*>(x + in_base + k + first + 8 * piece);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const __half* up = reinterpret_cast<const __half*>(&raw_up);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            value[j] = FUSED ? swiglu_value(h[j], up[j]) : __half2float(h[j]);
+            if (live) amax = fmaxf(amax, fabsf(value[j]));
+        }
+    } else {
+        for (int i = lane; i < width; i += 64) amax = fmaxf(amax, fabsf(load_value<FUSED, false>(x, nullptr, in_base, k, first + i)));
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+    const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
+    const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
+    if (lane == 0) s[(int64_t)row * groups + g] = stored;
+    const float scale = __half2float(stored);
+    const float inverse = __frcp_rn(scale);
+    if (vector) {
+        if (lane < width / 8) {
+            const float low[4] = {value[0], value[1], value[2], value[3]}, high[4] = {value[4], value[5], value[6], value[7]};
+            *reinterpret_cast<uint2*>(q + out_base + first + 8 * lane) =
+                make_uint2(quantise4(low, scale, inverse), quantise4(high, scale, inverse));
+        }
+    } else {
+        for (int i = lane; i < width; i += 64)
+            q[out_base + first + i] = quantise(load_value<FUSED, false>(x, nullptr, in_base, k, first + i), scale, inverse);
+    }
+}
+
 constexpr int kRotateBatch = 5;
 constexpr int kRotateWideRows = 256;  // up to one row per CU
 
@@ -433,25 +485,37 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ 
 // ---- host side -----------------------------------------------------------------------------
 // slots used: K, group, flags (bit0 masked, bit1 fused), capacity
 // few rows of long groups (decode): 16 waves per group, one 16-byte piece per thread
-bool a8_wide(const orx_function& f, int rows) { return f.flags == 0 && rows <= 256 && f.group >= 2048; }
+bool a8_wide(const orx_function& f, int rows) { return f.flags == 0 && rows <= 256 && f.group >= 4096; }
+// short groups, no mask: one wave per group
+bool a8_per_wave(const orx_function& f) { return !(f.flags & 1) && f.group <= 512; }
 
 int a8_geometry(const orx_function& f, int rows, Geometry* g) {
+    const uint32_t groups = ceil_div((uint32_t)f.K, (uint32_t)f.group);
+    if (a8_per_wave(f)) {
+        g->grid[0] = ceil_div((uint32_t)rows * groups, 4u);
+        g->block[0] = 256;
+        return ORX_OK;
+    }
     g->grid[0] = (uint32_t)rows;
-    g->grid[1] = ceil_div((uint32_t)f.K, (uint32_t)f.group);
+    g->grid[1] = groups;
     g->block[0] = a8_wide(f, rows) ? 1024 : 256;
     return ORX_OK;
 }
 
 int a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
-    (void)rows;
     const uint8_t* mask = pointer_arg<const uint8_t>(args, 0);
     int8_t* q = pointer_arg<int8_t>(args, 1);
     __half* s = pointer_arg<__half>(args, 2);
     const __half* x = pointer_arg<const __half>(args, 3);
     const dim3 grid(g.grid[0], g.grid[1]), block(256);
-    const int groups = (int)g.grid[1];
+    const int groups = (int)ceil_div((uint32_t)f.K, (uint32_t)f.group);
     const bool masked = f.flags & 1, fused = f.flags & 2;
-    if (g.block[0] == 1024)
+    if (a8_per_wave(f)) {
+        if (fused)
+            hipLaunchKernelGGL((a8_wave_kernel<true>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
+        else
+            hipLaunchKernelGGL((a8_wave_kernel<false>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
+    } else if (g.block[0] == 1024)
         hipLaunchKernelGGL((a8_kernel<false, false, 1024>), grid, dim3(1024), 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused && masked)
         hipLaunchKernelGGL((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
