@@ -26,6 +26,7 @@ int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
 int gemv_configure(orx_function* f, int codec, int passes_override);
 int gemv_prepare_device();
 bool gemv_serves_k_major(const orx_function& f, int rows);
+bool gemv_serves_fp16_input(const orx_function& f);
 // from k_stream.hip
 void stream_geometry(int n, Geometry* g);
 int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
@@ -545,6 +546,21 @@ int make_q4_projection(const Variant& v, orx_function* f) {
             f->workspace_bytes = bytes;
         else
             f->workspace = nullptr, (void)hipGetLastError();
+    }
+    // input_dtype=float16: A is the fp16 row and AS is written, not read (the kernel quantises the row)
+    const std::string input = v.string("input_dtype", "int8", &bad);
+    if (bad || (input != "int8" && input != "float16")) {
+        set_error("e8p_q4_projection: input_dtype must be int8 or float16");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (input == "float16") {
+        if (f->capacity != 1 || (f->algorithm != kAuto && f->algorithm != kGemv) || !gemv_serves_fp16_input(*f)) {
+            set_error("e8p_q4_projection: input_dtype=float16 is served for one row by the replicated-table GEMV "
+                      "(M = 1, algorithm auto or gemv, K up to 8192 with a layout that kernel reads)");
+            return ORX_ERR_BAD_VARIANT;
+        }
+        f->input_f16 = true;
+        f->algorithm = kGemv;
     }
     f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4},
                {"Out", ArgPointer, 2}, {"S", ArgPointer, 2},  {"W", ArgPointer, 16}};

@@ -314,7 +314,11 @@ constexpr uint32_t kSelNib1 = 0x0C0C0500u, kSelNib3 = 0x0C0C0700u, kSelMsk0 = 0x
 // registers for the whole kernel and the main loop reads LDS for table lookups only.
 // LAYOUT: lanes per row, + 64 for K-major codes.
 constexpr int kKMajorLayout = 64;
-template <int CODEC, int MR, int D, int LAYOUT, bool HOLD>
+// X16 (one activation row, K up to 8192): `a` holds the row as fp16 and the kernel quantises it
+// itself during set-up, by the rule of the activation quantiser (row maximum over 127, fp16 scale,
+// round to nearest even); every workgroup does so for itself, the first one also writes the scale
+// to `as`.  That saves the separate launch in front of a single-row projection.
+template <int CODEC, int MR, int D, int LAYOUT, bool HOLD, bool X16 = false>
 __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
@@ -371,16 +375,21 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     uint32_t* hi = planes;
     uint32_t* lo = planes + MR * groups;
     uint32_t* ov = planes + 2 * MR * groups;
+    static_assert(!X16 || MR == 1, "the fp16 input form serves one activation row");
     unsigned short as_bits[MR];
 #pragma unroll
-    for (int r = 0; r < MR; ++r) as_bits[r] = reinterpret_cast<const unsigned short*>(as)[min(r, m - 1)];
+    for (int r = 0; r < MR; ++r) as_bits[r] = X16 ? (unsigned short)0 : reinterpret_cast<const unsigned short*>(as)[min(r, m - 1)];
     const int entry_in_wave = lane >> 2, quarter = lane & 3;
     const int entry = wave * 16 + entry_in_wave;  // 16 waves x 16 entries
     uint32_t selector = book[entry];
     uint2 raw[MR];
+    uint4 raw_x16 = make_uint4(0u, 0u, 0u, 0u);
+    if (X16)
+        raw_x16 = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(a) + 8 * min(tid, groups - 1));
+    else
 #pragma unroll
-    for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
-        raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
+        for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
+            raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
     // The first chunks of the stream are requested in three instalments between the setup steps
     // rather than all at once: a workgroup's full ring is 80 KiB, and the small reads of waves
     // that start later would queue behind it in the CU's memory pipeline.
@@ -418,12 +427,59 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     // First use of a loaded value.  The empty statements pin that use here: without them the
     // compiler schedules the basis words ahead of the mask table and waits for the read at once.
     asm volatile("" : "+v"(selector));
+    if (!X16) {
 #pragma unroll
-    for (int r = 0; r < MR; ++r) asm volatile("" : "+v"(raw[r].x), "+v"(raw[r].y));
+        for (int r = 0; r < MR; ++r) asm volatile("" : "+v"(raw[r].x), "+v"(raw[r].y));
+    }
     {
         const uint32_t low = (uint32_t)selector_half(selector, quarter) & 15u;
         const uint32_t high = (uint32_t)selector_half(selector, quarter + 4) & 15u;
         replicate(0u, quad_or((low | high << 4) << (8 * quarter)));
+    }
+    if (X16) {
+        // row maximum: per thread, per wave, then over the 16 waves through LDS (one more barrier)
+        float* wave_max = reinterpret_cast<float*>(wave_sums + 3 * 16);  // the fourth row of sums is unused with one row
+        const __half* h = reinterpret_cast<const __half*>(&raw_x16);
+        float value[8];
+        float amax = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            value[j] = __half2float(h[j]);
+            if (tid < groups) amax = fmaxf(amax, fabsf(value[j]));
+        }
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+        if (lane == 0) wave_max[wave] = amax;
+        prefetch(0, 1);  // the row has arrived: the stream can start while the row is quantised
+        __syncthreads();
+        amax = wave_max[lane & 15];
+#pragma unroll
+        for (int offset = 8; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+        const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
+        const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
+        as_bits[0] = __half_as_ushort(stored);
+        if (blockIdx.x == 0 && tid == 0) *const_cast<__half*>(as) = stored;
+        const float scale = __half2float(stored);
+        const float inverse = __frcp_rn(scale);
+        // the product with the reciprocal decides, except within 2^-14 of a tie, where the correctly
+        // rounded quotient does (the product is within 2^-15 of the quotient)
+        float r[8];
+        float nearest = 1.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float guess = value[j] * inverse;
+            r[j] = rintf(guess);
+            nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
+        }
+        if (nearest < 6.103515625e-05f) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
+        }
+        uint32_t packed[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            packed[j >> 2] |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * (j & 3));
+        raw[0] = make_uint2(packed[0], packed[1]);
     }
     int wave_total[MR];  // sum of this wave's activations, valid in lane 63
 #pragma unroll
@@ -468,7 +524,7 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
         for (int r = 0; r < MR; ++r) wave_sums[r * 16 + wave] = wave_total[r];
     }
-    prefetch(0, 1);
+    if (!X16) prefetch(0, 1);
     __syncthreads();
     prefetch(1, D);
 
@@ -637,7 +693,13 @@ int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipSt
     const bool hold = f.K / 32 / (LPR & (kKMajorLayout - 1)) == D;  // a row's steps fill the ring exactly
     switch (mr_for(rows)) {
         case 1:
-            if (hold)
+            if (f.input_f16 && hold)
+                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true, true>), grid, block, g.shared, stream, a, w,
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            else if (f.input_f16)
+                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false, true>), grid, block, g.shared, stream, a, w,
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+            else if (hold)
                 hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
                                    ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
             else
@@ -903,6 +965,9 @@ int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t 
 
 int gemv_geometry_for(const orx_function& f, int rows, Geometry* g) { return gemv_geometry(f, rows, g); }
 
+// The fp16-input form exists in the replicated-table kernel, one row, one 16-byte piece per thread.
+bool gemv_serves_fp16_input(const orx_function& f) { return use_banked(f, 1) && f.K <= 8 * kBankedThreads; }
+
 // Fills the gemv-specific slots.  codec: 0 Q4 (u32 codes), 1 Q2 (u16 codes), 2 W8.
 int gemv_configure(orx_function* f, int codec, int passes_override) {
     if (f->capacity > 4) {
@@ -979,6 +1044,8 @@ int gemv_prepare_device() {
 #define ORX_OPT_IN_BANKED(depth, lanes)                       \
     ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, true>))     \
     ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, false>))    \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, true, true>))  \
+    ORX_OPT_IN((gemv_banked_kernel<kQ4, 1, depth, lanes, false, true>)) \
     ORX_OPT_IN((gemv_banked_kernel<kQ4, 2, depth, lanes, false>))    \
     ORX_OPT_IN((gemv_banked_kernel<kQ4, 4, depth, lanes, false>))
     ORX_OPT_IN_BANKED(4, 16) ORX_OPT_IN_BANKED(5, 16) ORX_OPT_IN_BANKED(6, 16)

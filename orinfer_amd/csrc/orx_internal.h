@@ -56,6 +56,7 @@ struct orx_function {
     int M = 0, N = 0, K = 0, E = 0, top_k = 0, H = 0, stride = 0, group = 0, tiles = 0, slots = 0;
     int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0;
     bool out_f32 = false;
+    bool input_f16 = false;  // single-row projection that quantises its fp16 activations itself
     const void* device_function = nullptr;  // for hipFuncGetAttributes
     // Device scratch owned by the handle (allocated when it is resolved on a machine with a
     // device, freed by orx_release): decoded int8 weights of a two-stage projection that serves

@@ -312,6 +312,39 @@ def test_int8_small_projection_symbol(m, block_m):
             gu.kernel("int8_small_projection", M=4, N=n, K=k, **bad)
 
 
+@pytest.mark.parametrize("n,k,packed_k", [(9728, 2560, 0), (17408, 5120, 0), (200, 1024, 0), (4096, 8192, 0),
+                                          (17408, 5120, 128), (136, 2048, 128)])
+def test_q4_gemv_quantises_fp16_input_itself(n, k, packed_k):
+    """input_dtype=float16: one launch gives what activation_quantization + e8p_q4_projection give."""
+    rng = np.random.default_rng(orc.SEED + n + k)
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    stored = gu.dev(packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k))
+    kern = gu.kernel("e8p_q4_projection", M=1, N=n, K=k, packed_k=packed_k, input_dtype="float16")
+    weights = orc.q4_integers(packed, TABLE)
+    out = torch.full((2, n), 9.0, dtype=torch.float16, device=gu.DEV)
+    a_scale = torch.full((2,), 7.0, dtype=torch.float16, device=gu.DEV)
+    for case in range(3):
+        x = rng.normal(size=(1, k)).astype(np.float16)
+        if case == 1:
+            x[0, :4] = [900, -900, 0, 1e-7]  # a large maximum: most codes are zero
+        if case == 2:
+            x[:] = 0                              # zero row: scale one, zero output
+        kern(A=gu.dev(x), AS=a_scale, Book=gu.book(), Out=out, S=gu.dev(scales), W=stored)
+        a_q, a_s = orc.a8(x)
+        np.testing.assert_array_equal(gu.host(a_scale)[:1], a_s[:, 0])
+        np.testing.assert_array_equal(gu.host(out)[:1], orc.project(a_q, a_s, weights, scales))
+        assert float(gu.host(a_scale)[1]) == 7.0 and (gu.host(out)[1] == 9).all()
+
+
+def test_q4_fp16_input_is_refused_where_no_kernel_serves_it():
+    for variant in (dict(M=2, N=256, K=1024), dict(M=1, N=256, K=1024, algorithm="mfma"), dict(M=1, N=256, K=16384),
+                    dict(M=1, N=256, K=1024, input_dtype="bfloat16")):
+        variant.setdefault("input_dtype", "float16")
+        with pytest.raises(Exception):
+            gu.kernel("e8p_q4_projection", **variant)
+
+
 def test_q4_embedding_gather_matches_oracle():
     rng = np.random.default_rng(orc.SEED + 40)
     vocab, hidden, cap = 50, 640, 16
