@@ -87,6 +87,7 @@ struct GemmParams {
     const int* tile_count;
     int64_t expert_weight_stride;  // bytes between experts in w
     int tile_rows;                 // rows a routed tile may hold (0: the kernel's own tile height)
+    int* partials;                 // split launches: int32 partial tiles, two slots per workgroup
 };
 
 template <int CODEC>
@@ -260,6 +261,224 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     }
 }
 
+// ---- the same tiles with the K steps dealt evenly to the workgroups ------------------------------
+// With a few hundred output tiles for 256 CUs (N = 17408 at 128 rows: 136 tiles) whole tiles leave
+// CUs idle or give some CUs twice the work, and a CU's share of the memory system bounds its tile.
+// Here the (tile, K step) units are numbered tile-major and workgroup g of G takes units
+// [g U / G, (g + 1) U / G): every CU pulls the same number of bytes.  A run of units that covers a
+// whole tile is finished in place; any other run leaves its int32 accumulators in one of the
+// workgroup's two partial slots (first run, last run), and gemm_split_finish_kernel adds the runs of
+// each tile (exact: integers) and rescales.  No atomics, no waiting between workgroups.
+constexpr int kSplitTile = 128;
+constexpr int kSplitSlotInts = kSplitTile * kSplitTile;
+
+__device__ __forceinline__ int64_t split_begin(int64_t units, int g, int groups) { return units * g / groups; }
+
+template <int CODEC>
+__global__ __launch_bounds__(256) void gemm_split_kernel(GemmParams p) {
+    constexpr int BM = kSplitTile, BN = kSplitTile, WAVES_M = 2;
+    constexpr int WAVES_N = 4 / WAVES_M;
+    constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
+    constexpr int A_CHUNKS = BM * 8 / 256;                        // uint4 per thread for A
+    constexpr int W_CHUNKS = BN * weight_chunks<CODEC>() / 256;   // uint4 per thread for weights
+    static_assert(A_CHUNKS >= 1 && W_CHUNKS >= 1, "tile too small for 256 threads");
+
+    __shared__ __align__(16) int8_t lds_a[BM * kPitch];
+    __shared__ __align__(16) int8_t lds_w[BN * kPitch];
+    __shared__ typename Tables<CODEC>::type tables;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int8_t* w_base = reinterpret_cast<const int8_t*>(p.w);
+    const __half* ws = p.ws;
+    const int tiles_n = (p.n + BN - 1) / BN, tiles_m = (p.m + BM - 1) / BM;
+    const int64_t units = (int64_t)tiles_m * tiles_n * (p.k / kBK);
+    const int64_t unit_begin = split_begin(units, blockIdx.x, gridDim.x), unit_end = split_begin(units, blockIdx.x + 1, gridDim.x);
+    int n0 = 0, row0 = 0, rows_here = 1;
+
+    if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, 256);
+
+    const int k_tiles = p.k / kBK;
+    v4u held_a[A_CHUNKS], held_w[W_CHUNKS];
+
+    auto load_tile = [&](int kt, v4u (&reg_a)[A_CHUNKS], v4u (&reg_w)[W_CHUNKS]) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            const int r = min(c >> 3, rows_here - 1), kc = c & 7;
+            reg_a[i] = *reinterpret_cast<const v4u*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            constexpr int PER_ROW = weight_chunks<CODEC>();
+            const int nn = min(n0 + c / PER_ROW, p.n - 1), q = c % PER_ROW;
+            int64_t byte;
+            if (CODEC == kW8)
+                byte = (int64_t)nn * p.k + kt * kBK + q * 16;
+            else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
+                byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
+            else  // (N, K/8 codes)
+                byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
+            reg_w[i] = *reinterpret_cast<const v4u*>(w_base + byte);
+        }
+    };
+
+    auto store_tile = [&](const v4u (&reg_a)[A_CHUNKS], const v4u (&reg_w)[W_CHUNKS]) {
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            *reinterpret_cast<v4u*>(lds_a + (c >> 3) * kPitch + (c & 7) * 16) = reg_a[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const int c = tid + 256 * i;
+            constexpr int PER_ROW = weight_chunks<CODEC>();
+            const int nn = c / PER_ROW, q = c % PER_ROW;
+            if constexpr (CODEC == kW8) {
+                *reinterpret_cast<v4u*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
+            } else if constexpr (CODEC == kQ4) {
+                // 4 u32 codes -> 32 weights at k offset q*32
+                const uint2 d0 = decode_q4(tables, reg_w[i].x), d1 = decode_q4(tables, reg_w[i].y);
+                const uint2 d2 = decode_q4(tables, reg_w[i].z), d3 = decode_q4(tables, reg_w[i].w);
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 32);
+                dst[0] = make_uint4(d0.x, d0.y, d1.x, d1.y);
+                dst[1] = make_uint4(d2.x, d2.y, d3.x, d3.y);
+            } else {
+                // 8 u16 codes -> 64 weights at k offset q*64
+                const uint32_t pair[4] = {reg_w[i].x, reg_w[i].y, reg_w[i].z, reg_w[i].w};
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 64);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint2 lo = decode_q2(tables, pair[j] & 0xFFFFu), hi = decode_q2(tables, pair[j] >> 16);
+                    dst[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+                }
+            }
+        }
+    };
+
+    __syncthreads();  // tables ready
+    for (int64_t unit = unit_begin; unit < unit_end;) {
+        const int tile = (int)(unit / k_tiles), kt_begin = (int)(unit - (int64_t)tile * k_tiles);
+        const int kt_end = (int)min((int64_t)k_tiles, kt_begin + (unit_end - unit));
+        n0 = (tile % tiles_n) * BN;
+        row0 = (tile / tiles_n) * BM;
+        rows_here = min(BM, p.m - row0);
+        v16i acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+        load_tile(kt_begin, held_a, held_w);
+        for (int kt = kt_begin; kt < kt_end; ++kt) {
+            store_tile(held_a, held_w);
+            __syncthreads();
+            if (kt + 1 < kt_end) load_tile(kt + 1, held_a, held_w);
+            const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
+#pragma unroll
+            for (int ks = 0; ks < kBK / 32; ++ks) {
+                v4i fa[TM], fb[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    fa[i] = *reinterpret_cast<const v4i*>(lds_a + ((wave_m * TM + i) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    fb[j] = *reinterpret_cast<const v4i*>(lds_w + ((wave_n * TN + j) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
+            __syncthreads();
+        }
+        const bool whole = kt_begin == 0 && kt_end == k_tiles;
+        if (!whole) {
+            // accumulator (i, j, r) of thread tid at ((i TN + j) 16 + r) 256 + tid: 1 KiB per store instruction
+            int* slot = p.partials + ((int64_t)blockIdx.x * 2 + (unit == unit_begin ? 0 : 1)) * kSplitSlotInts;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) slot[((i * TN + j) * 16 + r) * 256 + tid] = acc[i][j][r];
+        } else {
+    // epilogue: lane holds column (lane&31) and rows 8*(r/4) + 4*(lane>>5) + r%4 of each 32x32 block
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const int col = n0 + (wave_n * TN + j) * 32 + (lane & 31);
+        if (col >= p.n) continue;
+        const float wscale = __half2float(ws[col]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int local = (wave_m * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (local < rows_here) {
+                    const int64_t row = row0 + local;
+                    const float value = rescale(acc[i][j][r], wscale, __half2float(p.as[row]));
+                    if (p.out_f32)
+                        reinterpret_cast<float*>(p.out)[row * p.stride + col] = value;
+                    else
+                        reinterpret_cast<__half*>(p.out)[row * p.stride + col] = __float2half_rn(value);
+                }
+            }
+        }
+    }
+        }
+        unit += kt_end - kt_begin;
+    }
+}
+
+// Four workgroups per output tile, one per 32 x 32 block of every wave's 64 x 64: nothing to do when
+// one run covered the tile, else the sum of the tile's runs (in workgroup order) goes through the same
+// rescale and store as above.  A thread has 16 sums, so all loads of a run are in flight at once.
+__global__ __launch_bounds__(256) void gemm_split_finish_kernel(GemmParams p, int groups) {
+    constexpr int BM = kSplitTile, BN = kSplitTile, WAVES_N = 2, TM = 2, TN = 2;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int tiles_n = (p.n + BN - 1) / BN, tiles_m = (p.m + BM - 1) / BM;
+    const int k_tiles = p.k / kBK;
+    const int64_t units = (int64_t)tiles_m * tiles_n * k_tiles;
+    const int tile = blockIdx.x >> 2, i = (blockIdx.x >> 1) & 1, j = blockIdx.x & 1;
+    const int64_t first = (int64_t)tile * k_tiles, last = first + k_tiles;
+    int g = (int)(first * groups / units);
+    while (g > 0 && split_begin(units, g, groups) > first) --g;
+    while (split_begin(units, g + 1, groups) <= first) ++g;
+    if (split_begin(units, g, groups) <= first && split_begin(units, g + 1, groups) >= last) return;  // one run: done in place
+    int acc[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0;
+    for (; g < groups && split_begin(units, g, groups) < last; ++g) {
+        const int64_t begin = split_begin(units, g, groups);
+        const int64_t run_start = begin > first ? begin : first;
+        const int* slot = p.partials + ((int64_t)g * 2 + (run_start == begin ? 0 : 1)) * kSplitSlotInts;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] += slot[((i * TN + j) * 16 + r) * 256 + tid];
+    }
+    const int n0 = (tile % tiles_n) * BN, row0 = (tile / tiles_n) * BM;
+    const int rows_here = min(BM, p.m - row0);
+    const int col = n0 + (wave_n * TN + j) * 32 + (lane & 31);
+    if (col >= p.n) return;
+    const float wscale = __half2float(p.ws[col]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int local = (wave_m * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (local < rows_here) {
+            const int64_t row = row0 + local;
+            const float value = rescale(acc[r], wscale, __half2float(p.as[row]));
+            if (p.out_f32)
+                reinterpret_cast<float*>(p.out)[row * p.stride + col] = value;
+            else
+                reinterpret_cast<__half*>(p.out)[row * p.stride + col] = __float2half_rn(value);
+        }
+    }
+}
+
 // Whole-matrix decode to int8 (diagnostic; e8p_q4.py:267-302).  One thread per code.
 template <int CODEC>
 __global__ __launch_bounds__(256) void unpack_kernel(const void* __restrict__ w, const uint32_t* __restrict__ book,
@@ -352,6 +571,42 @@ bool use_expand(const orx_function& f, int rows) {
     return f.flags == kQ4 && f.workspace != nullptr && use_big(f, rows) && rows >= kExpandRows;
 }
 
+// Split launches serve the 128-row tiles when whole tiles would not spread evenly: up to two tiles
+// per CU.  The handle owns the partial slots (allocated when it is resolved).
+int split_groups() {
+    static int groups = 0;
+    if (groups == 0) {
+        int device = 0;
+        hipDeviceProp_t prop;
+        // two workgroups per CU: a single workgroup of four waves leaves every load latency exposed
+        groups = 2 * (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess &&
+                              prop.multiProcessorCount > 0
+                          ? prop.multiProcessorCount
+                          : 256);
+    }
+    return groups;
+}
+bool use_split(const orx_function& f, int rows) {
+    if (f.partials == nullptr || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
+    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows) || use_big(f, rows) || pick_bm(rows) != 128) return false;
+    const int64_t tiles = (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
+    // Measured at K = 5120 with N = 5120, 7168 and 17408: 40-272 tiles gain 10-40 % (two-stage codes
+    // 59 -> 44 us at 136 tiles, 53 -> 32 us at 80), 408 tiles lose; a handful of tiles is latency, not
+    // balance, and two launches would only add to it.
+    return tiles >= 8 && tiles <= (int64_t)split_groups() * 9 / 16 && tiles % (split_groups() / 2) != 0;
+}
+
+template <int CODEC>
+int launch_split(const GemmParams& p, hipStream_t stream) {
+    const int groups = split_groups();
+    hipLaunchKernelGGL((gemm_split_kernel<CODEC>), dim3(groups), dim3(256), 0, stream, p);
+    int code = hip_check(hipGetLastError(), "launch projection (mfma, split K steps)");
+    if (code != ORX_OK) return code;
+    const uint32_t tiles = ceil_div((uint32_t)p.n, 128u) * ceil_div((uint32_t)p.m, 128u);
+    hipLaunchKernelGGL(gemm_split_finish_kernel, dim3(4 * tiles), dim3(256), 0, stream, p, groups);
+    return hip_check(hipGetLastError(), "launch projection (mfma, sum of split tiles)");
+}
+
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_resident(f, rows)) {
@@ -364,6 +619,12 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     }
     if (use_big(f, rows)) {
         gemm_big_geometry(rows, f.N, f.flags == kQ4 && !use_expand(f, rows), g);
+        return ORX_OK;
+    }
+    if (use_split(f, rows)) {
+        g->grid[0] = (uint32_t)split_groups();
+        g->block[0] = 256;
+        g->shared = 0;
         return ORX_OK;
     }
     const int bm = f.tiles ? f.tiles : pick_bm(rows);
@@ -414,6 +675,10 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     if (use_big(f, rows))
         return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
                                f.out_f32, g, stream);
+    if (use_split(f, rows)) {
+        p.partials = static_cast<int*>(f.partials);
+        return launch_split<kQ4>(p, stream);
+    }
     return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
 
@@ -441,6 +706,10 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     if (use_big(f, rows))
         return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
                                stream);
+    if (use_split(f, rows)) {
+        p.partials = static_cast<int*>(f.partials);
+        return launch_split<kW8>(p, stream);
+    }
     return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
 
@@ -518,6 +787,18 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
             if (f->algorithm == kGemv && f->capacity > 4) return gemv_configure(f, codec, passes);  // reports the error
             f->block_m = probe.block_m;
             f->slots = probe.slots;  // ring depth of the replicated-table gemv, 0 = compact tables
+        }
+    }
+    // Partial slots of split launches (two 128 x 128 int32 tiles per workgroup): allocated here, never at
+    // launch.  Without a device (a build machine) or without memory the handle keeps whole tiles.
+    {
+        int devices = 0;
+        const bool split = v.boolean("split_k", true, &bad);  // diagnostic: false keeps whole tiles
+        if (bad) return ORX_ERR_BAD_VARIANT;
+        if (split && f->capacity > 64 && f->tiles == 0 && (f->algorithm == kAuto || f->algorithm == kMfma) &&
+            hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
+            if (hipMalloc(&f->partials, (size_t)split_groups() * 2 * kSplitSlotInts * sizeof(int)) != hipSuccess)
+                f->partials = nullptr, (void)hipGetLastError();
         }
     }
     f->geometry = projection_geometry;

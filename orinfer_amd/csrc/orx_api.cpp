@@ -263,6 +263,7 @@ int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
 
 int orx_release(orx_fn f) {
     if (f != nullptr && f->workspace != nullptr) (void)hipFree(f->workspace);
+    if (f != nullptr && f->partials != nullptr) (void)hipFree(f->partials);
     if (f != nullptr) delete f->inner;
     delete f;
     return ORX_OK;

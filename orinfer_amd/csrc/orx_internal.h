@@ -63,6 +63,8 @@ struct orx_function {
     // many rows.  Launches of one handle share it, so they must not overlap on different streams.
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
+    // int32 partial tiles of launches that split the K steps of output tiles over workgroups (owned).
+    void* partials = nullptr;
     // A handle composed of other kernels of the catalog keeps them here (owned).
     orx_function* inner = nullptr;
     // rows -> geometry; returns ORX_OK or an error code

@@ -345,6 +345,46 @@ def test_q4_fp16_input_is_refused_where_no_kernel_serves_it():
             gu.kernel("e8p_q4_projection", **variant)
 
 
+@pytest.mark.parametrize("codec,m,n,k,dtype", [("q4", 128, 8704, 512, "float16"), ("q4", 70, 8300, 384, "float16"),
+                                               ("w8", 128, 8704, 256, "float16"), ("w8", 300, 8450, 384, "float32"),
+                                               ("q4", 256, 17408, 256, "float16")])
+def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
+    """65-384 rows on the 128-row tiles: the K steps of the tiles are dealt evenly to one workgroup per
+    CU, runs that do not cover a whole tile meet as int32 partial sums.  Same bytes as whole tiles."""
+    rng = np.random.default_rng(orc.SEED + m + n)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.03, m).astype(np.float16)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    torch_dtype = torch.float16 if dtype == "float16" else torch.float32
+    stride = n + 8
+    if codec == "q4":
+        packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+        weights = orc.q4_integers(packed, TABLE)
+        symbol, stored = "e8p_q4_projection", gu.dev(packed)
+        call = lambda kern, out: kern(A=gu.dev(a), AS=gu.dev(a_s), Book=gu.book(), Out=out, S=gu.dev(scales), W=stored)
+    else:
+        weights = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        symbol, stored = "int8_projection", gu.dev(weights)
+        call = lambda kern, out: kern(A=gu.dev(a), Output=out, TokenScale=gu.dev(a_s), Weight=stored, WeightScale=gu.dev(scales))
+    variant = dict(M=m, N=n, K=k, output_dtype=dtype, output_stride=stride)
+    split = gu.kernel(symbol, **variant)
+    whole = gu.kernel(symbol, split_k=False, **variant)
+    grid_split, grid_whole = tuple(split.geometry()[0]), tuple(whole.geometry()[0])
+    assert grid_split[1] == 1 and grid_whole[0] == -(-n // 128) and grid_whole[1] == -(-m // 128)
+    out = torch.full((m + 1, stride), 9.0, dtype=torch_dtype, device=gu.DEV)
+    other = torch.full((m + 1, stride), 9.0, dtype=torch_dtype, device=gu.DEV)
+    call(split, out)
+    call(whole, other)
+    assert torch.equal(out, other)
+    want = orc.project(a, a_s, weights, scales, out_dtype=np.float16 if dtype == "float16" else np.float32)
+    np.testing.assert_array_equal(gu.host(out)[:m, :n], want)
+    assert (gu.host(out)[m] == 9).all() and (gu.host(out)[:, n:] == 9).all()
+    # again into the same buffers: the partial slots carry nothing over
+    out.fill_(9)
+    call(split, out)
+    assert torch.equal(out, other)
+
+
 def test_q4_embedding_gather_matches_oracle():
     rng = np.random.default_rng(orc.SEED + 40)
     vocab, hidden, cap = 50, 640, 16
