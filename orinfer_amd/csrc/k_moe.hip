@@ -7,6 +7,7 @@
 // the result is deterministic and every kernel is replayable inside a captured graph.
 #include <hip/hip_fp16.h>
 
+#include "a8_device.h"
 #include "orx_internal.h"
 
 namespace orx {
@@ -391,6 +392,52 @@ __global__ __launch_bounds__(256) void expert_dispatch_kernel(const int8_t* __re
     for (int g = threadIdx.x; g < groups; g += 256) ds[(int64_t)slot * groups + g] = scale[(int64_t)row * groups + g];
 }
 
+// The same with the quantiser in front (un-rotated activations): A is the fp16 row, every assignment
+// quantises its token row by the A8 rule (one scale per row) straight into its slot.  The row is
+// quantised top_k times over, which costs less than a launch of its own and a round trip of the codes.
+__global__ __launch_bounds__(256) void quantize_dispatch_kernel(const __half* __restrict__ x, int8_t* __restrict__ d,
+                                                                __half* __restrict__ ds, const int* __restrict__ ids,
+                                                                const int* __restrict__ relative,
+                                                                const int* __restrict__ row_offsets,
+                                                                int* __restrict__ slot_map, int h, int top_k) {
+    __shared__ float wave_max[4];
+    const int assignment = blockIdx.x, tid = threadIdx.x;
+    const int row = assignment / top_k;
+    const __half* src = x + (int64_t)row * h;
+    const int pieces = h / 8;  // the host guarantees h % 8 == 0 and 16-byte aligned rows
+    // the row's first piece is requested before the slot's chain of dependent reads, and stays in
+    // registers (the whole row when h <= 2048)
+    uint4 kept = reinterpret_cast<const uint4*>(src)[min(tid, pieces - 1)];
+    const int slot = row_offsets[ids[assignment]] + relative[assignment];
+    if (tid == 0) slot_map[assignment] = slot;
+    int8_t* dst = d + (int64_t)slot * h;
+    float amax = 0.f;
+    for (int i = tid; i < pieces; i += 256) {
+        const uint4 raw = i == tid ? kept : reinterpret_cast<const uint4*>(src)[i];
+        const __half2* pairs = reinterpret_cast<const __half2*>(&raw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float2 f = __half22float2(pairs[j]);
+            amax = fmaxf(amax, fmaxf(fabsf(f.x), fabsf(f.y)));
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    const __half stored = a8_scale(amax);
+    if (tid == 0) ds[slot] = stored;
+    const float scale = __half2float(stored), inverse = __frcp_rn(scale);
+    for (int i = tid; i < pieces; i += 256) {
+        const uint4 raw = i == tid ? kept : reinterpret_cast<const uint4*>(src)[i];
+        const __half* v = reinterpret_cast<const __half*>(&raw);
+        const float low[4] = {__half2float(v[0]), __half2float(v[1]), __half2float(v[2]), __half2float(v[3])};
+        const float high[4] = {__half2float(v[4]), __half2float(v[5]), __half2float(v[6]), __half2float(v[7])};
+        reinterpret_cast<uint2*>(dst)[i] = make_uint2(quantise4(low, scale, inverse), quantise4(high, scale, inverse));
+    }
+}
+
 // grid (M, ceil(H/256)): fp32 accumulate in rank order, one fp16 cast.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const __half* __restrict__ expert, __half* __restrict__ output,
                                                           const float* __restrict__ prob, const __half* __restrict__ shared,
@@ -697,6 +744,13 @@ int dispatch_geometry(const orx_function& f, int rows, Geometry* g) {
     return ORX_OK;
 }
 int dispatch_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
+    if (f.flags & 1) {  // fp16 rows, quantised on the way (Scale is not read)
+        hipLaunchKernelGGL(quantize_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const __half>(args, 0),
+                           pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 2), pointer_arg<const int>(args, 3),
+                           pointer_arg<const int>(args, 4), pointer_arg<const int>(args, 5), pointer_arg<int>(args, 7), f.H,
+                           f.top_k);
+        return hip_check(hipGetLastError(), "launch expert_dispatch (fp16 rows)");
+    }
     hipLaunchKernelGGL(expert_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int8_t>(args, 0),
                        pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 2), pointer_arg<const int>(args, 3),
                        pointer_arg<const int>(args, 4), pointer_arg<const int>(args, 5),
@@ -713,9 +767,18 @@ int make_dispatch(const Variant& v, orx_function* f) {
         set_error("expert_dispatch: invalid MoE activation dispatch dimensions");
         return ORX_ERR_BAD_VARIANT;
     }
-    f->args = {{"A", ArgPointer, 1},          {"D", ArgPointer, 1},          {"DS", ArgPointer, 2},
+    // input_dtype=float16: A holds fp16 rows, quantised by the A8 rule on the way to their slots (one scale
+    // per row); Scale is then not read and may be null
+    const std::string input = v.string("input_dtype", "int8", &bad);
+    if (bad || (input != "int8" && input != "float16") || (input == "float16" && (f->group != f->H || f->H % 8))) {
+        set_error("expert_dispatch: input_dtype must be int8 or float16 (float16: one scale per row, H a multiple of 8)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    const bool fp16_rows = input == "float16";
+    f->flags = fp16_rows ? 1 : 0;
+    f->args = {{"A", ArgPointer, fp16_rows ? 16u : 1u}, {"D", ArgPointer, fp16_rows ? 8u : 1u}, {"DS", ArgPointer, 2},
                {"IDs", ArgPointer, 4},        {"RelativeSlot", ArgPointer, 4}, {"RowOffsets", ArgPointer, 4},
-               {"Scale", ArgPointer, 2},      {"SlotMap", ArgPointer, 4}};
+               {"Scale", ArgPointer, fp16_rows ? 0x80000002u : 2u}, {"SlotMap", ArgPointer, 4}};
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = dispatch_geometry;
     f->launch = dispatch_launch;

@@ -17,6 +17,7 @@
 // * row scale, * sign), one fp16 cast; ids outside the vocabulary give zero rows.
 #include <hip/hip_fp16.h>
 
+#include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -53,37 +54,6 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     float r = scratch[0];
     for (int i = 1; i < waves; ++i) r = fmaxf(r, scratch[i]);
     return r;
-}
-
-// rint(value / scale), clamped: the product with the reciprocal decides, except within 2^-14 of a
-// tie, where the correctly rounded quotient does.  The product is within 4 units in the last place
-// of the quotient (|quotient| < 128.5, so 2^-15 at most), so the two round alike everywhere else;
-// the reference's kernel takes the same shortcut (kernels/cuda/model/rotation_a8.py:153-164).
-__device__ __forceinline__ int8_t quantise(float value, float scale, float inverse) {
-    const float guess = value * inverse;
-    float r = rintf(guess);
-    if (fabsf(fabsf(guess - r) - 0.5f) < 6.103515625e-05f) r = rintf(__fdiv_rn(value, scale));
-    return (int8_t)fmaxf(-127.f, fminf(127.f, r));
-}
-
-// Four codes packed into one word; one test (and, rarely, four exact quotients) for the four.
-__device__ __forceinline__ uint32_t quantise4(const float (&value)[4], float scale, float inverse) {
-    float r[4];
-    float nearest = 1.0f;  // smallest distance of a product from a tie
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float guess = value[j] * inverse;
-        r[j] = rintf(guess);
-        nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
-    }
-    if (nearest < 6.103515625e-05f) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
-    }
-    uint32_t packed = 0;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * j);
-    return packed;
 }
 
 // grid (rows, groups), 256 threads.

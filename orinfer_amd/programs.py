@@ -75,7 +75,7 @@ class MoeLayer:
     """Q2A8 expert layer: token-sort, grouped gate_up, SwiGLU->A8, grouped down, weighted combine."""
 
     def __init__(self, tokens, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales,
-                 block_m=32, packed_k=128, fused_metadata=None):
+                 block_m=32, packed_k=128, fused_metadata=None, fused_dispatch=True):
         self.tokens, self.experts, self.top_k = tokens, experts, top_k
         self.hidden, self.inter, self.block_m = hidden, intermediate, block_m
         assignments = tokens * top_k
@@ -120,8 +120,12 @@ class MoeLayer:
         self.k_histogram = Kernel("expert_histogram", **common)
         self.k_offsets = Kernel("expert_offsets", E=experts, block_m=block_m)
         self.k_tiles = Kernel("expert_tiles", block_m=block_m, **common)
+        # the dispatch quantises the fp16 rows on its way (one launch instead of quantiser + copy) where
+        # the row layout allows it
+        self.fused_dispatch = fused_dispatch and hidden % 8 == 0
         self.k_a8 = Kernel("activation_quantization", K=hidden)
-        self.k_dispatch = Kernel("expert_dispatch", H=hidden, **common)
+        self.k_dispatch = Kernel("expert_dispatch", H=hidden, **common,
+                                 **({"input_dtype": "float16"} if self.fused_dispatch else {}))
         grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k)
         self.k_gate_up = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, **grouped)
         self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
@@ -141,9 +145,13 @@ class MoeLayer:
                            TileOffsets=self.tile_offsets)
             self.k_tiles(stream=s, Counts=self.counts, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
                          TileRow=self.tile_row)
-        self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=self.tokens)
-        self.k_dispatch(stream=s, A=self.a_q, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
-                        RowOffsets=self.row_offsets, Scale=self.a_s, SlotMap=self.slot_map)
+        if self.fused_dispatch:
+            self.k_dispatch(stream=s, A=x16, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
+                            RowOffsets=self.row_offsets, Scale=None, SlotMap=self.slot_map)
+        else:
+            self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=self.tokens)
+            self.k_dispatch(stream=s, A=self.a_q, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
+                            RowOffsets=self.row_offsets, Scale=self.a_s, SlotMap=self.slot_map)
         routed = dict(Book=self.book, Counts=self.counts, Offsets=self.row_offsets, TileCount=self.tile_count,
                       TileExpert=self.tile_expert, TileRow=self.tile_row)
         self.k_gate_up(stream=s, A=self.d, AS=self.ds, C=self.gate_up_out, P=self.w1, WS=self.s1, **routed)

@@ -262,9 +262,10 @@ def test_combine_invalid_slots_and_shared_expert(m, h, slots):
     assert (np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)).all()
 
 
-def run_layer(c, bm, packed_k=128):
+def run_layer(c, bm, packed_k=128, fused_dispatch=True):
     layer = programs.MoeLayer(c["tokens"], c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
-                              c["gate_up_scales"], c["down"], c["down_scales"], block_m=bm, packed_k=packed_k)
+                              c["gate_up_scales"], c["down"], c["down_scales"], block_m=bm, packed_k=packed_k,
+                              fused_dispatch=fused_dispatch)
     layer.run(gu.dev(c["x"]), gu.dev(c["logits"]))
     gu.sync()
     return layer
@@ -281,10 +282,12 @@ def check_layer(c, layer, bm):
     np.testing.assert_array_equal(gu.host(layer.row_offsets), rows)
     np.testing.assert_array_equal(gu.host(layer.tile_count), total)
     a_q, a_s = orc.a8(c["x"])
-    np.testing.assert_array_equal(gu.host(layer.a_q), a_q)
+    if not layer.fused_dispatch:  # else the rows are quantised on their way to the slots
+        np.testing.assert_array_equal(gu.host(layer.a_q), a_q)
     d, ds, slot = orc.expert_dispatch(a_q, a_s, ids, rel, rows)
     np.testing.assert_array_equal(gu.host(layer.slot_map), slot)
     np.testing.assert_array_equal(gu.host(layer.d), d)
+    np.testing.assert_array_equal(gu.host(layer.ds), ds)
     w1 = np.stack([orc.q2_integers(x, TABLE) for x in c["gate_up"]])
     w2 = np.stack([orc.q2_integers(x, TABLE) for x in c["down"]])
     gate_up = orc.grouped_project(d, ds, w1, c["gate_up_scales"], counts, rows)
@@ -310,6 +313,7 @@ def test_moe_layer_small_end_to_end():
     c = workloads.config3(tokens=40, experts=16, top_k=4, hidden=256, intermediate=128)
     for bm in (32, 64):
         check_layer(c, run_layer(c, bm), bm)
+    check_layer(c, run_layer(c, 32, fused_dispatch=False), 32)  # quantiser and dispatch as two launches
 
 
 def test_config3_full_size_end_to_end():
@@ -605,3 +609,29 @@ def test_router_topk_warp_symbol(m, e, k, warps):
     for variant in (dict(E=100, top_k=4), dict(E=128, top_k=33), dict(E=128, top_k=4, warps=3)):
         with pytest.raises(Exception):
             gu.kernel("router_topk_warp", M=4, **variant)
+
+
+@pytest.mark.parametrize("m,e,k,h", [(37, 16, 4, 2048), (256, 128, 8, 2048), (5, 8, 2, 4096 + 8), (3, 4, 1, 64)])
+def test_expert_dispatch_quantises_fp16_rows(m, e, k, h):
+    """input_dtype=float16: the dispatch gives what activation_quantization + expert_dispatch give."""
+    rng = np.random.default_rng(orc.SEED + m + h)
+    x = rng.normal(size=(m, h)).astype(np.float16)
+    x[0] = 0
+    ids_np, _ = orc.router_topk(rng.normal(size=(m, e)).astype(np.float32), k)
+    counts, relative = orc.expert_histogram(ids_np, e)
+    offsets, _, _ = orc.expert_offsets(counts, 32)
+    a_q, a_s = orc.a8(x)
+    want_d, want_ds, want_map = orc.expert_dispatch(a_q, a_s, ids_np, relative, offsets)
+    d = torch.full((m * k + 1, h), 7, dtype=torch.int8, device=gu.DEV)
+    ds = torch.full((m * k + 1,), 3.0, dtype=torch.float16, device=gu.DEV)
+    slot_map = torch.full((m, k), -1, **I32)
+    gu.kernel("expert_dispatch", M=m, H=h, E=e, top_k=k, input_dtype="float16")(
+        A=gu.dev(x), D=d, DS=ds, IDs=gu.dev(ids_np), RelativeSlot=gu.dev(relative), RowOffsets=gu.dev(offsets), Scale=None,
+        SlotMap=slot_map)
+    np.testing.assert_array_equal(gu.host(d)[: m * k], want_d)
+    np.testing.assert_array_equal(gu.host(ds)[: m * k], want_ds[:, 0])
+    np.testing.assert_array_equal(gu.host(slot_map), want_map)
+    assert (gu.host(d)[m * k] == 7).all() and float(gu.host(ds)[m * k]) == 3.0
+    for variant in (dict(H=h, scale_group=h // 2), dict(H=36)):
+        with pytest.raises(Exception):
+            gu.kernel("expert_dispatch", M=m, E=e, top_k=k, input_dtype="float16", **variant)
