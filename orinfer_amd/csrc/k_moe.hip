@@ -459,6 +459,76 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const __half* __restri
     output[(int64_t)row * h + col] = __float2half_rn(acc);
 }
 
+// H a multiple of 8: a thread owns 8 consecutive columns (one 16-byte piece per rank), a workgroup
+// 2048 columns of one row.  Same operations per column as above, in the same order.
+__global__ __launch_bounds__(256) void moe_combine_wide_kernel(const __half* __restrict__ expert, __half* __restrict__ output,
+                                                               const float* __restrict__ prob,
+                                                               const __half* __restrict__ shared,
+                                                               const __half* __restrict__ shared_gate,
+                                                               const int* __restrict__ slot_map, int h, int slots,
+                                                               int top_k) {
+    const int row = blockIdx.x;
+    const int col = (blockIdx.y * 256 + threadIdx.x) * 8;
+    if (col >= h) return;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(expert) | reinterpret_cast<uintptr_t>(output) |
+                           reinterpret_cast<uintptr_t>(shared)) & 15) == 0;
+    auto load8 = [&](const __half* src, __half (&dst)[8]) {
+        if (aligned) {
+            *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(src);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[j] = src[j];
+        }
+    };
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    // Ranks in batches of 8: all slots, then all pieces, then the sums in rank order.  A skipped slot
+    // reads slot 0 and its term is not added, so the loads of a batch do not wait for one another.
+    for (int first = 0; first < top_k; first += 8) {
+        int slot[8];
+        float weight[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int rank = min(first + i, top_k - 1);
+            slot[i] = slot_map[(int64_t)row * top_k + rank];
+            weight[i] = prob[(int64_t)row * top_k + rank];
+        }
+        __align__(16) __half values[8][8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool valid = first + i < top_k && slot[i] >= 0 && slot[i] < slots;
+            load8(expert + (int64_t)(valid ? slot[i] : 0) * h + col, values[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool valid = first + i < top_k && slot[i] >= 0 && slot[i] < slots;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float sum = acc[j] + __half2float(values[i][j]) * weight[i];
+                acc[j] = valid ? sum : acc[j];
+            }
+        }
+    }
+    if (shared != nullptr) {
+        const float gate = __fdiv_rn(1.0f, 1.0f + expf(-__half2float(shared_gate[row])));
+        __align__(16) __half values[8];
+        load8(shared + (int64_t)row * h + col, values);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = acc[j] + gate * __half2float(values[j]);
+    }
+    __align__(16) __half result[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) result[j] = __float2half_rn(acc[j]);
+    __half* dst = output + (int64_t)row * h + col;
+    if (aligned) {
+        *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(result);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst[j] = result[j];
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------
 bool geometry_fields(const Variant& v, orx_function* f, bool need_m) {
     bool bad = false;
@@ -788,13 +858,20 @@ int make_dispatch(const Variant& v, orx_function* f) {
 
 int combine_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
-    g->grid[1] = ceil_div((uint32_t)f.H, 256u);
+    g->grid[1] = ceil_div((uint32_t)f.H, f.H % 8 == 0 ? 2048u : 256u);
     g->block[0] = 256;
     return ORX_OK;
 }
 int combine_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
     // dynamic decode has exactly top_k assignments per live row (moe.py:514-517)
     const int slots = f.dynamic_rows ? rows * f.top_k : f.slots;
+    if (f.H % 8 == 0) {
+        hipLaunchKernelGGL(moe_combine_wide_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
+                           pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), pointer_arg<const float>(args, 2),
+                           pointer_arg<const __half>(args, 3), pointer_arg<const __half>(args, 4),
+                           pointer_arg<const int>(args, 5), f.H, slots, f.top_k);
+        return hip_check(hipGetLastError(), "launch moe_combine");
+    }
     hipLaunchKernelGGL(moe_combine_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
                        pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), pointer_arg<const float>(args, 2),
                        pointer_arg<const __half>(args, 3), pointer_arg<const __half>(args, 4),

@@ -260,6 +260,11 @@ def test_combine_invalid_slots_and_shared_expert(m, h, slots):
     want = orc.moe_combine(ex, sm, prob).astype(np.float32)
     got = gu.host(out).astype(np.float32)
     assert (np.abs(got - want) <= 1e-2 + 1e-3 * np.abs(want)).all()
+    # an output that is only 8-byte aligned takes the element-wise stores: same bytes
+    flat = torch.zeros(m * h + 8, dtype=torch.float16, device=gu.DEV)
+    shifted = flat[4 : 4 + m * h].view(m, h)
+    kern(Expert=gu.dev(ex), Output=shifted, Prob=gu.dev(prob), Shared=None, SharedGate=None, SlotMap=gu.dev(sm))
+    assert torch.equal(shifted, out) and not flat[:4].any() and not flat[4 + m * h :].any()
 
 
 def run_layer(c, bm, packed_k=128, fused_dispatch=True):
