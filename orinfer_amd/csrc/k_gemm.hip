@@ -455,6 +455,7 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(GemmParams p, in
     for (int r = 0; r < 16; ++r) acc[r] = 0;
     for (; g < groups && split_begin(units, g, groups) < last; ++g) {
         const int64_t begin = split_begin(units, g, groups);
+        if (split_begin(units, g + 1, groups) == begin) continue;  // fewer units than workgroups: this one had none
         const int64_t run_start = begin > first ? begin : first;
         const int* slot = p.partials + ((int64_t)g * 2 + (run_start == begin ? 0 : 1)) * kSplitSlotInts;
 #pragma unroll

@@ -385,6 +385,24 @@ def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
     assert torch.equal(out, other)
 
 
+def test_split_launches_serve_k_major_codes_and_dynamic_rows():
+    rng = np.random.default_rng(orc.SEED + 91)
+    n, k, cap = 8704, 384, 256
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    weights = orc.q4_integers(packed, TABLE)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    kern = gu.kernel("e8p_q4_projection", M=cap, N=n, K=k, packed_k=128, dynamic_rows=True)
+    stored = gu.dev(orc.q4_pack_k(packed, 128))
+    for m in (200, 65, 130):
+        a = rng.integers(-128, 128, (cap, k), dtype=np.int8)
+        a_s = rng.uniform(0.01, 0.03, cap).astype(np.float16)
+        out = torch.full((cap, n), 9.0, dtype=torch.float16, device=gu.DEV)
+        assert tuple(kern.geometry(m)[0])[1] == 1  # one workgroup list: the split form
+        kern(A=gu.dev(a), AS=gu.dev(a_s), Book=gu.book(), Out=out, S=gu.dev(scales), W=stored, m=m)
+        np.testing.assert_array_equal(gu.host(out)[:m], orc.project(a[:m], a_s[:m], weights, scales))
+        assert (gu.host(out)[m:] == 9).all()
+
+
 def test_q4_embedding_gather_matches_oracle():
     rng = np.random.default_rng(orc.SEED + 40)
     vocab, hidden, cap = 50, 640, 16
