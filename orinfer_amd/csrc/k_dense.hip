@@ -30,7 +30,6 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
-constexpr int kMaxThreads = 1024;
 // Tables: entry i of the basis table ((h ^ 8) per coordinate) at byte i*256 + copy*8, entry u of the
 // sign/parity mask table at u*256 + 128 + copy*8, 16 copies each.  With the entry index in the
 // address's second byte, one v_perm_b32 builds a lookup address from a byte of the code.
