@@ -218,6 +218,21 @@ def main():
         t_both = timed_graph(lambda i, s: (main_case.quantize(s), main_case.project(i, s)), 2 * copies)
         extra["config1_m1_two_launches"] = {"a8_us": round(t_a8 * 1e6, 3), "gemv_us": sweep["1"]["us"],
                                             "both_us": round(t_both * 1e6, 3)}
+        # the production form of the step: signed block-128 rotation in front of the quantiser
+        signs1 = (torch.randint(0, 2, (main_case.k,), device="cuda", dtype=torch.int8) * 2 - 1)
+        rot1 = Kernel("rotate_activation_a8", M=1, K=main_case.k)
+        fused_rot = Kernel("e8p_q4_projection", M=1, N=main_case.n, K=main_case.k, input_dtype="float16", rotate=True)
+
+        def rotate_then_project(i, s):
+            rot1(stream=s, Q=main_case.a_q, S=main_case.a_s, Signs=signs1, X=main_case.x)
+            main_case.project(i, s)
+
+        t_rot_two = timed_graph(rotate_then_project, 2 * copies)
+        t_rot_one = timed_graph(lambda i, s: fused_rot(stream=s, A=main_case.x, AS=main_case.a_s, Book=book,
+                                                       Out=main_case.out, S=main_case.scales, Signs=signs1,
+                                                       W=main_case.weights[i % copies]), 2 * copies)
+        extra["config1_m1_rotated_input"] = {"rotate_a8_then_gemv_us": round(t_rot_two * 1e6, 3),
+                                             "one_launch_us": round(t_rot_one * 1e6, 3)}
         # the same projection on the reference's storage layout (K-major blocks of 128)
         k_major = {}
         for rows in (1, 8, 32):

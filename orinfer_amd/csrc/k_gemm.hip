@@ -21,7 +21,8 @@ namespace orx {
 
 // from k_gemv.hip
 int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
-                const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out);
+                const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out,
+                const int8_t* signs = nullptr);
 int gemv_geometry_for(const orx_function& f, int rows, Geometry* g);
 int gemv_configure(orx_function* f, int codec, int passes_override);
 int gemv_prepare_device();
@@ -644,9 +645,10 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.book = pointer_arg<const uint32_t>(args, 2);
     p.out = pointer_arg<void>(args, 3);
     p.ws = pointer_arg<const __half>(args, 4);
-    p.w = pointer_arg<const void>(args, 5);
+    const int8_t* signs = f.rotate_input ? pointer_arg<const int8_t>(args, 5) : nullptr;
+    p.w = pointer_arg<const void>(args, f.rotate_input ? 6 : 5);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
-    if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
+    if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out, signs);
     if (use_resident(f, rows)) {
         for (int first = 0; first < rows; first += 32) {
             const size_t out_offset = (size_t)first * f.stride * (f.out_f32 ? 4 : 2);
@@ -844,8 +846,17 @@ int make_q4_projection(const Variant& v, orx_function* f) {
         f->input_f16 = true;
         f->algorithm = kGemv;
     }
+    // rotate=true (fp16 input only): the signed block-128 rotation runs in front of the quantiser, Signs
+    // joins the buffers (kernels/cuda/model/rotation_a8.py:369-383 followed by the projection, in one launch)
+    f->rotate_input = v.boolean("rotate", false, &bad);
+    if (bad || (f->rotate_input && !f->input_f16)) {
+        set_error("e8p_q4_projection: rotate=true needs input_dtype=float16");
+        return ORX_ERR_BAD_VARIANT;
+    }
     f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4},
-               {"Out", ArgPointer, 2}, {"S", ArgPointer, 2},  {"W", ArgPointer, 16}};
+               {"Out", ArgPointer, 2}, {"S", ArgPointer, 2}};
+    if (f->rotate_input) f->args.push_back({"Signs", ArgPointer, 8});
+    f->args.push_back({"W", ArgPointer, 16});
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->launch = q4_launch;
     return ORX_OK;
@@ -1169,9 +1180,10 @@ int make_q2_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f,
 const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
-     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, packed_k=0|128, output_dtype=float16|float32, "
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|mfma, packed_k=0|128, output_dtype=float16|float32, "
+     "input_dtype=int8|float16, rotate=false, split_k=true, "
      "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0, decode_in_gemm=false",
-     "A,AS,Book,Out,S,W[,m]"},
+     "A,AS,Book,Out,S[,Signs],W[,m]"},
     {"int8_projection", make_w8_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "
      "block_m=0|32|64|128|256",

@@ -322,7 +322,7 @@ template <int CODEC, int MR, int D, int LAYOUT, bool HOLD, bool X16 = false>
 __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
-    int m, int out_f32) {
+    int m, int out_f32, const int8_t* __restrict__ signs) {
     extern __shared__ __align__(16) uint32_t lds[];
     constexpr int LPR = LAYOUT & (kKMajorLayout - 1);
     constexpr bool kKMajor = LAYOUT >= kKMajorLayout;
@@ -384,9 +384,11 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     uint32_t selector = book[entry];
     uint2 raw[MR];
     uint4 raw_x16 = make_uint4(0u, 0u, 0u, 0u);
-    if (X16)
+    uint2 sign_bytes = make_uint2(0u, 0u);
+    if (X16) {
         raw_x16 = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(a) + 8 * min(tid, groups - 1));
-    else
+        if (signs != nullptr) sign_bytes = *reinterpret_cast<const uint2*>(signs + 8 * min(tid, groups - 1));
+    } else
 #pragma unroll
         for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
             raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
@@ -441,12 +443,57 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
         float* wave_max = reinterpret_cast<float*>(wave_sums + 3 * 16);  // the fourth row of sums is unused with one row
         const __half* h = reinterpret_cast<const __half*>(&raw_x16);
         float value[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) value[j] = __half2float(h[j]);
+        if (signs != nullptr) {
+            // Signed block-128 rotation in front of the quantiser (kernels/cuda/model/rotation_a8.py:188-224):
+            // a block is the 8 values of each of 16 adjacent threads, so distances 1, 2 and 4 are inside
+            // the thread and 8..64 are lane exchanges at distance 1..8 inside a row of 16 lanes.  Every
+            // stage is one fp32 add or subtract in the reference's order; then one multiply by
+            // fp32(128^-1/2) and the fp16 boundary.
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                value[j] *= (float)(int8_t)((j < 4 ? sign_bytes.x : sign_bytes.y) >> (8 * (j & 3)));
+#pragma unroll
+            for (int distance = 1; distance < 8; distance <<= 1) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (j & distance) continue;
+                    const float left = value[j], right = value[j + distance];
+                    value[j] = left + right;
+                    value[j + distance] = left - right;
+                }
+            }
+#pragma unroll
+            for (int bit = 0; bit < 4; ++bit) {
+                const uint32_t flip = ((uint32_t)(lane >> bit) & 1u) << 31;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int own = __float_as_int(value[j]);
+                    int partner;
+                    if (bit == 0)
+                        partner = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+                    else if (bit == 1)
+                        partner = __builtin_amdgcn_update_dpp(0, own, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+                    else if (bit == 2) {
+                        partner = __builtin_amdgcn_update_dpp(own, own, 0x104, 0xF, 0x5, false);      // row_shl:4, banks 0, 2
+                        partner = __builtin_amdgcn_update_dpp(partner, own, 0x114, 0xF, 0xA, false);  // row_shr:4, banks 1, 3
+                    } else
+                        partner = __builtin_amdgcn_update_dpp(0, own, 0x128, 0xF, 0xF, true);  // row_ror:8
+                    value[j] = __int_as_float(partner) + __int_as_float(own ^ (int)flip);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float scaled = value[j] * 0.08838834764831845f;
+                asm volatile("" : "+v"(scaled));  // the fp16 cast rounds the fp32 product, not a fused multiply-convert
+                value[j] = __half2float(__float2half_rn(scaled));
+            }
+        }
         float amax = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            value[j] = __half2float(h[j]);
+        for (int j = 0; j < 8; ++j)
             if (tid < groups) amax = fmaxf(amax, fabsf(value[j]));
-        }
 #pragma unroll
         for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
         if (lane == 0) wave_max[wave] = amax;
@@ -686,6 +733,10 @@ int gemv_geometry(const orx_function& f, int rows, Geometry* g) {
     return ORX_OK;
 }
 
+// Sign vector of the rotation that the fp16-input form applies in front of its quantiser (null: none);
+// set by gemv_launch for the launch it is about to make on this thread.
+static thread_local const int8_t* pending_signs = nullptr;
+
 template <int D, int LPR>  // LPR: the kernel's LAYOUT (lanes per row, + 64 for K-major codes)
 int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
                        const uint4* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
@@ -695,24 +746,24 @@ int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipSt
         case 1:
             if (f.input_f16 && hold)
                 hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true, true>), grid, block, g.shared, stream, a, w,
-                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else if (f.input_f16)
                 hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false, true>), grid, block, g.shared, stream, a, w,
-                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else if (hold)
                 hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
-                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else
                 hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false>), grid, block, g.shared, stream, a, w, book,
-                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
         case 2:
             hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 2, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
-                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
         default:
             hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 4, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
-                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32);
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
     }
     return hip_check(hipGetLastError(), "launch projection (gemv, replicated tables)");
@@ -950,10 +1001,11 @@ bool gemv_serves_k_major(const orx_function& f, int rows) {
 // Launchers used by the projection factories.  Argument order is the caller's business:
 // they pass already-unmarshalled pointers.
 int gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const int8_t* a,
-                const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out) {
+                const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out, const int8_t* signs) {
     // LDS opt-in needs a device, so it happens at the first launch rather than at resolve time
     const int ready = gemv_prepare_device();
     if (ready != ORX_OK) return ready;
+    pending_signs = f.input_f16 ? signs : nullptr;
     if (f.packed_k != 0 && !gemv_serves_k_major(f, rows)) {
         set_error("%s: the gemv algorithm does not serve this K-major shape for %d rows", f.symbol.c_str(), rows);
         return ORX_ERR_BAD_VARIANT;

@@ -57,6 +57,7 @@ struct orx_function {
     int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0;
     bool out_f32 = false;
     bool input_f16 = false;  // single-row projection that quantises its fp16 activations itself
+    bool rotate_input = false;  // ... after the signed block-128 rotation (takes a Signs buffer)
     const void* device_function = nullptr;  // for hipFuncGetAttributes
     // Device scratch owned by the handle (allocated when it is resolved on a machine with a
     // device, freed by orx_release): decoded int8 weights of a two-stage projection that serves

@@ -53,6 +53,8 @@ ABI = {
     ("e8p_q4_embedding", (("M", 8), ("vocab", 1000), ("hidden", 5120))): ["Book", "IDs", "Output", "Scale", "Signs", "Weight", "m"],
     ("rotate_activation_a8", (("M", 8), ("K", 256), ("swiglu", True), ("dynamic_rows", True))): ["Q", "S", "Signs", "X", "m"],
     ("e8p_q4_projection", (("M", 1), ("N", 9728), ("K", 2560))): ["A", "AS", "Book", "Out", "S", "W"],
+    ("e8p_q4_projection", (("M", 1), ("N", 9728), ("K", 2560), ("input_dtype", "float16"), ("rotate", True))):
+        ["A", "AS", "Book", "Out", "S", "Signs", "W"],
     ("e8p_q4_projection", (("M", 64), ("N", 256), ("K", 256), ("dynamic_rows", True))):
         ["A", "AS", "Book", "Out", "S", "W", "m"],
     ("int8_projection", (("M", 8192), ("N", 4096), ("K", 4096))):

@@ -337,6 +337,34 @@ def test_q4_gemv_quantises_fp16_input_itself(n, k, packed_k):
         assert float(gu.host(a_scale)[1]) == 7.0 and (gu.host(out)[1] == 9).all()
 
 
+@pytest.mark.parametrize("n,k,packed_k", [(9728, 2560, 0), (17408, 5120, 0), (200, 1024, 0), (17408, 5120, 128)])
+def test_q4_gemv_rotates_and_quantises_fp16_input(n, k, packed_k):
+    """input_dtype=float16, rotate=true: one launch gives what rotate_activation_a8 + e8p_q4_projection give."""
+    rng = np.random.default_rng(orc.SEED + n + k + 1)
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    stored = gu.dev(packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k))
+    kern = gu.kernel("e8p_q4_projection", M=1, N=n, K=k, packed_k=packed_k, input_dtype="float16", rotate=True)
+    assert kern.arg_names == ["A", "AS", "Book", "Out", "S", "Signs", "W"]
+    weights = orc.q4_integers(packed, TABLE)
+    out = torch.full((2, n), 9.0, dtype=torch.float16, device=gu.DEV)
+    a_scale = torch.full((2,), 7.0, dtype=torch.float16, device=gu.DEV)
+    for case in range(3):
+        x = rng.normal(size=(1, k)).astype(np.float16)
+        if case == 1:
+            x[0, :4] = [900, -900, 0, 1e-7]
+        if case == 2:
+            x[:] = 0
+        kern(A=gu.dev(x), AS=a_scale, Book=gu.book(), Out=out, S=gu.dev(scales), Signs=gu.dev(signs), W=stored)
+        a_q, a_s = orc.rotate_a8(x, signs)
+        np.testing.assert_array_equal(gu.host(a_scale)[:1], a_s[:, 0])
+        np.testing.assert_array_equal(gu.host(out)[:1], orc.project(a_q, a_s, weights, scales))
+        assert float(gu.host(a_scale)[1]) == 7.0 and (gu.host(out)[1] == 9).all()
+    with pytest.raises(Exception):
+        gu.kernel("e8p_q4_projection", M=1, N=n, K=k, rotate=True)
+
+
 def test_q4_fp16_input_is_refused_where_no_kernel_serves_it():
     for variant in (dict(M=2, N=256, K=1024), dict(M=1, N=256, K=1024, algorithm="mfma"), dict(M=1, N=256, K=16384),
                     dict(M=1, N=256, K=1024, input_dtype="bfloat16")):
