@@ -550,11 +550,11 @@ bool use_stream(const orx_function& f, int rows) {
 bool use_resident(const orx_function& f, int rows) {
     if (f.flags != kQ4 || !dense_resident_eligible(f.N, f.K, f.packed_k)) return false;
     if (f.algorithm == kResident) return rows <= 128;
-    // from 3 rows: the GEMV's dot products grow with the row count (23 us at 3 and 4 rows of
-    // N=17408, K=5120), this kernel's MFMAs do not (19 us from 3 to 8 rows)
+    // from 2 rows: the GEMV's dot products grow with the row count (16.4 us at 2 rows, 23 us at 3 and 4
+    // rows of N=17408, K=5120), this kernel's MFMAs do not (15.6 us from 2 to 16 rows)
     // up to 64 rows as two launches of 32 (36 and 39 us at 48 and 64 rows against 42 and 48 us for
     // the streaming kernel)
-    return f.algorithm == kAuto && f.tiles == 0 && rows > (f.packed_k != 0 ? 1 : 2) && rows <= 64;
+    return f.algorithm == kAuto && f.tiles == 0 && rows > 1 && rows <= 64;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
