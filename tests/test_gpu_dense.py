@@ -82,7 +82,8 @@ def test_a8_edges_and_random():
     np.testing.assert_array_equal(gu.host(q), wq)
 
 
-@pytest.mark.parametrize("k,group", [(2560, 64), (384, 128), (100, 25), (7, 7)])
+@pytest.mark.parametrize("k,group", [(2560, 64), (384, 128), (100, 25), (7, 7), (5120, 5120), (16384, 8192), (9001, 9001),
+                                     (1024, 512), (4096, 4096)])
 def test_a8_groups_and_odd_shapes(k, group):
     rng = np.random.default_rng(orc.SEED + k)
     x = (rng.normal(size=(5, k)) * 3).astype(np.float16)
