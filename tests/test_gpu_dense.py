@@ -127,7 +127,7 @@ def test_swiglu_then_a8_and_fused_form_agree():
 
 
 # ---- signed block-128 rotation fused with A8 -------------------------------------------------
-@pytest.mark.parametrize("m,k", [(1, 128), (3, 384), (5, 2560), (2, 5120), (1, 17408)])
+@pytest.mark.parametrize("m,k", [(1, 128), (3, 384), (5, 2560), (2, 5120), (1, 17408), (260, 2304)])
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_rotate_activation_a8_matches_oracle(m, k, swiglu):
     rng = np.random.default_rng(orc.SEED + m + k)
