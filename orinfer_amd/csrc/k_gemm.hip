@@ -533,7 +533,8 @@ bool use_gemv(const orx_function& f, int rows) {
     // K-major codes: 1 row (13.4 us at N=17408, K=5120; the streaming kernel takes 17.2), and 2 rows
     // (16.4 us) where the batched-decode kernel (15.4 us) does not take the shape
     if (f.packed_k != 0) return rows <= 2 && gemv_serves_k_major(f, rows) && !use_resident(f, rows);
-    return rows <= 4 && !use_resident(f, rows);
+    // W8: 3 and 4 rows go to the streaming kernel (N = 5120, K = 17408: 25.9 us there against 32.2 us here)
+    return rows <= (f.flags == kW8 ? 2 : 4) && !use_resident(f, rows);
 }
 
 // weight-streaming kernel for up to 64 rows.  Two-stage codes of 65..128 rows go to the 128x128
@@ -590,8 +591,12 @@ int split_groups() {
 }
 bool use_split(const orx_function& f, int rows) {
     if (f.partials == nullptr || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
-    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows) || use_big(f, rows) || pick_bm(rows) != 128) return false;
+    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows) || use_big(f, rows)) return false;
     const int64_t tiles = (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
+    // 17-64 rows: the 32- and 64-row tiles give one workgroup per 128 channels, which leaves most CUs
+    // idle when N is small and K long (W8, N = 5120, K = 17408: 112 us at 32 rows as 40 whole tiles)
+    // (with 136 such tiles, N = 17408, the whole 32-row tiles win: 39.7 against 43.1 us)
+    if (pick_bm(rows) != 128 && tiles >= split_groups() / 8) return false;
     // Measured at K = 5120 with N = 5120, 7168 and 17408: 40-272 tiles gain 10-40 % (two-stage codes
     // 59 -> 44 us at 136 tiles, 53 -> 32 us at 80), 408 tiles lose; a handful of tiles is latency, not
     // balance, and two launches would only add to it.
@@ -798,7 +803,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         int devices = 0;
         const bool split = v.boolean("split_k", true, &bad);  // diagnostic: false keeps whole tiles
         if (bad) return ORX_ERR_BAD_VARIANT;
-        if (split && f->capacity > 64 && f->tiles == 0 && (f->algorithm == kAuto || f->algorithm == kMfma) &&
+        if (split && f->capacity > 16 && f->tiles == 0 && (f->algorithm == kAuto || f->algorithm == kMfma) &&
             hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
             if (hipMalloc(&f->partials, (size_t)split_groups() * 2 * kSplitSlotInts * sizeof(int)) != hipSuccess)
                 f->partials = nullptr, (void)hipGetLastError();

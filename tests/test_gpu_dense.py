@@ -376,7 +376,8 @@ def test_q4_fp16_input_is_refused_where_no_kernel_serves_it():
 
 @pytest.mark.parametrize("codec,m,n,k,dtype", [("q4", 128, 8704, 512, "float16"), ("q4", 70, 8300, 384, "float16"),
                                                ("w8", 128, 8704, 256, "float16"), ("w8", 300, 8450, 384, "float32"),
-                                               ("q4", 256, 17408, 256, "float16")])
+                                               ("q4", 256, 17408, 256, "float16"), ("w8", 40, 2048, 1024, "float16"),
+                                               ("w8", 17, 5120, 512, "float32")])
 def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
     """65-384 rows on the 128-row tiles: the K steps of the tiles are dealt evenly to one workgroup per
     CU, runs that do not cover a whole tile meet as int32 partial sums.  Same bytes as whole tiles."""
