@@ -562,8 +562,9 @@ bool use_resident(const orx_function& f, int rows) {
 // (from 385 rows: up to 384 the 128x128 tiles measure 73..77 us for two-stage codes at N=17408,
 // K=5120 against 86..93 us for decode-once + 256x256, and 54..60 us against 58..62 us for W8; at 512
 // rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
+bool split_preferred_to_big(const orx_function& f, int rows);
 bool use_big(const orx_function& f, int rows) {
-    return f.tiles == 256 || (f.tiles == 0 && rows > 384);
+    return f.tiles == 256 || (f.tiles == 0 && rows > 384 && !split_preferred_to_big(f, rows));
 }
 
 // Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel
@@ -589,23 +590,43 @@ int split_groups() {
     }
     return groups;
 }
-bool use_split(const orx_function& f, int rows) {
+// 128-row tiles of this launch, and whether their count suits a split launch: measured at K = 5120
+// with N = 5120, 7168 and 17408, 40-272 tiles gain 10-40 % (two-stage codes 59 -> 44 us at 136 tiles,
+// 53 -> 32 us at 80), 408 tiles lose; a handful of tiles is latency, not balance, and two launches would
+// only add to it; tiles that divide evenly over the CUs are balanced as they are.
+int64_t split_tiles(const orx_function& f, int rows) {
+    return (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
+}
+bool split_shape_ok(const orx_function& f, int rows) {
     if (f.partials == nullptr || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
-    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows) || use_big(f, rows)) return false;
-    const int64_t tiles = (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
-    // 17-64 rows: the 32- and 64-row tiles give one workgroup per 128 channels, which leaves most CUs
-    // idle when N is small and K long (W8, N = 5120, K = 17408: 112 us at 32 rows as 40 whole tiles)
-    // (with 136 such tiles, N = 17408, the whole 32-row tiles win: 39.7 against 43.1 us)
-    if (pick_bm(rows) != 128 && tiles >= split_groups() / 8) return false;
-    // Measured at K = 5120 with N = 5120, 7168 and 17408: 40-272 tiles gain 10-40 % (two-stage codes
-    // 59 -> 44 us at 136 tiles, 53 -> 32 us at 80), 408 tiles lose; a handful of tiles is latency, not
-    // balance, and two launches would only add to it.
+    const int64_t tiles = split_tiles(f, rows);
     return tiles >= 8 && tiles <= (int64_t)split_groups() * 9 / 16 && tiles % (split_groups() / 2) != 0;
+}
+// Above 384 rows the 256 x 256 kernel is the default, but with fewer such tiles than half the CUs it
+// leaves most of the chip idle (W8, N = 5120, K = 17408 at 512 rows: 40 tiles, 209 us; N = K = 4096:
+// 32 tiles, 48 us against 29 us at 384 rows): the split 128-row tiles take those launches.
+bool split_preferred_to_big(const orx_function& f, int rows) {
+    const int64_t big_tiles = (int64_t)ceil_div((uint32_t)f.N, 256u) * ceil_div((uint32_t)rows, 256u);
+    return big_tiles < split_groups() / 4 && split_shape_ok(f, rows);
+}
+bool use_split(const orx_function& f, int rows) {
+    if (!split_shape_ok(f, rows)) return false;
+    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows) || use_big(f, rows)) return false;
+    // 17-64 rows: the 32- and 64-row tiles give one workgroup per 128 channels, which leaves most CUs
+    // idle when N is small and K long (W8, N = 5120, K = 17408: 112 us at 32 rows as 40 whole tiles);
+    // with 136 such tiles (N = 17408) the whole 32-row tiles win, 39.7 against 43.1 us
+    if (pick_bm(rows) != 128 && split_tiles(f, rows) >= split_groups() / 8) return false;
+    return true;
+}
+// Workgroups of a split launch: two per CU, but at least 8 K steps each, so that the partial tiles
+// (64 KiB per run) stay small beside the operands a workgroup reads (32 KiB per K step).
+int split_groups_for(const orx_function& f, int rows) {
+    const int64_t units = split_tiles(f, rows) * (f.K / kBK);
+    return (int)std::max<int64_t>(1, std::min<int64_t>(split_groups(), units / 8));
 }
 
 template <int CODEC>
-int launch_split(const GemmParams& p, hipStream_t stream) {
-    const int groups = split_groups();
+int launch_split(const GemmParams& p, int groups, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_split_kernel<CODEC>), dim3(groups), dim3(256), 0, stream, p);
     int code = hip_check(hipGetLastError(), "launch projection (mfma, split K steps)");
     if (code != ORX_OK) return code;
@@ -629,7 +650,7 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (use_split(f, rows)) {
-        g->grid[0] = (uint32_t)split_groups();
+        g->grid[0] = (uint32_t)split_groups_for(f, rows);
         g->block[0] = 256;
         g->shared = 0;
         return ORX_OK;
@@ -685,7 +706,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
                                f.out_f32, g, stream);
     if (use_split(f, rows)) {
         p.partials = static_cast<int*>(f.partials);
-        return launch_split<kQ4>(p, stream);
+        return launch_split<kQ4>(p, split_groups_for(f, rows), stream);
     }
     return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
@@ -716,7 +737,7 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
                                stream);
     if (use_split(f, rows)) {
         p.partials = static_cast<int*>(f.partials);
-        return launch_split<kW8>(p, stream);
+        return launch_split<kW8>(p, split_groups_for(f, rows), stream);
     }
     return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
 }
