@@ -543,7 +543,12 @@ bool use_gemv(const orx_function& f, int rows) {
 // 16 rows: the 32/64/128-row tiles measure 27 / 31 / 40 us at 32 / 48 / 128 rows against 29 / 43 / 94.
 bool use_stream(const orx_function& f, int rows) {
     if (f.algorithm == kStream) return rows <= 64;
-    return f.algorithm == kAuto && f.tiles == 0 && rows <= (f.flags == kQ4 ? 64 : 16);
+    if (f.algorithm != kAuto || f.tiles != 0) return false;
+    if (f.flags == kQ4) return rows <= 64;
+    // W8 with weights that do not stay in cache: up to 32 rows (N = 17408, K = 5120 at 32 rows: 34.8 us
+    // against 39.0 us for the 32-row tiles; at 48 rows 49.0 against 42.5), up to 64 rows for matrices of
+    // at most 32 M weights (N = K = 4096 at 64 rows: 14.7 against 19.5 us)
+    return rows <= 32 || (rows <= 64 && (int64_t)f.N * f.K <= (int64_t)1 << 25);
 }
 
 // Resident two-stage kernel (32 rows per launch) where the streaming kernel would run and the shape
@@ -555,7 +560,10 @@ bool use_resident(const orx_function& f, int rows) {
     // rows of N=17408, K=5120), this kernel's MFMAs do not (15.6 us from 2 to 16 rows)
     // up to 64 rows as two launches of 32 (36 and 39 us at 48 and 64 rows against 42 and 48 us for
     // the streaming kernel)
-    return f.algorithm == kAuto && f.tiles == 0 && rows > 1 && rows <= 64;
+    // (the second launch pays for itself only on large matrices: N = 17408, K = 5120 at 48 rows 33 us
+    // against 39 us for the streaming kernel, but N = K = 5120 20 against 14.5 us)
+    const int limit = (int64_t)f.N * f.K >= ((int64_t)1 << 26) ? 64 : 32;
+    return f.algorithm == kAuto && f.tiles == 0 && rows > 1 && rows <= limit;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
