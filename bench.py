@@ -26,8 +26,8 @@ CACHE_BYTES = 256 << 20        # Infinity Cache
 # `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
 # same counter reads for a device copy of 44 564 480 bytes in the same run: FETCH_SIZE reads
 # 21 772.3 for 43 520 KiB (factor 1.9989), WRITE_SIZE reads 43 520.0 (factor 1.0).
-# Kernel (fp16-input GEMV): fetch 22 042.4 -> 45 117 341 B, write 272.0 -> 278 560 B.
-MEASURED_TRAFFIC_BYTES = 45_395_901
+# Kernel (fp16-input GEMV): fetch 22 042.5 -> 45 117 455 B  write 272.0 -> 278 560 B.
+MEASURED_TRAFFIC_BYTES = 45_396_015
 
 
 def parse():
