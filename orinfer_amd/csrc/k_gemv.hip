@@ -442,10 +442,13 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
         // row maximum: per thread, per wave, then over the 16 waves through LDS (one more barrier)
         float* wave_max = reinterpret_cast<float*>(wave_sums + 3 * 16);  // the fourth row of sums is unused with one row
         const __half* h = reinterpret_cast<const __half*>(&raw_x16);
+        // Waves past the end of the row (K / 8 pieces, one per thread) skip the per-value work: with
+        // four waves per SIMD in the same phase, their instructions would take issue slots from the rest.
+        const bool wave_live = __builtin_amdgcn_readfirstlane(wave) * 64 < groups;
         float value[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) value[j] = __half2float(h[j]);
-        if (signs != nullptr) {
+        for (int j = 0; j < 8; ++j) value[j] = wave_live ? __half2float(h[j]) : 0.f;
+        if (signs != nullptr && wave_live) {
             // Signed block-128 rotation in front of the quantiser (kernels/cuda/model/rotation_a8.py:188-224):
             // a block is the 8 values of each of 16 adjacent threads, so distances 1, 2 and 4 are inside
             // the thread and 8..64 are lane exchanges at distance 1..8 inside a row of 16 lanes.  Every
@@ -499,33 +502,39 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
         if (lane == 0) wave_max[wave] = amax;
         prefetch(0, 1);  // the row has arrived: the stream can start while the row is quantised
         __syncthreads();
+        // the 16 wave maxima, one per lane of a row, reduced with lane controls (no LDS round trips):
+        // quad permutes, then the mirror of each half row, then the mirror of the row
         amax = wave_max[lane & 15];
-#pragma unroll
-        for (int offset = 8; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+        amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0xB1, 0xF, 0xF, true)));
+        amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0x4E, 0xF, 0xF, true)));
+        amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0x141, 0xF, 0xF, true)));
+        amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(amax), 0x140, 0xF, 0xF, true)));
         const float raw_scale = fmaxf(__fdiv_rn(amax, 127.0f), 5.9604644775390625e-08f);
         const __half stored = amax > 0.f ? __float2half_rn(raw_scale) : __float2half_rn(1.0f);
         as_bits[0] = __half_as_ushort(stored);
         if (blockIdx.x == 0 && tid == 0) *const_cast<__half*>(as) = stored;
         const float scale = __half2float(stored);
-        const float inverse = __frcp_rn(scale);
+        const float inverse = __builtin_amdgcn_rcpf(scale);  // within one unit in the last place: inside the margin below
         // the product with the reciprocal decides, except within 2^-14 of a tie, where the correctly
         // rounded quotient does (the product is within 2^-15 of the quotient)
-        float r[8];
-        float nearest = 1.0f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float guess = value[j] * inverse;
-            r[j] = rintf(guess);
-            nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
-        }
-        if (nearest < 6.103515625e-05f) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
-        }
         uint32_t packed[2] = {0u, 0u};
+        if (wave_live) {
+            float r[8];
+            float nearest = 1.0f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            packed[j >> 2] |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * (j & 3));
+            for (int j = 0; j < 8; ++j) {
+                const float guess = value[j] * inverse;
+                r[j] = rintf(guess);
+                nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
+            }
+            if (nearest < 6.103515625e-05f) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                packed[j >> 2] |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * (j & 3));
+        }
         raw[0] = make_uint2(packed[0], packed[1]);
     }
     int wave_total[MR];  // sum of this wave's activations, valid in lane 63
