@@ -298,6 +298,17 @@ def main():
             single[name] = {"us": round(t * 1e6, 2), "GBps_codes": round(moved / t / 1e9, 1)}
             del bank
         extra["config3_single_token_routes"] = single
+        # the whole layer for one token: direct bank indexing against the token-sorted program
+        token_layer = programs.MoeTokenLayer(e3, k3, h3, i3, c3["gate_up"], c3["gate_up_scales"], c3["down"],
+                                             c3["down_scales"])
+        sorted_layer = programs.MoeLayer(1, e3, k3, h3, i3, c3["gate_up"], c3["gate_up_scales"], c3["down"],
+                                         c3["down_scales"], block_m=32)
+        x1, l1 = x3[:1].contiguous(), l3[:1].contiguous()
+        t_direct = timed_graph(lambda i, s: token_layer.run(x1, l1, stream=s), 20)
+        t_sorted = timed_graph(lambda i, s: sorted_layer.run(x1, l1, stream=s), 20)
+        extra["config3_single_token_layer"] = {"direct_routes_us": round(t_direct * 1e6, 2),
+                                               "token_sorted_us": round(t_sorted * 1e6, 2)}
+        del token_layer, sorted_layer
         torch.cuda.empty_cache()
         # config 4 layer linears
         c4 = workloads.config4()

@@ -160,3 +160,50 @@ class MoeLayer:
         self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
                        SlotMap=self.slot_map)
         return self.out
+
+
+class MoeTokenLayer:
+    """The same expert layer for ONE token: its routes index the expert banks directly
+    (kernels/cuda/model/integer_vq.py:380-444), so there is no sorting, no tile list and no dispatch copy:
+    router top-k, A8 of the row, gate/up of every route from the shared row, SwiGLU->A8 per route,
+    down per route, weighted combine."""
+
+    def __init__(self, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales):
+        self.experts, self.top_k, self.hidden, self.inter = experts, top_k, hidden, intermediate
+        self.w1 = _dev(codebook.q2_to_k_major(np.asarray(gate_up)))
+        self.w2 = _dev(codebook.q2_to_k_major(np.asarray(down)))
+        self.s1, self.s2 = _dev(gate_up_scales), _dev(down_scales)
+        self.book = _dev(codebook.raw_book())
+        f16 = dict(dtype=torch.float16, device="cuda")
+        i8 = dict(dtype=torch.int8, device="cuda")
+        self.ids = torch.empty((1, top_k), dtype=torch.int32, device="cuda")
+        self.prob = torch.empty((1, top_k), dtype=torch.float32, device="cuda")
+        self.a_q = torch.empty((1, hidden), **i8)
+        self.a_s = torch.empty((1, 1), **f16)
+        self.gate_up_out = torch.empty((top_k, 2 * intermediate), **f16)
+        self.h_q = torch.empty((top_k, intermediate), **i8)
+        self.h_s = torch.empty((top_k, 1), **f16)
+        self.down_out = torch.empty((top_k, hidden), **f16)
+        self.slot_map = torch.arange(top_k, dtype=torch.int32, device="cuda").view(1, top_k)  # route r is slot r
+        self.out = torch.empty((1, hidden), **f16)
+        common = dict(M=1, E=experts, top_k=top_k)
+        self.k_router = Kernel("router_topk", renormalize=True, **common)
+        self.k_a8 = Kernel("activation_quantization", K=hidden)
+        self.k_gate_up = Kernel("integer_e8p_gemv", E=experts, routes=top_k, N=2 * intermediate, K=hidden,
+                                shared_input=True)
+        self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
+        self.k_down = Kernel("integer_e8p_gemv", E=experts, routes=top_k, N=hidden, K=intermediate, shared_input=False)
+        self.k_combine = Kernel("moe_combine", H=hidden, slots=top_k, **common)
+
+    def run(self, x16, logits, stream=None):
+        s = stream
+        self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
+        self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=1)
+        self.k_gate_up(stream=s, A=self.a_q, AS=self.a_s, Book=self.book, C=self.gate_up_out, IDs=self.ids, P=self.w1,
+                       WS=self.s1)
+        self.k_swiglu_a8(stream=s, Mask=None, Q=self.h_q, S=self.h_s, X=self.gate_up_out, rows=self.top_k)
+        self.k_down(stream=s, A=self.h_q, AS=self.h_s, Book=self.book, C=self.down_out, IDs=self.ids, P=self.w2,
+                    WS=self.s2)
+        self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
+                       SlotMap=self.slot_map)
+        return self.out

@@ -640,3 +640,47 @@ def test_expert_dispatch_quantises_fp16_rows(m, e, k, h):
     for variant in (dict(H=h, scale_group=h // 2), dict(H=36)):
         with pytest.raises(Exception):
             gu.kernel("expert_dispatch", M=m, E=e, top_k=k, input_dtype="float16", **variant)
+
+
+def test_moe_token_layer_matches_the_routed_layer_of_one_token():
+    """One token through direct bank indexing gives what the token-sorted layer gives for it."""
+    c = workloads.config3(tokens=1, experts=32, top_k=4, hidden=512, intermediate=256)
+    layer = programs.MoeTokenLayer(c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
+                                   c["gate_up_scales"], c["down"], c["down_scales"])
+    x, logits = gu.dev(c["x"]), gu.dev(c["logits"])
+    layer.run(x, logits)
+    gu.sync()
+    ids, prob = orc.router_topk(c["logits"], c["top_k"], True)
+    np.testing.assert_array_equal(gu.host(layer.ids), ids)
+    a_q, a_s = orc.a8(c["x"])
+    w1 = np.stack([orc.q2_integers(m, TABLE) for m in c["gate_up"]])
+    w2 = np.stack([orc.q2_integers(m, TABLE) for m in c["down"]])
+    gate_up = orc.route_project(a_q, a_s[:, 0], w1, c["gate_up_scales"], ids, True)
+    np.testing.assert_array_equal(gu.host(layer.gate_up_out), gate_up)
+    # SwiGLU uses exp(): from here each stage is checked on the GPU's own input
+    h_q, h_s = gu.host(layer.h_q), gu.host(layer.h_s)
+    want_q, want_s = orc.a8(orc.swiglu_fp16(gate_up))
+    assert (h_q == want_q).mean() > 0.999
+    down = orc.route_project(h_q, h_s[:, 0], w2, c["down_scales"], ids, False)
+    np.testing.assert_array_equal(gu.host(layer.down_out), down)
+    staged = orc.moe_combine(down, np.arange(c["top_k"], dtype=np.int32)[None, :], gu.host(layer.prob)).astype(np.float32)
+    got = gu.host(layer.out).astype(np.float32)
+    assert (np.abs(got - staged) <= 1e-2 + 1e-3 * np.abs(staged)).all()
+    # and the token-sorted program on the same token
+    sorted_layer = run_layer(c, 32)
+    assert torch.equal(sorted_layer.out, layer.out)
+    # graph replay with another token
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            layer.run(x, logits, stream=stream.cuda_stream)
+    rng = np.random.default_rng(9)
+    logits.copy_(gu.dev(rng.normal(size=c["logits"].shape).astype(np.float32)))
+    x.copy_(gu.dev(rng.normal(size=c["x"].shape).astype(np.float16)))
+    graph.replay()
+    gu.sync()
+    replayed = layer.out.clone()
+    layer.run(x, logits)
+    gu.sync()
+    assert torch.equal(layer.out, replayed)
