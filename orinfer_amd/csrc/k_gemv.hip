@@ -18,6 +18,7 @@
 // scratch memory, no host reads.
 #include <hip/hip_fp16.h>
 
+#include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -856,8 +857,9 @@ constexpr int kRouteTableBytes = 256 * 16, kRouteMaskBytes = 256 * 8, kRoutePart
 __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
     const int8_t* __restrict__ a, const __half* __restrict__ as, const uint32_t* __restrict__ book, __half* __restrict__ c,
     const int32_t* __restrict__ ids, const uint16_t* __restrict__ p, const __half* __restrict__ ws, int experts, int n,
-    int k, int shared_input) {
+    int k, int shared_input, int x16) {
     extern __shared__ __align__(16) uint8_t route_lds[];
+    __shared__ float route_wave_max[kRouteWaves];
     uint4* table = reinterpret_cast<uint4*>(route_lds);                                    // entry, negated entry
     uint2* masks = reinterpret_cast<uint2*>(route_lds + kRouteTableBytes);                  // per u
     int* partial = reinterpret_cast<int*>(route_lds + kRouteTableBytes + kRouteMaskBytes);  // [waves][channels]
@@ -891,10 +893,55 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
         const uint32_t signs = u ^ (__popc(u) & 1u);
         masks[u] = make_uint2(sign_mask(signs), sign_mask(signs >> 2));
     }
-    for (int i = tid; i < k / 8; i += kRouteThreads) {
-        const uint2 bytes = reinterpret_cast<const uint2*>(a + (int64_t)row * k)[i];
-        reinterpret_cast<uint2*>(token)[i] = bytes;
-        token_sums[i] = __builtin_amdgcn_sdot4((int)bytes.y, 0x01010101, __builtin_amdgcn_sdot4((int)bytes.x, 0x01010101, 0, false), false);
+    float row_scale = 0.f;  // x16: fp32 value of the row's fp16 scale
+    if (x16) {
+        // `a` is the shared fp16 row: every workgroup quantises it by the A8 rule (row maximum over 127,
+        // fp16 scale, round to nearest even) on its way into LDS; the first one also writes the scale.
+        // Up to 4 pieces of 8 values per thread (K <= 16384) stay in registers between the two passes.
+        const __half* x = reinterpret_cast<const __half*>(a);
+        uint4 kept[4];
+        float amax = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + j * kRouteThreads;
+            kept[j] = make_uint4(0u, 0u, 0u, 0u);
+            if (i < k / 8) kept[j] = reinterpret_cast<const uint4*>(x)[i];
+            const __half2* pairs = reinterpret_cast<const __half2*>(&kept[j]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float2 f = __half22float2(pairs[e]);
+                amax = fmaxf(amax, fmaxf(fabsf(f.x), fabsf(f.y)));
+            }
+        }
+#pragma unroll
+        for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+        if (lane == 0) route_wave_max[wave] = amax;
+        __syncthreads();
+        amax = route_wave_max[0];
+#pragma unroll
+        for (int w = 1; w < kRouteWaves; ++w) amax = fmaxf(amax, route_wave_max[w]);
+        const __half stored = a8_scale(amax);
+        if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *const_cast<__half*>(as) = stored;
+        row_scale = __half2float(stored);
+        const float inverse = __builtin_amdgcn_rcpf(row_scale);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int i = tid + j * kRouteThreads;
+            if (i < k / 8) {
+                const __half* h = reinterpret_cast<const __half*>(&kept[j]);
+                const float low[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+                const float high[4] = {__half2float(h[4]), __half2float(h[5]), __half2float(h[6]), __half2float(h[7])};
+                const uint2 bytes = make_uint2(quantise4(low, row_scale, inverse), quantise4(high, row_scale, inverse));
+                reinterpret_cast<uint2*>(token)[i] = bytes;
+                token_sums[i] = __builtin_amdgcn_sdot4((int)bytes.y, 0x01010101, __builtin_amdgcn_sdot4((int)bytes.x, 0x01010101, 0, false), false);
+            }
+        }
+    } else {
+        for (int i = tid; i < k / 8; i += kRouteThreads) {
+            const uint2 bytes = reinterpret_cast<const uint2*>(a + (int64_t)row * k)[i];
+            reinterpret_cast<uint2*>(token)[i] = bytes;
+            token_sums[i] = __builtin_amdgcn_sdot4((int)bytes.y, 0x01010101, __builtin_amdgcn_sdot4((int)bytes.x, 0x01010101, 0, false), false);
+        }
     }
     __syncthreads();
     int acc = 0;
@@ -939,7 +986,8 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
             int total = 0;
 #pragma unroll
             for (int w = 0; w < kRouteWaves; ++w) total += partial[w * kRouteChannels + tid];
-            const float scaled = ((float)total * __half2float(ws[(int64_t)expert * n + out_channel])) * __half2float(as[row]);
+            const float token_scale = x16 ? row_scale : __half2float(as[row]);
+            const float scaled = ((float)total * __half2float(ws[(int64_t)expert * n + out_channel])) * token_scale;
             c[(int64_t)route * n + out_channel] = __float2half_rn(scaled);
         }
     }
@@ -966,7 +1014,7 @@ int route_gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStr
     const uint16_t* p = pointer_arg<const uint16_t>(args, 5);
     const __half* ws = pointer_arg<const __half>(args, 6);
     hipLaunchKernelGGL(route_gemv_kernel, dim3(g.grid[0], g.grid[1]), dim3(kRouteThreads), g.shared, stream, a, as, book, c, ids, p,
-                       ws, f.E, f.N, f.K, f.flags & 1);
+                       ws, f.E, f.N, f.K, f.flags & 1, f.input_f16 ? 1 : 0);
     return hip_check(hipGetLastError(), "launch integer_e8p_gemv");
 }
 
@@ -989,6 +1037,14 @@ int make_route_gemv(const Variant& v, orx_function* f) {
         return ORX_ERR_BAD_VARIANT;
     }
     f->flags = shared_input ? 1 : 0;
+    // input_dtype=float16 (shared row only): A is the fp16 row, quantised by every workgroup on its way into
+    // LDS; AS is written, not read
+    const std::string input = v.string("input_dtype", "int8", &bad);
+    if (bad || (input != "int8" && input != "float16") || (input == "float16" && (!shared_input || f->K > 16384))) {
+        set_error("integer_e8p_gemv: input_dtype must be int8 or float16 (float16: shared_input, K up to 16384)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->input_f16 = input == "float16";
     // 16-byte loads of A rows and P, 8-byte loads of Book
     f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 8}, {"C", ArgPointer, 2},
                {"IDs", ArgPointer, 4}, {"P", ArgPointer, 16}, {"WS", ArgPointer, 2}};
@@ -1121,7 +1177,7 @@ int gemv_prepare_device() {
 
 const Registration* gemv_registrations(int* count) {
     static const Registration rows[] = {
-    {"integer_e8p_gemv", make_route_gemv, "E, routes, N, K, shared_input, block_n=8", "A,AS,Book,C,IDs,P,WS"},
+    {"integer_e8p_gemv", make_route_gemv, "E, routes, N, K, shared_input, block_n=8, input_dtype=int8|float16", "A,AS,Book,C,IDs,P,WS"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;

@@ -165,7 +165,7 @@ class MoeLayer:
 class MoeTokenLayer:
     """The same expert layer for ONE token: its routes index the expert banks directly
     (kernels/cuda/model/integer_vq.py:380-444), so there is no sorting, no tile list and no dispatch copy:
-    router top-k, A8 of the row, gate/up of every route from the shared row, SwiGLU->A8 per route,
+    router top-k, gate/up of every route from the shared row (quantised on the way), SwiGLU->A8 per route,
     down per route, weighted combine."""
 
     def __init__(self, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales):
@@ -178,7 +178,6 @@ class MoeTokenLayer:
         i8 = dict(dtype=torch.int8, device="cuda")
         self.ids = torch.empty((1, top_k), dtype=torch.int32, device="cuda")
         self.prob = torch.empty((1, top_k), dtype=torch.float32, device="cuda")
-        self.a_q = torch.empty((1, hidden), **i8)
         self.a_s = torch.empty((1, 1), **f16)
         self.gate_up_out = torch.empty((top_k, 2 * intermediate), **f16)
         self.h_q = torch.empty((top_k, intermediate), **i8)
@@ -188,9 +187,9 @@ class MoeTokenLayer:
         self.out = torch.empty((1, hidden), **f16)
         common = dict(M=1, E=experts, top_k=top_k)
         self.k_router = Kernel("router_topk", renormalize=True, **common)
-        self.k_a8 = Kernel("activation_quantization", K=hidden)
+        # gate/up quantises the shared fp16 row itself (no launch for the A8 of one row)
         self.k_gate_up = Kernel("integer_e8p_gemv", E=experts, routes=top_k, N=2 * intermediate, K=hidden,
-                                shared_input=True)
+                                shared_input=True, input_dtype="float16")
         self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
         self.k_down = Kernel("integer_e8p_gemv", E=experts, routes=top_k, N=hidden, K=intermediate, shared_input=False)
         self.k_combine = Kernel("moe_combine", H=hidden, slots=top_k, **common)
@@ -198,8 +197,7 @@ class MoeTokenLayer:
     def run(self, x16, logits, stream=None):
         s = stream
         self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
-        self.k_a8(stream=s, Mask=None, Q=self.a_q, S=self.a_s, X=x16, rows=1)
-        self.k_gate_up(stream=s, A=self.a_q, AS=self.a_s, Book=self.book, C=self.gate_up_out, IDs=self.ids, P=self.w1,
+        self.k_gate_up(stream=s, A=x16, AS=self.a_s, Book=self.book, C=self.gate_up_out, IDs=self.ids, P=self.w1,
                        WS=self.s1)
         self.k_swiglu_a8(stream=s, Mask=None, Q=self.h_q, S=self.h_s, X=self.gate_up_out, rows=self.top_k)
         self.k_down(stream=s, A=self.h_q, AS=self.h_s, Book=self.book, C=self.down_out, IDs=self.ids, P=self.w2,

@@ -447,6 +447,32 @@ def test_route_gemv_production_table_and_repeated_experts(n, k, shared):
     np.testing.assert_array_equal(got[keep], want[keep])
 
 
+def test_route_gemv_quantises_a_shared_fp16_row():
+    rng = np.random.default_rng(orc.SEED + 55)
+    e, routes, n, k = 16, 4, 200, 2304
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    weights = np.stack([orc.q2_integers(c, TABLE) for c in codes])
+    stored = gu.dev(np.stack([orc.q2_pack_k128(c) for c in codes]))
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    ids = np.array([[3, 15, 0, 3]], np.int32)
+    kern = gu.kernel("integer_e8p_gemv", E=e, routes=routes, N=n, K=k, shared_input=True, input_dtype="float16")
+    out = torch.full((routes + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    scale = torch.full((2,), 5.0, dtype=torch.float16, device=gu.DEV)
+    for case in range(3):
+        x = rng.normal(size=(1, k)).astype(np.float16)
+        if case == 1:
+            x[0, :3] = [700, -700, 1e-7]
+        if case == 2:
+            x[:] = 0
+        kern(A=gu.dev(x), AS=scale, Book=gu.dev(orc.raw_table_words(TABLE)), C=out, IDs=gu.dev(ids), P=stored, WS=gu.dev(ws))
+        a_q, a_s = orc.a8(x)
+        np.testing.assert_array_equal(gu.host(scale)[:1], a_s[:, 0])
+        np.testing.assert_array_equal(gu.host(out)[:routes], orc.route_project(a_q, a_s[:, 0], weights, ws, ids, True))
+        assert float(gu.host(scale)[1]) == 5.0 and (gu.host(out)[routes] == 91).all()
+    with pytest.raises(Exception):
+        gu.kernel("integer_e8p_gemv", E=e, routes=routes, N=n, K=k, shared_input=False, input_dtype="float16")
+
+
 def test_route_gemv_refuses_bad_variants():
     for variant in (dict(E=4, routes=2, N=64, K=192, shared_input=True),
                     dict(E=4, routes=2, N=64, K=256),
@@ -656,6 +682,7 @@ def test_moe_token_layer_matches_the_routed_layer_of_one_token():
     w1 = np.stack([orc.q2_integers(m, TABLE) for m in c["gate_up"]])
     w2 = np.stack([orc.q2_integers(m, TABLE) for m in c["down"]])
     gate_up = orc.route_project(a_q, a_s[:, 0], w1, c["gate_up_scales"], ids, True)
+    np.testing.assert_array_equal(gu.host(layer.a_s), a_s)
     np.testing.assert_array_equal(gu.host(layer.gate_up_out), gate_up)
     # SwiGLU uses exp(): from here each stage is checked on the GPU's own input
     h_q, h_s = gu.host(layer.h_q), gu.host(layer.h_s)
