@@ -26,23 +26,29 @@ __device__ __forceinline__ int8_t quantise(float value, float scale, float inver
 }
 
 // Four codes packed into one word; one test (and, rarely, four exact quotients) for the four.
+// A product's distance from its rounded value is at most 0.5, so "within 2^-14 of a tie" is
+// "farther than 0.5 - 2^-14 from the rounded value".  The clamped integer plus 1.5 * 2^23 has the
+// integer in its low mantissa bits in two's complement: the low byte of that word is the int8 code.
 __device__ __forceinline__ uint32_t quantise4(const float (&value)[4], float scale, float inverse) {
     float r[4];
-    float nearest = 1.0f;  // smallest distance of a product from a tie
+    float farthest = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const float guess = value[j] * inverse;
         r[j] = rintf(guess);
-        nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
+        farthest = fmaxf(farthest, fabsf(guess - r[j]));
     }
-    if (nearest < 6.103515625e-05f) {
+    if (farthest > 0.49993896484375f) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
     }
-    uint32_t packed = 0;
+    uint32_t word[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) packed |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * j);
-    return packed;
+    for (int j = 0; j < 4; ++j) word[j] = __float_as_uint(__builtin_amdgcn_fmed3f(r[j], -127.f, 127.f) + 12582912.0f);
+    // byte 0 of the first operand's partner (second argument), then byte 0 of the first argument
+    const uint32_t low = __builtin_amdgcn_perm(word[1], word[0], 0x0C0C0400u);
+    const uint32_t high = __builtin_amdgcn_perm(word[3], word[2], 0x0C0C0400u);
+    return low | (high << 16);
 }
 
 }  // namespace orx

@@ -71,6 +71,8 @@ __global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ 
     const bool vector = !FUSED && !MASKED && (k % 8 == 0) && (group % 8 == 0) &&
                         ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 7) == 0);
     float amax = 0.f;
+    typedef _Float16 half_pair __attribute__((ext_vector_type(2)));
+    half_pair amax2 = {(_Float16)0.f, (_Float16)0.f};  // largest magnitudes so far as two fp16 lanes: comparing needs no conversion
     // a group of at most one 16-byte piece per thread stays in registers between the two passes
     // (only in the 16-wave form: carrying the piece through the loops costs the 4-wave form its
     // overlap of loads, 28 -> 48 us at 8192 x 5120)
@@ -81,13 +83,12 @@ __global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ 
         for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
             const uint4 raw = src[i];
             if (THREADS == 1024) kept = raw;
-            const __half2* h = reinterpret_cast<const __half2*>(&raw);
+            const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float2 f = __half22float2(h[j]);
-                amax = fmaxf(amax, fmaxf(fabsf(f.x), fabsf(f.y)));
-            }
+            for (int j = 0; j < 4; ++j)
+                amax2 = __builtin_elementwise_max(amax2, __builtin_bit_cast(half_pair, words[j] & 0x7FFF7FFFu));
         }
+        amax = fmaxf((float)amax2[0], (float)amax2[1]);
     } else {
         for (int i = threadIdx.x; i < width; i += blockDim.x)
             amax = fmaxf(amax, fabsf(load_value<FUSED, MASKED>(x, mask, in_base, k, first + i)));
