@@ -521,20 +521,25 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
         uint32_t packed[2] = {0u, 0u};
         if (wave_live) {
             float r[8];
-            float nearest = 1.0f;
+            float farthest = 0.f;  // a product is at most 0.5 from its rounded value: 0.5 at a tie
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float guess = value[j] * inverse;
                 r[j] = rintf(guess);
-                nearest = fminf(nearest, fabsf(fabsf(guess - r[j]) - 0.5f));
+                farthest = fmaxf(farthest, fabsf(guess - r[j]));
             }
-            if (nearest < 6.103515625e-05f) {
+            if (farthest > 0.49993896484375f) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) r[j] = rintf(__fdiv_rn(value[j], scale));
             }
+            // clamped integer + 1.5 * 2^23: the low byte of the word is the int8 code
+            uint32_t word[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
-                packed[j >> 2] |= ((uint32_t)(uint8_t)(int8_t)fmaxf(-127.f, fminf(127.f, r[j]))) << (8 * (j & 3));
+            for (int j = 0; j < 8; ++j) word[j] = __float_as_uint(__builtin_amdgcn_fmed3f(r[j], -127.f, 127.f) + 12582912.0f);
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+                packed[half] = __builtin_amdgcn_perm(word[4 * half + 1], word[4 * half], 0x0C0C0400u) |
+                               (__builtin_amdgcn_perm(word[4 * half + 3], word[4 * half + 2], 0x0C0C0400u) << 16);
         }
         raw[0] = make_uint2(packed[0], packed[1]);
     }
