@@ -56,11 +56,15 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
     return r;
 }
 
-// grid (rows, groups), 256 threads.
-template <bool FUSED, bool MASKED, int THREADS = 256>
+// grid (rows, groups), 256 threads.  STAGED (dynamic LDS of one group of fp16 values): a thread keeps
+// the 16-byte pieces it read for the maximum in LDS and quantises them from there.  With many rows
+// of long groups in flight the second read no longer hits the L2 cache (8192 rows of 17408: every
+// CU holds 8 rows of 34 KB), so it would cost HBM traffic a second time.
+template <bool FUSED, bool MASKED, int THREADS = 256, bool STAGED = false>
 __global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
                                                      int8_t* __restrict__ q, __half* __restrict__ s, int k, int group,
                                                      int groups) {
+    extern __shared__ __align__(16) uint4 staged[];
     __shared__ float scratch[THREADS / 64];
     const int row = blockIdx.x, g = blockIdx.y;
     const int first = g * group;
@@ -78,7 +82,27 @@ __global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ 
     // overlap of loads, 28 -> 48 us at 8192 x 5120)
     const bool held = THREADS == 1024 && vector && width / 8 <= THREADS;
     uint4 kept = make_uint4(0u, 0u, 0u, 0u);
-    if (vector) {
+    if (STAGED && vector) {
+        // four pieces per thread leave together (clamped, so unconditional): a long group would
+        // otherwise cost one load latency per piece
+        const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
+        const int pieces = width / 8;
+        for (int base = threadIdx.x; base < pieces; base += 4 * THREADS) {
+            uint4 raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) raw[u] = src[min(base + u * THREADS, pieces - 1)];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = base + u * THREADS;
+                if (i < pieces) staged[i] = raw[u];  // read back below by this thread only
+                const uint32_t words[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    amax2 = __builtin_elementwise_max(amax2, __builtin_bit_cast(half_pair, words[j] & 0x7FFF7FFFu));
+            }
+        }
+        amax = fmaxf((float)amax2[0], (float)amax2[1]);
+    } else if (vector) {
         const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
         for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
             const uint4 raw = src[i];
@@ -103,7 +127,7 @@ __global__ __launch_bounds__(THREADS) void a8_kernel(const __half* __restrict__ 
         const uint4* src = reinterpret_cast<const uint4*>(x + in_base + first);
         uint2* dst = reinterpret_cast<uint2*>(q + out_base + first);
         for (int i = threadIdx.x; i < width / 8; i += blockDim.x) {
-            const uint4 raw = held ? kept : src[i];
+            const uint4 raw = held ? kept : STAGED ? staged[i] : src[i];
             const __half* h = reinterpret_cast<const __half*>(&raw);
             const float low[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
             const float high[4] = {__half2float(h[4]), __half2float(h[5]), __half2float(h[6]), __half2float(h[7])};
@@ -459,6 +483,10 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const __half* __restrict__ 
 bool a8_wide(const orx_function& f, int rows) { return f.flags == 0 && rows <= 256 && f.group >= 4096; }
 // short groups, no mask: one wave per group
 bool a8_per_wave(const orx_function& f) { return !(f.flags & 1) && f.group <= 512; }
+// many rows of long groups: the pieces wait in LDS between the two passes (9 to 48 KiB per group: at least three of the four pieces a thread requests at once are real)
+bool a8_staged(const orx_function& f, int rows) {
+    return f.flags == 0 && !a8_wide(f, rows) && f.group % 8 == 0 && f.group >= 4608 && f.group <= 24576;
+}
 
 int a8_geometry(const orx_function& f, int rows, Geometry* g) {
     const uint32_t groups = ceil_div((uint32_t)f.K, (uint32_t)f.group);
@@ -470,6 +498,7 @@ int a8_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
     g->grid[1] = groups;
     g->block[0] = a8_wide(f, rows) ? 1024 : 256;
+    g->shared = a8_staged(f, rows) ? (uint32_t)f.group * 2u : 0u;
     return ORX_OK;
 }
 
@@ -488,6 +517,8 @@ int a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
             hipLaunchKernelGGL((a8_wave_kernel<false>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
     } else if (g.block[0] == 1024)
         hipLaunchKernelGGL((a8_kernel<false, false, 1024>), grid, dim3(1024), 0, stream, x, mask, q, s, f.K, f.group, groups);
+    else if (g.shared > 0)
+        hipLaunchKernelGGL((a8_kernel<false, false, 256, true>), grid, block, g.shared, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused && masked)
         hipLaunchKernelGGL((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused)

@@ -93,6 +93,20 @@ def test_a8_groups_and_odd_shapes(k, group):
     np.testing.assert_array_equal(gu.host(q), wq)
 
 
+@pytest.mark.parametrize("rows,k,group", [(300, 17408, 17408), (260, 16384, 8192), (259, 5120, 5120), (257, 24576, 24576), (258, 24584, 24584)])
+def test_a8_many_rows_of_long_groups(rows, k, group):
+    # above 256 rows, groups of 4608 to 24576 values wait in LDS between the maximum and the quantise
+    # pass; the last shape is just past that range and reads its input twice
+    rng = np.random.default_rng(orc.SEED + rows + k)
+    x = (rng.normal(size=(rows, k)) * 2).astype(np.float16)
+    x[1] = 0
+    x[2, -1] = 1000
+    q, s = gu.a8(gu.dev(x), group=group)
+    wq, ws = orc.a8(x, group)
+    np.testing.assert_array_equal(gu.host(s), ws)
+    np.testing.assert_array_equal(gu.host(q), wq)
+
+
 def test_a8_masked_columns():
     rng = np.random.default_rng(orc.SEED)
     x = rng.normal(size=(9, 512)).astype(np.float16)
