@@ -352,9 +352,10 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 // Residual add + RMSNorm in front of the rotation, one workgroup per row, same lane layout as
-// rotate_a8_kernel.  First pass: RO = fp32(X) + R, sum of squares.  Second pass: the fp32 sum is read
-// back by the thread that wrote it, Y = fp16((sum * rsqrt(mean + eps)) * (W + offset)), and that fp16
-// value goes through signs, butterflies and A8 as if rotate_a8_kernel had read Y.
+// rotate_a8_kernel.  First pass: RO = fp32(X) + R, sum of squares.  Second pass: the fp32 sum (kept
+// in registers, or read back by the thread that wrote it where the row is longer than the registers
+// hold), Y = fp16((sum * rsqrt(mean + eps)) * (W + offset)), and that fp16 value goes through signs,
+// butterflies and A8 as if rotate_a8_kernel had read Y.
 __global__ __launch_bounds__(256) void residual_norm_rotate_a8_kernel(
     const __half* __restrict__ x, const float* __restrict__ r, const __half* __restrict__ w, __half* __restrict__ y,
     float* __restrict__ ro, const int8_t* __restrict__ signs, int8_t* __restrict__ q, __half* __restrict__ s, int k,
@@ -366,7 +367,43 @@ __global__ __launch_bounds__(256) void residual_norm_rotate_a8_kernel(
     const int blocks = k / 128;  // even: k is a multiple of 256
     const int64_t base = (int64_t)row * k;
     float squares = 0.f;
-    for (int pair = wave; 2 * pair < blocks; pair += 4) {
+    // The first kHeld steps of a wave (all of them up to K = 5120): every load of both passes leaves
+    // at once, and the fp32 sums stay in registers for the second pass.  Longer rows go on in the
+    // loops below, which read their sums back.
+    constexpr int kHeld = 5;
+    float4 kept[kHeld];
+    uint2 held_w[kHeld];
+    uint32_t held_sign[kHeld];
+    {
+        uint2 raw[kHeld];
+        float4 residual[kHeld];
+#pragma unroll
+        for (int u = 0; u < kHeld; ++u) {  // clamped, so unconditional (blocks is even: a pair is live or not as a whole)
+            const int first = (min(2 * (wave + 4 * u), blocks - 2) + half_wave) * 128 + 4 * l32;
+            raw[u] = *reinterpret_cast<const uint2*>(x + base + first);
+            residual[u] = *reinterpret_cast<const float4*>(r + base + first);
+            held_w[u] = *reinterpret_cast<const uint2*>(w + first);
+            held_sign[u] = *reinterpret_cast<const uint32_t*>(signs + first);
+        }
+#pragma unroll
+        for (int u = 0; u < kHeld; ++u) {
+            if (2 * (wave + 4 * u) >= blocks) break;  // wave-uniform
+            const int first = (2 * (wave + 4 * u) + half_wave) * 128 + 4 * l32;
+            const __half* h = reinterpret_cast<const __half*>(&raw[u]);
+            float4 sum;
+            sum.x = __half2float(h[0]) + residual[u].x;
+            sum.y = __half2float(h[1]) + residual[u].y;
+            sum.z = __half2float(h[2]) + residual[u].z;
+            sum.w = __half2float(h[3]) + residual[u].w;
+            *reinterpret_cast<float4*>(ro + base + first) = sum;
+            kept[u] = sum;
+            squares += sum.x * sum.x;
+            squares += sum.y * sum.y;
+            squares += sum.z * sum.z;
+            squares += sum.w * sum.w;
+        }
+    }
+    for (int pair = wave + 4 * kHeld; 2 * pair < blocks; pair += 4) {
         const int first = (2 * pair + half_wave) * 128 + 4 * l32;
         const uint2 raw = *reinterpret_cast<const uint2*>(x + base + first);
         const __half* h = reinterpret_cast<const __half*>(&raw);
@@ -385,12 +422,8 @@ __global__ __launch_bounds__(256) void residual_norm_rotate_a8_kernel(
     const float total = block_sum(squares, sum_scratch);
     const float inverse = rsqrtf(__fdiv_rn(total, (float)k) + epsilon);
     float amax = 0.f;
-    for (int pair = wave; 2 * pair < blocks; pair += 4) {
-        const int first = (2 * pair + half_wave) * 128 + 4 * l32;
-        const float4 sum = *reinterpret_cast<const float4*>(ro + base + first);  // written above by this thread
-        const uint2 raw_w = *reinterpret_cast<const uint2*>(w + first);
+    auto second_pass = [&](int first, const float4& sum, const uint2& raw_w, uint32_t sign_word) {
         const __half* weight = reinterpret_cast<const __half*>(&raw_w);
-        const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
         const float values[4] = {sum.x, sum.y, sum.z, sum.w};
         __half normalized[4];
         float v[4];
@@ -407,6 +440,18 @@ __global__ __launch_bounds__(256) void residual_norm_rotate_a8_kernel(
         __half out[4];
         amax = fmaxf(amax, rotate_block(v, l32, out));
         *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
+    };
+#pragma unroll
+    for (int u = 0; u < kHeld; ++u) {
+        if (2 * (wave + 4 * u) >= blocks) break;  // wave-uniform
+        second_pass((2 * (wave + 4 * u) + half_wave) * 128 + 4 * l32, kept[u], held_w[u], held_sign[u]);
+    }
+    for (int pair = wave + 4 * kHeld; 2 * pair < blocks; pair += 4) {
+        const int first = (2 * pair + half_wave) * 128 + 4 * l32;
+        const float4 sum = *reinterpret_cast<const float4*>(ro + base + first);  // written above by this thread
+        const uint2 raw_w = *reinterpret_cast<const uint2*>(w + first);
+        const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+        second_pass(first, sum, raw_w, sign_word);
     }
     amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
     quantise_row(rotated, amax, q, s, row, k);
