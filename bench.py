@@ -26,8 +26,8 @@ CACHE_BYTES = 256 << 20        # Infinity Cache
 # `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
 # same counter reads for a device copy of 44 564 480 bytes in the same run: FETCH_SIZE reads
 # 21772.3 for 43 520 KiB (factor 1.9989), WRITE_SIZE reads 43 520.0 (factor 1.0).
-# Kernel (fp16-input GEMV): fetch 22043.9 -> 45 120 400 B, write 272.0 -> 278 560 B.
-MEASURED_TRAFFIC_BYTES = 45_398_960
+# Kernel (fp16-input GEMV): fetch 22044.0 -> 45 120 487 B, write 272.0 -> 278 560 B.
+MEASURED_TRAFFIC_BYTES = 45_399_047
 
 
 def parse():
