@@ -952,3 +952,71 @@ def test_config2_full_size_sampled_rows_and_linearity():
     colsum = c["weight"].astype(np.int64).sum(0)
     checksum = gu.host(a_q).astype(np.int64) @ colsum
     np.testing.assert_array_equal(gu.host(acc.double().sum(1)).astype(np.int64), checksum)
+
+
+# ---- configuration 4: one decoder layer's four projections at M = 8192 --------------------------
+_config4_cache = {}
+
+
+def _config4():
+    if "c" not in _config4_cache:
+        _config4_cache["c"] = workloads.config4()
+    return _config4_cache["c"]
+
+
+@pytest.mark.parametrize("name", [p[0] for p in workloads.LAYER_PROJECTIONS])
+def test_config4_full_size_sampled_rows_and_checksums(name):
+    """A8 with outlier channels + projection of every linear of the layer at M = 8192: the codes and
+    scales of the quantiser and the fp16 output bit-exact on 96 sampled rows x all N (oracle in
+    column blocks: the float64 form of the gate/up matrix alone would be 1.4 GB), and on ALL rows
+    acc(a) + acc(-a) == 0, row sums == a . colsum(W), column sums == colsum(a) . W."""
+    spec = _config4()[name]
+    rows_total, n, k = spec["rows"], spec["n"], spec["k"]
+    x = gu.dev(spec["x"])
+    a_q, a_s = gu.a8(x)
+    del x
+    rng = np.random.default_rng(4)
+    rows = np.sort(rng.choice(rows_total, 96, replace=False))
+    rows[0], rows[-1] = 0, rows_total - 1
+    wq, ws = orc.a8(spec["x"][rows])
+    got_q = gu.host(a_q)
+    np.testing.assert_array_equal(got_q[rows], wq)
+    np.testing.assert_array_equal(gu.host(a_s)[rows], ws)
+    # the outlier channels (x20) are where the row maxima sit: they must be the +-127 codes
+    outliers = np.argsort(np.abs(spec["x"][:64].astype(np.float32)).mean(0))[-max(1, k // 1000):]
+    assert (np.abs(got_q[rows][:, outliers]).max(1) == 127).all()
+    if spec["codec"] == "q4":
+        w_int = orc.q4_integers(spec["packed"], TABLE)
+        w_dev, s_dev = gu.dev(spec["packed"]), gu.dev(spec["scales"])
+        project = lambda a, s_tok, s_w, **kw: gu.q4_project(a, s_tok, w_dev, s_w, **kw)
+    else:
+        w_int = spec["weight"]
+        w_dev, s_dev = gu.dev(spec["weight"]), gu.dev(spec["scales"])
+        project = lambda a, s_tok, s_w, **kw: gu.w8_project(a, s_tok, w_dev, s_w, **kw)
+    out = project(a_q, a_s, s_dev)
+    got = gu.host(out[torch.from_numpy(rows).to(gu.DEV)])
+    del out
+    for first in range(0, n, 4096):
+        want = orc.project(wq, ws[:, 0], w_int[first:first + 4096], spec["scales"][first:first + 4096])
+        assert_close_fp16(got[:, first:first + 4096], want)
+        np.testing.assert_array_equal(got[:, first:first + 4096], want)
+    # size-independent properties over ALL rows, on the int32 accumulators (fp32 output, unit scales)
+    ones_m = torch.ones(rows_total, dtype=torch.float16, device=gu.DEV)
+    ones_n = torch.ones(n, dtype=torch.float16, device=gu.DEV)
+    acc = project(a_q, ones_m, ones_n, dtype=torch.float32)
+    assert float(acc.abs().max()) < 2.0 ** 24  # every accumulator is an exact fp32 value
+    neg = project(-a_q, ones_m, ones_n, dtype=torch.float32)
+    assert bool((acc + neg == 0).all())
+    del neg
+    row_sums = gu.host(acc.sum(1, dtype=torch.float64)).astype(np.int64)
+    col_sums = gu.host(acc.sum(0, dtype=torch.float64)).astype(np.int64)
+    del acc
+    w_colsum = np.zeros(k, np.int64)
+    for first in range(0, n, 4096):
+        w_colsum += w_int[first:first + 4096].sum(0, dtype=np.int64)
+    np.testing.assert_array_equal(row_sums, got_q.astype(np.int64) @ w_colsum)
+    a_colsum = got_q.sum(0, dtype=np.int64).astype(np.float64)
+    want_cols = np.concatenate([(w_int[first:first + 4096].astype(np.float64) @ a_colsum)
+                                for first in range(0, n, 4096)]).astype(np.int64)
+    np.testing.assert_array_equal(col_sums, want_cols)
+    torch.cuda.empty_cache()

@@ -176,6 +176,21 @@ def test_q4_exhaustive_fixture(table, clib):
     assert np.abs(w41).max() == 55 and (w41 % 2 != 0).all()  # 4*odd + odd is odd, |.| <= 44+11
 
 
+def test_q4_integers_gather_form_for_large_matrices_is_the_same_function(table, clib):
+    # above 2^20 codes q4_integers gathers from e8p_decode of all 65 536 codes: same values as the
+    # direct form (rows of it evaluated below the threshold) and as the C restatement
+    rng = np.random.default_rng(orc.SEED + 17)
+    packed = rng.integers(0, 2**32, (2100, 512), dtype=np.uint64).astype(np.uint32)
+    big = orc.q4_integers(packed, table)
+    assert big.dtype == np.int8 and big.shape == (2100, 4096)
+    for first in (0, 777, 2000):
+        np.testing.assert_array_equal(big[first:first + 100], orc.q4_integers(packed[first:first + 100], table))
+    cw = np.zeros((64, 4096), np.int8)
+    clib.orc_q4_integers(_ptr(table), _ptr(np.ascontiguousarray(packed[1500:1564])), ctypes.c_int64(64),
+                         ctypes.c_int64(4096), ctypes.c_int(4), ctypes.c_int(1), _ptr(cw))
+    np.testing.assert_array_equal(cw, big[1500:1564])
+
+
 def test_k_major_layouts_are_lossless():
     rng = np.random.default_rng(orc.SEED)
     packed = rng.integers(0, 2**32, (17, 48), dtype=np.uint64).astype(np.uint32)
