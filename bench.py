@@ -104,8 +104,9 @@ def main():
             self.a_s = torch.empty((self.rows, 1), dtype=torch.float16, device="cuda")
             self.out = torch.empty((self.rows, self.n), dtype=torch.float16, device="cuda")
             self.quant = Kernel("activation_quantization", K=self.k)
-            self.proj = Kernel("e8p_q4_projection", M=self.rows, N=self.n, K=self.k, algorithm=algorithm,
+            self.proj = Kernel("e8p_q4_projection", M=self.rows, N=self.n, K=self.k, algorithm=algorithm, workspace=True,
                                **({"packed_k": packed_k} if packed_k else {}))
+            self.proj.workspace()  # the caller's scratch, allocated before anything is captured
             # one row: the projection can quantise its fp16 row itself (one launch instead of two)
             self.fused = Kernel("e8p_q4_projection", M=1, N=self.n, K=self.k, input_dtype="float16",
                                 **({"packed_k": packed_k} if packed_k else {})) if fused_input else None
@@ -253,7 +254,8 @@ def main():
         o2 = torch.empty((c2["rows"], c2["n"]), dtype=torch.float16, device="cuda")
         w2, ws2 = dev(c2["weight"]), dev(c2["scales"])
         quant2 = Kernel("activation_quantization", K=c2["k"])
-        proj2 = Kernel("int8_projection", M=c2["rows"], N=c2["n"], K=c2["k"])
+        proj2 = Kernel("int8_projection", M=c2["rows"], N=c2["n"], K=c2["k"], workspace=True)
+        proj2.workspace()
         quant2(Mask=None, Q=a2, S=s2, X=x2, rows=c2["rows"])
         t = timed_graph(lambda i, s: proj2(stream=s, A=a2, Output=o2, TokenScale=s2, Weight=w2, WeightScale=ws2), 20)
         tq = timed_graph(lambda i, s: quant2(stream=s, Mask=None, Q=a2, S=s2, X=x2, rows=c2["rows"]), 20)
@@ -323,12 +325,13 @@ def main():
             quant = Kernel("activation_quantization", K=k)
             if spec["codec"] == "q4":
                 w = dev(spec["packed"])
-                proj = Kernel("e8p_q4_projection", M=rows, N=n, K=k)
+                proj = Kernel("e8p_q4_projection", M=rows, N=n, K=k, workspace=True)
                 run = lambda i, s: proj(stream=s, A=a, AS=sc, Book=book, Out=o, S=ws, W=w)
             else:
                 w = dev(spec["weight"])
-                proj = Kernel("int8_projection", M=rows, N=n, K=k)
+                proj = Kernel("int8_projection", M=rows, N=n, K=k, workspace=True)
                 run = lambda i, s: proj(stream=s, A=a, Output=o, TokenScale=sc, Weight=w, WeightScale=ws)
+            proj.workspace()
             tq = timed_graph(lambda i, s: quant(stream=s, Mask=None, Q=a, S=sc, X=x, rows=rows), 5)
             tp = timed_graph(run, 5)
             ops = workloads.algorithmic_ops(rows, n, k)

@@ -4,19 +4,30 @@
  * point: a `Kernel` record (symbol, grid, block, shared bytes, ordered args) is
  * resolved to a function handle and launched with `cuLaunchKernel(f, grid, block,
  * shared, stream, void** args, NULL)`.  This header is that entry point for HIP.
- * Nothing here allocates, synchronises or touches the host after the launch is
- * enqueued; every kernel reads its tables, scales and routing metadata from device
- * memory at run time, so a launch can be captured in a hipGraph and replayed after
- * the caller changed buffer contents.
+ * Nothing here allocates device memory (not at resolve, not at launch: a handle is
+ * host memory only), synchronises or touches the host after the launch is enqueued;
+ * every kernel reads its tables, scales and routing metadata from device memory at
+ * run time, so a launch can be captured in a hipGraph and replayed after the caller
+ * changed buffer contents.  The engine owns every buffer (AGENTS.md:41), scratch
+ * included: a kernel that wants scratch takes it as a `Workspace` buffer argument.
  *
  * Argument convention (crates/orinfer-engine/src/backend/cuda/mod.rs:282-299,319):
  * args[i] points at an 8-byte device pointer or at a 4-byte scalar.  The ORDER of
  * arguments per symbol is the generated host ABI of the reference (buffer names in
  * ASCII order, then scalars; dynamic-row kernels take `int32 m` last) and is
- * published by orx_arg_name() and orx_catalog().
+ * published by orx_arg_name() and orx_catalog().  The reference marshals
+ * Pointer, I32, U32, I64, U64 and F32 values; every kernel of this path takes device
+ * pointers and int32 row counts only, so those are the two kinds there are.
+ *
+ * Shapes: K is a multiple of 128 for every projection (the reference's int8 kernel
+ * also takes K % 64 == 0, int8_projection.py:29: not served here); two-stage codes are
+ * row-major (packed_k = 0) or K-major in blocks of 128 or 64 (packed_k = 128 | 64).
  *
  * Thread model: one thread per device session, one explicit stream
- * (backend/cuda/mod.rs:1-3).  Calls are re-entrant across distinct streams.
+ * (backend/cuda/mod.rs:1-3).  Handles are immutable after orx_resolve: launches of one
+ * handle, or of different handles, may run concurrently on distinct streams as long as
+ * their buffers (the Workspace included) are distinct.  One-time set-up inside the
+ * library is per device and safe to reach from several session threads.
  */
 #ifndef ORX_H
 #define ORX_H
@@ -36,6 +47,8 @@ extern "C" {
 #define ORX_ERR_BAD_GEOMETRY 10003     /* grid/block/shared do not fit the resolved kernel   */
 #define ORX_ERR_BAD_ARGUMENT 10004     /* null handle, null args, misaligned pointer         */
 #define ORX_ERR_ROWS 10005             /* dynamic rows outside 1..capacity                   */
+#define ORX_ERR_WORKSPACE 10006        /* the launch needs a Workspace and got none / too small a one */
+#define ORX_ERR_INTERNAL 10007         /* a C++ exception (out of host memory ...) stopped at the boundary */
 
 typedef struct orx_function* orx_fn;
 
@@ -48,7 +61,7 @@ typedef struct orx_function* orx_fn;
  *                      "{\"M\":1,\"N\":9728,\"K\":2560,\"algorithm\":\"gemv\"}", &f). */
 int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out);
 
-/* Drops a handle (cuModuleUnload in Session::cleanup). */
+/* Drops a handle (cuModuleUnload in Session::cleanup).  Host memory only. */
 int orx_release(orx_fn f);
 
 /* Replaces cuFuncGetAttribute(MAX_THREADS_PER_BLOCK / SHARED_SIZE_BYTES)
@@ -61,6 +74,17 @@ int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_by
  * variant's own M.  Fails with ORX_ERR_ROWS when rows exceeds the capacity. */
 int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes);
 
+/* Scratch the engine provides (AGENTS.md:41 "the engine owns every buffer"; the reference's
+ * kernels have none, so this has no counterpart there beyond the buffer table of
+ * crates/orinfer-model-sdk/src/artifact.rs:60-72 in which the engine would list it).  A
+ * projection resolved with `"workspace": true` takes one more buffer, `Workspace`, after its
+ * weights (256-byte aligned; contents need not be kept between launches; launches that overlap
+ * in time need distinct ones).  *bytes = what a launch of `rows` rows reads and writes there;
+ * rows <= 0 asks for the largest need of any row count up to the capacity, which is what an
+ * engine allocates once.  0 means the launch uses none and the pointer may be null.  Handles
+ * resolved without the key never use scratch (whole tiles, decode inside the GEMM). */
+int orx_workspace_bytes(orx_fn f, int32_t rows, uint64_t* bytes);
+
 /* Argument list of the resolved kernel, in launch order (contracts/abi.py:26-80 parses
  * the same from the generated host.txt).  kind: 0 = device pointer, 1 = int32 scalar. */
 int orx_arg_count(orx_fn f);
@@ -70,7 +94,10 @@ int orx_arg_kind(orx_fn f, int index);
 /* Replaces launch_kernel = cuLaunchKernel (backend/cuda/mod.rs:312-341).  Enqueues the
  * kernel on `hip_stream` (a hipStream_t, may be 0).  grid/block/shared must equal what
  * orx_geometry() returns for the row count passed in `m` (validated; the reference
- * validates records in kernels.rs:47-61).  Never blocks, never allocates. */
+ * validates records in kernels.rs:47-61).  Never blocks, never allocates.  A launch may
+ * enqueue more than one kernel (weight expansion + GEMM, split tiles + their sum, row slices
+ * of a batched-decode kernel): the recorded grid/block/shared are those of its main kernel and
+ * the whole launch is one node sequence under graph capture. */
 int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
                void* hip_stream, void** args);
 

@@ -136,23 +136,111 @@ def kernel_record(name, family, variant, bindings, rows=0):
     }
 
 
-def projection_records(slot, n, k, capacity, *, family="e8p_q4_projection", bindings=None):
-    """Row-specialised records of one projection slot under the naming rule `slot/rows/MIN-MAX`:
-    the decode kernel for 1..4 rows, the streaming kernel up to 128, the MFMA tiles above, each a
-    separately resolvable symbol whose geometry is recorded for the top of its range."""
-    ranges = [(1, min(4, capacity))]
-    if capacity > 4:
-        ranges.append((5, min(128, capacity)))
-    if capacity > 128:
-        ranges.append((129, capacity))
-    records = []
-    for low, high in ranges:
-        variant = dict(M=high, N=n, K=k, dynamic_rows=True)
-        names = lib.Kernel(family, **variant).arg_names
+# ---- dynamic-row launch contracts (crates/orinfer-model-sdk/src/operators/dynamic.rs:5-118) ---------
+def _constant(value):
+    return {"op": "constant", "value": int(value)}
+
+
+def _ceil_div_rows(divisor):
+    return {"op": "divide", "lhs": {"op": "add", "lhs": {"op": "rows"}, "rhs": _constant(divisor - 1)},
+            "rhs": _constant(divisor)}
+
+
+def evaluate_rows(expression, rows):
+    """RowExpression::evaluate (dynamic.rs:27-64): checked u32 arithmetic over the live row count."""
+    op = expression["op"]
+    if op == "constant":
+        return int(expression["value"])
+    if op == "rows":
+        return int(rows)
+    a, b = evaluate_rows(expression["lhs"], rows), evaluate_rows(expression["rhs"], rows)
+    if op in ("divide", "remainder") and b == 0:
+        raise ValueError("Invalid row expression arithmetic")
+    value = {"add": a + b, "subtract": a - b, "multiply": a * b, "divide": a // b if b else 0,
+             "remainder": a % b if b else 0, "minimum": min(a, b)}[op]
+    if not 0 <= value < 2**32:
+        raise ValueError("Invalid row expression arithmetic")
+    return value
+
+
+def _fit_rows(values):
+    """A RowExpression that gives values[rows] for every key of `values`, or None: a constant,
+    c * ceil(rows / d), or min(cap, c * ceil(rows / d) / 8) (the workgroups of a split launch)."""
+    rows = sorted(values)
+    if len({values[r] for r in rows}) == 1:
+        return _constant(values[rows[0]])
+    for d in (32, 64, 128, 256):
+        tiles = {r: -(-r // d) for r in rows}
+        if all(values[r] % tiles[r] == 0 for r in rows) and len({values[r] // tiles[r] for r in rows}) == 1:
+            c = values[rows[0]] // tiles[rows[0]]
+            expr = _ceil_div_rows(d) if c == 1 else {"op": "multiply", "lhs": _constant(c), "rhs": _ceil_div_rows(d)}
+            return expr
+    cap = max(values.values())
+    for d in (128,):
+        below = [r for r in rows if values[r] < cap]
+        if not below:
+            continue
+        r0 = below[0]
+        for c in range(values[r0] * 8 // -(-r0 // d), (values[r0] + 1) * 8 // -(-r0 // d) + 1):
+            expr = {"op": "minimum", "lhs": _constant(cap),
+                    "rhs": {"op": "divide", "lhs": {"op": "multiply", "lhs": _constant(c), "rhs": _ceil_div_rows(d)},
+                            "rhs": _constant(8)}}
+            if all(evaluate_rows(expr, r) == values[r] for r in rows):
+                return expr
+    return None
+
+
+def projection_program(slot, n, k, capacity, *, family="e8p_q4_projection", bindings=None, workspace=True, **extra):
+    """Row-specialised records of one projection slot under the naming rule `slot/rows/MIN-MAX`
+    (crates/orinfer-model-sdk/src/operators/rows.rs:14-58), each a separately resolvable symbol.
+
+    The library picks a kernel by the live row count, and kernels differ in block size and LDS
+    bytes.  A `Kernel` record fixes block and shared memory and a `DynamicBatchKernel` varies only the
+    grid and the `m` scalar (dynamic.rs:74-118), so the row domain 1..capacity is cut wherever block
+    or LDS bytes change, and further wherever the grid stops being one RowExpression of the rows.
+    Every range is checked row by row against the library's own geometry before it is emitted.
+    Returns {"kernels": [Kernel...], "dynamic": [DynamicBatchKernel...]} (ranges of one row count have
+    no dynamic entry: their grid is static)."""
+    def handle(top):
+        variant = dict(M=top, N=n, K=k, dynamic_rows=True, **extra)
+        if workspace:
+            variant["workspace"] = True
+        return variant, lib.Kernel(family, **variant)
+
+    _, whole = handle(capacity)
+    kernels, dynamic = [], []
+    low = 1
+    while low <= capacity:
+        block, shared = whole.geometry(low)[1:]
+        high = low
+        while high < capacity and whole.geometry(high + 1)[1:] == (block, shared):
+            high += 1
+        # the record of a range is resolved at the top of the range: its own dispatch must agree, and the
+        # grid over the range must be one expression per dimension; shrink the range until both hold
+        while True:
+            variant, kernel = handle(high)
+            geometry = {r: kernel.geometry(r) for r in range(low, high + 1)}
+            fits = [None] * 3
+            if all(g[1:] == (block, shared) for g in geometry.values()):
+                fits = [_fit_rows({r: g[0][d] for r, g in geometry.items()}) for d in range(3)]
+            if all(f is not None for f in fits):
+                break
+            high = low + (high - low) // 2
+        names = kernel.arg_names
         bound = dict(bindings or {a: a for a in names})
         bound["m"] = high
-        records.append(kernel_record(f"{slot}/rows/{low}-{high}", family, variant, bound, rows=high))
-    return records
+        name = f"{slot}/rows/{low}-{high}"
+        kernels.append(kernel_record(name, family, variant, bound, rows=high))
+        if high > low:
+            dynamic.append({"name": name, "capacity": high, "grid": fits,
+                            "arguments": [{"index": names.index("m"), "value": {"op": "rows"}}]})
+        low = high + 1
+    return {"kernels": kernels, "dynamic": dynamic}
+
+
+def projection_records(slot, n, k, capacity, **options):
+    """The `Kernel` records of projection_program()."""
+    return projection_program(slot, n, k, capacity, **options)["kernels"]
 
 
 def fixture_manifest(buffers, records, validation, *, rows=None):

@@ -404,19 +404,6 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
     }
 }
 
-int device_compute_units() {
-    static int units = 0;
-    if (units == 0) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess)
-            units = prop.multiProcessorCount;
-        else
-            (void)hipGetLastError();
-        if (units <= 0) units = 256;
-    }
-    return units;
-}
 
 // Channel blocks whose codes a lane holds at once: 3 (2 where the token fragments of a long K leave
 // less room); ring depths beyond that only delay the first MFMA.
@@ -440,14 +427,13 @@ constexpr uint32_t kLdsLimit = 160 * 1024;
 template <int W, int S, int CB>
 int launch_shape(const DenseParams& p, hipStream_t stream) {
     constexpr int P = held_blocks(S, CB);
-    static bool opted_in = false;
-    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
-        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_resident_kernel<W, S, CB, P>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
-                                   "hipFuncSetAttribute");
-        if (code != ORX_OK) return code;
-        opted_in = true;
-    }
+    static DeviceOnce opted_in;  // dynamic LDS above 64 KiB needs an opt-in per kernel and device
+    const int ready = opted_in.run([] {
+        return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_resident_kernel<W, S, CB, P>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
+                         "hipFuncSetAttribute");
+    });
+    if (ready != ORX_OK) return ready;
     const int workgroups = workgroups_for(p.m, p.k);
     hipLaunchKernelGGL((dense_resident_kernel<W, S, CB, P>), dim3(workgroups), dim3(W * 64), lds_bytes(p.n, workgroups),
                        stream, p);
@@ -467,14 +453,13 @@ bool specialized_fits(int n, int k, int packed_k) {
 
 template <int S, int CB, bool KM>
 int launch_specialized_shape(const DenseParams& p, hipStream_t stream) {
-    static bool opted_in = false;
-    if (!opted_in) {  // dynamic LDS above 64 KiB needs an opt-in per kernel
-        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_specialized_kernel<S, CB, KM>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
-                                   "hipFuncSetAttribute");
-        if (code != ORX_OK) return code;
-        opted_in = true;
-    }
+    static DeviceOnce opted_in;  // dynamic LDS above 64 KiB needs an opt-in per kernel and device
+    const int ready = opted_in.run([] {
+        return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&dense_specialized_kernel<S, CB, KM>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit),
+                         "hipFuncSetAttribute");
+    });
+    if (ready != ORX_OK) return ready;
     hipLaunchKernelGGL((dense_specialized_kernel<S, CB, KM>), dim3(device_compute_units()), dim3(kSpecThreads),
                        specialized_lds_bytes(p.n, p.k), stream, p);
     return hip_check(hipGetLastError(), "launch projection (resident, loader waves)");

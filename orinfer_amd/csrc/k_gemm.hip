@@ -66,6 +66,7 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
 enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4 };
+enum Flags2 { kNoSplit = 1, kNoExpand = 2 };  // orx_function::flags2 of a projection
 
 constexpr int kBK = 128;        // K bytes per tile step
 constexpr int kPitch = kBK + 16;  // LDS row pitch in bytes
@@ -89,6 +90,8 @@ struct GemmParams {
     int64_t expert_weight_stride;  // bytes between experts in w
     int tile_rows;                 // rows a routed tile may hold (0: the kernel's own tile height)
     int* partials;                 // split launches: int32 partial tiles, two slots per workgroup
+    const void* w2;                // gate/up + SwiGLU: the Up matrix (w is Gate) and its scales
+    const __half* ws2;
 };
 
 template <int CODEC>
@@ -110,9 +113,14 @@ __host__ __device__ constexpr int weight_chunks() {
     return CODEC == kQ4 ? 4 : CODEC == kQ2 ? 2 : 8;
 }
 
-template <int CODEC, int BM, int BN, int WAVES_M, bool GROUPED>
+// SWIGLU (W8 only): the tile's 128 weight rows are 64 Gate channels followed by the same 64 Up channels,
+// a wave's two column blocks are gate and up of the same 32 channels, and the epilogue rounds both
+// projections to fp16 and stores fp16(g / (1 + exp(-g)) * u) (int8_swiglu.py:10-57 with
+// integer_core.py:19-28, 261-264): no intermediate leaves the workgroup.
+template <int CODEC, int BM, int BN, int WAVES_M, bool GROUPED, bool SWIGLU = false>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     constexpr int WAVES_N = 4 / WAVES_M;
+    static_assert(!SWIGLU || (CODEC == kW8 && !GROUPED && BN == 128 && WAVES_N == 2), "gate/up tile shape");
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
     static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
     constexpr int A_CHUNKS = BM * 8 / 256;                        // uint4 per thread for A
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-    const int n0 = blockIdx.x * BN;
+    const int n0 = blockIdx.x * (SWIGLU ? BN / 2 : BN);
     int row0, rows_here;
     const int8_t* w_base = reinterpret_cast<const int8_t*>(p.w);
     const __half* ws = p.ws;
@@ -160,6 +168,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         for (int i = 0; i < W_CHUNKS; ++i) {
             const int c = tid + 256 * i;
             constexpr int PER_ROW = weight_chunks<CODEC>();
+            if constexpr (SWIGLU) {
+                const int r = c / PER_ROW, q = c % PER_ROW;
+                const int nn = min(n0 + (r & 63), p.n - 1);
+                const int8_t* side = reinterpret_cast<const int8_t*>(r < 64 ? p.w : p.w2);
+                reg_w[i] = *reinterpret_cast<const v4u*>(side + (int64_t)nn * p.k + kt * kBK + q * 16);
+                continue;
+            }
             const int nn = min(n0 + c / PER_ROW, p.n - 1), q = c % PER_ROW;
             int64_t byte;
             if (CODEC == kW8)
@@ -228,7 +243,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
                 fa[i] = *reinterpret_cast<const v4i*>(lds_a + ((wave_m * TM + i) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                fb[j] = *reinterpret_cast<const v4i*>(lds_w + ((wave_n * TN + j) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
+                fb[j] = *reinterpret_cast<const v4i*>(lds_w + ((SWIGLU ? j * 2 + wave_n : wave_n * TN + j) * 32 + frag_row) * kPitch + ks * 32 + frag_k);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -239,6 +254,28 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     }
 
     // epilogue: lane holds column (lane&31) and rows 8*(r/4) + 4*(lane>>5) + r%4 of each 32x32 block
+    if constexpr (SWIGLU) {
+        const int col = n0 + wave_n * 32 + (lane & 31);
+        if (col >= p.n) return;
+        const float gate_scale = __half2float(ws[col]), up_scale = __half2float(p.ws2[col]);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int local = (wave_m * TM + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (local < rows_here) {
+                    const int64_t row = row0 + local;
+                    const float token = __half2float(p.as[row]);
+                    const float g = __half2float(__float2half_rn(rescale(acc[i][0][r], gate_scale, token)));
+                    const float u = __half2float(__float2half_rn(rescale(acc[i][1][r], up_scale, token)));
+                    float value = __fdiv_rn(g, 1.0f + expf(-g)) * u;
+                    asm volatile("" : "+v"(value));  // the cast rounds the fp32 product, never a fused multiply-convert
+                    reinterpret_cast<__half*>(p.out)[row * p.stride + col] = __float2half_rn(value);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int col = n0 + (wave_n * TN + j) * 32 + (lane & 31);
@@ -580,24 +617,13 @@ bool use_big(const orx_function& f, int rows) {
 // again, and even a single tile row gains: the decode leaves the MFMA loop).
 constexpr int kExpandRows = 129;
 bool use_expand(const orx_function& f, int rows) {
-    return f.flags == kQ4 && f.workspace != nullptr && use_big(f, rows) && rows >= kExpandRows;
+    return f.flags == kQ4 && f.takes_workspace && (f.flags2 & kNoExpand) == 0 && use_big(f, rows) && rows >= kExpandRows;
 }
 
 // Split launches serve the 128-row tiles when whole tiles would not spread evenly: up to two tiles
-// per CU.  The handle owns the partial slots (allocated when it is resolved).
-int split_groups() {
-    static int groups = 0;
-    if (groups == 0) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        // two workgroups per CU: a single workgroup of four waves leaves every load latency exposed
-        groups = 2 * (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess &&
-                              prop.multiProcessorCount > 0
-                          ? prop.multiProcessorCount
-                          : 256);
-    }
-    return groups;
-}
+// per CU.  The partial slots are in the caller's Workspace.
+// two workgroups per CU: a single workgroup of four waves leaves every load latency exposed
+int split_groups() { return 2 * device_compute_units(); }
 // 128-row tiles of this launch, and whether their count suits a split launch: measured at K = 5120
 // with N = 5120, 7168 and 17408, 40-272 tiles gain 10-40 % (two-stage codes 59 -> 44 us at 136 tiles,
 // 53 -> 32 us at 80), 408 tiles lose; a handful of tiles is latency, not balance, and two launches would
@@ -606,7 +632,7 @@ int64_t split_tiles(const orx_function& f, int rows) {
     return (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
 }
 bool split_shape_ok(const orx_function& f, int rows) {
-    if (f.partials == nullptr || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
+    if (!f.takes_workspace || (f.flags2 & kNoSplit) || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
     const int64_t tiles = split_tiles(f, rows);
     return tiles >= 8 && tiles <= (int64_t)split_groups() * 9 / 16 && tiles % (split_groups() / 2) != 0;
 }
@@ -631,6 +657,16 @@ bool use_split(const orx_function& f, int rows) {
 int split_groups_for(const orx_function& f, int rows) {
     const int64_t units = split_tiles(f, rows) * (f.K / kBK);
     return (int)std::max<int64_t>(1, std::min<int64_t>(split_groups(), units / 8));
+}
+
+// Workspace bytes of a launch: the partial slots of a split launch, or the decoded weights of a
+// two-stage launch on the 256-row tiles.
+uint64_t projection_workspace(const orx_function& f, int rows) {
+    if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows)) return 0;
+    if (use_expand(f, rows)) return (uint64_t)f.N * f.K;
+    if (use_big(f, rows)) return 0;
+    if (use_split(f, rows)) return (uint64_t)split_groups_for(f, rows) * 2 * kSplitSlotInts * sizeof(int);
+    return 0;
 }
 
 template <int CODEC>
@@ -681,6 +717,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.ws = pointer_arg<const __half>(args, 4);
     const int8_t* signs = f.rotate_input ? pointer_arg<const int8_t>(args, 5) : nullptr;
     p.w = pointer_arg<const void>(args, f.rotate_input ? 6 : 5);
+    void* workspace = f.takes_workspace ? pointer_arg<void>(args, f.workspace_arg) : nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out, signs);
     if (use_resident(f, rows)) {
@@ -704,16 +741,16 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         return ORX_OK;
     }
     if (use_expand(f, rows)) {
-        const int code = q4_expand_launch(p.w, p.book, f.workspace, f.N, f.K, f.packed_k, stream);
+        const int code = q4_expand_launch(p.w, p.book, workspace, f.N, f.K, f.packed_k, stream);
         if (code != ORX_OK) return code;
-        return gemm_big_launch(false, p.a, f.workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0,
+        return gemm_big_launch(false, p.a, workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0,
                                f.out_f32, g, stream);
     }
     if (use_big(f, rows))
         return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
                                f.out_f32, g, stream);
     if (use_split(f, rows)) {
-        p.partials = static_cast<int*>(f.partials);
+        p.partials = static_cast<int*>(workspace);
         return launch_split<kQ4>(p, split_groups_for(f, rows), stream);
     }
     return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
@@ -728,6 +765,7 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, 3);
     p.ws = pointer_arg<const __half>(args, 4);
     p.book = nullptr;
+    void* workspace = f.takes_workspace ? pointer_arg<void>(args, f.workspace_arg) : nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = 0, p.out_f32 = f.out_f32;
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out);
     if (use_stream(f, rows)) {
@@ -744,7 +782,7 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
                                stream);
     if (use_split(f, rows)) {
-        p.partials = static_cast<int*>(f.partials);
+        p.partials = static_cast<int*>(workspace);
         return launch_split<kW8>(p, split_groups_for(f, rows), stream);
     }
     return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
@@ -826,17 +864,17 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
             f->slots = probe.slots;  // ring depth of the replicated-table gemv, 0 = compact tables
         }
     }
-    // Partial slots of split launches (two 128 x 128 int32 tiles per workgroup): allocated here, never at
-    // launch.  Without a device (a build machine) or without memory the handle keeps whole tiles.
+    // workspace=true: the launch takes a trailing `Workspace` buffer (the caller's; orx_workspace_bytes
+    // gives its size) and may then split the K steps of its tiles over the CUs (int32 partial tiles) or
+    // decode two-stage weights once per launch; without it the handle keeps whole tiles and decodes
+    // inside the GEMM.  split_k=false and decode_in_gemm=true switch the two uses off one by one.
     {
-        int devices = 0;
-        const bool split = v.boolean("split_k", true, &bad);  // diagnostic: false keeps whole tiles
+        f->takes_workspace = v.boolean("workspace", false, &bad);
+        const bool split = v.boolean("split_k", true, &bad);
+        const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);
         if (bad) return ORX_ERR_BAD_VARIANT;
-        if (split && f->capacity > 16 && f->tiles == 0 && (f->algorithm == kAuto || f->algorithm == kMfma) &&
-            hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
-            if (hipMalloc(&f->partials, (size_t)split_groups() * 2 * kSplitSlotInts * sizeof(int)) != hipSuccess)
-                f->partials = nullptr, (void)hipGetLastError();
-        }
+        f->flags2 = (split ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);
+        f->workspace_need = projection_workspace;
     }
     f->geometry = projection_geometry;
     // a projection handle launches one of several kernels depending on the live rows (1024-thread
@@ -849,22 +887,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
 int make_q4_projection(const Variant& v, orx_function* f) {
     int code = make_projection(v, f, kQ4);
     if (code != ORX_OK) return code;
-    // Scratch for the decoded weights of large-row launches: allocated here, never at launch
-    // (a launch may be under graph capture).  Without a device (a build machine) or without
-    // memory the handle simply keeps decoding inside the GEMM.
-    int devices = 0;
-    const bool wants_scratch = f->capacity >= kExpandRows && (f->algorithm == kAuto || f->algorithm == kMfma) &&
-                               (f->tiles == 0 || f->tiles == 256);
     bool bad = false;
-    const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);  // diagnostic: keep the decode inside the GEMM
-    if (bad) return ORX_ERR_BAD_VARIANT;
-    if (wants_scratch && !in_gemm && hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
-        const size_t bytes = (size_t)f->N * f->K;
-        if (hipMalloc(&f->workspace, bytes) == hipSuccess)
-            f->workspace_bytes = bytes;
-        else
-            f->workspace = nullptr, (void)hipGetLastError();
-    }
     // input_dtype=float16: A is the fp16 row and AS is written, not read (the kernel quantises the row)
     const std::string input = v.string("input_dtype", "int8", &bad);
     if (bad || (input != "int8" && input != "float16")) {
@@ -891,6 +914,7 @@ int make_q4_projection(const Variant& v, orx_function* f) {
                {"Out", ArgPointer, 2}, {"S", ArgPointer, 2}};
     if (f->rotate_input) f->args.push_back({"Signs", ArgPointer, 8});
     f->args.push_back({"W", ArgPointer, 16});
+    if (f->takes_workspace) f->args.push_back({"Workspace", ArgPointer, 256u | 0x80000000u});  // null where no launch needs it
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->launch = q4_launch;
     return ORX_OK;
@@ -901,6 +925,7 @@ int make_w8_projection(const Variant& v, orx_function* f) {
     if (code != ORX_OK) return code;
     f->args = {{"A", ArgPointer, 16},     {"Output", ArgPointer, 2},      {"TokenScale", ArgPointer, 2},
                {"Weight", ArgPointer, 16}, {"WeightScale", ArgPointer, 2}};
+    if (f->takes_workspace) f->args.push_back({"Workspace", ArgPointer, 256u | 0x80000000u});
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->launch = w8_launch;
     return ORX_OK;
@@ -925,66 +950,66 @@ int make_w8_small_projection(const Variant& v, orx_function* f) {
 
 // ---- W8 gate/up projections with the SwiGLU boundary (shared expert) ---------------------------
 // kernels/cuda/model/int8_swiglu.py:10-57 with integer_core.py:19-28: both projections are rounded
-// to fp16, then out = fp16((g / (1 + exp(-g))) * u) in fp32.  Built from the catalog's own int8
-// projection (two launches into the handle's fp16 scratch, row stride 2N) and one elementwise
-// kernel; the scratch is allocated when the handle is resolved.
-__global__ __launch_bounds__(256) void swiglu_pair_kernel(const __half* __restrict__ pair, __half* __restrict__ out, int n) {
-    const int row = blockIdx.x, col = blockIdx.y * 256 + threadIdx.x;
-    if (col >= n) return;
-    const float g = __half2float(pair[(int64_t)row * 2 * n + col]);
-    const float u = __half2float(pair[(int64_t)row * 2 * n + n + col]);
-    float value = __fdiv_rn(g, 1.0f + expf(-g)) * u;
-    asm volatile("" : "+v"(value));  // the cast rounds the fp32 product, never a fused multiply-convert
-    out[(int64_t)row * n + col] = __float2half_rn(value);
+// to fp16, then out = fp16((g / (1 + exp(-g))) * u) in fp32.  One launch: a workgroup owns 64 output
+// channels, holds the gate and the up accumulators of the same channels side by side (gemm_kernel's
+// SWIGLU form) and applies the boundary in its epilogue; nothing goes through memory in between.
+int int8_swiglu_geometry(const orx_function& f, int rows, Geometry* g) {
+    const int bm = rows <= 64 ? 64 : 128;
+    g->grid[0] = ceil_div((uint32_t)f.N, 64u);
+    g->grid[1] = ceil_div((uint32_t)rows, (uint32_t)bm);
+    g->block[0] = 256;
+    g->shared = 0;
+    return ORX_OK;
 }
 
 // A, Gate, GateScale, Output, TokenScale, Up, UpScale[, m]   (int8_swiglu.py:43-50 in generated-ABI order)
 int int8_swiglu_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
-    if (f.workspace == nullptr || f.inner == nullptr) {
-        set_error("%s: the handle was resolved without a device, its scratch is missing", f.symbol.c_str());
-        return ORX_ERR_BAD_ARGUMENT;
-    }
-    const int8_t* a = pointer_arg<const int8_t>(args, 0);
-    const __half* token_scale = pointer_arg<const __half>(args, 4);
-    __half* pair = static_cast<__half*>(f.workspace);
-    const void* weights[2] = {pointer_arg<const void>(args, 1), pointer_arg<const void>(args, 5)};
-    const __half* scales[2] = {pointer_arg<const __half>(args, 2), pointer_arg<const __half>(args, 6)};
-    for (int side = 0; side < 2; ++side) {
-        void* out = pair + (size_t)side * f.N;
-        void* inner_args[6] = {&a, &out, &token_scale, &weights[side], &scales[side], nullptr};
-        const int code = w8_launch(*f.inner, rows, g, stream, inner_args);
-        if (code != ORX_OK) return code;
-    }
-    hipLaunchKernelGGL(swiglu_pair_kernel, dim3((uint32_t)rows, ceil_div((uint32_t)f.N, 256u)), dim3(256), 0, stream, pair,
-                       pointer_arg<__half>(args, 3), f.N);
-    return hip_check(hipGetLastError(), "launch int8_swiglu (boundary)");
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.w = pointer_arg<const void>(args, 1);
+    p.ws = pointer_arg<const __half>(args, 2);
+    p.out = pointer_arg<void>(args, 3);
+    p.as = pointer_arg<const __half>(args, 4);
+    p.w2 = pointer_arg<const void>(args, 5);
+    p.ws2 = pointer_arg<const __half>(args, 6);
+    p.n = f.N, p.k = f.K, p.stride = f.N, p.m = rows, p.packed_k = 0, p.out_f32 = 0;
+    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    if (rows <= 64)
+        hipLaunchKernelGGL((gemm_kernel<kW8, 64, 128, 2, false, true>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemm_kernel<kW8, 128, 128, 2, false, true>), grid, block, 0, stream, p);
+    return hip_check(hipGetLastError(), "launch int8_swiglu");
 }
 
 int make_int8_swiglu(const Variant& v, orx_function* f) {
-    int code = make_projection(v, f, kW8);
-    if (code != ORX_OK) return code;
-    if (f->out_f32 || f->stride != f->N) {
-        set_error("int8_swiglu: fp16 output with row stride N only");
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    // the reference's tile hints (int8_swiglu.py:15-31): checked as it checks them, otherwise not used
+    const std::string algorithm = v.string("algorithm", "tensor_core", &bad);
+    const bool packed = algorithm == "dp4a";
+    const long long block_n = v.integer("block_n", 64, &bad), block_m = v.integer("block_m", packed ? 4 : 16, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % kBK || (int64_t)f->K * 128 * 128 > 2147483647LL) {
+        set_error("int8_swiglu: invalid decode INT8 SwiGLU geometry (M, N, K > 0, K a multiple of 128, K*2^14 < 2^31)");
         return ORX_ERR_BAD_VARIANT;
     }
+    if ((algorithm != "dp4a" && algorithm != "tensor_core" && algorithm != "auto" && algorithm != "mfma") ||
+        (packed && (block_m < 1 || block_m > 8 || (block_n != 4 && block_n != 8 && block_n != 16 && block_n != 32 && block_n != 64))) ||
+        (!packed && ((block_m != 16 && block_m != 32) || (block_n != 64 && block_n != 128)))) {
+        set_error("int8_swiglu: invalid INT8 SwiGLU algorithm or tile");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->stride = f->N;
+    f->flags = kW8;
     f->args = {{"A", ArgPointer, 16},         {"Gate", ArgPointer, 16}, {"GateScale", ArgPointer, 2}, {"Output", ArgPointer, 2},
                {"TokenScale", ArgPointer, 2}, {"Up", ArgPointer, 16},   {"UpScale", ArgPointer, 2}};
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
-    // the projections write fp16 pairs [rows, 2N]: same kernels, row stride 2N
-    f->inner = new orx_function(*f);
-    f->inner->stride = 2 * f->N;
-    f->inner->inner = nullptr;
-    int devices = 0;
-    if (hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
-        const size_t bytes = (size_t)f->capacity * 2 * f->N * sizeof(__half);
-        if (hipMalloc(&f->workspace, bytes) == hipSuccess)
-            f->workspace_bytes = bytes;
-        else
-            f->workspace = nullptr, (void)hipGetLastError();
-    } else {
-        (void)hipGetLastError();
-    }
+    f->geometry = int8_swiglu_geometry;
     f->launch = int8_swiglu_launch;
+    f->device_function = reinterpret_cast<const void*>(&gemm_kernel<kW8, 128, 128, 2, false, true>);
     return ORX_OK;
 }
 
@@ -1215,17 +1240,17 @@ const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|mfma, packed_k=0|128, output_dtype=float16|float32, "
-     "input_dtype=int8|float16, rotate=false, split_k=true, "
+     "input_dtype=int8|float16, rotate=false, workspace=false, split_k=true, "
      "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0, decode_in_gemm=false",
-     "A,AS,Book,Out,S[,Signs],W[,m]"},
+     "A,AS,Book,Out,S[,Signs],W[,Workspace][,m]"},
     {"int8_projection", make_w8_projection,
      "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma, output_dtype=float16|float32, output_stride=N, "
-     "block_m=0|32|64|128|256",
-     "A,Output,TokenScale,Weight,WeightScale[,m]"},
+     "block_m=0|32|64|128|256, workspace=false, split_k=true",
+     "A,Output,TokenScale,Weight,WeightScale[,Workspace][,m]"},
     {"int8_small_projection", make_w8_small_projection,
-     "M, N, K, dynamic_rows=false, output_dtype=float16|float32, output_stride=N, block_m=min(M,4) (1..8), block_n=4|8|16",
-     "A,Output,TokenScale,Weight,WeightScale[,m]"},
-    {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|mfma",
+     "M, N, K, dynamic_rows=false, output_dtype=float16|float32, output_stride=N, block_m=min(M,4) (1..8), block_n=4|8|16, workspace=false",
+     "A,Output,TokenScale,Weight,WeightScale[,Workspace][,m]"},
+    {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=tensor_core|dp4a, block_m, block_n (checked, not used)",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
     {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
      "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},

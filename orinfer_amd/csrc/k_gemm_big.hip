@@ -411,9 +411,7 @@ constexpr uint32_t kBigLdsQ4 = 4 * kTileBytes + sizeof(Q4ByteTables) > kBigLdsEp
 constexpr int kTM = ORX_BIG_TM, kTN = ORX_BIG_TN;
 constexpr int kBigThreads = (8 / kTM) * (8 / kTN) * 64;
 
-int prepare() {
-    static bool done = false;
-    if (done) return ORX_OK;
+int prepare_device() {
     int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<false, kTM, kTN>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds),
                          "hipFuncSetAttribute");
@@ -421,9 +419,11 @@ int prepare() {
     code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<true, kTM, kTN>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsQ4),
                      "hipFuncSetAttribute");
-    if (code != ORX_OK) return code;
-    done = true;
-    return ORX_OK;
+    return code;
+}
+int prepare() {
+    static DeviceOnce done;  // once per device, safe from several session threads
+    return done.run(prepare_device);
 }
 
 }  // namespace

@@ -698,17 +698,7 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 
 // ---- host side -----------------------------------------------------------------------------
 // slots: N, K, stride, capacity, block_m (= passes), flags (= codec), out_f32
-int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess)
-            cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
-    return cus;
-}
+int device_cus() { return device_compute_units(); }
 
 uint32_t gemv_lds_bytes(const orx_function& f, int mr) {
     const uint32_t planes = f.flags == kW8 ? (uint32_t)mr * f.K : (uint32_t)mr * (f.K / 8) * 8;
@@ -1141,10 +1131,8 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
     return ORX_OK;
 }
 
-int gemv_prepare_device() {
+static int gemv_opt_in_current_device() {
     // Dynamic LDS above 64 KiB needs an opt-in per kernel (kernels.rs:171-190 does the same on CUDA).
-    static bool done = false;
-    if (done) return ORX_OK;
     int limit = (int)kLdsLimit;  // the static tables take 2064 bytes of the 160 KiB
 #define ORX_OPT_IN(kernel)                                                                                   \
     {                                                                                                        \
@@ -1176,8 +1164,12 @@ int gemv_prepare_device() {
     ORX_OPT_IN_BANKED(4, kKMajorLayout + 16) ORX_OPT_IN_BANKED(5, kKMajorLayout + 16) ORX_OPT_IN_BANKED(6, kKMajorLayout + 16)
 #undef ORX_OPT_IN_BANKED
 #undef ORX_OPT_IN
-    done = true;
     return ORX_OK;
+}
+
+int gemv_prepare_device() {
+    static DeviceOnce done;  // once per device, safe from several session threads
+    return done.run(gemv_opt_in_current_device);
 }
 
 const Registration* gemv_registrations(int* count) {

@@ -406,19 +406,6 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     }
 }
 
-int device_compute_units() {
-    static int units = 0;
-    if (units == 0) {
-        int device = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&device) == hipSuccess && hipGetDeviceProperties(&prop, device) == hipSuccess)
-            units = prop.multiProcessorCount;
-        else
-            (void)hipGetLastError();
-        if (units <= 0) units = 256;
-    }
-    return units;
-}
 
 int ring_depth(int k) {
     const int kb = k / 128;
@@ -462,9 +449,8 @@ int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book
                             void* out, const int* counts, const int* offsets, const int* tile_expert,
                             const int* tile_row, const int* tile_count, int n, int k, int tiles, int packed_k,
                             hipStream_t stream) {
-    static bool opted_in = false;
-    if (!opted_in) {
-        // Dynamic LDS above 64 KiB needs an opt-in per kernel.
+    static DeviceOnce opted_in;  // dynamic LDS above 64 KiB needs an opt-in per kernel and device
+    const int ready = opted_in.run([] {
         const void* kernels[] = {reinterpret_cast<const void*>(&grouped_resident_kernel<3>),
                                  reinterpret_cast<const void*>(&grouped_resident_kernel<2>)};
         for (const void* kernel : kernels) {
@@ -472,8 +458,9 @@ int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book
                 hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit), "hipFuncSetAttribute");
             if (code != ORX_OK) return code;
         }
-        opted_in = true;
-    }
+        return (int)ORX_OK;
+    });
+    if (ready != ORX_OK) return ready;
     GroupedParams p = {};
     p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as;
     p.out = reinterpret_cast<__half*>(out);

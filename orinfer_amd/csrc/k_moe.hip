@@ -679,14 +679,13 @@ int metadata_geometry(const orx_function& f, int, Geometry* g) {
 // Counts, IDs, RelativeSlot, RowOffsets, TileCount, TileExpert, TileOffsets, TileRow[, m]
 // (moe.py:726-735 in generated-ABI order)
 int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
-    static bool opted_in = false;  // 64 KiB of counters at E = 1024 needs the LDS opt-in
-    if (!opted_in) {
-        const int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&route_metadata_kernel),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
-                                   "hipFuncSetAttribute");
-        if (code != ORX_OK) return code;
-        opted_in = true;
-    }
+    static DeviceOnce opted_in;  // 64 KiB of counters at E = 1024 needs the LDS opt-in
+    const int ready = opted_in.run([] {
+        return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&route_metadata_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024),
+                         "hipFuncSetAttribute");
+    });
+    if (ready != ORX_OK) return ready;
     hipLaunchKernelGGL(route_metadata_kernel, dim3(1), dim3(kMetaThreads), g.shared, s, pointer_arg<const int>(args, 1),
                        pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), pointer_arg<int>(args, 3),
                        pointer_arg<int>(args, 4), pointer_arg<int>(args, 5), pointer_arg<int>(args, 6),

@@ -6,7 +6,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <cmath>
+#include <memory>
+#include <new>
 
 #include "orx_internal.h"
 
@@ -26,6 +29,33 @@ int hip_check(hipError_t code, const char* operation) {
     // Same text shape as the reference's check(): "<op>: CUDA error <code>" (mod.rs:48-55).
     set_error("%s: HIP error %d (%s)", operation, (int)code, hipGetErrorName(code));
     return (int)code;
+}
+
+int current_device() {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return device;
+}
+
+int device_compute_units() {
+    static std::atomic<int> cached[64];
+    const int slot = current_device() & 63;
+    int units = cached[slot].load(std::memory_order_relaxed);
+    if (units == 0) {
+        hipDeviceProp_t prop;
+        int count = 0;
+        if (hipGetDeviceCount(&count) == hipSuccess && count > 0 &&
+            hipGetDeviceProperties(&prop, current_device()) == hipSuccess)
+            units = prop.multiProcessorCount;
+        else
+            (void)hipGetLastError();
+        if (units <= 0) units = 256;
+        cached[slot].store(units, std::memory_order_relaxed);
+    }
+    return units;
 }
 
 // ---- flat JSON object parser -------------------------------------------------------------
@@ -136,9 +166,12 @@ bool parse_variant(const char* json, Variant* out, std::string* error) {
 long long Variant::integer(const char* key, long long fallback, bool* bad) const {
     auto it = fields.find(key);
     if (it == fields.end() || it->second.kind == Value::Null) return fallback;
-    if (it->second.kind != Value::Number || std::floor(it->second.number) != it->second.number) {
+    // every integer of a variant is a shape, a count or a tile size and is stored in an int: a value
+    // outside the int range is refused here rather than wrapped by the casts of the factories
+    if (it->second.kind != Value::Number || std::floor(it->second.number) != it->second.number ||
+        !(std::fabs(it->second.number) <= 2147483647.0)) {
         *bad = true;
-        set_error("variant field %s must be an integer", key);
+        set_error("variant field %s must be an integer of at most 31 bits", key);
         return fallback;
     }
     return (long long)it->second.number;
@@ -191,14 +224,26 @@ const Registration* find(const char* symbol) {
 
 using namespace orx;
 
-extern "C" {
+namespace {
 
-int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
-    if (out == nullptr || symbol == nullptr) {
-        set_error("orx_resolve: null symbol or output");
-        return ORX_ERR_BAD_ARGUMENT;
+// No C++ exception crosses the C boundary: every entry point runs its body through guard().
+template <typename F>
+int guard(const char* entry, F&& body) {
+    try {
+        return body();
+    } catch (const std::bad_alloc&) {
+        set_error("%s: out of host memory", entry);
+        return ORX_ERR_INTERNAL;
+    } catch (const std::exception& e) {
+        set_error("%s: %s", entry, e.what());
+        return ORX_ERR_INTERNAL;
+    } catch (...) {
+        set_error("%s: unknown failure", entry);
+        return ORX_ERR_INTERNAL;
     }
-    *out = nullptr;
+}
+
+int resolve(const char* symbol, const char* variant_json, orx_fn* out) {
     // A package record has one `symbol` string and no place for a variant (artifact.rs:87-110), so
     // a symbol may carry it: "family?M=1&N=9728&K=2560&algorithm=gemv".  Values that are not
     // integers or true/false are taken as strings.
@@ -245,90 +290,38 @@ int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
         set_error("orx_resolve %s: %s", family.c_str(), why.c_str());
         return ORX_ERR_BAD_VARIANT;
     }
-    orx_function* f = new orx_function();
+    // the record owns host memory only, so every failure path is a plain delete
+    std::unique_ptr<orx_function> f(new orx_function());
     f->symbol = family;
-    int code = r->factory(variant, f);
-    if (code != ORX_OK) {
-        delete f;
-        return code;
-    }
+    const int code = r->factory(variant, f.get());
+    if (code != ORX_OK) return code;
     if (f->geometry == nullptr || f->launch == nullptr || f->args.empty()) {
-        delete f;
         set_error("orx_resolve %s: incomplete kernel record", symbol);
         return ORX_ERR_BAD_VARIANT;
     }
-    *out = f;
+    if (f->takes_workspace) {
+        f->workspace_arg = -1;
+        for (size_t i = 0; i < f->args.size(); ++i)
+            if (!strcmp(f->args[i].name, "Workspace")) f->workspace_arg = (int)i;
+        if (f->workspace_arg < 0 || f->workspace_need == nullptr) {
+            set_error("orx_resolve %s: incomplete workspace record", symbol);
+            return ORX_ERR_BAD_VARIANT;
+        }
+    }
+    *out = f.release();
     return ORX_OK;
 }
 
-int orx_release(orx_fn f) {
-    if (f != nullptr && f->workspace != nullptr) (void)hipFree(f->workspace);
-    if (f != nullptr && f->partials != nullptr) (void)hipFree(f->partials);
-    if (f != nullptr) delete f->inner;
-    delete f;
-    return ORX_OK;
-}
-
-int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
-    if (f == nullptr) {
-        set_error("orx_query: null handle");
-        return ORX_ERR_BAD_ARGUMENT;
-    }
-    hipFuncAttributes attr;
-    memset(&attr, 0, sizeof attr);
-    if (f->device_function != nullptr) {
-        int code = hip_check(hipFuncGetAttributes(&attr, f->device_function), "hipFuncGetAttributes");
-        if (code != ORX_OK) return code;
-    } else {
-        attr.maxThreadsPerBlock = 1024;
-    }
-    if (max_threads_per_block) *max_threads_per_block = (uint32_t)attr.maxThreadsPerBlock;
-    if (static_lds_bytes) *static_lds_bytes = (uint32_t)attr.sharedSizeBytes;
-    return ORX_OK;
-}
-
-int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes) {
-    if (f == nullptr) {
-        set_error("orx_geometry: null handle");
-        return ORX_ERR_BAD_ARGUMENT;
-    }
-    int live = rows <= 0 ? f->capacity : rows;
-    if (live > f->capacity || (!f->dynamic_rows && live != f->capacity)) {
-        // DynamicBatchKernel::launch rejects rows outside 1..capacity (operators/dynamic.rs:96-98).
-        set_error("%s: rows %d outside the kernel capacity %d", f->symbol.c_str(), live, f->capacity);
-        return ORX_ERR_ROWS;
-    }
-    Geometry g;
-    int code = f->geometry(*f, live, &g);
-    if (code != ORX_OK) return code;
-    for (int i = 0; i < 3; ++i) {
-        if (grid) grid[i] = g.grid[i];
-        if (block) block[i] = g.block[i];
-    }
-    if (shared_bytes) *shared_bytes = g.shared;
-    return ORX_OK;
-}
-
-int orx_arg_count(orx_fn f) { return f ? (int)f->args.size() : 0; }
-
-const char* orx_arg_name(orx_fn f, int index) {
-    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return "";
-    return f->args[index].name;
-}
-
-int orx_arg_kind(orx_fn f, int index) {
-    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return -1;
-    return (int)f->args[index].kind;
-}
-
-int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
-               void* hip_stream, void** args) {
+// Validates a launch against the record and returns the row count and geometry it runs with.
+int check_launch(const orx_function* f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+                 void** args, bool workspace_from_caller, int* rows_out, Geometry* want) {
     if (f == nullptr || grid == nullptr || block == nullptr || args == nullptr) {
         set_error("orx_launch: null handle, geometry or argument list");
         return ORX_ERR_BAD_ARGUMENT;
     }
     const int count = (int)f->args.size();
     for (int i = 0; i < count; ++i) {
+        if (i == f->workspace_arg && !workspace_from_caller) continue;  // replaced by the library's scratch
         if (args[i] == nullptr) {
             set_error("launch %s: argument %d (%s) is null", f->symbol.c_str(), i, f->args[i].name);
             return ORX_ERR_BAD_ARGUMENT;
@@ -355,50 +348,175 @@ int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32
             return ORX_ERR_ROWS;
         }
     }
-    Geometry want;
-    int code = f->geometry(*f, rows, &want);
+    int code = f->geometry(*f, rows, want);
     if (code != ORX_OK) return code;
     for (int i = 0; i < 3; ++i) {
-        if (grid[i] != want.grid[i] || block[i] != want.block[i]) {
+        if (grid[i] != want->grid[i] || block[i] != want->block[i]) {
             set_error("launch %s: geometry grid(%u,%u,%u) block(%u,%u,%u) does not fit the kernel, which needs "
                       "grid(%u,%u,%u) block(%u,%u,%u) for %d rows",
-                      f->symbol.c_str(), grid[0], grid[1], grid[2], block[0], block[1], block[2], want.grid[0],
-                      want.grid[1], want.grid[2], want.block[0], want.block[1], want.block[2], rows);
+                      f->symbol.c_str(), grid[0], grid[1], grid[2], block[0], block[1], block[2], want->grid[0],
+                      want->grid[1], want->grid[2], want->block[0], want->block[1], want->block[2], rows);
             return ORX_ERR_BAD_GEOMETRY;
         }
     }
-    if (shared_bytes != want.shared) {
-        set_error("launch %s: dynamic shared bytes %u, kernel needs %u", f->symbol.c_str(), shared_bytes, want.shared);
+    if (shared_bytes != want->shared) {
+        set_error("launch %s: dynamic shared bytes %u, kernel needs %u", f->symbol.c_str(), shared_bytes, want->shared);
         return ORX_ERR_BAD_GEOMETRY;
     }
-    return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), args);
+    *rows_out = rows;
+    return ORX_OK;
+}
+
+uint64_t workspace_need(const orx_function* f, int rows) {
+    return f->takes_workspace && f->workspace_need != nullptr ? f->workspace_need(*f, rows) : 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out) {
+    if (out == nullptr || symbol == nullptr) {
+        set_error("orx_resolve: null symbol or output");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    *out = nullptr;
+    return guard("orx_resolve", [&] { return resolve(symbol, variant_json, out); });
+}
+
+int orx_release(orx_fn f) {
+    delete f;  // host memory only: a handle owns nothing on the device
+    return ORX_OK;
+}
+
+int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
+    if (f == nullptr) {
+        set_error("orx_query: null handle");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    return guard("orx_query", [&] {
+        hipFuncAttributes attr;
+        memset(&attr, 0, sizeof attr);
+        if (f->device_function != nullptr) {
+            int code = hip_check(hipFuncGetAttributes(&attr, f->device_function), "hipFuncGetAttributes");
+            if (code != ORX_OK) return code;
+        } else {
+            attr.maxThreadsPerBlock = 1024;
+        }
+        if (max_threads_per_block) *max_threads_per_block = (uint32_t)attr.maxThreadsPerBlock;
+        if (static_lds_bytes) *static_lds_bytes = (uint32_t)attr.sharedSizeBytes;
+        return (int)ORX_OK;
+    });
+}
+
+int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes) {
+    if (f == nullptr) {
+        set_error("orx_geometry: null handle");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    return guard("orx_geometry", [&] {
+        int live = rows <= 0 ? f->capacity : rows;
+        if (live > f->capacity || (!f->dynamic_rows && live != f->capacity)) {
+            // DynamicBatchKernel::launch rejects rows outside 1..capacity (operators/dynamic.rs:96-98).
+            set_error("%s: rows %d outside the kernel capacity %d", f->symbol.c_str(), live, f->capacity);
+            return (int)ORX_ERR_ROWS;
+        }
+        Geometry g;
+        int code = f->geometry(*f, live, &g);
+        if (code != ORX_OK) return code;
+        for (int i = 0; i < 3; ++i) {
+            if (grid) grid[i] = g.grid[i];
+            if (block) block[i] = g.block[i];
+        }
+        if (shared_bytes) *shared_bytes = g.shared;
+        return (int)ORX_OK;
+    });
+}
+
+int orx_workspace_bytes(orx_fn f, int32_t rows, uint64_t* bytes) {
+    if (f == nullptr || bytes == nullptr) {
+        set_error("orx_workspace_bytes: null handle or output");
+        return ORX_ERR_BAD_ARGUMENT;
+    }
+    return guard("orx_workspace_bytes", [&] {
+        *bytes = 0;
+        if (rows > f->capacity || (rows > 0 && !f->dynamic_rows && rows != f->capacity)) {
+            set_error("%s: rows %d outside the kernel capacity %d", f->symbol.c_str(), rows, f->capacity);
+            return (int)ORX_ERR_ROWS;
+        }
+        if (rows > 0 || !f->dynamic_rows) {
+            *bytes = workspace_need(f, rows > 0 ? rows : f->capacity);
+            return (int)ORX_OK;
+        }
+        // rows <= 0 on a dynamic kernel: what the engine allocates once, the largest need of any row count
+        uint64_t most = 0;
+        for (int r = 1; r <= f->capacity; ++r) most = std::max(most, workspace_need(f, r));
+        *bytes = most;
+        return (int)ORX_OK;
+    });
+}
+
+int orx_arg_count(orx_fn f) { return f ? (int)f->args.size() : 0; }
+
+const char* orx_arg_name(orx_fn f, int index) {
+    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return "";
+    return f->args[index].name;
+}
+
+int orx_arg_kind(orx_fn f, int index) {
+    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return -1;
+    return (int)f->args[index].kind;
+}
+
+int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+               void* hip_stream, void** args) {
+    return guard("orx_launch", [&] {
+        int rows = 0;
+        Geometry want;
+        const int code = check_launch(f, grid, block, shared_bytes, args, true, &rows, &want);
+        if (code != ORX_OK) return code;
+        const uint64_t need = workspace_need(f, rows);
+        if (need != 0 && *reinterpret_cast<uint64_t*>(args[f->workspace_arg]) == 0) {
+            set_error("launch %s: %d rows need a Workspace of %llu bytes (orx_workspace_bytes), the buffer is null",
+                      f->symbol.c_str(), rows, (unsigned long long)need);
+            return (int)ORX_ERR_WORKSPACE;
+        }
+        return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), args);
+    });
 }
 
 const char* orx_last_error(void) { return g_error; }
 
 const char* orx_catalog(void) {
-    static std::string text;
-    if (text.empty()) {
-        std::string s = "{\"kernels\":[";
-        Table t[4];
-        tables(t);
-        bool first = true;
-        for (auto& table : t)
-            for (int i = 0; i < table.count; ++i) {
-                if (!first) s += ",";
-                first = false;
-                s += "{\"symbol\":\"";
-                s += table.rows[i].symbol;
-                s += "\",\"variant_keys\":\"";
-                s += table.rows[i].variant_keys;
-                s += "\",\"arguments\":\"";
-                s += table.rows[i].arguments;
-                s += "\"}";
-            }
-        s += "]}";
-        text = s;
-    }
-    return text.c_str();
+    // built once, also when two session threads ask at the same time
+    static const std::string* text = [] {
+        std::string* s = new (std::nothrow) std::string();
+        if (s == nullptr) return (const std::string*)nullptr;
+        try {
+            *s = "{\"kernels\":[";
+            Table t[4];
+            tables(t);
+            bool first = true;
+            for (auto& table : t)
+                for (int i = 0; i < table.count; ++i) {
+                    if (!first) *s += ",";
+                    first = false;
+                    *s += "{\"symbol\":\"";
+                    *s += table.rows[i].symbol;
+                    *s += "\",\"variant_keys\":\"";
+                    *s += table.rows[i].variant_keys;
+                    *s += "\",\"arguments\":\"";
+                    *s += table.rows[i].arguments;
+                    *s += "\"}";
+                }
+            *s += "]}";
+        } catch (...) {
+            delete s;
+            return (const std::string*)nullptr;
+        }
+        return (const std::string*)s;
+    }();
+    return text != nullptr ? text->c_str() : "{\"kernels\":[]}";
 }
 
 }  // extern "C"

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <map>
 #include <string>
 #include <vector>
@@ -54,23 +55,23 @@ struct orx_function {
     int capacity = 0;           // largest row count (M of the variant)
     // shape / configuration
     int M = 0, N = 0, K = 0, E = 0, top_k = 0, H = 0, stride = 0, group = 0, tiles = 0, slots = 0;
-    int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0;
+    int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0, flags2 = 0;
     bool out_f32 = false;
     bool input_f16 = false;  // single-row projection that quantises its fp16 activations itself
     bool rotate_input = false;  // ... after the signed block-128 rotation (takes a Signs buffer)
     const void* device_function = nullptr;  // for hipFuncGetAttributes
-    // Device scratch owned by the handle (allocated when it is resolved on a machine with a
-    // device, freed by orx_release): decoded int8 weights of a two-stage projection that serves
-    // many rows.  Launches of one handle share it, so they must not overlap on different streams.
-    void* workspace = nullptr;
-    size_t workspace_bytes = 0;
-    // int32 partial tiles of launches that split the K steps of output tiles over workgroups (owned).
-    void* partials = nullptr;
-    // A handle composed of other kernels of the catalog keeps them here (owned).
-    orx_function* inner = nullptr;
+    // The handle owns no device memory.  A kernel that needs scratch beyond its inputs and outputs
+    // (int32 partial tiles of split launches, int8 weights decoded once per launch) takes it from the
+    // caller as a trailing `Workspace` buffer when the variant says `workspace=true`; without it the
+    // handle keeps to the kernels that need none.  workspace_arg = index of that argument or -1.
+    bool takes_workspace = false;
+    int workspace_arg = -1;
+    // bytes of Workspace a launch of `rows` rows reads and writes (0: none needed)
+    uint64_t (*workspace_need)(const orx_function&, int rows) = nullptr;
     // rows -> geometry; returns ORX_OK or an error code
     int (*geometry)(const orx_function&, int rows, orx::Geometry*) = nullptr;
     // enqueue on stream; args already validated for count/alignment
+    // (the launch reads its Workspace pointer, if it takes one, from args[workspace_arg])
     int (*launch)(const orx_function&, int rows, const orx::Geometry&, hipStream_t, void** args) = nullptr;
 };
 
@@ -102,5 +103,24 @@ static inline T* pointer_arg(void** args, int index) {
 static inline int int_arg(void** args, int index) { return *reinterpret_cast<int32_t*>(args[index]); }
 
 static inline uint32_t ceil_div(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+// The device current on the calling thread (0 if there is none, as on a build machine).
+int current_device();
+// Compute units of the current device (256 where no device answers).  Cached per device.
+int device_compute_units();
+
+// One-time set-up that has to happen once per DEVICE (function attributes are per device), safe to
+// reach from several session threads: the set-up itself is idempotent, the flag is atomic.
+struct DeviceOnce {
+    std::atomic<uint64_t> done{0};
+    template <typename F>
+    int run(F&& setup) {
+        const uint64_t bit = 1ull << (current_device() & 63);
+        if (done.load(std::memory_order_acquire) & bit) return ORX_OK;
+        const int code = setup();
+        if (code == ORX_OK) done.fetch_or(bit, std::memory_order_release);
+        return code;
+    }
+};
 
 }  // namespace orx

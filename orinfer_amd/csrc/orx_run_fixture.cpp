@@ -293,6 +293,14 @@ int run(const std::string& manifest_path, std::ostringstream& report) {
                 if (it == buffers.end()) die("kernel " + symbol->text + ": unknown buffer " + name->text);
                 const size_t offset = (size_t)as_number(arg.get("offset"), 0);
                 if (offset >= it->second.bytes) die("kernel " + symbol->text + ": offset beyond buffer " + name->text);
+                // the engine sizes a Workspace buffer from orx_workspace_bytes before it accepts the record
+                if (std::string(orx_arg_name(record.function, (int)a)) == "Workspace") {
+                    uint64_t need = 0;
+                    orx(orx_workspace_bytes(record.function, rows, &need), "orx_workspace_bytes");
+                    if (it->second.bytes - offset < need)
+                        die("kernel " + symbol->text + ": Workspace buffer " + name->text + " holds " +
+                            std::to_string(it->second.bytes - offset) + " bytes, the launch needs " + std::to_string(need));
+                }
                 record.pointer_values[a] = reinterpret_cast<uint64_t>(static_cast<char*>(it->second.device) + offset);
             } else if (arg.get("null")) {
                 record.pointer_values[a] = 0;

@@ -18,10 +18,12 @@ ORX_ERR_BAD_VARIANT = 10002
 ORX_ERR_BAD_GEOMETRY = 10003
 ORX_ERR_BAD_ARGUMENT = 10004
 ORX_ERR_ROWS = 10005
+ORX_ERR_WORKSPACE = 10006
+ORX_ERR_INTERNAL = 10007
 
 EXPORTS = (
     "orx_resolve", "orx_release", "orx_query", "orx_geometry", "orx_arg_count", "orx_arg_name",
-    "orx_arg_kind", "orx_launch", "orx_last_error", "orx_catalog",
+    "orx_arg_kind", "orx_launch", "orx_last_error", "orx_catalog", "orx_workspace_bytes",
 )
 
 
@@ -67,6 +69,8 @@ def library():
         lib.orx_launch.argtypes = [ctypes.c_void_p, u32x3, u32x3, ctypes.c_uint32, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_void_p)]
         lib.orx_launch.restype = ctypes.c_int
+        lib.orx_workspace_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_uint64)]
+        lib.orx_workspace_bytes.restype = ctypes.c_int
         lib.orx_last_error.argtypes = []
         lib.orx_last_error.restype = ctypes.c_char_p
         lib.orx_catalog.argtypes = []
@@ -103,6 +107,7 @@ class Kernel:
         self.symbol = symbol
         self.variant = dict(variant)
         self._handle = ctypes.c_void_p()
+        self._workspace = None
         lib = library()
         _check(lib.orx_resolve(symbol.encode(), json.dumps(self.variant).encode(), ctypes.byref(self._handle)))
         count = lib.orx_arg_count(self._handle)
@@ -125,6 +130,25 @@ class Kernel:
         shared = ctypes.c_uint32()
         _check(library().orx_geometry(self._handle, int(rows), grid, block, ctypes.byref(shared)))
         return tuple(grid), tuple(block), shared.value
+
+    def workspace_bytes(self, rows=0):
+        """Bytes of `Workspace` a launch of `rows` rows uses (rows = 0: the most any row count needs)."""
+        need = ctypes.c_uint64()
+        _check(library().orx_workspace_bytes(self._handle, int(rows), ctypes.byref(need)))
+        return need.value
+
+    def workspace(self):
+        """This caller's Workspace buffer for the kernel, allocated once at the largest need (torch memory:
+        the caller owns it, as the engine owns every buffer).  None when the kernel takes or needs none."""
+        if "Workspace" not in self.arg_names:
+            return None
+        if self._workspace is None:
+            need = self.workspace_bytes(0)
+            if need:
+                import torch
+
+                self._workspace = torch.empty(need, dtype=torch.uint8, device="cuda")
+        return self._workspace
 
     def launch_raw(self, grid, block, shared, stream, values):
         """values: ABI-ordered list of device addresses (int) / int32 scalars.  Mirrors launch_kernel."""
@@ -151,6 +175,8 @@ class Kernel:
 
     def __call__(self, stream=None, **named):
         """Launch with arguments given by name (any order); unknown or missing names raise."""
+        if "Workspace" in self.arg_names and "Workspace" not in named:
+            named["Workspace"] = self.workspace()
         unknown = set(named) - set(self.arg_names)
         if unknown:
             raise OrxError(ORX_ERR_BAD_ARGUMENT, f"{self.symbol} has no arguments {sorted(unknown)}")

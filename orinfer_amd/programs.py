@@ -43,7 +43,9 @@ class QuantizedLinear:
         self.a_s = torch.empty((capacity, 1), dtype=torch.float16, device="cuda")
         self.out = torch.empty((capacity, self.n), dtype=torch.float16, device="cuda")
         self.quantizer = Kernel("activation_quantization", K=self.k)
-        variant = dict(M=capacity, N=self.n, K=self.k, dynamic_rows=True, algorithm=algorithm)
+        # workspace=True: the projection takes a `Workspace` buffer (allocated below, once, at the size
+        # orx_workspace_bytes reports) for split tiles and decode-once launches
+        variant = dict(M=capacity, N=self.n, K=self.k, dynamic_rows=True, algorithm=algorithm, workspace=True)
         if block_m:
             variant["block_m"] = block_m
         if codec == "q4":
@@ -52,6 +54,7 @@ class QuantizedLinear:
             self.projection = Kernel("e8p_q4_projection", **variant)
         else:
             self.projection = Kernel("int8_projection", **variant)
+        self.workspace = self.projection.workspace()
 
     def quantize(self, x16, stream=None):
         rows = x16.shape[0]
@@ -61,10 +64,10 @@ class QuantizedLinear:
     def project(self, rows, stream=None):
         if self.codec == "q4":
             self.projection(stream=stream, A=self.a_q, AS=self.a_s, Book=self.book, Out=self.out, S=self.scales,
-                            W=self.weight, m=rows)
+                            W=self.weight, Workspace=self.workspace, m=rows)
         else:
             self.projection(stream=stream, A=self.a_q, Output=self.out, TokenScale=self.a_s, Weight=self.weight,
-                            WeightScale=self.scales, m=rows)
+                            WeightScale=self.scales, Workspace=self.workspace, m=rows)
         return self.out[:rows]
 
     def run(self, x16, stream=None):

@@ -25,7 +25,7 @@ def declared_symbols():
 
 def test_header_symbols_are_exported():
     names = declared_symbols()
-    assert len(names) == 10 and set(names) == set(lib.EXPORTS)
+    assert len(names) == len(lib.EXPORTS) and set(names) == set(lib.EXPORTS)
     raw = ctypes.CDLL(str(lib.LIBRARY_PATH))
     for name in names:
         assert getattr(raw, name) is not None, name
@@ -166,6 +166,51 @@ def test_launch_record_is_validated_before_anything_is_enqueued():
         with pytest.raises(lib.OrxError) as err:
             dynamic.launch_raw(grid, block, shared, 0, fake + [rows])
         assert err.value.code == lib.ORX_ERR_ROWS
+
+
+def test_handles_own_no_device_memory_and_say_what_workspace_they_need():
+    """orx_resolve allocates nothing: scratch is a `Workspace` buffer the engine sizes from
+    orx_workspace_bytes (AGENTS.md:41: the engine owns every buffer).  A thousand handles resolve in
+    host memory only (the GPU test of the same name checks the device's free memory)."""
+    plain = lib.Kernel("e8p_q4_projection", M=8192, N=7168, K=5120, dynamic_rows=True)
+    assert plain.arg_names == ["A", "AS", "Book", "Out", "S", "W", "m"]           # the reference's list, unchanged
+    assert plain.workspace_bytes(0) == 0 and plain.workspace() is None
+    q4 = lib.Kernel("e8p_q4_projection", M=8192, N=7168, K=5120, dynamic_rows=True, workspace=True)
+    assert q4.arg_names == ["A", "AS", "Book", "Out", "S", "W", "Workspace", "m"]
+    assert q4.workspace_bytes(8192) == 7168 * 5120                                # int8 weights decoded once per launch
+    assert q4.workspace_bytes(1) == 0 and q4.workspace_bytes(32) == 0             # GEMV / batched decode: none
+    split = q4.workspace_bytes(256)                                                # 2 x 56 tiles of 128: K steps split over the CUs
+    assert split > 0 and split % (2 * 128 * 128 * 4) == 0 and split <= 512 * 2 * 128 * 128 * 4
+    assert q4.workspace_bytes(0) == max(split, 7168 * 5120)
+    assert q4.geometry(256) != plain.geometry(256)                                 # whole tiles without a workspace
+    w8 = lib.Kernel("int8_projection", M=512, N=5120, K=17408, workspace=True)
+    assert w8.arg_names == ["A", "Output", "TokenScale", "Weight", "WeightScale", "Workspace"]
+    assert w8.workspace_bytes(0) == w8.workspace_bytes(512) > 0
+    for off in (dict(split_k=False), dict(algorithm="gemv", M=4)):
+        assert lib.Kernel("int8_projection", **{**dict(M=256, N=5120, K=5120, workspace=True), **off}).workspace_bytes(0) == 0
+    with pytest.raises(lib.OrxError) as err:
+        q4.workspace_bytes(8193)
+    assert err.value.code == lib.ORX_ERR_ROWS
+    # a launch that needs the buffer refuses a null one before anything is enqueued; one that does not, takes it
+    grid, block, shared = q4.geometry(8192)
+    fake = [256] * 6
+    with pytest.raises(lib.OrxError) as err:
+        q4.launch_raw(grid, block, shared, 0, fake + [0, 8192])
+    assert err.value.code == lib.ORX_ERR_WORKSPACE and str(7168 * 5120) in str(err.value)
+    with pytest.raises(lib.OrxError) as err:
+        q4.launch_raw(grid, block, shared, 0, fake + [128, 8192])                 # not 256-byte aligned
+    assert err.value.code == lib.ORX_ERR_BAD_ARGUMENT
+    handles = [lib.Kernel("e8p_q4_projection", M=64 + i, N=17408, K=5120, dynamic_rows=True, workspace=True)
+               for i in range(1000)]
+    assert all(h.workspace_bytes(0) > 0 for h in handles[2:])
+    assert lib.library().orx_workspace_bytes(None, 0, None) == lib.ORX_ERR_BAD_ARGUMENT
+
+
+def test_variant_integers_are_range_checked():
+    for variant in (dict(M=4294967297, N=128, K=128), dict(M=1, N=2**31, K=128), dict(M=1, N=128, K=-2**40)):
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel("e8p_q4_projection", **variant)
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT, variant
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -62,23 +62,44 @@ def test_symbol_carries_its_variant():
 
 
 def test_kernel_records_follow_the_package_schema():
-    records = container.projection_records("decoder.0.qkv", 7168, 5120, 8192)
-    assert [r["name"] for r in records] == ["decoder.0.qkv/rows/1-4", "decoder.0.qkv/rows/5-128",
-                                            "decoder.0.qkv/rows/129-8192"]
+    program = container.projection_program("decoder.0.qkv", 7168, 5120, 8192)
+    records, dynamic = program["kernels"], {d["name"]: d for d in program["dynamic"]}
+    # the ranges partition 1..capacity (operators/rows.rs:14-58 parses MIN-MAX out of the name)
+    bounds = [tuple(int(v) for v in r["name"].rsplit("/", 1)[1].split("-")) for r in records]
+    assert bounds[0][0] == 1 and bounds[-1][1] == 8192
+    assert all(a[1] + 1 == b[0] for a, b in zip(bounds, bounds[1:])) and all(lo <= hi for lo, hi in bounds)
+    assert all(r["name"].startswith("decoder.0.qkv/rows/") for r in records)
     keys = {"name", "module", "source", "host_abi", "symbol", "grid", "block", "shared_memory_bytes", "cooperative", "args"}
-    for record in records:
+    for record, (low, high) in zip(records, bounds):
         assert set(record) == keys and record["cooperative"] is False
         assert record["symbol"].startswith("e8p_q4_projection?M=")
         for identity in (record["module"], record["source"], record["host_abi"]):
             assert set(identity) == {"file", "sha256"} and len(identity["sha256"]) == 64
-        assert [a.get("name", "m") for a in record["args"]] == ["A", "AS", "Book", "Out", "S", "W", "m"]
+        assert [a.get("name", "m") for a in record["args"]] == ["A", "AS", "Book", "Out", "S", "W", "Workspace", "m"]
         assert record["args"][-1]["kind"] == "i32" and all(a["kind"] == "buffer" for a in record["args"][:-1])
         threads = record["block"][0] * record["block"][1] * record["block"][2]
         assert 0 < threads <= 1024 and all(g > 0 for g in record["grid"])   # artifact.rs validate_geometry
-        # the record resolves and its launch geometry is what the library would use
+        # the record resolves; block and LDS bytes hold for EVERY row count of its range, and the grid is
+        # the record's RowExpression of the rows: what DynamicBatchKernel::launch computes (dynamic.rs:93-118)
+        # is a launch the library accepts, with no query of its own per launch
         kernel = lib.Kernel(record["symbol"])
-        rows = record["args"][-1]["value"]
-        assert kernel.geometry(rows) == (tuple(record["grid"]), tuple(record["block"]), record["shared_memory_bytes"])
+        assert record["args"][-1]["value"] == high == kernel.variant.get("M", high)
+        assert kernel.geometry(high) == (tuple(record["grid"]), tuple(record["block"]), record["shared_memory_bytes"])
+        contract = dynamic.get(record["name"])
+        assert (contract is None) == (low == high)
+        for rows in sorted({low, high, (low + high) // 2, min(high, low + 1), max(low, high - 1)}):
+            grid, block, shared = kernel.geometry(rows)
+            assert (block, shared) == (tuple(record["block"]), record["shared_memory_bytes"])
+            if contract is not None:
+                assert tuple(container.evaluate_rows(e, rows) for e in contract["grid"]) == grid
+        if contract is not None:
+            assert contract["capacity"] == high and contract["arguments"] == [{"index": 7, "value": {"op": "rows"}}]
+            assert [container.evaluate_rows(e, high) for e in contract["grid"]] == record["grid"]  # validate_binding
+    assert len(records) <= 8
+    with pytest.raises(ValueError):
+        container.evaluate_rows({"op": "subtract", "lhs": {"op": "constant", "value": 1}, "rhs": {"op": "rows"}}, 2)
+    plain = container.projection_records("decoder.0.o", 5120, 5120, 4, workspace=False)
+    assert [a.get("name", "m") for a in plain[0]["args"]] == ["A", "AS", "Book", "Out", "S", "W", "m"]
     json.loads(container.dumps(records[0]))
     sliced = container.kernel_record("embed", "e8p_q4_embedding", dict(M=8, vocab=100, hidden=256),
                                      dict(Book="Book", IDs=("Tokens", 64), Output="Hidden", Scale="Scale", Signs="Signs",
@@ -110,8 +131,9 @@ def test_container_to_records_to_fixture_run(tmp_path):
                 {"name": "Out", "bytes": 4 * n * 2, "fill": 0}]
     rotate = container.kernel_record("layer.rotate/rows/1-4", "rotate_activation_a8", dict(M=4, K=k, dynamic_rows=True),
                                      dict(Q="A", S="AS", Signs="Signs", X="X", m=rows), rows=rows)
-    project = container.projection_records("layer.proj", n, k, 4, bindings=dict(A="A", AS="AS", Book="Book", Out="Out",
-                                                                                  S="S", W="W"))[0]
+    project = [r for r in container.projection_records("layer.proj", n, k, 4, workspace=False,
+                                                        bindings=dict(A="A", AS="AS", Book="Book", Out="Out", S="S", W="W"))
+               if int(r["name"].rsplit("/", 1)[1].split("-")[0]) <= rows <= r["args"][-1]["value"]][0]
     project["args"][-1]["value"] = rows
     manifest = container.fixture_manifest(buffers, [rotate, project],
                                           dict(output="Out", output_dtype="f16", reference="Out.f32",

@@ -360,7 +360,8 @@ def test_q4_gemv_rotates_and_quantises_fp16_input(n, k, packed_k):
     scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
     signs = rng.choice(np.array([-1, 1], np.int8), k)
     stored = gu.dev(packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k))
-    kern = gu.kernel("e8p_q4_projection", M=1, N=n, K=k, packed_k=packed_k, input_dtype="float16", rotate=True)
+    kern = gu.kernel("e8p_q4_projection", M=1, N=n, K=k, packed_k=packed_k, input_dtype="float16", rotate=True,
+                     workspace=False)
     assert kern.arg_names == ["A", "AS", "Book", "Out", "S", "Signs", "W"]
     weights = orc.q4_integers(packed, TABLE)
     out = torch.full((2, n), 9.0, dtype=torch.float16, device=gu.DEV)
@@ -467,7 +468,8 @@ def test_q4_embedding_gather_matches_oracle():
     assert not got[3].any() and not got[4].any() and not got[6].any() and (got[len(ids):] == 3).all()
 
 
-@pytest.mark.parametrize("m,n,k", [(1, 96, 256), (6, 200, 1024), (70, 130, 384), (300, 260, 256)])
+@pytest.mark.parametrize("m,n,k", [(1, 96, 256), (6, 200, 1024), (70, 130, 384), (300, 260, 256), (64, 512, 2048),
+                                   (129, 64, 128)])
 def test_int8_swiglu_gate_up_boundary(m, n, k):
     rng = np.random.default_rng(orc.SEED + m + n)
     a_q = rng.integers(-127, 128, (m, k), dtype=np.int8)
@@ -479,8 +481,10 @@ def test_int8_swiglu_gate_up_boundary(m, n, k):
                                             TokenScale=gu.dev(a_s), Up=gu.dev(up), UpScale=gu.dev(us))
     got = gu.host(out)
     want = orc.int8_swiglu(a_q, a_s, gate, gs, up, us)
-    # exp() may differ in the last place between the device and libm: one fp16 step at most
+    # the two projections inside are exact integers rounded to fp16 as the oracle rounds them; only exp()
+    # may differ in the last place between the device and libm: one fp16 step at most, rarely
     np.testing.assert_allclose(got[:m].astype(np.float32), want.astype(np.float32), rtol=1e-3, atol=1e-2)
+    assert ulps_fp16(got[:m], want).max() <= 1
     assert np.mean(got[:m] == want) > 0.99 and (got[m:] == 2).all()
 
 
@@ -784,7 +788,7 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
 @pytest.mark.parametrize("packed_k", [0, 128])
 @pytest.mark.parametrize("decode_in_gemm", [False, True], ids=["decode-once", "decode-in-gemm"])
 def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
-    """From 512 rows on the two-stage weights are decoded once into the handle's scratch and the
+    """From 512 rows on the two-stage weights are decoded once into the caller's Workspace and the
     int8 kernel runs on them; `decode_in_gemm` keeps the decode inside the GEMM.  Same bits either
     way, also when the weights change between launches of one handle and under graph replay."""
     rng = np.random.default_rng(orc.SEED + 31 + packed_k)
@@ -792,12 +796,14 @@ def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     other = rng.integers(0, 2**32, packed.shape, dtype=np.uint32)
     store = (lambda p: p) if packed_k == 0 else (lambda p: orc.q4_pack_k(p, 128))
-    variant = dict(M=1024, N=n, K=k, dynamic_rows=True, output_stride=n + 3)
+    # split_k=False: so few 256-row tiles would otherwise go to the split 128-row tiles
+    variant = dict(M=1024, N=n, K=k, dynamic_rows=True, output_stride=n + 3, split_k=False)
     if packed_k:
         variant["packed_k"] = packed_k
     if decode_in_gemm:
         variant["decode_in_gemm"] = True
-    kern = gu.lib.Kernel("e8p_q4_projection", **variant)
+    kern = gu.lib.Kernel("e8p_q4_projection", workspace=True, **variant)
+    assert kern.workspace_bytes(700) == (0 if decode_in_gemm else n * k) and kern.workspace_bytes(3) == 0
     d_a, d_as, d_s, d_book = gu.dev(a_q), gu.dev(a_s), gu.dev(scales), gu.book()
     d_w = gu.dev(store(packed))
     out = torch.full((1024, n + 3), 7.0, dtype=torch.float16, device=gu.DEV)
@@ -880,7 +886,7 @@ def test_launch_rejects_bad_geometry_rows_and_alignment():
     w = torch.zeros((128, 32), dtype=torch.int32, device=gu.DEV)
     ws = torch.ones(128, dtype=torch.float16, device=gu.DEV)
     out = torch.zeros((8, 128), dtype=torch.float16, device=gu.DEV)
-    values = [a, s, gu.book(), out, ws, w, 8]
+    values = [a, s, gu.book(), out, ws, w, None, 8]    # 8 rows use no Workspace: a null one is taken
     grid, block, shared = kern.geometry(8)
     stream = torch.cuda.current_stream().cuda_stream
     with pytest.raises(lib.OrxError) as e:
@@ -1020,3 +1026,45 @@ def test_config4_full_size_sampled_rows_and_checksums(name):
                                 for first in range(0, n, 4096)]).astype(np.int64)
     np.testing.assert_array_equal(col_sums, want_cols)
     torch.cuda.empty_cache()
+
+
+# ---- scratch is the caller's ---------------------------------------------------------------------
+def test_resolving_handles_takes_no_device_memory():
+    torch.cuda.synchronize()
+    gu.lib.Kernel("int8_projection", M=8, N=128, K=128)  # the library's one-time set-up, if any
+    free_before = torch.cuda.mem_get_info()[0]
+    handles = [gu.lib.Kernel("e8p_q4_projection", M=4096 + i, N=17408, K=5120, dynamic_rows=True, workspace=True)
+               for i in range(1000)]
+    handles += [gu.lib.Kernel("int8_swiglu", M=512 + i, N=1024, K=2048, dynamic_rows=True) for i in range(100)]
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert handles[0].workspace_bytes(0) == 17408 * 5120
+
+
+def test_two_handles_on_two_streams_with_their_own_workspaces_stay_bit_exact():
+    """Launches of different handles (and of one handle) overlap on distinct streams as long as their
+    buffers, the Workspace included, are distinct: split tiles on one stream, decode-once on the other."""
+    rng = np.random.default_rng(orc.SEED + 77)
+    cases = []
+    for m, n, k in ((256, 5120, 1024), (640, 777, 640)):
+        a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+        kern = gu.lib.Kernel("e8p_q4_projection", M=m, N=n, K=k, workspace=True)
+        assert kern.workspace_bytes(m) > 0
+        want = orc.project(a_q, a_s, orc.q4_integers(packed, TABLE), scales)
+        cases.append((kern, gu.dev(a_q), gu.dev(a_s), gu.dev(packed), gu.dev(scales), want))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    # two launches of each handle in flight at once: each (handle, stream) pair has its own workspace and output
+    outs, spaces = {}, {}
+    for c, (kern, a, s, w, ws, want) in enumerate(cases):
+        for t in range(2):
+            outs[c, t] = torch.zeros(want.shape, dtype=torch.float16, device=gu.DEV)
+            spaces[c, t] = torch.empty(kern.workspace_bytes(0), dtype=torch.uint8, device=gu.DEV)
+    torch.cuda.synchronize()
+    for repeat in range(6):
+        for c, (kern, a, s, w, ws, want) in enumerate(cases):
+            for t in range(2):
+                kern(stream=streams[t].cuda_stream, A=a, AS=s, Book=gu.book(), Out=outs[c, t], S=ws, W=w,
+                     Workspace=spaces[c, t])
+    torch.cuda.synchronize()
+    for c, (kern, a, s, w, ws, want) in enumerate(cases):
+        for t in range(2):
+            np.testing.assert_array_equal(gu.host(outs[c, t]), want)
