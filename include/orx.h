@@ -101,6 +101,22 @@ int orx_arg_kind(orx_fn f, int index);
 int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
                void* hip_stream, void** args);
 
+/* Size of the library's own scratch, one copy per device for the life of the process. */
+#define ORX_STATIC_SCRATCH_BYTES (64u << 20)
+
+/* No counterpart in the reference.  For callers that cannot allocate device memory at all -- code
+ * that is already under hipGraph capture when it learns its shapes, tight serving loops and
+ * harnesses that forbid hipMalloc: orx_launch for a handle resolved with `"workspace": true`, with
+ * the Workspace argument ignored (its slot in `args` may be null) and the library's static device
+ * array of ORX_STATIC_SCRATCH_BYTES used in its place.  Everything else -- geometry check,
+ * arguments, results -- is orx_launch's.  A launch that needs more than ORX_STATIC_SCRATCH_BYTES
+ * (orx_workspace_bytes tells) fails with ORX_ERR_WORKSPACE and enqueues nothing.  Calls no
+ * allocator.  All calls on one device share that device's array: calls that overlap in time on
+ * one device (two streams) race; calls in stream order do not (nothing in the array has to
+ * survive from one launch to the next, and nothing has to be zero when a launch starts). */
+int orx_launch_static_scratch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+                              void* hip_stream, void** args);
+
 /* Thread-local text of the last failure on this thread (mod.rs:48-55 formats
  * "<op>: CUDA error <code>").  Never NULL. */
 const char* orx_last_error(void);

@@ -222,6 +222,36 @@ const Registration* find(const char* symbol) {
 }  // namespace
 }  // namespace orx
 
+// ---- library-owned scratch for callers that cannot allocate ------------------------------------
+// orx_launch_static_scratch() runs a launch on this array instead of a caller's Workspace.  The name
+// `scratch` is a host-side stand-in for the symbol, not a device address: the address is asked for
+// once per device (hipGetSymbolAddress, with that device current) and only that pointer is ever
+// handed to a kernel.  Every device the library runs on holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[ORX_STATIC_SCRATCH_BYTES];
+
+namespace orx {
+namespace {
+std::atomic<void*> g_scratch_address[64];
+
+// Address of `scratch` on the current device; looked up on the first call per device.
+int static_scratch_address(void** out) {
+    const int slot = current_device() & 63;
+    void* address = g_scratch_address[slot].load(std::memory_order_acquire);
+    if (address == nullptr) {
+        const int code = hip_check(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+        if (code != ORX_OK) return code;
+        if (address == nullptr || reinterpret_cast<uintptr_t>(address) % 256 != 0) {
+            set_error("hipGetSymbolAddress(scratch): unusable address %p", address);
+            return ORX_ERR_INTERNAL;
+        }
+        g_scratch_address[slot].store(address, std::memory_order_release);
+    }
+    *out = address;
+    return ORX_OK;
+}
+}  // namespace
+}  // namespace orx
+
 using namespace orx;
 
 namespace {
@@ -306,6 +336,15 @@ int resolve(const char* symbol, const char* variant_json, orx_fn* out) {
         if (f->workspace_arg < 0 || f->workspace_need == nullptr) {
             set_error("orx_resolve %s: incomplete workspace record", symbol);
             return ORX_ERR_BAD_VARIANT;
+        }
+        // set-up for orx_launch_static_scratch on the device current now (resolve is never under graph
+        // capture, the first launch may be); a machine without a device simply has nothing to look up
+        int devices = 0;
+        if (hipGetDeviceCount(&devices) == hipSuccess && devices > 0) {
+            void* unused = nullptr;
+            (void)static_scratch_address(&unused);
+        } else {
+            (void)hipGetLastError();
         }
     }
     *out = f.release();
@@ -482,6 +521,38 @@ int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32
             return (int)ORX_ERR_WORKSPACE;
         }
         return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), args);
+    });
+}
+
+int orx_launch_static_scratch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
+                              void* hip_stream, void** args) {
+    return guard("orx_launch_static_scratch", [&] {
+        int rows = 0;
+        Geometry want;
+        const int code = check_launch(f, grid, block, shared_bytes, args, false, &rows, &want);
+        if (code != ORX_OK) return code;
+        if (!f->takes_workspace)  // nothing to replace: the plain launch
+            return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), args);
+        const uint64_t need = workspace_need(f, rows);
+        if (need > (uint64_t)ORX_STATIC_SCRATCH_BYTES) {
+            set_error("launch %s: %d rows need %llu bytes of scratch, the library's static scratch holds %llu "
+                      "(ORX_STATIC_SCRATCH_BYTES): pass a Workspace to orx_launch instead",
+                      f->symbol.c_str(), rows, (unsigned long long)need, (unsigned long long)ORX_STATIC_SCRATCH_BYTES);
+            return (int)ORX_ERR_WORKSPACE;
+        }
+        void* address = nullptr;
+        const int found = static_scratch_address(&address);
+        if (found != ORX_OK) return found;
+        // the caller's argument list with the Workspace slot pointing at the library's scratch
+        const size_t count = f->args.size();
+        void* patched[64];
+        if (count > 64) {
+            set_error("launch %s: too many arguments", f->symbol.c_str());
+            return (int)ORX_ERR_INTERNAL;
+        }
+        for (size_t i = 0; i < count; ++i) patched[i] = args[i];
+        patched[f->workspace_arg] = &address;
+        return f->launch(*f, rows, want, reinterpret_cast<hipStream_t>(hip_stream), patched);
     });
 }
 

@@ -24,6 +24,7 @@ ORX_ERR_INTERNAL = 10007
 EXPORTS = (
     "orx_resolve", "orx_release", "orx_query", "orx_geometry", "orx_arg_count", "orx_arg_name",
     "orx_arg_kind", "orx_launch", "orx_last_error", "orx_catalog", "orx_workspace_bytes",
+    "orx_launch_static_scratch",
 )
 
 
@@ -69,6 +70,8 @@ def library():
         lib.orx_launch.argtypes = [ctypes.c_void_p, u32x3, u32x3, ctypes.c_uint32, ctypes.c_void_p,
                                    ctypes.POINTER(ctypes.c_void_p)]
         lib.orx_launch.restype = ctypes.c_int
+        lib.orx_launch_static_scratch.argtypes = lib.orx_launch.argtypes
+        lib.orx_launch_static_scratch.restype = ctypes.c_int
         lib.orx_workspace_bytes.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_uint64)]
         lib.orx_workspace_bytes.restype = ctypes.c_int
         lib.orx_last_error.argtypes = []
@@ -150,8 +153,9 @@ class Kernel:
                 self._workspace = torch.empty(need, dtype=torch.uint8, device="cuda")
         return self._workspace
 
-    def launch_raw(self, grid, block, shared, stream, values):
-        """values: ABI-ordered list of device addresses (int) / int32 scalars.  Mirrors launch_kernel."""
+    def launch_raw(self, grid, block, shared, stream, values, static_scratch=False):
+        """values: ABI-ordered list of device addresses (int) / int32 scalars.  Mirrors launch_kernel.
+        static_scratch: through orx_launch_static_scratch (the library's scratch replaces Workspace)."""
         if len(values) != len(self.arg_names):
             raise OrxError(ORX_ERR_BAD_ARGUMENT,
                            f"{self.symbol} takes {len(self.arg_names)} arguments {self.arg_names}, got {len(values)}")
@@ -160,7 +164,8 @@ class Kernel:
             storage.append(ctypes.c_uint64(_pointer_of(value)) if kind == 0 else ctypes.c_int32(int(value)))
         pointers = (ctypes.c_void_p * len(storage))(*[ctypes.cast(ctypes.byref(s), ctypes.c_void_p) for s in storage])
         g, b = (ctypes.c_uint32 * 3)(*grid), (ctypes.c_uint32 * 3)(*block)
-        _check(library().orx_launch(self._handle, g, b, int(shared), ctypes.c_void_p(int(stream)), pointers))
+        entry = library().orx_launch_static_scratch if static_scratch else library().orx_launch
+        _check(entry(self._handle, g, b, int(shared), ctypes.c_void_p(int(stream)), pointers))
 
     def launch(self, *values, rows=0, stream=None):
         """Launch with ABI-ordered arguments on `stream` (default: torch's current stream)."""
