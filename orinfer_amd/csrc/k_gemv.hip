@@ -393,9 +393,9 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
         for (int r = 0; r < MR; ++r)  // unconditional, clamped: a predicated load would be waited for at once
             raw[r] = *reinterpret_cast<const uint2*>(a + (int64_t)min(r, m - 1) * k + 8 * min(tid, groups - 1));
-    // The first chunks of the stream are requested in three instalments between the setup steps
-    // rather than all at once: a workgroup's full ring is 80 KiB, and the small reads of waves
-    // that start later would queue behind it in the CU's memory pipeline.
+    // The first chunks of the stream are requested in two instalments (when the small reads are back,
+    // and after the barrier) rather than all at once: a workgroup's full ring is 80 KiB, and the small
+    // reads of workgroups that start later would wait behind the bursts of the early ones.
     const char* first_base = base_of(first_task);
     const uint32_t first_offset = lane_offset(first_task);
     auto prefetch = [&](int from, int to) {
@@ -434,6 +434,12 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
         for (int r = 0; r < MR; ++r) asm volatile("" : "+v"(raw[r].x), "+v"(raw[r].y));
     }
+    // The wave's small reads are back: two chunks of the stream go out now and are in flight while the
+    // tables are built (measured against one chunk just before the barrier: 6.8 -> 6.4 us at N=9728,
+    // K=2560, 13.4 -> 12.8 us for the fp16-input form at N=17408, K=5120).  Earlier, or more of them,
+    // and the small reads of workgroups that start later wait behind the bursts in the L2 queues
+    // (set-up data back after 2.1-3.9 us instead of 1.2-2.0 us) and nothing is gained.
+    prefetch(0, 2);
     {
         const uint32_t low = (uint32_t)selector_half(selector, quarter) & 15u;
         const uint32_t high = (uint32_t)selector_half(selector, quarter + 4) & 15u;
@@ -501,7 +507,6 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
         for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
         if (lane == 0) wave_max[wave] = amax;
-        prefetch(0, 1);  // the row has arrived: the stream can start while the row is quantised
         __syncthreads();
         // the 16 wave maxima, one per lane of a row, reduced with lane controls (no LDS round trips):
         // quad permutes, then the mirror of each half row, then the mirror of the row
@@ -586,9 +591,8 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
 #pragma unroll
         for (int r = 0; r < MR; ++r) wave_sums[r * 16 + wave] = wave_total[r];
     }
-    if (!X16) prefetch(0, 1);
     __syncthreads();
-    prefetch(1, D);
+    prefetch(2, D);
 
     const uint32_t column = kMskBase + 4u * (uint32_t)lane;
     // sum of each activation row (scalar), the steps at which this lane's column holds an
