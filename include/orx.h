@@ -21,7 +21,10 @@
  *
  * Shapes: K is a multiple of 128 for every projection (the reference's int8 kernel
  * also takes K % 64 == 0, int8_projection.py:29: not served here); two-stage codes are
- * row-major (packed_k = 0) or K-major in blocks of 128 or 64 (packed_k = 128 | 64).
+ * row-major (packed_k = 0) or K-major in blocks of 128 or 64 (packed_k = 128 | 64,
+ * e8p_q4.py:78-80,250).  Blocks of 64 are read by the streaming and the MFMA tile
+ * kernels at every row count; the one-row GEMV and the resident kernel read row-major
+ * codes and blocks of 128 only (production stores 128, models/qwen35/build.py:212).
  *
  * Thread model: one thread per device session, one explicit stream
  * (backend/cuda/mod.rs:1-3).  Handles are immutable after orx_resolve: launches of one

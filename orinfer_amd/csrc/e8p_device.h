@@ -182,6 +182,14 @@ __device__ __forceinline__ uint2 decode_q2(const Q2ByteTables& t, uint32_t code)
     return make_uint2(b.x ^ m.x, b.y ^ m.y);
 }
 
+// Byte offset of the 16-byte chunk `q` (0..3: 32 weights each) of weight row `row` in the 128-wide
+// K step `kt` of two-stage codes stored K-major, (K/packed_k, N, packed_k/8) u32 with packed_k = 128
+// or 64 (kernels/cuda/model/e8p_q4.py:250).
+__device__ __forceinline__ int64_t q4_k_major_chunk(int packed_k, int n, int row, int kt, int q) {
+    if (packed_k == 128) return ((int64_t)kt * n + row) * 64 + q * 16;
+    return ((int64_t)(kt * 2 + (q >> 1)) * n + row) * 32 + (q & 1) * 16;
+}
+
 // fp32 epilogue shared by every projection: (float(acc) * ws) * as, two separate roundings
 // (kernels/cuda/model/integer_core.py:19-22).
 __device__ __forceinline__ float rescale(int acc, float weight_scale, float token_scale) {

@@ -79,7 +79,7 @@ struct GemmParams {
     const __half* as;
     void* out;
     int n, k, stride, m;
-    int packed_k;  // 0 row-major codes, 128 K-major blocks
+    int packed_k;  // 0 row-major codes, 128 or 64 K-major blocks
     int out_f32;
     // grouped only
     const int* counts;
@@ -181,6 +181,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
                 byte = (int64_t)nn * p.k + kt * kBK + q * 16;
             else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
                 byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
+            else if (p.packed_k == 64)  // (K/64, N, 8 two-stage codes): two block rows per K step
+                byte = q4_k_major_chunk(64, p.n, nn, kt, q);
             else  // (N, K/8 codes)
                 byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
             reg_w[i] = *reinterpret_cast<const v4u*>(w_base + byte);
@@ -357,6 +359,8 @@ __global__ __launch_bounds__(256) void gemm_split_kernel(GemmParams p) {
                 byte = (int64_t)nn * p.k + kt * kBK + q * 16;
             else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
                 byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
+            else if (p.packed_k == 64)  // (K/64, N, 8 two-stage codes): two block rows per K step
+                byte = q4_k_major_chunk(64, p.n, nn, kt, q);
             else  // (N, K/8 codes)
                 byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
             reg_w[i] = *reinterpret_cast<const v4u*>(w_base + byte);
@@ -815,8 +819,8 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         set_error("%s: output_dtype must be float16 or float32", name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->packed_k != 0 && (f->packed_k != 128 || codec == kW8)) {
-        set_error("%s: packed_k must be 0 or 128 (codes only)", name);
+    if (f->packed_k != 0 && ((f->packed_k != 128 && f->packed_k != 64) || codec == kW8)) {
+        set_error("%s: packed_k must be 0, 64 or 128 (codes only)", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->tiles != 0 && f->tiles != 32 && f->tiles != 64 && f->tiles != 128 && f->tiles != 256) {
@@ -846,12 +850,12 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         set_error("%s: the stream algorithm serves up to 64 rows, variant asks for %d", name, f->capacity);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv && f->packed_k != 0 && (codec != kQ4 || f->K % 256 != 0)) {
-        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0), or K-major two-stage codes with K a multiple of 256",
+    if (f->algorithm == kGemv && f->packed_k != 0 && (codec != kQ4 || f->packed_k != 128 || f->K % 256 != 0)) {
+        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0), or K-major two-stage codes in 128-wide blocks with K a multiple of 256",
                   name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv || (f->algorithm == kAuto && (f->packed_k == 0 || (codec == kQ4 && f->K % 256 == 0)))) {
+    if (f->algorithm == kGemv || (f->algorithm == kAuto && (f->packed_k == 0 || (codec == kQ4 && f->packed_k == 128 && f->K % 256 == 0)))) {
         orx_function probe = *f;
         if (probe.capacity > 4) probe.capacity = 4;
         int code = gemv_configure(&probe, codec, passes);
@@ -1239,7 +1243,7 @@ int make_q2_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f,
 const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
-     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|mfma, packed_k=0|128, output_dtype=float16|float32, "
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|mfma, packed_k=0|64|128, output_dtype=float16|float32, "
      "input_dtype=int8|float16, rotate=false, workspace=false, split_k=true, "
      "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0, decode_in_gemm=false",
      "A,AS,Book,Out,S[,Signs],W[,Workspace][,m]"},

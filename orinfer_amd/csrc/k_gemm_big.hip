@@ -145,8 +145,8 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
             const int c = tid + kThreads * i;      // chunk id: row = c / 4, quarter = c % 4
             const int row = min(c >> 2, cols_here - 1), q = c & 3;
             int64_t byte;
-            if (p.packed_k == 128)
-                byte = ((int64_t)kt * p.n + col0 + row) * 64 + q * 16;
+            if (p.packed_k != 0)
+                byte = q4_k_major_chunk(p.packed_k, p.n, col0 + row, kt, q);
             else
                 byte = ((int64_t)(col0 + row) * (p.k / kStep) + kt) * 64 + q * 16;
             code_regs[set][i] = *reinterpret_cast<const v4u*>(reinterpret_cast<const int8_t*>(p.w) + byte);
@@ -446,6 +446,9 @@ __global__ __launch_bounds__(512) void q4_expand_kernel(const uint4* __restrict_
         if (packed_k == 128) {  // (K/128, N, 16) u32: four chunks per row and K block
             const int64_t kt = c / ((int64_t)n * 4), rest = c % ((int64_t)n * 4);
             row = rest >> 2, k0 = kt * 128 + (rest & 3) * 32;
+        } else if (packed_k == 64) {  // (K/64, N, 8) u32: two chunks per row and K block
+            const int64_t kb = c / ((int64_t)n * 2), rest = c % ((int64_t)n * 2);
+            row = rest >> 1, k0 = kb * 64 + (rest & 1) * 32;
         } else {
             row = c / per_row, k0 = (c % per_row) * 32;
         }

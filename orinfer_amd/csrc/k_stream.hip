@@ -116,6 +116,8 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         int64_t byte;
         if (CODEC == kW8 || p.packed_k == 0)
             byte = ((int64_t)w_row * k_blocks + kb) * BB + half * LANE_BYTES;
+        else if (p.packed_k == 64)  // two-stage codes in 64-wide K blocks: this lane's half is one block row
+            byte = ((int64_t)(kb * 2 + half) * p.n + w_row) * LANE_BYTES;
         else
             byte = ((int64_t)kb * p.n + w_row) * BB + half * LANE_BYTES;
         return reinterpret_cast<const uint4*>(w_base + byte);

@@ -432,14 +432,15 @@ def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
     assert torch.equal(out, other)
 
 
-def test_split_launches_serve_k_major_codes_and_dynamic_rows():
+@pytest.mark.parametrize("packed_k", [128, 64])
+def test_split_launches_serve_k_major_codes_and_dynamic_rows(packed_k):
     rng = np.random.default_rng(orc.SEED + 91)
     n, k, cap = 8704, 384, 256
     packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
     weights = orc.q4_integers(packed, TABLE)
     scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
-    kern = gu.kernel("e8p_q4_projection", M=cap, N=n, K=k, packed_k=128, dynamic_rows=True)
-    stored = gu.dev(orc.q4_pack_k(packed, 128))
+    kern = gu.kernel("e8p_q4_projection", M=cap, N=n, K=k, packed_k=packed_k, dynamic_rows=True)
+    stored = gu.dev(orc.q4_pack_k(packed, packed_k))
     for m in (200, 65, 130):
         a = rng.integers(-128, 128, (cap, k), dtype=np.int8)
         a_s = rng.uniform(0.01, 0.03, cap).astype(np.float16)
@@ -579,7 +580,7 @@ def test_q4_gemv_activation_extremes(m, pattern, variant):
     np.testing.assert_array_equal(gu.host(got).astype(np.int64), acc.astype(np.int64))
 
 
-@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
 @pytest.mark.parametrize("m", [1, 7, 32, 33, 64, 65, 128, 129, 300])
 def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
     # check_e8p_q4.py:123-193: N=65, K=256, fp32 out, stride N+3, sentinel 91 beyond the tails
@@ -587,7 +588,7 @@ def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
     n, k = 65, 256
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :2] = [-128, 127]
-    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
     storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
     gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
                   dtype=torch.float32, algorithm="mfma", packed_k=packed_k)
@@ -597,7 +598,7 @@ def test_q4_mfma_rows_tails_stride_and_sentinels(m, packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
-@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
 @pytest.mark.parametrize("m", [5, 8, 31, 32, 33, 64])
 def test_q4_stream_rows_tails_stride_and_sentinels(m, packed_k):
     # same construction as the MFMA tail test, through the weight-streaming kernel; K=640 gives the
@@ -606,7 +607,7 @@ def test_q4_stream_rows_tails_stride_and_sentinels(m, packed_k):
     n, k = 97, 640
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :2] = [-128, 127]
-    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
     w = orc.q4_integers(packed, TABLE)
     storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
     gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
@@ -770,13 +771,13 @@ def test_w8_dynamic_capacity_stride_extremes(m):
     assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
 
 
-@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
 def test_q4_big_tile_tails_stride_sentinels(packed_k):
     rng = np.random.default_rng(orc.SEED + 9)
     m, n, k = 257 + 130, 300, 384
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :2] = [-128, 127]
-    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, 128)
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
     storage = torch.full((m + 2, n + 5), 91.0, dtype=torch.float32, device=gu.DEV)
     gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 5,
                   dtype=torch.float32, algorithm="mfma", packed_k=packed_k, block_m=256)
@@ -785,7 +786,7 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
-@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
 @pytest.mark.parametrize("decode_in_gemm", [False, True], ids=["decode-once", "decode-in-gemm"])
 def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
     """From 512 rows on the two-stage weights are decoded once into the caller's Workspace and the
@@ -795,7 +796,7 @@ def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
     m, n, k = 700, 333, 640
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     other = rng.integers(0, 2**32, packed.shape, dtype=np.uint32)
-    store = (lambda p: p) if packed_k == 0 else (lambda p: orc.q4_pack_k(p, 128))
+    store = (lambda p: p) if packed_k == 0 else (lambda p: orc.q4_pack_k(p, packed_k))
     # split_k=False: so few 256-row tiles would otherwise go to the split 128-row tiles
     variant = dict(M=1024, N=n, K=k, dynamic_rows=True, output_stride=n + 3, split_k=False)
     if packed_k:
