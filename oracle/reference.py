@@ -462,6 +462,34 @@ def expert_dispatch(a_q, a_scale, ids, relative, row_offsets):
     return d, ds, slot_map
 
 
+def rotate_expert_a8(x, signs, ids=None, relative=None, row_offsets=None, swiglu=False, scatter=True):
+    """Rotation + A8 with the routed hand-over of the same launch (rotation_a8.py:452-531, :558-604).
+
+    The row's codes and scale are those of `rotate_a8`.  Without `ids`: (Q, S, Sum) with Sum the
+    integer sum of each row's codes (:499, :530).  With routing, slot = RowOffsets[IDs] +
+    RelativeSlot (:502, :597): scatter gives (Q, S, D, DS, SlotMap, Sum) with the codes, the scale
+    and the sum copied to every slot of the row (:503-510); shared gives (Q, S, DS, SlotMap, Sum)
+    with Sum per row (:596-599).  The reference leaves the codes as two planes of unsigned
+    nibbles, low = q & 15 and high = (q >> 4) & 15 (:489-491): `nibble_planes` gives those.
+    """
+    q, s = rotate_a8(x, signs, swiglu)
+    total = q.astype(np.int32).sum(axis=1).astype(np.int32)
+    if ids is None:
+        return q, s, total
+    d, ds, slot_map = expert_dispatch(q, s, ids, relative, row_offsets)
+    if not scatter:
+        return q, s, ds, slot_map, total
+    slot_sum = np.zeros(d.shape[0], np.int32)
+    slot_sum[slot_map] = total[:, None]
+    return q, s, d, ds, slot_map, slot_sum
+
+
+def nibble_planes(q):
+    """int8 codes -> (low, high) unsigned nibbles of the two's-complement byte (rotation_a8.py:489-491)."""
+    b = np.asarray(q, np.int8).view(np.uint8)
+    return b & 15, b >> 4
+
+
 def moe_combine(expert_out, slot_map, prob, shared=None, shared_gate=None):
     """out = sum_rank fp32(Expert[slot])*prob (+ sigmoid(gate)*shared), one fp16 cast (moe.py:498-554).
 
@@ -516,20 +544,21 @@ def raw_table_words(table):
     return np.ascontiguousarray(np.asarray(table, np.int8)).view("<u4").reshape(256, 2)
 
 
-def moe_layer(x, logits, gate_up_codes, gate_up_scales, down_codes, down_scales, table, top_k, block_m=16):
+def moe_layer(x, logits, gate_up_codes, gate_up_scales, down_codes, down_scales, table, top_k, block_m=16, signs=None):
     """Whole Q2A8 expert layer in the reference's program order
     (tests/cuda/operators/flash_next_quantized.py:117-135; kernels/cuda/model/moe.py):
     top-k -> histogram/offsets -> A8 -> dispatch -> grouped gate_up -> SwiGLU fp16 -> A8 ->
     grouped down -> weighted combine.
 
     gate_up_codes u16 [E, 2I, H/8], down_codes u16 [E, H, I/8] (row-major per expert).
+    `signs`: the input is rotated before the A8 (rotation_a8.py:558-604).
     Returns a dict of every intermediate so kernels can be checked stage by stage.
     """
     e = gate_up_codes.shape[0]
     ids, prob = router_topk(logits, top_k, True)
     counts, relative = expert_histogram(ids, e)
     row_offsets, tile_offsets, tile_count = expert_offsets(counts, block_m)
-    a_q, a_s = a8(x)
+    a_q, a_s = a8(x) if signs is None else rotate_a8(x, signs)
     d, ds, slot_map = expert_dispatch(a_q, a_s, ids, relative, row_offsets)
     w1 = np.stack([q2_integers(gate_up_codes[i], table) for i in range(e)])
     w2 = np.stack([q2_integers(down_codes[i], table) for i in range(e)])

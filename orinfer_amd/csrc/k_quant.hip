@@ -261,14 +261,14 @@ constexpr int kRotateWideRows = 256;  // up to one row per CU
 // a wave takes two blocks of 128 channels per step (one per half
 // wave), a lane holds 4 consecutive channels: stages 1 and 2 are local, stages 4..64 are lane
 // exchanges at distance 1..16.  The rotated fp16 row is kept in LDS for the second pass.
-template <bool SWIGLU, int THREADS = 256>
-__global__ __launch_bounds__(THREADS) void rotate_a8_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
-                                                            int8_t* __restrict__ q, __half* __restrict__ s, int k) {
-    extern __shared__ __align__(16) __half rotated[];  // k halves
-    __shared__ float scratch[THREADS / 64];
+// The rotation pass of one row: the rotated fp16 values go to `rotated` (LDS), the return value is the
+// largest magnitude this thread has seen.
+template <bool SWIGLU, int THREADS>
+__device__ __forceinline__ float rotate_row_to_lds(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                   __half* rotated, int row, int k) {
     constexpr int kWaves = THREADS / 64;
     constexpr int kBatch = THREADS == 256 ? kRotateBatch : 2;  // steps whose loads leave together
-    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int half_wave = lane >> 5, l32 = lane & 31;
     const int blocks = k / 128;
     const int64_t in_base = (int64_t)row * (SWIGLU ? 2 * k : k);
@@ -307,8 +307,78 @@ __global__ __launch_bounds__(THREADS) void rotate_a8_kernel(const __half* __rest
             if (live) *reinterpret_cast<uint2*>(rotated + first) = *reinterpret_cast<const uint2*>(out);
         }
     }
+    return amax;
+}
+
+template <bool SWIGLU, int THREADS = 256>
+__global__ __launch_bounds__(THREADS) void rotate_a8_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                            int8_t* __restrict__ q, __half* __restrict__ s, int k) {
+    extern __shared__ __align__(16) __half rotated[];  // k halves
+    __shared__ float scratch[THREADS / 64];
+    const int row = blockIdx.x;
+    float amax = rotate_row_to_lds<SWIGLU, THREADS>(x, signs, rotated, row, k);
     amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated`
     quantise_row(rotated, amax, q, s, row, k);
+}
+
+// rotate_expert_a8 (kernels/cuda/model/rotation_a8.py:386-422, body :452-531, entry points :558-604):
+// the rotation and the A8 rule of rotate_a8_kernel with the routed hand-over to the expert GEMMs in the
+// same launch.  The reference's expert GEMMs multiply 4-bit planes, so its kernel leaves the codes as
+// two nibble planes plus their sum; the expert GEMMs here multiply int8 rows, so the codes stay whole:
+//   routing "scatter": D[slot] = codes and DS[slot] = scale for each of the row's top_k slots
+//                      (slot = RowOffsets[IDs[row, c]] + RelativeSlot[row, c]), SlotMap[row, c] = slot;
+//   routing "shared":  Q[row] = codes, and only DS[slot] and SlotMap are written per assignment;
+//   no routing:        Q[row], S[row] (and Sum[row]) alone.
+// S[row] is always written; Q (scatter) and Sum may be null.  Sum is the integer sum of a row's codes
+// (per slot under scatter, per row otherwise), the term the reference's unsigned-nibble product needs.
+constexpr int kRouteScatter = 1, kRouteShared = 2;
+constexpr int kMaxRouteChoices = 64;
+template <bool SWIGLU, int THREADS>
+__global__ __launch_bounds__(THREADS) void rotate_expert_kernel(
+    const __half* __restrict__ x, const int8_t* __restrict__ signs, int8_t* __restrict__ q, __half* __restrict__ s,
+    int8_t* __restrict__ d, __half* __restrict__ ds, const int* __restrict__ ids, const int* __restrict__ relative,
+    const int* __restrict__ row_offsets, int* __restrict__ slot_map, int* __restrict__ sum, int k, int top_k,
+    int routing) {
+    extern __shared__ __align__(16) __half rotated[];  // k halves
+    __shared__ float scratch[THREADS / 64];
+    __shared__ int slot_of[kMaxRouteChoices];
+    __shared__ int wave_sum[THREADS / 64];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    if (routing != 0 && tid < top_k) {  // requested first: two dependent reads, hidden behind the rotation
+        const int assignment = row * top_k + tid;
+        const int slot = row_offsets[ids[assignment]] + relative[assignment];
+        slot_of[tid] = slot;
+        slot_map[assignment] = slot;
+    }
+    float amax = rotate_row_to_lds<SWIGLU, THREADS>(x, signs, rotated, row, k);
+    amax = block_max(amax, scratch);  // includes the barrier that publishes `rotated` and `slot_of`
+    const __half stored = a8_scale(amax);
+    if (tid == 0) s[row] = stored;
+    if (routing != 0 && tid < top_k) ds[slot_of[tid]] = stored;
+    const float scale = __half2float(stored), inverse = __frcp_rn(scale);
+    int total = 0;
+    for (int i = tid; i < k / 4; i += THREADS) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(rotated + 4 * i);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const float values[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+        const uint32_t word = quantise4(values, scale, inverse);
+        total += (int)(int8_t)word + (int)(int8_t)(word >> 8) + (int)(int8_t)(word >> 16) + ((int)word >> 24);
+        if (q != nullptr) *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = word;
+        if (routing == kRouteScatter)
+            for (int c = 0; c < top_k; ++c) *reinterpret_cast<uint32_t*>(d + (int64_t)slot_of[c] * k + 4 * i) = word;
+    }
+    if (sum == nullptr) return;  // uniform: one pointer for the whole launch
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) total += __shfl_xor(total, offset, 64);
+    if ((tid & 63) == 0) wave_sum[tid >> 6] = total;
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < THREADS / 64; ++w) total += wave_sum[w];
+        if (routing == kRouteScatter)
+            for (int c = 0; c < top_k; ++c) sum[slot_of[c]] = total;
+        else
+            sum[row] = total;
+    }
 }
 
 // The rotation alone (kernels/cuda/model/integer_vq.py:447-486): Y = fp16(rotated * 128^-1/2), the
@@ -651,6 +721,97 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// rotate_expert_a8: buffers in ASCII order.  scatter: D,DS,IDs,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X;
+// shared: the same without D; no routing: Q,S,Signs,Sum,X.  slots used: K, top_k, E, flags (bit1 swiglu),
+// algorithm (routing).
+int rotate_expert_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    int8_t *q, *d = nullptr;
+    __half *s, *ds = nullptr;
+    const int *ids = nullptr, *relative = nullptr, *row_offsets = nullptr;
+    int *slot_map = nullptr, *sum;
+    const int8_t* signs;
+    const __half* x;
+    if (f.algorithm == 0) {
+        q = pointer_arg<int8_t>(args, 0), s = pointer_arg<__half>(args, 1), signs = pointer_arg<const int8_t>(args, 2);
+        sum = pointer_arg<int>(args, 3), x = pointer_arg<const __half>(args, 4);
+    } else {
+        int i = 0;
+        if (f.algorithm == kRouteScatter) d = pointer_arg<int8_t>(args, i++);
+        ds = pointer_arg<__half>(args, i++), ids = pointer_arg<const int>(args, i++), q = pointer_arg<int8_t>(args, i++);
+        relative = pointer_arg<const int>(args, i++), row_offsets = pointer_arg<const int>(args, i++);
+        s = pointer_arg<__half>(args, i++), signs = pointer_arg<const int8_t>(args, i++);
+        slot_map = pointer_arg<int>(args, i++), sum = pointer_arg<int>(args, i++), x = pointer_arg<const __half>(args, i++);
+    }
+    const dim3 grid(g.grid[0]), block(g.block[0]);
+#define ORX_ROTATE_EXPERT(SW, TH)                                                                                     \
+    hipLaunchKernelGGL((rotate_expert_kernel<SW, TH>), grid, block, g.shared, stream, x, signs, q, s, d, ds, ids,      \
+                       relative, row_offsets, slot_map, sum, f.K, f.top_k, f.algorithm)
+    if (g.block[0] == 1024) {
+        if (f.flags & 2) ORX_ROTATE_EXPERT(true, 1024);
+        else ORX_ROTATE_EXPERT(false, 1024);
+    } else if (f.flags & 2) {
+        ORX_ROTATE_EXPERT(true, 256);
+    } else {
+        ORX_ROTATE_EXPERT(false, 256);
+    }
+#undef ORX_ROTATE_EXPERT
+    return hip_check(hipGetLastError(), "launch rotate_expert_a8");
+}
+
+int make_rotate_expert(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("K", 0, &bad);
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    f->top_k = (int)v.integer("top_k", 1, &bad);
+    f->E = (int)v.integer("experts", 1, &bad);
+    const bool swiglu = v.boolean("swiglu", false, &bad);
+    const bool reciprocal = v.boolean("reciprocal", true, &bad);
+    const bool group_major = v.boolean("group_major", false, &bad);
+    const std::string routing = v.string("routing", "none", &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    (void)reciprocal;  // both forms of the reference give the same codes (the reciprocal one divides near ties)
+    if (f->M <= 0 || f->K <= 0 || f->K % 128 || f->K > 32768) {
+        set_error("rotate_expert_a8: need M > 0 and K a multiple of 128 up to 32768");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (routing != "none" && routing != "shared" && routing != "scatter") {
+        set_error("rotate_expert_a8: routing must be none, shared or scatter");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->top_k < 1 || f->top_k > f->E || f->top_k > kMaxRouteChoices) {
+        set_error("rotate_expert_a8: need 1 <= top_k <= experts and top_k <= %d", kMaxRouteChoices);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (group_major) {
+        set_error("rotate_expert_a8: group_major lays out 4-bit planes for 64-wide K blocks; the expert GEMMs here "
+                  "multiply int8 rows, so there is no such layout");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = swiglu ? 2 : 0;
+    f->algorithm = routing == "scatter" ? kRouteScatter : routing == "shared" ? kRouteShared : 0;
+    const uint32_t nullable = 0x80000000u;
+    if (f->algorithm == 0) {
+        f->args = {{"Q", ArgPointer, 4}, {"S", ArgPointer, 2}, {"Signs", ArgPointer, 4}, {"Sum", ArgPointer, nullable | 4u},
+                   {"X", ArgPointer, 8}};
+    } else {
+        if (f->algorithm == kRouteScatter) f->args.push_back({"D", ArgPointer, 4});
+        const uint32_t q_align = f->algorithm == kRouteScatter ? nullable | 4u : 4u;
+        for (const ArgSpec& a : std::initializer_list<ArgSpec>{{"DS", ArgPointer, 2}, {"IDs", ArgPointer, 4},
+                                                               {"Q", ArgPointer, q_align}, {"RelativeSlot", ArgPointer, 4},
+                                                               {"RowOffsets", ArgPointer, 4}, {"S", ArgPointer, 2},
+                                                               {"Signs", ArgPointer, 4}, {"SlotMap", ArgPointer, 4},
+                                                               {"Sum", ArgPointer, nullable | 4u}, {"X", ArgPointer, 8}})
+            f->args.push_back(a);
+    }
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = nullptr;  // 256- and 1024-thread kernels serve this symbol
+    f->geometry = rotate_a8_geometry;
+    f->launch = rotate_expert_launch;
+    return ORX_OK;
+}
+
 // slots used: K, flags (bit1 swiglu)
 int rotate_geometry(const orx_function&, int rows, Geometry* g) {
     g->grid[0] = (uint32_t)rows;
@@ -808,6 +969,9 @@ const Registration* quant_registrations(int* count) {
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
     {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
+    {"rotate_expert_a8", make_rotate_expert,
+     "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, routing=none|shared|scatter, top_k=1, experts=1",
+     "[D,]DS,IDs,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X[,m] (no routing: Q,S,Signs,Sum,X[,m])"},
     {"rotate_activation", make_rotate, "M, K, swiglu=false", "Signs,X,Y"},
     {"residual_norm_rotate_a8", make_residual_rotate, "M, K=5120, dynamic_rows=false, zero_centered=true",
      "Q,R,RO,S,Signs,W,X,Y[,m]"},

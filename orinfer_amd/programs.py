@@ -78,7 +78,7 @@ class MoeLayer:
     """Q2A8 expert layer: token-sort, grouped gate_up, SwiGLU->A8, grouped down, weighted combine."""
 
     def __init__(self, tokens, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales,
-                 block_m=32, packed_k=128, fused_metadata=None, fused_dispatch=True):
+                 block_m=32, packed_k=128, fused_metadata=None, fused_dispatch=True, signs=None):
         self.tokens, self.experts, self.top_k = tokens, experts, top_k
         self.hidden, self.inter, self.block_m = hidden, intermediate, block_m
         assignments = tokens * top_k
@@ -129,6 +129,13 @@ class MoeLayer:
         self.k_a8 = Kernel("activation_quantization", K=hidden)
         self.k_dispatch = Kernel("expert_dispatch", H=hidden, **common,
                                  **({"input_dtype": "float16"} if self.fused_dispatch else {}))
+        # signs: the layer's input is rotated first (block-128 signed Hadamard); rotation, A8 and the
+        # scatter to the expert-sorted slots are one launch (kernels/cuda/model/rotation_a8.py:558-604)
+        self.signs = None if signs is None else _dev(np.asarray(signs, np.int8))
+        self.k_rotate_dispatch = None
+        if signs is not None:
+            self.k_rotate_dispatch = Kernel("rotate_expert_a8", M=tokens, K=hidden, routing="scatter", top_k=top_k,
+                                            experts=experts)
         grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k)
         self.k_gate_up = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, **grouped)
         self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
@@ -148,7 +155,11 @@ class MoeLayer:
                            TileOffsets=self.tile_offsets)
             self.k_tiles(stream=s, Counts=self.counts, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
                          TileRow=self.tile_row)
-        if self.fused_dispatch:
+        if self.k_rotate_dispatch is not None:
+            self.k_rotate_dispatch(stream=s, D=self.d, DS=self.ds, IDs=self.ids, Q=None, RelativeSlot=self.relative,
+                                   RowOffsets=self.row_offsets, S=self.a_s, Signs=self.signs, SlotMap=self.slot_map,
+                                   Sum=None, X=x16)
+        elif self.fused_dispatch:
             self.k_dispatch(stream=s, A=x16, D=self.d, DS=self.ds, IDs=self.ids, RelativeSlot=self.relative,
                             RowOffsets=self.row_offsets, Scale=None, SlotMap=self.slot_map)
         else:

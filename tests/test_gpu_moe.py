@@ -267,10 +267,10 @@ def test_combine_invalid_slots_and_shared_expert(m, h, slots):
     assert torch.equal(shifted, out) and not flat[:4].any() and not flat[4 + m * h :].any()
 
 
-def run_layer(c, bm, packed_k=128, fused_dispatch=True):
+def run_layer(c, bm, packed_k=128, fused_dispatch=True, signs=None):
     layer = programs.MoeLayer(c["tokens"], c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
                               c["gate_up_scales"], c["down"], c["down_scales"], block_m=bm, packed_k=packed_k,
-                              fused_dispatch=fused_dispatch)
+                              fused_dispatch=fused_dispatch, signs=signs)
     layer.run(gu.dev(c["x"]), gu.dev(c["logits"]))
     gu.sync()
     return layer
@@ -286,8 +286,8 @@ def check_layer(c, layer, bm):
     np.testing.assert_array_equal(gu.host(layer.counts), counts)
     np.testing.assert_array_equal(gu.host(layer.row_offsets), rows)
     np.testing.assert_array_equal(gu.host(layer.tile_count), total)
-    a_q, a_s = orc.a8(c["x"])
-    if not layer.fused_dispatch:  # else the rows are quantised on their way to the slots
+    a_q, a_s = orc.a8(c["x"]) if layer.signs is None else orc.rotate_a8(c["x"], gu.host(layer.signs))
+    if layer.signs is None and not layer.fused_dispatch:  # else the rows are quantised on their way to the slots
         np.testing.assert_array_equal(gu.host(layer.a_q), a_q)
     d, ds, slot = orc.expert_dispatch(a_q, a_s, ids, rel, rows)
     np.testing.assert_array_equal(gu.host(layer.slot_map), slot)
@@ -309,7 +309,7 @@ def check_layer(c, layer, bm):
     staged = orc.moe_combine(down, slot, gu.host(layer.prob)).astype(np.float32)
     assert (np.abs(got - staged) <= 1e-2 + 1e-3 * np.abs(staged)).all()
     full = orc.moe_layer(c["x"], c["logits"], c["gate_up"], c["gate_up_scales"], c["down"], c["down_scales"], TABLE,
-                         c["top_k"], bm)["out"].astype(np.float32)
+                         c["top_k"], bm, signs=None if layer.signs is None else gu.host(layer.signs))["out"].astype(np.float32)
     rel_l2 = np.linalg.norm(got - full) / np.linalg.norm(full)
     assert rel_l2 < 0.003  # flash_next_quantized.py:117-135 accepts the expert FFN at this bar
 
@@ -319,6 +319,8 @@ def test_moe_layer_small_end_to_end():
     for bm in (32, 64):
         check_layer(c, run_layer(c, bm), bm)
     check_layer(c, run_layer(c, 32, fused_dispatch=False), 32)  # quantiser and dispatch as two launches
+    signs = np.random.default_rng(3).choice(np.array([-1, 1], np.int8), c["hidden"])
+    check_layer(c, run_layer(c, 32, signs=signs), 32)  # rotated input: rotation, A8 and scatter in one launch
 
 
 def test_config3_full_size_end_to_end():
@@ -711,3 +713,79 @@ def test_moe_token_layer_matches_the_routed_layer_of_one_token():
     layer.run(x, logits)
     gu.sync()
     assert torch.equal(layer.out, replayed)
+
+
+@pytest.mark.parametrize("swiglu", [False, True], ids=["rows", "swiglu"])
+@pytest.mark.parametrize("m,e,k,h", [(37, 64, 10, 640), (5, 512, 10, 5120), (300, 16, 2, 128)])
+def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, h, swiglu):
+    """rotate_expert_a8: bit-exact against the oracle for every routing form, and the same bits as
+    rotate_activation_a8 followed by expert_dispatch; rows beyond the live count stay untouched."""
+    rng = np.random.default_rng(orc.SEED + 3 * m + h + swiglu)
+    x = rng.normal(size=(m, 2 * h if swiglu else h)).astype(np.float16)
+    x[1] = 0
+    signs = rng.choice(np.array([-1, 1], np.int8), h)
+    ids_np, _ = orc.router_topk(rng.normal(size=(m, e)).astype(np.float32), k)
+    counts, relative = orc.expert_histogram(ids_np, e)
+    offsets, _, _ = orc.expert_offsets(counts, 32)
+    want_q, want_s, want_d, want_ds, want_map, want_sum = orc.rotate_expert_a8(x, signs, ids_np, relative, offsets, swiglu)
+    cap = m + 3
+    pad = lambda a: np.concatenate([a, np.zeros((cap - m,) + a.shape[1:], a.dtype)])
+    d_x, d_signs = gu.dev(pad(x)), gu.dev(signs)
+    d_ids, d_rel, d_off = gu.dev(pad(ids_np)), gu.dev(pad(relative)), gu.dev(offsets)
+    fresh = lambda: dict(
+        q=torch.full((cap, h), 7, dtype=torch.int8, device=gu.DEV), s=torch.full((cap,), 3.0, dtype=torch.float16, device=gu.DEV),
+        d=torch.full((cap * k, h), 7, dtype=torch.int8, device=gu.DEV),
+        ds=torch.full((cap * k,), 3.0, dtype=torch.float16, device=gu.DEV), slot_map=torch.full((cap, k), -1, **I32),
+        total=torch.full((cap * k,), -5, **I32))
+    common = dict(M=cap, K=h, swiglu=swiglu, dynamic_rows=True)
+
+    # scatter: codes, scale and sum land in every slot of the row
+    o = fresh()
+    kern = gu.kernel("rotate_expert_a8", routing="scatter", top_k=k, experts=e, **common)
+    kern(D=o["d"], DS=o["ds"], IDs=d_ids, Q=o["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=o["s"], Signs=d_signs,
+         SlotMap=o["slot_map"], Sum=o["total"], X=d_x, m=m)
+    np.testing.assert_array_equal(gu.host(o["q"])[:m], want_q)
+    np.testing.assert_array_equal(gu.host(o["s"])[:m], want_s[:, 0])
+    np.testing.assert_array_equal(gu.host(o["d"])[: m * k], want_d)
+    np.testing.assert_array_equal(gu.host(o["ds"])[: m * k], want_ds[:, 0])
+    np.testing.assert_array_equal(gu.host(o["slot_map"])[:m], want_map)
+    np.testing.assert_array_equal(gu.host(o["total"])[: m * k], want_sum)
+    assert (gu.host(o["q"])[m:] == 7).all() and (gu.host(o["d"])[m * k:] == 7).all()
+    assert (gu.host(o["ds"])[m * k:] == 3).all() and (gu.host(o["slot_map"])[m:] == -1).all()
+    assert (gu.host(o["total"])[m * k:] == -5).all() and (gu.host(o["s"])[m:] == 3).all()
+    # Q and Sum are optional under scatter
+    lean = fresh()
+    kern(D=lean["d"], DS=lean["ds"], IDs=d_ids, Q=None, RelativeSlot=d_rel, RowOffsets=d_off, S=lean["s"], Signs=d_signs,
+         SlotMap=lean["slot_map"], Sum=None, X=d_x, m=m)
+    assert torch.equal(lean["d"], o["d"]) and torch.equal(lean["ds"], o["ds"]) and torch.equal(lean["slot_map"], o["slot_map"])
+
+    # the two launches it replaces give the same bits
+    two = fresh()
+    gu.kernel("rotate_activation_a8", **common)(Q=two["q"], S=two["s"], Signs=d_signs, X=d_x, m=m)
+    gu.kernel("expert_dispatch", M=cap, H=h, E=e, top_k=k, dynamic_rows=True)(
+        A=two["q"], D=two["d"], DS=two["ds"], IDs=d_ids, RelativeSlot=d_rel, RowOffsets=d_off, Scale=two["s"],
+        SlotMap=two["slot_map"], m=m)
+    for name in ("q", "s", "d", "ds", "slot_map"):
+        assert torch.equal(two[name], o[name]), name
+
+    # shared: the codes stay in Q, every assignment gets its scale and slot
+    sh = fresh()
+    gu.kernel("rotate_expert_a8", routing="shared", top_k=k, experts=e, **common)(
+        DS=sh["ds"], IDs=d_ids, Q=sh["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=sh["s"], Signs=d_signs,
+        SlotMap=sh["slot_map"], Sum=sh["total"], X=d_x, m=m)
+    assert torch.equal(sh["q"], o["q"]) and torch.equal(sh["ds"], o["ds"]) and torch.equal(sh["slot_map"], o["slot_map"])
+    np.testing.assert_array_equal(gu.host(sh["total"])[:m], want_q.astype(np.int32).sum(1))
+    assert (gu.host(sh["total"])[m:] == -5).all()
+
+    # no routing: codes, scale and the row sum
+    plain = fresh()
+    gu.kernel("rotate_expert_a8", **common)(Q=plain["q"], S=plain["s"], Signs=d_signs, Sum=plain["total"], X=d_x, m=m)
+    assert torch.equal(plain["q"], o["q"]) and torch.equal(plain["s"], o["s"])
+    np.testing.assert_array_equal(gu.host(plain["total"])[:m], want_q.astype(np.int32).sum(1))
+
+
+def test_rotate_expert_a8_refuses_what_it_does_not_serve():
+    for variant in (dict(K=192), dict(routing="broadcast"), dict(routing="scatter", top_k=9, experts=8),
+                    dict(routing="scatter", top_k=65, experts=128), dict(group_major=True), dict(M=0)):
+        with pytest.raises(Exception):
+            gu.kernel("rotate_expert_a8", **{**dict(M=4, K=256), **variant})

@@ -652,3 +652,40 @@ def test_int8_swiglu_is_the_fp16_pair_through_the_swiglu_boundary():
     assert float(orc.project(np.full((1, 128), 127, np.int8), np.array([1.0], np.float16), -np.full((1, 128), 127, np.int8),
                              np.array([2.0**-6], np.float16))[0, 0]) == -32256.0  # fp16(-32258.0)
     assert float(big[0, 0]) == 0.0
+
+
+def test_rotate_expert_a8_is_rotation_then_dispatch_and_its_sum_closes_the_nibble_identity():
+    """The fused hand-over adds no arithmetic: its pieces are `rotate_a8` (pinned by the Sylvester
+    matrix above) and `expert_dispatch` (pinned by enumeration).  What is new is Sum; the reference
+    needs it because its planes are unsigned nibbles: sum_k (low + 16 high) - 256 [q < 0] = sum_k q,
+    and an int dot with unsigned planes is repaired by exactly that term."""
+    rng = np.random.default_rng(orc.SEED + 77)
+    m, k, e, top_k = 9, 256, 6, 3
+    x = rng.normal(size=(m, k)).astype(np.float16)
+    x[4] = 0
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    ids = np.stack([rng.choice(e, top_k, replace=False) for _ in range(m)]).astype(np.int32)
+    counts, relative = orc.expert_histogram(ids, e)
+    offsets, _, _ = orc.expert_offsets(counts, 16)
+    q, s, d, ds, slot_map, slot_sum = orc.rotate_expert_a8(x, signs, ids, relative, offsets)
+    want_q, want_s = orc.rotate_a8(x, signs)
+    assert np.array_equal(q, want_q) and np.array_equal(s, want_s)
+    assert sorted(slot_map.ravel().tolist()) == list(range(m * top_k))  # a permutation of the slots
+    for row in range(m):
+        for rank in range(top_k):
+            slot = slot_map[row, rank]
+            assert offsets[ids[row, rank]] <= slot < offsets[ids[row, rank]] + counts[ids[row, rank]]
+            assert np.array_equal(d[slot], q[row]) and ds[slot, 0] == s[row, 0]
+            assert slot_sum[slot] == int(q[row].astype(np.int64).sum())
+    low, high = orc.nibble_planes(q)
+    assert low.max() <= 15 and high.max() <= 15
+    unsigned = low.astype(np.int64) + 16 * high.astype(np.int64)
+    assert np.array_equal(unsigned - 256 * (q < 0), q.astype(np.int64))
+    w = rng.integers(-8, 8, (5, k)).astype(np.int64)
+    repaired = unsigned @ w.T - 256 * ((q < 0).astype(np.int64) @ w.T)
+    assert np.array_equal(repaired, q.astype(np.int64) @ w.T)
+    # shared routing and no routing keep the per-row sum
+    q2, s2, ds2, map2, row_sum = orc.rotate_expert_a8(x, signs, ids, relative, offsets, scatter=False)
+    assert np.array_equal(map2, slot_map) and np.array_equal(ds2, ds) and np.array_equal(row_sum, q.astype(np.int32).sum(1))
+    q3, s3, sum3 = orc.rotate_expert_a8(x, signs)
+    assert np.array_equal(sum3, row_sum) and row_sum[4] == 0 and s[4, 0] == 1
