@@ -22,12 +22,32 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA (5.0 POP/s)
 CACHE_BYTES = 256 << 20        # Infinity Cache
 
-# HBM bytes per launch of the contract kernel from two `rocprofv3 --pmc` runs of
-# `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the
-# same counter reads for a device copy of 44 564 480 bytes in the same run: FETCH_SIZE reads
-# 21772.3 for 43 520 KiB (factor 1.9989), WRITE_SIZE reads 43 520.0 (factor 1.0).
-# Kernel (fp16-input GEMV): fetch 22044.0 -> 45 120 487 B, write 272.0 -> 278 560 B.
-MEASURED_TRAFFIC_BYTES = 45_399_047
+# HBM bytes per launch of the contract kernel come from the committed counter summary (two
+# `rocprofv3 --pmc` runs of `bench.py --traffic-probe`: FETCH_SIZE, then WRITE_SIZE, each scaled by what
+# the same counter reads for a device copy of known size in the same run).  The summary records the
+# launch it was taken on; `measured_traffic` gives nothing when that is not what the handle launches now.
+TRAFFIC_SUMMARY = ROOT / "profiles" / "gemv_q4_config1_m1_hbm_traffic.txt"
+
+
+def measured_traffic(geometry):
+    """(bytes per launch, kernel name) from the counter summary, or (None, None) when the summary is
+    absent, unreadable or was taken on a launch with another grid, block or LDS size."""
+    try:
+        fields = {}
+        for line in TRAFFIC_SUMMARY.read_text().splitlines():
+            if line.startswith("bench-traffic:"):
+                for item in line[len("bench-traffic:"):].split(";"):
+                    key, _, value = item.strip().partition("=")
+                    fields[key] = value.strip()
+        grid, block, shared = geometry
+        if (int(fields["grid"]), int(fields["block"]), int(fields["lds"])) != (grid[0], block[0], shared):
+            return None, None
+        copy_kib = float(fields["copy_kib"])
+        fetch = float(fields["kernel_fetch"]) * copy_kib / float(fields["copy_fetch"])
+        write = float(fields["kernel_write"]) * copy_kib / float(fields["copy_write"])
+        return int(round((fetch + write) * 1024)), fields["kernel"]
+    except (OSError, KeyError, ValueError, ZeroDivisionError):
+        return None, None
 
 
 def parse():
@@ -143,8 +163,10 @@ def main():
         for i in range(copies):
             main_case.step(i, stream.cuda_stream)
         torch.cuda.synchronize()
+        grid, block, shared = main_case.fused.geometry(1)
         print(json.dumps({"traffic_probe": {"copy_bytes_read": probe.numel(), "copy_bytes_written": probe.numel(),
-                                            "projection_launches": copies, "algorithmic_bytes": bytes_c1}}))
+                                            "projection_launches": copies, "algorithmic_bytes": bytes_c1,
+                                            "grid": grid[0], "block": block[0], "lds": shared}}))
         return
     for i in range(args.warmup):
         main_case.step(i, stream.cuda_stream)
@@ -168,6 +190,15 @@ def main():
     # for comparison: the same GEMV on a row that is already int8 (the quantiser is then a launch of its own)
     main_case.quantize(stream.cuda_stream)
     plain_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(min(args.steps, 260), copies))
+    traffic_bytes, traffic_kernel = measured_traffic(main_case.fused.geometry(1))
+    # config 0 (the reference's own CPU-runnable shape) on the same kernel: a second roofline entry
+    c0 = workloads.config0()
+    b0 = workloads.algorithmic_bytes_q4(1, c0["n"], c0["k"])
+    case0 = Q4Case(c0, -(-2 * CACHE_BYTES // (c0["n"] * c0["k"] // 2)), fused_input=True)
+    t0_fused = timed_graph(lambda i, s: case0.project_fp16(i, s), 480)
+    case0.quantize(stream.cuda_stream)
+    t0_plain = timed_graph(lambda i, s: case0.project(i, s), 480)
+    del case0
     result = {
         "metric": "Q4A8 GEMV HBM GB/s (% of peak) + GEMM int8 TOPS (% MFMA peak), 1 GPU",
         "value": round(bytes_c1 / step_seconds / 1e9, 1),
@@ -184,24 +215,25 @@ def main():
         "config": {"workload": "BASELINE config 1: Q4A8 linear K=5120 N=17408, M=1 decode GEMV, step = A8 + projection "
                                "of one fp16 row (one launch: the GEMV quantises the row during its set-up)",
                    "weight_copies_rotated": copies, "algorithmic_bytes_per_step": bytes_c1},
-        "roofline": {"bound": "hbm", "kernel": "gemv_banked_kernel<Q4, 1 row, fp16 input>", "achieved": round(achieved, 1),
+        "roofline": {"bound": "hbm", "kernel": traffic_kernel or "gemv_banked_kernel<Q4, 1 row, fp16 input>",
+                     "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": traffic_bytes,
                      "same_kernel_int8_input": {"us_per_launch": round(plain_seconds * 1e6, 3),
                                                 "achieved": round(bytes_c1 / plain_seconds / 1e9, 1),
-                                                "frac": round(bytes_c1 / plain_seconds / 1e9 / HBM_PEAK_GBS, 4)}},
+                                                "frac": round(bytes_c1 / plain_seconds / 1e9 / HBM_PEAK_GBS, 4)},
+                     "config0": {"workload": "BASELINE config 0: Q4A8 linear K=2560 N=9728, M=1, fp16 row in",
+                                 "bound": "hbm", "algorithmic_bytes": b0, "us_per_launch": round(t0_fused * 1e6, 3),
+                                 "achieved": round(b0 / t0_fused / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": round(b0 / t0_fused / 1e9 / HBM_PEAK_GBS, 4),
+                                 "int8_input_us_per_launch": round(t0_plain * 1e6, 3)}},
     }
 
     extra = {}
     if not args.no_extra:
-        # config 0 GEMV
-        c0 = workloads.config0()
-        b0 = workloads.algorithmic_bytes_q4(1, c0["n"], c0["k"])
-        case0 = Q4Case(c0, -(-2 * CACHE_BYTES // (c0["n"] * c0["k"] // 2)))
-        t = timed_graph(lambda i, s: case0.project(i, s), 480)
-        extra["config0_q4a8_gemv_m1"] = {"us": round(t * 1e6, 3), "GBps": round(b0 / t / 1e9, 1),
-                                         "frac_hbm": round(b0 / t / 1e9 / HBM_PEAK_GBS, 4), "bytes": b0}
-        del case0
+        # config 0 GEMV (int8 row in; the fp16-row form is `roofline.config0`)
+        extra["config0_q4a8_gemv_m1"] = {"us": round(t0_plain * 1e6, 3), "GBps": round(b0 / t0_plain / 1e9, 1),
+                                         "frac_hbm": round(b0 / t0_plain / 1e9 / HBM_PEAK_GBS, 4), "bytes": b0}
         # config 1 sweep
         sweep = {}
         for rows in (1, 8, 32, 128, 512):
