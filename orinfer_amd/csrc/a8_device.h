@@ -51,4 +51,13 @@ __device__ __forceinline__ uint32_t quantise4(const float (&value)[4], float sca
     return low | (high << 16);
 }
 
+// fp16(silu(gate) * up) in fp32 with a stable sigmoid (kernels/cuda/operators/op04_swiglu.py:6-17).
+__device__ __forceinline__ float swiglu_value(__half gate, __half up) {
+    const float g = __half2float(gate), u = __half2float(up);
+    const float e = expf(-fabsf(g));
+    const float sigmoid = __fdiv_rn(g >= 0.f ? 1.0f : e, 1.0f + e);  // one division serves both signs of the gate
+    // one fp16 rounding here: the value a downstream quantiser sees is the materialised fp16
+    return __half2float(__float2half_rn((g * sigmoid) * u));
+}
+
 }  // namespace orx

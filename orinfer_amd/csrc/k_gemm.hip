@@ -37,13 +37,11 @@ bool dense_resident_eligible(int n, int k, int packed_k);
 void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g);
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
-bool grouped_resident_eligible(int n, int k, int block_m, int tiles);
+bool grouped_resident_eligible(int n, int k, int block_m, int tiles, int input, int epilogue, int slots);
 bool grouped_resident_preferred(int rows, int experts, int n);
-void grouped_resident_geometry(int k, Geometry* g);
-int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                            void* out, const int* counts, const int* offsets, const int* tile_expert,
-                            const int* tile_row, const int* tile_count, int n, int k, int tiles, int packed_k,
-                            hipStream_t stream);
+void grouped_resident_geometry(int k, int input, int slots, Geometry* g);
+int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, int packed_k, int input, int epilogue,
+                            int slots, hipStream_t stream);
 int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, const int* counts, const int* offsets, const int* tile_expert, const int* tile_row,
                           const int* tile_count, int n, int k, int tiles, int block_m, int packed_k,
@@ -1022,16 +1020,18 @@ int make_int8_swiglu(const Variant& v, orx_function* f) {
 // (tests/cuda/operators/e8p_decode.py:72-84; kernels/cuda/model/e8p_decode.py:60-73 without Patch)
 // Resident kernel: forced by `algorithm=resident`, chosen by `auto` once the routed rows give every
 // CU a unit of its own.
+// flags2: input form (0 int8 rows per slot, 1 int8 token rows gathered by slot, 2 fp16 rows quantised while
+// staged) + 4 * epilogue (0 plain, 1 SwiGLU).  Anything but 0 is a form of the resident kernel.
 bool grouped_uses_resident(const orx_function& f) {
-    if (f.algorithm == kResident) return true;
-    return f.algorithm == kAuto && grouped_resident_eligible(f.N, f.K, f.block_m, f.tiles) &&
+    if (f.algorithm == kResident || f.flags2 != 0) return true;
+    return f.algorithm == kAuto && grouped_resident_eligible(f.N, f.K, f.block_m, f.tiles, 0, 0, f.capacity) &&
            grouped_resident_preferred(f.capacity, f.E, f.N);
 }
 
 int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
     (void)rows;
     if (grouped_uses_resident(f)) {
-        grouped_resident_geometry(f.K, g);
+        grouped_resident_geometry(f.K, f.flags2 & 3, f.capacity, g);
         return ORX_OK;
     }
     if (f.block_m <= 64 && f.algorithm != kMfma) {
@@ -1044,25 +1044,36 @@ int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
     return ORX_OK;
 }
 
+// position of a buffer in the handle's argument list, -1 when this form has none
+int grouped_arg(const orx_function& f, const char* name) {
+    for (size_t i = 0; i < f.args.size(); ++i)
+        if (std::string(f.args[i].name) == name) return (int)i;
+    return -1;
+}
+
 int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
+    auto buffer = [&](const char* name) -> void* {
+        const int at = grouped_arg(f, name);
+        return at < 0 ? nullptr : pointer_arg<void>(args, at);
+    };
+    GroupedBuffers b;
+    b.a = buffer("A"), b.as = buffer("AS"), b.book = reinterpret_cast<const uint32_t*>(buffer("Book"));
+    b.out = buffer("C"), b.counts = reinterpret_cast<const int*>(buffer("Counts"));
+    b.offsets = reinterpret_cast<const int*>(buffer("Offsets")), b.w = buffer("P");
+    b.tile_count = reinterpret_cast<const int*>(buffer("TileCount"));
+    b.tile_expert = reinterpret_cast<const int*>(buffer("TileExpert"));
+    b.tile_row = reinterpret_cast<const int*>(buffer("TileRow")), b.ws = buffer("WS");
+    b.slot_token = reinterpret_cast<const int*>(buffer("SlotToken"));
+    b.row_max = reinterpret_cast<const int*>(buffer("RowMax")), b.act = buffer("Act"), b.q = buffer("Q");
+    if (grouped_uses_resident(f))
+        return grouped_resident_launch(b, f.N, f.K, f.tiles, f.packed_k, f.flags2 & 3, f.flags2 >> 2, f.capacity, stream);
     GemmParams p = {};
-    p.a = pointer_arg<const int8_t>(args, 0);
-    p.as = pointer_arg<const __half>(args, 1);
-    p.book = pointer_arg<const uint32_t>(args, 2);
-    p.out = pointer_arg<void>(args, 3);
-    p.counts = pointer_arg<const int>(args, 4);
-    p.offsets = pointer_arg<const int>(args, 5);
-    p.w = pointer_arg<const void>(args, 6);
-    p.tile_count = pointer_arg<const int>(args, 7);
-    p.tile_expert = pointer_arg<const int>(args, 8);
-    p.tile_row = pointer_arg<const int>(args, 9);
-    p.ws = pointer_arg<const __half>(args, 10);
+    p.a = reinterpret_cast<const int8_t*>(b.a), p.as = reinterpret_cast<const __half*>(b.as), p.book = b.book, p.out = b.out;
+    p.counts = b.counts, p.offsets = b.offsets, p.w = b.w, p.tile_count = b.tile_count, p.tile_expert = b.tile_expert;
+    p.tile_row = b.tile_row, p.ws = reinterpret_cast<const __half*>(b.ws);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
-    if (grouped_uses_resident(f))
-        return grouped_resident_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
-                                       p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.packed_k, stream);
     if (f.block_m <= 64 && f.algorithm != kMfma)
         return stream_grouped_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
                                      p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.block_m, f.packed_k, stream);
@@ -1079,8 +1090,18 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     f->block_m = (int)v.integer("block_m", 32, &bad);
     f->packed_k = (int)v.integer("packed_k", 128, &bad);
     const std::string grouped_algorithm = v.string("algorithm", "auto", &bad);
+    const std::string input = v.string("input_dtype", "int8", &bad);
+    const bool gather = v.boolean("gather", false, &bad);
+    const std::string epilogue = v.string("epilogue", "none", &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
+    if ((input != "int8" && input != "float16") || (epilogue != "none" && epilogue != "swiglu") ||
+        (input == "float16" && (gather || epilogue != "none"))) {
+        set_error("%s: input_dtype int8 (optionally gather=true, epilogue=swiglu) or float16 (rows with RowMax, plain epilogue)",
+                  name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags2 = (input == "float16" ? 2 : gather ? 1 : 0) + (epilogue == "swiglu" ? 4 : 0);
     if (grouped_algorithm != "auto" && grouped_algorithm != "mfma" && grouped_algorithm != "stream" &&
         grouped_algorithm != "resident") {
         set_error("%s: algorithm must be auto, stream, resident or mfma", name);
@@ -1103,15 +1124,46 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
         set_error("%s: packed_k must be 128 (K-major) or 0 (row-major per expert)", name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kResident && !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles)) {
+    if (f->algorithm == kResident && !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles, 0, 0, f->capacity)) {
         set_error("%s: algorithm=resident needs block_m=32, at most 1024 tiles, N a multiple of 32 and K/128 even or a multiple of 3, K <= 2304",
                   name);
         return ORX_ERR_BAD_VARIANT;
     }
-    f->args = {{"A", ArgPointer, 16},         {"AS", ArgPointer, 2},         {"Book", ArgPointer, 4},
-               {"C", ArgPointer, 2},          {"Counts", ArgPointer, 4},     {"Offsets", ArgPointer, 4},
-               {"P", ArgPointer, 16},         {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
-               {"TileRow", ArgPointer, 4},    {"WS", ArgPointer, 2}};
+    // gather=true: A and AS are per token, SlotToken names every slot's token, and the kernel gathers the rows
+    // while it stages a tile (no dispatch copy).  epilogue=swiglu: N = gate | up; Act (slots, N/2) receives
+    // fp16(silu(gate) * up), RowMax (slots, zero before the launch) is raised to the fp32 bits of every slot's
+    // largest |Act|, and C may be null.  input_dtype=float16: A holds such fp16 rows and RowMax their maxima; the
+    // rows are quantised by the A8 rule while staged, and AS and Q (either may be null) receive scales and codes.
+    // All three are forms of the resident kernel: served where `auto` picks it, or by name.
+    if (f->flags2 != 0) {
+        if ((f->algorithm != kAuto && f->algorithm != kResident) ||
+            !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles, f->flags2 & 3, f->flags2 >> 2, f->capacity) ||
+            (f->algorithm == kAuto && !grouped_resident_preferred(f->capacity, f->E, f->N))) {
+            set_error("%s: gather, epilogue=swiglu and input_dtype=float16 are forms of the resident kernel (block_m=32, "
+                      "at most 4096 gathered slots, K <= 1024 for float16 rows) where the routed rows fill the chip", name);
+            return ORX_ERR_BAD_VARIANT;
+        }
+    }
+    {
+        const uint32_t nullable = 0x80000000u;
+        const bool rows16 = (f->flags2 & 3) == 2, gathered = (f->flags2 & 3) == 1, swiglu = (f->flags2 >> 2) == 1;
+        f->args.clear();
+        f->args.push_back({"A", ArgPointer, 16});
+        f->args.push_back({"AS", ArgPointer, rows16 ? nullable | 2u : 2u});
+        if (swiglu) f->args.push_back({"Act", ArgPointer, 8});
+        f->args.push_back({"Book", ArgPointer, 4});
+        f->args.push_back({"C", ArgPointer, swiglu ? nullable | 8u : 2u});
+        f->args.push_back({"Counts", ArgPointer, 4});
+        f->args.push_back({"Offsets", ArgPointer, 4});
+        f->args.push_back({"P", ArgPointer, 16});
+        if (rows16) f->args.push_back({"Q", ArgPointer, nullable | 8u});
+        if (rows16 || swiglu) f->args.push_back({"RowMax", ArgPointer, 4});
+        if (gathered) f->args.push_back({"SlotToken", ArgPointer, 4});
+        f->args.push_back({"TileCount", ArgPointer, 4});
+        f->args.push_back({"TileExpert", ArgPointer, 4});
+        f->args.push_back({"TileRow", ArgPointer, 4});
+        f->args.push_back({"WS", ArgPointer, 2});
+    }
     f->geometry = grouped_geometry;
     f->launch = grouped_launch;
     // several kernels with different block sizes serve this symbol: report the device-wide limits
@@ -1256,10 +1308,12 @@ const Registration* gemm_registrations(int* count) {
      "A,Output,TokenScale,Weight,WeightScale[,Workspace][,m]"},
     {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=tensor_core|dp4a, block_m, block_n (checked, not used)",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
-    {"e8p_decode_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
-     "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
-    {"integer_vq_grouped", make_q2_grouped, "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma",
-     "A,AS,Book,C,Counts,Offsets,P,TileCount,TileExpert,TileRow,WS"},
+    {"e8p_decode_grouped", make_q2_grouped,
+     "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
+     "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
+    {"integer_vq_grouped", make_q2_grouped,
+     "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
+     "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
     {"integer_experts", make_integer_experts,
      "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},

@@ -22,11 +22,21 @@
 //    staged rows are reused).  What does not divide evenly is finished in a second phase where a
 //    32-channel block is split over K between the waves and summed with LDS integer atomics
 //    (integer addition is exact in any order), so no CU has to run a whole extra unit.
+//  * Three launches of the expert layer can disappear into this kernel (INPUT, EPILOGUE):
+//    - the dispatch copy: int8 token rows are gathered through the slot -> token map while a tile is
+//      staged (kInputGather), so nobody copies a token's row top_k times into slot order;
+//    - the SwiGLU -> A8 launch between the two projections: with kEpilogueSwiglu a wave owns 16 gate
+//      and the 16 matching up channels, so gate and up of one (token, channel) sit in one lane; the
+//      epilogue writes fp16(silu(gate) * up) and raises the slot's largest magnitude with an
+//      integer atomic max (non-negative fp32 bits order like integers).  The next projection
+//      (kInputAct) reads those fp16 rows and maxima and quantises them while it stages a tile.
+//    The arithmetic of every value is that of the separate launches, so the bits are the same.
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
 #include <cmath>
 
+#include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -44,14 +54,27 @@ constexpr uint32_t kBasisBase = 0;             // 256 entries x 16 copies x 8 by
 constexpr uint32_t kMaskBase = 32768;
 constexpr uint32_t kInfoBase = 65536;          // (expert, first row, rows) of every routed tile
 constexpr int kMaxTiles = 1024;
-constexpr uint32_t kSumBase = kInfoBase + kMaxTiles * 12;  // phase-two sums, then the staged token rows
+constexpr uint32_t kRowStatBase = kInfoBase + kMaxTiles * 12;  // per staged row: largest magnitude (32 ints), scale (32 halves)
+constexpr uint32_t kSumBase = kRowStatBase + 256;          // phase-two sums, then the staged token rows
 constexpr int kRowPad = 16;
 constexpr int kSumStride = 33;                 // ints per token row of a phase-two sum block
 constexpr int kSumBlock = 32 * kSumStride;     // ints
 constexpr int kMaxPieces = 5;                  // 16-byte pieces a thread stages per tile (K <= 2560)
+constexpr int kMaxHalfPieces = 4;              // fp16 input: 16-byte pieces of 8 values per thread and tile (K <= 1024)
+constexpr int kMaxSlots = 4096;                // rows gathered by slot: the slot -> token map sits in LDS as u16
+enum { kInputInt8 = 0, kInputGather = 1, kInputAct = 2 };
+enum { kEpiloguePlain = 0, kEpilogueSwiglu = 1 };
 
 struct GroupedParams {
-    const int8_t* a;
+    const int8_t* a;               // kInputInt8: (slots, K) int8; kInputGather: (tokens, K) int8
+    const __half* x;               // kInputAct: (slots, K) fp16
+    const int* slot_token;         // kInputGather: token of every slot
+    const int* row_max_in;         // kInputAct: fp32 bits of every slot's largest magnitude
+    __half* as_out;                // kInputAct: the row scales, written once per slot (may be null)
+    int8_t* q_out;                 // kInputAct: the codes, written once per slot (may be null)
+    __half* act;                   // kEpilogueSwiglu: (slots, N/2) fp16(silu(gate) * up)
+    int* row_max_out;              // kEpilogueSwiglu: raised to the fp32 bits of the slot's largest |act|
+    int slots;
     const uint8_t* w;
     const uint32_t* book;
     const __half* ws;
@@ -84,19 +107,23 @@ __host__ __device__ inline Split phase_two_split(int kb_count) {
 }
 
 // D: K blocks per ring group (the ring depth); K/128 is a multiple of it.
-template <int D>
+template <int D, int INPUT = kInputInt8, int EPILOGUE = kEpiloguePlain>
 __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParams p) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, frag = lane & 31;
     const int kb_count = p.k / 128;
-    const int spans = (p.n + kSpan - 1) / kSpan;
+    // channels a unit covers: 512 outputs, or 256 gate + the 256 matching up channels
+    const int inner = p.n / 2;  // kEpilogueSwiglu: N = gate | up
+    const int spans = EPILOGUE == kEpilogueSwiglu ? (inner + kSpan / 2 - 1) / (kSpan / 2) : (p.n + kSpan - 1) / kSpan;
     const int groups = (int)gridDim.x, group = (int)blockIdx.x;
     const Split split = phase_two_split(kb_count);
     const uint32_t tile_base = kSumBase + (uint32_t)split.per_pass * kSumBlock * 4;
     const int tile_stride = p.k + kRowPad;
     int* sums = reinterpret_cast<int*>(lds + kSumBase);
+    __half* row_scale = reinterpret_cast<__half*>(lds + kRowStatBase);     // kInputAct: scales of the staged rows
+    uint16_t* slot_tokens = reinterpret_cast<uint16_t*>(lds + tile_base + 32 * tile_stride);  // kInputGather
 
     // ---- set-up: two round trips to memory, then one barrier ------------------------------------
     // First trip: the selector table (waves 0-3 build the basis table from it, waves 4-7 the mask
@@ -121,6 +148,8 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
         for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
     }
     for (int i = tid; i < split.per_pass * kSumBlock; i += kThreads) sums[i] = 0;
+    if constexpr (INPUT == kInputGather)  // same trip as the tile list: nothing below waits for slot -> token -> row
+        for (int i = tid; i < p.slots; i += kThreads) slot_tokens[i] = (uint16_t)p.slot_token[i];
     if (listed_here) {
         int* info = reinterpret_cast<int*>(lds + kInfoBase) + 3 * tid;
         info[0] = my_expert, info[1] = my_offset + my_first, info[2] = min(32, my_count - my_first);
@@ -144,7 +173,8 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     int leftover = units - full * groups;
     const int passes = (leftover * kWaves + groups * split.per_pass - 1) / (groups * split.per_pass);
     int my_units = full, first_unit = group * full;
-    if (passes > max(1, kb_count / 8)) {
+    // (phase two reads int8 rows from memory and has the plain epilogue)
+    if (INPUT == kInputAct || EPILOGUE == kEpilogueSwiglu || passes > max(1, kb_count / 8)) {
         first_unit += min(group, leftover);
         if (group < leftover) ++my_units;
         leftover = 0;
@@ -152,8 +182,10 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
 
     // ---- weight stream of this lane ----------------------------------------------------------
     const int64_t kb_step = p.k_major ? (int64_t)p.n * 32 : 32;
+    // kEpilogueSwiglu: n0 is the wave's first inner channel; lanes 0-15 of a half wave stream the gate
+    // rows n0.., lanes 16-31 the up rows inner + n0..
     auto lane_weights = [&](int expert, int n0) -> const uint8_t* {
-        const int64_t row = n0 + frag;
+        const int64_t row = EPILOGUE == kEpilogueSwiglu ? (frag < 16 ? n0 + frag : inner + n0 + frag - 16) : n0 + frag;
         const int64_t offset = p.k_major ? row * 32 : row * kb_count * 32;
         return p.w + (int64_t)expert * p.expert_weight_stride + offset + half * 16;
     };
@@ -174,27 +206,83 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     // Register arrays hold the native vector type: an array of HIP's uint4 struct that is filled in
     // one lambda and read in another is kept in scratch memory by the compiler.
     v4u held[kMaxPieces];
+    int held_max[INPUT == kInputAct ? kMaxHalfPieces : 1];
     const int row_pieces = p.k / 16;
+    const int half_pieces = p.k / 8;  // kInputAct: pieces of 8 fp16 values per row
     auto stage_load = [&](const Tile& t) {
         // unconditional loads of clamped pieces, so that all of them are in flight together
-        const v4u* src = reinterpret_cast<const v4u*>(p.a + (int64_t)(t.rows > 0 ? t.row0 : 0) * p.k);
-        const int last_piece = max(t.rows * row_pieces, 1) - 1;
+        const int first_row = t.rows > 0 ? t.row0 : 0;
+        if constexpr (INPUT == kInputInt8) {
+            const v4u* src = reinterpret_cast<const v4u*>(p.a + (int64_t)first_row * p.k);
+            const int last_piece = max(t.rows * row_pieces, 1) - 1;
 #pragma unroll
-        for (int i = 0; i < kMaxPieces; ++i) held[i] = src[min(tid + i * kThreads, last_piece)];
-    };
-    auto stage_store = [&](const Tile& t) {
-        const int pieces = t.rows * row_pieces;
+            for (int i = 0; i < kMaxPieces; ++i) held[i] = src[min(tid + i * kThreads, last_piece)];
+        } else if constexpr (INPUT == kInputGather) {
+            const int last_piece = max(t.rows * row_pieces, 1) - 1;
 #pragma unroll
-        for (int i = 0; i < kMaxPieces; ++i) {
-            const int piece = tid + i * kThreads;
-            if (piece < pieces) {
+            for (int i = 0; i < kMaxPieces; ++i) {
+                const int piece = min(tid + i * kThreads, last_piece);
                 const int row = piece / row_pieces, col = piece - row * row_pieces;
-                *reinterpret_cast<v4u*>(lds + tile_base + row * tile_stride + col * 16) = held[i];
+                const int64_t token = slot_tokens[first_row + row];
+                held[i] = *reinterpret_cast<const v4u*>(p.a + token * p.k + col * 16);
+            }
+        } else {
+            const int last_piece = max(t.rows * half_pieces, 1) - 1;
+#pragma unroll
+            for (int i = 0; i < kMaxHalfPieces; ++i) {
+                const int piece = min(tid + i * kThreads, last_piece);
+                const int row = piece / half_pieces;
+                held[i] = reinterpret_cast<const v4u*>(p.x + (int64_t)first_row * p.k)[piece];
+                held_max[i] = p.row_max_in[first_row + row];
             }
         }
     };
+    // `publish`: this workgroup holds the tile's first span, so it is the one that writes the
+    // tile's scales (and codes) to memory for whoever wants to look at them.
+    auto stage_store = [&](const Tile& t, bool publish) {
+        if constexpr (INPUT != kInputAct) {
+            const int pieces = t.rows * row_pieces;
+#pragma unroll
+            for (int i = 0; i < kMaxPieces; ++i) {
+                const int piece = tid + i * kThreads;
+                if (piece < pieces) {
+                    const int row = piece / row_pieces, col = piece - row * row_pieces;
+                    *reinterpret_cast<v4u*>(lds + tile_base + row * tile_stride + col * 16) = held[i];
+                }
+            }
+        } else {
+            const int pieces = t.rows * half_pieces;
+#pragma unroll
+            for (int i = 0; i < kMaxHalfPieces; ++i) {
+                const int piece = tid + i * kThreads;
+                if (piece < pieces) {
+                    const int row = piece / half_pieces, col = piece - row * half_pieces;
+                    const __half stored = a8_scale(__int_as_float(held_max[i]));
+                    const float scale = __half2float(stored), inverse = __frcp_rn(scale);
+                    const __half* h = reinterpret_cast<const __half*>(&held[i]);
+                    const float low[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+                    const float high[4] = {__half2float(h[4]), __half2float(h[5]), __half2float(h[6]), __half2float(h[7])};
+                    const uint2 codes = make_uint2(quantise4(low, scale, inverse), quantise4(high, scale, inverse));
+                    *reinterpret_cast<uint2*>(lds + tile_base + row * tile_stride + col * 8) = codes;
+                    if (col == 0) row_scale[row] = stored;
+                    if (publish) {
+                        if (col == 0 && p.as_out != nullptr) p.as_out[t.row0 + row] = stored;
+                        if (p.q_out != nullptr)
+                            *reinterpret_cast<uint2*>(p.q_out + (int64_t)(t.row0 + row) * p.k + col * 8) = codes;
+                    }
+                }
+            }
+        }
+    };
+    // scale of the token in slot `row`
+    auto token_scale_of = [&](int64_t row) -> __half {
+        if constexpr (INPUT == kInputGather) return p.as[slot_tokens[row]];
+        return p.as[row];
+    };
 
     // accumulator register r of a lane: channel 8*(r/4) + 4*half + r%4 of the block, token `frag`
+    // (kEpilogueSwiglu: channels 0-15 of the block are gate channels n0.., 16-31 the up channels
+    // inner + n0.., so registers r and r + 8 hold gate and up of one inner channel)
     struct Scales {
         uint2 weight[4];  // four fp16 channel scales per 8-channel step
         __half token;
@@ -203,25 +291,65 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
         Scales s;
         const __half* scales = p.ws + (int64_t)expert * p.n + n0 + 4 * half;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) s.weight[j] = *reinterpret_cast<const uint2*>(scales + 8 * j);
-        s.token = p.as[row];
+        for (int j = 0; j < 4; ++j) {
+            const int at = EPILOGUE == kEpilogueSwiglu ? (j < 2 ? 8 * j : inner + 8 * (j - 2)) : 8 * j;
+            s.weight[j] = *reinterpret_cast<const uint2*>(scales + at);
+        }
+        if constexpr (INPUT != kInputAct) s.token = token_scale_of(row);
         return s;
     };
-    auto store_block = [&](const v16i& acc, const Scales& scales, int64_t row, int n0) {
+    auto channel_scales = [](const uint2& bits, float (&s)[4]) {
+        const __half2 s01 = *reinterpret_cast<const __half2*>(&bits.x), s23 = *reinterpret_cast<const __half2*>(&bits.y);
+        s[0] = __low2float(s01), s[1] = __high2float(s01), s[2] = __low2float(s23), s[3] = __high2float(s23);
+    };
+    auto pack4 = [](const __half (&h)[4]) {
+        uint2 packed;
+        packed.x = (uint32_t)__half_as_ushort(h[0]) | (uint32_t)__half_as_ushort(h[1]) << 16;
+        packed.y = (uint32_t)__half_as_ushort(h[2]) | (uint32_t)__half_as_ushort(h[3]) << 16;
+        return packed;
+    };
+    auto store_block = [&](const v16i& acc, const Scales& scales, int64_t row, int n0, bool live) {
         const float token_scale = __half2float(scales.token);
-        __half* dst = p.out + row * p.n + n0 + 4 * half;
+        if constexpr (EPILOGUE == kEpiloguePlain) {
+            if (!live) return;
+            __half* dst = p.out + row * p.n + n0 + 4 * half;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint2 bits = scales.weight[j];
-            const __half2 s01 = *reinterpret_cast<const __half2*>(&bits.x), s23 = *reinterpret_cast<const __half2*>(&bits.y);
-            const float s[4] = {__low2float(s01), __high2float(s01), __low2float(s23), __high2float(s23)};
-            __half h[4];
+            for (int j = 0; j < 4; ++j) {
+                float s[4];
+                channel_scales(scales.weight[j], s);
+                __half h[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) h[i] = __float2half_rn(rescale(acc[4 * j + i], s[i], token_scale));
-            uint2 packed;
-            packed.x = (uint32_t)__half_as_ushort(h[0]) | (uint32_t)__half_as_ushort(h[1]) << 16;
-            packed.y = (uint32_t)__half_as_ushort(h[2]) | (uint32_t)__half_as_ushort(h[3]) << 16;
-            *reinterpret_cast<uint2*>(dst + 8 * j) = packed;
+                for (int i = 0; i < 4; ++i) h[i] = __float2half_rn(rescale(acc[4 * j + i], s[i], token_scale));
+                *reinterpret_cast<uint2*>(dst + 8 * j) = pack4(h);
+            }
+        } else {
+            float amax = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float sg[4], su[4];
+                channel_scales(scales.weight[j], sg);
+                channel_scales(scales.weight[j + 2], su);
+                __half gate[4], up[4], value[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    gate[i] = __float2half_rn(rescale(acc[4 * j + i], sg[i], token_scale));
+                    up[i] = __float2half_rn(rescale(acc[4 * (j + 2) + i], su[i], token_scale));
+                    const float v = swiglu_value(gate[i], up[i]);  // already rounded to fp16
+                    value[i] = __float2half_rn(v);
+                    amax = fmaxf(amax, fabsf(v));
+                }
+                if (live) {
+                    const int64_t at = n0 + 8 * j + 4 * half;
+                    *reinterpret_cast<uint2*>(p.act + row * inner + at) = pack4(value);
+                    if (p.out != nullptr) {
+                        *reinterpret_cast<uint2*>(p.out + row * p.n + at) = pack4(gate);
+                        *reinterpret_cast<uint2*>(p.out + row * p.n + inner + at) = pack4(up);
+                    }
+                }
+            }
+            // the two half waves hold different channels of the same token
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            if (live && half == 0) atomicMax(p.row_max_out + row, __float_as_int(amax));
         }
     };
 
@@ -233,9 +361,11 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
         if (u < my_units) {
             const int index = first_unit + u;
             unit.tile = index / spans;
-            unit.n0 = (index - unit.tile * spans) * kSpan + wave * 32;
+            const int span = index - unit.tile * spans;
+            unit.n0 = EPILOGUE == kEpilogueSwiglu ? span * (kSpan / 2) + wave * 16 : span * kSpan + wave * 32;
             const Tile t = tile_info(unit.tile);
-            unit.expert = t.expert, unit.row0 = t.row0, unit.rows = unit.n0 < p.n ? t.rows : 0;
+            unit.expert = t.expert, unit.row0 = t.row0;
+            unit.rows = unit.n0 < (EPILOGUE == kEpilogueSwiglu ? inner : p.n) ? t.rows : 0;
         }
         return unit;
     };
@@ -263,7 +393,9 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
         return piece;
     };
     auto piece_rows = [&](const Piece& piece) {
-        return p.a + (int64_t)(piece.tile.row0 + min(frag, piece.tile.rows - 1)) * p.k + half * 64;
+        int64_t row = piece.tile.row0 + min(frag, piece.tile.rows - 1);
+        if constexpr (INPUT == kInputGather) row = slot_tokens[row];
+        return p.a + row * p.k + half * 64;
     };
     const Piece early = piece_of(0);
     uint4 early_codes = make_uint4(0, 0, 0, 0), early_tokens[4];
@@ -291,7 +423,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
             } else {
                 __syncthreads();  // every wave has finished with the rows staged before
             }
-            stage_store(staged_tile);
+            stage_store(staged_tile, (first_unit + u) % spans == 0);
             staged = cur.tile;
             __syncthreads();
         }
@@ -312,7 +444,8 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
                 for (int d = 0; d < D; ++d) ring[d] = fetch(weights, d);
             }
             const int64_t row = cur.row0 + min(frag, cur.rows - 1);
-            const Scales scales = load_scales(cur.expert, row, cur.n0);
+            Scales scales = load_scales(cur.expert, row, cur.n0);
+            if constexpr (INPUT == kInputAct) scales.token = row_scale[min(frag, cur.rows - 1)];
             const uint8_t* rows = lds + tile_base + min(frag, cur.rows - 1) * tile_stride + half * 64;
             v16i acc;
 #pragma unroll
@@ -342,7 +475,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
 #pragma unroll
                 for (int s = 0; s < 4; ++s) early_tokens[s] = fragment[s];
             }
-            if (frag < cur.rows) store_block(acc, scales, row, cur.n0);
+            store_block(acc, scales, row, cur.n0, frag < cur.rows);
         }
     }
 
@@ -400,7 +533,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
             const int64_t row = t.row0 + token;
             const int total = sums[e * kSumBlock + token * kSumStride + channel];
             const float value = rescale(total, __half2float(p.ws[(int64_t)t.expert * p.n + n0 + channel]),
-                                        __half2float(p.as[row]));
+                                        __half2float(token_scale_of(row)));
             p.out[row * p.n + n0 + channel] = __float2half_rn(value);
         }
     }
@@ -412,9 +545,10 @@ int ring_depth(int k) {
     return kb % 2 == 0 ? 2 : kb % 3 == 0 ? 3 : 0;
 }
 
-uint32_t resident_lds_bytes(int k) {
+uint32_t resident_lds_bytes(int k, int input, int slots) {
     const Split split = phase_two_split(k / 128);
-    return kSumBase + (uint32_t)split.per_pass * kSumBlock * 4u + 32u * (uint32_t)(k + kRowPad);
+    const uint32_t rows = kSumBase + (uint32_t)split.per_pass * kSumBlock * 4u + 32u * (uint32_t)(k + kRowPad);
+    return rows + (input == kInputGather ? (((uint32_t)slots * 2u + 15u) & ~15u) : 0u);
 }
 
 constexpr uint32_t kLdsLimit = 160 * 1024;
@@ -422,10 +556,15 @@ constexpr uint32_t kLdsLimit = 160 * 1024;
 }  // namespace
 
 // Shapes the resident kernel takes: tiles of at most 32 rows, whole 32-channel blocks, a K whose
-// blocks divide into ring groups and whose staged rows fit beside the tables.
-bool grouped_resident_eligible(int n, int k, int block_m, int tiles) {
+// blocks divide into ring groups and whose staged rows fit beside the tables.  Gathered rows keep
+// the slot -> token map in LDS; fp16 rows are held in registers while a tile is quantised, which
+// bounds K; the SwiGLU epilogue pairs 16 gate with 16 up channels per wave.
+bool grouped_resident_eligible(int n, int k, int block_m, int tiles, int input, int epilogue, int slots) {
+    if (input == kInputGather && slots > kMaxSlots) return false;
+    if (input == kInputAct && k > kMaxHalfPieces * kThreads * 8 / 32) return false;
+    if (epilogue == kEpilogueSwiglu && n % 32 != 0) return false;  // inner = N/2 a multiple of 16
     return block_m == 32 && n % 32 == 0 && k % 128 == 0 && ring_depth(k) > 0 && tiles <= kMaxTiles &&
-           k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k) <= kLdsLimit;
+           k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k, input, slots) <= kLdsLimit;
 }
 
 // Worth it once the routed tiles give most CUs a unit of their own; below that the streaming
@@ -438,21 +577,27 @@ bool grouped_resident_preferred(int rows, int experts, int n) {
     return tiles * ((n + kSpan - 1) / kSpan) >= 0.8 * device_compute_units();
 }
 
-void grouped_resident_geometry(int k, Geometry* g) {
+void grouped_resident_geometry(int k, int input, int slots, Geometry* g) {
     g->grid[0] = (uint32_t)device_compute_units();
     g->grid[1] = g->grid[2] = 1;
     g->block[0] = kThreads;
-    g->shared = resident_lds_bytes(k);
+    g->shared = resident_lds_bytes(k, input, slots);
 }
 
-int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                            void* out, const int* counts, const int* offsets, const int* tile_expert,
-                            const int* tile_row, const int* tile_count, int n, int k, int tiles, int packed_k,
-                            hipStream_t stream) {
+int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, int packed_k, int input, int epilogue,
+                            int slots, hipStream_t stream) {
     static DeviceOnce opted_in;  // dynamic LDS above 64 KiB needs an opt-in per kernel and device
     const int ready = opted_in.run([] {
-        const void* kernels[] = {reinterpret_cast<const void*>(&grouped_resident_kernel<3>),
-                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2>)};
+        const void* kernels[] = {reinterpret_cast<const void*>(&grouped_resident_kernel<3, kInputInt8, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2, kInputInt8, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<3, kInputGather, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2, kInputGather, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<3, kInputAct, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2, kInputAct, kEpiloguePlain>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<3, kInputInt8, kEpilogueSwiglu>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2, kInputInt8, kEpilogueSwiglu>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<3, kInputGather, kEpilogueSwiglu>),
+                                 reinterpret_cast<const void*>(&grouped_resident_kernel<2, kInputGather, kEpilogueSwiglu>)};
         for (const void* kernel : kernels) {
             const int code = hip_check(
                 hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsLimit), "hipFuncSetAttribute");
@@ -461,20 +606,46 @@ int grouped_resident_launch(const int8_t* a, const void* w, const uint32_t* book
         return (int)ORX_OK;
     });
     if (ready != ORX_OK) return ready;
+    const int depth = ring_depth(k);
+    if (depth == 0 || input < 0 || input > 2 || epilogue < 0 || epilogue > 1 || (input == kInputAct && epilogue != 0)) {
+        set_error("routed projection: K=%d, input %d, epilogue %d is not a form of the resident kernel", k, input, epilogue);
+        return ORX_ERR_BAD_VARIANT;
+    }
     GroupedParams p = {};
-    p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as;
-    p.out = reinterpret_cast<__half*>(out);
-    p.counts = counts, p.offsets = offsets, p.tile_expert = tile_expert, p.tile_row = tile_row, p.tile_count = tile_count;
+    if (input == kInputAct) {
+        p.x = reinterpret_cast<const __half*>(b.a), p.as_out = reinterpret_cast<__half*>(const_cast<void*>(b.as));
+        p.row_max_in = b.row_max, p.q_out = reinterpret_cast<int8_t*>(b.q);
+    } else {
+        p.a = reinterpret_cast<const int8_t*>(b.a), p.as = reinterpret_cast<const __half*>(b.as);
+        p.slot_token = b.slot_token;
+    }
+    if (epilogue == kEpilogueSwiglu) p.act = reinterpret_cast<__half*>(b.act), p.row_max_out = const_cast<int*>(b.row_max);
+    p.slots = slots;
+    p.w = reinterpret_cast<const uint8_t*>(b.w), p.book = b.book, p.ws = reinterpret_cast<const __half*>(b.ws);
+    p.out = reinterpret_cast<__half*>(b.out);
+    p.counts = b.counts, p.offsets = b.offsets, p.tile_expert = b.tile_expert, p.tile_row = b.tile_row;
+    p.tile_count = b.tile_count;
     p.n = n, p.k = k, p.k_major = packed_k != 0, p.tile_capacity = tiles;
     p.expert_weight_stride = (int64_t)n * (k / 8) * 2;
     Geometry g;
-    grouped_resident_geometry(k, &g);
+    grouped_resident_geometry(k, input, slots, &g);
     const dim3 grid(g.grid[0]), block(kThreads);
-    switch (ring_depth(k)) {
-        case 3: hipLaunchKernelGGL(grouped_resident_kernel<3>, grid, block, g.shared, stream, p); break;
-        case 2: hipLaunchKernelGGL(grouped_resident_kernel<2>, grid, block, g.shared, stream, p); break;
-        default: set_error("routed projection: K=%d does not divide into ring groups", k); return ORX_ERR_BAD_VARIANT;
+#define ORX_GROUPED(D, IN, EP) hipLaunchKernelGGL((grouped_resident_kernel<D, IN, EP>), grid, block, g.shared, stream, p)
+#define ORX_GROUPED_DEPTH(IN, EP)           \
+    do {                                    \
+        if (depth == 3) ORX_GROUPED(3, IN, EP); \
+        else ORX_GROUPED(2, IN, EP);        \
+    } while (0)
+    if (epilogue == kEpiloguePlain) {
+        if (input == kInputInt8) ORX_GROUPED_DEPTH(kInputInt8, kEpiloguePlain);
+        else if (input == kInputGather) ORX_GROUPED_DEPTH(kInputGather, kEpiloguePlain);
+        else ORX_GROUPED_DEPTH(kInputAct, kEpiloguePlain);
+    } else {
+        if (input == kInputInt8) ORX_GROUPED_DEPTH(kInputInt8, kEpilogueSwiglu);
+        else ORX_GROUPED_DEPTH(kInputGather, kEpilogueSwiglu);
     }
+#undef ORX_GROUPED_DEPTH
+#undef ORX_GROUPED
     return hip_check(hipGetLastError(), "launch routed projection (resident)");
 }
 

@@ -57,13 +57,58 @@ __device__ __forceinline__ float wave_sum(float v) {
 // One wave per row; each lane keeps ceil(E/64) keys in registers.  Key = ordered score in the
 // high word, (E - id) in the low word, so one max picks the score and the lowest id on ties.
 constexpr int kMaxLocal = 16;  // E <= 1024
-template <int LOCAL>  // keys per lane: ceil(E / 64) rounded up to a power of two
-__global__ __launch_bounds__(256) void router_topk_kernel(const float* __restrict__ logits, int* __restrict__ ids,
-                                                          float* __restrict__ prob, int m, int e, int top_k,
-                                                          int renormalize) {
+// The A8 quantiser of one row of fp16 values by one wave (the rule of a8_device.h).
+__device__ __forceinline__ void wave_quantise_row(const __half* __restrict__ x, int8_t* __restrict__ q,
+                                                  __half* __restrict__ s, int row, int h, int lane) {
+    constexpr int kHeldPieces = 4;  // 16-byte pieces a lane keeps in registers (the whole row up to h = 2048)
+    const int pieces = h / 8;
+    const uint4* row_pieces = reinterpret_cast<const uint4*>(x + (int64_t)row * h);
+    uint4 held[kHeldPieces];
+#pragma unroll
+    for (int i = 0; i < kHeldPieces; ++i) held[i] = row_pieces[min(lane + 64 * i, pieces - 1)];
+    auto piece_at = [&](int i) { return i < kHeldPieces ? held[i] : row_pieces[lane + 64 * i]; };
+    float amax = 0.f;
+    for (int i = 0; lane + 64 * i < pieces; ++i) {
+        const uint4 raw = piece_at(i);
+        const __half2* pairs = reinterpret_cast<const __half2*>(&raw);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float2 f = __half22float2(pairs[j]);
+            amax = fmaxf(amax, fmaxf(fabsf(f.x), fabsf(f.y)));
+        }
+    }
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
+    const __half stored = a8_scale(amax);
+    if (lane == 0) s[row] = stored;
+    const float scale = __half2float(stored), inverse = __frcp_rn(scale);
+    for (int i = 0; lane + 64 * i < pieces; ++i) {
+        const uint4 raw = piece_at(i);
+        const __half* v = reinterpret_cast<const __half*>(&raw);
+        const float low[4] = {__half2float(v[0]), __half2float(v[1]), __half2float(v[2]), __half2float(v[3])};
+        const float high[4] = {__half2float(v[4]), __half2float(v[5]), __half2float(v[6]), __half2float(v[7])};
+        reinterpret_cast<uint2*>(q + (int64_t)row * h)[lane + 64 * i] =
+            make_uint2(quantise4(low, scale, inverse), quantise4(high, scale, inverse));
+    }
+}
+
+// QUANT (quantize_hidden): four more waves per workgroup quantise the same four tokens' hidden rows
+// by the A8 rule while the first four select the routes (the expert projections gather these rows
+// by slot, so a row is quantised once, not once per route, and it costs no launch of its own).
+template <int LOCAL, bool QUANT>  // LOCAL keys per lane: ceil(E / 64) rounded up to a power of two
+__global__ __launch_bounds__(QUANT ? 512 : 256) void router_topk_kernel(const float* __restrict__ logits,
+                                                                        int* __restrict__ ids, float* __restrict__ prob, int m,
+                                                                        int e, int top_k, int renormalize,
+                                                                        const __half* __restrict__ x, int8_t* __restrict__ q,
+                                                                        __half* __restrict__ s, int h) {
     const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6;
+    const int row = blockIdx.x * 4 + (wave & 3);
     if (row >= m) return;
+    if (QUANT && wave >= 4) {
+        wave_quantise_row(x, q, s, row, h, lane);
+        return;
+    }
     unsigned long long keys[LOCAL];
     float all_exp = 0.f;
     float local_max = -INFINITY;
@@ -258,7 +303,8 @@ constexpr int kMetaWaves = 16, kMetaThreads = kMetaWaves * 64;
 __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
     const int* __restrict__ ids, int* __restrict__ counts, int* __restrict__ relative, int* __restrict__ row_offsets,
     int* __restrict__ tile_count, int* __restrict__ tile_expert, int* __restrict__ tile_offsets, int* __restrict__ tile_row,
-    int m, int experts, int top_k, int block_m) {
+    int* __restrict__ slot_map, int* __restrict__ slot_token, int* __restrict__ row_max, int m, int experts, int top_k,
+    int block_m) {
     extern __shared__ int meta_lds[];
     int* counters = meta_lds;                          // [kMetaWaves][experts]
     int* wave_rows = counters + kMetaWaves * experts;  // [kMetaWaves]
@@ -308,8 +354,11 @@ __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
     }
     __syncthreads();
     // global relative slots, written once and coalesced
-    for (int at = tid; at < assignments; at += kMetaThreads)
-        relative[at] = local[at] + counters[(at / per_wave) * experts + local_id[at]];
+    for (int at = tid; at < assignments; at += kMetaThreads) {
+        const int slot_in_expert = local[at] + counters[(at / per_wave) * experts + local_id[at]];
+        relative[at] = slot_in_expert;
+        local[at] = slot_in_expert;
+    }
     // exclusive scans of count and ceil(count / block_m) over the experts (one per thread)
     const int tiles = (count + block_m - 1) / block_m;
     int row_scan = count, tile_scan = tiles;
@@ -326,14 +375,27 @@ __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
         tile_total += wave_tiles[w];
     }
     if (tid == 0) tile_count[0] = tile_total;
+    // (the barrier above also ended the reads of the counter rows: row 0 now takes the row offsets)
     if (tid < experts) {
         const int first_tile = tile_base + tile_scan - tiles;
         row_offsets[tid] = row_base + row_scan - count;
+        if (slot_map != nullptr) counters[tid] = row_base + row_scan - count;
         tile_offsets[tid] = first_tile;
         for (int t = 0; t < tiles; ++t) {
             tile_expert[first_tile + t] = tid;
             tile_row[first_tile + t] = t * block_m;
         }
+    }
+    // slot_maps: what the dispatch would compute, slot = RowOffsets[expert] + RelativeSlot, and its
+    // inverse (the token of every slot), so that no launch has to copy rows into slot order; and the
+    // per-slot maxima the expert projection's SwiGLU epilogue raises start at zero
+    if (slot_map == nullptr) return;
+    __syncthreads();
+    for (int at = tid; at < assignments; at += kMetaThreads) {
+        const int slot = counters[local_id[at]] + local[at];
+        slot_map[at] = slot;
+        slot_token[slot] = at / top_k;
+        row_max[at] = 0;
     }
 }
 
@@ -540,26 +602,35 @@ bool geometry_fields(const Variant& v, orx_function* f, bool need_m) {
     return !bad;
 }
 
-int rows_geometry_router(const orx_function&, int rows, Geometry* g) {
+int rows_geometry_router(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, 4u);
-    g->block[0] = 256;
+    g->block[0] = f.H > 0 ? 512 : 256;  // quantize_hidden: four more waves quantise the four tokens' rows
     return ORX_OK;
 }
+// IDs, Logits, Prob[, Q, S, X][, m]
 int router_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
     const float* logits = pointer_arg<const float>(args, 1);
     int* ids = pointer_arg<int>(args, 0);
     float* prob = pointer_arg<float>(args, 2);
-    const dim3 grid(g.grid[0]), block(256);
-    if (f.E <= 64)
-        hipLaunchKernelGGL(router_topk_kernel<1>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
-    else if (f.E <= 128)
-        hipLaunchKernelGGL(router_topk_kernel<2>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
-    else if (f.E <= 256)
-        hipLaunchKernelGGL(router_topk_kernel<4>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
-    else if (f.E <= 512)
-        hipLaunchKernelGGL(router_topk_kernel<8>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
-    else
-        hipLaunchKernelGGL(router_topk_kernel<16>, grid, block, 0, s, logits, ids, prob, rows, f.E, f.top_k, f.flags);
+    const __half* x = f.H > 0 ? pointer_arg<const __half>(args, 5) : nullptr;
+    int8_t* q = f.H > 0 ? pointer_arg<int8_t>(args, 3) : nullptr;
+    __half* scale = f.H > 0 ? pointer_arg<__half>(args, 4) : nullptr;
+    const dim3 grid(g.grid[0]), block(g.block[0]);
+#define ORX_ROUTER(LOCAL)                                                                                              \
+    do {                                                                                                               \
+        if (f.H > 0)                                                                                                   \
+            hipLaunchKernelGGL((router_topk_kernel<LOCAL, true>), grid, block, 0, s, logits, ids, prob, rows, f.E,     \
+                               f.top_k, f.flags, x, q, scale, f.H);                                                    \
+        else                                                                                                           \
+            hipLaunchKernelGGL((router_topk_kernel<LOCAL, false>), grid, block, 0, s, logits, ids, prob, rows, f.E,    \
+                               f.top_k, f.flags, x, q, scale, f.H);                                                    \
+    } while (0)
+    if (f.E <= 64) ORX_ROUTER(1);
+    else if (f.E <= 128) ORX_ROUTER(2);
+    else if (f.E <= 256) ORX_ROUTER(4);
+    else if (f.E <= 512) ORX_ROUTER(8);
+    else ORX_ROUTER(16);
+#undef ORX_ROUTER
     return hip_check(hipGetLastError(), "launch router_topk");
 }
 int make_router(const Variant& v, orx_function* f) {
@@ -571,11 +642,18 @@ int make_router(const Variant& v, orx_function* f) {
         set_error("router_topk: invalid MoE router dimensions (need top_k <= min(E,64), E <= 1024)");
         return ORX_ERR_BAD_VARIANT;
     }
+    // quantize_hidden=H: the launch also writes the A8 codes Q (M, H) and scales S (M) of the fp16 rows X (M, H)
+    f->H = (int)v.integer("quantize_hidden", 0, &bad);
+    if (bad || f->H < 0 || f->H % 8) {
+        set_error("router_topk: quantize_hidden must be a multiple of 8");
+        return ORX_ERR_BAD_VARIANT;
+    }
     f->args = {{"IDs", ArgPointer, 4}, {"Logits", ArgPointer, 4}, {"Prob", ArgPointer, 4}};
+    if (f->H > 0) f->args.push_back({"Q", ArgPointer, 8}), f->args.push_back({"S", ArgPointer, 2}), f->args.push_back({"X", ArgPointer, 16});
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = rows_geometry_router;
     f->launch = router_launch;
-    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel<16>);
+    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel<16, false>);
     return ORX_OK;
 }
 
@@ -676,8 +754,8 @@ int metadata_geometry(const orx_function& f, int, Geometry* g) {
     g->shared = (uint32_t)((kMetaWaves * f.E + 2 * kMetaWaves + 2 * f.M * f.top_k) * sizeof(int));
     return ORX_OK;
 }
-// Counts, IDs, RelativeSlot, RowOffsets, TileCount, TileExpert, TileOffsets, TileRow[, m]
-// (moe.py:726-735 in generated-ABI order)
+// Counts, IDs, RelativeSlot, [RowMax,] RowOffsets, [SlotMap, SlotToken,] TileCount, TileExpert, TileOffsets, TileRow[, m]
+// (moe.py:726-735 in generated-ABI order; slot_maps=true adds the two slot tables and the zeroed RowMax)
 int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
     static DeviceOnce opted_in;  // 64 KiB of counters at E = 1024 needs the LDS opt-in
     const int ready = opted_in.run([] {
@@ -686,10 +764,14 @@ int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStrea
                          "hipFuncSetAttribute");
     });
     if (ready != ORX_OK) return ready;
+    const bool maps = f.flags & 1;
+    const int offsets_at = maps ? 4 : 3, tiles_at = maps ? 7 : 4;
     hipLaunchKernelGGL(route_metadata_kernel, dim3(1), dim3(kMetaThreads), g.shared, s, pointer_arg<const int>(args, 1),
-                       pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), pointer_arg<int>(args, 3),
-                       pointer_arg<int>(args, 4), pointer_arg<int>(args, 5), pointer_arg<int>(args, 6),
-                       pointer_arg<int>(args, 7), rows, f.E, f.top_k, f.block_m);
+                       pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), pointer_arg<int>(args, offsets_at),
+                       pointer_arg<int>(args, tiles_at), pointer_arg<int>(args, tiles_at + 1),
+                       pointer_arg<int>(args, tiles_at + 2), pointer_arg<int>(args, tiles_at + 3),
+                       maps ? pointer_arg<int>(args, 5) : nullptr, maps ? pointer_arg<int>(args, 6) : nullptr,
+                       maps ? pointer_arg<int>(args, 3) : nullptr, rows, f.E, f.top_k, f.block_m);
     return hip_check(hipGetLastError(), "launch route_metadata");
 }
 int make_metadata(const Variant& v, orx_function* f) {
@@ -703,9 +785,16 @@ int make_metadata(const Variant& v, orx_function* f) {
         set_error("route_metadata: need E <= 1024, top_k <= E, a valid block_m and M*top_k small enough for LDS");
         return ORX_ERR_BAD_VARIANT;
     }
-    f->args = {{"Counts", ArgPointer, 4},     {"IDs", ArgPointer, 4},        {"RelativeSlot", ArgPointer, 4},
-               {"RowOffsets", ArgPointer, 4}, {"TileCount", ArgPointer, 4},  {"TileExpert", ArgPointer, 4},
-               {"TileOffsets", ArgPointer, 4}, {"TileRow", ArgPointer, 4}};
+    const bool slot_maps = v.boolean("slot_maps", false, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    f->flags = slot_maps ? 1 : 0;
+    f->args = {{"Counts", ArgPointer, 4}, {"IDs", ArgPointer, 4}, {"RelativeSlot", ArgPointer, 4}};
+    if (slot_maps) f->args.push_back({"RowMax", ArgPointer, 4});
+    f->args.push_back({"RowOffsets", ArgPointer, 4});
+    if (slot_maps) f->args.push_back({"SlotMap", ArgPointer, 4}), f->args.push_back({"SlotToken", ArgPointer, 4});
+    for (const ArgSpec& a : std::initializer_list<ArgSpec>{{"TileCount", ArgPointer, 4}, {"TileExpert", ArgPointer, 4},
+                                                           {"TileOffsets", ArgPointer, 4}, {"TileRow", ArgPointer, 4}})
+        f->args.push_back(a);
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = metadata_geometry;
     f->launch = metadata_launch;
@@ -901,13 +990,14 @@ int make_combine(const Variant& v, orx_function* f) {
 
 const Registration* moe_registrations(int* count) {
     static const Registration rows[] = {
-    {"router_topk", make_router, "M, E=512, top_k=10, renormalize=true, dynamic_rows=false", "IDs,Logits,Prob[,m]"},
+    {"router_topk", make_router, "M, E=512, top_k=10, renormalize=true, dynamic_rows=false, quantize_hidden=0",
+     "IDs,Logits,Prob[,Q,S,X][,m]"},
     {"router_topk_warp", make_router_warp, "M, E, top_k, dynamic_rows=false, warps=4", "IDs,Logits,Prob[,m]"},
     {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
     {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
-    {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false",
-     "Counts,IDs,RelativeSlot,RowOffsets,TileCount,TileExpert,TileOffsets,TileRow[,m]"},
+    {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false, slot_maps=false",
+     "Counts,IDs,RelativeSlot[,RowMax],RowOffsets[,SlotMap,SlotToken],TileCount,TileExpert,TileOffsets,TileRow[,m]"},
     {"single_route_metadata", make_single_metadata, "E=512, top_k=10, capacity=11",
      "Counts,IDs,Offsets,Relative,TileCount,TileExpert,TileOffsets,TileRow"},
     {"expert_partition_offsets", make_partition_offsets, "experts, hot_m, cold_m, cold_rows",

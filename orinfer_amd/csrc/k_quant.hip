@@ -24,14 +24,6 @@
 namespace orx {
 namespace {
 
-__device__ __forceinline__ float swiglu_value(__half gate, __half up) {
-    const float g = __half2float(gate), u = __half2float(up);
-    const float e = expf(-fabsf(g));
-    const float sigmoid = __fdiv_rn(g >= 0.f ? 1.0f : e, 1.0f + e);  // one division serves both signs of the gate
-    // one fp16 rounding here: the value a downstream quantiser sees is the materialised fp16
-    return __half2float(__float2half_rn((g * sigmoid) * u));
-}
-
 template <bool FUSED, bool MASKED>
 __device__ __forceinline__ float load_value(const __half* __restrict__ x, const uint8_t* __restrict__ mask,
                                             int64_t row_base, int k, int col) {

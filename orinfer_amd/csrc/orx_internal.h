@@ -109,6 +109,25 @@ int current_device();
 // Compute units of the current device (256 where no device answers).  Cached per device.
 int device_compute_units();
 
+// Buffers of a routed expert projection as the resident kernel takes them (null where a form has none).
+struct GroupedBuffers {
+    const void* a = nullptr;        // rows: int8 (slots, K); gathered: int8 (tokens, K); fp16 (slots, K) values to quantise
+    const void* as = nullptr;       // row scales (per slot, or per token when gathered); an output for fp16 rows
+    const void* w = nullptr;
+    const uint32_t* book = nullptr;
+    const void* ws = nullptr;       // fp16 channel scales (E, N)
+    void* out = nullptr;            // fp16 (slots, N); optional with the SwiGLU epilogue
+    const int* counts = nullptr;
+    const int* offsets = nullptr;
+    const int* tile_expert = nullptr;
+    const int* tile_row = nullptr;
+    const int* tile_count = nullptr;
+    const int* slot_token = nullptr;  // gathered rows: token of every slot
+    const int* row_max = nullptr;     // fp32 bits of every slot's largest magnitude: read with fp16 rows, raised by the SwiGLU epilogue
+    void* act = nullptr;              // SwiGLU epilogue: fp16 (slots, N/2)
+    void* q = nullptr;                // fp16 rows: the codes, optional
+};
+
 // One-time set-up that has to happen once per DEVICE (function attributes are per device), safe to
 // reach from several session threads: the set-up itself is idempotent, the flag is atomic.
 struct DeviceOnce {

@@ -11,7 +11,7 @@ import numpy as np
 import torch
 
 from . import codebook
-from .lib import Kernel
+from .lib import ORX_ERR_BAD_VARIANT, Kernel, OrxError
 
 
 def _dev(array):
@@ -78,7 +78,8 @@ class MoeLayer:
     """Q2A8 expert layer: token-sort, grouped gate_up, SwiGLU->A8, grouped down, weighted combine."""
 
     def __init__(self, tokens, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales,
-                 block_m=32, packed_k=128, fused_metadata=None, fused_dispatch=True, signs=None):
+                 block_m=32, packed_k=128, fused_metadata=None, fused_dispatch=True, signs=None, fused_stages=None,
+                 keep_intermediates=False, grouped_algorithm="auto"):
         self.tokens, self.experts, self.top_k = tokens, experts, top_k
         self.hidden, self.inter, self.block_m = hidden, intermediate, block_m
         assignments = tokens * top_k
@@ -136,14 +137,42 @@ class MoeLayer:
         if signs is not None:
             self.k_rotate_dispatch = Kernel("rotate_expert_a8", M=tokens, K=hidden, routing="scatter", top_k=top_k,
                                             experts=experts)
-        grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k)
+        grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k,
+                       algorithm=grouped_algorithm)
         self.k_gate_up = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, **grouped)
         self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
         self.k_down = Kernel("e8p_decode_grouped", N=hidden, K=intermediate, **grouped)
+        # Five launches instead of seven where the resident expert kernel takes the shapes:
+        #   router top-k that also quantises every token's row (once per token, not once per route),
+        #   metadata that also writes SlotMap, its inverse and zeroed per-slot maxima,
+        #   gate_up that gathers the int8 token rows by slot while it stages a tile (no dispatch copy) and
+        #     whose epilogue writes fp16(silu(gate) * up) and raises every slot's largest magnitude,
+        #   down that quantises those fp16 rows while it stages a tile (no SwiGLU->A8 launch),
+        #   combine.
+        # The library refuses the variants it does not serve that way, and the seven-launch program stays.
+        self.fused_stages = False
+        self.keep_intermediates = keep_intermediates
+        if fused_stages is not False and fused_metadata and signs is None and hidden % 8 == 0:
+            try:
+                self.k_router_a8 = Kernel("router_topk", renormalize=True, quantize_hidden=hidden, **common)
+                self.k_metadata_slots = Kernel("route_metadata", block_m=block_m, slot_maps=True, **common)
+                self.k_gate_up_fused = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, gather=True,
+                                              epilogue="swiglu", **grouped)
+                self.k_down_fused = Kernel("e8p_decode_grouped", N=hidden, K=intermediate, input_dtype="float16",
+                                           **grouped)
+                self.slot_token = torch.empty(assignments, **i32)
+                self.row_max = torch.empty(assignments, **i32)
+                self.act = torch.empty((assignments, intermediate), **f16)
+                self.fused_stages = True
+            except OrxError as error:
+                if fused_stages or error.code != ORX_ERR_BAD_VARIANT:
+                    raise
         self.k_combine = Kernel("moe_combine", H=hidden, slots=assignments, **common)
 
     def run(self, x16, logits, stream=None):
         s = stream
+        if self.fused_stages:
+            return self._run_fused(x16, logits, s)
         self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
         if self.k_metadata is not None:
             self.k_metadata(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative,
@@ -171,6 +200,24 @@ class MoeLayer:
         self.k_gate_up(stream=s, A=self.d, AS=self.ds, C=self.gate_up_out, P=self.w1, WS=self.s1, **routed)
         self.k_swiglu_a8(stream=s, Mask=None, Q=self.h_q, S=self.h_s, X=self.gate_up_out, rows=self.assignments)
         self.k_down(stream=s, A=self.h_q, AS=self.h_s, C=self.down_out, P=self.w2, WS=self.s2, **routed)
+        self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
+                       SlotMap=self.slot_map)
+        return self.out
+
+
+    def _run_fused(self, x16, logits, s):
+        keep = self.keep_intermediates
+        self.k_router_a8(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob, Q=self.a_q, S=self.a_s, X=x16)
+        self.k_metadata_slots(stream=s, Counts=self.counts, IDs=self.ids, RelativeSlot=self.relative, RowMax=self.row_max,
+                              RowOffsets=self.row_offsets, SlotMap=self.slot_map, SlotToken=self.slot_token,
+                              TileCount=self.tile_count, TileExpert=self.tile_expert, TileOffsets=self.tile_offsets,
+                              TileRow=self.tile_row)
+        routed = dict(Book=self.book, Counts=self.counts, Offsets=self.row_offsets, TileCount=self.tile_count,
+                      TileExpert=self.tile_expert, TileRow=self.tile_row)
+        self.k_gate_up_fused(stream=s, A=self.a_q, AS=self.a_s, Act=self.act, C=self.gate_up_out if keep else None,
+                             P=self.w1, RowMax=self.row_max, SlotToken=self.slot_token, WS=self.s1, **routed)
+        self.k_down_fused(stream=s, A=self.act, AS=self.h_s if keep else None, C=self.down_out, P=self.w2,
+                          Q=self.h_q if keep else None, RowMax=self.row_max, WS=self.s2, **routed)
         self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
                        SlotMap=self.slot_map)
         return self.out

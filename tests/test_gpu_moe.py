@@ -267,10 +267,12 @@ def test_combine_invalid_slots_and_shared_expert(m, h, slots):
     assert torch.equal(shifted, out) and not flat[:4].any() and not flat[4 + m * h :].any()
 
 
-def run_layer(c, bm, packed_k=128, fused_dispatch=True, signs=None):
+def run_layer(c, bm, packed_k=128, fused_dispatch=True, signs=None, fused_stages=False, **more):
     layer = programs.MoeLayer(c["tokens"], c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
                               c["gate_up_scales"], c["down"], c["down_scales"], block_m=bm, packed_k=packed_k,
-                              fused_dispatch=fused_dispatch, signs=signs)
+                              fused_dispatch=fused_dispatch, signs=signs, fused_stages=fused_stages,
+                              keep_intermediates=True, **more)
+    assert fused_stages is None or layer.fused_stages == bool(fused_stages)
     layer.run(gu.dev(c["x"]), gu.dev(c["logits"]))
     gu.sync()
     return layer
@@ -291,8 +293,15 @@ def check_layer(c, layer, bm):
         np.testing.assert_array_equal(gu.host(layer.a_q), a_q)
     d, ds, slot = orc.expert_dispatch(a_q, a_s, ids, rel, rows)
     np.testing.assert_array_equal(gu.host(layer.slot_map), slot)
-    np.testing.assert_array_equal(gu.host(layer.d), d)
-    np.testing.assert_array_equal(gu.host(layer.ds), ds)
+    if layer.fused_stages:  # the rows stay per token; the projection gathers them through the slot -> token map
+        np.testing.assert_array_equal(gu.host(layer.a_q), a_q)
+        np.testing.assert_array_equal(gu.host(layer.a_s), a_s)
+        token_of = np.empty(slot.size, np.int32)
+        token_of[slot.ravel()] = np.repeat(np.arange(slot.shape[0], dtype=np.int32), slot.shape[1])
+        np.testing.assert_array_equal(gu.host(layer.slot_token), token_of)
+    else:
+        np.testing.assert_array_equal(gu.host(layer.d), d)
+        np.testing.assert_array_equal(gu.host(layer.ds), ds)
     w1 = np.stack([orc.q2_integers(x, TABLE) for x in c["gate_up"]])
     w2 = np.stack([orc.q2_integers(x, TABLE) for x in c["down"]])
     gate_up = orc.grouped_project(d, ds, w1, c["gate_up_scales"], counts, rows)
@@ -303,6 +312,15 @@ def check_layer(c, layer, bm):
     act = orc.swiglu_fp16(gate_up)
     want_q, want_s = orc.a8(act)
     assert (act_gpu_q == want_q).mean() > 0.999 and (act_gpu_s == want_s).mean() > 0.99
+    if layer.fused_stages:
+        # the fp16 values between the two projections and their per-slot maxima; the codes are the
+        # A8 rule applied to exactly those values
+        act_gpu = gu.host(layer.act)
+        assert (act_gpu == act).mean() > 0.999
+        np.testing.assert_array_equal(gu.host(layer.row_max).view(np.float32), np.abs(act_gpu.astype(np.float32)).max(1))
+        exact_q, exact_s = orc.a8(act_gpu)
+        np.testing.assert_array_equal(act_gpu_q, exact_q)
+        np.testing.assert_array_equal(act_gpu_s, exact_s)
     down = orc.grouped_project(act_gpu_q, act_gpu_s, w2, c["down_scales"], counts, rows)
     np.testing.assert_array_equal(gu.host(layer.down_out), down)
     got = gu.host(layer.out).astype(np.float32)
@@ -321,11 +339,30 @@ def test_moe_layer_small_end_to_end():
     check_layer(c, run_layer(c, 32, fused_dispatch=False), 32)  # quantiser and dispatch as two launches
     signs = np.random.default_rng(3).choice(np.array([-1, 1], np.int8), c["hidden"])
     check_layer(c, run_layer(c, 32, signs=signs), 32)  # rotated input: rotation, A8 and scatter in one launch
+    # five launches: no dispatch copy, no SwiGLU->A8 launch between the two expert projections
+    wide = workloads.config3(tokens=70, experts=16, top_k=4, hidden=768, intermediate=384)  # K/128 = 6 and 3
+    for packed_k in (128, 0):
+        check_layer(wide, run_layer(wide, 32, packed_k=packed_k, fused_stages=True, grouped_algorithm="resident"), 32)
 
 
 def test_config3_full_size_end_to_end():
     c = workloads.config3()
     check_layer(c, run_layer(c, 32), 32)
+
+
+def test_config3_full_size_end_to_end_in_five_launches():
+    """What `MoeLayer` runs by default at this size: router that also quantises the token rows, metadata
+    with the slot tables, gate_up that gathers the rows by slot and ends in SwiGLU, down that quantises the
+    fp16 rows while it stages them, combine."""
+    c = workloads.config3()
+    layer = run_layer(c, 32, fused_stages=None)
+    assert layer.fused_stages
+    check_layer(c, layer, 32)
+    lean = programs.MoeLayer(c["tokens"], c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
+                             c["gate_up_scales"], c["down"], c["down_scales"], block_m=32)  # no intermediates kept
+    lean.run(gu.dev(c["x"]), gu.dev(c["logits"]))
+    gu.sync()
+    assert lean.fused_stages and torch.equal(lean.out, layer.out)
 
 
 def test_moe_layer_graph_replay_with_new_routing():
@@ -789,3 +826,31 @@ def test_rotate_expert_a8_refuses_what_it_does_not_serve():
                     dict(routing="scatter", top_k=65, experts=128), dict(group_major=True), dict(M=0)):
         with pytest.raises(Exception):
             gu.kernel("rotate_expert_a8", **{**dict(M=4, K=256), **variant})
+
+
+@pytest.mark.parametrize("m,e,k,h", [(256, 128, 8, 2048), (5, 64, 4, 4096), (33, 512, 10, 136)])
+def test_router_quantises_the_hidden_rows_in_the_same_launch(m, e, k, h):
+    """quantize_hidden: ids and probabilities as without it, plus the A8 codes and scales of the rows."""
+    rng = np.random.default_rng(orc.SEED + m + h)
+    logits = rng.normal(size=(m, e)).astype(np.float32)
+    x = (rng.normal(size=(m, h)) * rng.uniform(0.1, 4.0, (m, 1))).astype(np.float16)
+    x[m // 2] = 0
+    cap = m + 2
+    ids = torch.full((cap, k), -1, **I32)
+    prob = torch.full((cap, k), -1.0, dtype=torch.float32, device=gu.DEV)
+    q = torch.full((cap, h), 7, dtype=torch.int8, device=gu.DEV)
+    s = torch.full((cap,), 3.0, dtype=torch.float16, device=gu.DEV)
+    pad = lambda a: np.concatenate([a, np.zeros((cap - m,) + a.shape[1:], a.dtype)])
+    gu.kernel("router_topk", M=cap, E=e, top_k=k, dynamic_rows=True, quantize_hidden=h)(
+        IDs=ids, Logits=gu.dev(pad(logits)), Prob=prob, Q=q, S=s, X=gu.dev(pad(x)), m=m)
+    plain_ids = torch.full((cap, k), -1, **I32)
+    plain_prob = torch.full((cap, k), -1.0, dtype=torch.float32, device=gu.DEV)
+    gu.kernel("router_topk", M=cap, E=e, top_k=k, dynamic_rows=True)(IDs=plain_ids, Logits=gu.dev(pad(logits)),
+                                                                     Prob=plain_prob, m=m)
+    assert torch.equal(ids, plain_ids) and torch.equal(prob, plain_prob)
+    want_ids, _ = orc.router_topk(logits, k, True)
+    np.testing.assert_array_equal(gu.host(ids)[:m], want_ids)
+    want_q, want_s = orc.a8(x)
+    np.testing.assert_array_equal(gu.host(q)[:m], want_q)
+    np.testing.assert_array_equal(gu.host(s)[:m], want_s[:, 0])
+    assert (gu.host(q)[m:] == 7).all() and (gu.host(s)[m:] == 3).all() and (gu.host(ids)[m:] == -1).all()
