@@ -254,3 +254,44 @@ def test_workload_sizes_and_algorithmic_bytes():
     assert np.array_equal(case["packed"], again["packed"]) and np.array_equal(case["x"], again["x"])
     small = workloads.config1(8, n=256, k=256)
     assert small["x"].shape == (8, 256) and np.array_equal(small["packed"], workloads.config1(1, n=256, k=256)["packed"])
+
+
+def test_argument_lists_of_the_fused_expert_layer_forms():
+    """Buffer names stay in ASCII order when a form adds buffers, and forms the resident expert kernel
+    does not serve are refused at resolve time (so a program can fall back to the separate launches)."""
+    def names(symbol, **variant):
+        return lib.Kernel(symbol, **variant).arg_names
+
+    assert names("router_topk", M=8, E=64, top_k=4, quantize_hidden=256) == ["IDs", "Logits", "Prob", "Q", "S", "X"]
+    assert names("router_topk", M=8, E=64, top_k=4, dynamic_rows=True) == ["IDs", "Logits", "Prob", "m"]
+    assert names("route_metadata", M=8, E=64, top_k=4, block_m=32, slot_maps=True) == [
+        "Counts", "IDs", "RelativeSlot", "RowMax", "RowOffsets", "SlotMap", "SlotToken", "TileCount", "TileExpert",
+        "TileOffsets", "TileRow"]
+    grouped = dict(rows=2048, E=128, tiles=192, block_m=32, algorithm="resident")
+    plain = ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "TileCount", "TileExpert", "TileRow", "WS"]
+    assert names("e8p_decode_grouped", N=1024, K=2048, **grouped) == plain
+    assert names("e8p_decode_grouped", N=1024, K=2048, gather=True, epilogue="swiglu", **grouped) == [
+        "A", "AS", "Act", "Book", "C", "Counts", "Offsets", "P", "RowMax", "SlotToken", "TileCount", "TileExpert",
+        "TileRow", "WS"]
+    assert names("e8p_decode_grouped", N=2048, K=512, input_dtype="float16", **grouped) == [
+        "A", "AS", "Book", "C", "Counts", "Offsets", "P", "Q", "RowMax", "TileCount", "TileExpert", "TileRow", "WS"]
+    for listed in (plain, names("rotate_expert_a8", M=4, K=256, routing="scatter", top_k=2, experts=8)):
+        assert listed == sorted(listed)
+    assert names("rotate_expert_a8", M=4, K=256, routing="shared", top_k=2, experts=8, dynamic_rows=True) == [
+        "DS", "IDs", "Q", "RelativeSlot", "RowOffsets", "S", "Signs", "SlotMap", "Sum", "X", "m"]
+    assert names("rotate_expert_a8", M=4, K=256) == ["Q", "S", "Signs", "Sum", "X"]
+    refused = (
+        ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, rows=8192, E=128, tiles=512, block_m=32, algorithm="resident")),
+        ("e8p_decode_grouped", dict(N=2048, K=2048, input_dtype="float16", **grouped)),          # K > 1024 for fp16 rows
+        ("e8p_decode_grouped", dict(N=2048, K=512, input_dtype="float16", epilogue="swiglu", **grouped)),
+        ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, rows=2048, E=128, tiles=192, block_m=64)),
+        ("e8p_decode_grouped", dict(N=1024, K=2048, epilogue="swiglu", rows=2048, E=128, tiles=192, block_m=32,
+                                    algorithm="stream")),
+        ("rotate_expert_a8", dict(M=4, K=256, group_major=True)),
+        ("rotate_expert_a8", dict(M=4, K=256, routing="scatter", top_k=65, experts=128)),
+        ("router_topk", dict(M=8, E=64, top_k=4, quantize_hidden=100)),
+    )
+    for symbol, variant in refused:
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel(symbol, **variant)
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT, (symbol, variant)
