@@ -118,7 +118,9 @@ def kernel_record(name, family, variant, bindings, rows=0):
         if arg_name not in bindings:
             raise KeyError(f"{family}: no binding for argument {arg_name}")
         bound = bindings[arg_name]
-        if kind == 1:
+        if bound is None:
+            args.append({"kind": "null"})  # an optional buffer that this program does not use
+        elif kind == 1:
             args.append({"kind": "i32", "value": int(bound)})
         elif isinstance(bound, tuple):
             args.append({"kind": "buffer_slice", "name": bound[0], "offset": int(bound[1])})
@@ -243,6 +245,58 @@ def projection_records(slot, n, k, capacity, **options):
     return projection_program(slot, n, k, capacity, **options)["kernels"]
 
 
+def expert_layer_program(slot, tokens, experts, top_k, hidden, intermediate, *, block_m=32, packed_k=128,
+                         grouped_algorithm="auto", buffers=None):
+    """The routed Q2A8 expert layer as five `Kernel` records in launch order (the program of
+    `programs.MoeLayer` where the resident expert kernel applies): router top-k that also quantises
+    the token rows, routing metadata with the slot tables, gate_up (rows gathered by slot, SwiGLU
+    epilogue), down (fp16 rows quantised while staged), weighted combine.
+
+    buffers: overrides of the default buffer names, which are the argument names prefixed where two
+    launches would collide (`GateUpCodes`/`DownCodes`, `GateUpScales`/`DownScales`, ...).  Returns the
+    records and a dict name -> byte size of every buffer the program touches."""
+    assignments = tokens * top_k
+    tiles = (assignments + block_m - 1) // block_m + min(experts, assignments)
+    common = dict(M=tokens, E=experts, top_k=top_k)
+    grouped = dict(rows=assignments, E=experts, tiles=tiles, block_m=block_m, packed_k=packed_k,
+                   algorithm=grouped_algorithm)
+    name = dict(buffers or {})
+    b = lambda key: name.get(key, key)
+    routed = dict(Book=b("Book"), Counts=b("Counts"), Offsets=b("RowOffsets"), TileCount=b("TileCount"),
+                  TileExpert=b("TileExpert"), TileRow=b("TileRow"))
+    records = [
+        kernel_record(f"{slot}.router", "router_topk", dict(renormalize=True, quantize_hidden=hidden, **common),
+                      dict(IDs=b("IDs"), Logits=b("Logits"), Prob=b("Prob"), Q=b("A8"), S=b("A8Scale"), X=b("X"))),
+        kernel_record(f"{slot}.metadata", "route_metadata", dict(block_m=block_m, slot_maps=True, **common),
+                      dict(Counts=b("Counts"), IDs=b("IDs"), RelativeSlot=b("RelativeSlot"), RowMax=b("RowMax"),
+                           RowOffsets=b("RowOffsets"), SlotMap=b("SlotMap"), SlotToken=b("SlotToken"),
+                           TileCount=b("TileCount"), TileExpert=b("TileExpert"), TileOffsets=b("TileOffsets"),
+                           TileRow=b("TileRow"))),
+        kernel_record(f"{slot}.gate_up", "e8p_decode_grouped",
+                      dict(N=2 * intermediate, K=hidden, gather=True, epilogue="swiglu", **grouped),
+                      dict(A=b("A8"), AS=b("A8Scale"), Act=b("Act"), C=None, P=b("GateUpCodes"), RowMax=b("RowMax"),
+                           SlotToken=b("SlotToken"), WS=b("GateUpScales"), **routed)),
+        kernel_record(f"{slot}.down", "e8p_decode_grouped",
+                      dict(N=hidden, K=intermediate, input_dtype="float16", **grouped),
+                      dict(A=b("Act"), AS=None, C=b("ExpertOut"), P=b("DownCodes"), Q=None, RowMax=b("RowMax"),
+                           WS=b("DownScales"), **routed)),
+        kernel_record(f"{slot}.combine", "moe_combine", dict(H=hidden, slots=assignments, **common),
+                      dict(Expert=b("ExpertOut"), Output=b("Output"), Prob=b("Prob"), Shared=None, SharedGate=None,
+                           SlotMap=b("SlotMap"))),
+    ]
+    sizes = {
+        b("X"): tokens * hidden * 2, b("Logits"): tokens * experts * 4, b("IDs"): assignments * 4,
+        b("Prob"): assignments * 4, b("A8"): tokens * hidden, b("A8Scale"): tokens * 2, b("Counts"): experts * 4,
+        b("RelativeSlot"): assignments * 4, b("RowMax"): assignments * 4, b("RowOffsets"): experts * 4,
+        b("SlotMap"): assignments * 4, b("SlotToken"): assignments * 4, b("TileCount"): 4, b("TileExpert"): tiles * 4,
+        b("TileOffsets"): experts * 4, b("TileRow"): tiles * 4, b("Act"): assignments * intermediate * 2,
+        b("ExpertOut"): assignments * hidden * 2, b("Output"): tokens * hidden * 2, b("Book"): 1024,
+        b("GateUpCodes"): experts * 2 * intermediate * hidden // 4, b("DownCodes"): experts * hidden * intermediate // 4,
+        b("GateUpScales"): experts * 2 * intermediate * 2, b("DownScales"): experts * hidden * 2,
+    }
+    return records, sizes
+
+
 def fixture_manifest(buffers, records, validation, *, rows=None):
     """The same records as a manifest of the `orx_run_fixture` runner (buffers: name -> bytes | array file)."""
     kernels = []
@@ -254,6 +308,8 @@ def fixture_manifest(buffers, records, validation, *, rows=None):
                 args.append({"buffer": arg["name"]})
             elif arg["kind"] == "buffer_slice":
                 args.append({"buffer": arg["name"], "offset": arg["offset"]})
+            elif arg["kind"] == "null":
+                args.append({"null": True})
             else:
                 args.append({"i32": arg["value"]})
         entry = {"symbol": record["symbol"], "grid": record["grid"], "block": record["block"],

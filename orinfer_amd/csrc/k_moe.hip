@@ -653,7 +653,8 @@ int make_router(const Variant& v, orx_function* f) {
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = rows_geometry_router;
     f->launch = router_launch;
-    f->device_function = reinterpret_cast<const void*>(&router_topk_kernel<16, false>);
+    f->device_function = f->H > 0 ? reinterpret_cast<const void*>(&router_topk_kernel<16, true>)
+                                  : reinterpret_cast<const void*>(&router_topk_kernel<16, false>);
     return ORX_OK;
 }
 

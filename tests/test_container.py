@@ -143,3 +143,38 @@ def test_container_to_records_to_fixture_run(tmp_path):
                           timeout=120)
     report = json.loads(done.stdout.strip().splitlines()[-1])
     assert done.returncode == 0 and report["ok"] and report["relative_l2"] < 1e-3, (report, done.stderr)
+
+
+@pytest.mark.gpu
+def test_expert_layer_records_run_through_the_fixture_runner(tmp_path):
+    """The five-launch expert layer as package records, resolved and launched by the C++ fixture runner
+    (a separate process that knows only the C ABI): oracle output within the expert-FFN bar of
+    flash_next_quantized.py:117-135, graph capture, poisoned-output, zero-input and restored replays."""
+    from orinfer_amd import workloads
+    c = workloads.config3(tokens=70, experts=16, top_k=4, hidden=768, intermediate=384)
+    records, sizes = container.expert_layer_program("layer.moe", c["tokens"], c["experts"], c["top_k"], c["hidden"],
+                                                    c["intermediate"], grouped_algorithm="resident")
+    assert [r["name"].rsplit(".", 1)[1] for r in records] == ["router", "metadata", "gate_up", "down", "combine"]
+    want = orc.moe_layer(c["x"], c["logits"], c["gate_up"], c["gate_up_scales"], c["down"], c["down_scales"], orc.basis(),
+                         c["top_k"], 32)["out"].astype(np.float32)
+    want.tofile(tmp_path / "Output.f32")
+    data = {"X": c["x"], "Logits": c["logits"], "Book": codebook.book(),
+            "GateUpCodes": codebook.q2_to_k_major(np.asarray(c["gate_up"])), "GateUpScales": c["gate_up_scales"],
+            "DownCodes": codebook.q2_to_k_major(np.asarray(c["down"])), "DownScales": c["down_scales"]}
+    buffers = []
+    for name, size in sizes.items():
+        if name in data:
+            array = np.ascontiguousarray(data[name])
+            assert array.nbytes == size, name
+            array.tofile(tmp_path / f"{name}.bin")
+            buffers.append({"name": name, "file": f"{name}.bin", "bytes": size})
+        else:
+            buffers.append({"name": name, "bytes": size, "fill": 0})
+    manifest = container.fixture_manifest(buffers, records,
+                                          dict(output="Output", output_dtype="f16", reference="Output.f32",
+                                               relative_l2_tolerance=3e-3, zero_input="X", repetitions=5))
+    (tmp_path / "manifest.json").write_text(json.dumps(manifest))
+    done = subprocess.run([str(build.FIXTURE_RUNNER), str(tmp_path / "manifest.json")], capture_output=True, text=True,
+                          timeout=120)
+    report = json.loads(done.stdout.strip().splitlines()[-1])
+    assert done.returncode == 0 and report["ok"] and report["relative_l2"] < 3e-3, (report, done.stderr)

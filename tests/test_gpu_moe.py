@@ -854,3 +854,30 @@ def test_router_quantises_the_hidden_rows_in_the_same_launch(m, e, k, h):
     np.testing.assert_array_equal(gu.host(q)[:m], want_q)
     np.testing.assert_array_equal(gu.host(s)[:m], want_s[:, 0])
     assert (gu.host(q)[m:] == 7).all() and (gu.host(s)[m:] == 3).all() and (gu.host(ids)[m:] == -1).all()
+
+
+def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
+    """`orx_query` is what an engine checks a record's block against before it accepts the record
+    (backend/cuda/kernels.rs:150-170): every form's limit must hold the block its geometry asks for."""
+    grouped = dict(rows=2048, E=128, tiles=192, block_m=32)
+    forms = [
+        ("router_topk", dict(M=256, E=128, top_k=8)),
+        ("router_topk", dict(M=256, E=128, top_k=8, quantize_hidden=2048)),
+        ("router_topk", dict(M=256, E=1024, top_k=8, quantize_hidden=2048)),
+        ("route_metadata", dict(M=256, E=128, top_k=8, block_m=32, slot_maps=True)),
+        ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, epilogue="swiglu", **grouped)),
+        ("e8p_decode_grouped", dict(N=2048, K=512, input_dtype="float16", **grouped)),
+        ("e8p_decode_grouped", dict(N=2048, K=512, **grouped)),
+        ("rotate_expert_a8", dict(M=256, K=2048, routing="scatter", top_k=8, experts=128)),
+        ("rotate_expert_a8", dict(M=8192, K=5120)),
+        ("expert_dispatch", dict(M=256, H=2048, E=128, top_k=8, input_dtype="float16")),
+        ("moe_combine", dict(M=256, H=2048, slots=2048, E=128, top_k=8)),
+        ("int8_swiglu", dict(M=64, N=512, K=256)),
+        ("e8p_q4_projection", dict(M=8192, N=5120, K=5120, dynamic_rows=True, workspace=True)),
+    ]
+    for symbol, variant in forms:
+        kern = gu.lib.Kernel(symbol, **variant)
+        threads, _ = kern.query()
+        for rows in ({1, variant["M"]} if variant.get("dynamic_rows") else {0}):
+            block = kern.geometry(rows)[1]
+            assert block[0] * block[1] * block[2] <= threads, (symbol, variant, rows, block, threads)
