@@ -54,7 +54,7 @@ constexpr uint32_t kBasisBase = 0;             // 256 entries x 16 copies x 8 by
 constexpr uint32_t kMaskBase = 32768;
 constexpr uint32_t kInfoBase = 65536;          // (expert, first row, rows) of every routed tile
 constexpr int kMaxTiles = 1024;
-constexpr uint32_t kRowStatBase = kInfoBase + kMaxTiles * 12;  // per staged row: largest magnitude (32 ints), scale (32 halves)
+constexpr uint32_t kRowStatBase = kInfoBase + kMaxTiles * 12;  // fp16 rows quantised while staged: the scale of every staged row
 constexpr uint32_t kSumBase = kRowStatBase + 256;          // phase-two sums, then the staged token rows
 constexpr int kRowPad = 16;
 constexpr int kSumStride = 33;                 // ints per token row of a phase-two sum block

@@ -95,17 +95,20 @@ __device__ __forceinline__ void wave_quantise_row(const __half* __restrict__ x, 
 // QUANT (quantize_hidden): four more waves per workgroup quantise the same four tokens' hidden rows
 // by the A8 rule while the first four select the routes (the expert projections gather these rows
 // by slot, so a row is quantised once, not once per route, and it costs no launch of its own).
+// With 16 keys per lane the selection wants more registers than a 512-thread workgroup leaves a
+// wave, so there each wave quantises its own token's row after it has selected the routes.
+template <int LOCAL, bool QUANT>
+constexpr int router_threads() { return QUANT && LOCAL <= 8 ? 512 : 256; }
 template <int LOCAL, bool QUANT>  // LOCAL keys per lane: ceil(E / 64) rounded up to a power of two
-__global__ __launch_bounds__(QUANT ? 512 : 256) void router_topk_kernel(const float* __restrict__ logits,
-                                                                        int* __restrict__ ids, float* __restrict__ prob, int m,
-                                                                        int e, int top_k, int renormalize,
-                                                                        const __half* __restrict__ x, int8_t* __restrict__ q,
-                                                                        __half* __restrict__ s, int h) {
+__global__ __launch_bounds__((router_threads<LOCAL, QUANT>())) void router_topk_kernel(
+    const float* __restrict__ logits, int* __restrict__ ids, float* __restrict__ prob, int m, int e, int top_k,
+    int renormalize, const __half* __restrict__ x, int8_t* __restrict__ q, __half* __restrict__ s, int h) {
+    constexpr bool kQuantiserWaves = router_threads<LOCAL, QUANT>() == 512;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int row = blockIdx.x * 4 + (wave & 3);
     if (row >= m) return;
-    if (QUANT && wave >= 4) {
+    if (kQuantiserWaves && wave >= 4) {
         wave_quantise_row(x, q, s, row, h, lane);
         return;
     }
@@ -151,6 +154,7 @@ __global__ __launch_bounds__(QUANT ? 512 : 256) void router_topk_kernel(const fl
     }
     const float selected_sum = wave_sum(lane < top_k ? mine : 0.f);
     if (lane < top_k) prob[(int64_t)row * top_k + lane] = __fdiv_rn(mine, renormalize ? selected_sum : all_exp);
+    if (QUANT && !kQuantiserWaves) wave_quantise_row(x, q, s, row, h, lane);
 }
 
 // Block-wide exclusive prefix of a 0/1 flag; returns this thread's prefix and the block total.
@@ -604,7 +608,8 @@ bool geometry_fields(const Variant& v, orx_function* f, bool need_m) {
 
 int rows_geometry_router(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, 4u);
-    g->block[0] = f.H > 0 ? 512 : 256;  // quantize_hidden: four more waves quantise the four tokens' rows
+    // quantize_hidden: four more waves quantise the four tokens' rows (up to 8 keys per lane, E <= 512)
+    g->block[0] = f.H > 0 && f.E <= 512 ? 512 : 256;
     return ORX_OK;
 }
 // IDs, Logits, Prob[, Q, S, X][, m]
@@ -653,8 +658,16 @@ int make_router(const Variant& v, orx_function* f) {
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = rows_geometry_router;
     f->launch = router_launch;
-    f->device_function = f->H > 0 ? reinterpret_cast<const void*>(&router_topk_kernel<16, true>)
-                                  : reinterpret_cast<const void*>(&router_topk_kernel<16, false>);
+    // the instantiation this variant launches (its thread limit is what orx_query reports)
+#define ORX_ROUTER_FN(LOCAL)                                                                \
+    (f->H > 0 ? reinterpret_cast<const void*>(&router_topk_kernel<LOCAL, true>)             \
+              : reinterpret_cast<const void*>(&router_topk_kernel<LOCAL, false>))
+    f->device_function = f->E <= 64    ? ORX_ROUTER_FN(1)
+                         : f->E <= 128 ? ORX_ROUTER_FN(2)
+                         : f->E <= 256 ? ORX_ROUTER_FN(4)
+                         : f->E <= 512 ? ORX_ROUTER_FN(8)
+                                       : ORX_ROUTER_FN(16);
+#undef ORX_ROUTER_FN
     return ORX_OK;
 }
 

@@ -828,7 +828,7 @@ def test_rotate_expert_a8_refuses_what_it_does_not_serve():
             gu.kernel("rotate_expert_a8", **{**dict(M=4, K=256), **variant})
 
 
-@pytest.mark.parametrize("m,e,k,h", [(256, 128, 8, 2048), (5, 64, 4, 4096), (33, 512, 10, 136)])
+@pytest.mark.parametrize("m,e,k,h", [(256, 128, 8, 2048), (5, 64, 4, 4096), (33, 512, 10, 136), (7, 1024, 8, 256)])
 def test_router_quantises_the_hidden_rows_in_the_same_launch(m, e, k, h):
     """quantize_hidden: ids and probabilities as without it, plus the A8 codes and scales of the rows."""
     rng = np.random.default_rng(orc.SEED + m + h)
