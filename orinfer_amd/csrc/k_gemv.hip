@@ -20,6 +20,7 @@
 
 #include "a8_device.h"
 #include "e8p_device.h"
+#include "moe_device.h"
 #include "orx_internal.h"
 
 namespace orx {
@@ -856,12 +857,24 @@ constexpr int kRouteTableBytes = 256 * 16, kRouteMaskBytes = 256 * 8, kRoutePart
 //   q[j] = +-t[j] + c,  c = 1 - 2 * parity   =>   a . q = a . (+-t) + c * sum(a)
 // with +-t picked per byte between the table entry and its negation (both prepared per entry at
 // set-up), the byte masks of u prepared per u, and the sums of every 8 token bytes prepared once.
+//
+// Two launches of the one-token expert layer can run inside this kernel's set-up:
+//   LOCAL > 0 (route_logits): `ids` is an output.  Wave 0 of every workgroup selects the token's
+//     routes from `logits` (the router's rule, moe_device.h) while the others build the tables; the
+//     first workgroup writes ids and probabilities for the combine.  Selecting eight routes of one
+//     token costs a wave about a microsecond; a router launch in front costs three to four.
+//   x16 == 2 (fused_swiglu): `a` holds fp16 gate|up rows, one per route; the row becomes
+//     fp16(silu(gate) * up), then A8 codes, on its way into LDS (the SwiGLU -> A8 launch between the
+//     two projections disappears); the first workgroup of a route writes its scale.
+template <int LOCAL>
 __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
     const int8_t* __restrict__ a, const __half* __restrict__ as, const uint32_t* __restrict__ book, __half* __restrict__ c,
     const int32_t* __restrict__ ids, const uint16_t* __restrict__ p, const __half* __restrict__ ws, int experts, int n,
-    int k, int shared_input, int x16) {
+    int k, int shared_input, int x16, const float* __restrict__ logits, float* __restrict__ prob, int renormalize) {
     extern __shared__ __align__(16) uint8_t route_lds[];
     __shared__ float route_wave_max[kRouteWaves];
+    __shared__ int selected_ids[64];
+    __shared__ float selected_prob[64];
     uint4* table = reinterpret_cast<uint4*>(route_lds);                                    // entry, negated entry
     uint2* masks = reinterpret_cast<uint2*>(route_lds + kRouteTableBytes);                  // per u
     int* partial = reinterpret_cast<int*>(route_lds + kRouteTableBytes + kRouteMaskBytes);  // [waves][channels]
@@ -870,23 +883,29 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int route = blockIdx.y;
-    const int expert = ids[route];
-    if ((unsigned)expert >= (unsigned)experts) return;  // nothing to index: the row stays as it was
+    const int routes = (int)gridDim.y;
+    int expert = LOCAL > 0 ? 0 : ids[route];
+    if (LOCAL == 0 && (unsigned)expert >= (unsigned)experts) return;  // nothing to index: the row stays as it was
     const int row = shared_input ? 0 : route;
     const int blocks = k / 128;
     const int channel = blockIdx.x * kRouteChannels + (lane >> 1);
     const int half = lane & 1;
     const bool live = channel < n;
     // codes of this lane: 16 bytes per K block, K blocks wave, wave + 8, ...; the first kRouteDepth
-    // loads leave before anything else
-    const uint4* codes = reinterpret_cast<const uint4*>(p + (((int64_t)expert * blocks) * n + (live ? channel : 0)) * 16) + half;
+    // loads leave before anything else (once the expert is known)
     const int64_t block_stride = (int64_t)n * 2;  // uint4 per K block
+    const uint4* codes = nullptr;
     uint4 held[kRouteDepth];
+    auto request_codes = [&]() {
+        codes = reinterpret_cast<const uint4*>(p + (((int64_t)expert * blocks) * n + (live ? channel : 0)) * 16) + half;
 #pragma unroll
-    for (int d = 0; d < kRouteDepth; ++d) {
-        const int kb = wave + d * kRouteWaves;
-        held[d] = kb < blocks ? codes[kb * block_stride] : make_uint4(0u, 0u, 0u, 0u);
-    }
+        for (int d = 0; d < kRouteDepth; ++d) {
+            const int kb = wave + d * kRouteWaves;
+            held[d] = kb < blocks ? codes[kb * block_stride] : make_uint4(0u, 0u, 0u, 0u);
+        }
+    };
+    if (LOCAL == 0) request_codes();
+    if (LOCAL > 0 && wave == 0) select_routes<LOCAL == 0 ? 1 : LOCAL>(logits, selected_ids, selected_prob, 0, experts, routes, renormalize, lane);
     if (tid < 256) {
         const uint2 entry = reinterpret_cast<const uint2*>(book)[tid];
         table[tid] = make_uint4(entry.x, entry.y, negate_bytes(entry.x), negate_bytes(entry.y));
@@ -896,18 +915,40 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
         masks[u] = make_uint2(sign_mask(signs), sign_mask(signs >> 2));
     }
     float row_scale = 0.f;  // x16: fp32 value of the row's fp16 scale
+    // the routes are known after the next barrier (the one of the row maximum where there is one)
+    auto routes_published = [&]() {
+        if (LOCAL == 0) return;
+        expert = selected_ids[route];
+        request_codes();
+        if (blockIdx.x == 0 && blockIdx.y == 0 && tid < routes) {
+            const_cast<int32_t*>(ids)[tid] = selected_ids[tid];
+            prob[tid] = selected_prob[tid];
+        }
+    };
     if (x16) {
-        // `a` is the shared fp16 row: every workgroup quantises it by the A8 rule (row maximum over 127,
-        // fp16 scale, round to nearest even) on its way into LDS; the first one also writes the scale.
-        // Up to 4 pieces of 8 values per thread (K <= 16384) stay in registers between the two passes.
-        const __half* x = reinterpret_cast<const __half*>(a);
+        // `a` is an fp16 row (the shared token row, or with x16 == 2 this route's gate|up row, which
+        // first becomes fp16(silu(gate) * up)): every workgroup quantises it by the A8 rule (row maximum
+        // over 127, fp16 scale, round to nearest even) on its way into LDS; the first one also writes
+        // the scale.  Up to 4 pieces of 8 values per thread (K <= 16384) stay in registers between the
+        // two passes.
+        const bool swiglu_rows = x16 == 2;
+        const __half* x = reinterpret_cast<const __half*>(a) + (swiglu_rows ? (int64_t)route * 2 * k : 0);
         uint4 kept[4];
         float amax = 0.f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int i = tid + j * kRouteThreads;
             kept[j] = make_uint4(0u, 0u, 0u, 0u);
-            if (i < k / 8) kept[j] = reinterpret_cast<const uint4*>(x)[i];
+            if (i < k / 8) {
+                kept[j] = reinterpret_cast<const uint4*>(x)[i];
+                if (swiglu_rows) {
+                    const uint4 up_bits = reinterpret_cast<const uint4*>(x + k)[i];
+                    __half* gate = reinterpret_cast<__half*>(&kept[j]);
+                    const __half* up = reinterpret_cast<const __half*>(&up_bits);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) gate[e] = __float2half_rn(swiglu_value(gate[e], up[e]));
+                }
+            }
             const __half2* pairs = reinterpret_cast<const __half2*>(&kept[j]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -919,11 +960,12 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
         for (int offset = 32; offset > 0; offset >>= 1) amax = fmaxf(amax, __shfl_xor(amax, offset, 64));
         if (lane == 0) route_wave_max[wave] = amax;
         __syncthreads();
+        routes_published();
         amax = route_wave_max[0];
 #pragma unroll
         for (int w = 1; w < kRouteWaves; ++w) amax = fmaxf(amax, route_wave_max[w]);
         const __half stored = a8_scale(amax);
-        if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *const_cast<__half*>(as) = stored;
+        if (blockIdx.x == 0 && (swiglu_rows || blockIdx.y == 0) && tid == 0) const_cast<__half*>(as)[swiglu_rows ? route : 0] = stored;
         row_scale = __half2float(stored);
         const float inverse = __builtin_amdgcn_rcpf(row_scale);
 #pragma unroll
@@ -939,6 +981,10 @@ __global__ __launch_bounds__(kRouteThreads) void route_gemv_kernel(
             }
         }
     } else {
+        if (LOCAL > 0) {
+            __syncthreads();
+            routes_published();
+        }
         for (int i = tid; i < k / 8; i += kRouteThreads) {
             const uint2 bytes = reinterpret_cast<const uint2*>(a + (int64_t)row * k)[i];
             reinterpret_cast<uint2*>(token)[i] = bytes;
@@ -1005,18 +1051,31 @@ int route_gemv_geometry(const orx_function& f, int rows, Geometry* g) {
     return ORX_OK;
 }
 
-// A, AS, Book, C, IDs, P, WS: the buffers of integer_vq.py:388-395 in generated-ABI order
+// A, AS, Book, C, IDs, [Logits,] P, [Prob,] WS: the buffers of integer_vq.py:388-395 in generated-ABI order
+// slots used: flags bit0 shared_input, bit1 fused_swiglu, bit2 route_logits, bit3 renormalize
 int route_gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
+    const bool routing = f.flags & 4;
     const int8_t* a = pointer_arg<const int8_t>(args, 0);
     const __half* as = pointer_arg<const __half>(args, 1);
     const uint32_t* book = pointer_arg<const uint32_t>(args, 2);
     __half* c = pointer_arg<__half>(args, 3);
     const int32_t* ids = pointer_arg<const int32_t>(args, 4);
-    const uint16_t* p = pointer_arg<const uint16_t>(args, 5);
-    const __half* ws = pointer_arg<const __half>(args, 6);
-    hipLaunchKernelGGL(route_gemv_kernel, dim3(g.grid[0], g.grid[1]), dim3(kRouteThreads), g.shared, stream, a, as, book, c, ids, p,
-                       ws, f.E, f.N, f.K, f.flags & 1, f.input_f16 ? 1 : 0);
+    const float* logits = routing ? pointer_arg<const float>(args, 5) : nullptr;
+    const uint16_t* p = pointer_arg<const uint16_t>(args, routing ? 6 : 5);
+    float* prob = routing ? pointer_arg<float>(args, 7) : nullptr;
+    const __half* ws = pointer_arg<const __half>(args, routing ? 8 : 6);
+    const int x16 = f.input_f16 ? ((f.flags & 2) ? 2 : 1) : 0;
+    const dim3 grid(g.grid[0], g.grid[1]), block(kRouteThreads);
+#define ORX_ROUTE_GEMV(LOCAL)                                                                                      \
+    hipLaunchKernelGGL(route_gemv_kernel<LOCAL>, grid, block, g.shared, stream, a, as, book, c, ids, p, ws, f.E, f.N, f.K, \
+                       f.flags & 1, x16, logits, prob, (f.flags >> 3) & 1)
+    if (!routing) ORX_ROUTE_GEMV(0);
+    else if (f.E <= 64) ORX_ROUTE_GEMV(1);
+    else if (f.E <= 128) ORX_ROUTE_GEMV(2);
+    else if (f.E <= 256) ORX_ROUTE_GEMV(4);
+    else ORX_ROUTE_GEMV(8);
+#undef ORX_ROUTE_GEMV
     return hip_check(hipGetLastError(), "launch integer_e8p_gemv");
 }
 
@@ -1039,18 +1098,39 @@ int make_route_gemv(const Variant& v, orx_function* f) {
         return ORX_ERR_BAD_VARIANT;
     }
     f->flags = shared_input ? 1 : 0;
-    // input_dtype=float16 (shared row only): A is the fp16 row, quantised by every workgroup on its way into
-    // LDS; AS is written, not read
+    // input_dtype=float16: A is fp16 and AS is written, not read.  With shared_input it is the one token row,
+    // quantised by every workgroup on its way into LDS; with fused_swiglu (no shared input) it holds one
+    // gate|up row of 2K values per route, which becomes fp16(silu(gate) * up) and then A8 codes.
     const std::string input = v.string("input_dtype", "int8", &bad);
-    if (bad || (input != "int8" && input != "float16") || (input == "float16" && (!shared_input || f->K > 16384))) {
-        set_error("integer_e8p_gemv: input_dtype must be int8 or float16 (float16: shared_input, K up to 16384)");
+    const bool fused_swiglu = v.boolean("fused_swiglu", false, &bad);
+    if (bad || (input != "int8" && input != "float16") || (input == "float16" && f->K > 16384) ||
+        (input == "float16" && shared_input == fused_swiglu) || (fused_swiglu && input != "float16")) {
+        set_error("integer_e8p_gemv: input_dtype must be int8 or float16 (float16: the shared row, or with fused_swiglu "
+                  "one gate|up row per route; K up to 16384)");
         return ORX_ERR_BAD_VARIANT;
     }
     f->input_f16 = input == "float16";
+    if (fused_swiglu) f->flags |= 2;
+    // route_logits=true: IDs is written, not read: every workgroup selects the token's `routes` routes from
+    // Logits (1, E) by the router's rule, the first one writes IDs and Prob (renormalize as router_topk)
+    const bool route_logits = v.boolean("route_logits", false, &bad);
+    const bool renormalize = v.boolean("renormalize", true, &bad);
+    if (bad || (route_logits && (f->E > 512 || f->M > 64 || f->M > f->E))) {
+        set_error("integer_e8p_gemv: route_logits needs E <= 512 and routes <= min(E, 64)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (route_logits) f->flags |= 4 | (renormalize ? 8 : 0);
     // 16-byte loads of A rows and P, 8-byte loads of Book
-    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 8}, {"C", ArgPointer, 2},
-               {"IDs", ArgPointer, 4}, {"P", ArgPointer, 16}, {"WS", ArgPointer, 2}};
-    f->device_function = reinterpret_cast<const void*>(&route_gemv_kernel);
+    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 8}, {"C", ArgPointer, 2}, {"IDs", ArgPointer, 4}};
+    if (route_logits) f->args.push_back({"Logits", ArgPointer, 4});
+    f->args.push_back({"P", ArgPointer, 16});
+    if (route_logits) f->args.push_back({"Prob", ArgPointer, 4});
+    f->args.push_back({"WS", ArgPointer, 2});
+    f->device_function = !route_logits  ? reinterpret_cast<const void*>(&route_gemv_kernel<0>)
+                         : f->E <= 64  ? reinterpret_cast<const void*>(&route_gemv_kernel<1>)
+                         : f->E <= 128 ? reinterpret_cast<const void*>(&route_gemv_kernel<2>)
+                         : f->E <= 256 ? reinterpret_cast<const void*>(&route_gemv_kernel<4>)
+                                       : reinterpret_cast<const void*>(&route_gemv_kernel<8>);
     f->geometry = route_gemv_geometry;
     f->launch = route_gemv_launch;
     return ORX_OK;
@@ -1181,7 +1261,9 @@ int gemv_prepare_device() {
 
 const Registration* gemv_registrations(int* count) {
     static const Registration rows[] = {
-    {"integer_e8p_gemv", make_route_gemv, "E, routes, N, K, shared_input, block_n=8, input_dtype=int8|float16", "A,AS,Book,C,IDs,P,WS"},
+    {"integer_e8p_gemv", make_route_gemv,
+     "E, routes, N, K, shared_input, block_n=8, input_dtype=int8|float16, fused_swiglu=false, route_logits=false, renormalize=true",
+     "A,AS,Book,C,IDs[,Logits],P[,Prob],WS"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;

@@ -229,7 +229,7 @@ class MoeTokenLayer:
     router top-k, gate/up of every route from the shared row (quantised on the way), SwiGLU->A8 per route,
     down per route, weighted combine."""
 
-    def __init__(self, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales):
+    def __init__(self, experts, top_k, hidden, intermediate, gate_up, gate_up_scales, down, down_scales, fused=None):
         self.experts, self.top_k, self.hidden, self.inter = experts, top_k, hidden, intermediate
         self.w1 = _dev(codebook.q2_to_k_major(np.asarray(gate_up)))
         self.w2 = _dev(codebook.q2_to_k_major(np.asarray(down)))
@@ -254,9 +254,32 @@ class MoeTokenLayer:
         self.k_swiglu_a8 = Kernel("activation_quantization", K=intermediate, fused=True)
         self.k_down = Kernel("integer_e8p_gemv", E=experts, routes=top_k, N=hidden, K=intermediate, shared_input=False)
         self.k_combine = Kernel("moe_combine", H=hidden, slots=top_k, **common)
+        # Three launches instead of five where the library has the forms (up to 512 experts): gate/up selects
+        # the token's routes itself while it builds its tables (no router launch), down turns the fp16 gate|up
+        # rows into SwiGLU -> A8 codes on their way into LDS (no launch in between).
+        self.fused = False
+        if fused is not False:
+            try:
+                routes = dict(E=experts, routes=top_k)
+                self.k_gate_up_routing = Kernel("integer_e8p_gemv", N=2 * intermediate, K=hidden, shared_input=True,
+                                                input_dtype="float16", route_logits=True, renormalize=True, **routes)
+                self.k_down_swiglu = Kernel("integer_e8p_gemv", N=hidden, K=intermediate, shared_input=False,
+                                            input_dtype="float16", fused_swiglu=True, **routes)
+                self.fused = True
+            except OrxError as error:
+                if fused or error.code != ORX_ERR_BAD_VARIANT:
+                    raise
 
     def run(self, x16, logits, stream=None):
         s = stream
+        if self.fused:
+            self.k_gate_up_routing(stream=s, A=x16, AS=self.a_s, Book=self.book, C=self.gate_up_out, IDs=self.ids,
+                                   Logits=logits, P=self.w1, Prob=self.prob, WS=self.s1)
+            self.k_down_swiglu(stream=s, A=self.gate_up_out, AS=self.h_s, Book=self.book, C=self.down_out, IDs=self.ids,
+                               P=self.w2, WS=self.s2)
+            self.k_combine(stream=s, Expert=self.down_out, Output=self.out, Prob=self.prob, Shared=None, SharedGate=None,
+                           SlotMap=self.slot_map)
+            return self.out
         self.k_router(stream=s, IDs=self.ids, Logits=logits, Prob=self.prob)
         self.k_gate_up(stream=s, A=x16, AS=self.a_s, Book=self.book, C=self.gate_up_out, IDs=self.ids, P=self.w1,
                        WS=self.s1)

@@ -711,7 +711,8 @@ def test_moe_token_layer_matches_the_routed_layer_of_one_token():
     """One token through direct bank indexing gives what the token-sorted layer gives for it."""
     c = workloads.config3(tokens=1, experts=32, top_k=4, hidden=512, intermediate=256)
     layer = programs.MoeTokenLayer(c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
-                                   c["gate_up_scales"], c["down"], c["down_scales"])
+                                   c["gate_up_scales"], c["down"], c["down_scales"], fused=False)
+    assert not layer.fused
     x, logits = gu.dev(c["x"]), gu.dev(c["logits"])
     layer.run(x, logits)
     gu.sync()
@@ -735,6 +736,16 @@ def test_moe_token_layer_matches_the_routed_layer_of_one_token():
     # and the token-sorted program on the same token
     sorted_layer = run_layer(c, 32)
     assert torch.equal(sorted_layer.out, layer.out)
+    # three launches (gate/up selects the routes itself, down applies SwiGLU -> A8 to its input): same bits
+    three = programs.MoeTokenLayer(c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
+                                   c["gate_up_scales"], c["down"], c["down_scales"])
+    assert three.fused
+    three.ids.fill_(-1)
+    three.run(x, logits)
+    gu.sync()
+    for name in ("ids", "prob", "a_s", "gate_up_out", "h_s", "down_out", "out"):
+        assert torch.equal(getattr(three, name), getattr(layer, name)), name
+    layer = three  # the graph replay below runs the three-launch program
     # graph replay with another token
     stream = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
@@ -881,3 +892,25 @@ def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
         for rows in ({1, variant["M"]} if variant.get("dynamic_rows") else {0}):
             block = kern.geometry(rows)[1]
             assert block[0] * block[1] * block[2] <= threads, (symbol, variant, rows, block, threads)
+
+
+@pytest.mark.parametrize("e,k,h,i", [(128, 8, 2048, 512), (512, 10, 1024, 384), (64, 64, 256, 128)])
+def test_one_token_layer_in_three_launches_gives_the_bits_of_five(e, k, h, i):
+    c = workloads.config3(tokens=1, experts=e, top_k=k, hidden=h, intermediate=i)
+    x, logits = gu.dev(c["x"]), gu.dev(c["logits"])
+    layers = []
+    for fused in (False, True):
+        layer = programs.MoeTokenLayer(e, k, h, i, c["gate_up"], c["gate_up_scales"], c["down"], c["down_scales"],
+                                       fused=fused)
+        layer.run(x, logits)
+        gu.sync()
+        layers.append(layer)
+    want_ids, want_prob = orc.router_topk(c["logits"], k, True)
+    np.testing.assert_array_equal(gu.host(layers[1].ids), want_ids)
+    np.testing.assert_allclose(gu.host(layers[1].prob), want_prob, atol=2e-6, rtol=2e-5)
+    for name in ("ids", "prob", "a_s", "gate_up_out", "h_s", "down_out", "out"):
+        assert torch.equal(getattr(layers[1], name), getattr(layers[0], name)), name
+    for variant in (dict(shared_input=True, input_dtype="float16", fused_swiglu=True), dict(shared_input=False, input_dtype="float16"),
+                    dict(shared_input=False, fused_swiglu=True), dict(shared_input=True, route_logits=True, E=1024)):
+        with pytest.raises(Exception):
+            gu.kernel("integer_e8p_gemv", **{**dict(E=e, routes=k, N=h, K=i), **variant})
