@@ -60,6 +60,9 @@ def parse():
     p.add_argument("--traffic-probe", action="store_true",
                    help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a plain copy of known size, then the "
                         "contract kernel once per weight copy, eagerly; no timing")
+    p.add_argument("--mfma-probe", action="store_true",
+                   help="the int8 matrix pipe alone: v_mfma_i32_32x32x32_i8 back to back from registers, with zero and "
+                        "with random operands (the ceiling the GEMM fractions are read against); no other workload")
     return p.parse_args()
 
 
@@ -149,6 +152,24 @@ def main():
                 self.quantize(s)
                 self.project(i, s)
 
+    if args.mfma_probe:
+        # rates of the matrix pipe by itself; long launches, so that the power controller has settled
+        iterations = 20000
+        out = torch.empty(1024, dtype=torch.int32, device="cuda")
+        report = {}
+        for operands in ("zero", "random"):
+            probe = Kernel("int8_mfma_probe", iterations=iterations, operands=operands)
+            cus = probe.geometry()[0][0]
+            for _ in range(2):
+                probe(stream=stream.cuda_stream, Out=out)
+            torch.cuda.synchronize()
+            seconds = timed_graph(lambda i, s: probe(stream=s, Out=out), 4)
+            ops = cus * 8 * iterations * 8 * 65536.0
+            report[operands] = {"ms_per_launch": round(seconds * 1e3, 3), "TOPS": round(ops / seconds / 1e12, 1),
+                                "frac_int8_peak": round(ops / seconds / 1e12 / INT8_PEAK_TOPS, 4)}
+        print(json.dumps({"int8_mfma_probe": dict(report, compute_units=cus, waves_per_cu=8, iterations=iterations,
+                                                  ops_per_launch=cus * 8 * iterations * 8 * 65536)}))
+        return
     # ---- contract workload: config 1, M=1 ----
     c1 = workloads.config1(1)
     bytes_c1 = workloads.algorithmic_bytes_q4(1, c1["n"], c1["k"])

@@ -295,3 +295,11 @@ def test_argument_lists_of_the_fused_expert_layer_forms():
         with pytest.raises(lib.OrxError) as err:
             lib.Kernel(symbol, **variant)
         assert err.value.code == lib.ORX_ERR_BAD_VARIANT, (symbol, variant)
+
+
+def test_matrix_pipe_probe_is_a_catalogued_diagnostic():
+    kern = lib.Kernel("int8_mfma_probe", iterations=100, operands="zero")
+    assert kern.arg_names == ["Out"] and kern.geometry()[1][0] == 512
+    for bad in (dict(iterations=0), dict(operands="ones")):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("int8_mfma_probe", **bad)
