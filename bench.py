@@ -63,6 +63,9 @@ def parse():
     p.add_argument("--mfma-probe", action="store_true",
                    help="the int8 matrix pipe alone: v_mfma_i32_32x32x32_i8 back to back from registers, with zero and "
                         "with random operands (the ceiling the GEMM fractions are read against); no other workload")
+    p.add_argument("--read-probe", action="store_true",
+                   help="a plain streaming read of 12.5, 44.6 and 178 MB (the code bytes of configs 0 and 1 and four times "
+                        "that), rotating more buffers than the caches hold: the rate that bounds the GEMV; no other workload")
     return p.parse_args()
 
 
@@ -169,6 +172,25 @@ def main():
                                 "frac_int8_peak": round(ops / seconds / 1e12 / INT8_PEAK_TOPS, 4)}
         print(json.dumps({"int8_mfma_probe": dict(report, compute_units=cus, waves_per_cu=8, iterations=iterations,
                                                   ops_per_launch=cus * 8 * iterations * 8 * 65536)}))
+        return
+    if args.read_probe:
+        out = torch.zeros(1, dtype=torch.int32, device="cuda")
+        report = {}
+        for label, size in (("config0_codes", 9728 * 2560 // 2), ("config1_codes", 17408 * 5120 // 2),
+                            ("four_times_config1", 4 * 17408 * 5120 // 2)):
+            sources = [torch.empty(size, dtype=torch.uint8, device="cuda").random_(0, 256)
+                       for _ in range(-(-2 * CACHE_BYTES // size))]
+            best = None
+            for per_cu in (4, 8, 16):
+                probe = Kernel("hbm_read_probe", bytes=size, workgroups_per_cu=per_cu)
+                seconds = timed_graph(lambda i, s: probe(stream=s, Out=out, Source=sources[i % len(sources)]),
+                                      max(2 * len(sources), 26))
+                if best is None or seconds < best[0]:
+                    best = (seconds, per_cu)
+            report[label] = {"bytes": size, "us_per_launch": round(best[0] * 1e6, 3), "GBps": round(size / best[0] / 1e9, 1),
+                             "frac_hbm_peak": round(size / best[0] / 1e9 / HBM_PEAK_GBS, 4), "workgroups_per_cu": best[1]}
+            del sources
+        print(json.dumps({"hbm_read_probe": report}))
         return
     # ---- contract workload: config 1, M=1 ----
     c1 = workloads.config1(1)

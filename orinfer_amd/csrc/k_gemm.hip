@@ -48,7 +48,6 @@ int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, 
                           hipStream_t stream);
 // from k_gemm_big.hip
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g);
-int make_mfma_probe(const Variant& v, orx_function* f);
 int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int n, int k, int packed_k,
                      hipStream_t stream);
 int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
@@ -1318,7 +1317,6 @@ const Registration* gemm_registrations(int* count) {
     {"integer_experts", make_integer_experts,
      "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},
-    {"int8_mfma_probe", make_mfma_probe, "iterations=20000, operands=random|zero (diagnostic: the matrix pipe alone)", "Out"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     };

@@ -471,77 +471,6 @@ int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int
     return hip_check(hipGetLastError(), "launch two-stage weight expansion");
 }
 
-// ---- int8_mfma_probe: what the matrix pipe sustains by itself ---------------------------------
-// A diagnostic, not part of the path: eight waves per CU issue v_mfma_i32_32x32x32_i8 back to back
-// from registers (no memory, no LDS), with all-zero operands or with eight random fragments per
-// operand rotated through the instructions.  The two rates differ by what the data costs in power:
-// it is the ceiling that the projections' int8 fractions should be read against.
-namespace {
-template <bool RANDOM>
-__global__ __launch_bounds__(512) void mfma_probe_kernel(int* out, int iterations) {
-    v4i fa[8], fb[8];
-    uint32_t x = (threadIdx.x + blockIdx.x * 512u) * 2654435761u + 12345u;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            x ^= x << 13, x ^= x >> 17, x ^= x << 5;
-            fa[i][j] = RANDOM ? (int)x : 0;
-            x ^= x << 13, x ^= x >> 17, x ^= x << 5;
-            fb[i][j] = RANDOM ? (int)x : 0;
-        }
-    v16i acc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[i][j] = 0;
-    for (int it = 0; it < iterations; ++it) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[(i + 3) & 7], acc[i], 0, 0, 0);
-    }
-    int folded = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 16; ++j) folded ^= acc[i][j];
-    // one word per workgroup, so that the loop cannot be removed; the value carries no meaning
-    if (threadIdx.x == 0) out[blockIdx.x] = folded;
-}
-
-int mfma_probe_geometry(const orx_function&, int, Geometry* g) {
-    g->grid[0] = (uint32_t)device_compute_units();
-    g->block[0] = 512;
-    return ORX_OK;
-}
-int mfma_probe_launch(const orx_function& f, int, const Geometry& g, hipStream_t stream, void** args) {
-    int* out = pointer_arg<int>(args, 0);
-    if (f.flags)
-        hipLaunchKernelGGL(mfma_probe_kernel<true>, dim3(g.grid[0]), dim3(512), 0, stream, out, f.K);
-    else
-        hipLaunchKernelGGL(mfma_probe_kernel<false>, dim3(g.grid[0]), dim3(512), 0, stream, out, f.K);
-    return hip_check(hipGetLastError(), "launch int8_mfma_probe");
-}
-}  // namespace
-
-// Out: one int32 per CU (at least 1024 of them).  Operations per launch: CUs * 8 waves * iterations * 8 * 65536.
-int make_mfma_probe(const Variant& v, orx_function* f) {
-    bool bad = false;
-    f->K = (int)v.integer("iterations", 20000, &bad);
-    const std::string operands = v.string("operands", "random", &bad);
-    if (bad || f->K <= 0 || f->K > (1 << 24) || (operands != "random" && operands != "zero")) {
-        set_error("int8_mfma_probe: iterations in 1..2^24, operands random|zero");
-        return ORX_ERR_BAD_VARIANT;
-    }
-    f->flags = operands == "random";
-    f->M = f->capacity = 1;
-    f->args = {{"Out", ArgPointer, 4}};
-    f->geometry = mfma_probe_geometry;
-    f->launch = mfma_probe_launch;
-    f->device_function = f->flags ? reinterpret_cast<const void*>(&mfma_probe_kernel<true>)
-                                  : reinterpret_cast<const void*>(&mfma_probe_kernel<false>);
-    return ORX_OK;
-}
-
 void gemm_big_geometry(int rows, int n, bool q4, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTile) * ceil_div((uint32_t)n, (uint32_t)kTile);
     g->grid[1] = g->grid[2] = 1;

@@ -205,14 +205,16 @@ struct Table {
     const Registration* rows;
     int count;
 };
-void tables(Table out[4]) {
+constexpr int kTables = 5;
+void tables(Table out[kTables]) {
     out[0].rows = quant_registrations(&out[0].count);
     out[1].rows = gemv_registrations(&out[1].count);
     out[2].rows = gemm_registrations(&out[2].count);
     out[3].rows = moe_registrations(&out[3].count);
+    out[4].rows = probe_registrations(&out[4].count);
 }
 const Registration* find(const char* symbol) {
-    Table t[4];
+    Table t[kTables];
     tables(t);
     for (auto& table : t)
         for (int i = 0; i < table.count; ++i)
@@ -565,7 +567,7 @@ const char* orx_catalog(void) {
         if (s == nullptr) return (const std::string*)nullptr;
         try {
             *s = "{\"kernels\":[";
-            Table t[4];
+            Table t[kTables];
             tables(t);
             bool first = true;
             for (auto& table : t)

@@ -95,6 +95,7 @@ const Registration* quant_registrations(int* count);
 const Registration* gemv_registrations(int* count);
 const Registration* gemm_registrations(int* count);
 const Registration* moe_registrations(int* count);
+const Registration* probe_registrations(int* count);
 
 template <typename T>
 static inline T* pointer_arg(void** args, int index) {

@@ -303,3 +303,11 @@ def test_matrix_pipe_probe_is_a_catalogued_diagnostic():
     for bad in (dict(iterations=0), dict(operands="ones")):
         with pytest.raises(lib.OrxError):
             lib.Kernel("int8_mfma_probe", **bad)
+
+
+def test_plain_read_probe_is_a_catalogued_diagnostic():
+    kern = lib.Kernel("hbm_read_probe", bytes=44564480, workgroups_per_cu=4)
+    assert kern.arg_names == ["Out", "Source"] and kern.geometry()[1][0] == 256
+    for bad in (dict(bytes=1000), dict(bytes=16384, workgroups_per_cu=0)):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("hbm_read_probe", **bad)
