@@ -234,6 +234,12 @@ def main():
     main_case.quantize(stream.cuda_stream)
     plain_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(min(args.steps, 260), copies))
     traffic_bytes, traffic_kernel = measured_traffic(main_case.fused.geometry(1))
+    # what a read of the same code bytes reaches on this box when nothing is done with them
+    read_probe = Kernel("hbm_read_probe", bytes=c1["n"] * c1["k"] // 2, workgroups_per_cu=4)
+    probe_out = torch.zeros(1, dtype=torch.int32, device="cuda")
+    read_seconds = timed_graph(lambda i, s: read_probe(stream=s, Out=probe_out, Source=main_case.weights[i % copies]),
+                               max(min(args.steps, 260), copies))
+    read_rate = c1["n"] * c1["k"] // 2 / read_seconds / 1e9
     # config 0 (the reference's own CPU-runnable shape) on the same kernel: a second roofline entry
     c0 = workloads.config0()
     b0 = workloads.algorithmic_bytes_q4(1, c0["n"], c0["k"])
@@ -262,6 +268,9 @@ def main():
                      "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": traffic_bytes,
+                     "plain_read_of_the_codes": {"us_per_launch": round(read_seconds * 1e6, 3), "GBps": round(read_rate, 1),
+                                                 "frac": round(read_rate / HBM_PEAK_GBS, 4),
+                                                 "kernel_vs_plain_read": round(achieved / read_rate, 4)},
                      "same_kernel_int8_input": {"us_per_launch": round(plain_seconds * 1e6, 3),
                                                 "achieved": round(bytes_c1 / plain_seconds / 1e9, 1),
                                                 "frac": round(bytes_c1 / plain_seconds / 1e9 / HBM_PEAK_GBS, 4)},
