@@ -66,6 +66,9 @@ def parse():
     p.add_argument("--read-probe", action="store_true",
                    help="a plain streaming read of 12.5, 44.6 and 178 MB (the code bytes of configs 0 and 1 and four times "
                         "that), rotating more buffers than the caches hold: the rate that bounds the GEMV; no other workload")
+    p.add_argument("--lds-probe", action="store_true",
+                   help="random 4-byte reads of a 256-entry LDS table stored once, 32 and 64 times (what a code's decode "
+                        "lookups cost); no other workload")
     return p.parse_args()
 
 
@@ -172,6 +175,18 @@ def main():
                                 "frac_int8_peak": round(ops / seconds / 1e12 / INT8_PEAK_TOPS, 4)}
         print(json.dumps({"int8_mfma_probe": dict(report, compute_units=cus, waves_per_cu=8, iterations=iterations,
                                                   ops_per_launch=cus * 8 * iterations * 8 * 65536)}))
+        return
+    if args.lds_probe:
+        out = torch.zeros(1, dtype=torch.int32, device="cuda")
+        iterations, report = 2000, {}
+        for copies in (1, 32, 64):
+            probe = Kernel("lds_lookup_probe", iterations=iterations, copies=copies)
+            seconds = timed_graph(lambda i, s: probe(stream=s, Out=out), 8)
+            wave_instructions_per_cu = 16 * iterations * 8
+            report[f"copies_{copies}"] = {"us_per_launch": round(seconds * 1e6, 2),
+                                          "ns_per_wave_lookup_per_cu": round(seconds * 1e9 / wave_instructions_per_cu, 3),
+                                          "lane_lookups_per_ns_per_cu": round(64 * wave_instructions_per_cu / seconds / 1e9, 2)}
+        print(json.dumps({"lds_lookup_probe": dict(report, waves_per_cu=16, iterations=iterations, lookups_per_iteration=8)}))
         return
     if args.read_probe:
         out = torch.zeros(1, dtype=torch.int32, device="cuda")

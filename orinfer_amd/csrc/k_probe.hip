@@ -132,10 +132,83 @@ int make_read_probe(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// ---- lds_lookup_probe: random 4-byte reads of a 256-entry table in LDS -------------------------
+// The decode of every E8P code is two such lookups per stage.  `copies` is how often the table is
+// stored: entry e, copy c at word e * copies + c, and lane l reads copy l mod copies; 1 is a compact
+// 1 KiB table (the lanes of a wave collide in the banks), 64 gives every lane its own bank.  Sixteen
+// waves per CU issue eight independent lookups per iteration; nothing else competes for the LDS.
+namespace {
+typedef __attribute__((address_space(3))) const uint32_t lds_word;
+template <int COPIES>
+__global__ __launch_bounds__(1024) void lds_lookup_probe_kernel(uint32_t* out, int iterations) {
+    extern __shared__ uint32_t probe_table[];
+    for (int i = threadIdx.x; i < 256 * COPIES; i += 1024) probe_table[i] = (uint32_t)i * 2654435761u;
+    __syncthreads();
+    const uint32_t column = ((threadIdx.x & 63u) % COPIES) * 4u;
+    uint32_t x = threadIdx.x * 2654435761u + blockIdx.x + 1u, folded = 0;
+    for (int it = 0; it < iterations; ++it) {
+        x ^= x << 13, x ^= x >> 17, x ^= x << 5;
+        const uint32_t y = x ^ (x >> 7) ^ 0x9E3779B9u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t a0 = ((x >> (8 * j)) & 255u) * (COPIES * 4u) + column;
+            const uint32_t a1 = ((y >> (8 * j)) & 255u) * (COPIES * 4u) + column;
+            folded ^= *reinterpret_cast<lds_word*>(a0);
+            folded ^= *reinterpret_cast<lds_word*>(a1);
+        }
+    }
+    if (folded == 0x1234567u) out[0] = folded;  // keeps the lookups alive; practically never true
+}
+int lds_probe_geometry(const orx_function& f, int, Geometry* g) {
+    g->grid[0] = (uint32_t)device_compute_units();
+    g->block[0] = 1024;
+    g->shared = 256u * (uint32_t)f.tiles * 4u;
+    return ORX_OK;
+}
+template <int COPIES>
+int lds_probe_launch_as(const orx_function& f, const Geometry& g, hipStream_t stream, uint32_t* out) {
+    static DeviceOnce opted_in;  // 64 copies are 64 KiB of dynamic LDS
+    const int ready = opted_in.run([] {
+        return hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&lds_lookup_probe_kernel<COPIES>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024),
+                         "hipFuncSetAttribute");
+    });
+    if (ready != ORX_OK) return ready;
+    hipLaunchKernelGGL(lds_lookup_probe_kernel<COPIES>, dim3(g.grid[0]), dim3(1024), g.shared, stream, out, f.K);
+    return hip_check(hipGetLastError(), "launch lds_lookup_probe");
+}
+int lds_probe_launch(const orx_function& f, int, const Geometry& g, hipStream_t stream, void** args) {
+    uint32_t* out = pointer_arg<uint32_t>(args, 0);
+    if (f.tiles == 1) return lds_probe_launch_as<1>(f, g, stream, out);
+    if (f.tiles == 32) return lds_probe_launch_as<32>(f, g, stream, out);
+    return lds_probe_launch_as<64>(f, g, stream, out);
+}
+}  // namespace
+
+// Out: one word.  Lane lookups per launch: CUs * 1024 * iterations * 8 (wave instructions: a 64th of that).
+int make_lds_probe(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->K = (int)v.integer("iterations", 2000, &bad);
+    f->tiles = (int)v.integer("copies", 64, &bad);
+    if (bad || f->K <= 0 || f->K > (1 << 24) || (f->tiles != 1 && f->tiles != 32 && f->tiles != 64)) {
+        set_error("lds_lookup_probe: iterations in 1..2^24, copies 1|32|64");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->M = f->capacity = 1;
+    f->args = {{"Out", ArgPointer, 4}};
+    f->geometry = lds_probe_geometry;
+    f->launch = lds_probe_launch;
+    f->device_function = f->tiles == 1    ? reinterpret_cast<const void*>(&lds_lookup_probe_kernel<1>)
+                         : f->tiles == 32 ? reinterpret_cast<const void*>(&lds_lookup_probe_kernel<32>)
+                                          : reinterpret_cast<const void*>(&lds_lookup_probe_kernel<64>);
+    return ORX_OK;
+}
+
 const Registration* probe_registrations(int* count) {
     static const Registration rows[] = {
     {"int8_mfma_probe", make_mfma_probe, "iterations=20000, operands=random|zero (diagnostic: the matrix pipe alone)", "Out"},
     {"hbm_read_probe", make_read_probe, "bytes, workgroups_per_cu=8 (diagnostic: a plain streaming read)", "Out,Source"},
+    {"lds_lookup_probe", make_lds_probe, "iterations=2000, copies=64|32|1 (diagnostic: random table reads in LDS)", "Out"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;

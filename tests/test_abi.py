@@ -311,3 +311,10 @@ def test_plain_read_probe_is_a_catalogued_diagnostic():
     for bad in (dict(bytes=1000), dict(bytes=16384, workgroups_per_cu=0)):
         with pytest.raises(lib.OrxError):
             lib.Kernel("hbm_read_probe", **bad)
+
+
+def test_lds_lookup_probe_is_a_catalogued_diagnostic():
+    kern = lib.Kernel("lds_lookup_probe", iterations=10, copies=32)
+    assert kern.arg_names == ["Out"] and kern.geometry()[1:] == ((1024, 1, 1), 256 * 32 * 4)
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("lds_lookup_probe", copies=16)
