@@ -914,3 +914,18 @@ def test_one_token_layer_in_three_launches_gives_the_bits_of_five(e, k, h, i):
                     dict(shared_input=False, fused_swiglu=True), dict(shared_input=True, route_logits=True, E=1024)):
         with pytest.raises(Exception):
             gu.kernel("integer_e8p_gemv", **{**dict(E=e, routes=k, N=h, K=i), **variant})
+
+
+@pytest.mark.parametrize("fused_stages", [False, True], ids=["seven-launches", "five-launches"])
+def test_expert_layer_when_every_token_names_the_same_experts(fused_stages):
+    """The skew a router can produce: all 150 tokens choose the same four of sixteen experts, so those
+    experts have five tiles each (the last one ragged) and the other twelve none."""
+    c = workloads.config3(tokens=150, experts=16, top_k=4, hidden=768, intermediate=384)
+    logits = np.random.default_rng(11).normal(size=c["logits"].shape).astype(np.float32) * 0.01
+    logits[:, [3, 7, 8, 15]] += 5.0
+    c = dict(c, logits=logits)
+    layer = run_layer(c, 32, fused_stages=fused_stages, grouped_algorithm="resident")
+    counts = gu.host(layer.counts)
+    assert sorted(np.nonzero(counts)[0].tolist()) == [3, 7, 8, 15] and (counts[[3, 7, 8, 15]] == 150).all()
+    assert int(gu.host(layer.tile_count)[0]) == 20
+    check_layer(c, layer, 32)
