@@ -764,7 +764,7 @@ def test_moe_token_layer_matches_the_routed_layer_of_one_token():
 
 
 @pytest.mark.parametrize("swiglu", [False, True], ids=["rows", "swiglu"])
-@pytest.mark.parametrize("m,e,k,h", [(37, 64, 10, 640), (5, 512, 10, 5120), (300, 16, 2, 128)])
+@pytest.mark.parametrize("m,e,k,h", [(37, 64, 10, 640), (5, 512, 10, 5120), (300, 16, 2, 128), (3, 128, 64, 256)])
 def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, h, swiglu):
     """rotate_expert_a8: bit-exact against the oracle for every routing form, and the same bits as
     rotate_activation_a8 followed by expert_dispatch; rows beyond the live count stay untouched."""
@@ -929,3 +929,24 @@ def test_expert_layer_when_every_token_names_the_same_experts(fused_stages):
     assert sorted(np.nonzero(counts)[0].tolist()) == [3, 7, 8, 15] and (counts[[3, 7, 8, 15]] == 150).all()
     assert int(gu.host(layer.tile_count)[0]) == 20
     check_layer(c, layer, 32)
+
+
+def test_five_launches_at_the_largest_gathered_batch_give_the_bits_of_seven():
+    """512 tokens x top-8 = 4096 slots, the most the slot -> token table in LDS holds; one token more and
+    the layer keeps the seven-launch order by itself."""
+    c = workloads.config3(tokens=512)
+    x, logits = gu.dev(c["x"]), gu.dev(c["logits"])
+    outs = []
+    for fused in (False, None):
+        layer = programs.MoeLayer(c["tokens"], c["experts"], c["top_k"], c["hidden"], c["intermediate"], c["gate_up"],
+                                  c["gate_up_scales"], c["down"], c["down_scales"], block_m=32, fused_stages=fused)
+        assert layer.fused_stages == (fused is None)
+        layer.run(x, logits)
+        gu.sync()
+        outs.append(layer.out.clone())
+        del layer
+    assert torch.equal(outs[0], outs[1])
+    bigger = workloads.config3(tokens=513)
+    layer = programs.MoeLayer(513, bigger["experts"], bigger["top_k"], bigger["hidden"], bigger["intermediate"],
+                              bigger["gate_up"], bigger["gate_up_scales"], bigger["down"], bigger["down_scales"], block_m=32)
+    assert not layer.fused_stages
