@@ -39,7 +39,7 @@ int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, 
                           void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 bool grouped_resident_eligible(int n, int k, int block_m, int tiles, int input, int epilogue, int slots);
 bool grouped_resident_preferred(int rows, int experts, int n);
-void grouped_resident_geometry(int k, int input, int slots, Geometry* g);
+void grouped_resident_geometry(int k, int input, int epilogue, int slots, Geometry* g);
 int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, int packed_k, int input, int epilogue,
                             int slots, hipStream_t stream);
 int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
@@ -1031,7 +1031,7 @@ bool grouped_uses_resident(const orx_function& f) {
 int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
     (void)rows;
     if (grouped_uses_resident(f)) {
-        grouped_resident_geometry(f.K, f.flags2 & 3, f.capacity, g);
+        grouped_resident_geometry(f.K, f.flags2 & 3, f.flags2 >> 2, f.capacity, g);
         return ORX_OK;
     }
     if (f.block_m <= 64 && f.algorithm != kMfma) {
@@ -1140,7 +1140,7 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
             !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles, f->flags2 & 3, f->flags2 >> 2, f->capacity) ||
             (f->algorithm == kAuto && !grouped_resident_preferred(f->capacity, f->E, f->N))) {
             set_error("%s: gather, epilogue=swiglu and input_dtype=float16 are forms of the resident kernel (block_m=32, "
-                      "at most 4096 gathered slots, K <= 1024 for float16 rows) where the routed rows fill the chip", name);
+                      "gathered slots that fit LDS beside the staged rows, K <= 1024 for float16 rows) where the routed rows fill the chip", name);
             return ORX_ERR_BAD_VARIANT;
         }
     }

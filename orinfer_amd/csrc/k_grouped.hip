@@ -61,7 +61,7 @@ constexpr int kSumStride = 33;                 // ints per token row of a phase-
 constexpr int kSumBlock = 32 * kSumStride;     // ints
 constexpr int kMaxPieces = 5;                  // 16-byte pieces a thread stages per tile (K <= 2560)
 constexpr int kMaxHalfPieces = 4;              // fp16 input: 16-byte pieces of 8 values per thread and tile (K <= 1024)
-constexpr int kMaxSlots = 4096;                // rows gathered by slot: the slot -> token map sits in LDS as u16
+constexpr int kMaxSlots = 8192;                // rows gathered by slot: the slot -> token map sits in LDS as u16
 enum { kInputInt8 = 0, kInputGather = 1, kInputAct = 2 };
 enum { kEpiloguePlain = 0, kEpilogueSwiglu = 1 };
 
@@ -119,7 +119,9 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     const int spans = EPILOGUE == kEpilogueSwiglu ? (inner + kSpan / 2 - 1) / (kSpan / 2) : (p.n + kSpan - 1) / kSpan;
     const int groups = (int)gridDim.x, group = (int)blockIdx.x;
     const Split split = phase_two_split(kb_count);
-    const uint32_t tile_base = kSumBase + (uint32_t)split.per_pass * kSumBlock * 4;
+    // forms without a phase two (see below) have no sum blocks, and the staged rows start where those would
+    constexpr bool kPhaseTwo = INPUT != kInputAct && EPILOGUE == kEpiloguePlain;
+    const uint32_t tile_base = kSumBase + (kPhaseTwo ? (uint32_t)split.per_pass * kSumBlock * 4 : 0u);
     const int tile_stride = p.k + kRowPad;
     int* sums = reinterpret_cast<int*>(lds + kSumBase);
     __half* row_scale = reinterpret_cast<__half*>(lds + kRowStatBase);     // kInputAct: scales of the staged rows
@@ -147,7 +149,8 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
 #pragma unroll
         for (int i = 0; i < 8; ++i) *reinterpret_cast<uint4*>(dst + 16 * i) = pair;
     }
-    for (int i = tid; i < split.per_pass * kSumBlock; i += kThreads) sums[i] = 0;
+    if (kPhaseTwo)
+        for (int i = tid; i < split.per_pass * kSumBlock; i += kThreads) sums[i] = 0;
     if constexpr (INPUT == kInputGather)  // same trip as the tile list: nothing below waits for slot -> token -> row
         for (int i = tid; i < p.slots; i += kThreads) slot_tokens[i] = (uint16_t)p.slot_token[i];
     if (listed_here) {
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void grouped_resident_kernel(GroupedParam
     const int passes = (leftover * kWaves + groups * split.per_pass - 1) / (groups * split.per_pass);
     int my_units = full, first_unit = group * full;
     // (phase two reads int8 rows from memory and has the plain epilogue)
-    if (INPUT == kInputAct || EPILOGUE == kEpilogueSwiglu || passes > max(1, kb_count / 8)) {
+    if (!kPhaseTwo || passes > max(1, kb_count / 8)) {
         first_unit += min(group, leftover);
         if (group < leftover) ++my_units;
         leftover = 0;
@@ -545,9 +548,10 @@ int ring_depth(int k) {
     return kb % 2 == 0 ? 2 : kb % 3 == 0 ? 3 : 0;
 }
 
-uint32_t resident_lds_bytes(int k, int input, int slots) {
+uint32_t resident_lds_bytes(int k, int input, int epilogue, int slots) {
     const Split split = phase_two_split(k / 128);
-    const uint32_t rows = kSumBase + (uint32_t)split.per_pass * kSumBlock * 4u + 32u * (uint32_t)(k + kRowPad);
+    const bool phase_two = input != kInputAct && epilogue == kEpiloguePlain;  // the others have no sum blocks
+    const uint32_t rows = kSumBase + (phase_two ? (uint32_t)split.per_pass * kSumBlock * 4u : 0u) + 32u * (uint32_t)(k + kRowPad);
     return rows + (input == kInputGather ? (((uint32_t)slots * 2u + 15u) & ~15u) : 0u);
 }
 
@@ -564,7 +568,7 @@ bool grouped_resident_eligible(int n, int k, int block_m, int tiles, int input, 
     if (input == kInputAct && k > kMaxHalfPieces * kThreads * 8 / 32) return false;
     if (epilogue == kEpilogueSwiglu && n % 32 != 0) return false;  // inner = N/2 a multiple of 16
     return block_m == 32 && n % 32 == 0 && k % 128 == 0 && ring_depth(k) > 0 && tiles <= kMaxTiles &&
-           k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k, input, slots) <= kLdsLimit;
+           k / 16 <= kMaxPieces * kThreads / 32 && resident_lds_bytes(k, input, epilogue, slots) <= kLdsLimit;
 }
 
 // Worth it once the routed tiles give most CUs a unit of their own; below that the streaming
@@ -577,11 +581,11 @@ bool grouped_resident_preferred(int rows, int experts, int n) {
     return tiles * ((n + kSpan - 1) / kSpan) >= 0.8 * device_compute_units();
 }
 
-void grouped_resident_geometry(int k, int input, int slots, Geometry* g) {
+void grouped_resident_geometry(int k, int input, int epilogue, int slots, Geometry* g) {
     g->grid[0] = (uint32_t)device_compute_units();
     g->grid[1] = g->grid[2] = 1;
     g->block[0] = kThreads;
-    g->shared = resident_lds_bytes(k, input, slots);
+    g->shared = resident_lds_bytes(k, input, epilogue, slots);
 }
 
 int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, int packed_k, int input, int epilogue,
@@ -628,7 +632,7 @@ int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, in
     p.n = n, p.k = k, p.k_major = packed_k != 0, p.tile_capacity = tiles;
     p.expert_weight_stride = (int64_t)n * (k / 8) * 2;
     Geometry g;
-    grouped_resident_geometry(k, input, slots, &g);
+    grouped_resident_geometry(k, input, epilogue, slots, &g);
     const dim3 grid(g.grid[0]), block(kThreads);
 #define ORX_GROUPED(D, IN, EP) hipLaunchKernelGGL((grouped_resident_kernel<D, IN, EP>), grid, block, g.shared, stream, p)
 #define ORX_GROUPED_DEPTH(IN, EP)           \

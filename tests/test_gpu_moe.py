@@ -932,9 +932,9 @@ def test_expert_layer_when_every_token_names_the_same_experts(fused_stages):
 
 
 def test_five_launches_at_the_largest_gathered_batch_give_the_bits_of_seven():
-    """512 tokens x top-8 = 4096 slots, the most the slot -> token table in LDS holds; one token more and
+    """1024 tokens x top-8 = 8192 slots, the most the slot -> token table in LDS holds; one token more and
     the layer keeps the seven-launch order by itself."""
-    c = workloads.config3(tokens=512)
+    c = workloads.config3(tokens=1024)
     x, logits = gu.dev(c["x"]), gu.dev(c["logits"])
     outs = []
     for fused in (False, None):
@@ -946,7 +946,7 @@ def test_five_launches_at_the_largest_gathered_batch_give_the_bits_of_seven():
         outs.append(layer.out.clone())
         del layer
     assert torch.equal(outs[0], outs[1])
-    bigger = workloads.config3(tokens=513)
-    layer = programs.MoeLayer(513, bigger["experts"], bigger["top_k"], bigger["hidden"], bigger["intermediate"],
+    bigger = workloads.config3(tokens=1025)
+    layer = programs.MoeLayer(1025, bigger["experts"], bigger["top_k"], bigger["hidden"], bigger["intermediate"],
                               bigger["gate_up"], bigger["gate_up_scales"], bigger["down"], bigger["down_scales"], block_m=32)
     assert not layer.fused_stages
