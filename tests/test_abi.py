@@ -320,3 +320,46 @@ def test_lds_lookup_probe_is_a_catalogued_diagnostic():
     assert kern.arg_names == ["Out"] and kern.geometry()[1:] == ((1024, 1, 1), 256 * 32 * 4)
     with pytest.raises(lib.OrxError):
         lib.Kernel("lds_lookup_probe", copies=16)
+
+
+def test_session_threads_resolve_and_query_concurrently():
+    """Two or more session threads may resolve, inspect and release handles at the same time (one-time
+    set-up is atomic, errors are thread-local): every thread sees the answers a single thread sees."""
+    import threading
+
+    variants = [("e8p_q4_projection", dict(M=1, N=9728, K=2560)), ("int8_projection", dict(M=256, N=5120, K=5120, workspace=True)),
+                ("router_topk", dict(M=64, E=128, top_k=8, quantize_hidden=2048)),
+                ("e8p_decode_grouped", dict(rows=2048, E=128, tiles=192, N=1024, K=2048, block_m=32, algorithm="resident")),
+                ("rotate_expert_a8", dict(M=16, K=512, routing="scatter", top_k=4, experts=32))]
+    expected = []
+    for symbol, variant in variants:
+        kern = lib.Kernel(symbol, **variant)
+        expected.append((kern.arg_names, kern.geometry(), kern.workspace_bytes() if "workspace" in variant else 0))
+    catalog = lib.catalog()
+    failures = []
+
+    def session(index):
+        try:
+            for round_ in range(40):
+                symbol, variant = variants[(index + round_) % len(variants)]
+                kern = lib.Kernel(symbol, **variant)
+                want = expected[(index + round_) % len(variants)]
+                got = (kern.arg_names, kern.geometry(), kern.workspace_bytes() if "workspace" in variant else 0)
+                if got != want or lib.catalog() != catalog:
+                    failures.append((index, symbol))
+                try:
+                    lib.Kernel("e8p_q4_projection", M=1, N=128, K=100 + index)  # a refusal with a thread-local message
+                    failures.append((index, "accepted a bad K"))
+                except lib.OrxError as error:
+                    if str(100 + index) not in str(error) and "K" not in str(error):
+                        failures.append((index, str(error)))
+                del kern
+        except Exception as error:  # noqa: BLE001 - reported below
+            failures.append((index, repr(error)))
+
+    threads = [threading.Thread(target=session, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures[:5]
