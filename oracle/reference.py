@@ -160,11 +160,15 @@ def q2_pack_k128(indices):
 
 
 def q2_repack_k64(packed):
-    """(E,K/128,N,16) u16 -> (E,K/64,N,8), codes unchanged (vq.py:121-128)."""
-    e, g, n, _ = packed.shape
-    return np.ascontiguousarray(packed.reshape(e, g, n, 2, 8).transpose(0, 1, 3, 2, 4)).reshape(
-        e, g * 2, n, 8
-    )
+    """(E,K/128,N,16) u16 -> (E,K/64,N,8), codes unchanged (vq.py:121-128): K block 2g holds the first
+    eight codes of every row of group g, block 2g + 1 the other eight."""
+    experts, groups, rows, per_row = packed.shape
+    if per_row != 16:
+        raise ValueError("expected sixteen codes per row and group of 128")
+    blocks = np.empty((experts, 2 * groups, rows, 8), packed.dtype)
+    blocks[:, 0::2] = packed[..., :8]
+    blocks[:, 1::2] = packed[..., 8:]
+    return blocks
 
 
 # --------------------------------------------------------------------------
@@ -211,20 +215,22 @@ def swiglu_fp16(gu):
 def rotate(x, signs):
     """Signed block-128 Hadamard rotation in fp32 (python/orinfer_build/quantization/vq.py:20-31).
 
-    y = x * signs, then seven butterfly stages h = 1, 2, .. 64 inside every block of 128
-    (left + right, left - right), then one multiply by fp32(128 ** -0.5).  Every step is a
-    single fp32 operation, so a kernel that runs the stages in the same order is bit-exact.
+    y = x * signs, then seven butterfly stages with partner distance 1, 2, .. 64 inside every block
+    of 128: the element whose distance bit is clear becomes itself + partner, the other one
+    partner - itself; then one multiply by fp32(128 ** -0.5).  Every step is a single fp32
+    operation, so a kernel that runs the stages in the same order is bit-exact.
     """
-    x = np.asarray(x, dtype=np.float32)
-    signs = np.asarray(signs)
-    if x.shape[-1] % 128 or signs.shape != (x.shape[-1],) or not np.isin(signs, [-1, 1]).all():
+    values = np.asarray(x, dtype=np.float32)
+    flips = np.asarray(signs)
+    width = values.shape[-1]
+    if width % 128 != 0 or flips.shape != (width,) or np.any(np.abs(flips) != 1):
         raise ValueError("block-128 rotation needs one +-1 sign per input channel")
-    y = (x * signs.astype(np.float32)).astype(np.float32)
-    for stage in range(7):
-        h = 1 << stage
-        block = y.reshape(*y.shape[:-1], -1, 2 * h)
-        left, right = block[..., :h].copy(), block[..., h:].copy()
-        block[..., :h], block[..., h:] = left + right, left - right
+    y = values * flips.astype(np.float32)
+    position = np.arange(width)
+    for distance in (1, 2, 4, 8, 16, 32, 64):
+        partner = y[..., position ^ distance]
+        upper = (position & distance) != 0
+        y = np.where(upper, partner - y, y + partner).astype(np.float32)
     return (y * np.float32(128**-0.5)).astype(np.float32)
 
 
