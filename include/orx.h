@@ -25,6 +25,14 @@
  * e8p_q4.py:78-80,250).  Blocks of 64 are read by the streaming and the MFMA tile
  * kernels at every row count; the one-row GEMV and the resident kernel read row-major
  * codes and blocks of 128 only (production stores 128, models/qwen35/build.py:212).
+ * Single-stage (routed expert) codes are decoded by an XOR identity that needs a basis
+ * without zero coordinates, which the E8P basis is (quantization/vq.py:96-118 has the
+ * same contract); `integer_vq_grouped` also takes the reference decoder's other options
+ * (integer_vq.py:111-258): basis=any (selector ids for zero coordinates), one selector
+ * table per expert (shared_table=false: Book is (E,256,1)), patch words (patched=true:
+ * Patch is (E,K/128,N) u16), tile lists of 8 or 16 rows and K-major blocks of 64.  These
+ * run on the MFMA tile kernel only.  The symbol always lists Patch, as the reference's
+ * host ABI does; without patched=true it is never read and may be null.
  *
  * Thread model: one thread per device session, one explicit stream
  * (backend/cuda/mod.rs:1-3).  Handles are immutable after orx_resolve: launches of one

@@ -138,12 +138,25 @@ def q4_integers(packed, table, coefficients=(4, 1)):
     return w.reshape(packed.shape[0], packed.shape[1] * 8).astype(np.int8)
 
 
-def q2_integers(indices, table):
-    """Single-stage int8 weights from u16 [N, K/8] (vq.py:185-195, without patches)."""
+def q2_integers(indices, table, patches=None):
+    """Single-stage int8 weights from u16 [N, K/8] (vq.py:184-194).
+
+    `patches` [N, K/128] u16 overrides at most one weight per row and group of 128: bit 15 says the
+    word is valid, bits 0-6 give the position inside the group, bits 7-14 the int8 value.
+    """
     indices = np.asarray(indices)
     if indices.dtype != np.uint16 or indices.ndim != 2:
         raise ValueError("expected u16 [N, K/8]")
-    return e8p_decode(indices, table).reshape(indices.shape[0], indices.shape[1] * 8)
+    weights = e8p_decode(indices, table).reshape(indices.shape[0], indices.shape[1] * 8).copy()
+    if patches is not None:
+        words = np.asarray(patches)
+        if words.dtype != np.uint16 or words.shape != (weights.shape[0], weights.shape[1] // 128):
+            raise ValueError("expected one u16 patch word per row and group of 128")
+        for row, group in zip(*np.nonzero(words >> 15)):
+            word = int(words[row, group])
+            stored = (word >> 7) & 255
+            weights[row, 128 * group + (word & 127)] = stored - 256 if stored > 127 else stored
+    return weights
 
 
 def q4_pack_k(packed, packed_k):

@@ -182,6 +182,42 @@ __device__ __forceinline__ uint2 decode_q2(const Q2ByteTables& t, uint32_t code)
     return make_uint2(b.x ^ m.x, b.y ^ m.y);
 }
 
+// Single-stage decode for any selector table, zero coordinates included (the selector decoder of
+// kernels/cuda/model/integer_vq.py:163-192 takes them; the XOR identity above does not): where the
+// basis value is zero the weight is 1 - 2p whatever the sign bit says, so those bytes are replaced.
+struct Q2GeneralTables {
+    uint2 basis[256];  // t
+    uint2 mask[256];   // mask3
+    uint2 zero[256];   // 0xFF where t == 0
+};
+
+__device__ __forceinline__ uint2 byte_zero_mask(uint32_t selector) {
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (((selector >> (4 * j)) & 3u) == 3u) lo |= 0xFFu << (8 * j);
+        if (((selector >> (4 * (j + 4))) & 3u) == 3u) hi |= 0xFFu << (8 * j);
+    }
+    return make_uint2(lo, hi);
+}
+
+__device__ __forceinline__ void build_tables(Q2GeneralTables& t, const uint32_t* __restrict__ book, int tid, int threads) {
+    for (int i = tid; i < 256; i += threads) {
+        const uint32_t s = book[i];
+        t.basis[i] = byte_basis_signed(s);
+        t.zero[i] = byte_zero_mask(s);
+        t.mask[i] = byte_mask_signed((uint32_t)i);
+    }
+}
+
+__device__ __forceinline__ uint2 decode_q2(const Q2GeneralTables& t, uint32_t code) {
+    const uint2 b = t.basis[(code >> 8) & 255u];
+    const uint2 m = t.mask[code & 255u];
+    const uint2 z = t.zero[(code >> 8) & 255u];
+    const uint32_t offset = (__popc(code & 255u) & 1u) ? 0xFFFFFFFFu : 0x01010101u;  // 1 - 2p in every byte
+    return make_uint2(((b.x ^ m.x) & ~z.x) | (offset & z.x), ((b.y ^ m.y) & ~z.y) | (offset & z.y));
+}
+
 // Byte offset of the 16-byte chunk `q` (0..3: 32 weights each) of weight row `row` in the 128-wide
 // K step `kt` of two-stage codes stored K-major, (K/packed_k, N, packed_k/8) u32 with packed_k = 128
 // or 64 (kernels/cuda/model/e8p_q4.py:250).

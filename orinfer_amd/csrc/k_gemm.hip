@@ -14,6 +14,8 @@
 // MFMAs of tile t.  Grouped (expert) tiles take (expert, first row, count) from device lists.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -90,6 +92,9 @@ struct GemmParams {
     int* partials;                 // split launches: int32 partial tiles, two slots per workgroup
     const void* w2;                // gate/up + SwiGLU: the Up matrix (w is Gate) and its scales
     const __half* ws2;
+    // routed single-stage codes, general form
+    const uint16_t* patch;         // (E, K/128, N) patch words or null
+    int book_stride;               // selector words between the experts' tables (0: one table for all)
 };
 
 template <int CODEC>
@@ -115,10 +120,16 @@ __host__ __device__ constexpr int weight_chunks() {
 // a wave's two column blocks are gate and up of the same 32 channels, and the epilogue rounds both
 // projections to fp16 and stores fp16(g / (1 + exp(-g)) * u) (int8_swiglu.py:10-57 with
 // integer_core.py:19-28, 261-264): no intermediate leaves the workgroup.
-template <int CODEC, int BM, int BN, int WAVES_M, bool GROUPED, bool SWIGLU = false>
+//
+// GENERAL (routed single-stage codes only; kernels/cuda/model/integer_vq.py:111-214): the selector table may
+// hold zero coordinates and may differ per expert (`book_stride`), the K-major blocks may be 64 wide, and
+// one weight per row and 128-wide K group may be overridden by a patch word: bit 15 valid, bits 7-14 the
+// int8 value, bits 0-6 the position in the group (integer_vq.py:193-202, quantization/vq.py:184-194).
+template <int CODEC, int BM, int BN, int WAVES_M, bool GROUPED, bool SWIGLU = false, bool GENERAL = false>
 __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     constexpr int WAVES_N = 4 / WAVES_M;
     static_assert(!SWIGLU || (CODEC == kW8 && !GROUPED && BN == 128 && WAVES_N == 2), "gate/up tile shape");
+    static_assert(!GENERAL || (CODEC == kQ2 && GROUPED && !SWIGLU), "the general decode is the routed single-stage one");
     constexpr int TM = BM / WAVES_M / 32, TN = BN / WAVES_N / 32;
     static_assert(TM >= 1 && TN >= 1, "wave tile must hold at least one 32x32 block");
     constexpr int A_CHUNKS = BM * 8 / 256;                        // uint4 per thread for A
@@ -127,7 +138,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
     __shared__ __align__(16) int8_t lds_a[BM * kPitch];
     __shared__ __align__(16) int8_t lds_w[BN * kPitch];
-    __shared__ typename Tables<CODEC>::type tables;
+    __shared__ typename std::conditional<GENERAL, Q2GeneralTables, typename Tables<CODEC>::type>::type tables;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
@@ -135,6 +146,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     int row0, rows_here;
     const int8_t* w_base = reinterpret_cast<const int8_t*>(p.w);
     const __half* ws = p.ws;
+    const uint32_t* book = p.book;
+    const uint16_t* patch = nullptr;
     if (GROUPED) {
         const int tile = blockIdx.y;
         if (tile >= p.tile_count[0]) return;
@@ -145,12 +158,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         if (rows_here <= 0) return;
         w_base += (int64_t)expert * p.expert_weight_stride;
         ws += (int64_t)expert * p.n;
+        if constexpr (GENERAL) {
+            book += (int64_t)expert * p.book_stride;
+            if (p.patch != nullptr) patch = p.patch + (int64_t)expert * (p.k / kBK) * p.n;
+        }
     } else {
         row0 = blockIdx.y * BM;
         rows_here = min(BM, p.m - row0);
     }
 
-    if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, 256);
+    if constexpr (CODEC != kW8) build_tables(tables, book, tid, 256);
 
     const int k_tiles = p.k / kBK;
     v4u held_a[A_CHUNKS], held_w[W_CHUNKS];
@@ -179,15 +196,16 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
                 byte = (int64_t)nn * p.k + kt * kBK + q * 16;
             else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
                 byte = ((int64_t)kt * p.n + nn) * (PER_ROW * 16) + q * 16;
-            else if (p.packed_k == 64)  // (K/64, N, 8 two-stage codes): two block rows per K step
-                byte = q4_k_major_chunk(64, p.n, nn, kt, q);
+            else if (p.packed_k == 64)  // (K/64, N, 8 codes): two block rows per K step
+                byte = CODEC == kQ2 ? ((int64_t)(kt * 2 + q) * p.n + nn) * 16 : q4_k_major_chunk(64, p.n, nn, kt, q);
             else  // (N, K/8 codes)
                 byte = ((int64_t)nn * k_tiles + kt) * (PER_ROW * 16) + q * 16;
             reg_w[i] = *reinterpret_cast<const v4u*>(w_base + byte);
         }
     };
 
-    auto store_tile = [&](const v4u (&reg_a)[A_CHUNKS], const v4u (&reg_w)[W_CHUNKS]) {
+    auto store_tile = [&](int kt, const v4u (&reg_a)[A_CHUNKS], const v4u (&reg_w)[W_CHUNKS]) {
+        (void)kt;
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + 256 * i;
@@ -216,6 +234,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
                     const uint2 lo = decode_q2(tables, pair[j] & 0xFFFFu), hi = decode_q2(tables, pair[j] >> 16);
                     dst[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
                 }
+                if constexpr (GENERAL) {
+                    // the thread that decoded the half group a patch points into overwrites that weight
+                    // (its own earlier stores to LDS are ordered before this one)
+                    if (patch != nullptr && n0 + nn < p.n) {
+                        const uint32_t word = patch[(int64_t)kt * p.n + n0 + nn];
+                        if ((word & 0x8000u) && ((word & 127u) >> 6) == (uint32_t)q)
+                            lds_w[nn * kPitch + (word & 127u)] = (int8_t)((word >> 7) & 255u);
+                    }
+                }
             }
         }
     };
@@ -231,7 +258,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     load_tile(0, held_a, held_w);
     __syncthreads();  // tables ready
     for (int kt = 0; kt < k_tiles; ++kt) {
-        store_tile(held_a, held_w);
+        store_tile(kt, held_a, held_w);
         __syncthreads();
         if (kt + 1 < k_tiles) load_tile(kt + 1, held_a, held_w);
         const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
@@ -563,6 +590,18 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
             break;
     }
     return hip_check(hipGetLastError(), "launch projection (mfma)");
+}
+
+// routed single-stage codes, general decode (any selector table, per-expert tables, patches, 64-wide blocks)
+int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStream_t stream) {
+    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    if (bm <= 32)
+        hipLaunchKernelGGL((gemm_kernel<kQ2, 32, 128, 1, true, false, true>), grid, block, 0, stream, p);
+    else if (bm == 64)
+        hipLaunchKernelGGL((gemm_kernel<kQ2, 64, 128, 2, true, false, true>), grid, block, 0, stream, p);
+    else
+        hipLaunchKernelGGL((gemm_kernel<kQ2, 128, 128, 2, true, false, true>), grid, block, 0, stream, p);
+    return hip_check(hipGetLastError(), "launch routed projection (general decode)");
 }
 
 bool use_resident(const orx_function& f, int rows);
@@ -1022,7 +1061,11 @@ int make_int8_swiglu(const Variant& v, orx_function* f) {
 // CU a unit of its own.
 // flags2: input form (0 int8 rows per slot, 1 int8 token rows gathered by slot, 2 fp16 rows quantised while
 // staged) + 4 * epilogue (0 plain, 1 SwiGLU).  Anything but 0 is a form of the resident kernel.
+// H (integer_vq_grouped only): 1 general decode, 2 patched, 4 one selector table per expert, 8 the list has a Patch.
+enum GroupedForm { kGeneralDecode = 1, kPatched = 2, kExpertTables = 4, kTakesPatch = 8 };
+
 bool grouped_uses_resident(const orx_function& f) {
+    if (f.H & kGeneralDecode) return false;
     if (f.algorithm == kResident || f.flags2 != 0) return true;
     return f.algorithm == kAuto && grouped_resident_eligible(f.N, f.K, f.block_m, f.tiles, 0, 0, f.capacity) &&
            grouped_resident_preferred(f.capacity, f.E, f.N);
@@ -1034,7 +1077,7 @@ int grouped_geometry(const orx_function& f, int rows, Geometry* g) {
         grouped_resident_geometry(f.K, f.flags2 & 3, f.flags2 >> 2, f.capacity, g);
         return ORX_OK;
     }
-    if (f.block_m <= 64 && f.algorithm != kMfma) {
+    if (f.block_m <= 64 && f.algorithm != kMfma && !(f.H & kGeneralDecode)) {
         stream_grouped_geometry(f.N, f.tiles, g);
         return ORX_OK;
     }
@@ -1074,6 +1117,12 @@ int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     p.tile_row = b.tile_row, p.ws = reinterpret_cast<const __half*>(b.ws);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
+    if (f.H & kGeneralDecode) {
+        p.patch = (f.H & kPatched) ? reinterpret_cast<const uint16_t*>(buffer("Patch")) : nullptr;
+        p.book_stride = (f.H & kExpertTables) ? 256 : 0;
+        p.tile_rows = f.block_m;
+        return launch_mfma_general(f.block_m, p, g, stream);
+    }
     if (f.block_m <= 64 && f.algorithm != kMfma)
         return stream_grouped_launch(p.a, p.w, p.book, p.ws, p.as, p.out, p.counts, p.offsets, p.tile_expert,
                                      p.tile_row, p.tile_count, f.N, f.K, f.tiles, f.block_m, f.packed_k, stream);
@@ -1093,8 +1142,17 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     const std::string input = v.string("input_dtype", "int8", &bad);
     const bool gather = v.boolean("gather", false, &bad);
     const std::string epilogue = v.string("epilogue", "none", &bad);
+    // integer_vq_grouped carries the reference's Patch buffer and its decoder options (integer_vq.py:217-258)
+    const bool vq = f->symbol == "integer_vq_grouped";
+    const bool patched = vq && v.boolean("patched", false, &bad);
+    const bool shared_table = !vq || v.boolean("shared_table", true, &bad);
+    const std::string basis = vq ? v.string("basis", "spread29", &bad) : std::string("spread29");
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
+    if (basis != "spread29" && basis != "any") {
+        set_error("%s: basis must be spread29 (no zero coordinates: the XOR decoders) or any (selector ids 0-7)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
     if ((input != "int8" && input != "float16") || (epilogue != "none" && epilogue != "swiglu") ||
         (input == "float16" && (gather || epilogue != "none"))) {
         set_error("%s: input_dtype int8 (optionally gather=true, epilogue=swiglu) or float16 (rows with RowMax, plain epilogue)",
@@ -1116,12 +1174,22 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
         set_error("%s: invalid E8P decode geometry", name);  // e8p_decode.py:52
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->block_m != 32 && f->block_m != 64 && f->block_m != 128) {
-        set_error("%s: block_m must be 32, 64 or 128 (rows per routed tile)", name);
+    const bool small_tile = vq && (f->block_m == 8 || f->block_m == 16);
+    if (f->block_m != 32 && f->block_m != 64 && f->block_m != 128 && !small_tile) {
+        set_error("%s: block_m must be 32, 64 or 128 (rows per routed tile%s)", name, vq ? "; also 8 or 16 here" : "");
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->packed_k != 128 && f->packed_k != 0) {
-        set_error("%s: packed_k must be 128 (K-major) or 0 (row-major per expert)", name);
+    if (f->packed_k != 128 && f->packed_k != 0 && !(vq && f->packed_k == 64)) {
+        set_error("%s: packed_k must be 128 (K-major)%s or 0 (row-major per expert)", name, vq ? ", 64" : "");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    // Zero coordinates, per-expert tables, patches, 8- and 16-row tile lists and 64-wide blocks are served by
+    // the MFMA tiles with the general decode.
+    const bool general = patched || !shared_table || basis == "any" || small_tile || f->packed_k == 64;
+    f->H = (general ? kGeneralDecode : 0) | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | (vq ? kTakesPatch : 0);
+    if (general && (f->flags2 != 0 || (f->algorithm != kAuto && f->algorithm != kMfma))) {
+        set_error("%s: patched, shared_table=false, basis=any, block_m 8|16 and packed_k=64 run on the MFMA tiles "
+                  "(algorithm auto or mfma, int8 rows, plain epilogue)", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->algorithm == kResident && !grouped_resident_eligible(f->N, f->K, f->block_m, f->tiles, 0, 0, f->capacity)) {
@@ -1156,6 +1224,8 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
         f->args.push_back({"Counts", ArgPointer, 4});
         f->args.push_back({"Offsets", ArgPointer, 4});
         f->args.push_back({"P", ArgPointer, 16});
+        // (E, K/128, N) u16 when patched; the reference binds a one-element dummy otherwise: never read, may be null
+        if (vq) f->args.push_back({"Patch", ArgPointer, patched ? 2u : nullable | 2u});
         if (rows16) f->args.push_back({"Q", ArgPointer, nullable | 8u});
         if (rows16 || swiglu) f->args.push_back({"RowMax", ArgPointer, 4});
         if (gathered) f->args.push_back({"SlotToken", ArgPointer, 4});
@@ -1312,8 +1382,9 @@ const Registration* gemm_registrations(int* count) {
      "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
     {"integer_vq_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
-     "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
+     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, patched=false, shared_table=true, basis=spread29|any, "
+     "algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
+     "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
     {"integer_experts", make_integer_experts,
      "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},

@@ -363,3 +363,34 @@ def test_session_threads_resolve_and_query_concurrently():
     for t in threads:
         t.join()
     assert not failures, failures[:5]
+
+
+def test_integer_vq_grouped_takes_the_reference_patch_buffer():
+    """integer_vq_grouped lists Patch like the reference's routed prim_func (integer_vq.py:230-258) in the
+    sorted host order; e8p_decode_grouped has none (e8p_decode.py:64).  The decoder options that the XOR
+    kernels do not take run on the MFMA tiles and refuse the other algorithms."""
+    shape = dict(rows=99, E=3, tiles=16, N=65, K=256)
+    want = ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "Patch", "TileCount", "TileExpert", "TileRow", "WS"]
+    for extra in (dict(), dict(patched=True), dict(shared_table=False), dict(basis="any"), dict(block_m=8),
+                  dict(block_m=16, patched=True, shared_table=False), dict(packed_k=64), dict(packed_k=0, patched=True)):
+        kern = lib.Kernel("integer_vq_grouped", **shape, **extra)
+        assert kern.arg_names == want, extra
+        grid, block, _ = kern.geometry()
+        if extra:
+            assert tuple(grid)[:2] == (1, 16) and tuple(block)[0] == 256, extra
+    assert "Patch" not in lib.Kernel("e8p_decode_grouped", **shape).arg_names
+    for symbol, bad in (("integer_vq_grouped", dict(patched=True, algorithm="stream")),
+                        ("integer_vq_grouped", dict(basis="any", algorithm="resident")),
+                        ("integer_vq_grouped", dict(basis="e8")),
+                        ("integer_vq_grouped", dict(block_m=24)),
+                        ("integer_vq_grouped", dict(packed_k=32)),
+                        ("e8p_decode_grouped", dict(block_m=8)),
+                        ("e8p_decode_grouped", dict(packed_k=64))):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel(symbol, **shape, **bad)
+    # the fused forms keep their places around Patch
+    fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16")
+    assert fused.arg_names == ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "Patch", "Q", "RowMax", "TileCount",
+                               "TileExpert", "TileRow", "WS"]
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", patched=True)

@@ -950,3 +950,96 @@ def test_five_launches_at_the_largest_gathered_batch_give_the_bits_of_seven():
     layer = programs.MoeLayer(1025, bigger["experts"], bigger["top_k"], bigger["hidden"], bigger["intermediate"],
                               bigger["gate_up"], bigger["gate_up_scales"], bigger["down"], bigger["down_scales"], block_m=32)
     assert not layer.fused_stages
+
+
+# The selector decoder's whole domain, after tests/cuda/operators/e8p_selector.py:23-94: tables drawn from
+# {0, +-2, +-6, +-10} (zero coordinates included), one table per expert or one for all, patch words on or
+# off (with the word that test plants: valid, value -128, last position), tile lists of 8 to 64 rows with
+# one row more than a tile, N = 65, unit power-of-two scales so that the result is the integer itself.
+@pytest.mark.parametrize("packed_k", [128, 64, 0])
+@pytest.mark.parametrize("bm,m,patched,shared", [(8, 1, False, True), (8, 3, True, False), (16, 17, True, True),
+                                                 (32, 33, False, False), (64, 65, False, True), (128, 130, True, False)])
+def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
+    rng = np.random.default_rng(orc.SEED + bm + packed_k)
+    e, n, k = 3, 65, 256
+    tables, codes, patches = [], [], []
+    for expert in range(e):
+        t = rng.choice(np.array([-10, -6, -2, 0, 2, 6, 10], np.int8), (256, 8))
+        tables.append(tables[0] if shared and expert else t)
+        codes.append(rng.integers(0, 65536, (n, k // 8), dtype=np.uint16))
+        words = rng.integers(0, 65536, (n, k // 128), dtype=np.uint16)
+        words[0, 0] = 32768 | (128 << 7) | 127
+        patches.append(words)
+    codes = np.stack(codes)
+    patch_np = np.stack([w.T for w in patches])  # (E, K/128, N)
+    book_np = np.stack([orc.selector_table(t) for t in (tables[:1] if shared else tables)])
+    weights = np.stack([orc.q2_integers(codes[x], tables[x], patches[x] if patched else None) for x in range(e)])
+    ws = np.full((e, n), 0.015625, np.float16)
+    counts_np = np.full(e, m, np.int32)
+    rows = e * m
+    a_q = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    a_s = np.full(rows, 0.0078125, np.float16)
+    offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+    cap = orc.tile_capacity(rows, e, bm)
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+    k128 = np.stack([orc.q2_pack_k128(c) for c in codes])
+    stored = codes if packed_k == 0 else k128 if packed_k == 128 else orc.q2_repack_k64(k128)
+    kern = gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
+                     patched=patched, shared_table=shared, basis="any")
+    out = torch.full((rows + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    book, patch = gu.dev(book_np), gu.dev(patch_np) if patched else None
+    counts = gu.dev(counts_np)
+    args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=book, C=out, Counts=counts, Offsets=gu.dev(offsets_np),
+                P=gu.dev(stored), Patch=patch, TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
+    kern(**args)
+    want = orc.grouped_project(a_q, a_s[:, None], weights, ws, counts_np, offsets_np)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows] == 91).all()
+    # every result is the exact integer dot product: 2^-6 * 2^-7 * sum, |sum| < 2^24 / ... fits fp16 only if small,
+    # so compare the integers where they are representable
+    exact = np.stack([a_q[x * m:(x + 1) * m].astype(np.int64) @ weights[x].astype(np.int64).T for x in range(e)]).reshape(rows, n)
+    small = np.abs(exact) < 2048
+    np.testing.assert_array_equal(got[:rows][small].astype(np.float64) * 8192, exact[small])
+    # tables and patches are read at launch time: an all-zero table leaves 1 - 2p and the patches
+    book.copy_(gu.dev(np.stack([orc.selector_table(np.zeros((256, 8), np.int8))] * book_np.shape[0])))
+    zero_w = np.stack([orc.q2_integers(codes[x], np.zeros((256, 8), np.int8), patches[x] if patched else None) for x in range(e)])
+    kern(**args)
+    np.testing.assert_array_equal(gu.host(out)[:rows], orc.grouped_project(a_q, a_s[:, None], zero_w, ws, counts_np, offsets_np))
+    book.copy_(gu.dev(book_np))
+    if patched:
+        patch.zero_()
+        plain = np.stack([orc.q2_integers(codes[x], tables[x]) for x in range(e)])
+        kern(**args)
+        np.testing.assert_array_equal(gu.host(out)[:rows], orc.grouped_project(a_q, a_s[:, None], plain, ws, counts_np, offsets_np))
+        patch.copy_(gu.dev(patch_np))
+    # an expert without rows is skipped
+    out.fill_(91)
+    counts[0] = 0
+    kern(**args)
+    got = gu.host(out)
+    assert (got[:m] == 91).all()
+    np.testing.assert_array_equal(got[m:rows], want[m:])
+
+
+def test_integer_vq_grouped_default_form_matches_e8p_decode_grouped():
+    # without decoder options the symbol runs the same kernels as e8p_decode_grouped; Patch may be null or a dummy
+    rng = np.random.default_rng(orc.SEED + 5)
+    e, n, k, bm = 6, 160, 256, 32
+    counts_np = np.array([3, 0, 40, 32, 1, 9], np.int32)
+    rows = int(counts_np.sum())
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.03, rows).astype(np.float16)
+    offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+    cap = orc.tile_capacity(rows, e, bm)
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    want = orc.grouped_project(a_q, a_s[:, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np, offsets_np)
+    for patch in (None, gu.dev(np.zeros(1, np.uint16))):
+        out = torch.full((rows, n), 55.0, dtype=torch.float16, device=gu.DEV)
+        gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm)(
+            A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=gu.dev(counts_np), Offsets=gu.dev(offsets_np),
+            P=gu.dev(stored), Patch=patch, TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
+        np.testing.assert_array_equal(gu.host(out), want)

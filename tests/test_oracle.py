@@ -689,3 +689,51 @@ def test_rotate_expert_a8_is_rotation_then_dispatch_and_its_sum_closes_the_nibbl
     assert np.array_equal(map2, slot_map) and np.array_equal(ds2, ds) and np.array_equal(row_sum, q.astype(np.int32).sum(1))
     q3, s3, sum3 = orc.rotate_expert_a8(x, signs)
     assert np.array_equal(sum3, row_sum) and row_sum[4] == 0 and s[4, 0] == 1
+
+
+def test_q2_patches_override_one_weight_per_row_and_group(table):
+    """Patch words (vq.py:184-194; the word the reference's own test plants, tests/cuda/operators/e8p_selector.py:38):
+    checked against a scalar loop over every (row, group) and on hand-built words."""
+    rng = np.random.default_rng(orc.SEED + 77)
+    n, k = 11, 384
+    codes = rng.integers(0, 65536, (n, k // 8), dtype=np.uint16)
+    words = rng.integers(0, 65536, (n, k // 128), dtype=np.uint16)
+    words[0, 0] = 32768 | (128 << 7) | 127  # valid, value byte 0x80 = -128, last position of group 0
+    words[1, 1] = (5 << 7) | 3              # not valid: ignored
+    plain = orc.q2_integers(codes, table)
+    got = orc.q2_integers(codes, table, words)
+    assert got[0, 127] == -128 and got[1, 128 + 3] == plain[1, 128 + 3]
+    want = plain.copy()
+    changed = 0
+    for row in range(n):
+        for group in range(k // 128):
+            word = int(words[row, group])
+            if word & 0x8000:
+                value = (word >> 7) & 0xFF
+                want[row, group * 128 + (word % 128)] = value - 256 if value >= 128 else value
+                changed += 1
+    np.testing.assert_array_equal(got, want)
+    assert int((got != plain).sum()) <= changed and changed > 5
+    # no valid bit anywhere: nothing changes; wrong shape is refused
+    np.testing.assert_array_equal(orc.q2_integers(codes, table, words & np.uint16(0x7FFF)), plain)
+    with pytest.raises(ValueError):
+        orc.q2_integers(codes, table, words[:, :2])
+
+
+def test_decode_with_zero_coordinates_and_the_selector_table_for_them():
+    """Tables with zeros (the selector decoder's domain, vq.py:74-93): a zero coordinate decodes to 1 - 2p
+    whatever its sign bit says, and its selector nibble is 3."""
+    rng = np.random.default_rng(orc.SEED + 78)
+    general = rng.choice(np.array([-10, -6, -2, 0, 2, 6, 10], np.int8), (256, 8))
+    general[7] = 0
+    book = orc.selector_table(general)
+    assert int(book[7, 0]) == 0x33333333
+    decoded = orc.e8p_decode(ALL, general).reshape(256, 256, 8)  # [basis row, low byte, coordinate]
+    parity = np.array([bin(u).count("1") & 1 for u in range(256)])
+    for u in (0, 1, 2, 0x55, 0xFE, 0xFF):
+        assert decoded[7, u].tolist() == [1 - 2 * parity[u]] * 8
+    zero_row, zero_col = np.nonzero(general == 0)
+    np.testing.assert_array_equal(decoded[zero_row, :, zero_col], np.broadcast_to(1 - 2 * parity, (len(zero_row), 256)))
+    some = rng.integers(0, 65536, 300)
+    np.testing.assert_array_equal(orc.e8p_decode(some.astype(np.uint16), general),
+                                  [orc.e8p_decode_scalar(c, general) for c in some])
