@@ -19,8 +19,9 @@
  * Pointer, I32, U32, I64, U64 and F32 values; every kernel of this path takes device
  * pointers and int32 row counts only, so those are the two kinds there are.
  *
- * Shapes: K is a multiple of 128 for every projection (the reference's int8 kernel
- * also takes K % 64 == 0, int8_projection.py:29: not served here); two-stage codes are
+ * Shapes: K is a multiple of 128 for codes and of 64 for int8 weights (int8_projection.py:29;
+ * a K that ends in half a step of 128 is served by the MFMA tile kernel at every row count);
+ * two-stage codes are
  * row-major (packed_k = 0) or K-major in blocks of 128 or 64 (packed_k = 128 | 64,
  * e8p_q4.py:78-80,250).  Blocks of 64 are read by the streaming and the MFMA tile
  * kernels at every row count; the one-row GEMV and the resident kernel read row-major

@@ -169,15 +169,21 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
 
     if constexpr (CODEC != kW8) build_tables(tables, book, tid, 256);
 
-    const int k_tiles = p.k / kBK;
+    // int8 weights may end in half a K step (K a multiple of 64, int8_projection.py:29): the missing halves of
+    // both operands are zeros.  Codes always come in whole steps.
+    const int k_tiles = CODEC == kW8 ? (p.k + kBK - 1) / kBK : p.k / kBK;
     v4u held_a[A_CHUNKS], held_w[W_CHUNKS];
+    const v4u zero_chunk = {0u, 0u, 0u, 0u};
 
     auto load_tile = [&](int kt, v4u (&reg_a)[A_CHUNKS], v4u (&reg_w)[W_CHUNKS]) {
 #pragma unroll
         for (int i = 0; i < A_CHUNKS; ++i) {
             const int c = tid + 256 * i;
             const int r = min(c >> 3, rows_here - 1), kc = c & 7;
-            reg_a[i] = *reinterpret_cast<const v4u*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
+            if (CODEC == kW8 && kt * kBK + kc * 16 >= p.k)
+                reg_a[i] = zero_chunk;
+            else
+                reg_a[i] = *reinterpret_cast<const v4u*>(p.a + (int64_t)(row0 + r) * p.k + kt * kBK + kc * 16);
         }
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) {
@@ -192,6 +198,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             }
             const int nn = min(n0 + c / PER_ROW, p.n - 1), q = c % PER_ROW;
             int64_t byte;
+            if (CODEC == kW8 && kt * kBK + q * 16 >= p.k) {
+                reg_w[i] = zero_chunk;
+                continue;
+            }
             if (CODEC == kW8)
                 byte = (int64_t)nn * p.k + kt * kBK + q * 16;
             else if (p.packed_k == 128)  // (K/128, N, 16 codes): one block row is PER_ROW*16 bytes
@@ -650,6 +660,7 @@ bool use_resident(const orx_function& f, int rows) {
 // rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
 bool split_preferred_to_big(const orx_function& f, int rows);
 bool use_big(const orx_function& f, int rows) {
+    if (f.K % kBK) return false;  // half a K step at the end: the 32-128 row tiles only
     return f.tiles == 256 || (f.tiles == 0 && rows > 384 && !split_preferred_to_big(f, rows));
 }
 
@@ -844,8 +855,9 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
     // validate_shape + K*128*127 < 2^31 (q4_projection.py:33-35, int8_projection.py:29)
-    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % kBK || (int64_t)f->K * 128 * 128 > 2147483647LL) {
-        set_error("%s: need M,N,K > 0, K a multiple of 128 and K*2^14 < 2^31", name);
+    const bool half_step = codec == kW8 && f->K % kBK == 64;  // int8_projection.py:29 takes K % 64 == 0
+    if (f->M <= 0 || f->N <= 0 || f->K <= 0 || (f->K % kBK && !half_step) || (int64_t)f->K * 128 * 128 > 2147483647LL) {
+        set_error("%s: need M,N,K > 0, K a multiple of 128 (of 64 for int8 weights) and K*2^14 < 2^31", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->stride < f->N) {
@@ -876,6 +888,14 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     if (f->algorithm < 0) {
         set_error("%s: algorithm must be auto, gemv, stream, resident or mfma", name);
         return ORX_ERR_BAD_VARIANT;
+    }
+    if (half_step) {
+        // a K that ends in half a step is served by the 32/64/128-row MFMA tiles at every row count
+        if ((f->algorithm != kAuto && f->algorithm != kMfma) || f->tiles == 256) {
+            set_error("%s: K = %d is not a multiple of 128: served by the MFMA tiles (algorithm auto or mfma, block_m up to 128)", name, f->K);
+            return ORX_ERR_BAD_VARIANT;
+        }
+        f->algorithm = kMfma;
     }
     if (f->algorithm == kResident &&
         (codec != kQ4 || f->capacity > 128 || !dense_resident_eligible(f->N, f->K, f->packed_k))) {
@@ -914,7 +934,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         const bool split = v.boolean("split_k", true, &bad);
         const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);
         if (bad) return ORX_ERR_BAD_VARIANT;
-        f->flags2 = (split ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);
+        f->flags2 = (split && !half_step ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);
         f->workspace_need = projection_workspace;
     }
     f->geometry = projection_geometry;

@@ -394,3 +394,17 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
                                "TileExpert", "TileRow", "WS"]
     with pytest.raises(lib.OrxError):
         lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", patched=True)
+
+
+def test_int8_weights_take_k_in_steps_of_64():
+    """int8_projection.py:29 accepts K % 64 == 0; codes come in whole groups of 128 only."""
+    kern = lib.Kernel("int8_projection", M=512, N=130, K=192, dynamic_rows=True)
+    for rows, tile in ((1, 32), (33, 64), (500, 128)):
+        grid, block, shared = kern.geometry(rows)
+        assert tuple(grid)[:2] == (2, -(-rows // tile)) and tuple(block)[0] == 256, rows
+    for symbol, bad in (("int8_projection", dict(K=192, algorithm="gemv")), ("int8_projection", dict(K=192, block_m=256)),
+                        ("int8_projection", dict(K=96)), ("e8p_q4_projection", dict(K=192))):
+        variant = dict(M=8, N=130, K=128)
+        variant.update(bad)
+        with pytest.raises(lib.OrxError):
+            lib.Kernel(symbol, **variant)

@@ -771,6 +771,26 @@ def test_w8_dynamic_capacity_stride_extremes(m):
     assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
 
 
+@pytest.mark.parametrize("k", [64, 192, 2752])
+@pytest.mark.parametrize("m", [1, 5, 33, 100, 200, 500])
+def test_w8_k_ends_in_half_a_step(m, k):
+    # int8_projection.py:29 takes any K that is a multiple of 64; the last K step is then half empty.
+    # A sentinel row sits right behind the activations and the weights, so a read past K would change the sums.
+    rng = np.random.default_rng(orc.SEED + m + k)
+    n, stride = 130, 136
+    x = rng.integers(-128, 128, (m + 1, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n + 1, k), dtype=np.int8)
+    x[m], w[n] = 127, 127
+    ws = (rng.uniform(0.2, 1.0, n) * 0.003).astype(np.float16)
+    ts = (rng.uniform(0.2, 1.0, m) * 0.005).astype(np.float16)
+    storage = torch.full((m + 2, stride), 99.0, dtype=torch.float32, device=gu.DEV)
+    gu.w8_project(gu.dev(x)[:m], gu.dev(ts), gu.dev(w)[:n], gu.dev(ws), dynamic=True, capacity=512, out=storage, stride=stride,
+                  dtype=torch.float32)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(x[:m], ts, w[:n], ws, np.float32))
+    assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
+
+
 @pytest.mark.parametrize("packed_k", [0, 64, 128])
 def test_q4_big_tile_tails_stride_sentinels(packed_k):
     rng = np.random.default_rng(orc.SEED + 9)
