@@ -30,7 +30,7 @@
  * without zero coordinates, which the E8P basis is (quantization/vq.py:96-118 has the
  * same contract); `integer_vq_grouped` also takes the reference decoder's other options
  * (integer_vq.py:111-258): basis=any (selector ids for zero coordinates), one selector
- * table per expert (shared_table=false: Book is (E,256,1)), patch words (patched=true:
+ * table per expert (shared_table=false, the reference's default: Book is (E,256,1)), patch words (patched=true:
  * Patch is (E,K/128,N) u16), tile lists of 8 or 16 rows and K-major blocks of 64.  These
  * run on the MFMA tile kernel only.  The symbol always lists Patch, as the reference's
  * host ABI does; without patched=true it is never read and may be null.

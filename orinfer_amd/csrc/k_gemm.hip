@@ -95,6 +95,7 @@ struct GemmParams {
     // routed single-stage codes, general form
     const uint16_t* patch;         // (E, K/128, N) patch words or null
     int book_stride;               // selector words between the experts' tables (0: one table for all)
+    int direct_rows;               // > 0: no tile list; expert blockIdx.z owns rows [z * direct_rows, (z + 1) * direct_rows)
 };
 
 template <int CODEC>
@@ -149,12 +150,19 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
     const uint32_t* book = p.book;
     const uint16_t* patch = nullptr;
     if (GROUPED) {
-        const int tile = blockIdx.y;
-        if (tile >= p.tile_count[0]) return;
-        const int expert = p.tile_expert[tile];
-        const int first = p.tile_row[tile];
-        row0 = p.offsets[expert] + first;
-        rows_here = min(p.tile_rows > 0 ? min(BM, p.tile_rows) : BM, p.counts[expert] - first);
+        int expert, first;
+        if (GENERAL && p.direct_rows > 0) {  // every expert has the same number of rows (integer_vq.py:217-228)
+            expert = blockIdx.z, first = blockIdx.y * BM;
+            row0 = expert * p.direct_rows + first;
+            rows_here = min(BM, p.direct_rows - first);
+        } else {
+            const int tile = blockIdx.y;
+            if (tile >= p.tile_count[0]) return;
+            expert = p.tile_expert[tile];
+            first = p.tile_row[tile];
+            row0 = p.offsets[expert] + first;
+            rows_here = min(p.tile_rows > 0 ? min(BM, p.tile_rows) : BM, p.counts[expert] - first);
+        }
         if (rows_here <= 0) return;
         w_base += (int64_t)expert * p.expert_weight_stride;
         ws += (int64_t)expert * p.n;
@@ -604,7 +612,7 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
 
 // routed single-stage codes, general decode (any selector table, per-expert tables, patches, 64-wide blocks)
 int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStream_t stream) {
-    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    const dim3 grid(g.grid[0], g.grid[1], g.grid[2]), block(256);
     if (bm <= 32)
         hipLaunchKernelGGL((gemm_kernel<kQ2, 32, 128, 1, true, false, true>), grid, block, 0, stream, p);
     else if (bm == 64)
@@ -1165,7 +1173,7 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     // integer_vq_grouped carries the reference's Patch buffer and its decoder options (integer_vq.py:217-258)
     const bool vq = f->symbol == "integer_vq_grouped";
     const bool patched = vq && v.boolean("patched", false, &bad);
-    const bool shared_table = !vq || v.boolean("shared_table", true, &bad);
+    const bool shared_table = !vq || v.boolean("shared_table", false, &bad);  // the reference's default (integer_vq.py:308)
     const std::string basis = vq ? v.string("basis", "spread29", &bad) : std::string("spread29");
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
@@ -1258,6 +1266,69 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     f->launch = grouped_launch;
     // several kernels with different block sizes serve this symbol: report the device-wide limits
     f->device_function = nullptr;
+    return ORX_OK;
+}
+
+// ---- integer_vq: every expert multiplies its own M rows (integer_vq.py:217-228, 262-300) -------------------
+// A, AS, Book, C, P, Patch, WS.  A is (E*M, K); expert e owns rows [e*M, (e+1)*M).  Runs on the MFMA tiles with
+// the general decode: any selector table, shared or per expert, patch words, blocks of 128 or 64 or row-major.
+int vq_direct_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)f.N, 128u);
+    g->grid[1] = ceil_div((uint32_t)f.M, (uint32_t)f.block_m);
+    g->grid[2] = (uint32_t)f.E;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+
+int vq_direct_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0), p.as = pointer_arg<const __half>(args, 1);
+    p.book = pointer_arg<const uint32_t>(args, 2), p.out = pointer_arg<void>(args, 3), p.w = pointer_arg<const void>(args, 4);
+    p.patch = (f.H & kPatched) ? pointer_arg<const uint16_t>(args, 5) : nullptr;
+    p.ws = pointer_arg<const __half>(args, 6);
+    p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
+    p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
+    p.book_stride = (f.H & kExpertTables) ? 256 : 0;
+    p.direct_rows = f.M;
+    return launch_mfma_general(f.block_m, p, g, stream);
+}
+
+int make_vq_direct(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->E = (int)v.integer("E", 0, &bad);
+    f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    const int block_m = (int)v.integer("block_m", 32, &bad);
+    f->packed_k = (int)v.integer("packed_k", 128, &bad);
+    const bool patched = v.boolean("patched", false, &bad);
+    const bool shared_table = v.boolean("shared_table", false, &bad);  // integer_vq.py:271
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->E <= 0 || f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 || (int64_t)f->K * 128 * 128 > 2147483647LL ||
+        (int64_t)f->E * f->M > 2147483647LL) {
+        set_error("integer_vq: invalid integer VQ geometry");  // integer_vq.py:86
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (block_m != 8 && block_m != 16 && block_m != 32 && block_m != 64) {
+        set_error("integer_vq: invalid VQ row tile (block_m 8, 16, 32 or 64)");  // integer_vq.py:89-90
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->packed_k != 128 && f->packed_k != 64 && f->packed_k != 0) {
+        set_error("integer_vq: packed_k must be 128 or 64 (K-major) or 0 (row-major per expert)");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->capacity = f->E * f->M;
+    f->block_m = block_m < 32 ? 32 : block_m;  // 8 and 16 rows ride in a 32-row tile: the row ranges are the same
+    f->H = kGeneralDecode | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | kTakesPatch;
+    const uint32_t nullable = 0x80000000u;
+    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4}, {"C", ArgPointer, 2},
+               {"P", ArgPointer, 16}, {"Patch", ArgPointer, patched ? 2u : nullable | 2u}, {"WS", ArgPointer, 2}};
+    f->geometry = vq_direct_geometry;
+    f->launch = vq_direct_launch;
+    f->device_function = block_m <= 32 ? reinterpret_cast<const void*>(&gemm_kernel<kQ2, 32, 128, 1, true, false, true>)
+                                       : reinterpret_cast<const void*>(&gemm_kernel<kQ2, 64, 128, 2, true, false, true>);
     return ORX_OK;
 }
 
@@ -1401,8 +1472,11 @@ const Registration* gemm_registrations(int* count) {
     {"e8p_decode_grouped", make_q2_grouped,
      "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
+    {"integer_vq", make_vq_direct,
+     "E, M (rows of every expert), N, K, block_m=32|8|16|64, packed_k=128|64|0, patched=false, shared_table=false",
+     "A,AS,Book,C,P,Patch,WS"},
     {"integer_vq_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, patched=false, shared_table=true, basis=spread29|any, "
+     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, patched=false, shared_table=false, basis=spread29|any, "
      "algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
     {"integer_experts", make_integer_experts,

@@ -371,16 +371,17 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
     kernels do not take run on the MFMA tiles and refuse the other algorithms."""
     shape = dict(rows=99, E=3, tiles=16, N=65, K=256)
     want = ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "Patch", "TileCount", "TileExpert", "TileRow", "WS"]
-    for extra in (dict(), dict(patched=True), dict(shared_table=False), dict(basis="any"), dict(block_m=8),
-                  dict(block_m=16, patched=True, shared_table=False), dict(packed_k=64), dict(packed_k=0, patched=True)):
+    for extra in (dict(shared_table=True), dict(patched=True), dict(), dict(shared_table=True, basis="any"), dict(block_m=8),
+                  dict(block_m=16, patched=True, shared_table=True), dict(packed_k=64), dict(packed_k=0, patched=True)):
         kern = lib.Kernel("integer_vq_grouped", **shape, **extra)
         assert kern.arg_names == want, extra
         grid, block, _ = kern.geometry()
-        if extra:
+        if extra != dict(shared_table=True):  # one table per expert is the reference's default (integer_vq.py:308)
             assert tuple(grid)[:2] == (1, 16) and tuple(block)[0] == 256, extra
     assert "Patch" not in lib.Kernel("e8p_decode_grouped", **shape).arg_names
     for symbol, bad in (("integer_vq_grouped", dict(patched=True, algorithm="stream")),
-                        ("integer_vq_grouped", dict(basis="any", algorithm="resident")),
+                        ("integer_vq_grouped", dict(algorithm="stream")),
+                        ("integer_vq_grouped", dict(shared_table=True, basis="any", algorithm="resident")),
                         ("integer_vq_grouped", dict(basis="e8")),
                         ("integer_vq_grouped", dict(block_m=24)),
                         ("integer_vq_grouped", dict(packed_k=32)),
@@ -389,11 +390,22 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
         with pytest.raises(lib.OrxError):
             lib.Kernel(symbol, **shape, **bad)
     # the fused forms keep their places around Patch
-    fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16")
+    fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", shared_table=True)
     assert fused.arg_names == ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "Patch", "Q", "RowMax", "TileCount",
                                "TileExpert", "TileRow", "WS"]
     with pytest.raises(lib.OrxError):
-        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", patched=True)
+        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", shared_table=True,
+                   patched=True)
+    # the form without a tile list: every expert multiplies its own M rows (integer_vq.py:217-228)
+    direct = lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, block_m=16, patched=True)
+    assert direct.arg_names == ["A", "AS", "Book", "C", "P", "Patch", "WS"]
+    grid, block, _ = direct.geometry()
+    assert tuple(grid) == (1, 1, 3) and tuple(block)[0] == 256
+    for bad in (dict(block_m=128), dict(K=200), dict(packed_k=32), dict(M=0)):
+        variant = dict(E=3, M=17, N=65, K=256)
+        variant.update(bad)
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("integer_vq", **variant)
 
 
 def test_int8_weights_take_k_in_steps_of_64():

@@ -1023,7 +1023,8 @@ def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
 
 
 def test_integer_vq_grouped_default_form_matches_e8p_decode_grouped():
-    # without decoder options the symbol runs the same kernels as e8p_decode_grouped; Patch may be null or a dummy
+    # with one table for all experts and no other decoder option the symbol runs the same kernels as
+    # e8p_decode_grouped; Patch may be null or a dummy
     rng = np.random.default_rng(orc.SEED + 5)
     e, n, k, bm = 6, 160, 256, 32
     counts_np = np.array([3, 0, 40, 32, 1, 9], np.int32)
@@ -1039,7 +1040,41 @@ def test_integer_vq_grouped_default_form_matches_e8p_decode_grouped():
     want = orc.grouped_project(a_q, a_s[:, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np, offsets_np)
     for patch in (None, gu.dev(np.zeros(1, np.uint16))):
         out = torch.full((rows, n), 55.0, dtype=torch.float16, device=gu.DEV)
-        gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm)(
+        gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, shared_table=True)(
             A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=gu.dev(counts_np), Offsets=gu.dev(offsets_np),
             P=gu.dev(stored), Patch=patch, TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
         np.testing.assert_array_equal(gu.host(out), want)
+
+
+@pytest.mark.parametrize("packed_k", [128, 64, 0])
+@pytest.mark.parametrize("bm,m,patched,shared", [(8, 1, False, True), (8, 3, True, False), (16, 17, True, True),
+                                                 (32, 33, False, False), (64, 65, False, True)])
+def test_integer_vq_direct_form(bm, m, patched, shared, packed_k):
+    # the cases of tests/cuda/operators/e8p_selector.py:23-94 through the symbol without a tile list:
+    # expert e multiplies rows [e*m, (e+1)*m)
+    rng = np.random.default_rng(orc.SEED + 3 * bm + packed_k)
+    e, n, k = 3, 65, 256
+    tables, patches = [], []
+    for expert in range(e):
+        t = rng.choice(np.array([-10, -6, -2, 0, 2, 6, 10], np.int8), (256, 8))
+        tables.append(tables[0] if shared and expert else t)
+        words = rng.integers(0, 65536, (n, k // 128), dtype=np.uint16)
+        words[0, 0] = 32768 | (128 << 7) | 127
+        patches.append(words)
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    weights = np.stack([orc.q2_integers(codes[x], tables[x], patches[x] if patched else None) for x in range(e)])
+    ws = np.full((e, n), 0.015625, np.float16)
+    a_q = rng.integers(-128, 128, (e * m, k), dtype=np.int8)
+    a_s = np.full(e * m, 0.0078125, np.float16)
+    k128 = np.stack([orc.q2_pack_k128(c) for c in codes])
+    stored = codes if packed_k == 0 else k128 if packed_k == 128 else orc.q2_repack_k64(k128)
+    book_np = np.stack([orc.selector_table(t) for t in (tables[:1] if shared else tables)])
+    out = torch.full((e * m + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    kern = gu.kernel("integer_vq", E=e, M=m, N=n, K=k, block_m=bm, packed_k=packed_k, patched=patched, shared_table=shared)
+    kern(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.dev(book_np), C=out, P=gu.dev(stored),
+         Patch=gu.dev(np.stack([w.T for w in patches])) if patched else None, WS=gu.dev(ws))
+    counts = np.full(e, m, np.int32)
+    want = orc.grouped_project(a_q, a_s[:, None], weights, ws, counts, np.arange(e, dtype=np.int32) * m)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:e * m], want)
+    assert (got[e * m] == 91).all()
