@@ -859,9 +859,15 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     f->tiles = (int)v.integer("block_m", 0, &bad);  // forced MFMA row tile, 0 = by row count
     const int passes = (int)v.integer("gemv_passes", 0, &bad);
     const std::string dtype = v.string("output_dtype", "float16", &bad);
-    const std::string algorithm = v.string("algorithm", "auto", &bad);
+    std::string algorithm = v.string("algorithm", "auto", &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
+    // The reference's factories name their schedules tensor_core, dp4a and int4_direct and take row tiles of
+    // 1-8, 16, 96 and 192 as well (e8p_q4.py:143-215, int8_projection.py:15-48): those are choices among SM87
+    // kernels, so they are accepted and the library picks its own kernel by the live rows.  Its other tile
+    // keys (block_n, block_k, stages, tail_m, group_m, cache_scales, an integer split_k) are not read.
+    if (algorithm == "tensor_core" || algorithm == "dp4a" || algorithm == "int4_direct") algorithm = "auto";
+    if ((f->tiles >= 1 && f->tiles <= 8) || f->tiles == 16 || f->tiles == 96 || f->tiles == 192) f->tiles = 0;
     // validate_shape + K*128*127 < 2^31 (q4_projection.py:33-35, int8_projection.py:29)
     const bool half_step = codec == kW8 && f->K % kBK == 64;  // int8_projection.py:29 takes K % 64 == 0
     if (f->M <= 0 || f->N <= 0 || f->K <= 0 || (f->K % kBK && !half_step) || (int64_t)f->K * 128 * 128 > 2147483647LL) {
@@ -939,7 +945,8 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     // inside the GEMM.  split_k=false and decode_in_gemm=true switch the two uses off one by one.
     {
         f->takes_workspace = v.boolean("workspace", false, &bad);
-        const bool split = v.boolean("split_k", true, &bad);
+        // (an integer split_k is the reference's K partition of its direct INT4 schedule: not a request here)
+        const bool split = v.fields.count("split_k") && v.fields.at("split_k").kind == Value::Number ? true : v.boolean("split_k", true, &bad);
         const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);
         if (bad) return ORX_ERR_BAD_VARIANT;
         f->flags2 = (split && !half_step ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);

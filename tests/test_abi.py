@@ -420,3 +420,22 @@ def test_int8_weights_take_k_in_steps_of_64():
         variant.update(bad)
         with pytest.raises(lib.OrxError):
             lib.Kernel(symbol, **variant)
+
+
+def test_projections_take_the_reference_factories_schedule_names():
+    """e8p_q4.projection(algorithm="tensor_core"|"dp4a"|"int4_direct", block_m=8.., split_k=1|2|4, ...) and
+    int8_projection(block_m=16.., block_n, block_k, stages, ...) (e8p_q4.py:143-215, int8_projection.py:15-48) pick
+    among SM87 kernels; the same keyword set resolves here to the handle that picks by row count."""
+    plain = lib.Kernel("e8p_q4_projection", M=64, N=512, K=1024, dynamic_rows=True)
+    for extra in (dict(algorithm="tensor_core", block_m=8, block_n=64, block_k=128, stages=2),
+                  dict(algorithm="dp4a", block_m=4, block_n=8),
+                  dict(algorithm="int4_direct", block_m=8, block_n=128, packed_k=128, basis_nonzero=True, split_k=2),
+                  dict(algorithm="tensor_core", block_m=96, group_m=4, cache_scales=True, tail_m=16)):
+        variant = dict(M=64, N=512, K=1024, dynamic_rows=True)
+        variant.update(extra)
+        kern = lib.Kernel("e8p_q4_projection", **variant)
+        if extra.get("packed_k", 0) == 0:
+            for rows in (1, 8, 64):
+                assert kern.geometry(rows) == plain.geometry(rows), (extra, rows)
+    w8 = lib.Kernel("int8_projection", M=256, N=512, K=1024, block_m=16, block_n=64, block_k=64, stages=2)
+    assert w8.geometry() == lib.Kernel("int8_projection", M=256, N=512, K=1024).geometry()
