@@ -236,17 +236,20 @@ __global__ __launch_bounds__(kMetaThreads) void route_metadata_kernel(
     int* local_id = local + assignments;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    for (int i = tid; i < kMetaWaves * experts; i += kMetaThreads) counters[i] = 0;
-    __syncthreads();
     // this wave's run of assignments, a multiple of 64 long
     const int per_wave = ((assignments + kMetaWaves - 1) / kMetaWaves + 63) & ~63;
     const int first = wave * per_wave, last = min(assignments, first + per_wave);
+    // the ids of the first two steps travel while the counters are cleared (2048 assignments are two steps per wave)
+    const int early_id[2] = {first + lane < last ? ids[first + lane] : -1, first + 64 + lane < last ? ids[first + 64 + lane] : -1};
+    for (int i = tid; i < kMetaWaves * experts; i += kMetaThreads) counters[i] = 0;
+    __syncthreads();
     int* mine = counters + wave * experts;
     const int id_bits = 32 - __builtin_clz(max(experts - 1, 1));
     for (int base = first; base < last; base += 64) {
         const int at = base + lane;
         const bool valid = at < last;
-        const int id = valid ? ids[at] : -1;
+        const int step = (base - first) >> 6;
+        const int id = step == 0 ? early_id[0] : step == 1 ? early_id[1] : valid ? ids[at] : -1;
         const int running = valid ? mine[id] : 0;  // nobody has written this expert in this step yet
         // the lanes that hold the same expert, found one id bit at a time
         unsigned long long same = __ballot(valid);
