@@ -39,6 +39,10 @@ bool dense_resident_eligible(int n, int k, int packed_k);
 void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g);
 int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                           void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
+bool dense_wide_eligible(int n, int k, int packed_k);
+void dense_wide_geometry(int n, Geometry* g);
+int dense_wide_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out,
+                      int rows, int n, int k, int stride, int packed_k, int out_f32, const Geometry& g, hipStream_t stream);
 bool grouped_resident_eligible(int n, int k, int block_m, int tiles, int input, int epilogue, int slots);
 bool grouped_resident_preferred(int rows, int experts, int n);
 void grouped_resident_geometry(int k, int input, int epilogue, int slots, Geometry* g);
@@ -65,7 +69,7 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
-enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4 };
+enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4, kWide = 5 };
 enum Flags2 { kNoSplit = 1, kNoExpand = 2 };  // orx_function::flags2 of a projection
 
 constexpr int kBK = 128;        // K bytes per tile step
@@ -622,8 +626,24 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
     return hip_check(hipGetLastError(), "launch routed projection (general decode)");
 }
 
+// Channel runs per CU over the whole K (k_wide.hip): two-stage codes, `algorithm=wide` by name, and by
+// `auto` at 65..128 rows while K is short enough.  Its time is 10 us + 0.4..0.55 us per K step of 128 whatever
+// N is (up to 96 channels per CU), where the split 128 x 128 tiles pay for N K: measured at 65-128 rows,
+// K-major and row-major alike, K = 1024: 9 against 23 us (N = 1024); 2560: 16-17 against 26-28 (N = 9728);
+// 4096: 20-23 against 29 (N = 11008), 17-20 against 23 (N = 4096); 5120: 31-32 against 40 (N = 17408),
+// 21-25 against 27-30 (N = 5120, 7168), 55-62 against 62-63 (N = 34816); 8192: 30-36 against 32 (N = 8192),
+// 70-83 against 72-74 (N = 28672); 9728 and up: slower (N = 5120, K = 17408: 56-69 against 41).  Below 65
+// rows the batched-decode kernels are as fast or faster except at N = 17408 (30 against 31-34 us), above 128
+// rows a second pass doubles the time (58-62 against 57 us at 160-256 rows).
+bool use_wide(const orx_function& f, int rows) {
+    if (f.flags != kQ4 || !dense_wide_eligible(f.N, f.K, f.packed_k)) return false;
+    if (f.algorithm == kWide) return true;
+    return f.algorithm == kAuto && f.tiles == 0 && rows >= 65 && rows <= 128 && f.K <= 6144;
+}
+
 bool use_resident(const orx_function& f, int rows);
 bool use_gemv(const orx_function& f, int rows) {
+    if (use_wide(f, rows)) return false;
     if (f.algorithm == kGemv) return true;
     if (f.algorithm != kAuto) return false;
     // K-major codes: 1 row (13.4 us at N=17408, K=5120; the streaming kernel takes 17.2), and 2 rows
@@ -722,6 +742,7 @@ int split_groups_for(const orx_function& f, int rows) {
 // Workspace bytes of a launch: the partial slots of a split launch, or the decoded weights of a
 // two-stage launch on the 256-row tiles.
 uint64_t projection_workspace(const orx_function& f, int rows) {
+    if (use_wide(f, rows)) return 0;
     if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows)) return 0;
     if (use_expand(f, rows)) return (uint64_t)f.N * f.K;
     if (use_big(f, rows)) return 0;
@@ -740,6 +761,10 @@ int launch_split(const GemmParams& p, int groups, hipStream_t stream) {
 }
 
 int projection_geometry(const orx_function& f, int rows, Geometry* g) {
+    if (use_wide(f, rows)) {
+        dense_wide_geometry(f.N, g);
+        return ORX_OK;
+    }
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_resident(f, rows)) {
         dense_resident_geometry(rows, f.N, f.K, f.packed_k, g);
@@ -779,6 +804,8 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.w = pointer_arg<const void>(args, f.rotate_input ? 6 : 5);
     void* workspace = f.takes_workspace ? pointer_arg<void>(args, f.workspace_arg) : nullptr;
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
+    if (use_wide(f, rows))
+        return dense_wide_launch(p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32, g, stream);
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out, signs);
     if (use_resident(f, rows)) {
         for (int first = 0; first < rows; first += 32) {
@@ -897,10 +924,15 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
                    : algorithm == "mfma"   ? kMfma
                    : algorithm == "stream"   ? kStream
                    : algorithm == "resident" ? kResident
+                   : algorithm == "wide"     ? kWide
                    : algorithm == "auto"     ? kAuto
                                              : -1;
     if (f->algorithm < 0) {
-        set_error("%s: algorithm must be auto, gemv, stream, resident or mfma", name);
+        set_error("%s: algorithm must be auto, gemv, stream, resident, wide or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kWide && (codec != kQ4 || !dense_wide_eligible(f->N, f->K, f->packed_k))) {
+        set_error("%s: algorithm=wide serves two-stage codes, row-major or K-major in blocks of 128", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (half_step) {
@@ -1463,7 +1495,7 @@ int make_q2_unpack(const Variant& v, orx_function* f) { return make_unpack(v, f,
 const Registration* gemm_registrations(int* count) {
     static const Registration rows[] = {
     {"e8p_q4_projection", make_q4_projection,
-     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|mfma, packed_k=0|64|128, output_dtype=float16|float32, "
+     "M, N, K, dynamic_rows=false, algorithm=auto|gemv|stream|resident|wide|mfma, packed_k=0|64|128, output_dtype=float16|float32, "
      "input_dtype=int8|float16, rotate=false, workspace=false, split_k=true, "
      "output_stride=N, block_m=0|32|64|128|256, gemv_passes=0, decode_in_gemm=false",
      "A,AS,Book,Out,S[,Signs],W[,Workspace][,m]"},

@@ -209,7 +209,8 @@ def test_handles_own_no_device_memory_and_say_what_workspace_they_need():
     assert err.value.code == lib.ORX_ERR_BAD_ARGUMENT
     handles = [lib.Kernel("e8p_q4_projection", M=64 + i, N=17408, K=5120, dynamic_rows=True, workspace=True)
                for i in range(1000)]
-    assert all(h.workspace_bytes(0) > 0 for h in handles[2:])
+    # up to 128 rows no launch of such a handle needs scratch (K = 5120: the channel-run kernel serves 65..128 rows)
+    assert all(h.workspace_bytes(0) == 0 for h in handles[:65]) and all(h.workspace_bytes(0) > 0 for h in handles[65:])
     assert lib.library().orx_workspace_bytes(None, 0, None) == lib.ORX_ERR_BAD_ARGUMENT
 
 

@@ -412,8 +412,10 @@ def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
         symbol, stored = "int8_projection", gu.dev(weights)
         call = lambda kern, out: kern(A=gu.dev(a), Output=out, TokenScale=gu.dev(a_s), Weight=stored, WeightScale=gu.dev(scales))
     variant = dict(M=m, N=n, K=k, output_dtype=dtype, output_stride=stride)
-    if m <= 64:
-        variant["algorithm"] = "mfma"  # `auto` gives so few rows of so small a matrix to the streaming kernel
+    if m <= 64 or (codec == "q4" and m <= 128):
+        # `auto` gives so few rows of so small a matrix to the streaming kernel, and 65..128 rows of two-stage
+        # codes with a short K to the channel-run kernel
+        variant["algorithm"] = "mfma"
     split = gu.kernel(symbol, **variant)
     whole = gu.kernel(symbol, split_k=False, **variant)
     grid_split, grid_whole = tuple(split.geometry()[0]), tuple(whole.geometry()[0])
@@ -789,6 +791,28 @@ def test_w8_k_ends_in_half_a_step(m, k):
     got = gu.host(storage)
     np.testing.assert_array_equal(got[:m, :n], orc.project(x[:m], ts, w[:n], ws, np.float32))
     assert (got[m:] == 99).all() and (got[:m, n:] == 99).all()
+
+
+# Channel runs per CU over the whole K (`algorithm=wide`): one and two row passes, a last pass of one row,
+# runs of 2, 97 (two channel passes, the second with one channel) and 100 channels per CU, a K of one step
+# and of many, both code layouts, strided fp32 output with sentinels, extremes outside the A8 range.
+@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("m,n,k", [(33, 300, 384), (64, 24832, 128), (100, 1000, 640), (128, 300, 5120), (129, 515, 256),
+                                   (200, 25600, 256), (256, 300, 1024)])
+def test_q4_channel_run_kernel(m, n, k, packed_k):
+    rng = np.random.default_rng(orc.SEED + m + n + k)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :4] = [-128, -1, 0, 127]
+    a_q[m - 1, -2:] = [127, -128]
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
+    storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
+    gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3, dtype=torch.float32,
+                  algorithm="wide", packed_k=packed_k)
+    got = gu.host(storage)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, orc.q4_integers(packed, TABLE), scales, np.float32))
+    assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+    out16 = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), algorithm="wide", packed_k=packed_k)
+    np.testing.assert_array_equal(gu.host(out16), orc.project(a_q, a_s, orc.q4_integers(packed, TABLE), scales))
 
 
 @pytest.mark.parametrize("packed_k", [0, 64, 128])
