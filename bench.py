@@ -57,6 +57,9 @@ def parse():
     p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--no-extra", action="store_true", help="only the contract workload")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--rows-probe", type=int, default=0, metavar="ROWS",
+                   help="launch config 1's projection at ROWS rows once per weight copy, eagerly, and exit (for counter runs of "
+                        "the kernel that serves that row count)")
     p.add_argument("--traffic-probe", action="store_true",
                    help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a plain copy of known size, then the "
                         "contract kernel once per weight copy, eagerly; no timing")
@@ -212,6 +215,15 @@ def main():
     bytes_c1 = workloads.algorithmic_bytes_q4(1, c1["n"], c1["k"])
     copies = -(-2 * CACHE_BYTES // (c1["n"] * c1["k"] // 2))  # aggregate footprint >= 2x the cache
     main_case = Q4Case(c1, copies, fused_input=True)
+    if args.rows_probe:
+        case = Q4Case(workloads.config1(args.rows_probe), copies)
+        case.quantize(stream.cuda_stream)
+        for i in range(copies):
+            case.project(i, stream.cuda_stream)
+        torch.cuda.synchronize()
+        grid, block, shared = case.proj.geometry(args.rows_probe)
+        print(json.dumps({"rows_probe": {"rows": args.rows_probe, "launches": copies, "grid": list(grid), "block": list(block), "lds": shared}}))
+        return
     if args.traffic_probe:
         # counter calibration: a device copy reads and writes exactly `probe.numel()` bytes
         probe = torch.empty(c1["n"] * c1["k"] // 2, dtype=torch.uint8, device="cuda").random_(0, 256)
