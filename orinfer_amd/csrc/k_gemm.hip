@@ -627,7 +627,7 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
 }
 
 // Channel runs per CU over the whole K (k_wide.hip): two-stage codes, `algorithm=wide` by name, and by
-// `auto` at 65..128 rows while K is short enough.  Its time is 10 us + 0.4..0.55 us per K step of 128 whatever
+// `auto` at 65..128 rows (33..64 rows of large matrices) while K is short enough.  Its time is 10 us + 0.4..0.55 us per K step of 128 whatever
 // N is (up to 96 channels per CU), where the split 128 x 128 tiles pay for N K: measured at 65-128 rows,
 // K-major and row-major alike, K = 1024: 9 against 23 us (N = 1024); 2560: 16-17 against 26-28 (N = 9728);
 // 4096: 20-23 against 29 (N = 11008), 17-20 against 23 (N = 4096); 5120: 31-32 against 40 (N = 17408),
@@ -638,7 +638,12 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
 bool use_wide(const orx_function& f, int rows) {
     if (f.flags != kQ4 || !dense_wide_eligible(f.N, f.K, f.packed_k)) return false;
     if (f.algorithm == kWide) return true;
-    return f.algorithm == kAuto && f.tiles == 0 && rows >= 65 && rows <= 128 && f.K <= 6144;
+    if (f.algorithm != kAuto || f.tiles != 0 || f.K > 6144) return false;
+    if (rows >= 65 && rows <= 128) return true;
+    // 33..64 rows of a large matrix would be two batched-decode launches: one pass here is faster while a CU's
+    // run fits one channel pass (N = 17408, K = 5120: 29.9 / 30.2 / 30.4 us at 33 / 48 / 64 rows against 31.2 / 31.8 /
+    // 34.3; N = 34816, two channel passes: 51-53 against 49-54, left alone)
+    return rows >= 33 && rows <= 64 && (int64_t)f.N * f.K >= ((int64_t)1 << 26) && f.N <= 96 * device_compute_units();
 }
 
 bool use_resident(const orx_function& f, int rows);
