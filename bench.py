@@ -309,6 +309,9 @@ def main():
     }
 
     extra = {}
+    # launches per graph for kernels of tens of microseconds: at least a hundred, so that a replay lasts milliseconds
+    # (a 26-launch graph of the 128-row projection reads 38-40 us per launch, a 260-launch one settles at 34.6)
+    short_graph = 8 * copies
     if not args.no_extra:
         # config 0 GEMV (int8 row in; the fp16-row form is `roofline.config0`)
         extra["config0_q4a8_gemv_m1"] = {"us": round(t0_plain * 1e6, 3), "GBps": round(b0 / t0_plain / 1e9, 1),
@@ -317,7 +320,7 @@ def main():
         sweep = {}
         for rows in (1, 8, 32, 128, 512):
             case = Q4Case(workloads.config1(rows), copies)
-            t = timed_graph(lambda i, s: case.project(i, s), 2 * copies)
+            t = timed_graph(lambda i, s: case.project(i, s), short_graph)
             b = workloads.algorithmic_bytes_q4(rows, case.n, case.k)
             ops = workloads.algorithmic_ops(rows, case.n, case.k)
             sweep[str(rows)] = {"us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
@@ -326,8 +329,8 @@ def main():
             del case
         extra["config1_q4a8_sweep"] = sweep
         # the same decode step as two launches (quantiser, then the projection on int8 rows)
-        t_a8 = timed_graph(lambda i, s: main_case.quantize(s), 2 * copies)
-        t_both = timed_graph(lambda i, s: (main_case.quantize(s), main_case.project(i, s)), 2 * copies)
+        t_a8 = timed_graph(lambda i, s: main_case.quantize(s), short_graph)
+        t_both = timed_graph(lambda i, s: (main_case.quantize(s), main_case.project(i, s)), short_graph)
         extra["config1_m1_two_launches"] = {"a8_us": round(t_a8 * 1e6, 3), "gemv_us": sweep["1"]["us"],
                                             "both_us": round(t_both * 1e6, 3)}
         # the production form of the step: signed block-128 rotation in front of the quantiser
@@ -339,17 +342,17 @@ def main():
             rot1(stream=s, Q=main_case.a_q, S=main_case.a_s, Signs=signs1, X=main_case.x)
             main_case.project(i, s)
 
-        t_rot_two = timed_graph(rotate_then_project, 2 * copies)
+        t_rot_two = timed_graph(rotate_then_project, short_graph)
         t_rot_one = timed_graph(lambda i, s: fused_rot(stream=s, A=main_case.x, AS=main_case.a_s, Book=book,
                                                        Out=main_case.out, S=main_case.scales, Signs=signs1,
-                                                       W=main_case.weights[i % copies]), 2 * copies)
+                                                       W=main_case.weights[i % copies]), short_graph)
         extra["config1_m1_rotated_input"] = {"rotate_a8_then_gemv_us": round(t_rot_two * 1e6, 3),
                                              "one_launch_us": round(t_rot_one * 1e6, 3)}
         # the same projection on the reference's storage layout (K-major blocks of 128)
         k_major = {}
         for rows in (1, 8, 32):
             case = Q4Case(workloads.config1(rows), copies, packed_k=128)
-            t = timed_graph(lambda i, s: case.project(i, s), 2 * copies)
+            t = timed_graph(lambda i, s: case.project(i, s), short_graph)
             b = workloads.algorithmic_bytes_q4(rows, case.n, case.k)
             k_major[str(rows)] = {"us": round(t * 1e6, 3), "GBps": round(b / t / 1e9, 1),
                                   "frac_hbm": round(b / t / 1e9 / HBM_PEAK_GBS, 4)}
@@ -383,7 +386,7 @@ def main():
         layer = programs.MoeLayer(c3["tokens"], c3["experts"], c3["top_k"], c3["hidden"], c3["intermediate"],
                                   c3["gate_up"], c3["gate_up_scales"], c3["down"], c3["down_scales"], block_m=32)
         x3, l3 = dev(c3["x"]), dev(c3["logits"])
-        t = timed_graph(lambda i, s: layer.run(x3, l3, stream=s), 20)
+        t = timed_graph(lambda i, s: layer.run(x3, l3, stream=s), 100)
         counts = layer.counts.cpu().numpy()
         touched = int((counts > 0).sum())
         code_bytes = touched * (c3["hidden"] * 2 * c3["intermediate"] + c3["intermediate"] * c3["hidden"]) // 4
@@ -406,7 +409,7 @@ def main():
             kern = Kernel("integer_e8p_gemv", E=e3, routes=k3, N=n, K=k, shared_input=shared)
             ws_dev = dev(scales)
             t = timed_graph(lambda i, st: kern(stream=st, A=a, AS=a_scale, Book=raw_book, C=out, IDs=routes, P=bank,
-                                               WS=ws_dev), 20)
+                                               WS=ws_dev), 100)
             moved = k3 * n * k // 4
             single[name] = {"us": round(t * 1e6, 2), "GBps_codes": round(moved / t / 1e9, 1)}
             del bank
@@ -417,8 +420,8 @@ def main():
         sorted_layer = programs.MoeLayer(1, e3, k3, h3, i3, c3["gate_up"], c3["gate_up_scales"], c3["down"],
                                          c3["down_scales"], block_m=32)
         x1, l1 = x3[:1].contiguous(), l3[:1].contiguous()
-        t_direct = timed_graph(lambda i, s: token_layer.run(x1, l1, stream=s), 20)
-        t_sorted = timed_graph(lambda i, s: sorted_layer.run(x1, l1, stream=s), 20)
+        t_direct = timed_graph(lambda i, s: token_layer.run(x1, l1, stream=s), 100)
+        t_sorted = timed_graph(lambda i, s: sorted_layer.run(x1, l1, stream=s), 100)
         extra["config3_single_token_layer"] = {"direct_routes_us": round(t_direct * 1e6, 2),
                                                "token_sorted_us": round(t_sorted * 1e6, 2)}
         del token_layer, sorted_layer
