@@ -13,6 +13,10 @@ Every function cites the reference file:line it follows.  Pinning status:
 * e8p_decode()           pinned by the scalar formula, the palette decoders and
                          the XOR/nibble identities of the reference's test_vq.py
 * q4_integers()          pinned by the exhaustive 65 536-code fixture
+* q2_integers()          decode as above; the patch words by a scalar loop over every
+                         (row, group) and the word the reference's own test plants
+                         (tests/cuda/operators/e8p_selector.py:38); tables with zero
+                         coordinates by the scalar decode and the 1 - 2p rule
 * a8()                   pinned by closed-form edge cases (ties, clamp, floor)
 * project()/rescale()    pinned by brute-force int64 dots and power-of-two KATs
 * router_topk()/metadata pinned by stable argsort / enumeration
