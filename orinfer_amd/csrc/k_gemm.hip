@@ -998,6 +998,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
 }
 
 int make_q4_projection(const Variant& v, orx_function* f) {
+    if (!two_stage_coefficients_ok(v, "e8p_q4_projection")) return ORX_ERR_BAD_VARIANT;
     int code = make_projection(v, f, kQ4);
     if (code != ORX_OK) return code;
     bool bad = false;
@@ -1425,6 +1426,7 @@ int make_integer_experts(const Variant& v, orx_function* f) {
     f->block_m = (int)v.integer("block_m", 16, &bad);
     f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
     const std::string codec = v.string("codec", "e8p_q4", &bad);
+    if (!bad && codec == "e8p_q4" && !two_stage_coefficients_ok(v, "integer_experts")) return ORX_ERR_BAD_VARIANT;
     // the reference's tile hints: checked as it checks them (moe.py:72-88), otherwise not used
     const long long block_n = v.integer("block_n", 64, &bad), block_k = v.integer("block_k", 128, &bad);
     const long long stages = v.integer("stages", 2, &bad), minimum_blocks = v.integer("minimum_blocks", 1, &bad);
@@ -1475,6 +1477,7 @@ int unpack_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
 }
 
 int make_unpack(const Variant& v, orx_function* f, int codec) {
+    if (codec == kQ4 && !two_stage_coefficients_ok(v, "e8p_q4_unpack")) return ORX_ERR_BAD_VARIANT;
     bool bad = false;
     f->N = (int)v.integer("N", 0, &bad);
     f->K = (int)v.integer("K", 0, &bad);

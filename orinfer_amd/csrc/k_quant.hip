@@ -904,6 +904,7 @@ int q4_embedding_launch(const orx_function& f, int rows, const Geometry& g, hipS
 }
 
 int make_q4_embedding(const Variant& v, orx_function* f) {
+    if (!two_stage_coefficients_ok(v, "e8p_q4_embedding")) return ORX_ERR_BAD_VARIANT;
     bool bad = false;
     f->capacity = f->M = (int)v.integer("M", 0, &bad);
     f->N = (int)v.integer("vocab", 0, &bad);

@@ -129,6 +129,31 @@ bool parse_variant(const char* json, Variant* out, std::string* error) {
         } else if (!strncmp(c.p, "null", 4)) {
             v.kind = Value::Null;
             c.p += 4;
+        } else if (*c.p == '[') {
+            // a flat list of integers (the reference factories' tuples, e.g. coefficients=(4, 1)) is kept as the
+            // string "4,1"
+            ++c.p;
+            v.kind = Value::String;
+            for (;;) {
+                c.skip();
+                if (*c.p == ']') break;
+                char* end = nullptr;
+                const long long item = strtoll(c.p, &end, 10);
+                if (end == c.p) {
+                    *error = "list of " + key + " must hold integers";
+                    return false;
+                }
+                c.p = end;
+                if (!v.text.empty()) v.text += ",";
+                v.text += std::to_string(item);
+                c.skip();
+                if (*c.p == ',') ++c.p;
+                else if (*c.p != ']') {
+                    *error = "bad list for " + key;
+                    return false;
+                }
+            }
+            ++c.p;
         } else {
             char* end = nullptr;
             v.number = strtod(c.p, &end);
@@ -197,6 +222,19 @@ std::string Variant::string(const char* key, const char* fallback, bool* bad) co
         return fallback;
     }
     return it->second.text;
+}
+
+// The two-stage codec's weights are 4 * coarse + residual (quantization/e8p_q4.py:19-29 allows other coprime
+// pairs; the model builder accepts [4, 1] only, models/qwen35/test_build.py:695-709, and so do the kernels here).
+bool two_stage_coefficients_ok(const Variant& v, const char* symbol) {
+    bool bad = false;
+    std::string given = v.string("coefficients", "4,1", &bad);
+    given.erase(std::remove(given.begin(), given.end(), ' '), given.end());
+    if (bad || given != "4,1") {
+        set_error("%s: coefficients must be (4, 1): the kernels decode 4 * coarse + residual", symbol);
+        return false;
+    }
+    return true;
 }
 
 // ---- catalog -------------------------------------------------------------------------------

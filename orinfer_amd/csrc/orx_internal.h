@@ -30,6 +30,8 @@ struct Variant {
 };
 
 bool parse_variant(const char* json, Variant* out, std::string* error);
+// false (with the error set) unless the variant's `coefficients` are absent or (4, 1)
+bool two_stage_coefficients_ok(const Variant& v, const char* symbol);
 
 enum ArgKind { ArgPointer = 0, ArgI32 = 1 };
 struct ArgSpec {

@@ -440,3 +440,18 @@ def test_projections_take_the_reference_factories_schedule_names():
                 assert kern.geometry(rows) == plain.geometry(rows), (extra, rows)
     w8 = lib.Kernel("int8_projection", M=256, N=512, K=1024, block_m=16, block_n=64, block_k=64, stages=2)
     assert w8.geometry() == lib.Kernel("int8_projection", M=256, N=512, K=1024).geometry()
+
+
+def test_two_stage_coefficients_other_than_4_1_are_refused():
+    """quantization/e8p_q4.py:19-29 allows other coprime pairs, the model builder only [4, 1]
+    (models/qwen35/test_build.py:695-709): the kernels decode 4 * coarse + residual and say so."""
+    shape = dict(M=4, N=256, K=512)
+    for good in (dict(), dict(coefficients=[4, 1]), dict(coefficients="4,1"), dict(coefficients="4, 1")):
+        lib.Kernel("e8p_q4_projection", **shape, **good)
+    for symbol, base in (("e8p_q4_projection", shape), ("e8p_q4_unpack", dict(N=256, K=512))):
+        for bad in ([3, 1], [7, 2], "5,2", [4], [4, 1, 0]):
+            with pytest.raises(lib.OrxError) as err:
+                lib.Kernel(symbol, **base, coefficients=bad)
+            assert err.value.code == lib.ORX_ERR_BAD_VARIANT and "coefficients" in str(err.value)
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("e8p_q4_projection", **shape, coefficients=[4.5, 1])
