@@ -70,7 +70,10 @@ typedef struct orx_function* orx_fn;
  * reference bakes into a cubin at compile time (shape, tile, layout, dtype), the way
  * package `Definition`s do (crates/orinfer-model-sdk/src/catalog.rs:32-50).
  * Example: orx_resolve("e8p_q4_projection",
- *                      "{\"M\":1,\"N\":9728,\"K\":2560,\"algorithm\":\"gemv\"}", &f). */
+ *                      "{\"M\":1,\"N\":9728,\"K\":2560,\"algorithm\":\"gemv\"}", &f).
+ * Values are integers, strings, booleans or flat lists of integers.  A key the family does
+ * not know is refused (ORX_ERR_BAD_VARIANT, the message lists the family's keys), as the
+ * reference's factories raise on an unknown keyword: no option is ever ignored silently. */
 int orx_resolve(const char* symbol, const char* variant_json, orx_fn* out);
 
 /* Drops a handle (cuModuleUnload in Session::cleanup).  Host memory only. */

@@ -899,6 +899,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     // kernels, so they are accepted and the library picks its own kernel by the live rows.  Its other tile
     // keys (block_n, block_k, stages, tail_m, group_m, cache_scales, an integer split_k) are not read.
     if (algorithm == "tensor_core" || algorithm == "dp4a" || algorithm == "int4_direct") algorithm = "auto";
+    for (const char* hint : {"block_n", "block_k", "stages", "tail_m", "group_m", "cache_scales", "basis_nonzero", "minimum_blocks"}) v.accept(hint);
     if ((f->tiles >= 1 && f->tiles <= 8) || f->tiles == 16 || f->tiles == 96 || f->tiles == 192) f->tiles = 0;
     // validate_shape + K*128*127 < 2^31 (q4_projection.py:33-35, int8_projection.py:29)
     const bool half_step = codec == kW8 && f->K % kBK == 64;  // int8_projection.py:29 takes K % 64 == 0
@@ -983,7 +984,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     {
         f->takes_workspace = v.boolean("workspace", false, &bad);
         // (an integer split_k is the reference's K partition of its direct INT4 schedule: not a request here)
-        const bool split = v.fields.count("split_k") && v.fields.at("split_k").kind == Value::Number ? true : v.boolean("split_k", true, &bad);
+        const bool split = v.has("split_k") && v.fields.at("split_k").kind == Value::Number ? true : v.boolean("split_k", true, &bad);
         const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);
         if (bad) return ORX_ERR_BAD_VARIANT;
         f->flags2 = (split && !half_step ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);

@@ -189,6 +189,7 @@ bool parse_variant(const char* json, Variant* out, std::string* error) {
 }
 
 long long Variant::integer(const char* key, long long fallback, bool* bad) const {
+    (*read)[key] = true;
     auto it = fields.find(key);
     if (it == fields.end() || it->second.kind == Value::Null) return fallback;
     // every integer of a variant is a shape, a count or a tile size and is stored in an int: a value
@@ -203,6 +204,7 @@ long long Variant::integer(const char* key, long long fallback, bool* bad) const
 }
 
 bool Variant::boolean(const char* key, bool fallback, bool* bad) const {
+    (*read)[key] = true;
     auto it = fields.find(key);
     if (it == fields.end() || it->second.kind == Value::Null) return fallback;
     if (it->second.kind != Value::Bool) {
@@ -214,6 +216,7 @@ bool Variant::boolean(const char* key, bool fallback, bool* bad) const {
 }
 
 std::string Variant::string(const char* key, const char* fallback, bool* bad) const {
+    (*read)[key] = true;
     auto it = fields.find(key);
     if (it == fields.end() || it->second.kind == Value::Null) return fallback;
     if (it->second.kind != Value::String) {
@@ -365,6 +368,12 @@ int resolve(const char* symbol, const char* variant_json, orx_fn* out) {
     f->symbol = family;
     const int code = r->factory(variant, f.get());
     if (code != ORX_OK) return code;
+    for (const auto& field : variant.fields) {
+        if (!variant.read->count(field.first)) {
+            set_error("orx_resolve %s: unknown variant key %s (keys: %s)", family.c_str(), field.first.c_str(), r->variant_keys);
+            return ORX_ERR_BAD_VARIANT;
+        }
+    }
     if (f->geometry == nullptr || f->launch == nullptr || f->args.empty()) {
         set_error("orx_resolve %s: incomplete kernel record", symbol);
         return ORX_ERR_BAD_VARIANT;

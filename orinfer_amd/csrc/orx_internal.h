@@ -6,6 +6,7 @@
 
 #include <atomic>
 #include <map>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -22,7 +23,16 @@ struct Value {
 
 struct Variant {
     std::map<std::string, Value> fields;
-    bool has(const char* key) const { return fields.count(key) != 0; }
+    // Keys a factory has looked at.  orx_resolve refuses a variant with a key nobody read: a misspelt or
+    // unsupported option must not silently resolve to the default behaviour (the reference's factories raise
+    // on an unknown keyword).  `accept` marks a key that is understood and deliberately not used.
+    // (shared by the copies a factory hands to another factory)
+    std::shared_ptr<std::map<std::string, bool>> read = std::make_shared<std::map<std::string, bool>>();
+    void accept(const char* key) const { (*read)[key] = true; }
+    bool has(const char* key) const {
+        (*read)[key] = true;
+        return fields.count(key) != 0;
+    }
     // Integer field with a default; sets `bad` if the field exists but is not an integer.
     long long integer(const char* key, long long fallback, bool* bad) const;
     bool boolean(const char* key, bool fallback, bool* bad) const;

@@ -455,3 +455,26 @@ def test_two_stage_coefficients_other_than_4_1_are_refused():
             assert err.value.code == lib.ORX_ERR_BAD_VARIANT and "coefficients" in str(err.value)
     with pytest.raises(lib.OrxError):
         lib.Kernel("e8p_q4_projection", **shape, coefficients=[4.5, 1])
+
+
+def test_unknown_variant_keys_are_refused():
+    """A key no factory reads (a typo, an option of another symbol) fails the resolve and the message lists the
+    symbol's keys, as a reference factory raises on an unknown keyword; the reference's own tile hints are known."""
+    for symbol, variant, stray in (("e8p_q4_projection", dict(M=4, N=256, K=512), dict(output_strid=300)),
+                                   ("e8p_q4_projection", dict(M=4, N=256, K=512), dict(patched=True)),
+                                   ("int8_projection", dict(M=4, N=256, K=512), dict(packed=128)),
+                                   ("router_topk", dict(M=4, E=64, top_k=4), dict(quantise_hidden=512)),
+                                   ("e8p_decode_grouped", dict(rows=64, E=4, tiles=8, N=256, K=256), dict(shared_table=True)),
+                                   ("activation_quantization", dict(K=512), dict(groups=4)),
+                                   ("moe_combine", dict(M=4, top_k=2, H=256), dict(shared=True))):
+        lib.Kernel(symbol, **variant)
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel(symbol, **variant, **stray)
+        key = next(iter(stray))
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT and key in str(err.value) and "keys:" in str(err.value), (symbol, str(err.value))
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("swiglu?I=128&J=3")
+    # hints of the reference factories that choose among its own kernels are accepted and change nothing
+    lib.Kernel("e8p_q4_projection", M=4, N=256, K=512, block_n=64, block_k=128, stages=2, tail_m=0, group_m=0, cache_scales=False,
+               basis_nonzero=True, split_k=1)
+    lib.Kernel("int8_projection", M=64, N=256, K=512, block_n=128, block_k=64, stages=2)
