@@ -1221,8 +1221,24 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     const bool patched = vq && v.boolean("patched", false, &bad);
     const bool shared_table = !vq || v.boolean("shared_table", false, &bad);  // the reference's default (integer_vq.py:308)
     const std::string basis = vq ? v.string("basis", "spread29", &bad) : std::string("spread29");
+    // The reference factories' other keywords (integer_vq.py:300-322, e8p_decode.py:36-58): `kind` is e8p; Book is
+    // the (256, 1) selector table, which the reference calls shortbook + selectorbook (its raw-basis and sign-table
+    // forms of Book are not read here); the rest chooses among its own schedules and is accepted as a hint.
+    const std::string kind = v.string("kind", "e8p", &bad);
+    const bool selector_book = v.boolean("selectorbook", true, &bad) && v.boolean("shortbook", true, &bad);
+    for (const char* hint : {"block_n", "num_stages", "stages", "byte_permute", "group_n", "warp_decode", "split_k", "parity_xor",
+                             "warp_private"})
+        v.accept(hint);
+    // dynamic_rows: the reference's kernel then takes the live row count as a trailing `m` (integer_vq.py:234-258
+    // with kernels/shared/rows.py); the tile lists already bound every row these kernels touch, so `m` is taken
+    // and only checked against the capacity
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
+    if (kind != "e8p" || !selector_book) {
+        set_error("%s: kind must be e8p and Book the (256, 1) selector table (shortbook and selectorbook)", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
     if (basis != "spread29" && basis != "any") {
         set_error("%s: basis must be spread29 (no zero coordinates: the XOR decoders) or any (selector ids 0-7)", name);
         return ORX_ERR_BAD_VARIANT;
@@ -1307,6 +1323,7 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
         f->args.push_back({"TileExpert", ArgPointer, 4});
         f->args.push_back({"TileRow", ArgPointer, 4});
         f->args.push_back({"WS", ArgPointer, 2});
+        if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     }
     f->geometry = grouped_geometry;
     f->launch = grouped_launch;
@@ -1351,7 +1368,14 @@ int make_vq_direct(const Variant& v, orx_function* f) {
     f->packed_k = (int)v.integer("packed_k", 128, &bad);
     const bool patched = v.boolean("patched", false, &bad);
     const bool shared_table = v.boolean("shared_table", false, &bad);  // integer_vq.py:271
+    const std::string kind = v.string("kind", "e8p", &bad);
+    const bool selector_book = v.boolean("selectorbook", true, &bad) && v.boolean("shortbook", true, &bad);
+    for (const char* hint : {"block_n", "num_stages", "byte_permute"}) v.accept(hint);
     if (bad) return ORX_ERR_BAD_VARIANT;
+    if (kind != "e8p" || !selector_book) {
+        set_error("integer_vq: kind must be e8p and Book the (256, 1) selector table (shortbook and selectorbook)");
+        return ORX_ERR_BAD_VARIANT;
+    }
     if (f->E <= 0 || f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 || (int64_t)f->K * 128 * 128 > 2147483647LL ||
         (int64_t)f->E * f->M > 2147483647LL) {
         set_error("integer_vq: invalid integer VQ geometry");  // integer_vq.py:86
@@ -1518,15 +1542,15 @@ const Registration* gemm_registrations(int* count) {
     {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=tensor_core|dp4a, block_m, block_n (checked, not used)",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
     {"e8p_decode_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
-     "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
+     "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, dynamic_rows=false, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
+     "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_vq", make_vq_direct,
      "E, M (rows of every expert), N, K, block_m=32|8|16|64, packed_k=128|64|0, patched=false, shared_table=false",
      "A,AS,Book,C,P,Patch,WS"},
     {"integer_vq_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, patched=false, shared_table=false, basis=spread29|any, "
+     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, dynamic_rows=false, patched=false, shared_table=false, basis=spread29|any, "
      "algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
-     "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS"},
+     "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_experts", make_integer_experts,
      "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},

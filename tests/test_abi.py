@@ -478,3 +478,21 @@ def test_unknown_variant_keys_are_refused():
     lib.Kernel("e8p_q4_projection", M=4, N=256, K=512, block_n=64, block_k=128, stages=2, tail_m=0, group_m=0, cache_scales=False,
                basis_nonzero=True, split_k=1)
     lib.Kernel("int8_projection", M=64, N=256, K=512, block_n=128, block_k=64, stages=2)
+
+
+def test_routed_decode_symbols_take_the_reference_factories_keywords():
+    """integer_vq_grouped(..., kind="e8p", shortbook=True, selectorbook=True, byte_permute=True, num_stages, block_n)
+    as tests/cuda/operators/e8p_selector.py:66-79 calls it; the reference's other Book forms are refused."""
+    shape = dict(rows=99, E=3, tiles=16, N=65, K=256)
+    hints = dict(kind="e8p", shared_table=True, patched=False, block_m=32, block_n=128, shortbook=True, selectorbook=True,
+                 num_stages=1, byte_permute=True)
+    assert lib.Kernel("integer_vq_grouped", **shape, **hints).geometry() == lib.Kernel("integer_vq_grouped", **shape, shared_table=True).geometry()
+    lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, kind="e8p", shortbook=True, selectorbook=True, num_stages=2, block_n=128, byte_permute=True)
+    lib.Kernel("e8p_decode_grouped", **shape, block_n=32, split_k=2, parity_xor=True)
+    dynamic = lib.Kernel("integer_vq_grouped", **shape, shared_table=True, dynamic_rows=True)
+    assert dynamic.arg_names[-1] == "m" and dynamic.arg_names[:-1] == lib.Kernel("integer_vq_grouped", **shape, shared_table=True).arg_names
+    for bad in (dict(selectorbook=False), dict(shortbook=False), dict(kind="scalar")):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("integer_vq_grouped", **shape, **bad)
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, **bad)

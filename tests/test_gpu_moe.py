@@ -1078,3 +1078,35 @@ def test_integer_vq_direct_form(bm, m, patched, shared, packed_k):
     got = gu.host(out)
     np.testing.assert_array_equal(got[:e * m], want)
     assert (got[e * m] == 91).all()
+
+
+@pytest.mark.parametrize("symbol", ["e8p_decode_grouped", "integer_vq_grouped"])
+def test_grouped_q2_with_dynamic_rows_takes_m_last(symbol):
+    # dynamic_rows (integer_vq.py:234-258): the same launch with the live row count as a trailing scalar
+    rng = np.random.default_rng(orc.SEED + 17)
+    e, n, k, bm = 5, 160, 256, 32
+    counts_np = np.array([3, 0, 40, 32, 9], np.int32)
+    rows, cap_rows = int(counts_np.sum()), 128
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    a_q = rng.integers(-127, 128, (cap_rows, k), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.03, cap_rows).astype(np.float16)
+    offsets_np, tile_offsets, total = orc.expert_offsets(counts_np, bm)
+    cap = orc.tile_capacity(cap_rows, e, bm)
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    extra = dict(shared_table=True) if symbol == "integer_vq_grouped" else {}
+    kern = gu.kernel(symbol, rows=cap_rows, E=e, tiles=cap, N=n, K=k, block_m=bm, dynamic_rows=True, **extra)
+    assert kern.arg_names[-1] == "m"
+    out = torch.full((cap_rows, n), 55.0, dtype=torch.float16, device=gu.DEV)
+    args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=gu.dev(counts_np), Offsets=gu.dev(offsets_np),
+                P=gu.dev(stored), TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws), m=rows)
+    if symbol == "integer_vq_grouped":
+        args["Patch"] = None
+    kern(**args)
+    want = orc.grouped_project(a_q[:rows], a_s[:rows, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np, offsets_np)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows:] == 55).all()
+    with pytest.raises(gu.lib.OrxError):
+        kern(**{**args, "m": cap_rows + 1})
