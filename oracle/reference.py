@@ -21,6 +21,11 @@ Every function cites the reference file:line it follows.  Pinning status:
 * project()/rescale()    pinned by brute-force int64 dots and power-of-two KATs
 * router_topk()/metadata pinned by stable argsort / enumeration
 * swiglu(), combine()    pinned by direct formula on tiny inputs
+* split_planes(), nibble_table(), nibble_decode(), plane_project()
+                         the plane words by the reference's mask-and-shift form and its
+                         test's low + 16 high == permuted codes; the nibble decode by
+                         2y + 1 == e8p_decode() over all 65 536 codes; plane_project by
+                         project() on the same integers and a planted Sum
 * rotate(), rotate_a8()  pinned by the Sylvester Hadamard matrix (exact on small
                          integers), dot preservation and the involution of the
                          reference's test_vq.py:123-130
@@ -511,6 +516,128 @@ def nibble_planes(q):
     """int8 codes -> (low, high) unsigned nibbles of the two's-complement byte (rotation_a8.py:489-491)."""
     b = np.asarray(q, np.int8).view(np.uint8)
     return b & 15, b >> 4
+
+
+# --------------------------------------------------------------------------
+# Nibble planes: the A8 hand-over of the reference's INT4 expert kernels
+# --------------------------------------------------------------------------
+# Nibble i of a plane word holds coordinate PLANE_ORDER[i] of its eight codes
+# (kernels/cuda/model/e8p_core.py:63-78, rotation_a8.py:489-491).
+PLANE_ORDER = (0, 2, 1, 3, 4, 6, 5, 7)
+
+
+def split_planes(a_q):
+    """int8 (rows, K) -> (Low, High, Sum): u32 (rows, K/8) words and the int32 row sums.
+
+    a = low + 16 * high with low the unsigned and high the signed nibble of the byte
+    (kernels/cuda/model/e8p_exact.py:3-4, :18-46); the words take the eight nibbles in
+    PLANE_ORDER.  Sum is what the exact kernels add back for w = 2y + 1.
+    """
+    a_q = np.asarray(a_q, np.int8)
+    rows, k = a_q.shape
+    b = a_q.view(np.uint8).reshape(rows, k // 8, 8)[:, :, list(PLANE_ORDER)].astype(np.uint32)
+    shifts = np.arange(0, 32, 4, dtype=np.uint32)
+    low = np.bitwise_or.reduce((b & 15) << shifts, axis=-1).astype(np.uint32)
+    high = np.bitwise_or.reduce((b >> 4) << shifts, axis=-1).astype(np.uint32)
+    return low, high, a_q.astype(np.int32).sum(axis=1).astype(np.int32)
+
+
+def planes_group_major(words):
+    """(rows, K/8) plane words -> (K/64, rows, 8): K64-major (kernels/cuda/model/e8p_prefill.py:55-56, :79-80)."""
+    rows, w = words.shape
+    return np.ascontiguousarray(words.reshape(rows, w // 8, 8).transpose(1, 0, 2))
+
+
+def planes_row_major(words):
+    """Inverse of `planes_group_major`."""
+    g, rows, _ = words.shape
+    return np.ascontiguousarray(words.transpose(1, 0, 2)).reshape(rows, g * 8)
+
+
+def planes_values(low, high):
+    """(rows, K/8) words -> int64 (rows, K) values low_u4 + 16 * high_s4 in K order."""
+    shifts = np.arange(0, 32, 4, dtype=np.uint32)
+    lo = ((np.asarray(low, np.uint32)[..., None] >> shifts) & 15).astype(np.int64)
+    hi = ((np.asarray(high, np.uint32)[..., None] >> shifts) & 15).astype(np.int64)
+    hi = np.where(hi >= 8, hi - 16, hi)
+    inverse = np.argsort(PLANE_ORDER)
+    return (lo + 16 * hi)[..., inverse].reshape(low.shape[0], low.shape[1] * 8)
+
+
+def nibble_table(selectors):
+    """Selector words -> words of signed nibbles (w - 1) / 2 at even parity, in PLANE_ORDER.
+
+    python/orinfer_build/quantization/vq.py:105-118 (and `direct_nibble_basis`,
+    kernels/cuda/model/e8p_core.py:45-60): id 0..2 are +1, +3, +5, id 4..6 their negatives;
+    zero coordinates (id 3, 7) have no nibble form and are refused.
+    """
+    sel = np.asarray(selectors, np.uint32).reshape(-1)
+    shifts = np.arange(0, 32, 4, dtype=np.uint32)
+    ids = (sel[:, None] >> shifts) & 7
+    if np.any((ids & 3) == 3) or np.any(sel & np.uint32(0x88888888)):
+        raise ValueError("the nibble form needs a nonzero spread29 basis")
+    half = np.array([1, 3, 5, 0, -1, -3, -5, 0], np.int32)[ids]
+    words = np.bitwise_or.reduce((half[:, list(PLANE_ORDER)] & 15).astype(np.uint32) << shifts, axis=1)
+    return words.astype(np.uint32).reshape(-1, 1)
+
+
+def nibble_decode(codes, nibbles):
+    """u16 codes -> int64 (..., 8) values y = (w - 1) / 2 in K order, from a nibble table.
+
+    kernels/cuda/model/e8p_core.py:7-10: sign bit SIGN_BITS[j] negates coordinate j's nibble
+    (xor 0xe: the stored values are odd), odd parity lowers every nibble by one (xor 1) and
+    flips the first coordinate's sign as well.
+    """
+    codes = np.asarray(codes, np.uint16).astype(np.uint32)
+    book = np.asarray(nibbles, np.uint32).reshape(-1)[codes >> 8]
+    low = codes & 255
+    parity = np.zeros_like(low)
+    for bit in range(8):
+        parity ^= (low >> bit) & 1
+    out = np.empty(codes.shape + (8,), np.int64)
+    for position, coordinate in enumerate(PLANE_ORDER):
+        nib = (book >> np.uint32(4 * position)) & 15
+        flip = (low >> SIGN_BITS[coordinate]) & 1
+        nib = nib ^ (flip * 0xE) ^ parity
+        if position == 0:
+            nib = nib ^ (parity * 0xE)
+        out[..., coordinate] = np.where(nib >= 8, nib.astype(np.int64) - 16, nib.astype(np.int64))
+    return out
+
+
+def plane_project(low, high, total, half_weights, weight_scale, token_scale, coefficient_sum=1):
+    """Out = rescale(2 * sum_k y[n, k] * (low + 16 high)[m, k] + coefficient_sum * Sum[m]).
+
+    kernels/cuda/model/e8p_core.py:173-189 (single-stage, coefficient_sum 1) and :154-170
+    (two-stage: y = 4 y_coarse + y_fine, coefficient_sum 5); `total` is taken as given, as
+    the kernels take their Sum argument.  Integer arithmetic wraps at 32 bits as theirs does.
+    """
+    a = planes_values(low, high)
+    acc = a @ np.asarray(half_weights, np.int64).T
+    value = 2 * acc + coefficient_sum * np.asarray(total, np.int64)[:, None]
+    value = ((value + 2**31) % 2**32 - 2**31).astype(np.int32)
+    return rescale(value, weight_scale, token_scale)
+
+
+def dispatch_planes(a_q, a_scale, ids, relative, row_offsets):
+    """A8 rows -> K64-major planes at their routed slots (kernels/cuda/model/e8p_prefill.py:565-622).
+
+    Returns (Low, High, Sum, DS, SlotMap) with slot = RowOffsets[IDs] + RelativeSlot.
+    """
+    m, top_k = ids.shape
+    low, high, total = split_planes(a_q)
+    slot_map = (np.asarray(row_offsets)[ids] + relative).astype(np.int32)
+    slots = m * top_k
+    out_low = np.zeros((slots, low.shape[1]), np.uint32)
+    out_high = np.zeros_like(out_low)
+    out_sum = np.zeros(slots, np.int32)
+    ds = np.zeros((slots, 1), np.float16)
+    scale = np.asarray(a_scale, np.float16).reshape(m)
+    for row in range(m):
+        for rank in range(top_k):
+            slot = slot_map[row, rank]
+            out_low[slot], out_high[slot], out_sum[slot], ds[slot, 0] = low[row], high[row], total[row], scale[row]
+    return planes_group_major(out_low), planes_group_major(out_high), out_sum, ds, slot_map
 
 
 def moe_combine(expert_out, slot_map, prob, shared=None, shared_gate=None):

@@ -644,9 +644,15 @@ int make_a8(const Variant& v, orx_function* f) {
     const bool masked = v.boolean("masked", false, &bad);
     const bool fused = v.boolean("fused", false, &bad);
     f->capacity = (int)v.integer("M", 1 << 24, &bad);
+    // op30_activation_quantization.py:84: a block size of the reference's kernel; the block here follows the row
+    const int threads = (int)v.integer("threads", 256, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     if (f->K <= 0 || f->group <= 0 || f->group > f->K || f->capacity < 1) {
         set_error("activation_quantization: need K > 0 and 0 < group_size <= K");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (threads != 128 && threads != 256 && threads != 512) {
+        set_error("activation_quantization: threads is 128, 256 or 512");
         return ORX_ERR_BAD_VARIANT;
     }
     f->flags = (masked ? 1 : 0) | (fused ? 2 : 0);
@@ -696,6 +702,10 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     f->capacity = f->M = (int)v.integer("M", 0, &bad);
     f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
     const bool swiglu = v.boolean("swiglu", false, &bad);
+    // rotation_a8.py:373-383: reciprocal picks one of two roundings that give the same codes (the reciprocal one
+    // divides near ties), registers picks where the reference's kernel keeps the butterflies
+    v.boolean("reciprocal", true, &bad);
+    v.boolean("registers", false, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     // rotation_a8.py:425-427: K a positive multiple of 128; the row has to fit LDS as fp16
     if (f->M <= 0 || f->K <= 0 || f->K % 128 || f->K > 32768) {
@@ -958,10 +968,10 @@ int make_swiglu(const Variant& v, orx_function* f) {
 
 const Registration* quant_registrations(int* count) {
     static const Registration rows[] = {
-    {"activation_quantization", make_a8, "K, group_size=null, masked=false, fused=false, M=capacity",
+    {"activation_quantization", make_a8, "K, group_size=null, masked=false, fused=false, threads=256, M=capacity",
      "Mask,Q,S,X,rows"},
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
-    {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, dynamic_rows=false", "Q,S,Signs,X[,m]"},
+    {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, registers=false", "Q,S,Signs,X[,m]"},
     {"rotate_expert_a8", make_rotate_expert,
      "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, routing=none|shared|scatter, top_k=1, experts=1",
      "[D,]DS,IDs,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X[,m] (no routing: Q,S,Signs,Sum,X[,m])"},

@@ -246,13 +246,14 @@ struct Table {
     const Registration* rows;
     int count;
 };
-constexpr int kTables = 5;
+constexpr int kTables = 6;
 void tables(Table out[kTables]) {
     out[0].rows = quant_registrations(&out[0].count);
     out[1].rows = gemv_registrations(&out[1].count);
     out[2].rows = gemm_registrations(&out[2].count);
     out[3].rows = moe_registrations(&out[3].count);
     out[4].rows = probe_registrations(&out[4].count);
+    out[5].rows = plane_registrations(&out[5].count);
 }
 const Registration* find(const char* symbol) {
     Table t[kTables];

@@ -108,6 +108,7 @@ const Registration* gemv_registrations(int* count);
 const Registration* gemm_registrations(int* count);
 const Registration* moe_registrations(int* count);
 const Registration* probe_registrations(int* count);
+const Registration* plane_registrations(int* count);
 
 template <typename T>
 static inline T* pointer_arg(void** args, int index) {

@@ -89,6 +89,24 @@ ABI = {
         ["A", "D", "DS", "IDs", "RelativeSlot", "RowOffsets", "Scale", "SlotMap"],
     ("moe_combine", (("M", 64), ("H", 2048), ("dynamic_rows", True))):
         ["Expert", "Output", "Prob", "Shared", "SharedGate", "SlotMap", "m"],
+    # the nibble-plane family: crates/orinfer-models/src/flash_next/experts.rs:207-215 binds the exact kernel as
+    # AS, Book, Counts, High, Low, Offsets, Out, P, Sum, TC, TE, TR, WS and the split as A, High, Low, Sum
+    ("split_a8", (("rows", 64), ("K", 2048))): ["A", "High", "Low", "Sum"],
+    ("split_prefill_a8", (("rows", 64), ("K", 2048), ("dynamic_rows", True))): ["A", "High", "Low", "Sum", "m"],
+    ("split_routed_prefill_a8", (("rows", 640), ("K", 2048), ("experts", 128), ("block_m", 16))):
+        ["A", "Counts", "High", "Low", "Offsets", "Sum", "TC", "TE", "TR"],
+    ("dispatch_prefill_a8", (("M", 64),)):
+        ["A", "DS", "High", "IDs", "Low", "RelativeSlot", "RowOffsets", "Scale", "SlotMap", "Sum"],
+    ("pack_expert_tokens", (("M", 64), ("K", 2048), ("E", 128), ("top_k", 8))):
+        ["A", "High", "IDs", "Low", "RelativeSlot", "RowOffsets", "SlotMap", "Sources", "Sum", "m"],
+    ("expand_expert_slots", (("M", 64), ("K", 2048), ("top_k", 8))):
+        ["DS", "High", "Low", "Scale", "Sources", "SrcHigh", "SrcLow", "SrcSum", "Sum", "m"],
+    ("e8p_exact_grouped", (("rows", 640), ("E", 128), ("tiles", 200), ("N", 1024), ("K", 2048), ("block_m", 8), ("stages", 3),
+                           ("warp_private", True))):
+        ["AS", "Book", "Counts", "High", "Low", "Offsets", "Out", "P", "Sum", "TC", "TE", "TR", "WS"],
+    ("e8p_prefill_grouped", (("rows", 640), ("E", 128), ("tiles", 200), ("N", 1024), ("K", 2048), ("dynamic_rows", True),
+                             ("codec", "e8p_q4"), ("block_m", 32))):
+        ["AS", "Book", "Counts", "High", "Low", "Offsets", "Out", "P", "Sum", "TC", "TE", "TR", "WS", "m"],
 }
 
 
@@ -496,3 +514,81 @@ def test_routed_decode_symbols_take_the_reference_factories_keywords():
             lib.Kernel("integer_vq_grouped", **shape, **bad)
         with pytest.raises(lib.OrxError):
             lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, **bad)
+
+
+REFERENCE_KEYWORDS = {
+    # every keyword of the reference's factory with a value it accepts (signatures read from kernels/cuda/model/*.py and
+    # kernels/cuda/operators/op30_activation_quantization.py): a package record written for the reference resolves here
+    "activation_quantization": dict(K=512, group_size=128, masked=False, threads=512),
+    "rotate_activation_a8": dict(M=8, K=512, swiglu=False, reciprocal=False, dynamic_rows=True, registers=True),
+    "rotate_expert_a8": dict(M=8, K=512, swiglu=False, reciprocal=True, dynamic_rows=False, routing="scatter", top_k=2, experts=8,
+                             group_major=False),
+    "residual_norm_rotate_a8": dict(M=8, K=512, dynamic_rows=True, zero_centered=True),
+    "integer_experts": dict(M=8, N=256, K=512, E=8, top_k=2, codec="e8p_q4", block_m=16, block_n=64, block_k=128, stages=2,
+                            dynamic_rows=False, tail_m=0, minimum_blocks=1),
+    "expert_histogram": dict(M=8, E=8, top_k=2, dynamic_rows=True),
+    "expert_offsets": dict(E=8, block_m=16),
+    "expert_tiles": dict(M=8, E=8, top_k=2, block_m=16, dynamic_rows=True),
+    "expert_dispatch": dict(M=8, H=512, E=8, top_k=2, scale_group=512, dynamic_rows=True),
+    "router_topk_warp": dict(M=8, E=64, top_k=4, dynamic_rows=True, warps=4),
+    "router_topk": dict(M=8, E=64, top_k=4, renormalize=True, dynamic_rows=True),
+    "moe_combine": dict(M=8, H=512, slots=16, top_k=2, dynamic_rows=False),
+    "single_route_metadata": dict(E=64, top_k=8, capacity=16),
+    "route_metadata": dict(M=8, E=64, top_k=8, block_m=16, dynamic_rows=True),
+    "int8_swiglu": dict(M=8, N=256, K=512, block_n=64, dynamic_rows=True, algorithm="tensor_core", block_m=16),
+    "int8_projection": dict(M=64, N=256, K=512, output_dtype="float16", block_m=64, block_n=128, block_k=64, group_m=4,
+                            dynamic_rows=True, output_stride=260, tail_m=16, cache_scales=True),
+    "int8_small_projection": dict(M=4, N=256, K=512, output_dtype="float32", dynamic_rows=True, block_m=4, block_n=8,
+                                  output_stride=256),
+    "expert_partition_offsets": dict(experts=8, hot_m=64, cold_m=16, cold_rows=16),
+    "expert_partition_tiles": dict(M=8, experts=8, top_k=2, hot_m=64, cold_m=16, cold_rows=16, dynamic_rows=True),
+    "e8p_decode_grouped": dict(rows=64, E=8, tiles=16, N=256, K=512, block_n=32, split_k=2, parity_xor=True, packed_k=128),
+    "integer_vq": dict(E=3, M=17, N=65, K=256, kind="e8p", shared_table=True, block_n=128, patched=True, shortbook=True,
+                       num_stages=2, block_m=16, byte_permute=True, selectorbook=True, packed_k=64),
+    "integer_vq_grouped": dict(rows=64, E=8, tiles=16, N=256, K=512, kind="e8p", shared_table=False, block_n=128, patched=True,
+                               shortbook=True, num_stages=1, block_m=8, byte_permute=True, selectorbook=True, warp_decode=True,
+                               split_k=2, parity_xor=True, group_n=2, packed_k=64, dynamic_rows=True),
+    "integer_e8p_gemv": dict(E=8, routes=2, N=256, K=512, shared_input=True, block_n=8),
+    "rotate_activation": dict(M=8, K=512, swiglu=True),
+    "split_a8": dict(rows=8, K=512, dynamic_rows=True),
+    "split_prefill_a8": dict(rows=8, K=512, dynamic_rows=False),
+    "split_routed_prefill_a8": dict(rows=64, K=512, experts=8, block_m=16, dynamic_rows=True),
+    "dispatch_prefill_a8": dict(M=8, K=512, E=8, top_k=2, dynamic_rows=True),
+    "pack_expert_tokens": dict(M=8, K=512, E=8, top_k=2),
+    "expand_expert_slots": dict(M=8, K=512, top_k=2),
+    "e8p_exact_grouped": dict(rows=64, E=8, tiles=16, N=256, K=512, block_m=16, stages=4, dynamic_rows=True, warp_private=False),
+    "e8p_prefill_grouped": dict(rows=64, E=8, tiles=16, N=256, K=512, dynamic_rows=False, sparse_rows=True, row_major=False,
+                                codec="e8p_q2", minimum_blocks=2, block_m=32, block_n=64, specialize_tails=True,
+                                merge_routed_tiles=True),
+}
+
+
+@pytest.mark.parametrize("symbol", list(REFERENCE_KEYWORDS))
+def test_every_keyword_of_the_reference_factory_resolves(symbol):
+    kernel = lib.Kernel(symbol, **REFERENCE_KEYWORDS[symbol])
+    assert kernel.arg_names
+    with pytest.raises(lib.OrxError, match="unknown variant key"):
+        lib.Kernel(symbol, **REFERENCE_KEYWORDS[symbol], no_such_option=1)
+
+
+def test_plane_kernels_refuse_what_the_reference_refuses():
+    # e8p_exact.py:57-70, e8p_prefill.py:160-183
+    shape = dict(rows=64, E=8, tiles=16, N=256, K=512)
+    for bad in (dict(block_m=32), dict(stages=5), dict(stages=1), dict(K=500), dict(K=131200)):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("e8p_exact_grouped", **{**shape, **bad})
+    for bad in (dict(block_m=8), dict(block_n=32), dict(codec="w8"), dict(codec="e8p_q4", block_n=64), dict(minimum_blocks=17),
+                dict(specialize_tails=True, block_m=16), dict(specialize_tails=True, block_m=32, codec="e8p_q4"),
+                dict(merge_routed_tiles=True, block_m=32)):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("e8p_prefill_grouped", **{**shape, **bad})
+    for bad in (dict(rows=0, K=512), dict(rows=8, K=192)):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("split_a8", **bad)
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("split_routed_prefill_a8", rows=64, K=512, experts=8, block_m=6)
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("dispatch_prefill_a8", M=8, K=512, E=4, top_k=5)
+    # the exact kernel launches no more tiles than the live rows can fill (e8p_exact.py:76)
+    dynamic = lib.Kernel("e8p_exact_grouped", **shape, block_m=8, dynamic_rows=True)
+    assert dynamic.geometry(8)[0][1] == 1 + 8 and dynamic.geometry(64)[0][1] == 16

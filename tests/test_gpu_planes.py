@@ -1,0 +1,289 @@
+"""GPU parity for the nibble-plane hand-over (A8 as two planes of 4-bit words) and the grouped GEMMs that take it.
+
+The cases follow the reference's own test of these kernels (tests/cuda/operators/e8p_exact.py): random bases from
+{+-2, +-6, +-10}, extreme codes planted in every row, tile lists with tails, the plane words checked through
+low + 16 high == permuted codes, outputs equal to the int8 grouped kernel's on the same code bank.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import reference as orc
+
+from . import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+I32 = dict(dtype=torch.int32, device=gu.DEV)
+
+SHAPES = [  # (block_m, counts, N, K): tests/cuda/operators/e8p_exact.py:35-45
+    (8, [1, 0], 160, 640),
+    (8, [7, 8], 160, 640),
+    (16, [17, 16], 160, 640),
+    (32, [33, 32], 160, 640),
+    (16, [3, 0], 129, 128),
+    (16, [5, 9], 257, 2560),
+    (8, [9, 17], 1280, 2560),
+    (16, [17, 33], 2560, 640),
+]
+
+
+def planted_rows(rng, rows, k):
+    a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    a[:, :4] = np.array([-128, -1, 0, 127], np.int8)
+    return a
+
+
+def tile_list(counts, bm):
+    offsets, tile_offsets, total = orc.expert_offsets(np.asarray(counts, np.int32), bm)
+    cap = sum(counts) // bm + len(counts) + 1
+    te, tr = orc.expert_tiles(np.asarray(counts, np.int32), tile_offsets, bm, cap)
+    return offsets, te, tr, total, cap
+
+
+def empty_planes(rows, k, group_major):
+    shape = (k // 64, rows, 8) if group_major else (rows, k // 8)
+    return torch.full(shape, -1, **I32), torch.full(shape, -1, **I32)
+
+
+@pytest.mark.parametrize("rows,k", [(1, 128), (5, 640), (67, 2560), (130, 5120)])
+@pytest.mark.parametrize("group_major", [False, True])
+def test_split_a8_words_and_sums(rows, k, group_major):
+    rng = np.random.default_rng(orc.SEED + rows)
+    a = planted_rows(rng, rows, k)
+    low, high = empty_planes(rows + 1, k, group_major) if not group_major else empty_planes(rows, k, True)
+    total = torch.full((rows + 1,), -7, **I32)
+    symbol = "split_prefill_a8" if group_major else "split_a8"
+    gu.kernel(symbol, rows=rows, K=k)(A=gu.dev(a), High=high, Low=low, Sum=total)
+    want_low, want_high, want_sum = orc.split_planes(a)
+    got_low, got_high = gu.host(low, np.uint32), gu.host(high, np.uint32)
+    if group_major:
+        got_low, got_high = orc.planes_row_major(got_low), orc.planes_row_major(got_high)
+    else:
+        assert (got_low[rows] == 0xFFFFFFFF).all() and (got_high[rows] == 0xFFFFFFFF).all()
+        got_low, got_high = got_low[:rows], got_high[:rows]
+    np.testing.assert_array_equal(got_low, want_low)
+    np.testing.assert_array_equal(got_high, want_high)
+    np.testing.assert_array_equal(gu.host(total)[:rows], want_sum)
+    assert gu.host(total)[rows] == -7
+    # the reference's own statement of the planes (e8p_exact.py:196-206)
+    shifts = np.arange(0, 32, 4, dtype=np.uint64)
+    lo = ((got_low.astype(np.uint64)[..., None] >> shifts) & 15).astype(np.int64).reshape(rows, k)
+    hi = ((got_high.astype(np.uint64)[..., None] >> shifts) & 15).astype(np.int64).reshape(rows, k)
+    hi = np.where(hi >= 8, hi - 16, hi)
+    permuted = a.reshape(rows, k // 8, 8)[:, :, [0, 2, 1, 3, 4, 6, 5, 7]].reshape(rows, k)
+    np.testing.assert_array_equal(lo + 16 * hi, permuted.astype(np.int64))
+
+
+def test_split_a8_dynamic_rows_strides_follow_the_live_rows():
+    rng = np.random.default_rng(orc.SEED)
+    capacity, m, k = 40, 13, 256
+    a = planted_rows(rng, capacity, k)
+    low, high = empty_planes(capacity, k, True)
+    total = torch.full((capacity,), -7, **I32)
+    gu.kernel("split_prefill_a8", rows=capacity, K=k, dynamic_rows=True)(A=gu.dev(a), High=high, Low=low, Sum=total, m=m)
+    want_low, want_high, want_sum = orc.split_planes(a[:m])
+    words = k // 64 * m * 8
+    np.testing.assert_array_equal(gu.host(low, np.uint32).reshape(-1)[:words], orc.planes_group_major(want_low).reshape(-1))
+    np.testing.assert_array_equal(gu.host(high, np.uint32).reshape(-1)[:words], orc.planes_group_major(want_high).reshape(-1))
+    assert (gu.host(low, np.uint32).reshape(-1)[words:] == 0xFFFFFFFF).all()
+    np.testing.assert_array_equal(gu.host(total)[:m], want_sum)
+    assert (gu.host(total)[m:] == -7).all()
+
+
+def test_split_routed_prefill_a8_touches_the_rows_of_the_tiles_only():
+    rng = np.random.default_rng(orc.SEED + 1)
+    counts, bm, k = [5, 0, 9, 3], 8, 384
+    rows = sum(counts) + 2  # two rows that belong to no expert
+    a = planted_rows(rng, rows, k)
+    offsets, tile_offsets, total = orc.expert_offsets(np.asarray(counts, np.int32), bm)
+    cap = (rows + bm - 1) // bm + min(len(counts), rows)
+    te, tr = orc.expert_tiles(np.asarray(counts, np.int32), tile_offsets, bm, cap)
+    low, high = empty_planes(rows, k, True)
+    sums = torch.full((rows,), -7, **I32)
+    gu.kernel("split_routed_prefill_a8", rows=rows, K=k, experts=len(counts), block_m=bm)(
+        A=gu.dev(a), Counts=gu.dev(np.asarray(counts, np.int32)), High=high, Low=low, Offsets=gu.dev(offsets), Sum=sums,
+        TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr))
+    want_low, want_high, want_sum = orc.split_planes(a)
+    live = sum(counts)
+    got_low, got_high = orc.planes_row_major(gu.host(low, np.uint32)), orc.planes_row_major(gu.host(high, np.uint32))
+    np.testing.assert_array_equal(got_low[:live], want_low[:live])
+    np.testing.assert_array_equal(got_high[:live], want_high[:live])
+    np.testing.assert_array_equal(gu.host(sums)[:live], want_sum[:live])
+    assert (got_low[live:] == 0xFFFFFFFF).all() and (gu.host(sums)[live:] == -7).all()
+
+
+def routed(rng, m, e, top_k):
+    ids = np.stack([rng.choice(e, top_k, replace=False) for _ in range(m)]).astype(np.int32)
+    counts, relative = orc.expert_histogram(ids, e)
+    offsets, _, _ = orc.expert_offsets(counts, 16)
+    return ids, relative, offsets
+
+
+@pytest.mark.parametrize("m,k,e,top_k", [(1, 128, 4, 1), (9, 640, 16, 4), (33, 2560, 64, 10)])
+def test_dispatch_prefill_a8(m, k, e, top_k):
+    rng = np.random.default_rng(orc.SEED + m)
+    a = planted_rows(rng, m, k)
+    scale = rng.uniform(0.01, 0.03, (m, 1)).astype(np.float16)
+    ids, relative, offsets = routed(rng, m, e, top_k)
+    slots = m * top_k
+    low, high = empty_planes(slots, k, True)
+    sums, slot_map = torch.full((slots,), -7, **I32), torch.full((m, top_k), -7, **I32)
+    ds = torch.zeros((slots, 1), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("dispatch_prefill_a8", M=m, K=k, E=e, top_k=top_k)(
+        A=gu.dev(a), DS=ds, High=high, IDs=gu.dev(ids), Low=low, RelativeSlot=gu.dev(relative), RowOffsets=gu.dev(offsets),
+        Scale=gu.dev(scale), SlotMap=slot_map, Sum=sums)
+    want = orc.dispatch_planes(a, scale, ids, relative, offsets)
+    for got, expected in zip((gu.host(low, np.uint32), gu.host(high, np.uint32), gu.host(sums), gu.host(ds), gu.host(slot_map)), want):
+        np.testing.assert_array_equal(got, expected)
+
+
+def test_pack_expert_tokens_then_expand_expert_slots_equals_dispatch():
+    rng = np.random.default_rng(orc.SEED + 2)
+    capacity, m, k, e, top_k = 24, 19, 640, 16, 4
+    a = planted_rows(rng, capacity, k)
+    scale = rng.uniform(0.01, 0.03, (capacity, 1)).astype(np.float16)
+    ids, relative, offsets = routed(rng, m, e, top_k)
+    slots = m * top_k
+    src_low, src_high = empty_planes(m, k, True)
+    src_sum, sources = torch.full((m,), -7, **I32), torch.full((slots,), -7, **I32)
+    slot_map = torch.full((m, top_k), -7, **I32)
+    gu.kernel("pack_expert_tokens", M=capacity, K=k, E=e, top_k=top_k)(
+        A=gu.dev(a), High=src_high, IDs=gu.dev(ids), Low=src_low, RelativeSlot=gu.dev(relative), RowOffsets=gu.dev(offsets),
+        SlotMap=slot_map, Sources=sources, Sum=src_sum, m=m)
+    want_low, want_high, want_sum = orc.split_planes(a[:m])
+    np.testing.assert_array_equal(gu.host(src_low, np.uint32), orc.planes_group_major(want_low))
+    np.testing.assert_array_equal(gu.host(src_high, np.uint32), orc.planes_group_major(want_high))
+    np.testing.assert_array_equal(gu.host(src_sum), want_sum)
+    want = orc.dispatch_planes(a[:m], scale[:m], ids, relative, offsets)
+    np.testing.assert_array_equal(gu.host(slot_map), want[4])
+    inverse = np.empty(slots, np.int32)
+    inverse[want[4]] = np.arange(m, dtype=np.int32)[:, None]
+    np.testing.assert_array_equal(gu.host(sources), inverse)
+    low, high = empty_planes(slots, k, True)
+    sums = torch.full((slots,), -7, **I32)
+    ds = torch.zeros((slots, 1), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("expand_expert_slots", M=capacity, K=k, top_k=top_k)(
+        DS=ds, High=high, Low=low, Scale=gu.dev(scale), Sources=sources, SrcHigh=src_high, SrcLow=src_low, SrcSum=src_sum,
+        Sum=sums, m=m)
+    for got, expected in zip((gu.host(low, np.uint32), gu.host(high, np.uint32), gu.host(sums), gu.host(ds)), want[:4]):
+        np.testing.assert_array_equal(got, expected)
+
+
+def grouped_case(rng, counts, n, k, basis):
+    e, rows = len(counts), sum(counts)
+    a = planted_rows(rng, rows, k)
+    raw = rng.integers(0, 65536, (e, k // 128, n, 16), dtype=np.uint16)  # K128 blocks, as the reference's bank
+    codes = np.ascontiguousarray(raw.transpose(0, 2, 1, 3)).reshape(e, n, k // 8)
+    ws = (rng.random((e, n)) / 16).astype(np.float16)
+    scale = (rng.random(rows) / 16).astype(np.float16)
+    weights = np.stack([orc.q2_integers(c, basis) for c in codes])
+    return a, raw, codes, ws, scale, weights
+
+
+@pytest.mark.parametrize("bm,counts,n,k", SHAPES)
+def test_exact_and_prefill_grouped_match_the_int8_kernel(bm, counts, n, k):
+    rng = np.random.default_rng(orc.SEED + bm + n)
+    basis = rng.choice(np.array([-10, -6, -2, 2, 6, 10], np.int8), (256, 8))
+    selector = orc.selector_table(basis)
+    nibble = orc.nibble_table(selector)
+    e, rows = len(counts), sum(counts)
+    a, raw, codes, ws, scale, weights = grouped_case(rng, counts, n, k, basis)
+    offsets, te, tr, total, cap = tile_list(counts, bm)
+    counts_np = np.asarray(counts, np.int32)
+    want = orc.grouped_project(a, scale[:, None], weights, ws, counts_np, offsets)
+    routing = dict(Counts=gu.dev(counts_np), Offsets=gu.dev(offsets))
+    # the int8 kernel on the same bank in K64 blocks
+    ref = torch.full((rows, n), float("nan"), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, kind="e8p", shared_table=True, block_m=bm,
+              block_n=128, shortbook=True, selectorbook=True, packed_k=64, basis="any")(
+        A=gu.dev(a), AS=gu.dev(scale), Book=gu.dev(selector[None]), C=ref, P=gu.dev(orc.q2_repack_k64(raw)), Patch=None,
+        TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws), **routing)
+    np.testing.assert_array_equal(gu.host(ref), want)
+    a_dev = gu.dev(a)
+    forms = []
+    if bm <= 16:
+        forms += [("e8p_exact_grouped", dict(block_m=bm, stages=s), False) for s in (2, 3, 4) if k // 64 >= s - 1]
+    if bm >= 16:
+        forms += [("e8p_prefill_grouped", dict(block_m=bm), True), ("e8p_prefill_grouped", dict(block_m=bm, row_major=True), False)]
+    for symbol, options, group_major in forms:
+        low, high = empty_planes(rows, k, group_major)
+        sums = torch.full((rows,), -7, **I32)
+        gu.kernel("split_prefill_a8" if group_major else "split_a8", rows=rows, K=k)(A=a_dev, High=high, Low=low, Sum=sums)
+        out = torch.full((rows, n), float("nan"), dtype=torch.float16, device=gu.DEV)
+        kern = gu.kernel(symbol, rows=rows, E=e, tiles=cap, N=n, K=k, **options)
+        args = dict(AS=gu.dev(scale), Book=gu.dev(nibble[None]), High=high, Low=low, Out=out, P=gu.dev(orc.q2_repack_k64(raw)),
+                    Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws), **routing)
+        kern(**args)
+        assert torch.equal(out, ref), (symbol, options)
+        # Sum is an input like any other: the kernels add what they are given (e8p_core.py:186)
+        planted = rng.integers(-1000, 1000, rows).astype(np.int32)
+        sums.copy_(gu.dev(planted))
+        kern(**args)
+        half = np.stack([orc.nibble_decode(c, nibble).reshape(n, k) for c in codes])
+        expected = np.zeros((rows, n), np.float16)
+        got_low, got_high = gu.host(low, np.uint32), gu.host(high, np.uint32)
+        if group_major:
+            got_low, got_high = orc.planes_row_major(got_low), orc.planes_row_major(got_high)
+        for x, c in enumerate(counts):
+            r = slice(int(offsets[x]), int(offsets[x]) + c)
+            expected[r] = orc.plane_project(got_low[r], got_high[r], planted[r], half[x], ws[x], scale[r])
+        np.testing.assert_array_equal(gu.host(out), expected)
+        # zero activations with their sums give zero (the reference's graph replay on a.zero_())
+        low.zero_(), high.zero_(), sums.zero_()
+        kern(**args)
+        assert bool((out == 0).all())
+
+
+@pytest.mark.parametrize("bm,counts,n,k", [(16, [17, 16], 160, 640), (32, [33, 5, 0, 70], 257, 1280), (16, [3, 0], 129, 128)])
+def test_prefill_grouped_two_stage_codes(bm, counts, n, k):
+    # codec e8p_q4: K-major blocks of 128 u32 codes, Book = selector words (e8p_prefill.py:468-469, :492-493)
+    rng = np.random.default_rng(orc.SEED + bm + k)
+    basis = orc.basis()
+    e, rows = len(counts), sum(counts)
+    a = planted_rows(rng, rows, k)
+    packed = rng.integers(0, 2**32, (e, n, k // 8), dtype=np.uint32)
+    weights = np.stack([orc.q4_integers(p, basis) for p in packed])
+    stored = np.stack([orc.q4_pack_k(p, 128) for p in packed])
+    ws = (rng.random((e, n)) / 64).astype(np.float16)
+    scale = (rng.random(rows) / 16).astype(np.float16)
+    offsets, te, tr, total, cap = tile_list(counts, bm)
+    counts_np = np.asarray(counts, np.int32)
+    want = orc.grouped_project(a, scale[:, None], weights, ws, counts_np, offsets)
+    low, high = empty_planes(rows, k, True)
+    sums = torch.full((rows,), -7, **I32)
+    gu.kernel("split_prefill_a8", rows=rows, K=k)(A=gu.dev(a), High=high, Low=low, Sum=sums)
+    out = torch.full((rows + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("e8p_prefill_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, codec="e8p_q4", block_m=bm)(
+        AS=gu.dev(scale), Book=gu.book(), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets), Out=out,
+        P=gu.dev(stored), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws))
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows] == 91).all()
+
+
+def test_prefill_grouped_merges_adjacent_tiles_of_a_shared_list_and_takes_live_rows():
+    # merge_routed_tiles: the list steps by 16 rows, a workgroup takes 32 (e8p_prefill.py:188, :497-498);
+    # dynamic rows: the plane stride is the live row count (e8p_prefill.py:186-187)
+    rng = np.random.default_rng(orc.SEED + 9)
+    basis = orc.basis()
+    nibble = orc.nibble_table(orc.selector_table(basis))
+    counts, n, k, capacity = [40, 0, 16, 7], 192, 512, 80
+    e, rows = len(counts), sum(counts)
+    a, raw, codes, ws, scale, weights = grouped_case(rng, counts, n, k, basis)
+    counts_np = np.asarray(counts, np.int32)
+    offsets, tile_offsets, total = orc.expert_offsets(counts_np, 16)
+    cap = capacity // 16 + e + 1
+    te, tr = orc.expert_tiles(counts_np, tile_offsets, 16, cap)
+    want = orc.grouped_project(a, scale[:, None], weights, ws, counts_np, offsets)
+    low, high = empty_planes(capacity, k, True)
+    sums = torch.full((capacity,), -7, **I32)
+    gu.kernel("split_prefill_a8", rows=capacity, K=k, dynamic_rows=True)(A=gu.dev(a), High=high, Low=low, Sum=sums, m=rows)
+    out = torch.full((capacity, n), 91.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("e8p_prefill_grouped", rows=capacity, E=e, tiles=cap, N=n, K=k, block_m=32, specialize_tails=True,
+              merge_routed_tiles=True, dynamic_rows=True, sparse_rows=True, minimum_blocks=2)(
+        AS=gu.dev(scale), Book=gu.dev(nibble[None]), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets),
+        Out=out, P=gu.dev(orc.q2_repack_k64(raw)), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws),
+        m=rows)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows:] == 91).all()

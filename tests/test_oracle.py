@@ -737,3 +737,93 @@ def test_decode_with_zero_coordinates_and_the_selector_table_for_them():
     some = rng.integers(0, 65536, 300)
     np.testing.assert_array_equal(orc.e8p_decode(some.astype(np.uint16), general),
                                   [orc.e8p_decode_scalar(c, general) for c in some])
+
+
+def test_plane_words_follow_the_reference_masks_and_its_test():
+    """split_planes against the mask-and-shift form of kernels/cuda/model/e8p_core.py:63-78 and against the statement of
+    tests/cuda/operators/e8p_exact.py:196-206 (low + 16 high == codes permuted by [0, 2, 1, 3, 4, 6, 5, 7])."""
+    rng = np.random.default_rng(orc.SEED)
+    a = rng.integers(-128, 128, (7, 256), dtype=np.int8)
+    a[:, :4] = np.array([-128, -1, 0, 127], np.int8)
+    low, high, total = orc.split_planes(a)
+    x = a.view("<u4").reshape(7, 32, 2)[:, :, 0]
+    y = a.view("<u4").reshape(7, 32, 2)[:, :, 1]
+    np.testing.assert_array_equal(low, (x & 0x0F0F) | ((x >> 12) & 0xF0F0) | ((y << 16) & 0x0F0F0000) | ((y << 4) & 0xF0F00000))
+    np.testing.assert_array_equal(high, ((x >> 4) & 0x0F0F) | ((x >> 16) & 0xF0F0) | ((y << 12) & 0x0F0F0000) | (y & 0xF0F00000))
+    # a word by hand: codes -128, -1, 0, 127, 5, -3, 17, -16 are bytes 80 FF 00 7F 05 FD 11 F0; low nibbles
+    # 0 F 0 F 5 D 1 0 and high nibbles 8 F 0 7 0 F 1 F land at positions [0, 2, 1, 3, 4, 6, 5, 7]
+    hand = np.array([[-128, -1, 0, 127, 5, -3, 17, -16] * 16], np.int8)
+    hl, hh, ht = orc.split_planes(hand)
+    assert hl[0, 0] == 0x0D15FF00 and hh[0, 0] == 0xFF107F08 and ht[0] == 16
+    shifts = np.arange(0, 32, 4, dtype=np.uint64)
+    lo = ((low.astype(np.uint64)[..., None] >> shifts) & 15).astype(np.int64).reshape(7, 256)
+    hi = ((high.astype(np.uint64)[..., None] >> shifts) & 15).astype(np.int64).reshape(7, 256)
+    hi = np.where(hi >= 8, hi - 16, hi)
+    np.testing.assert_array_equal(lo + 16 * hi, a.reshape(7, 32, 8)[:, :, [0, 2, 1, 3, 4, 6, 5, 7]].reshape(7, 256))
+    np.testing.assert_array_equal(orc.planes_values(low, high), a)
+    np.testing.assert_array_equal(total, a.astype(np.int64).sum(axis=1))
+    grouped = orc.planes_group_major(low)
+    assert grouped.shape == (4, 7, 8) and grouped[2, 5, 3] == low[5, 19]
+    np.testing.assert_array_equal(orc.planes_row_major(grouped), low)
+
+
+def test_nibble_table_and_decode_are_the_selector_decode_halved(table):
+    """2 y + 1 == e8p_decode over all 65 536 codes, on the real basis and on a random nonzero one
+    (python/orinfer_build/quantization/vq.py:105-118, kernels/cuda/model/e8p_core.py:7-10); the table itself against
+    the literal palette of vq.py:115 for one row; zero coordinates are refused."""
+    codes = np.arange(65536, dtype=np.uint16)
+    rng = np.random.default_rng(orc.SEED)
+    for basis in (table, rng.choice(np.array([-10, -6, -2, 2, 6, 10], np.int8), (256, 8))):
+        nibbles = orc.nibble_table(orc.selector_table(basis))
+        assert nibbles.shape == (256, 1) and nibbles.dtype == np.uint32
+        np.testing.assert_array_equal(2 * orc.nibble_decode(codes, nibbles) + 1, orc.e8p_decode(codes, basis))
+    row = np.array([[2, -6, 10, -2, 6, -10, 2, 6]] * 256, np.int8)
+    # halves 1 -3 5 -1 3 -5 1 3 in the order [0, 2, 1, 3, 4, 6, 5, 7]: 1, 5, -3, -1, 3, 1, -5, 3
+    assert orc.nibble_table(orc.selector_table(row))[0, 0] == 0x3B13FD51
+    zeros = table.copy()
+    zeros[3, 2] = 0
+    with pytest.raises(ValueError):
+        orc.nibble_table(orc.selector_table(zeros))
+
+
+def test_plane_project_is_project_when_sum_is_the_row_sum_and_adds_what_it_is_given(table):
+    """2 (y . a) + Sum == w . a for w = 2 y + 1 (kernels/cuda/model/e8p_exact.py:3-4); two-stage codes:
+    y = 4 y_coarse + y_fine and 5 Sum (e8p_core.py:154-170); a planted Sum moves every integer by its difference."""
+    rng = np.random.default_rng(orc.SEED + 4)
+    n, k, rows = 9, 256, 5
+    a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    low, high, total = orc.split_planes(a)
+    ws = np.full(n, 2.0 ** -7, np.float16)
+    scale = np.full(rows, 2.0 ** -6, np.float16)
+    codes = rng.integers(0, 65536, (n, k // 8), dtype=np.uint16)
+    nibbles = orc.nibble_table(orc.selector_table(table))
+    y = orc.nibble_decode(codes, nibbles).reshape(n, k)
+    np.testing.assert_array_equal(orc.plane_project(low, high, total, y, ws, scale), orc.project(a, scale, orc.q2_integers(codes, table), ws))
+    packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    y4 = 4 * orc.nibble_decode((packed & 0xFFFF).astype(np.uint16), nibbles) + orc.nibble_decode((packed >> 16).astype(np.uint16), nibbles)
+    np.testing.assert_array_equal(orc.plane_project(low, high, total, y4.reshape(n, k), ws, scale, 5),
+                                  orc.project(a, scale, orc.q4_integers(packed, table), ws))
+    moved = orc.plane_project(low, high, total + 64, y, ws, scale).astype(np.float64)
+    plain = orc.project(a, scale, orc.q2_integers(codes, table), ws).astype(np.float64)
+    exact = np.abs(a.astype(np.int64) @ orc.q2_integers(codes, table).astype(np.int64).T) < 1900
+    np.testing.assert_array_equal((moved - plain)[exact] * 8192, 64)
+
+
+def test_dispatch_planes_copies_every_token_to_its_slots():
+    rng = np.random.default_rng(orc.SEED + 6)
+    m, k, e, top_k = 6, 128, 5, 2
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    scale = rng.uniform(0.01, 0.03, (m, 1)).astype(np.float16)
+    ids = np.stack([rng.choice(e, top_k, replace=False) for _ in range(m)]).astype(np.int32)
+    counts, relative = orc.expert_histogram(ids, e)
+    offsets, _, _ = orc.expert_offsets(counts, 16)
+    low, high, total, ds, slot_map = orc.dispatch_planes(a, scale, ids, relative, offsets)
+    assert low.shape == (k // 64, m * top_k, 8) and sorted(slot_map.reshape(-1)) == list(range(m * top_k))
+    wl, wh, wt = orc.split_planes(a)
+    for row in range(m):
+        for rank in range(top_k):
+            slot = slot_map[row, rank]
+            np.testing.assert_array_equal(orc.planes_row_major(low)[slot], wl[row])
+            np.testing.assert_array_equal(orc.planes_row_major(high)[slot], wh[row])
+            assert total[slot] == wt[row] and ds[slot, 0] == scale[row, 0]
+            assert offsets[ids[row, rank]] <= slot < offsets[ids[row, rank]] + counts[ids[row, rank]]
