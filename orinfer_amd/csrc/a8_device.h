@@ -60,4 +60,20 @@ __device__ __forceinline__ float swiglu_value(__half gate, __half up) {
     return __half2float(__float2half_rn((g * sigmoid) * u));
 }
 
+// ---- nibble planes ------------------------------------------------------------------------------
+// The reference's INT4 expert kernels take A8 codes as two planes of u32 words: nibble i of a word holds the low
+// (unsigned) or high (signed) nibble of code {0,2,1,3,4,6,5,7}[i] of its group of eight
+// (kernels/cuda/model/e8p_core.py:63-78, rotation_a8.py:489-491).  x = codes 0..3, y = codes 4..7, one byte each.
+__device__ __forceinline__ uint32_t low_word_first(uint32_t x) { return (x & 0x00000F0Fu) | ((x >> 12) & 0x0000F0F0u); }
+__device__ __forceinline__ uint32_t low_word_second(uint32_t y) { return ((y << 16) & 0x0F0F0000u) | ((y << 4) & 0xF0F00000u); }
+__device__ __forceinline__ uint32_t high_word_first(uint32_t x) { return ((x >> 4) & 0x00000F0Fu) | ((x >> 16) & 0x0000F0F0u); }
+__device__ __forceinline__ uint32_t high_word_second(uint32_t y) { return ((y << 12) & 0x0F0F0000u) | (y & 0xF0F00000u); }
+__device__ __forceinline__ uint32_t low_word(uint32_t x, uint32_t y) { return low_word_first(x) | low_word_second(y); }
+__device__ __forceinline__ uint32_t high_word(uint32_t x, uint32_t y) { return high_word_first(x) | high_word_second(y); }
+
+// Word j of plane row `row`: row-major (rows, K/8), or K64-major (K/64, rows, 8) (kernels/cuda/model/e8p_prefill.py:79-80)
+__device__ __forceinline__ int64_t plane_index(int group_major, int plane_rows, int words, int64_t row, int j) {
+    return group_major ? ((int64_t)(j >> 3) * plane_rows + row) * 8 + (j & 7) : row * words + j;
+}
+
 }  // namespace orx

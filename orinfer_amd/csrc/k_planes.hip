@@ -16,6 +16,7 @@
 
 #include <algorithm>
 
+#include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
 
@@ -30,14 +31,6 @@ constexpr int kPlaneWaves = kPlaneThreads / 64;
 constexpr int kMaxChoices = 64;  // routes of one token: one lane each
 
 // ---- packing ------------------------------------------------------------------------------------
-
-// x = codes 0..3, y = codes 4..7 of one group of eight, one byte each (e8p_core.py:63-78)
-__device__ __forceinline__ uint32_t low_word(uint32_t x, uint32_t y) {
-    return (x & 0x00000F0Fu) | ((x >> 12) & 0x0000F0F0u) | ((y << 16) & 0x0F0F0000u) | ((y << 4) & 0xF0F00000u);
-}
-__device__ __forceinline__ uint32_t high_word(uint32_t x, uint32_t y) {
-    return ((x >> 4) & 0x00000F0Fu) | ((x >> 16) & 0x0000F0F0u) | ((y << 12) & 0x0F0F0000u) | (y & 0xF0F00000u);
-}
 
 enum PlaneMode { kSplitRows = 0, kSplitTiles = 1, kDispatchSlots = 2, kPackTokens = 3 };
 
@@ -57,10 +50,6 @@ struct PlaneParams {
     int *slot_map, *sources;
     int top_k;
 };
-
-__device__ __forceinline__ int64_t plane_index(int group_major, int plane_rows, int words, int64_t row, int j) {
-    return group_major ? ((int64_t)(j >> 3) * plane_rows + row) * 8 + (j & 7) : row * words + j;
-}
 
 // One wave packs row `src` of A into the plane rows `dst` (lane r holds the r-th of `copies` destinations,
 // or every lane the one destination when copies == 0) and returns the row's sum in every lane.

@@ -17,6 +17,8 @@
 // * row scale, * sign), one fp16 cast; ids outside the vocabulary give zero rows.
 #include <hip/hip_fp16.h>
 
+#include <cstring>
+
 #include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
@@ -315,12 +317,13 @@ __global__ __launch_bounds__(THREADS) void rotate_a8_kernel(const __half* __rest
 
 // rotate_expert_a8 (kernels/cuda/model/rotation_a8.py:386-422, body :452-531, entry points :558-604):
 // the rotation and the A8 rule of rotate_a8_kernel with the routed hand-over to the expert GEMMs in the
-// same launch.  The reference's expert GEMMs multiply 4-bit planes, so its kernel leaves the codes as
-// two nibble planes plus their sum; the expert GEMMs here multiply int8 rows, so the codes stay whole:
-//   routing "scatter": D[slot] = codes and DS[slot] = scale for each of the row's top_k slots
+// same launch.  The reference's kernel leaves the codes as two nibble planes plus their sum for its INT4
+// expert GEMMs (Low, High: u32 words, row-major, or K64-major under group_major); the int8 expert GEMMs here
+// take whole rows, so the kernel can write those instead (D):
+//   routing "scatter": Low/High[slot] (and D[slot]) = codes, DS[slot] = scale for each of the row's top_k slots
 //                      (slot = RowOffsets[IDs[row, c]] + RelativeSlot[row, c]), SlotMap[row, c] = slot;
-//   routing "shared":  Q[row] = codes, and only DS[slot] and SlotMap are written per assignment;
-//   no routing:        Q[row], S[row] (and Sum[row]) alone.
+//   routing "shared":  Low/High[row] and Q[row] = codes, and only DS[slot] and SlotMap are written per assignment;
+//   no routing:        Low/High[row], Q[row], S[row] (and Sum[row]) alone.
 // S[row] is always written; Q (scatter) and Sum may be null.  Sum is the integer sum of a row's codes
 // (per slot under scatter, per row otherwise), the term the reference's unsigned-nibble product needs.
 constexpr int kRouteScatter = 1, kRouteShared = 2;
@@ -329,8 +332,8 @@ template <bool SWIGLU, int THREADS>
 __global__ __launch_bounds__(THREADS) void rotate_expert_kernel(
     const __half* __restrict__ x, const int8_t* __restrict__ signs, int8_t* __restrict__ q, __half* __restrict__ s,
     int8_t* __restrict__ d, __half* __restrict__ ds, const int* __restrict__ ids, const int* __restrict__ relative,
-    const int* __restrict__ row_offsets, int* __restrict__ slot_map, int* __restrict__ sum, int k, int top_k,
-    int routing) {
+    const int* __restrict__ row_offsets, int* __restrict__ slot_map, int* __restrict__ sum, uint32_t* __restrict__ low,
+    uint32_t* __restrict__ high, int plane_rows, int group_major, int k, int top_k, int routing) {
     extern __shared__ __align__(16) __half rotated[];  // k halves
     __shared__ float scratch[THREADS / 64];
     __shared__ int slot_of[kMaxRouteChoices];
@@ -356,8 +359,26 @@ __global__ __launch_bounds__(THREADS) void rotate_expert_kernel(
         const uint32_t word = quantise4(values, scale, inverse);
         total += (int)(int8_t)word + (int)(int8_t)(word >> 8) + (int)(int8_t)(word >> 16) + ((int)word >> 24);
         if (q != nullptr) *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + 4 * i) = word;
-        if (routing == kRouteScatter)
+        if (routing == kRouteScatter && d != nullptr)
             for (int c = 0; c < top_k; ++c) *reinterpret_cast<uint32_t*>(d + (int64_t)slot_of[c] * k + 4 * i) = word;
+        if (low != nullptr) {
+            // threads 2j and 2j + 1 hold the two halves of plane word j (the trip count is even, so both are here)
+            const bool second = i & 1;
+            uint32_t lo = second ? low_word_second(word) : low_word_first(word);
+            uint32_t hi = second ? high_word_second(word) : high_word_first(word);
+            lo |= __shfl_xor(lo, 1, 64), hi |= __shfl_xor(hi, 1, 64);
+            if (!second) {
+                if (routing == kRouteScatter) {
+                    for (int c = 0; c < top_k; ++c) {
+                        const int64_t at = plane_index(group_major, plane_rows, k >> 3, slot_of[c], i >> 1);
+                        low[at] = lo, high[at] = hi;
+                    }
+                } else {
+                    const int64_t at = plane_index(group_major, plane_rows, k >> 3, row, i >> 1);
+                    low[at] = lo, high[at] = hi;
+                }
+            }
+        }
     }
     if (sum == nullptr) return;  // uniform: one pointer for the whole launch
 #pragma unroll
@@ -723,32 +744,34 @@ int make_rotate_a8(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
-// rotate_expert_a8: buffers in ASCII order.  scatter: D,DS,IDs,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X;
-// shared: the same without D; no routing: Q,S,Signs,Sum,X.  slots used: K, top_k, E, flags (bit1 swiglu),
-// algorithm (routing).
+// rotate_expert_a8: buffers in ASCII order, looked up by name (the list depends on the routing and on the hand-over).
+// slots used: K, top_k, E, flags (bit1 swiglu, bit2 K64-major planes), algorithm (routing).
 int rotate_expert_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
-    (void)rows;
-    int8_t *q, *d = nullptr;
-    __half *s, *ds = nullptr;
-    const int *ids = nullptr, *relative = nullptr, *row_offsets = nullptr;
-    int *slot_map = nullptr, *sum;
-    const int8_t* signs;
-    const __half* x;
-    if (f.algorithm == 0) {
-        q = pointer_arg<int8_t>(args, 0), s = pointer_arg<__half>(args, 1), signs = pointer_arg<const int8_t>(args, 2);
-        sum = pointer_arg<int>(args, 3), x = pointer_arg<const __half>(args, 4);
-    } else {
-        int i = 0;
-        if (f.algorithm == kRouteScatter) d = pointer_arg<int8_t>(args, i++);
-        ds = pointer_arg<__half>(args, i++), ids = pointer_arg<const int>(args, i++), q = pointer_arg<int8_t>(args, i++);
-        relative = pointer_arg<const int>(args, i++), row_offsets = pointer_arg<const int>(args, i++);
-        s = pointer_arg<__half>(args, i++), signs = pointer_arg<const int8_t>(args, i++);
-        slot_map = pointer_arg<int>(args, i++), sum = pointer_arg<int>(args, i++), x = pointer_arg<const __half>(args, i++);
-    }
+    auto find = [&](const char* name) -> void* {
+        for (size_t i = 0; i < f.args.size(); ++i)
+            if (!strcmp(f.args[i].name, name)) return pointer_arg<void>(args, (int)i);
+        return nullptr;
+    };
+    int8_t* q = static_cast<int8_t*>(find("Q"));
+    int8_t* d = static_cast<int8_t*>(find("D"));
+    __half* s = static_cast<__half*>(find("S"));
+    __half* ds = static_cast<__half*>(find("DS"));
+    const int* ids = static_cast<const int*>(find("IDs"));
+    const int* relative = static_cast<const int*>(find("RelativeSlot"));
+    const int* row_offsets = static_cast<const int*>(find("RowOffsets"));
+    int* slot_map = static_cast<int*>(find("SlotMap"));
+    int* sum = static_cast<int*>(find("Sum"));
+    uint32_t* low = static_cast<uint32_t*>(find("Low"));
+    uint32_t* high = static_cast<uint32_t*>(find("High"));
+    const int8_t* signs = static_cast<const int8_t*>(find("Signs"));
+    const __half* x = static_cast<const __half*>(find("X"));
+    // planes have one row per slot under scatter, one per token otherwise; K64-major strides follow the live rows
+    const int plane_rows = f.algorithm == kRouteScatter ? rows * f.top_k : rows;
+    const int group_major = (f.flags & 4) ? 1 : 0;
     const dim3 grid(g.grid[0]), block(g.block[0]);
-#define ORX_ROTATE_EXPERT(SW, TH)                                                                                     \
+#define ORX_ROTATE_EXPERT(SW, TH)                                                                                      \
     hipLaunchKernelGGL((rotate_expert_kernel<SW, TH>), grid, block, g.shared, stream, x, signs, q, s, d, ds, ids,      \
-                       relative, row_offsets, slot_map, sum, f.K, f.top_k, f.algorithm)
+                       relative, row_offsets, slot_map, sum, low, high, plane_rows, group_major, f.K, f.top_k, f.algorithm)
     if (g.block[0] == 1024) {
         if (f.flags & 2) ORX_ROTATE_EXPERT(true, 1024);
         else ORX_ROTATE_EXPERT(false, 1024);
@@ -769,11 +792,12 @@ int make_rotate_expert(const Variant& v, orx_function* f) {
     f->top_k = (int)v.integer("top_k", 1, &bad);
     f->E = (int)v.integer("experts", 1, &bad);
     const bool swiglu = v.boolean("swiglu", false, &bad);
-    const bool reciprocal = v.boolean("reciprocal", true, &bad);
+    v.boolean("reciprocal", true, &bad);  // both forms of the reference give the same codes (the reciprocal one divides near ties)
     const bool group_major = v.boolean("group_major", false, &bad);
     const std::string routing = v.string("routing", "none", &bad);
+    // planes: the reference's buffers (Low, High for its INT4 expert GEMMs); int8: whole rows for the int8 expert GEMMs
+    const std::string hand_over = v.string("hand_over", "planes", &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
-    (void)reciprocal;  // both forms of the reference give the same codes (the reciprocal one divides near ties)
     if (f->M <= 0 || f->K <= 0 || f->K % 128 || f->K > 32768) {
         set_error("rotate_expert_a8: need M > 0 and K a multiple of 128 up to 32768");
         return ORX_ERR_BAD_VARIANT;
@@ -786,22 +810,35 @@ int make_rotate_expert(const Variant& v, orx_function* f) {
         set_error("rotate_expert_a8: need 1 <= top_k <= experts and top_k <= %d", kMaxRouteChoices);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (group_major) {
-        set_error("rotate_expert_a8: group_major lays out 4-bit planes for 64-wide K blocks; the expert GEMMs here "
-                  "multiply int8 rows, so there is no such layout");
+    if (hand_over != "planes" && hand_over != "int8") {
+        set_error("rotate_expert_a8: hand_over must be planes or int8");
         return ORX_ERR_BAD_VARIANT;
     }
-    f->flags = swiglu ? 2 : 0;
+    const bool planes = hand_over == "planes";
+    if (group_major && (routing != "none" || !planes)) {  // rotation_a8.py:409-410
+        set_error("rotate_expert_a8: K64-major planes need contiguous expert rows (no routing) and hand_over=planes");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = (swiglu ? 2 : 0) | (group_major ? 4 : 0);
     f->algorithm = routing == "scatter" ? kRouteScatter : routing == "shared" ? kRouteShared : 0;
     const uint32_t nullable = 0x80000000u;
+    const ArgSpec high = {"High", ArgPointer, 4}, low = {"Low", ArgPointer, 4};
     if (f->algorithm == 0) {
-        f->args = {{"Q", ArgPointer, 4}, {"S", ArgPointer, 2}, {"Signs", ArgPointer, 4}, {"Sum", ArgPointer, nullable | 4u},
-                   {"X", ArgPointer, 8}};
+        // rotate_split_a8: X, Signs, Q, S, Low, High, Sum; rotate_pack_a8 (K64-major) has no Q (rotation_a8.py:536-571)
+        if (planes) f->args = {high, low};
+        if (!group_major) f->args.push_back({"Q", ArgPointer, 4});
+        for (const ArgSpec& a : std::initializer_list<ArgSpec>{{"S", ArgPointer, 2}, {"Signs", ArgPointer, 4},
+                                                               {"Sum", ArgPointer, nullable | 4u}, {"X", ArgPointer, 8}})
+            f->args.push_back(a);
     } else {
-        if (f->algorithm == kRouteScatter) f->args.push_back({"D", ArgPointer, 4});
+        // rotate_dispatch_a8 (rotation_a8.py:573-604); the int8 hand-over has D (scatter) in place of Low and High
+        if (!planes && f->algorithm == kRouteScatter) f->args.push_back({"D", ArgPointer, 4});
+        f->args.push_back({"DS", ArgPointer, 2});
+        if (planes) f->args.push_back(high);
+        f->args.push_back({"IDs", ArgPointer, 4});
+        if (planes) f->args.push_back(low);
         const uint32_t q_align = f->algorithm == kRouteScatter ? nullable | 4u : 4u;
-        for (const ArgSpec& a : std::initializer_list<ArgSpec>{{"DS", ArgPointer, 2}, {"IDs", ArgPointer, 4},
-                                                               {"Q", ArgPointer, q_align}, {"RelativeSlot", ArgPointer, 4},
+        for (const ArgSpec& a : std::initializer_list<ArgSpec>{{"Q", ArgPointer, q_align}, {"RelativeSlot", ArgPointer, 4},
                                                                {"RowOffsets", ArgPointer, 4}, {"S", ArgPointer, 2},
                                                                {"Signs", ArgPointer, 4}, {"SlotMap", ArgPointer, 4},
                                                                {"Sum", ArgPointer, nullable | 4u}, {"X", ArgPointer, 8}})
@@ -973,8 +1010,10 @@ const Registration* quant_registrations(int* count) {
     {"swiglu", make_swiglu, "I, M=capacity", "X,Y,rows"},
     {"rotate_activation_a8", make_rotate_a8, "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, registers=false", "Q,S,Signs,X[,m]"},
     {"rotate_expert_a8", make_rotate_expert,
-     "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, routing=none|shared|scatter, top_k=1, experts=1",
-     "[D,]DS,IDs,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X[,m] (no routing: Q,S,Signs,Sum,X[,m])"},
+     "M, K, swiglu=false, reciprocal=true, dynamic_rows=false, routing=none|shared|scatter, top_k=1, experts=1, "
+     "group_major=false, hand_over=planes|int8",
+     "DS,High,IDs,Low,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X[,m] (no routing: High,Low,Q,S,Signs,Sum,X[,m]; "
+     "group_major: no Q; hand_over=int8: no High, Low and D first under scatter)"},
     {"rotate_activation", make_rotate, "M, K, swiglu=false", "Signs,X,Y"},
     {"residual_norm_rotate_a8", make_residual_rotate, "M, K=5120, dynamic_rows=false, zero_centered=true",
      "Q,R,RO,S,Signs,W,X,Y[,m]"},

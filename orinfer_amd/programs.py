@@ -136,7 +136,7 @@ class MoeLayer:
         self.k_rotate_dispatch = None
         if signs is not None:
             self.k_rotate_dispatch = Kernel("rotate_expert_a8", M=tokens, K=hidden, routing="scatter", top_k=top_k,
-                                            experts=experts)
+                                            experts=experts, hand_over="int8")
         grouped = dict(rows=assignments, E=experts, tiles=self.tile_capacity, block_m=block_m, packed_k=packed_k,
                        algorithm=grouped_algorithm)
         self.k_gate_up = Kernel("e8p_decode_grouped", N=2 * intermediate, K=hidden, **grouped)

@@ -296,9 +296,18 @@ def test_argument_lists_of_the_fused_expert_layer_forms():
         "A", "AS", "Book", "C", "Counts", "Offsets", "P", "Q", "RowMax", "TileCount", "TileExpert", "TileRow", "WS"]
     for listed in (plain, names("rotate_expert_a8", M=4, K=256, routing="scatter", top_k=2, experts=8)):
         assert listed == sorted(listed)
-    assert names("rotate_expert_a8", M=4, K=256, routing="shared", top_k=2, experts=8, dynamic_rows=True) == [
-        "DS", "IDs", "Q", "RelativeSlot", "RowOffsets", "S", "Signs", "SlotMap", "Sum", "X", "m"]
-    assert names("rotate_expert_a8", M=4, K=256) == ["Q", "S", "Signs", "Sum", "X"]
+    # the reference's lists (kernels/cuda/model/rotation_a8.py:536-589 in generated-ABI order): nibble planes Low and High
+    routed = ["DS", "High", "IDs", "Low", "Q", "RelativeSlot", "RowOffsets", "S", "Signs", "SlotMap", "Sum", "X"]
+    assert names("rotate_expert_a8", M=4, K=256, routing="shared", top_k=2, experts=8, dynamic_rows=True) == routed + ["m"]
+    assert names("rotate_expert_a8", M=4, K=256, routing="scatter", top_k=2, experts=8) == routed
+    assert names("rotate_expert_a8", M=4, K=256) == ["High", "Low", "Q", "S", "Signs", "Sum", "X"]
+    assert names("rotate_expert_a8", M=4, K=256, group_major=True) == ["High", "Low", "S", "Signs", "Sum", "X"]
+    # whole int8 rows for the int8 expert GEMMs: D (scatter) in place of the planes
+    assert names("rotate_expert_a8", M=4, K=256, routing="scatter", top_k=2, experts=8, hand_over="int8") == [
+        "D", "DS", "IDs", "Q", "RelativeSlot", "RowOffsets", "S", "Signs", "SlotMap", "Sum", "X"]
+    assert names("rotate_expert_a8", M=4, K=256, routing="shared", top_k=2, experts=8, hand_over="int8") == [
+        "DS", "IDs", "Q", "RelativeSlot", "RowOffsets", "S", "Signs", "SlotMap", "Sum", "X"]
+    assert names("rotate_expert_a8", M=4, K=256, hand_over="int8") == ["Q", "S", "Signs", "Sum", "X"]
     refused = (
         ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, rows=8200, E=128, tiles=512, block_m=32, algorithm="resident")),
         # without the SwiGLU epilogue the kernel keeps its phase-two sums in LDS, which leaves room for fewer slots
@@ -308,7 +317,9 @@ def test_argument_lists_of_the_fused_expert_layer_forms():
         ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, rows=2048, E=128, tiles=192, block_m=64)),
         ("e8p_decode_grouped", dict(N=1024, K=2048, epilogue="swiglu", rows=2048, E=128, tiles=192, block_m=32,
                                     algorithm="stream")),
-        ("rotate_expert_a8", dict(M=4, K=256, group_major=True)),
+        ("rotate_expert_a8", dict(M=4, K=256, group_major=True, routing="shared", top_k=2, experts=8)),  # rotation_a8.py:409
+        ("rotate_expert_a8", dict(M=4, K=256, group_major=True, hand_over="int8")),
+        ("rotate_expert_a8", dict(M=4, K=256, hand_over="fp8")),
         ("rotate_expert_a8", dict(M=4, K=256, routing="scatter", top_k=65, experts=128)),
         ("router_topk", dict(M=8, E=64, top_k=4, quantize_hidden=100)),
     )

@@ -786,10 +786,11 @@ def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, 
         ds=torch.full((cap * k,), 3.0, dtype=torch.float16, device=gu.DEV), slot_map=torch.full((cap, k), -1, **I32),
         total=torch.full((cap * k,), -5, **I32))
     common = dict(M=cap, K=h, swiglu=swiglu, dynamic_rows=True)
+    int8 = dict(hand_over="int8", **common)
 
     # scatter: codes, scale and sum land in every slot of the row
     o = fresh()
-    kern = gu.kernel("rotate_expert_a8", routing="scatter", top_k=k, experts=e, **common)
+    kern = gu.kernel("rotate_expert_a8", routing="scatter", top_k=k, experts=e, **int8)
     kern(D=o["d"], DS=o["ds"], IDs=d_ids, Q=o["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=o["s"], Signs=d_signs,
          SlotMap=o["slot_map"], Sum=o["total"], X=d_x, m=m)
     np.testing.assert_array_equal(gu.host(o["q"])[:m], want_q)
@@ -818,7 +819,7 @@ def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, 
 
     # shared: the codes stay in Q, every assignment gets its scale and slot
     sh = fresh()
-    gu.kernel("rotate_expert_a8", routing="shared", top_k=k, experts=e, **common)(
+    gu.kernel("rotate_expert_a8", routing="shared", top_k=k, experts=e, **int8)(
         DS=sh["ds"], IDs=d_ids, Q=sh["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=sh["s"], Signs=d_signs,
         SlotMap=sh["slot_map"], Sum=sh["total"], X=d_x, m=m)
     assert torch.equal(sh["q"], o["q"]) and torch.equal(sh["ds"], o["ds"]) and torch.equal(sh["slot_map"], o["slot_map"])
@@ -827,14 +828,61 @@ def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, 
 
     # no routing: codes, scale and the row sum
     plain = fresh()
-    gu.kernel("rotate_expert_a8", **common)(Q=plain["q"], S=plain["s"], Signs=d_signs, Sum=plain["total"], X=d_x, m=m)
+    gu.kernel("rotate_expert_a8", **int8)(Q=plain["q"], S=plain["s"], Signs=d_signs, Sum=plain["total"], X=d_x, m=m)
     assert torch.equal(plain["q"], o["q"]) and torch.equal(plain["s"], o["s"])
     np.testing.assert_array_equal(gu.host(plain["total"])[:m], want_q.astype(np.int32).sum(1))
+
+    # the reference's own hand-over (rotation_a8.py:489-531): the same codes as two planes of nibble words
+    def planes(rows, group_major=False):
+        shape = (h // 64, rows, 8) if group_major else (rows, h // 8)
+        return torch.full(shape, -1, **I32), torch.full(shape, -1, **I32)
+
+    def check(low, high, codes, group_major=False):
+        want_low, want_high, _ = orc.split_planes(codes)
+        got_low, got_high = gu.host(low, np.uint32), gu.host(high, np.uint32)
+        rows = codes.shape[0]
+        if group_major:  # the stride is the live row count
+            words = h // 64 * rows * 8
+            assert (got_low.reshape(-1)[words:] == 0xFFFFFFFF).all() and (got_high.reshape(-1)[words:] == 0xFFFFFFFF).all()
+            got_low = orc.planes_row_major(got_low.reshape(-1)[:words].reshape(h // 64, rows, 8))
+            got_high = orc.planes_row_major(got_high.reshape(-1)[:words].reshape(h // 64, rows, 8))
+        else:
+            assert (got_low[rows:] == 0xFFFFFFFF).all() and (got_high[rows:] == 0xFFFFFFFF).all()
+        np.testing.assert_array_equal(got_low[:rows], want_low)
+        np.testing.assert_array_equal(got_high[:rows], want_high)
+
+    p = fresh()
+    low, high = planes(cap * k)
+    gu.kernel("rotate_expert_a8", routing="scatter", top_k=k, experts=e, **common)(
+        DS=p["ds"], High=high, IDs=d_ids, Low=low, Q=p["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=p["s"], Signs=d_signs,
+        SlotMap=p["slot_map"], Sum=p["total"], X=d_x, m=m)
+    check(low, high, want_d)
+    for name in ("q", "s", "ds", "slot_map", "total"):
+        assert torch.equal(p[name], o[name]), name
+    p = fresh()
+    low, high = planes(cap)
+    gu.kernel("rotate_expert_a8", routing="shared", top_k=k, experts=e, **common)(
+        DS=p["ds"], High=high, IDs=d_ids, Low=low, Q=p["q"], RelativeSlot=d_rel, RowOffsets=d_off, S=p["s"], Signs=d_signs,
+        SlotMap=p["slot_map"], Sum=p["total"], X=d_x, m=m)
+    check(low, high, want_q)
+    for name in ("q", "s", "ds", "slot_map", "total"):
+        assert torch.equal(p[name], sh[name]), name
+    p = fresh()
+    low, high = planes(cap)
+    gu.kernel("rotate_expert_a8", **common)(High=high, Low=low, Q=p["q"], S=p["s"], Signs=d_signs, Sum=p["total"], X=d_x, m=m)
+    check(low, high, want_q)
+    assert torch.equal(p["q"], plain["q"]) and torch.equal(p["s"], plain["s"]) and torch.equal(p["total"], plain["total"])
+    p = fresh()
+    low, high = planes(cap, True)
+    gu.kernel("rotate_expert_a8", group_major=True, **common)(High=high, Low=low, S=p["s"], Signs=d_signs, Sum=p["total"], X=d_x, m=m)
+    check(low, high, want_q, True)
+    assert torch.equal(p["s"], plain["s"]) and torch.equal(p["total"], plain["total"])
 
 
 def test_rotate_expert_a8_refuses_what_it_does_not_serve():
     for variant in (dict(K=192), dict(routing="broadcast"), dict(routing="scatter", top_k=9, experts=8),
-                    dict(routing="scatter", top_k=65, experts=128), dict(group_major=True), dict(M=0)):
+                    dict(routing="scatter", top_k=65, experts=128), dict(group_major=True, routing="shared", top_k=1, experts=2),
+                    dict(M=0)):
         with pytest.raises(Exception):
             gu.kernel("rotate_expert_a8", **{**dict(M=4, K=256), **variant})
 
@@ -879,7 +927,7 @@ def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
         ("e8p_decode_grouped", dict(N=1024, K=2048, gather=True, epilogue="swiglu", **grouped)),
         ("e8p_decode_grouped", dict(N=2048, K=512, input_dtype="float16", **grouped)),
         ("e8p_decode_grouped", dict(N=2048, K=512, **grouped)),
-        ("rotate_expert_a8", dict(M=256, K=2048, routing="scatter", top_k=8, experts=128)),
+        ("rotate_expert_a8", dict(M=256, K=2048, routing="scatter", top_k=8, experts=128, hand_over="int8")),
         ("rotate_expert_a8", dict(M=8192, K=5120)),
         ("expert_dispatch", dict(M=256, H=2048, E=128, top_k=8, input_dtype="float16")),
         ("moe_combine", dict(M=256, H=2048, slots=2048, E=128, top_k=8)),

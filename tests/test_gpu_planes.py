@@ -287,3 +287,46 @@ def test_prefill_grouped_merges_adjacent_tiles_of_a_shared_list_and_takes_live_r
     got = gu.host(out)
     np.testing.assert_array_equal(got[:rows], want)
     assert (got[rows:] == 91).all()
+
+
+def test_rotated_planes_into_the_exact_kernel_equal_int8_rows_into_the_int8_kernel():
+    # one routed expert projection both ways: rotate_expert_a8 writes planes at the slots and e8p_exact_grouped reads them
+    # (the reference's pairing, flash_next/experts.rs:207-215), or it writes int8 rows and e8p_decode_grouped reads those
+    rng = np.random.default_rng(orc.SEED + 11)
+    m, e, top_k, h, n, bm = 21, 8, 2, 512, 192, 16
+    basis = orc.basis()
+    x = rng.normal(size=(m, h)).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), h)
+    ids, _ = orc.router_topk(rng.normal(size=(m, e)).astype(np.float32), top_k)
+    counts, relative = orc.expert_histogram(ids, e)
+    offsets, tile_offsets, total = orc.expert_offsets(counts, bm)
+    slots = m * top_k
+    cap = orc.tile_capacity(slots, e, bm)
+    te, tr = orc.expert_tiles(counts, tile_offsets, bm, cap)
+    raw = rng.integers(0, 65536, (e, h // 128, n, 16), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    routing = dict(IDs=gu.dev(ids), RelativeSlot=gu.dev(relative), RowOffsets=gu.dev(offsets), Signs=gu.dev(signs), X=gu.dev(x))
+    shape = dict(M=m, K=h, routing="scatter", top_k=top_k, experts=e)
+    tiles = dict(Counts=gu.dev(counts), Offsets=gu.dev(offsets))
+    q = torch.empty((m, h), dtype=torch.int8, device=gu.DEV)
+    s = torch.empty((m,), dtype=torch.float16, device=gu.DEV)
+    ds = torch.empty((slots,), dtype=torch.float16, device=gu.DEV)
+    slot_map, sums = torch.empty((m, top_k), **I32), torch.empty((slots,), **I32)
+    d = torch.empty((slots, h), dtype=torch.int8, device=gu.DEV)
+    gu.kernel("rotate_expert_a8", hand_over="int8", **shape)(D=d, DS=ds, Q=q, S=s, SlotMap=slot_map, Sum=sums, **routing)
+    ref = torch.full((slots, n), float("nan"), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("e8p_decode_grouped", rows=slots, E=e, tiles=cap, N=n, K=h, block_m=32)(
+        A=d, AS=ds, Book=gu.book(), C=ref, P=gu.dev(raw), TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr),
+        WS=gu.dev(ws), **tiles)
+    low, high = empty_planes(slots, h, False)
+    ds2, sums2 = torch.empty_like(ds), torch.empty_like(sums)
+    gu.kernel("rotate_expert_a8", **shape)(DS=ds2, High=high, Low=low, Q=q, S=s, SlotMap=slot_map, Sum=sums2, **routing)
+    out = torch.full((slots, n), float("nan"), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("e8p_exact_grouped", rows=slots, E=e, tiles=cap, N=n, K=h, block_m=bm)(
+        AS=ds2, Book=gu.dev(orc.nibble_table(orc.selector_table(basis))[None]), High=high, Low=low, Out=out,
+        P=gu.dev(orc.q2_repack_k64(raw)), Sum=sums2, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws), **tiles)
+    assert torch.equal(out, ref) and not bool(torch.isnan(out).any())
+    want_q, want_s, want_d, want_ds, want_map, want_sum = orc.rotate_expert_a8(x, signs, ids, relative, offsets)
+    codes = np.ascontiguousarray(raw.transpose(0, 2, 1, 3)).reshape(e, n, h // 8)
+    weights = np.stack([orc.q2_integers(c, basis) for c in codes])
+    np.testing.assert_array_equal(gu.host(out), orc.grouped_project(want_d, want_ds, weights, ws, counts, offsets))
