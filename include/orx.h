@@ -35,6 +35,13 @@
  * run on the MFMA tile kernel only.  The symbol always lists Patch, as the reference's
  * host ABI does; without patched=true it is never read and may be null.
  *
+ * The reference's INT4-exact expert kernels (e8p_exact.py, e8p_prefill.py) take A8 rows as two planes
+ * of nibble words, Low and High, with the rows' integer sums: split_a8, split_prefill_a8,
+ * split_routed_prefill_a8, dispatch_prefill_a8, pack_expert_tokens, expand_expert_slots and
+ * rotate_expert_a8 write them, e8p_exact_grouped and e8p_prefill_grouped multiply them (on int8
+ * MFMA, the nibbles put back together on the way into LDS; Sum is added as given).  Same symbols,
+ * variant keys and argument order as the reference (flash_next/experts.rs:207-215).
+ *
  * Thread model: one thread per device session, one explicit stream
  * (backend/cuda/mod.rs:1-3).  Handles are immutable after orx_resolve: launches of one
  * handle, or of different handles, may run concurrently on distinct streams as long as
