@@ -572,7 +572,14 @@ __global__ __launch_bounds__(256) void gemm_split_finish_kernel(GemmParams p, in
 // Whole-matrix decode to int8 (diagnostic; e8p_q4.py:267-302).  One thread per code.
 template <int CODEC>
 __global__ __launch_bounds__(256) void unpack_kernel(const void* __restrict__ w, const uint32_t* __restrict__ book,
-                                                     uint2* __restrict__ out, int n, int k, int packed_k) {
+                                                     uint2* __restrict__ out, int n, int k, int packed_k,
+                                                     const int* __restrict__ counts) {
+    // banks of routed experts (grid y): only the experts that have rows are decoded (kernels/cuda/model/moe.py:147-173)
+    if (counts != nullptr) {
+        if (counts[blockIdx.y] <= 0) return;
+        w = reinterpret_cast<const int8_t*>(w) + (int64_t)blockIdx.y * n * (k / 8) * (CODEC == kQ4 ? 4 : 2);
+        out += (int64_t)blockIdx.y * n * (k / 8);
+    }
     __shared__ typename Tables<CODEC>::type tables;
     build_tables(tables, book, threadIdx.x, 256);
     __syncthreads();
@@ -1495,10 +1502,45 @@ int unpack_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
     uint2* out = pointer_arg<uint2>(args, 1);
     const void* w = pointer_arg<const void>(args, 2);
     if (f.flags == kQ4)
-        hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k);
+        hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
     else
-        hipLaunchKernelGGL((unpack_kernel<kQ2>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k);
+        hipLaunchKernelGGL((unpack_kernel<kQ2>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
     return hip_check(hipGetLastError(), "launch unpack");
+}
+
+// expand_experts (kernels/cuda/model/moe.py:146-173): Book, Counts, Out, W.  slots used: N, K, E
+int expand_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = ceil_div((uint32_t)((int64_t)f.N * (f.K / 8)), 256u);
+    g->grid[1] = (uint32_t)f.E;
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int expand_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const void>(args, 3),
+                       pointer_arg<const uint32_t>(args, 0), pointer_arg<uint2>(args, 2), f.N, f.K, 128,
+                       pointer_arg<const int>(args, 1));
+    return hip_check(hipGetLastError(), "launch expand_experts");
+}
+int make_expand_experts(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->E = (int)v.integer("E", 0, &bad);
+    const int block_n = (int)v.integer("block_n", 64, &bad), block_k = (int)v.integer("block_k", 256, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // moe.py:152-153: whole tiles of the reference's kernel; the codes come in K-major blocks of 128
+    if (f->N <= 0 || f->K <= 0 || f->E <= 0 || block_n <= 0 || block_k <= 0 || f->N % block_n || f->K % block_k || f->K % 128) {
+        set_error("expand_experts: need N, K, E > 0, N a multiple of block_n, K a multiple of block_k and of 128");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->capacity = 1;
+    f->args = {{"Book", ArgPointer, 4}, {"Counts", ArgPointer, 4}, {"Out", ArgPointer, 8}, {"W", ArgPointer, 4}};
+    f->geometry = expand_geometry;
+    f->launch = expand_launch;
+    f->device_function = reinterpret_cast<const void*>(&unpack_kernel<kQ4>);
+    return ORX_OK;
 }
 
 int make_unpack(const Variant& v, orx_function* f, int codec) {
@@ -1556,6 +1598,7 @@ const Registration* gemm_registrations(int* count) {
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
+    {"expand_experts", make_expand_experts, "N, K, E, block_n=64, block_k=256", "Book,Counts,Out,W"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;

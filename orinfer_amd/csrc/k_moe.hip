@@ -110,6 +110,58 @@ __global__ __launch_bounds__(256) void expert_histogram_kernel(const int* __rest
     if (threadIdx.x == 0) counts[expert] = base;
 }
 
+// ---- the histogram in three launches over segments of the assignment list (kernels/cuda/model/moe.py:556-656) ----
+// local:   grid (segments, E).  Partial[e, s] = assignments of segment s routed to expert e, Slots[i] = rank of
+//          assignment i among those of its expert inside its segment.
+// offsets: grid E.  Offsets[e, s] = exclusive prefix of Partial[e, :], Counts[e] = their sum.
+// finish:  Slots[i] += Offsets[IDs[i], segment of i]: the token-major stable slot of expert_histogram.
+// Partial and Offsets are (E, segments) with the segments of the live rows.
+__global__ __launch_bounds__(256) void histogram_local_kernel(const int* __restrict__ ids, int* __restrict__ partial,
+                                                              int* __restrict__ slots, int assignments, int block,
+                                                              int segments) {
+    __shared__ int wave_totals[4];
+    const int segment = blockIdx.x, expert = blockIdx.y;
+    int base = 0;
+    for (int first = 0; first < block; first += 256) {
+        const int i = segment * block + first + threadIdx.x;
+        const bool match = first + (int)threadIdx.x < block && i < assignments && ids[i] == expert;
+        int total;
+        const int prefix = block_flag_scan(match, wave_totals, &total);
+        if (match) slots[i] = base + prefix;
+        base += total;
+    }
+    if (threadIdx.x == 0) partial[(int64_t)expert * segments + segment] = base;
+}
+
+__global__ __launch_bounds__(64) void histogram_offsets_kernel(const int* __restrict__ partial, int* __restrict__ offsets,
+                                                               int* __restrict__ counts, int segments) {
+    const int expert = blockIdx.x, lane = threadIdx.x;
+    const int per = (segments + 63) / 64;
+    const int begin = min(lane * per, segments), end = min(begin + per, segments);
+    const int* row = partial + (int64_t)expert * segments;
+    int mine = 0;
+    for (int j = begin; j < end; ++j) mine += row[j];
+    int inclusive = mine;
+#pragma unroll
+    for (int offset = 1; offset < 64; offset <<= 1) {
+        const int other = __shfl_up(inclusive, offset, 64);
+        if (lane >= offset) inclusive += other;
+    }
+    int running = inclusive - mine;
+    for (int j = begin; j < end; ++j) {
+        offsets[(int64_t)expert * segments + j] = running;
+        running += row[j];
+    }
+    if (lane == 63) counts[expert] = inclusive;
+}
+
+__global__ __launch_bounds__(256) void histogram_finish_kernel(const int* __restrict__ ids, const int* __restrict__ offsets,
+                                                               int* __restrict__ slots, int assignments, int block,
+                                                               int segments) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < assignments) slots[i] += offsets[(int64_t)ids[i] * segments + i / block];
+}
+
 // one block: exclusive prefixes of counts and of ceil(counts/bm); TileCount = total tiles.
 __global__ __launch_bounds__(256) void expert_offsets_kernel(const int* __restrict__ counts, int* __restrict__ row_offsets,
                                                              int* __restrict__ tile_count, int* __restrict__ tile_offsets,
@@ -631,6 +683,61 @@ int make_histogram(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// expert_histogram_local / _offsets / _finish (moe.py:556-656).  slots used: M, E, top_k (the reference's K), group (block),
+// algorithm (0 local, 1 offsets, 2 finish)
+int segmented_geometry(const orx_function& f, int rows, Geometry* g) {
+    const uint32_t assignments = (uint32_t)rows * (uint32_t)f.top_k, segments = ceil_div(assignments, (uint32_t)f.group);
+    if (f.algorithm == 0) {
+        g->grid[0] = segments, g->grid[1] = (uint32_t)f.E, g->block[0] = 256;
+    } else if (f.algorithm == 1) {
+        g->grid[0] = (uint32_t)f.E, g->block[0] = 64;
+    } else {
+        g->grid[0] = ceil_div(assignments, 256u), g->block[0] = 256;
+    }
+    return ORX_OK;
+}
+int segmented_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    const int assignments = rows * f.top_k, segments = (assignments + f.group - 1) / f.group;
+    const dim3 grid(g.grid[0], g.grid[1]), block(g.block[0]);
+    if (f.algorithm == 0)  // IDs, Partial, Slots
+        hipLaunchKernelGGL(histogram_local_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0), pointer_arg<int>(args, 1),
+                           pointer_arg<int>(args, 2), assignments, f.group, segments);
+    else if (f.algorithm == 1)  // Counts, Offsets, Partial
+        hipLaunchKernelGGL(histogram_offsets_kernel, grid, block, 0, s, pointer_arg<const int>(args, 2),
+                           pointer_arg<int>(args, 1), pointer_arg<int>(args, 0), segments);
+    else  // IDs, Offsets, Slots
+        hipLaunchKernelGGL(histogram_finish_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0),
+                           pointer_arg<const int>(args, 1), pointer_arg<int>(args, 2), assignments, f.group, segments);
+    return hip_check(hipGetLastError(), "launch segmented expert histogram");
+}
+int make_segmented(const Variant& v, orx_function* f, int stage) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->E = (int)v.integer("E", 512, &bad);
+    f->top_k = (int)v.integer("K", 10, &bad);
+    f->group = (int)v.integer("block", 1024, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (f->M <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || (f->group != 512 && f->group != 1024 && f->group != 2048)) {
+        set_error("%s: need M, E > 0, 1 <= K <= E and block 512, 1024 or 2048", f->symbol.c_str());
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->algorithm = stage;
+    if (stage == 0) f->args = {{"IDs", ArgPointer, 4}, {"Partial", ArgPointer, 4}, {"Slots", ArgPointer, 4}};
+    if (stage == 1) f->args = {{"Counts", ArgPointer, 4}, {"Offsets", ArgPointer, 4}, {"Partial", ArgPointer, 4}};
+    if (stage == 2) f->args = {{"IDs", ArgPointer, 4}, {"Offsets", ArgPointer, 4}, {"Slots", ArgPointer, 4}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = segmented_geometry;
+    f->launch = segmented_launch;
+    f->device_function = stage == 0   ? reinterpret_cast<const void*>(&histogram_local_kernel)
+                         : stage == 1 ? reinterpret_cast<const void*>(&histogram_offsets_kernel)
+                                      : reinterpret_cast<const void*>(&histogram_finish_kernel);
+    return ORX_OK;
+}
+int make_histogram_local(const Variant& v, orx_function* f) { return make_segmented(v, f, 0); }
+int make_histogram_offsets(const Variant& v, orx_function* f) { return make_segmented(v, f, 1); }
+int make_histogram_finish(const Variant& v, orx_function* f) { return make_segmented(v, f, 2); }
+
 int one_block_geometry(const orx_function&, int, Geometry* g) {
     g->block[0] = 256;
     return ORX_OK;
@@ -929,6 +1036,12 @@ const Registration* moe_registrations(int* count) {
      "IDs,Logits,Prob[,Q,S,X][,m]"},
     {"router_topk_warp", make_router_warp, "M, E, top_k, dynamic_rows=false, warps=4", "IDs,Logits,Prob[,m]"},
     {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
+    {"expert_histogram_local", make_histogram_local, "M, E=512, K=10 (routes per token), block=1024|512|2048, dynamic_rows=false",
+     "IDs,Partial,Slots[,m]"},
+    {"expert_histogram_offsets", make_histogram_offsets, "M, E=512, K=10, block=1024|512|2048, dynamic_rows=false",
+     "Counts,Offsets,Partial[,m]"},
+    {"expert_histogram_finish", make_histogram_finish, "M, E=512, K=10, block=1024|512|2048, dynamic_rows=false",
+     "IDs,Offsets,Slots[,m]"},
     {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
     {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false, slot_maps=false",

@@ -394,6 +394,63 @@ __global__ __launch_bounds__(THREADS) void rotate_expert_kernel(
     }
 }
 
+// The rotation and the quantiser as two launches over tiles of block_k channels, for few long rows
+// (kernels/cuda/model/rotation_a8.py:266-365): rotate_activation_tiles writes the rotated fp16 values and each tile's
+// largest magnitude, quantize_rotation_tiles takes the row maximum of the tile maxima and quantises its tile.
+// grid (rows, ceil(K / block_k)).  With plane_rows the up rows follow the gate rows as a second plane of X.
+template <bool SWIGLU>
+__global__ __launch_bounds__(256) void rotate_tiles_kernel(const __half* __restrict__ x, const int8_t* __restrict__ signs,
+                                                           __half* __restrict__ rotated, float* __restrict__ maxima, int k,
+                                                           int block_k, int64_t row_stride, int64_t up_delta) {
+    __shared__ float scratch[4];
+    const int row = blockIdx.x, tile = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int half_wave = lane >> 5, l32 = lane & 31;
+    const int first_block = tile * (block_k / 128), end_block = min(first_block + block_k / 128, k / 128);
+    const int64_t in_base = (int64_t)row * row_stride;
+    float amax = 0.f;
+    for (int pair = wave; first_block + 2 * pair < end_block; pair += 4) {  // wave-uniform trip count
+        const int block = first_block + 2 * pair + half_wave;
+        const bool live = block < end_block;
+        const int first = (live ? block : first_block) * 128 + 4 * l32;
+        const uint2 raw = *reinterpret_cast<const uint2*>(x + in_base + first);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const uint32_t sign_word = *reinterpret_cast<const uint32_t*>(signs + first);
+        uint2 raw_up = make_uint2(0u, 0u);
+        if (SWIGLU) raw_up = *reinterpret_cast<const uint2*>(x + in_base + up_delta + first);
+        const __half* up = reinterpret_cast<const __half*>(&raw_up);
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float value = SWIGLU ? swiglu_value(h[j], up[j]) : __half2float(h[j]);
+            v[j] = live ? value * (float)(int8_t)(sign_word >> (8 * j)) : 0.f;
+        }
+        __half out[4];
+        amax = fmaxf(amax, rotate_block(v, l32, out));
+        if (live) *reinterpret_cast<uint2*>(rotated + (int64_t)row * k + first) = *reinterpret_cast<const uint2*>(out);
+    }
+    amax = block_max(amax, scratch);
+    if (tid == 0) maxima[(int64_t)row * gridDim.y + tile] = amax;
+}
+
+__global__ __launch_bounds__(256) void quantize_tiles_kernel(const __half* __restrict__ rotated, const float* __restrict__ maxima,
+                                                             int8_t* __restrict__ q, __half* __restrict__ s, int k, int block_k) {
+    __shared__ float scratch[4];
+    const int row = blockIdx.x, tile = blockIdx.y, tiles = gridDim.y, tid = threadIdx.x;
+    float amax = 0.f;
+    for (int j = tid; j < tiles; j += 256) amax = fmaxf(amax, maxima[(int64_t)row * tiles + j]);
+    amax = block_max(amax, scratch);
+    const __half stored = a8_scale(amax);
+    if (tile == 0 && tid == 0) s[row] = stored;
+    const float scale = __half2float(stored), inverse = __frcp_rn(scale);
+    const int first = tile * block_k, width = min(block_k, k - first);
+    for (int i = tid; i < width / 4; i += 256) {
+        const uint2 raw = *reinterpret_cast<const uint2*>(rotated + (int64_t)row * k + first + 4 * i);
+        const __half* h = reinterpret_cast<const __half*>(&raw);
+        const float values[4] = {__half2float(h[0]), __half2float(h[1]), __half2float(h[2]), __half2float(h[3])};
+        *reinterpret_cast<uint32_t*>(q + (int64_t)row * k + first + 4 * i) = quantise4(values, scale, inverse);
+    }
+}
+
 // The rotation alone (kernels/cuda/model/integer_vq.py:447-486): Y = fp16(rotated * 128^-1/2), the
 // values rotate_a8_kernel quantises.  Same lane layout; nothing is kept in LDS.
 template <bool SWIGLU>
@@ -910,6 +967,94 @@ int residual_rotate_launch(const orx_function& f, int rows, const Geometry& g, h
     return hip_check(hipGetLastError(), "launch residual_norm_rotate_a8");
 }
 
+// rotate_activation_tiles / quantize_rotation_tiles.  slots used: K, group (block_k), flags (bit1 swiglu), slots (plane_rows)
+int tiles_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = (uint32_t)rows;
+    g->grid[1] = ceil_div((uint32_t)f.K, (uint32_t)f.group);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+// Maxima, Rotated, Signs, X[, m]
+int rotate_tiles_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    float* maxima = pointer_arg<float>(args, 0);
+    __half* rotated = pointer_arg<__half>(args, 1);
+    const int8_t* signs = pointer_arg<const int8_t>(args, 2);
+    const __half* x = pointer_arg<const __half>(args, 3);
+    const dim3 grid(g.grid[0], g.grid[1]), block(256);
+    if (f.flags & 2) {
+        const int64_t stride = f.slots ? f.K : 2 * (int64_t)f.K, up = f.slots ? (int64_t)f.slots * f.K : f.K;
+        hipLaunchKernelGGL((rotate_tiles_kernel<true>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group, stride, up);
+    } else {
+        hipLaunchKernelGGL((rotate_tiles_kernel<false>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group,
+                           (int64_t)f.K, (int64_t)0);
+    }
+    return hip_check(hipGetLastError(), "launch rotate_activation_tiles");
+}
+// Maxima, Q, Rotated, S[, m]
+int quantize_tiles_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows;
+    hipLaunchKernelGGL(quantize_tiles_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const __half>(args, 2),
+                       pointer_arg<const float>(args, 0), pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 3), f.K, f.group);
+    return hip_check(hipGetLastError(), "launch quantize_rotation_tiles");
+}
+bool tile_shape_ok(const orx_function& f) {
+    const int bk = f.group;
+    return f.M > 0 && f.K > 0 && f.K % 128 == 0 && (bk == 128 || bk == 256 || bk == 512 || bk == 1024 || bk == 2048);
+}
+int make_rotate_tiles(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->group = (int)v.integer("block_k", 512, &bad);
+    const bool swiglu = v.boolean("swiglu", false, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    f->slots = (int)v.integer("plane_rows", 0, &bad);
+    const bool registers = v.boolean("registers", false, &bad);
+    const int threads = (int)v.integer("threads", 128, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (!tile_shape_ok(*f)) {  // rotation_a8.py:279-280
+        set_error("rotate_activation_tiles: need M > 0, K a multiple of 128 and block_k 128, 256, 512, 1024 or 2048");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->slots < 0 || (f->slots && (!swiglu || f->slots < f->M))) {  // rotation_a8.py:281-286
+        set_error("rotate_activation_tiles: plane_rows needs swiglu and at least M rows");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    // rotation_a8.py:227-228, :287-288: block sizes of the reference's two kernels; the block here is 256 threads
+    if ((!registers && threads != 128) ||
+        (registers && ((threads != 64 && threads != 128 && threads != 256 && threads != 512) || f->group % (threads * 4)))) {
+        set_error("rotate_activation_tiles: threads is 128, or with registers 64..512 with block_k a multiple of 4 threads");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->flags = swiglu ? 2 : 0;
+    f->args = {{"Maxima", ArgPointer, 4}, {"Rotated", ArgPointer, 8}, {"Signs", ArgPointer, 4}, {"X", ArgPointer, 8}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = swiglu ? reinterpret_cast<const void*>(&rotate_tiles_kernel<true>)
+                                : reinterpret_cast<const void*>(&rotate_tiles_kernel<false>);
+    f->geometry = tiles_geometry;
+    f->launch = rotate_tiles_launch;
+    return ORX_OK;
+}
+int make_quantize_tiles(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    f->group = (int)v.integer("block_k", 512, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (!tile_shape_ok(*f)) {  // rotation_a8.py:332-333
+        set_error("quantize_rotation_tiles: need M > 0, K a multiple of 128 and block_k 128, 256, 512, 1024 or 2048");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"Maxima", ArgPointer, 4}, {"Q", ArgPointer, 4}, {"Rotated", ArgPointer, 8}, {"S", ArgPointer, 2}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = reinterpret_cast<const void*>(&quantize_tiles_kernel);
+    f->geometry = tiles_geometry;
+    f->launch = quantize_tiles_launch;
+    return ORX_OK;
+}
+
 int make_residual_rotate(const Variant& v, orx_function* f) {
     bool bad = false;
     f->K = (int)v.integer("K", 5120, &bad);
@@ -953,7 +1098,8 @@ int q4_embedding_launch(const orx_function& f, int rows, const Geometry& g, hipS
 int make_q4_embedding(const Variant& v, orx_function* f) {
     if (!two_stage_coefficients_ok(v, "e8p_q4_embedding")) return ORX_ERR_BAD_VARIANT;
     bool bad = false;
-    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    // the reference's factory calls the row capacity `capacity` (kernels/cuda/model/e8p_q4.py:84)
+    f->capacity = f->M = (int)v.integer(v.has("capacity") ? "capacity" : "M", 0, &bad);
     f->N = (int)v.integer("vocab", 0, &bad);
     f->K = (int)v.integer("hidden", 0, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
@@ -1015,9 +1161,12 @@ const Registration* quant_registrations(int* count) {
      "DS,High,IDs,Low,Q,RelativeSlot,RowOffsets,S,Signs,SlotMap,Sum,X[,m] (no routing: High,Low,Q,S,Signs,Sum,X[,m]; "
      "group_major: no Q; hand_over=int8: no High, Low and D first under scatter)"},
     {"rotate_activation", make_rotate, "M, K, swiglu=false", "Signs,X,Y"},
+    {"rotate_activation_tiles", make_rotate_tiles,
+     "M, K, block_k=512, swiglu=false, dynamic_rows=false, plane_rows=0, registers=false, threads=128", "Maxima,Rotated,Signs,X[,m]"},
+    {"quantize_rotation_tiles", make_quantize_tiles, "M, K, block_k=512, dynamic_rows=false", "Maxima,Q,Rotated,S[,m]"},
     {"residual_norm_rotate_a8", make_residual_rotate, "M, K=5120, dynamic_rows=false, zero_centered=true",
      "Q,R,RO,S,Signs,W,X,Y[,m]"},
-    {"e8p_q4_embedding", make_q4_embedding, "M, vocab, hidden", "Book,IDs,Output,Scale,Signs,Weight,m"},
+    {"e8p_q4_embedding", make_q4_embedding, "M (or capacity), vocab, hidden", "Book,IDs,Output,Scale,Signs,Weight,m"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));
     return rows;

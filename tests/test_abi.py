@@ -561,6 +561,18 @@ REFERENCE_KEYWORDS = {
                                split_k=2, parity_xor=True, group_n=2, packed_k=64, dynamic_rows=True),
     "integer_e8p_gemv": dict(E=8, routes=2, N=256, K=512, shared_input=True, block_n=8),
     "rotate_activation": dict(M=8, K=512, swiglu=True),
+    "rotate_activation_tiles": dict(M=8, K=1024, block_k=1024, swiglu=True, dynamic_rows=True, plane_rows=8, registers=True,
+                                    threads=256),
+    "quantize_rotation_tiles": dict(M=8, K=1024, block_k=256, dynamic_rows=True),
+    "expert_histogram_local": dict(M=64, E=16, K=4, block=512, dynamic_rows=True),
+    "expert_histogram_offsets": dict(M=64, E=16, K=4, block=2048, dynamic_rows=False),
+    "expert_histogram_finish": dict(M=64, E=16, K=4, block=1024, dynamic_rows=True),
+    "expand_experts": dict(N=256, K=512, E=8, block_n=64, block_k=256),
+    "e8p_q4_embedding": dict(capacity=8, vocab=1000, hidden=512),
+    "e8p_q4_projection": dict(M=8, N=256, K=512, coefficients=[4, 1], algorithm="tensor_core", block_m=8, block_n=64, block_k=128,
+                              stages=2, dynamic_rows=False, output_dtype="float16", output_stride=256, packed_k=0,
+                              basis_nonzero=False, split_k=1, tail_m=0, group_m=0, cache_scales=False),
+    "e8p_q4_unpack": dict(N=256, K=512, coefficients=[4, 1], packed_k=64),
     "split_a8": dict(rows=8, K=512, dynamic_rows=True),
     "split_prefill_a8": dict(rows=8, K=512, dynamic_rows=False),
     "split_routed_prefill_a8": dict(rows=64, K=512, experts=8, block_m=16, dynamic_rows=True),

@@ -1135,3 +1135,56 @@ def test_diagnostic_probes_run_and_leave_their_inputs_alone():
         gu.kernel("lds_lookup_probe", iterations=20, copies=copies)(Out=word)
     gu.sync()
     assert torch.equal(source, before) and int(word.item()) == 5
+
+
+@pytest.mark.parametrize("m,k,block_k,swiglu,planes", [(3, 5120, 512, False, False), (1, 17408, 2048, False, False),
+                                                       (5, 640, 256, True, False), (4, 1152, 1024, True, True),
+                                                       (2, 128, 128, False, False)])
+def test_rotation_in_tiles_gives_the_one_launch_codes(m, k, block_k, swiglu, planes):
+    # kernels/cuda/model/rotation_a8.py:266-365: rotate_activation_tiles then quantize_rotation_tiles
+    rng = np.random.default_rng(orc.SEED + m + k)
+    x = (rng.normal(size=(m, 2 * k if swiglu else k)) * rng.uniform(0.2, 3.0, (m, 1))).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), k)
+    cap = m + 2
+    blocks = (k + block_k - 1) // block_k
+    plane_rows = cap + 1 if planes else 0
+    if planes:  # gate rows, then the up rows as a second plane
+        stacked = np.zeros((cap + plane_rows, k), np.float16)
+        stacked[:m], stacked[plane_rows:plane_rows + m] = x[:, :k], x[:, k:]
+        d_x = gu.dev(stacked)
+    else:
+        d_x = gu.dev(np.concatenate([x, np.zeros((cap - m, x.shape[1]), np.float16)]))
+    rotated = torch.full((cap, k), 9.0, dtype=torch.float16, device=gu.DEV)
+    maxima = torch.full((m, blocks), -1.0, dtype=torch.float32, device=gu.DEV)
+    variant = dict(M=cap, K=k, block_k=block_k, dynamic_rows=True)
+    gu.kernel("rotate_activation_tiles", swiglu=swiglu, plane_rows=plane_rows, **variant)(
+        Maxima=maxima, Rotated=rotated, Signs=gu.dev(signs), X=d_x, m=m)
+    single = torch.empty((m, k), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("rotate_activation", M=m, K=k, swiglu=swiglu)(Signs=gu.dev(signs), X=gu.dev(x), Y=single)
+    assert torch.equal(rotated[:m], single) and bool((rotated[m:] == 9).all())
+    values = np.abs(gu.host(single).astype(np.float32))
+    padded = np.zeros((m, blocks * block_k), np.float32)
+    padded[:, :k] = values
+    np.testing.assert_array_equal(gu.host(maxima), padded.reshape(m, blocks, block_k).max(axis=2))
+    q = torch.full((cap, k), 77, dtype=torch.int8, device=gu.DEV)
+    s = torch.full((cap,), 5.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("quantize_rotation_tiles", **variant)(Maxima=maxima, Q=q, Rotated=rotated, S=s, m=m)
+    want_q = torch.empty((m, k), dtype=torch.int8, device=gu.DEV)
+    want_s = torch.empty((m,), dtype=torch.float16, device=gu.DEV)
+    gu.kernel("rotate_activation_a8", M=m, K=k, swiglu=swiglu)(Q=want_q, S=want_s, Signs=gu.dev(signs), X=gu.dev(x))
+    assert torch.equal(q[:m], want_q) and torch.equal(s[:m], want_s)
+    assert bool((q[m:] == 77).all()) and bool((s[m:] == 5).all())
+    if not swiglu:
+        oracle_q, oracle_s = orc.rotate_a8(x, signs)
+        np.testing.assert_array_equal(gu.host(q)[:m], oracle_q)
+        np.testing.assert_array_equal(gu.host(s)[:m], oracle_s[:, 0])
+
+
+def test_rotation_tiles_refuse_what_the_reference_refuses():
+    for bad in (dict(block_k=384), dict(K=192), dict(plane_rows=8), dict(swiglu=True, plane_rows=2), dict(threads=256),
+                dict(registers=True, threads=512, block_k=1024), dict(registers=True, threads=96)):
+        with pytest.raises(Exception):
+            gu.kernel("rotate_activation_tiles", **{**dict(M=4, K=1024), **bad})
+    gu.kernel("rotate_activation_tiles", M=4, K=1024, registers=True, threads=256, block_k=1024)
+    with pytest.raises(Exception):
+        gu.kernel("quantize_rotation_tiles", M=4, K=1024, block_k=64)

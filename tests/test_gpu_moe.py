@@ -1158,3 +1158,52 @@ def test_grouped_q2_with_dynamic_rows_takes_m_last(symbol):
     assert (got[rows:] == 55).all()
     with pytest.raises(gu.lib.OrxError):
         kern(**{**args, "m": cap_rows + 1})
+
+
+@pytest.mark.parametrize("m,e,k,block,capacity", [(300, 16, 4, 512, 300), (1, 8, 2, 1024, 1), (700, 64, 10, 2048, 900),
+                                                  (513, 5, 1, 512, 513)])
+def test_segmented_histogram_in_three_launches_gives_expert_histogram(m, e, k, block, capacity):
+    # kernels/cuda/model/moe.py:556-656: per-segment ranks and partial counts, their prefixes, the final slots
+    rng = np.random.default_rng(orc.SEED + m)
+    ids_np = np.stack([rng.choice(e, k, replace=False) for _ in range(m)]).astype(np.int32)
+    want_counts, want_rel = orc.expert_histogram(ids_np, e)
+    segments = (m * k + block - 1) // block
+    ids = torch.full((capacity, k), -1, **I32)
+    ids[:m] = gu.dev(ids_np)
+    partial, offsets = torch.full((e, segments), -3, **I32), torch.full((e, segments), -3, **I32)
+    slots, counts = torch.full((capacity, k), -3, **I32), torch.full((e,), -3, **I32)
+    common = dict(M=capacity, E=e, K=k, block=block, dynamic_rows=capacity != m)
+    live = dict(m=m) if capacity != m else {}
+    gu.kernel("expert_histogram_local", **common)(IDs=ids, Partial=partial, Slots=slots, **live)
+    flat = ids_np.reshape(-1)
+    want_partial = np.stack([[np.count_nonzero(flat[s * block:(s + 1) * block] == x) for s in range(segments)] for x in range(e)])
+    np.testing.assert_array_equal(gu.host(partial), want_partial)
+    local = gu.host(slots)[:m].reshape(-1)
+    for i in (0, m * k // 2, m * k - 1):  # rank of an assignment among those of its expert inside its segment
+        assert local[i] == np.count_nonzero(flat[i // block * block:i] == flat[i])
+    gu.kernel("expert_histogram_offsets", **common)(Counts=counts, Offsets=offsets, Partial=partial, **live)
+    np.testing.assert_array_equal(gu.host(offsets), np.cumsum(want_partial, axis=1) - want_partial)
+    np.testing.assert_array_equal(gu.host(counts), want_counts)
+    gu.kernel("expert_histogram_finish", **common)(IDs=ids, Offsets=offsets, Slots=slots, **live)
+    np.testing.assert_array_equal(gu.host(slots)[:m], want_rel)
+    assert (gu.host(slots)[m:] == -3).all()
+
+
+def test_expand_experts_decodes_the_banks_of_experts_with_rows():
+    # kernels/cuda/model/moe.py:146-173
+    rng = np.random.default_rng(orc.SEED + 8)
+    e, n, k = 5, 128, 512
+    packed = rng.integers(0, 2**32, (e, n, k // 8), dtype=np.uint32)
+    stored = np.stack([orc.q4_pack_k(p, 128) for p in packed])
+    counts = np.array([3, 0, 1, 0, 40], np.int32)
+    out = torch.full((e, n, k), 99, dtype=torch.int8, device=gu.DEV)
+    gu.kernel("expand_experts", N=n, K=k, E=e)(Book=gu.book(), Counts=gu.dev(counts), Out=out, W=gu.dev(stored))
+    got = gu.host(out)
+    for x in range(e):
+        if counts[x]:
+            np.testing.assert_array_equal(got[x], orc.q4_integers(packed[x], TABLE))
+        else:
+            assert (got[x] == 99).all()
+    for bad in (dict(N=100), dict(K=384), dict(E=0), dict(block_n=48)):
+        with pytest.raises(Exception):
+            gu.kernel("expand_experts", **{**dict(N=n, K=k, E=e), **bad})
