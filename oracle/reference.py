@@ -17,6 +17,9 @@ Every function cites the reference file:line it follows.  Pinning status:
                          (row, group) and the word the reference's own test plants
                          (tests/cuda/operators/e8p_selector.py:38); tables with zero
                          coordinates by the scalar decode and the 1 - 2p rule
+* row_q4_integers()      pinned by the reference's own known answer (every signed nibble,
+                         quantization/test_row_q4.py:11-16) and by the byte-permute form of
+                         kernels/cuda/model/q4_projection.py:23-29 emulated on all 65 536 words
 * a8()                   pinned by closed-form edge cases (ties, clamp, floor)
 * project()/rescale()    pinned by brute-force int64 dots and power-of-two KATs
 * router_topk()/metadata pinned by stable argsort / enumeration
@@ -166,6 +169,24 @@ def q2_integers(indices, table, patches=None):
             stored = (word >> 7) & 255
             weights[row, 128 * group + (word & 127)] = stored - 256 if stored > 127 else stored
     return weights
+
+
+ROW_Q4_MAGNITUDES = (3, 10, 19, 31, 46, 67, 93, 127)  # python/orinfer_build/quantization/row_q4.py:15
+
+
+def row_q4_integers(packed, magnitudes=ROW_Q4_MAGNITUDES):
+    """Row-scaled scalar Q4: uint8 (N, K/2), two nibbles per byte, low nibble first -> int8 (N, K).
+
+    python/orinfer_build/quantization/row_q4.py:45-51: weight = magnitudes[nibble & 7], negated for
+    nibbles 8..15.  The kernels bind the same bytes as (N, K/4) u16
+    (kernels/cuda/model/q4_projection.py:66, :165).
+    """
+    packed = np.asarray(packed)
+    if packed.dtype == np.uint16:
+        packed = np.ascontiguousarray(packed).view(np.uint8)
+    codes = np.stack((packed & 15, packed >> 4), axis=-1).reshape(packed.shape[0], -1)
+    values = np.asarray(magnitudes, np.int8)[codes & 7]
+    return np.where(codes < 8, values, -values).astype(np.int8)
 
 
 def q4_pack_k(packed, packed_k):

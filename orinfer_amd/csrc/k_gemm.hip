@@ -18,6 +18,7 @@
 
 #include "e8p_device.h"
 #include "orx_internal.h"
+#include "row_q4_device.h"
 
 namespace orx {
 
@@ -34,6 +35,8 @@ bool gemv_serves_fp16_input(const orx_function& f);
 void stream_geometry(int n, Geometry* g);
 int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
+int stream_row_q4_launch(const int8_t* a, const void* w, uint32_t magnitudes_low, uint32_t magnitudes_high, const __half* ws,
+                         const __half* as, void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
 bool dense_resident_eligible(int n, int k, int packed_k);
 void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g);
@@ -68,7 +71,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
+enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2, kS4 = 3 };  // kS4: row-scaled scalar Q4 nibbles (q4_projection.py)
 enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4, kWide = 5 };
 enum Flags2 { kNoSplit = 1, kNoExpand = 2 };  // orx_function::flags2 of a projection
 
@@ -100,6 +103,7 @@ struct GemmParams {
     const uint16_t* patch;         // (E, K/128, N) patch words or null
     int book_stride;               // selector words between the experts' tables (0: one table for all)
     int direct_rows;               // > 0: no tile list; expert blockIdx.z owns rows [z * direct_rows, (z + 1) * direct_rows)
+    uint32_t magnitudes_low, magnitudes_high;  // scalar Q4: the eight magnitudes, one per byte
 };
 
 template <int CODEC>
@@ -114,11 +118,15 @@ template <>
 struct Tables<kW8> {
     struct type {};
 };
+template <>
+struct Tables<kS4> {
+    struct type {};
+};
 
 // Number of 16-byte global chunks of weight stream per output row per K step.
 template <int CODEC>
 __host__ __device__ constexpr int weight_chunks() {
-    return CODEC == kQ4 ? 4 : CODEC == kQ2 ? 2 : 8;
+    return CODEC == kQ4 || CODEC == kS4 ? 4 : CODEC == kQ2 ? 2 : 8;
 }
 
 // SWIGLU (W8 only): the tile's 128 weight rows are 64 Gate channels followed by the same 64 Up channels,
@@ -179,7 +187,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         rows_here = min(BM, p.m - row0);
     }
 
-    if constexpr (CODEC != kW8) build_tables(tables, book, tid, 256);
+    if constexpr (CODEC == kQ4 || CODEC == kQ2) build_tables(tables, book, tid, 256);
 
     // int8 weights may end in half a K step (K a multiple of 64, int8_projection.py:29): the missing halves of
     // both operands are zeros.  Codes always come in whole steps.
@@ -240,6 +248,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             const int nn = c / PER_ROW, q = c % PER_ROW;
             if constexpr (CODEC == kW8) {
                 *reinterpret_cast<v4u*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
+            } else if constexpr (CODEC == kS4) {
+                // 64 nibbles -> 32 weights at k offset q*32
+                const uint32_t in[4] = {reg_w[i].x, reg_w[i].y, reg_w[i].z, reg_w[i].w};
+                uint32_t out[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    out[2 * j] = decode_row_q4(in[j], p.magnitudes_low, p.magnitudes_high);
+                    out[2 * j + 1] = decode_row_q4(in[j] >> 16, p.magnitudes_low, p.magnitudes_high);
+                }
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 32);
+                dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
+                dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
             } else if constexpr (CODEC == kQ4) {
                 // 4 u32 codes -> 32 weights at k offset q*32
                 const uint2 d0 = decode_q4(tables, reg_w[i].x), d1 = decode_q4(tables, reg_w[i].y);
@@ -427,6 +447,18 @@ __global__ __launch_bounds__(256) void gemm_split_kernel(GemmParams p) {
             const int nn = c / PER_ROW, q = c % PER_ROW;
             if constexpr (CODEC == kW8) {
                 *reinterpret_cast<v4u*>(lds_w + nn * kPitch + q * 16) = reg_w[i];
+            } else if constexpr (CODEC == kS4) {
+                // 64 nibbles -> 32 weights at k offset q*32
+                const uint32_t in[4] = {reg_w[i].x, reg_w[i].y, reg_w[i].z, reg_w[i].w};
+                uint32_t out[8];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    out[2 * j] = decode_row_q4(in[j], p.magnitudes_low, p.magnitudes_high);
+                    out[2 * j + 1] = decode_row_q4(in[j] >> 16, p.magnitudes_low, p.magnitudes_high);
+                }
+                uint4* dst = reinterpret_cast<uint4*>(lds_w + nn * kPitch + q * 32);
+                dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
+                dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
             } else if constexpr (CODEC == kQ4) {
                 // 4 u32 codes -> 32 weights at k offset q*32
                 const uint2 d0 = decode_q4(tables, reg_w[i].x), d1 = decode_q4(tables, reg_w[i].y);
@@ -1053,6 +1085,214 @@ int make_w8_projection(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// ---- row-scaled scalar Q4 (kernels/cuda/model/q4_projection.py; python/orinfer_build/quantization/row_q4.py) ----
+// W is (N, K/4) u16: four nibbles per word, weight = +-magnitudes[nibble & 7], negative when bit 3 is set.  Same
+// activations, accumulation and rescale as every other projection.  Up to 64 rows the weight-streaming kernel
+// reads the nibbles once; above, the 128-wide MFMA tiles decode them into LDS; from 512 rows with a Workspace they
+// are decoded once per launch and the int8 256 x 256 kernel runs.
+// slots used: M/capacity, N, K, stride, out_f32, H (magnitudes 0-3 as bytes), group (magnitudes 4-7)
+__global__ __launch_bounds__(256) void row_q4_unpack_kernel(const uint32_t* __restrict__ w, uint2* __restrict__ out,
+                                                            int64_t pairs, uint32_t low, uint32_t high) {
+    // one u32 = two words = eight weights
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pairs; i += (int64_t)gridDim.x * 256) {
+        const uint32_t v = w[i];
+        out[i] = make_uint2(decode_row_q4(v, low, high), decode_row_q4(v >> 16, low, high));
+    }
+}
+
+int row_q4_unpack(const void* w, void* out, int n, int k, uint32_t low, uint32_t high, hipStream_t stream) {
+    const int64_t pairs = (int64_t)n * (k / 8);
+    const int blocks = (int)std::min<int64_t>((pairs + 255) / 256, 4096);
+    hipLaunchKernelGGL(row_q4_unpack_kernel, dim3(blocks), dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(w),
+                       reinterpret_cast<uint2*>(out), pairs, low, high);
+    return hip_check(hipGetLastError(), "launch unpack_q4");
+}
+
+constexpr int kRowQ4BigRows = 512;
+bool row_q4_expands(const orx_function& f, int rows) { return f.takes_workspace && rows >= kRowQ4BigRows; }
+
+uint64_t row_q4_workspace(const orx_function& f, int rows) {
+    return (rows == 0 ? f.capacity >= kRowQ4BigRows : row_q4_expands(f, rows)) ? (uint64_t)f.N * f.K : 0;
+}
+
+int row_q4_geometry(const orx_function& f, int rows, Geometry* g) {
+    if (rows <= 64) {
+        stream_geometry(f.N, g);
+        return ORX_OK;
+    }
+    if (row_q4_expands(f, rows)) {
+        gemm_big_geometry(rows, f.N, false, g);
+        return ORX_OK;
+    }
+    g->grid[0] = ceil_div((uint32_t)f.N, 128u);
+    g->grid[1] = ceil_div((uint32_t)rows, 128u);
+    g->block[0] = 256;
+    g->shared = 0;
+    return ORX_OK;
+}
+
+// A, AS, Out, S, W[, Workspace][, m]   (crates/orinfer-models/src/flash_next/q4.rs:176-196 binds A, AS, Out, S, W)
+int row_q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    GemmParams p = {};
+    p.a = pointer_arg<const int8_t>(args, 0);
+    p.as = pointer_arg<const __half>(args, 1);
+    p.out = pointer_arg<void>(args, 2);
+    p.ws = pointer_arg<const __half>(args, 3);
+    p.w = pointer_arg<const void>(args, 4);
+    p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.out_f32 = f.out_f32;
+    p.magnitudes_low = (uint32_t)f.H, p.magnitudes_high = (uint32_t)f.group;
+    if (rows <= 64)
+        return stream_row_q4_launch(p.a, p.w, p.magnitudes_low, p.magnitudes_high, p.ws, p.as, p.out, rows, f.N, f.K, f.stride,
+                                    f.out_f32, stream);
+    if (row_q4_expands(f, rows)) {
+        void* workspace = pointer_arg<void>(args, f.workspace_arg);
+        const int code = row_q4_unpack(p.w, workspace, f.N, f.K, p.magnitudes_low, p.magnitudes_high, stream);
+        if (code != ORX_OK) return code;
+        return gemm_big_launch(false, p.a, workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
+                               stream);
+    }
+    hipLaunchKernelGGL((gemm_kernel<kS4, 128, 128, 2, false>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, p);
+    return hip_check(hipGetLastError(), "launch scalar Q4 projection (mfma)");
+}
+
+// `magnitudes`: eight strictly increasing integers in 1..127 (q4_projection.py:17-21)
+bool row_q4_magnitudes(const Variant& v, const char* symbol, uint32_t* low, uint32_t* high) {
+    bool bad = false;
+    std::string given = v.string("magnitudes", "3,10,19,31,46,67,93,127", &bad);
+    int values[8], count = 0, previous = 0;
+    bool ok = !bad;
+    size_t at = 0;
+    while (ok && at <= given.size() && count < 9) {
+        size_t end = given.find(',', at);
+        if (end == std::string::npos) end = given.size();
+        const std::string piece = given.substr(at, end - at);
+        char* rest = nullptr;
+        const long value = strtol(piece.c_str(), &rest, 10);
+        if (piece.empty() || rest == piece.c_str() || value <= previous || value > 127 || count == 8) ok = false;
+        while (ok && *rest == ' ') ++rest;
+        if (ok && *rest != 0) ok = false;
+        if (ok) values[count++] = previous = (int)value;
+        at = end + 1;
+        if (end == given.size()) break;
+    }
+    if (!ok || count != 8) {
+        set_error("%s: magnitudes are eight strictly increasing integers in 1..127", symbol);
+        return false;
+    }
+    *low = *high = 0;
+    for (int i = 0; i < 4; ++i) *low |= (uint32_t)values[i] << (8 * i), *high |= (uint32_t)values[4 + i] << (8 * i);
+    return true;
+}
+
+bool row_q4_shape(const char* symbol, orx_function* f) {
+    // q4_projection.py:32-35: block-128 geometry, the int32 accumulator holds a whole row
+    if (f->M > 0 && f->N > 0 && f->K > 0 && f->K % 128 == 0 && (int64_t)f->K * 128 * 127 <= 2147483647ll) return true;
+    set_error("%s: need M, N, K > 0, K a multiple of 128 and K * 128 * 127 < 2^31", symbol);
+    return false;
+}
+
+int finish_row_q4(const Variant& v, orx_function* f, const std::string& dtype) {
+    const char* symbol = f->symbol.c_str();
+    uint32_t low, high;
+    if (!row_q4_shape(symbol, f) || !row_q4_magnitudes(v, symbol, &low, &high)) return ORX_ERR_BAD_VARIANT;
+    if (dtype != "float16" && dtype != "float32") {
+        set_error("%s: output_dtype must be float16 or float32", symbol);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->stride < f->N) {
+        set_error("%s: output_stride must hold a whole row", symbol);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->capacity = f->M;
+    f->out_f32 = dtype == "float32";
+    f->H = (int)low, f->group = (int)high;
+    f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Out", ArgPointer, f->out_f32 ? 4u : 2u}, {"S", ArgPointer, 2},
+               {"W", ArgPointer, 16}};
+    if (f->takes_workspace) {
+        f->workspace_arg = (int)f->args.size();
+        f->args.push_back({"Workspace", ArgPointer, 256u | 0x80000000u});
+        f->workspace_need = row_q4_workspace;
+    }
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->device_function = nullptr;  // several kernels serve the symbol
+    f->geometry = row_q4_geometry;
+    f->launch = row_q4_launch;
+    return ORX_OK;
+}
+
+// q4_projection (q4_projection.py:125-183)
+int make_row_q4_projection(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    const int bn = (int)v.integer("BN", 64, &bad), bk = (int)v.integer("BK", 128, &bad);
+    const std::string dtype = v.string("output_dtype", "float16", &bad);
+    const int block_m = (int)v.integer("block_m", 8, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const int stages = (int)v.integer("stages", 2, &bad);
+    f->stride = (int)v.integer("output_stride", f->N, &bad);
+    const int tail_m = (int)v.integer("tail_m", 0, &bad), group_m = (int)v.integer("group_m", 0, &bad);
+    f->takes_workspace = v.boolean("workspace", false, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // tile choices of the reference's kernel, checked as it checks them (q4_projection.py:142-150); the row count picks here
+    if ((bn != 32 && bn != 64 && bn != 128) || bk <= 0 || bk % 128 || (f->K > 0 && f->K % bk) ||
+        (block_m != 8 && block_m != 16 && block_m != 32 && block_m != 64 && block_m != 128) || (stages != 1 && stages != 2) ||
+        (group_m != 0 && group_m != 1 && group_m != 2 && group_m != 4 && group_m != 8) || tail_m < 0) {
+        set_error("q4_projection: BN 32|64|128, BK a multiple of 128 that divides K, block_m 8..128, stages 1|2, group_m 0|1|2|4|8");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    return finish_row_q4(v, f, dtype);
+}
+
+// q4_gemv (q4_projection.py:38-78): the reference's DP4A form for tiles of up to 8 rows; A is the same bytes read as int32
+int make_row_q4_gemv(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->M = (int)v.integer("M", 0, &bad);
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    const int bn = (int)v.integer("BN", 16, &bad);
+    const std::string dtype = v.string("output_dtype", "float16", &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const int block_m = (int)v.integer("block_m", std::max(1, std::min(f->M, 8)), &bad);
+    f->stride = (int)v.integer("output_stride", f->N, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    if (block_m < 1 || block_m > 8 || (bn != 4 && bn != 8 && bn != 16)) {  // q4_projection.py:53-54
+        set_error("q4_gemv: block_m 1..8 and BN 4, 8 or 16");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    return finish_row_q4(v, f, dtype);
+}
+
+// unpack_q4 (q4_projection.py:186-213): Output, W.  slots used: N, K, H, group
+int row_q4_unpack_geometry(const orx_function& f, int rows, Geometry* g) {
+    (void)rows;
+    g->grid[0] = (uint32_t)std::min<int64_t>(((int64_t)f.N * (f.K / 8) + 255) / 256, 4096);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int row_q4_unpack_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
+    (void)rows, (void)g;
+    return row_q4_unpack(pointer_arg<const void>(args, 1), pointer_arg<void>(args, 0), f.N, f.K, (uint32_t)f.H, (uint32_t)f.group,
+                         stream);
+}
+int make_row_q4_unpack(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->N = (int)v.integer("N", 0, &bad);
+    f->K = (int)v.integer("K", 0, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    f->M = 1;
+    uint32_t low, high;
+    if (!row_q4_shape("unpack_q4", f) || !row_q4_magnitudes(v, "unpack_q4", &low, &high)) return ORX_ERR_BAD_VARIANT;
+    f->capacity = 1;
+    f->H = (int)low, f->group = (int)high;
+    f->args = {{"Output", ArgPointer, 8}, {"W", ArgPointer, 4}};
+    f->geometry = row_q4_unpack_geometry;
+    f->launch = row_q4_unpack_launch;
+    f->device_function = reinterpret_cast<const void*>(&row_q4_unpack_kernel);
+    return ORX_OK;
+}
+
 // kernels/cuda/model/int8_projection.py:65-107: the reference's DP4A form for up to 8-row tiles.  Same
 // buffers and arithmetic as int8_projection; here the row count picks the kernel, so the tile hints
 // are checked as the reference checks them and dropped.
@@ -1598,6 +1838,14 @@ const Registration* gemm_registrations(int* count) {
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
+    {"q4_projection", make_row_q4_projection,
+     "M, N, K, BN=64, BK=128, output_dtype=float16|float32, magnitudes=[3,10,19,31,46,67,93,127], block_m=8, dynamic_rows=false, "
+     "stages=2, output_stride=N, tail_m=0, group_m=0, workspace=false",
+     "A,AS,Out,S,W[,Workspace][,m]"},
+    {"q4_gemv", make_row_q4_gemv,
+     "M, N, K, BN=16, output_dtype=float16|float32, magnitudes=[...], dynamic_rows=false, block_m=min(M,8), output_stride=N",
+     "A,AS,Out,S,W[,m]"},
+    {"unpack_q4", make_row_q4_unpack, "N, K, magnitudes=[3,10,19,31,46,67,93,127]", "Output,W"},
     {"expand_experts", make_expand_experts, "N, K, E, block_n=64, block_k=256", "Book,Counts,Out,W"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));

@@ -19,6 +19,7 @@
 
 #include "e8p_device.h"
 #include "orx_internal.h"
+#include "row_q4_device.h"
 
 namespace orx {
 namespace {
@@ -26,7 +27,7 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2 };
+enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2, kS4 = 3 };  // kS4: row-scaled scalar Q4 nibbles
 
 struct StreamParams {
     const int8_t* a;
@@ -45,6 +46,7 @@ struct StreamParams {
     const int* tile_row;
     const int* tile_count;
     int64_t expert_weight_stride;  // bytes between experts in w
+    uint32_t magnitudes_low, magnitudes_high;  // scalar Q4: the eight magnitudes, one per byte
 };
 
 template <int CODEC>
@@ -59,6 +61,10 @@ template <>
 struct StreamTables<kW8> {
     struct type {};
 };
+template <>
+struct StreamTables<kS4> {
+    struct type {};
+};
 
 constexpr int kWaves = 8;             // waves per workgroup
 constexpr int kThreads = kWaves * 64;
@@ -66,7 +72,7 @@ constexpr int kThreads = kWaves * 64;
 // bytes of weight stream per output row per 128-wide K block
 template <int CODEC>
 __host__ __device__ constexpr int block_bytes() {
-    return CODEC == kQ4 ? 64 : CODEC == kQ2 ? 32 : 128;
+    return CODEC == kQ4 || CODEC == kS4 ? 64 : CODEC == kQ2 ? 32 : 128;
 }
 
 // CB = column blocks of 32 token rows (1 or 2); SPLITS = waves that share one group of 32 output
@@ -100,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         ws += (int64_t)expert * p.n;
     }
 
-    if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, kThreads);
+    if constexpr (CODEC == kQ4 || CODEC == kQ2) build_tables(tables, p.book, tid, kThreads);
 
     // K blocks of this wave
     const int k_blocks = p.k / 128;
@@ -114,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
     constexpr int LOADS = LANE_BYTES / 16;      // 16-byte loads per K block: Q4 2, Q2 1, W8 4
     auto weight_pointer = [&](int kb) -> const uint4* {
         int64_t byte;
-        if (CODEC == kW8 || p.packed_k == 0)
+        if (CODEC == kW8 || CODEC == kS4 || p.packed_k == 0)
             byte = ((int64_t)w_row * k_blocks + kb) * BB + half * LANE_BYTES;
         else if (p.packed_k == 64)  // two-stage codes in 64-wide K blocks: this lane's half is one block row
             byte = ((int64_t)(kb * 2 + half) * p.n + w_row) * LANE_BYTES;
@@ -175,6 +181,16 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
                 const uint2 lo = decode_q2(tables, c[s] & 0xFFFFu), hi = decode_q2(tables, c[s] >> 16);
                 wf[s] = make_uint4(lo.x, lo.y, hi.x, hi.y);
             }
+        } else if constexpr (CODEC == kS4) {
+            // a lane's 32 bytes are 64 nibbles: 16 weights per fragment are one 8-byte run
+            const uint32_t c[8] = {codes[0].x, codes[0].y, codes[0].z, codes[0].w,
+                                   codes[1].x, codes[1].y, codes[1].z, codes[1].w};
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                wf[s] = make_uint4(decode_row_q4(c[2 * s], p.magnitudes_low, p.magnitudes_high),
+                                   decode_row_q4(c[2 * s] >> 16, p.magnitudes_low, p.magnitudes_high),
+                                   decode_row_q4(c[2 * s + 1], p.magnitudes_low, p.magnitudes_high),
+                                   decode_row_q4(c[2 * s + 1] >> 16, p.magnitudes_low, p.magnitudes_high));
         } else {
 #pragma unroll
             for (int s = 0; s < 4; ++s) wf[s] = codes[s];
@@ -250,6 +266,18 @@ int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* boo
     if (codec == kQ4) return launch_codec<kQ4, false, kDenseSplits>(cb, p, grid, stream);
     if (codec == kQ2) return launch_codec<kQ2, false, kDenseSplits>(cb, p, grid, stream);
     return launch_codec<kW8, false, kDenseSplits>(cb, p, grid, stream);
+}
+
+// Row-scaled scalar Q4 (kernels/cuda/model/q4_projection.py): W is (N, K/4) u16, rows <= 64
+int stream_row_q4_launch(const int8_t* a, const void* w, uint32_t magnitudes_low, uint32_t magnitudes_high, const __half* ws,
+                         const __half* as, void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream) {
+    StreamParams p = {};
+    p.a = a, p.w = w, p.ws = ws, p.as = as, p.out = out;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32;
+    p.magnitudes_low = magnitudes_low, p.magnitudes_high = magnitudes_high;
+    Geometry g;
+    stream_geometry(n, &g);
+    return launch_codec<kS4, false, kDenseSplits>(rows <= 32 ? 1 : 2, p, dim3(g.grid[0]), stream);
 }
 
 // Routed single-stage experts: one tile = (expert, first row, count <= block_m), block_m 32 or 64.

@@ -16,7 +16,7 @@ def kernel(symbol, **variant):
     # the split-tile and decode-once launches are what the tests run (workspace=False asks for the rest)
     if symbol in WORKSPACE_SYMBOLS:
         variant.setdefault("workspace", True)
-    key = (symbol, tuple(sorted(variant.items())))
+    key = (symbol, tuple(sorted((k, tuple(v) if isinstance(v, list) else v) for k, v in variant.items())))
     if key not in _cache:
         _cache[key] = lib.Kernel(symbol, **variant)
     return _cache[key]

@@ -573,6 +573,11 @@ REFERENCE_KEYWORDS = {
                               stages=2, dynamic_rows=False, output_dtype="float16", output_stride=256, packed_k=0,
                               basis_nonzero=False, split_k=1, tail_m=0, group_m=0, cache_scales=False),
     "e8p_q4_unpack": dict(N=256, K=512, coefficients=[4, 1], packed_k=64),
+    "q4_projection": dict(M=64, N=256, K=512, BN=64, BK=256, output_dtype="float32", magnitudes=[3, 10, 19, 31, 46, 67, 93, 127],
+                          block_m=16, dynamic_rows=True, stages=1, output_stride=260, tail_m=8, group_m=4),
+    "q4_gemv": dict(M=4, N=256, K=512, BN=8, output_dtype="float16", magnitudes=[1, 2, 3, 4, 5, 6, 7, 8], dynamic_rows=True,
+                    block_m=4, output_stride=256),
+    "unpack_q4": dict(N=256, K=512, magnitudes=[3, 10, 19, 31, 46, 67, 93, 127]),
     "split_a8": dict(rows=8, K=512, dynamic_rows=True),
     "split_prefill_a8": dict(rows=8, K=512, dynamic_rows=False),
     "split_routed_prefill_a8": dict(rows=64, K=512, experts=8, block_m=16, dynamic_rows=True),
@@ -615,3 +620,23 @@ def test_plane_kernels_refuse_what_the_reference_refuses():
     # the exact kernel launches no more tiles than the live rows can fill (e8p_exact.py:76)
     dynamic = lib.Kernel("e8p_exact_grouped", **shape, block_m=8, dynamic_rows=True)
     assert dynamic.geometry(8)[0][1] == 1 + 8 and dynamic.geometry(64)[0][1] == 16
+
+
+def test_scalar_q4_symbols_bind_as_the_reference_does_and_refuse_what_it_refuses():
+    # crates/orinfer-models/src/flash_next/q4.rs:176-196 binds A, AS, Out, S, W; kernels/cuda/model/q4_projection.py:17-35, :53-54, :142-150
+    assert lib.Kernel("q4_projection", M=8, N=256, K=512).arg_names == ["A", "AS", "Out", "S", "W"]
+    assert lib.Kernel("q4_gemv", M=8, N=256, K=512, dynamic_rows=True).arg_names == ["A", "AS", "Out", "S", "W", "m"]
+    big = lib.Kernel("q4_projection", M=1024, N=256, K=512, workspace=True, dynamic_rows=True)
+    assert big.arg_names == ["A", "AS", "Out", "S", "W", "Workspace", "m"]
+    assert big.workspace_bytes() == 256 * 512 and big.workspace_bytes(64) == 0 and big.workspace_bytes(600) == 256 * 512
+    assert lib.Kernel("unpack_q4", N=256, K=512).arg_names == ["Output", "W"]
+    shape = dict(M=8, N=256, K=512)
+    for bad in (dict(magnitudes=[3, 10, 19, 31, 46, 67, 93]), dict(magnitudes=[3, 10, 19, 31, 46, 67, 93, 128]),
+                dict(magnitudes=[0, 10, 19, 31, 46, 67, 93, 127]), dict(magnitudes=[3, 3, 19, 31, 46, 67, 93, 127]),
+                dict(magnitudes=[3, 10, 19, 31, 46, 67, 93, 127, 127]), dict(K=500), dict(K=133120), dict(BN=48), dict(BK=384),
+                dict(block_m=4), dict(stages=3), dict(group_m=3), dict(output_stride=255), dict(output_dtype="bfloat16")):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("q4_projection", **{**shape, **bad})
+    for bad in (dict(block_m=9), dict(BN=32), dict(block_m=0)):
+        with pytest.raises(lib.OrxError):
+            lib.Kernel("q4_gemv", **{**shape, **bad})

@@ -1188,3 +1188,60 @@ def test_rotation_tiles_refuse_what_the_reference_refuses():
     gu.kernel("rotate_activation_tiles", M=4, K=1024, registers=True, threads=256, block_k=1024)
     with pytest.raises(Exception):
         gu.kernel("quantize_rotation_tiles", M=4, K=1024, block_k=64)
+
+
+@pytest.mark.parametrize("m,n,k,symbol", [(3, 333, 640, "q4_projection"), (3, 333, 640, "q4_gemv"), (1, 9728, 2560, "q4_gemv"),
+                                          (33, 200, 1024, "q4_projection"), (64, 129, 256, "q4_projection"),
+                                          (65, 260, 384, "q4_projection"), (130, 1000, 1280, "q4_projection"),
+                                          (700, 300, 512, "q4_projection")])
+def test_scalar_q4_projection_at_every_row_range(m, n, k, symbol):
+    # kernels/cuda/model/q4_projection.py; the check of python/orinfer_build/quantization/check_e8p_q4.py:195-214
+    # (random u16 words, rows in -128..127, unit token scales, fp32 out) plus fp16 with scales, strides and live rows
+    rng = np.random.default_rng(orc.SEED + m + n)
+    words = rng.integers(0, 65536, (n, k // 4), dtype=np.uint16)
+    weights = orc.row_q4_integers(words)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    ws = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    cap, stride = m + 3, n + 5
+    pad = np.concatenate([a, np.zeros((cap - m, k), np.int8)])
+    ones = np.ones(cap, np.float16)
+    extra = {} if symbol == "q4_gemv" else dict(workspace=True)
+    kern = gu.kernel(symbol, M=cap, N=n, K=k, dynamic_rows=True, output_dtype="float32", output_stride=stride, **extra)
+    out = torch.full((cap, stride), -7.0, dtype=torch.float32, device=gu.DEV)
+    args = dict(A=gu.dev(pad), AS=gu.dev(ones), Out=out, S=gu.dev(ws), W=gu.dev(words), m=m)
+    kern(**args)
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:m, :n], orc.project(a, ones[:m], weights, ws, np.float32))
+    assert (got[m:] == -7).all() and (got[:, n:] == -7).all()
+    # unit weight scales: the int32 accumulators themselves
+    args["S"] = gu.dev(np.ones(n, np.float16))
+    kern(**args)
+    np.testing.assert_array_equal(gu.host(out)[:m, :n], (a.astype(np.int64) @ weights.astype(np.int64).T).astype(np.float32))
+    scales = rng.uniform(0.01, 0.03, cap).astype(np.float16)
+    half = torch.full((cap, n), 9.0, dtype=torch.float16, device=gu.DEV)
+    plain = gu.kernel(symbol, M=cap, N=n, K=k, dynamic_rows=True)
+    plain(A=gu.dev(pad), AS=gu.dev(scales), Out=half, S=gu.dev(ws), W=gu.dev(words), m=m)
+    np.testing.assert_array_equal(gu.host(half)[:m], orc.project(a, scales[:m], weights, ws))
+    assert bool((half[m:] == 9).all())
+
+
+def test_scalar_q4_other_magnitudes_extremes_and_unpack():
+    rng = np.random.default_rng(orc.SEED + 77)
+    n, k, m = 160, 512, 5
+    magnitudes = [1, 2, 5, 9, 33, 64, 100, 127]
+    words = rng.integers(0, 65536, (n, k // 4), dtype=np.uint16)
+    words[0] = 0xFFFF  # -127 everywhere
+    words[1] = 0x7777  # +127 everywhere
+    weights = orc.row_q4_integers(words, magnitudes)
+    assert (weights[0] == -127).all() and (weights[1] == 127).all()
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    a[0] = -128
+    out = torch.empty((m, n), dtype=torch.float32, device=gu.DEV)
+    gu.kernel("q4_projection", M=m, N=n, K=k, magnitudes=magnitudes, output_dtype="float32")(
+        A=gu.dev(a), AS=gu.dev(np.ones(m, np.float16)), Out=out, S=gu.dev(np.ones(n, np.float16)), W=gu.dev(words))
+    np.testing.assert_array_equal(gu.host(out), (a.astype(np.int64) @ weights.astype(np.int64).T).astype(np.float32))
+    assert gu.host(out)[0, 0] == 128 * 127 * k
+    unpacked = torch.full((n + 1, k), 55, dtype=torch.int8, device=gu.DEV)
+    gu.kernel("unpack_q4", N=n, K=k, magnitudes=magnitudes)(Output=unpacked, W=gu.dev(words))
+    np.testing.assert_array_equal(gu.host(unpacked)[:n], weights)
+    assert bool((unpacked[n] == 55).all())

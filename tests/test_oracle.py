@@ -827,3 +827,26 @@ def test_dispatch_planes_copies_every_token_to_its_slots():
             np.testing.assert_array_equal(orc.planes_row_major(high)[slot], wh[row])
             assert total[slot] == wt[row] and ds[slot, 0] == scale[row, 0]
             assert offsets[ids[row, rank]] <= slot < offsets[ids[row, rank]] + counts[ids[row, rank]]
+
+
+def test_row_q4_every_signed_nibble_and_the_byte_permute_form():
+    """The reference's known answer (python/orinfer_build/quantization/test_row_q4.py:11-16) and its kernel's decode
+    (kernels/cuda/model/q4_projection.py:23-29: two byte permutes, xor with the sign bytes, + 1 where negative)
+    emulated on every u16 word."""
+    codes = np.tile(np.arange(16, dtype=np.uint8), (1, 8))
+    packed = codes[:, ::2] | (codes[:, 1::2] << 4)
+    expected = np.tile(np.r_[orc.ROW_Q4_MAGNITUDES, -np.asarray(orc.ROW_Q4_MAGNITUDES)], (1, 8))
+    np.testing.assert_array_equal(orc.row_q4_integers(packed), expected)
+    magnitudes = (1, 2, 5, 9, 33, 64, 100, 126)
+    table = np.array(magnitudes, np.uint8)
+    words = np.arange(65536, dtype=np.uint32)
+    selector = words & 0x7777
+    sign_selector = (words >> 1) & 0x4444
+    got = np.empty((65536, 4), np.int64)
+    for i in range(4):
+        value = table[(selector >> (4 * i)) & 7].astype(np.uint32)           # __byte_perm(lo, hi, selector), byte i
+        sign = np.where(((sign_selector >> (4 * i)) & 7) >= 4, 0xFF, 0).astype(np.uint32)  # __byte_perm(0, ~0, ...)
+        byte = ((value ^ sign) + (sign & 1)) & 0xFF
+        got[:, i] = byte.astype(np.uint8).view(np.int8)
+    want = orc.row_q4_integers(words.astype(np.uint16).reshape(-1, 1), magnitudes)
+    np.testing.assert_array_equal(got, want)
