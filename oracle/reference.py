@@ -410,6 +410,16 @@ def router_topk(logits, top_k, renormalize=True):
     return ids, (num / den).astype(np.float32)
 
 
+def router_projection(x, w):
+    """Logits fp32 (m, E) and SharedGate fp16 (m,) = x (m, H) . w (E + 1, H)^T (kernels/cuda/model/moe.py:15-49).
+
+    fp16 operands with fp32 accumulation in the kernels; here the products are summed in float64 and
+    rounded once, and the tests bound the difference by the fp32 rounding of the partial sums.
+    """
+    full = np.asarray(x, np.float16).astype(np.float64) @ np.asarray(w, np.float16).astype(np.float64).T
+    return full[:, :-1].astype(np.float32), full[:, -1].astype(np.float16)
+
+
 def expert_histogram(ids, experts):
     """Counts[E], RelativeSlot[M,k]; assignment order token-major, rank-minor (moe.py:177-210)."""
     ids = np.asarray(ids, np.int32)

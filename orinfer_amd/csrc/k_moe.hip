@@ -110,6 +110,53 @@ __global__ __launch_bounds__(256) void expert_histogram_kernel(const int* __rest
     if (threadIdx.x == 0) counts[expert] = base;
 }
 
+// router_projection (kernels/cuda/model/moe.py:15-49): Logits[m, E] fp32 and SharedGate[m] fp16 = X[m, H] . W[E + 1, H]^T,
+// fp16 operands, fp32 accumulation.  Floating point: the order of the additions is this kernel's own.
+// grid (ceil(m / 32), ceil((E + 1) / 32)), four waves: each takes a quarter of H with v_mfma_f32_32x32x16_f16, operands
+// straight from global memory (a lane reads 16 contiguous bytes of its row), and the quarters are added through LDS.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+__global__ __launch_bounds__(256) void router_projection_kernel(const __half* __restrict__ x, const __half* __restrict__ w,
+                                                                float* __restrict__ logits, __half* __restrict__ shared_gate,
+                                                                int rows, int h, int experts) {
+    __shared__ float partial[3][32][33];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int frag = lane & 31, half = lane >> 5;
+    const int row0 = blockIdx.x * 32, col0 = blockIdx.y * 32;
+    const __half* x_row = x + (int64_t)min(row0 + frag, rows - 1) * h + half * 8;
+    const __half* w_row = w + (int64_t)min(col0 + frag, experts) * h + half * 8;
+    const int steps = h / 16;  // H is a multiple of 128
+    const int first = steps * wave / 4, last = steps * (wave + 1) / 4;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll 4
+    for (int step = first; step < last; ++step) {
+        const v8h a = *reinterpret_cast<const v8h*>(x_row + step * 16);
+        const v8h b = *reinterpret_cast<const v8h*>(w_row + step * 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+    // lane holds column `frag` and rows 8 (r / 4) + 4 half + r % 4
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) partial[wave - 1][8 * (r >> 2) + 4 * half + (r & 3)][frag] = acc[r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    const int col = col0 + frag;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int local = 8 * (r >> 2) + 4 * half + (r & 3), row = row0 + local;
+        const float value = (acc[r] + partial[0][local][frag]) + (partial[1][local][frag] + partial[2][local][frag]);
+        if (row < rows) {
+            if (col < experts)
+                logits[(int64_t)row * experts + col] = value;
+            else if (col == experts)
+                shared_gate[row] = __float2half_rn(value);
+        }
+    }
+}
+
 // ---- the histogram in three launches over segments of the assignment list (kernels/cuda/model/moe.py:556-656) ----
 // local:   grid (segments, E).  Partial[e, s] = assignments of segment s routed to expert e, Slots[i] = rank of
 //          assignment i among those of its expert inside its segment.
@@ -683,6 +730,41 @@ int make_histogram(const Variant& v, orx_function* f) {
     return ORX_OK;
 }
 
+// router_projection: Logits, SharedGate, W, X[, m].  slots used: M, H, E
+int router_projection_geometry(const orx_function& f, int rows, Geometry* g) {
+    g->grid[0] = ceil_div((uint32_t)rows, 32u);
+    g->grid[1] = ceil_div((uint32_t)f.E + 1u, 32u);
+    g->block[0] = 256;
+    return ORX_OK;
+}
+int router_projection_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
+    hipLaunchKernelGGL(router_projection_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s, pointer_arg<const __half>(args, 3),
+                       pointer_arg<const __half>(args, 2), pointer_arg<float>(args, 0), pointer_arg<__half>(args, 1), rows, f.H, f.E);
+    return hip_check(hipGetLastError(), "launch router_projection");
+}
+int make_router_projection(const Variant& v, orx_function* f) {
+    bool bad = false;
+    f->capacity = f->M = (int)v.integer("M", 0, &bad);
+    f->H = (int)v.integer("H", 0, &bad);
+    f->E = (int)v.integer("E", 0, &bad);
+    f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
+    const int bm = (int)v.integer("block_m", 16, &bad), bn = (int)v.integer("block_n", 32, &bad);
+    const int bk = (int)v.integer("block_k", 128, &bad), stages = (int)v.integer("stages", 2, &bad);
+    if (bad) return ORX_ERR_BAD_VARIANT;
+    // moe.py:20-28: tile choices of the reference's kernel, checked as it checks them; H in whole K steps
+    if (f->M <= 0 || f->H <= 0 || f->E <= 0 || (bm != 16 && bm != 32 && bm != 64 && bm != 128) || (bn != 32 && bn != 64 && bn != 128) ||
+        (bk != 128 && bk != 256) || f->H % bk || (stages != 1 && stages != 2)) {
+        set_error("router_projection: need M, H, E > 0, block_m 16..128, block_n 32|64|128, block_k 128|256 dividing H, stages 1|2");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->args = {{"Logits", ArgPointer, 4}, {"SharedGate", ArgPointer, 2}, {"W", ArgPointer, 16}, {"X", ArgPointer, 16}};
+    if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
+    f->geometry = router_projection_geometry;
+    f->launch = router_projection_launch;
+    f->device_function = reinterpret_cast<const void*>(&router_projection_kernel);
+    return ORX_OK;
+}
+
 // expert_histogram_local / _offsets / _finish (moe.py:556-656).  slots used: M, E, top_k (the reference's K), group (block),
 // algorithm (0 local, 1 offsets, 2 finish)
 int segmented_geometry(const orx_function& f, int rows, Geometry* g) {
@@ -1034,6 +1116,8 @@ const Registration* moe_registrations(int* count) {
     static const Registration rows[] = {
     {"router_topk", make_router, "M, E=512, top_k=10, renormalize=true, dynamic_rows=false, quantize_hidden=0",
      "IDs,Logits,Prob[,Q,S,X][,m]"},
+    {"router_projection", make_router_projection, "M, H, E, dynamic_rows=false, block_m=16, block_n=32, block_k=128, stages=2",
+     "Logits,SharedGate,W,X[,m]"},
     {"router_topk_warp", make_router_warp, "M, E, top_k, dynamic_rows=false, warps=4", "IDs,Logits,Prob[,m]"},
     {"expert_histogram", make_histogram, "M, E=512, top_k=10, dynamic_rows=false", "Counts,IDs,RelativeSlot[,m]"},
     {"expert_histogram_local", make_histogram_local, "M, E=512, K=10 (routes per token), block=1024|512|2048, dynamic_rows=false",

@@ -578,6 +578,7 @@ REFERENCE_KEYWORDS = {
     "q4_gemv": dict(M=4, N=256, K=512, BN=8, output_dtype="float16", magnitudes=[1, 2, 3, 4, 5, 6, 7, 8], dynamic_rows=True,
                     block_m=4, output_stride=256),
     "unpack_q4": dict(N=256, K=512, magnitudes=[3, 10, 19, 31, 46, 67, 93, 127]),
+    "router_projection": dict(M=64, H=2048, E=128, dynamic_rows=True, block_m=32, block_n=64, block_k=256, stages=1),
     "split_a8": dict(rows=8, K=512, dynamic_rows=True),
     "split_prefill_a8": dict(rows=8, K=512, dynamic_rows=False),
     "split_routed_prefill_a8": dict(rows=64, K=512, experts=8, block_m=16, dynamic_rows=True),

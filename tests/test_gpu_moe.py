@@ -1207,3 +1207,33 @@ def test_expand_experts_decodes_the_banks_of_experts_with_rows():
     for bad in (dict(N=100), dict(K=384), dict(E=0), dict(block_n=48)):
         with pytest.raises(Exception):
             gu.kernel("expand_experts", **{**dict(N=n, K=k, E=e), **bad})
+
+
+@pytest.mark.parametrize("m,h,e", [(1, 128, 1), (37, 2048, 128), (256, 2048, 128), (130, 2560, 512), (5, 384, 33)])
+def test_router_projection_logits_and_shared_gate(m, h, e):
+    # floating point (fp16 operands, fp32 accumulation): every logit within 2^-15 of the sum of the magnitudes of its
+    # products (H fp32 roundings of partial sums would allow H * 2^-24 of it; H <= 2560 here), the gate within one fp16 step
+    rng = np.random.default_rng(orc.SEED + m + e)
+    x = rng.normal(size=(m, h)).astype(np.float16)
+    w = (rng.normal(size=(e + 1, h)) * 0.05).astype(np.float16)
+    cap = m + 3
+    logits = torch.full((cap, e), 7.0, dtype=torch.float32, device=gu.DEV)
+    gate = torch.full((cap,), 7.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("router_projection", M=cap, H=h, E=e, dynamic_rows=True)(
+        Logits=logits, SharedGate=gate, W=gu.dev(w), X=gu.dev(np.concatenate([x, np.zeros((cap - m, h), np.float16)])), m=m)
+    want_logits, want_gate = orc.router_projection(x, w)
+    bound = (np.abs(x.astype(np.float64)) @ np.abs(w.astype(np.float64)).T) * 2.0 ** -15
+    got = gu.host(logits)
+    assert (np.abs(got[:m].astype(np.float64) - want_logits) <= bound[:, :e] + 1e-30).all()
+    got_gate = gu.host(gate)[:m].astype(np.float64)
+    assert (np.abs(got_gate - want_gate.astype(np.float64)) <= np.abs(want_gate.astype(np.float64)) * 2.0 ** -10 + bound[:, e]).all()
+    assert (got[m:] == 7).all() and (gu.host(gate)[m:] == 7).all()
+    # the ranking that follows is the one of the exact logits wherever they are farther apart than the bound
+    ids = torch.empty((m, min(4, e)), **I32)
+    prob = torch.empty((m, min(4, e)), dtype=torch.float32, device=gu.DEV)
+    gu.kernel("router_topk", M=m, E=e, top_k=min(4, e))(IDs=ids, Logits=logits[:m].contiguous(), Prob=prob)
+    want_ids, _ = orc.router_topk(got[:m], min(4, e))
+    np.testing.assert_array_equal(gu.host(ids), want_ids)
+    for bad in (dict(H=100), dict(block_k=512), dict(block_m=8), dict(stages=3), dict(E=0)):
+        with pytest.raises(Exception):
+            gu.kernel("router_projection", **{**dict(M=4, H=256, E=8), **bad})
