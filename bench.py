@@ -479,6 +479,62 @@ def main():
                                                         "frac_hbm": round(moved / tf / 1e9 / HBM_PEAK_GBS, 4),
                                                         "bytes": moved}
         del x, q, res, res_out, y
+
+        # ---- the reference's other factories on the path, at the same shapes ----
+        # row-scaled scalar Q4 (q4_projection): config 1's matrix as nibbles, six weight copies in rotation
+        rng = np.random.default_rng(11)
+        n4, k4 = c1["n"], c1["k"]
+        nibbles = [dev(rng.integers(0, 65536, (n4, k4 // 4), dtype=np.uint16)) for _ in range(6)]
+        s4 = dev(c1["scales"])
+        scalar = {}
+        for rows in (1, 32, 512):
+            a4 = torch.randint(-127, 128, (rows, k4), dtype=torch.int8, device="cuda")
+            as4 = torch.rand((rows,), dtype=torch.float16, device="cuda") * 0.02 + 0.01
+            o4 = torch.empty((rows, n4), dtype=torch.float16, device="cuda")
+            kern = Kernel("q4_projection", M=rows, N=n4, K=k4, workspace=True)
+            ws4 = kern.workspace()
+            t = timed_graph(lambda i, st: kern(stream=st, A=a4, AS=as4, Out=o4, S=s4, W=nibbles[i % 6], Workspace=ws4), 24)
+            code_bytes = n4 * k4 // 2
+            scalar[str(rows)] = {"us": round(t * 1e6, 2), "weight_GBps": round(code_bytes / t / 1e9, 1),
+                                 "TOPS": round(2 * rows * n4 * k4 / t / 1e12, 1)}
+        extra["scalar_q4_projection_config1_shape"] = scalar
+        del nibbles
+        # nibble planes: config 3's gate_up through split_prefill_a8 + e8p_prefill_grouped (16-row tiles)
+        e3, slots3, h3, n3 = 128, 2048, 2048, 1024
+        ids3 = dev(np.stack([rng.choice(e3, 8, replace=False) for _ in range(256)]).astype(np.int32))
+        cap3 = (slots3 + 15) // 16 + min(e3, slots3)
+        i32 = dict(dtype=torch.int32, device="cuda")
+        counts3, relative3 = torch.zeros((e3,), **i32), torch.zeros((256, 8), **i32)
+        offsets3, tile_offsets3, total3 = torch.zeros((e3,), **i32), torch.zeros((e3,), **i32), torch.zeros((1,), **i32)
+        te3, tr3 = torch.zeros((cap3,), **i32), torch.zeros((cap3,), **i32)
+        Kernel("route_metadata", M=256, E=e3, top_k=8, block_m=16)(
+            Counts=counts3, IDs=ids3, RelativeSlot=relative3, RowOffsets=offsets3, TileCount=total3, TileExpert=te3,
+            TileOffsets=tile_offsets3, TileRow=tr3)
+        a3 = torch.randint(-127, 128, (slots3, h3), dtype=torch.int8, device="cuda")
+        low3 = torch.empty((h3 // 64, slots3, 8), dtype=torch.int32, device="cuda")
+        high3, sum3 = torch.empty_like(low3), torch.empty((slots3,), dtype=torch.int32, device="cuda")
+        split = Kernel("split_prefill_a8", rows=slots3, K=h3)
+        t_split = timed_graph(lambda i, st: split(stream=st, A=a3, High=high3, Low=low3, Sum=sum3), 40)
+        p3 = dev(rng.integers(0, 65536, (e3, h3 // 64, n3, 8), dtype=np.uint16))
+        nib3 = dev(codebook.nibble_book())
+        ws3 = dev(rng.uniform(0.005, 0.02, (e3, n3)).astype(np.float16))
+        as3 = torch.rand((slots3,), dtype=torch.float16, device="cuda") * 0.02 + 0.01
+        o3 = torch.empty((slots3, n3), dtype=torch.float16, device="cuda")
+        grouped = Kernel("e8p_prefill_grouped", rows=slots3, E=e3, tiles=cap3, N=n3, K=h3, block_m=16)
+        routing3 = dict(Counts=counts3, Offsets=offsets3, TC=total3, TE=te3, TR=tr3)
+        t_planes = timed_graph(lambda i, st: grouped(stream=st, AS=as3, Book=nib3, High=high3, Low=low3, Out=o3, P=p3, Sum=sum3,
+                                                     WS=ws3, **routing3), 40)
+        extra["config3_gate_up_on_nibble_planes"] = {"split_prefill_a8_us": round(t_split * 1e6, 2),
+                                                     "e8p_prefill_grouped_us": round(t_planes * 1e6, 2),
+                                                     "tiles_of_16_rows": int(total3.cpu()[0])}
+        # router projection: 256 tokens x 2048 -> 128 logits + the shared expert's gate
+        xr = torch.randn((256, 2048), dtype=torch.float16, device="cuda")
+        wr = torch.randn((129, 2048), dtype=torch.float16, device="cuda") * 0.05
+        lr = torch.empty((256, 128), dtype=torch.float32, device="cuda")
+        gr = torch.empty((256,), dtype=torch.float16, device="cuda")
+        proj = Kernel("router_projection", M=256, H=2048, E=128)
+        t_proj = timed_graph(lambda i, st: proj(stream=st, Logits=lr, SharedGate=gr, W=wr, X=xr), 100)
+        extra["config3_router_projection"] = {"us": round(t_proj * 1e6, 2)}
     result["extra"] = extra
 
     # ---- CPU baseline: the oracle's C restatement on the contract workload, all host cores ----

@@ -48,6 +48,24 @@ def book():
     return selector_table(basis())
 
 
+def nibble_book(table=None):
+    """(1, 256, 1) u32 nibble words, the `Book` of `e8p_exact_grouped` and of `e8p_prefill_grouped` with single-stage
+    codes: nibble i = (t_j / 2) & 15 for j = [0, 2, 1, 3, 4, 6, 5, 7][i] (python/orinfer_build/quantization/vq.py:105-118).
+    Needs a basis without zeros."""
+    t = np.asarray(basis() if table is None else table)
+    if t.dtype != np.int8 or t.shape != (256, 8) or not np.isin(np.abs(t.astype(np.int32)), (2, 6, 10)).all():
+        raise ValueError("the nibble form needs the int8 [256,8] basis with entries of +-2, +-6, +-10")
+    half = (t.astype(np.int32) // 2)[:, [0, 2, 1, 3, 4, 6, 5, 7]] & 15
+    shifts = np.arange(0, 32, 4, dtype=np.uint32)
+    return np.bitwise_or.reduce(half.astype(np.uint32) << shifts, axis=1).astype(np.uint32).reshape(1, 256, 1)
+
+
+def q2_to_k64(blocks):
+    """(E, K/128, N, 16) u16 -> (E, K/64, N, 8): the K-major blocks of 64 the plane kernels read (vq.py:121-128)."""
+    e, g, n, _ = blocks.shape
+    return np.ascontiguousarray(blocks.reshape(e, g, n, 2, 8).transpose(0, 1, 3, 2, 4)).reshape(e, g * 2, n, 8)
+
+
 def raw_book(table=None):
     """The 256 x 8 int8 table as (256, 2) u32 words: the `Book` of the raw-table kernels
     (`integer_e8p_gemv`; python/orinfer_build/quantization/vq.py:203)."""

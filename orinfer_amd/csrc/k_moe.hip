@@ -112,25 +112,26 @@ __global__ __launch_bounds__(256) void expert_histogram_kernel(const int* __rest
 
 // router_projection (kernels/cuda/model/moe.py:15-49): Logits[m, E] fp32 and SharedGate[m] fp16 = X[m, H] . W[E + 1, H]^T,
 // fp16 operands, fp32 accumulation.  Floating point: the order of the additions is this kernel's own.
-// grid (ceil(m / 32), ceil((E + 1) / 32)), four waves: each takes a quarter of H with v_mfma_f32_32x32x16_f16, operands
-// straight from global memory (a lane reads 16 contiguous bytes of its row), and the quarters are added through LDS.
+// grid (ceil(m / 32), ceil((E + 1) / 32)), eight waves: each takes an eighth of H with v_mfma_f32_32x32x16_f16, operands
+// straight from global memory (a lane reads 16 contiguous bytes of its row), and the eighths are added through LDS.
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-__global__ __launch_bounds__(256) void router_projection_kernel(const __half* __restrict__ x, const __half* __restrict__ w,
+constexpr int kProjectionWaves = 8;
+__global__ __launch_bounds__(kProjectionWaves * 64) void router_projection_kernel(const __half* __restrict__ x, const __half* __restrict__ w,
                                                                 float* __restrict__ logits, __half* __restrict__ shared_gate,
                                                                 int rows, int h, int experts) {
-    __shared__ float partial[3][32][33];
+    __shared__ float partial[kProjectionWaves - 1][32][33];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int frag = lane & 31, half = lane >> 5;
     const int row0 = blockIdx.x * 32, col0 = blockIdx.y * 32;
     const __half* x_row = x + (int64_t)min(row0 + frag, rows - 1) * h + half * 8;
     const __half* w_row = w + (int64_t)min(col0 + frag, experts) * h + half * 8;
     const int steps = h / 16;  // H is a multiple of 128
-    const int first = steps * wave / 4, last = steps * (wave + 1) / 4;
+    const int first = steps * wave / kProjectionWaves, last = steps * (wave + 1) / kProjectionWaves;
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll 4
+#pragma unroll 8
     for (int step = first; step < last; ++step) {
         const v8h a = *reinterpret_cast<const v8h*>(x_row + step * 16);
         const v8h b = *reinterpret_cast<const v8h*>(w_row + step * 16);
@@ -147,7 +148,9 @@ __global__ __launch_bounds__(256) void router_projection_kernel(const __half* __
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         const int local = 8 * (r >> 2) + 4 * half + (r & 3), row = row0 + local;
-        const float value = (acc[r] + partial[0][local][frag]) + (partial[1][local][frag] + partial[2][local][frag]);
+        float value = acc[r];
+#pragma unroll
+        for (int other = 0; other < kProjectionWaves - 1; ++other) value += partial[other][local][frag];
         if (row < rows) {
             if (col < experts)
                 logits[(int64_t)row * experts + col] = value;
@@ -734,11 +737,11 @@ int make_histogram(const Variant& v, orx_function* f) {
 int router_projection_geometry(const orx_function& f, int rows, Geometry* g) {
     g->grid[0] = ceil_div((uint32_t)rows, 32u);
     g->grid[1] = ceil_div((uint32_t)f.E + 1u, 32u);
-    g->block[0] = 256;
+    g->block[0] = kProjectionWaves * 64;
     return ORX_OK;
 }
 int router_projection_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(router_projection_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s, pointer_arg<const __half>(args, 3),
+    hipLaunchKernelGGL(router_projection_kernel, dim3(g.grid[0], g.grid[1]), dim3(g.block[0]), 0, s, pointer_arg<const __half>(args, 3),
                        pointer_arg<const __half>(args, 2), pointer_arg<float>(args, 0), pointer_arg<__half>(args, 1), rows, f.H, f.E);
     return hip_check(hipGetLastError(), "launch router_projection");
 }

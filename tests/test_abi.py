@@ -260,6 +260,16 @@ def test_package_codebook_matches_oracle(golden_basis):
     assert np.array_equal(codebook.raw_book(golden_basis[::-1]), ref.raw_table_words(golden_basis[::-1]))
 
 
+def test_package_nibble_book_and_k64_blocks_match_oracle(golden_basis):
+    assert np.array_equal(codebook.nibble_book().reshape(256, 1), ref.nibble_table(ref.selector_table(golden_basis)))
+    raw = np.random.default_rng(3).integers(0, 65536, (2, 3, 5, 16), dtype=np.uint16)
+    assert np.array_equal(codebook.q2_to_k64(raw), ref.q2_repack_k64(raw))
+    zeros = golden_basis.copy()
+    zeros[7, 1] = 0
+    with pytest.raises(ValueError):
+        codebook.nibble_book(zeros)
+
+
 def test_workload_sizes_and_algorithmic_bytes():
     # N*K/2 + 2N + M*K + 2M + 2*M*N + 1024 (Q4) and N*K + 2N + M*K + 2M + 2*M*N (W8)
     assert workloads.algorithmic_bytes_q4(1, 9728, 2560) == 12_494_338
