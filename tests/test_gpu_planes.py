@@ -330,3 +330,51 @@ def test_rotated_planes_into_the_exact_kernel_equal_int8_rows_into_the_int8_kern
     codes = np.ascontiguousarray(raw.transpose(0, 2, 1, 3)).reshape(e, n, h // 8)
     weights = np.stack([orc.q2_integers(c, basis) for c in codes])
     np.testing.assert_array_equal(gu.host(out), orc.grouped_project(want_d, want_ds, weights, ws, counts, offsets))
+
+
+def test_split_then_exact_grouped_replayed_from_a_graph_with_changed_inputs():
+    # the replay sequence of tests/cuda/operators/e8p_exact.py:208-227: zeroed rows, new rows, the first rows again;
+    # the tile list, the counts and Book are read on the device at every replay
+    rng = np.random.default_rng(orc.SEED + 21)
+    basis = orc.basis()
+    bm, counts, n, k = 16, [17, 33], 320, 640
+    e, rows = len(counts), sum(counts)
+    a, raw, codes, ws, scale, weights = grouped_case(rng, counts, n, k, basis)
+    offsets, te, tr, total, cap = tile_list(counts, bm)
+    counts_np = np.asarray(counts, np.int32)
+    d_a = gu.dev(a)
+    low, high = empty_planes(rows, k, False)
+    sums = torch.empty((rows,), **I32)
+    out = torch.empty((rows, n), dtype=torch.float16, device=gu.DEV)
+    d_counts = gu.dev(counts_np)
+    split = gu.kernel("split_a8", rows=rows, K=k)
+    gemm = gu.kernel("e8p_exact_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm)
+    args = dict(AS=gu.dev(scale), Book=gu.dev(orc.nibble_table(orc.selector_table(basis))[None]), Counts=d_counts, High=high,
+                Low=low, Offsets=gu.dev(offsets), Out=out, P=gu.dev(orc.q2_repack_k64(raw)), Sum=sums, TC=gu.dev(total),
+                TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws))
+    split(A=d_a, High=high, Low=low, Sum=sums)
+    gemm(**args)
+    gu.sync()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            split(stream=side.cuda_stream, A=d_a, High=high, Low=low, Sum=sums)
+            gemm(stream=side.cuda_stream, **args)
+    first = a.copy()
+    for rows_now in (np.zeros_like(a), planted_rows(rng, rows, k), first):
+        d_a.copy_(gu.dev(rows_now))
+        out.fill_(float("nan"))
+        gu.sync()
+        graph.replay()
+        gu.sync()
+        np.testing.assert_array_equal(gu.host(out), orc.grouped_project(rows_now, scale[:, None], weights, ws, counts_np, offsets))
+    # an expert that lost its rows between replays is skipped
+    d_counts[0] = 0
+    out.fill_(5.0)
+    gu.sync()
+    graph.replay()
+    gu.sync()
+    got = gu.host(out)
+    assert (got[:counts[0]] == 5).all()
+    np.testing.assert_array_equal(got[counts[0]:], orc.grouped_project(first, scale[:, None], weights, ws, counts_np, offsets)[counts[0]:])
