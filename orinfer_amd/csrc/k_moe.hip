@@ -7,6 +7,8 @@
 // the result is deterministic and every kernel is replayable inside a captured graph.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "a8_device.h"
 #include "moe_device.h"
 #include "orx_internal.h"
@@ -112,42 +114,54 @@ __global__ __launch_bounds__(256) void expert_histogram_kernel(const int* __rest
 
 // router_projection (kernels/cuda/model/moe.py:15-49): Logits[m, E] fp32 and SharedGate[m] fp16 = X[m, H] . W[E + 1, H]^T,
 // fp16 operands, fp32 accumulation.  Floating point: the order of the additions is this kernel's own.
-// grid (ceil(m / 32), ceil((E + 1) / 32)), eight waves: each takes an eighth of H with v_mfma_f32_32x32x16_f16, operands
-// straight from global memory (a lane reads 16 contiguous bytes of its row), and the eighths are added through LDS.
+// grid (ceil(m / T), ceil((E + 1) / T)) with T = 16 up to 1024 rows and 32 above, eight waves: each takes an eighth of H,
+// operands straight from global memory (a lane reads 16 contiguous bytes of its row), the eighths are added through LDS.
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 constexpr int kProjectionWaves = 8;
-__global__ __launch_bounds__(kProjectionWaves * 64) void router_projection_kernel(const __half* __restrict__ x, const __half* __restrict__ w,
-                                                                float* __restrict__ logits, __half* __restrict__ shared_gate,
-                                                                int rows, int h, int experts) {
-    __shared__ float partial[kProjectionWaves - 1][32][33];
+constexpr int kProjectionSmallRows = 1024;  // up to here 16 x 16 tiles: four times the workgroups, each pulls half the rows
+// TILE 32: v_mfma_f32_32x32x16_f16, a lane holds row (lane % 32) and 8 values of k at 8 (lane / 32);
+// TILE 16: v_mfma_f32_16x16x32_f16, a lane holds row (lane % 16) and 8 values of k at 8 (lane / 16).
+template <int TILE>
+__global__ __launch_bounds__(kProjectionWaves * 64) void router_projection_kernel(const __half* __restrict__ x,
+                                                                                  const __half* __restrict__ w,
+                                                                                  float* __restrict__ logits,
+                                                                                  __half* __restrict__ shared_gate, int rows,
+                                                                                  int h, int experts) {
+    constexpr int STEP = TILE == 32 ? 16 : 32, REGS = TILE == 32 ? 16 : 4;
+    __shared__ float partial[kProjectionWaves - 1][TILE][TILE + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int frag = lane & 31, half = lane >> 5;
-    const int row0 = blockIdx.x * 32, col0 = blockIdx.y * 32;
-    const __half* x_row = x + (int64_t)min(row0 + frag, rows - 1) * h + half * 8;
-    const __half* w_row = w + (int64_t)min(col0 + frag, experts) * h + half * 8;
-    const int steps = h / 16;  // H is a multiple of 128
+    const int frag = lane % TILE, piece = lane / TILE;
+    const int row0 = blockIdx.x * TILE, col0 = blockIdx.y * TILE;
+    const __half* x_row = x + (int64_t)min(row0 + frag, rows - 1) * h + piece * 8;
+    const __half* w_row = w + (int64_t)min(col0 + frag, experts) * h + piece * 8;
+    const int steps = h / STEP;  // H is a multiple of 128
     const int first = steps * wave / kProjectionWaves, last = steps * (wave + 1) / kProjectionWaves;
-    v16f acc;
+    typename std::conditional<TILE == 32, v16f, v4f>::type acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    for (int r = 0; r < REGS; ++r) acc[r] = 0.f;
 #pragma unroll 8
     for (int step = first; step < last; ++step) {
-        const v8h a = *reinterpret_cast<const v8h*>(x_row + step * 16);
-        const v8h b = *reinterpret_cast<const v8h*>(w_row + step * 16);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+        const v8h a = *reinterpret_cast<const v8h*>(x_row + step * STEP);
+        const v8h b = *reinterpret_cast<const v8h*>(w_row + step * STEP);
+        if constexpr (TILE == 32)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc, 0, 0, 0);
     }
-    // lane holds column `frag` and rows 8 (r / 4) + 4 half + r % 4
+    // a lane holds column `frag`; TILE 32: rows 8 (r / 4) + 4 piece + r % 4, TILE 16: rows 4 piece + r
+    auto local_row = [&](int r) { return TILE == 32 ? 8 * (r >> 2) + 4 * piece + (r & 3) : 4 * piece + r; };
     if (wave > 0) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) partial[wave - 1][8 * (r >> 2) + 4 * half + (r & 3)][frag] = acc[r];
+        for (int r = 0; r < REGS; ++r) partial[wave - 1][local_row(r)][frag] = acc[r];
     }
     __syncthreads();
     if (wave > 0) return;
     const int col = col0 + frag;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int local = 8 * (r >> 2) + 4 * half + (r & 3), row = row0 + local;
+    for (int r = 0; r < REGS; ++r) {
+        const int local = local_row(r), row = row0 + local;
         float value = acc[r];
 #pragma unroll
         for (int other = 0; other < kProjectionWaves - 1; ++other) value += partial[other][local][frag];
@@ -735,14 +749,21 @@ int make_histogram(const Variant& v, orx_function* f) {
 
 // router_projection: Logits, SharedGate, W, X[, m].  slots used: M, H, E
 int router_projection_geometry(const orx_function& f, int rows, Geometry* g) {
-    g->grid[0] = ceil_div((uint32_t)rows, 32u);
-    g->grid[1] = ceil_div((uint32_t)f.E + 1u, 32u);
+    const uint32_t tile = rows <= kProjectionSmallRows ? 16u : 32u;
+    g->grid[0] = ceil_div((uint32_t)rows, tile);
+    g->grid[1] = ceil_div((uint32_t)f.E + 1u, tile);
     g->block[0] = kProjectionWaves * 64;
     return ORX_OK;
 }
 int router_projection_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(router_projection_kernel, dim3(g.grid[0], g.grid[1]), dim3(g.block[0]), 0, s, pointer_arg<const __half>(args, 3),
-                       pointer_arg<const __half>(args, 2), pointer_arg<float>(args, 0), pointer_arg<__half>(args, 1), rows, f.H, f.E);
+    const dim3 grid(g.grid[0], g.grid[1]), block(g.block[0]);
+    const __half *x = pointer_arg<const __half>(args, 3), *w = pointer_arg<const __half>(args, 2);
+    float* logits = pointer_arg<float>(args, 0);
+    __half* gate = pointer_arg<__half>(args, 1);
+    if (rows <= kProjectionSmallRows)
+        hipLaunchKernelGGL(router_projection_kernel<16>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
+    else
+        hipLaunchKernelGGL(router_projection_kernel<32>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
     return hip_check(hipGetLastError(), "launch router_projection");
 }
 int make_router_projection(const Variant& v, orx_function* f) {
@@ -764,7 +785,7 @@ int make_router_projection(const Variant& v, orx_function* f) {
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
     f->geometry = router_projection_geometry;
     f->launch = router_projection_launch;
-    f->device_function = reinterpret_cast<const void*>(&router_projection_kernel);
+    f->device_function = reinterpret_cast<const void*>(&router_projection_kernel<32>);
     return ORX_OK;
 }
 
