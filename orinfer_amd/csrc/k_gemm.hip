@@ -37,6 +37,11 @@ int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* boo
                   void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, hipStream_t stream);
 int stream_row_q4_launch(const int8_t* a, const void* w, uint32_t magnitudes_low, uint32_t magnitudes_high, const __half* ws,
                          const __half* as, void* out, int rows, int n, int k, int stride, bool out_f32, hipStream_t stream);
+// from k_rowq4.hip
+bool row_q4_gemv_serves(int rows, int k);
+void row_q4_gemv_geometry(int rows, int n, int k, Geometry* g);
+int row_q4_gemv_launch(const int8_t* a, const void* w, uint32_t low, uint32_t high, const __half* ws, const __half* as, void* out,
+                       int rows, int n, int k, int stride, bool out_f32, const Geometry& g, hipStream_t stream);
 void stream_grouped_geometry(int n, int tiles, Geometry* g);
 bool dense_resident_eligible(int n, int k, int packed_k);
 void dense_resident_geometry(int rows, int n, int k, int packed_k, Geometry* g);
@@ -1087,8 +1092,8 @@ int make_w8_projection(const Variant& v, orx_function* f) {
 
 // ---- row-scaled scalar Q4 (kernels/cuda/model/q4_projection.py; python/orinfer_build/quantization/row_q4.py) ----
 // W is (N, K/4) u16: four nibbles per word, weight = +-magnitudes[nibble & 7], negative when bit 3 is set.  Same
-// activations, accumulation and rescale as every other projection.  Up to 64 rows the weight-streaming kernel
-// reads the nibbles once; above, the 128-wide MFMA tiles decode them into LDS; from 512 rows with a Workspace they
+// activations, accumulation and rescale as every other projection.  One or two rows: a streaming GEMV (k_rowq4.hip);
+// up to 64 rows the weight-streaming MFMA kernel reads the nibbles once; above, the 128-wide MFMA tiles decode them into LDS; from 512 rows with a Workspace they
 // are decoded once per launch and the int8 256 x 256 kernel runs.
 // slots used: M/capacity, N, K, stride, out_f32, H (magnitudes 0-3 as bytes), group (magnitudes 4-7)
 __global__ __launch_bounds__(256) void row_q4_unpack_kernel(const uint32_t* __restrict__ w, uint2* __restrict__ out,
@@ -1116,6 +1121,10 @@ uint64_t row_q4_workspace(const orx_function& f, int rows) {
 }
 
 int row_q4_geometry(const orx_function& f, int rows, Geometry* g) {
+    if (row_q4_gemv_serves(rows, f.K)) {
+        row_q4_gemv_geometry(rows, f.N, f.K, g);
+        return ORX_OK;
+    }
     if (rows <= 64) {
         stream_geometry(f.N, g);
         return ORX_OK;
@@ -1141,6 +1150,9 @@ int row_q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
     p.w = pointer_arg<const void>(args, 4);
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.out_f32 = f.out_f32;
     p.magnitudes_low = (uint32_t)f.H, p.magnitudes_high = (uint32_t)f.group;
+    if (row_q4_gemv_serves(rows, f.K))
+        return row_q4_gemv_launch(p.a, p.w, p.magnitudes_low, p.magnitudes_high, p.ws, p.as, p.out, rows, f.N, f.K, f.stride,
+                                  f.out_f32, g, stream);
     if (rows <= 64)
         return stream_row_q4_launch(p.a, p.w, p.magnitudes_low, p.magnitudes_high, p.ws, p.as, p.out, rows, f.N, f.K, f.stride,
                                     f.out_f32, stream);

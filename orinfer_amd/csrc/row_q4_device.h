@@ -18,4 +18,11 @@ __device__ __forceinline__ uint32_t decode_row_q4(uint32_t word, uint32_t low, u
     return (magnitude ^ negative) + (negative & 0x01010101u);
 }
 
+// Four nibbles already spread one per byte (bits 0-3 of every byte) -> four int8 weights.
+__device__ __forceinline__ uint32_t decode_row_q4_bytes(uint32_t x, uint32_t low, uint32_t high) {
+    const uint32_t magnitude = __builtin_amdgcn_perm(high, low, x & 0x07070707u);
+    const uint32_t sign = (x >> 3) & 0x01010101u;
+    return (magnitude ^ (sign * 0xFFu)) + sign;
+}
+
 }  // namespace orx
