@@ -1191,6 +1191,7 @@ def test_rotation_tiles_refuse_what_the_reference_refuses():
 
 
 @pytest.mark.parametrize("m,n,k,symbol", [(3, 333, 640, "q4_projection"), (3, 333, 640, "q4_gemv"), (1, 9728, 2560, "q4_gemv"),
+                                          (2, 333, 640, "q4_gemv"), (1, 129, 128, "q4_projection"), (2, 5000, 3200, "q4_projection"),
                                           (33, 200, 1024, "q4_projection"), (64, 129, 256, "q4_projection"),
                                           (65, 260, 384, "q4_projection"), (130, 1000, 1280, "q4_projection"),
                                           (700, 300, 512, "q4_projection")])
