@@ -226,6 +226,58 @@ __device__ __forceinline__ int64_t q4_k_major_chunk(int packed_k, int n, int row
     return ((int64_t)(kt * 2 + (q >> 1)) * n + row) * 32 + (q & 1) * 16;
 }
 
+// ---- y = (w - 1) / 2 as bytes, from the reference's nibble words (quantization/vq.py:105-118) ----------------
+// sign-extends the four nibbles at bits 0-3 of every byte
+__device__ __forceinline__ uint32_t extend_nibbles(uint32_t t) { return t | ((t & 0x08080808u) * 0x1Eu); }
+
+// bytewise a + b of signed bytes whose sums fit a byte
+__device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
+    return ((a & 0x7F7F7F7Fu) + (b & 0x7F7F7F7Fu)) ^ ((a ^ b) & 0x80808080u);
+}
+
+// Tables of the INT4-exact expert kernels' decode (kernels/cuda/model/e8p_core.py:7-10, 45-60), one entry per thread
+// for threads 0..255.  `value[b]`: y of basis row b at even parity without sign bits; `change[u]`: what a code's low byte
+// u changes in it (a coordinate's sign bit negates its nibble: the stored values are odd, so xor 0xe; odd parity lowers
+// every nibble by one, xor 1, and flips the first coordinate's sign too).  Both as sign-extended bytes, the even nibbles
+// of the reference's word (coordinates 0, 1, 4, 5) in .x and the odd ones (2, 3, 6, 7) in .y: sign extension commutes
+// with xor, so a code decodes with two 8-byte lookups and two xors.  `selector_form`: Book holds selector words.
+__device__ __forceinline__ void build_half_tables(uint2* value, uint2* change, const uint32_t* book, bool selector_form, int entry) {
+    uint32_t word = book[entry];
+    if (selector_form) {
+        uint32_t nibbles = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int coordinate = (i & 4) | ((i & 1) << 1) | ((i & 2) >> 1);
+            nibbles |= ((uint32_t)selector_half(word, coordinate) & 15u) << (4 * i);
+        }
+        word = nibbles;
+    }
+    value[entry] = make_uint2(extend_nibbles(word & 0x0F0F0F0Fu), extend_nibbles((word >> 4) & 0x0F0F0F0Fu));
+    const uint32_t u = (uint32_t)entry, parity = __popc(u) & 1u;
+    const uint32_t bits = (u & 0x03u) | ((u & 0x30u) >> 2) | ((u & 0x0Cu) << 2) | (u & 0xC0u);  // nibble i <- sign bit
+    uint32_t spread = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) spread |= ((bits >> i) & 1u) << (4 * i + 1);
+    const uint32_t flip = (spread * 7u) ^ (parity * 0x1111111Fu);
+    change[entry] = make_uint2(extend_nibbles(flip & 0x0F0F0F0Fu), extend_nibbles((flip >> 4) & 0x0F0F0F0Fu));
+}
+
+__device__ __forceinline__ uint2 decode_half(const uint2* value, const uint2* change, uint32_t code) {
+    const uint2 v = value[(code >> 8) & 255u], c = change[code & 255u];
+    return make_uint2(v.x ^ c.x, v.y ^ c.y);
+}
+
+// two-stage code: y = 4 y_coarse + y_fine (coarse in the low half)
+__device__ __forceinline__ uint2 decode_half_q4(const uint2* value, const uint2* change, uint32_t code) {
+    const uint2 coarse = decode_half(value, change, code & 0xFFFFu), fine = decode_half(value, change, code >> 16);
+    return make_uint2(add_bytes((coarse.x & 0x3F3F3F3Fu) << 2, fine.x), add_bytes((coarse.y & 0x3F3F3F3Fu) << 2, fine.y));
+}
+
+// Eight activations from a low and a high plane word: byte = low nibble | high nibble << 4, even nibbles in .x
+__device__ __forceinline__ uint2 plane_bytes(uint32_t low, uint32_t high) {
+    return make_uint2((low & 0x0F0F0F0Fu) | ((high & 0x0F0F0F0Fu) << 4), ((low >> 4) & 0x0F0F0F0Fu) | (high & 0xF0F0F0F0u));
+}
+
 // fp32 epilogue shared by every projection: (float(acc) * ws) * as, two separate roundings
 // (kernels/cuda/model/integer_core.py:19-22).
 __device__ __forceinline__ float rescale(int acc, float weight_scale, float token_scale) {

@@ -21,6 +21,15 @@
 #include "orx_internal.h"
 
 namespace orx {
+
+// from k_stream.hip
+void stream_grouped_geometry(int n, int tiles, Geometry* g);
+int stream_planes_launch(bool two_stage, const uint32_t* low, const uint32_t* high, const int* sum, const void* w,
+                         const uint32_t* book, bool selector_book, const __half* ws, const __half* as, void* out,
+                         const int* counts, const int* offsets, const int* tile_expert, const int* tile_row, const int* tile_count,
+                         int n, int k, int rows, bool group_major, int tile_rows, int list_rows, const Geometry& g,
+                         hipStream_t stream);
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -169,22 +178,17 @@ struct PlaneGemmParams {
     int64_t expert_stride;  // bytes between the experts' codes
 };
 
-// sign-extends the four nibbles at bits 0-3 of every byte
-__device__ __forceinline__ uint32_t extend_nibbles(uint32_t t) { return t | ((t & 0x08080808u) * 0x1Eu); }
-
-// bytewise a + b of signed bytes whose sums fit a byte
-__device__ __forceinline__ uint32_t add_bytes(uint32_t a, uint32_t b) {
-    return ((a & 0x7F7F7F7Fu) + (b & 0x7F7F7F7Fu)) ^ ((a ^ b) & 0x80808080u);
-}
-
 // Q4: codes are u32 (coarse in the low half, weight 4; fine in the high half, weight 1) in blocks (K/128, N, 16);
 // else u16 in blocks (K/64, N, 8).
 template <bool Q4>
 __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmParams p) {
     __shared__ __align__(16) int8_t lds_a[kTileRows * kRowPitch];
     __shared__ __align__(16) int8_t lds_w[kTileChannels * kRowPitch];
-    __shared__ uint32_t book[256];   // nibble i: (w - 1) / 2 of coordinate {0,2,1,3,4,6,5,7}[i] at even parity, no sign bits
-    __shared__ uint32_t flips[256];  // what a code's low byte changes in those nibbles
+    // y = (w - 1) / 2 as sign-extended bytes, even nibbles of the reference's nibble word in .x, odd ones in .y: the value
+    // at even parity without sign bits per basis row, and what a code's low byte changes in it.  Sign extension
+    // commutes with xor, so a code is two 8-byte lookups and two xors.
+    __shared__ uint2 book[256];
+    __shared__ uint2 flips[256];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tile = blockIdx.y;
@@ -198,27 +202,7 @@ __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmPara
     const int8_t* codes = reinterpret_cast<const int8_t*>(p.codes) + (int64_t)expert * p.expert_stride;
     const __half* ws = p.ws + (int64_t)expert * p.n;
 
-    {
-        uint32_t word = p.book[tid];
-        if (p.selector_book) {  // e8p_core.py:45-60
-            uint32_t nibbles = 0;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int coordinate = (i & 4) | ((i & 1) << 1) | ((i & 2) >> 1);
-                nibbles |= ((uint32_t)selector_half(word, coordinate) & 15u) << (4 * i);
-            }
-            word = nibbles;
-        }
-        book[tid] = word;
-        // e8p_core.py:7-10: the sign bit of a coordinate negates its nibble (the stored values are odd: xor 0xe),
-        // odd parity lowers every nibble by one (xor 1) and flips the first coordinate's sign too
-        const uint32_t u = (uint32_t)tid, parity = __popc(u) & 1u;
-        const uint32_t bits = (u & 0x03u) | ((u & 0x30u) >> 2) | ((u & 0x0Cu) << 2) | (u & 0xC0u);  // nibble i <- bit
-        uint32_t spread = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) spread |= ((bits >> i) & 1u) << (4 * i + 1);
-        flips[tid] = (spread * 7u) ^ (parity * 0x1111111Fu);
-    }
+    build_half_tables(book, flips, p.book, p.selector_book != 0, tid);
 
     const int k_steps = p.k / kStepK;
     const int words = p.k >> 3;
@@ -248,20 +232,10 @@ __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmPara
         }
     };
 
-    auto half_weights = [&](uint32_t code, uint32_t& even, uint32_t& odd) {
-        const uint32_t v = book[(code >> 8) & 255u] ^ flips[code & 255u];
-        even = extend_nibbles(v & 0x0F0F0F0Fu);
-        odd = extend_nibbles((v >> 4) & 0x0F0F0F0Fu);
-    };
-
     auto store_step = [&]() {
         {
-            // byte = low nibble | high nibble << 4, even nibbles of a word first
-            const uint32_t x0 = (held_low.x & 0x0F0F0F0Fu) | ((held_high.x & 0x0F0F0F0Fu) << 4);
-            const uint32_t y0 = ((held_low.x >> 4) & 0x0F0F0F0Fu) | (held_high.x & 0xF0F0F0F0u);
-            const uint32_t x1 = (held_low.y & 0x0F0F0F0Fu) | ((held_high.y & 0x0F0F0F0Fu) << 4);
-            const uint32_t y1 = ((held_low.y >> 4) & 0x0F0F0F0Fu) | (held_high.y & 0xF0F0F0F0u);
-            *reinterpret_cast<uint4*>(lds_a + a_row * kRowPitch + a_piece * 16) = make_uint4(x0, y0, x1, y1);
+            const uint2 first = plane_bytes(held_low.x, held_high.x), second = plane_bytes(held_low.y, held_high.y);
+            *reinterpret_cast<uint4*>(lds_a + a_row * kRowPitch + a_piece * 16) = make_uint4(first.x, first.y, second.x, second.y);
         }
 #pragma unroll
         for (int i = 0; i < W_PIECES; ++i) {
@@ -272,11 +246,8 @@ __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmPara
                 uint32_t out[8];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    uint32_t ce, co, fe, fo;
-                    half_weights(in[j] & 0xFFFFu, ce, co);
-                    half_weights(in[j] >> 16, fe, fo);
-                    out[2 * j] = add_bytes((ce & 0x3F3F3F3Fu) << 2, fe);
-                    out[2 * j + 1] = add_bytes((co & 0x3F3F3F3Fu) << 2, fo);
+                    const uint2 y = decode_half_q4(book, flips, in[j]);
+                    out[2 * j] = y.x, out[2 * j + 1] = y.y;
                 }
                 uint4* dst = reinterpret_cast<uint4*>(lds_w + (c >> 2) * kRowPitch + (c & 3) * 32);
                 dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
@@ -285,10 +256,8 @@ __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmPara
                 uint4* dst = reinterpret_cast<uint4*>(lds_w + (c >> 1) * kRowPitch + (c & 1) * 64);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    uint32_t e0, o0, e1, o1;
-                    half_weights(in[j] & 0xFFFFu, e0, o0);
-                    half_weights(in[j] >> 16, e1, o1);
-                    dst[j] = make_uint4(e0, o0, e1, o1);
+                    const uint2 y0 = decode_half(book, flips, in[j] & 0xFFFFu), y1 = decode_half(book, flips, in[j] >> 16);
+                    dst[j] = make_uint4(y0.x, y0.y, y1.x, y1.y);
                 }
             }
         }
@@ -520,6 +489,10 @@ int plane_gemm_geometry(const orx_function& f, int rows, Geometry* g) {
     int tiles = f.tiles;
     // e8p_exact.py:76, e8p_prefill.py:189-192: no more tiles than the live rows can fill
     if (f.dynamic_rows) tiles = std::min(tiles, (rows + f.group - 1) / f.group + std::min(f.E, rows));
+    if (f.algorithm == 0) {  // the weight-streaming kernel
+        stream_grouped_geometry(f.N, std::max(tiles, 1), g);
+        return ORX_OK;
+    }
     g->grid[1] = (uint32_t)std::max(tiles, 1);
     g->block[0] = kPlaneThreads;
     return ORX_OK;
@@ -539,6 +512,10 @@ int plane_gemm_launch(const orx_function& f, int rows, const Geometry& g, hipStr
     p.n = f.N, p.k = f.K, p.rows = rows, p.tile_rows = f.block_m, p.list_rows = f.group;
     p.group_major = f.flags & 1, p.selector_book = (f.flags & 2) ? 1 : 0;
     p.expert_stride = (int64_t)f.N * f.K / ((f.flags & 2) ? 2 : 4);  // 4 or 2 bits per weight
+    if (f.algorithm == 0)
+        return stream_planes_launch((f.flags & 2) != 0, p.low, p.high, p.sum, p.codes, p.book, p.selector_book != 0, p.ws, p.as, p.out,
+                                    p.counts, p.offsets, p.tile_expert, p.tile_row, p.tile_count, f.N, f.K, rows, p.group_major != 0,
+                                    p.tile_rows, p.list_rows, g, stream);
     const dim3 grid(g.grid[0], g.grid[1]), block(g.block[0]);
     if (f.flags & 2)
         hipLaunchKernelGGL(plane_gemm_kernel<true>, grid, block, 0, stream, p);
@@ -547,7 +524,17 @@ int plane_gemm_launch(const orx_function& f, int rows, const Geometry& g, hipStr
     return hip_check(hipGetLastError(), "launch grouped GEMM on planes");
 }
 
-int finish_plane_gemm(const char* symbol, orx_function* f) {
+int finish_plane_gemm(const Variant& v, const char* symbol, orx_function* f) {
+    bool bad = false;
+    // stream: codes decoded straight into MFMA operands, K split over two waves (k_stream.hip); tiles: operands staged in
+    // LDS (plane_gemm_kernel).  Measured at 2048 slots in 177 tiles of 16 rows: N = 1024, K = 2048: 35.5 against 43.2 us;
+    // N = 2048, K = 512: 29.2 against 25.4 us (the streaming kernel's set-up is paid per 128 channels and tile).
+    const std::string algorithm = v.string("algorithm", "auto", &bad);
+    if (bad || (algorithm != "auto" && algorithm != "stream" && algorithm != "tiles")) {
+        set_error("%s: algorithm is auto, stream or tiles", symbol);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    f->algorithm = algorithm == "tiles" || (algorithm == "auto" && f->K < 1024) ? 1 : 0;
     if (f->M <= 0 || f->E <= 0 || f->tiles <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 ||
         (int64_t)f->K * 128 * 128 > 2147483647ll) {  // e8p_exact.py:60-61: the int32 accumulator holds a whole row
         set_error("%s: need rows, E, tiles, N > 0 and K a multiple of 128 with K * 128 * 128 < 2^31", symbol);
@@ -558,8 +545,9 @@ int finish_plane_gemm(const char* symbol, orx_function* f) {
                {"Sum", ArgPointer, 4},    {"TC", ArgPointer, 4},      {"TE", ArgPointer, 4},     {"TR", ArgPointer, 4},
                {"WS", ArgPointer, 2}};
     if (f->dynamic_rows) f->args.push_back({"m", ArgI32, 4});
-    f->device_function = (f->flags & 2) ? reinterpret_cast<const void*>(&plane_gemm_kernel<true>)
-                                        : reinterpret_cast<const void*>(&plane_gemm_kernel<false>);
+    f->device_function = f->algorithm == 0 ? nullptr  // 512 threads: the device's own limit
+                         : (f->flags & 2)  ? reinterpret_cast<const void*>(&plane_gemm_kernel<true>)
+                                           : reinterpret_cast<const void*>(&plane_gemm_kernel<false>);
     f->geometry = plane_gemm_geometry;
     f->launch = plane_gemm_launch;
     return ORX_OK;
@@ -584,7 +572,7 @@ int make_exact_grouped(const Variant& v, orx_function* f) {
         return ORX_ERR_BAD_VARIANT;
     }
     f->group = f->block_m, f->flags = 0;
-    return finish_plane_gemm("e8p_exact_grouped", f);
+    return finish_plane_gemm(v, "e8p_exact_grouped", f);
 }
 
 // e8p_prefill_grouped (e8p_prefill.py:132-561): K64-major planes (row-major on request), single-stage codes in
@@ -616,7 +604,7 @@ int make_prefill_grouped(const Variant& v, orx_function* f) {
     }
     f->group = merge ? f->block_m / 2 : f->block_m;  // e8p_prefill.py:188
     f->flags = (row_major ? 0 : 1) | (q4 ? 2 : 0);
-    return finish_plane_gemm("e8p_prefill_grouped", f);
+    return finish_plane_gemm(v, "e8p_prefill_grouped", f);
 }
 
 }  // namespace
@@ -632,11 +620,11 @@ const Registration* plane_registrations(int* count) {
         {"pack_expert_tokens", make_pack_tokens, "M, K, E, top_k", "A,High,IDs,Low,RelativeSlot,RowOffsets,SlotMap,Sources,Sum,m"},
         {"expand_expert_slots", make_expand_slots, "M, K, top_k", "DS,High,Low,Scale,Sources,SrcHigh,SrcLow,SrcSum,Sum,m"},
         {"e8p_exact_grouped", make_exact_grouped,
-         "rows, E, tiles, N, K, block_m=16|8, stages=2..4, dynamic_rows=false, warp_private=false",
+         "rows, E, tiles, N, K, block_m=16|8, stages=2..4, dynamic_rows=false, warp_private=false, algorithm=auto|stream|tiles",
          "AS,Book,Counts,High,Low,Offsets,Out,P,Sum,TC,TE,TR,WS[,m]"},
         {"e8p_prefill_grouped", make_prefill_grouped,
          "rows, E, tiles, N, K, dynamic_rows=false, sparse_rows=false, row_major=false, codec=e8p_q2|e8p_q4, "
-         "minimum_blocks=1, block_m=16|32, block_n=128|64, specialize_tails=false, merge_routed_tiles=false",
+         "minimum_blocks=1, block_m=16|32, block_n=128|64, specialize_tails=false, merge_routed_tiles=false, algorithm=auto|stream|tiles",
          "AS,Book,Counts,High,Low,Offsets,Out,P,Sum,TC,TE,TR,WS[,m]"},
     };
     *count = (int)(sizeof(rows) / sizeof(rows[0]));

@@ -17,6 +17,9 @@
 // half h owns bytes [64h, 64h+64) of every 128-byte K block, sub-step s the 16 bytes at 16s.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
+#include "a8_device.h"
 #include "e8p_device.h"
 #include "orx_internal.h"
 #include "row_q4_device.h"
@@ -47,6 +50,11 @@ struct StreamParams {
     const int* tile_count;
     int64_t expert_weight_stride;  // bytes between experts in w
     uint32_t magnitudes_low, magnitudes_high;  // scalar Q4: the eight magnitudes, one per byte
+    // PLANES: activations as two planes of nibble words with the rows' sums (e8p_exact.py, e8p_prefill.py)
+    const uint32_t* low;
+    const uint32_t* high;
+    const int* sum;
+    int plane_rows, group_major, selector_book, tile_rows, list_rows;
 };
 
 template <int CODEC>
@@ -77,12 +85,18 @@ __host__ __device__ constexpr int block_bytes() {
 
 // CB = column blocks of 32 token rows (1 or 2); SPLITS = waves that share one group of 32 output
 // channels, each taking a slice of K (8 for long K and few channels, 2 for the short K of experts).
-template <int CODEC, int CB, bool GROUPED, int SPLITS>
+// PLANES (routed codes only): the INT4-exact expert kernels' operands.  Activations come as low / high nibble planes and are
+// put back together in registers; weights are decoded as y = (w - 1) / 2 from the nibble Book; the integer is
+// 2 acc + c Sum[row] with the caller's Sum (c = 1, or 5 for two-stage codes; kernels/cuda/model/e8p_core.py:154-189).
+// The bytes of a group of eight keep the order (even nibbles, odd nibbles) on both operands.
+template <int CODEC, int CB, bool GROUPED, int SPLITS, bool PLANES = false>
 __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
+    static_assert(!PLANES || (GROUPED && CB == 1 && (CODEC == kQ2 || CODEC == kQ4)), "planes feed the routed tiles");
     constexpr int kSplits = SPLITS;
     constexpr int GROUPS = kWaves / SPLITS;   // channel groups per workgroup
     constexpr int kRows = 32;
-    __shared__ typename StreamTables<CODEC>::type tables;
+    __shared__ typename std::conditional<PLANES, StreamTables<kW8>, StreamTables<CODEC>>::type::type tables;
+    __shared__ uint2 half_value[PLANES ? 256 : 1], half_change[PLANES ? 256 : 1];
     __shared__ int partial[kWaves][kRows][33];  // one column block at a time; +1 keeps column reads conflict-free
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -99,14 +113,19 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         if (tile >= p.tile_count[0]) return;
         const int expert = p.tile_expert[tile];
         const int first = p.tile_row[tile];
+        if (PLANES && p.list_rows != p.tile_rows && first % p.tile_rows != 0) return;  // the second of two merged tiles
         row0 = p.offsets[expert] + first;
-        rows_here = min(CB * 32, p.counts[expert] - first);
+        rows_here = min(PLANES ? p.tile_rows : CB * 32, p.counts[expert] - first);
         if (rows_here <= 0) return;
         w_base += (int64_t)expert * p.expert_weight_stride;
         ws += (int64_t)expert * p.n;
     }
 
-    if constexpr (CODEC == kQ4 || CODEC == kQ2) build_tables(tables, p.book, tid, kThreads);
+    if constexpr (PLANES) {
+        if (tid < 256) build_half_tables(half_value, half_change, p.book, p.selector_book != 0, tid);
+    } else if constexpr (CODEC == kQ4 || CODEC == kQ2) {
+        build_tables(tables, p.book, tid, kThreads);
+    }
 
     // K blocks of this wave
     const int k_blocks = p.k / 128;
@@ -132,7 +151,9 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
     const int8_t* a_rows[CB];
 #pragma unroll
     for (int c = 0; c < CB; ++c)
-        a_rows[c] = p.a + (int64_t)(row0 + min(c * 32 + frag, rows_here - 1)) * p.k + half * 64;
+        a_rows[c] = PLANES ? nullptr : p.a + (int64_t)(row0 + min(c * 32 + frag, rows_here - 1)) * p.k + half * 64;
+    // PLANES: the lane's 64 activations of a K block are words [16 kb + 8 half, + 8) of its plane row
+    const int64_t plane_row = row0 + min(frag, rows_here - 1);
 
     v16i acc[CB];
 #pragma unroll
@@ -146,6 +167,14 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         const uint4* src = weight_pointer(kb);
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) c[i] = src[i];
+        if constexpr (PLANES) {
+            // a[0][0..1] hold the low words, a[0][2..3] the high words; they are combined when they are used
+            const int64_t at = plane_index(p.group_major, p.plane_rows, p.k >> 3, plane_row, kb * 16 + half * 8);
+            const uint4* low = reinterpret_cast<const uint4*>(p.low + at);
+            const uint4* high = reinterpret_cast<const uint4*>(p.high + at);
+            a[0][0] = low[0], a[0][1] = low[1], a[0][2] = high[0], a[0][3] = high[1];
+            return;
+        }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             const uint4* arow = reinterpret_cast<const uint4*>(a_rows[cb] + (int64_t)kb * 128);
@@ -166,7 +195,30 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         if (kb + 1 < kb_last) fetch(kb + 1, next_codes, next_act);
         // four row-operand fragments of 16 weights each
         uint4 wf[4];
-        if constexpr (CODEC == kQ4) {
+        if constexpr (PLANES) {
+            const uint32_t low[8] = {act[0][0].x, act[0][0].y, act[0][0].z, act[0][0].w, act[0][1].x, act[0][1].y, act[0][1].z, act[0][1].w};
+            const uint32_t high[8] = {act[0][2].x, act[0][2].y, act[0][2].z, act[0][2].w, act[0][3].x, act[0][3].y, act[0][3].z, act[0][3].w};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const uint2 first = plane_bytes(low[2 * s], high[2 * s]), second = plane_bytes(low[2 * s + 1], high[2 * s + 1]);
+                act[0][s] = make_uint4(first.x, first.y, second.x, second.y);
+            }
+            if constexpr (CODEC == kQ4) {
+                const uint32_t c[8] = {codes[0].x, codes[0].y, codes[0].z, codes[0].w, codes[1].x, codes[1].y, codes[1].z, codes[1].w};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint2 y0 = decode_half_q4(half_value, half_change, c[2 * s]), y1 = decode_half_q4(half_value, half_change, c[2 * s + 1]);
+                    wf[s] = make_uint4(y0.x, y0.y, y1.x, y1.y);
+                }
+            } else {
+                const uint32_t c[4] = {codes[0].x, codes[0].y, codes[0].z, codes[0].w};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint2 y0 = decode_half(half_value, half_change, c[s] & 0xFFFFu), y1 = decode_half(half_value, half_change, c[s] >> 16);
+                    wf[s] = make_uint4(y0.x, y0.y, y1.x, y1.y);
+                }
+            }
+        } else if constexpr (CODEC == kQ4) {
             const uint32_t c[8] = {codes[0].x, codes[0].y, codes[0].z, codes[0].w,
                                    codes[1].x, codes[1].y, codes[1].z, codes[1].w};
 #pragma unroll
@@ -223,6 +275,7 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
 #pragma unroll
             for (int s = 0; s < kSplits; ++s) total += partial[g * SPLITS + s][channel][local_token];
             const int64_t row = row0 + token;
+            if constexpr (PLANES) total = (int)(2u * (uint32_t)total + (CODEC == kQ4 ? 5u : 1u) * (uint32_t)p.sum[row]);
             const float value = rescale(total, __half2float(ws[col]), __half2float(p.as[row]));
             if (p.out_f32)
                 reinterpret_cast<float*>(p.out)[row * p.stride + col] = value;
@@ -266,6 +319,28 @@ int stream_launch(int codec, const int8_t* a, const void* w, const uint32_t* boo
     if (codec == kQ4) return launch_codec<kQ4, false, kDenseSplits>(cb, p, grid, stream);
     if (codec == kQ2) return launch_codec<kQ2, false, kDenseSplits>(cb, p, grid, stream);
     return launch_codec<kW8, false, kDenseSplits>(cb, p, grid, stream);
+}
+
+// Routed experts on nibble planes (e8p_exact_grouped, e8p_prefill_grouped): tiles of up to 32 rows; single-stage codes in
+// K-major blocks of 64 (two-stage: blocks of 128)
+int stream_planes_launch(bool two_stage, const uint32_t* low, const uint32_t* high, const int* sum, const void* w,
+                         const uint32_t* book, bool selector_book, const __half* ws, const __half* as, void* out,
+                         const int* counts, const int* offsets, const int* tile_expert, const int* tile_row, const int* tile_count,
+                         int n, int k, int rows, bool group_major, int tile_rows, int list_rows, const Geometry& g,
+                         hipStream_t stream) {
+    StreamParams p = {};
+    p.w = w, p.book = book, p.ws = ws, p.as = as, p.out = out;
+    p.n = n, p.k = k, p.stride = n, p.m = 0, p.packed_k = two_stage ? 128 : 64, p.out_f32 = 0;
+    p.counts = counts, p.offsets = offsets, p.tile_expert = tile_expert, p.tile_row = tile_row, p.tile_count = tile_count;
+    p.expert_weight_stride = (int64_t)n * k / (two_stage ? 2 : 4);
+    p.low = low, p.high = high, p.sum = sum, p.plane_rows = rows, p.group_major = group_major, p.selector_book = selector_book;
+    p.tile_rows = tile_rows, p.list_rows = list_rows;
+    const dim3 grid(g.grid[0], g.grid[1]);
+    if (two_stage)
+        hipLaunchKernelGGL((stream_kernel<kQ4, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
+    else
+        hipLaunchKernelGGL((stream_kernel<kQ2, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
+    return hip_check(hipGetLastError(), "launch routed projection on nibble planes (stream)");
 }
 
 // Row-scaled scalar Q4 (kernels/cuda/model/q4_projection.py): W is (N, K/4) u16, rows <= 64

@@ -631,6 +631,11 @@ def test_plane_kernels_refuse_what_the_reference_refuses():
     # the exact kernel launches no more tiles than the live rows can fill (e8p_exact.py:76)
     dynamic = lib.Kernel("e8p_exact_grouped", **shape, block_m=8, dynamic_rows=True)
     assert dynamic.geometry(8)[0][1] == 1 + 8 and dynamic.geometry(64)[0][1] == 16
+    # two kernels behind the symbols: 512-thread weight-streaming workgroups from K = 1024, 256-thread LDS tiles below
+    assert lib.Kernel("e8p_exact_grouped", **{**shape, "K": 2048}).geometry()[1][0] == 512 and dynamic.geometry()[1][0] == 256
+    assert lib.Kernel("e8p_exact_grouped", **shape, algorithm="stream").geometry()[1][0] == 512
+    with pytest.raises(lib.OrxError):
+        lib.Kernel("e8p_exact_grouped", **shape, algorithm="mfma")
 
 
 def test_scalar_q4_symbols_bind_as_the_reference_does_and_refuse_what_it_refuses():

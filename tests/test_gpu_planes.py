@@ -200,11 +200,14 @@ def test_exact_and_prefill_grouped_match_the_int8_kernel(bm, counts, n, k):
         TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws), **routing)
     np.testing.assert_array_equal(gu.host(ref), want)
     a_dev = gu.dev(a)
-    forms = []
+    forms = []  # both kernels behind the symbols: codes decoded into MFMA operands (stream) or staged in LDS (tiles)
     if bm <= 16:
-        forms += [("e8p_exact_grouped", dict(block_m=bm, stages=s), False) for s in (2, 3, 4) if k // 64 >= s - 1]
+        forms += [("e8p_exact_grouped", dict(block_m=bm, stages=s, algorithm=("stream", "tiles", "auto")[s - 2]), False)
+                  for s in (2, 3, 4) if k // 64 >= s - 1]
     if bm >= 16:
-        forms += [("e8p_prefill_grouped", dict(block_m=bm), True), ("e8p_prefill_grouped", dict(block_m=bm, row_major=True), False)]
+        forms += [("e8p_prefill_grouped", dict(block_m=bm, algorithm="stream"), True),
+                  ("e8p_prefill_grouped", dict(block_m=bm, algorithm="tiles"), True),
+                  ("e8p_prefill_grouped", dict(block_m=bm, row_major=True), False)]
     for symbol, options, group_major in forms:
         low, high = empty_planes(rows, k, group_major)
         sums = torch.full((rows,), -7, **I32)
@@ -253,12 +256,14 @@ def test_prefill_grouped_two_stage_codes(bm, counts, n, k):
     sums = torch.full((rows,), -7, **I32)
     gu.kernel("split_prefill_a8", rows=rows, K=k)(A=gu.dev(a), High=high, Low=low, Sum=sums)
     out = torch.full((rows + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
-    gu.kernel("e8p_prefill_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, codec="e8p_q4", block_m=bm)(
-        AS=gu.dev(scale), Book=gu.book(), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets), Out=out,
-        P=gu.dev(stored), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws))
-    got = gu.host(out)
-    np.testing.assert_array_equal(got[:rows], want)
-    assert (got[rows] == 91).all()
+    for algorithm in ("stream", "tiles"):
+        out.fill_(91.0)
+        gu.kernel("e8p_prefill_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, codec="e8p_q4", block_m=bm, algorithm=algorithm)(
+            AS=gu.dev(scale), Book=gu.book(), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets), Out=out,
+            P=gu.dev(stored), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws))
+        got = gu.host(out)
+        np.testing.assert_array_equal(got[:rows], want)
+        assert (got[rows] == 91).all()
 
 
 def test_prefill_grouped_merges_adjacent_tiles_of_a_shared_list_and_takes_live_rows():
@@ -279,14 +284,16 @@ def test_prefill_grouped_merges_adjacent_tiles_of_a_shared_list_and_takes_live_r
     sums = torch.full((capacity,), -7, **I32)
     gu.kernel("split_prefill_a8", rows=capacity, K=k, dynamic_rows=True)(A=gu.dev(a), High=high, Low=low, Sum=sums, m=rows)
     out = torch.full((capacity, n), 91.0, dtype=torch.float16, device=gu.DEV)
-    gu.kernel("e8p_prefill_grouped", rows=capacity, E=e, tiles=cap, N=n, K=k, block_m=32, specialize_tails=True,
-              merge_routed_tiles=True, dynamic_rows=True, sparse_rows=True, minimum_blocks=2)(
-        AS=gu.dev(scale), Book=gu.dev(nibble[None]), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets),
-        Out=out, P=gu.dev(orc.q2_repack_k64(raw)), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws),
-        m=rows)
-    got = gu.host(out)
-    np.testing.assert_array_equal(got[:rows], want)
-    assert (got[rows:] == 91).all()
+    for algorithm in ("stream", "tiles"):
+        out.fill_(91.0)
+        gu.kernel("e8p_prefill_grouped", rows=capacity, E=e, tiles=cap, N=n, K=k, block_m=32, specialize_tails=True,
+                  merge_routed_tiles=True, dynamic_rows=True, sparse_rows=True, minimum_blocks=2, algorithm=algorithm)(
+            AS=gu.dev(scale), Book=gu.dev(nibble[None]), Counts=gu.dev(counts_np), High=high, Low=low, Offsets=gu.dev(offsets),
+            Out=out, P=gu.dev(orc.q2_repack_k64(raw)), Sum=sums, TC=gu.dev(total), TE=gu.dev(te), TR=gu.dev(tr), WS=gu.dev(ws),
+            m=rows)
+        got = gu.host(out)
+        np.testing.assert_array_equal(got[:rows], want)
+        assert (got[rows:] == 91).all()
 
 
 def test_rotated_planes_into_the_exact_kernel_equal_int8_rows_into_the_int8_kernel():
