@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) void gemm_split_kernel(GemmParams p) {
     const int64_t unit_begin = split_begin(units, blockIdx.x, gridDim.x), unit_end = split_begin(units, blockIdx.x + 1, gridDim.x);
     int n0 = 0, row0 = 0, rows_here = 1;
 
-    if constexpr (CODEC != kW8) build_tables(tables, p.book, tid, 256);
+    if constexpr (CODEC == kQ4 || CODEC == kQ2) build_tables(tables, p.book, tid, 256);
 
     const int k_tiles = p.k / kBK;
     v4u held_a[A_CHUNKS], held_w[W_CHUNKS];
@@ -1115,9 +1115,20 @@ int row_q4_unpack(const void* w, void* out, int n, int k, uint32_t low, uint32_t
 
 constexpr int kRowQ4BigRows = 512;
 bool row_q4_expands(const orx_function& f, int rows) { return f.takes_workspace && rows >= kRowQ4BigRows; }
+// 65..511 rows: the K steps of the 128-row tiles dealt evenly to the CUs when whole tiles would not spread evenly
+// (the rule of the other codecs: 8 to 288 tiles that do not divide over the CUs)
+bool row_q4_splits(const orx_function& f, int rows) { return rows > 64 && !row_q4_expands(f, rows) && split_shape_ok(f, rows); }
 
 uint64_t row_q4_workspace(const orx_function& f, int rows) {
-    return (rows == 0 ? f.capacity >= kRowQ4BigRows : row_q4_expands(f, rows)) ? (uint64_t)f.N * f.K : 0;
+    if (rows == 0) {  // the most any row count needs: one probe per height in 128-row tiles
+        uint64_t most = 0;
+        for (int top = 128; top - 128 < std::min(f.capacity, kRowQ4BigRows); top += 128)
+            most = std::max(most, row_q4_workspace(f, std::min(top, f.capacity)));
+        return most;
+    }
+    if (row_q4_expands(f, rows)) return (uint64_t)f.N * f.K;
+    if (row_q4_splits(f, rows)) return (uint64_t)split_groups_for(f, rows) * 2 * kSplitSlotInts * sizeof(int);
+    return 0;
 }
 
 int row_q4_geometry(const orx_function& f, int rows, Geometry* g) {
@@ -1131,6 +1142,12 @@ int row_q4_geometry(const orx_function& f, int rows, Geometry* g) {
     }
     if (row_q4_expands(f, rows)) {
         gemm_big_geometry(rows, f.N, false, g);
+        return ORX_OK;
+    }
+    if (row_q4_splits(f, rows)) {
+        g->grid[0] = (uint32_t)split_groups_for(f, rows);
+        g->block[0] = 256;
+        g->shared = 0;
         return ORX_OK;
     }
     g->grid[0] = ceil_div((uint32_t)f.N, 128u);
@@ -1162,6 +1179,10 @@ int row_q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
         if (code != ORX_OK) return code;
         return gemm_big_launch(false, p.a, workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
                                stream);
+    }
+    if (row_q4_splits(f, rows)) {
+        p.partials = pointer_arg<int>(args, f.workspace_arg);
+        return launch_split<kS4>(p, split_groups_for(f, rows), stream);
     }
     hipLaunchKernelGGL((gemm_kernel<kS4, 128, 128, 2, false>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, p);
     return hip_check(hipGetLastError(), "launch scalar Q4 projection (mfma)");
