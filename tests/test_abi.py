@@ -644,7 +644,9 @@ def test_scalar_q4_symbols_bind_as_the_reference_does_and_refuse_what_it_refuses
     assert lib.Kernel("q4_gemv", M=8, N=256, K=512, dynamic_rows=True).arg_names == ["A", "AS", "Out", "S", "W", "m"]
     big = lib.Kernel("q4_projection", M=1024, N=256, K=512, workspace=True, dynamic_rows=True)
     assert big.arg_names == ["A", "AS", "Out", "S", "W", "Workspace", "m"]
-    assert big.workspace_bytes() == 256 * 512 and big.workspace_bytes(64) == 0 and big.workspace_bytes(600) == 256 * 512
+    assert big.workspace_bytes(64) == 0 and big.workspace_bytes(600) == 256 * 512
+    # 511 rows are 8 tiles of 128 x 128 over 4 K steps: 4 workgroups with two partial slots each
+    assert big.workspace_bytes(511) == 4 * 2 * 128 * 128 * 4 == big.workspace_bytes()
     # 65..511 rows: int32 partial tiles of a split launch where whole tiles would not spread evenly over the CUs
     mid = lib.Kernel("q4_projection", M=256, N=17408, K=5120, workspace=True, dynamic_rows=True)
     assert mid.workspace_bytes(128) == 512 * 2 * 128 * 128 * 4 == mid.workspace_bytes() and mid.workspace_bytes(64) == 0
