@@ -650,7 +650,7 @@ def test_scalar_q4_symbols_bind_as_the_reference_does_and_refuse_what_it_refuses
     # 65..511 rows: int32 partial tiles of a split launch where whole tiles would not spread evenly over the CUs
     mid = lib.Kernel("q4_projection", M=256, N=17408, K=5120, workspace=True, dynamic_rows=True)
     assert mid.workspace_bytes(128) == 512 * 2 * 128 * 128 * 4 == mid.workspace_bytes() and mid.workspace_bytes(64) == 0
-    assert mid.geometry(128)[0][0] == 512 and lib.Kernel("q4_projection", M=256, N=17408, K=5120).geometry(128)[0] == (136, 1, 1)
+    assert mid.geometry(128)[0][0] == 512 and lib.Kernel("q4_projection", M=128, N=17408, K=5120).geometry()[0] == (136, 1, 1)
     assert lib.Kernel("unpack_q4", N=256, K=512).arg_names == ["Output", "W"]
     shape = dict(M=8, N=256, K=512)
     for bad in (dict(magnitudes=[3, 10, 19, 31, 46, 67, 93]), dict(magnitudes=[3, 10, 19, 31, 46, 67, 93, 128]),
