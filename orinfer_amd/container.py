@@ -297,6 +297,33 @@ def expert_layer_program(slot, tokens, experts, top_k, hidden, intermediate, *, 
     return records, sizes
 
 
+def exact_expert_program(slot, rows, experts, top_k, n, k, *, block_m=8, stages=4, warp_private=True, buffers=None):
+    """One routed expert projection on nibble planes as the reference's decode programs record it
+    (python/orinfer_build/models/flash_next/expert_decode.py:23-75: `e8p_exact_grouped` with 8-row tiles behind the
+    split of the A8 rows): `split_a8` writes Low / High / Sum, `e8p_exact_grouped` multiplies them with the
+    K-major blocks of 64 (`codebook.q2_to_k64`) and the nibble Book (`codebook.nibble_book`).
+
+    rows: token rows; the projection sees rows * top_k routed rows.  Returns the two records and a dict
+    name -> byte size of every buffer they touch."""
+    slots = rows * top_k
+    tiles = (slots + block_m - 1) // block_m + min(experts, slots)
+    name = dict(buffers or {})
+    b = lambda key: name.get(key, key)
+    records = [
+        kernel_record(f"{slot}.split", "split_a8", dict(rows=slots, K=k),
+                      dict(A=b("A"), High=b("High"), Low=b("Low"), Sum=b("Sum"))),
+        kernel_record(f"{slot}.project", "e8p_exact_grouped",
+                      dict(rows=slots, E=experts, tiles=tiles, N=n, K=k, block_m=block_m, stages=stages,
+                           warp_private=warp_private),
+                      dict(AS=b("AS"), Book=b("Book"), Counts=b("Counts"), High=b("High"), Low=b("Low"), Offsets=b("Offsets"),
+                           Out=b("Out"), P=b("P"), Sum=b("Sum"), TC=b("TC"), TE=b("TE"), TR=b("TR"), WS=b("WS"))),
+    ]
+    sizes = {b("A"): slots * k, b("High"): slots * k // 2, b("Low"): slots * k // 2, b("Sum"): slots * 4, b("AS"): slots * 2,
+             b("Book"): 1024, b("Counts"): experts * 4, b("Offsets"): experts * 4, b("Out"): slots * n * 2,
+             b("P"): experts * n * k // 4, b("TC"): 4, b("TE"): tiles * 4, b("TR"): tiles * 4, b("WS"): experts * n * 2}
+    return records, sizes
+
+
 def fixture_manifest(buffers, records, validation, *, rows=None):
     """The same records as a manifest of the `orx_run_fixture` runner (buffers: name -> bytes | array file)."""
     kernels = []

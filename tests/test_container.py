@@ -178,3 +178,44 @@ def test_expert_layer_records_run_through_the_fixture_runner(tmp_path):
                           timeout=120)
     report = json.loads(done.stdout.strip().splitlines()[-1])
     assert done.returncode == 0 and report["ok"] and report["relative_l2"] < 3e-3, (report, done.stderr)
+
+
+@pytest.mark.gpu
+def test_exact_expert_records_run_through_the_fixture_runner(tmp_path):
+    """The reference's decode pairing on nibble planes (split_a8 -> e8p_exact_grouped, 8-row tiles) as package records,
+    resolved and launched by the C++ fixture runner: the oracle's output exactly, graph capture and the replays."""
+    rng = np.random.default_rng(orc.SEED + 31)
+    rows, experts, top_k, n, k, bm = 9, 8, 4, 320, 640, 8
+    slots = rows * top_k
+    ids = np.stack([rng.choice(experts, top_k, replace=False) for _ in range(rows)]).astype(np.int32)
+    counts, _ = orc.expert_histogram(ids, experts)
+    offsets, tile_offsets, total = orc.expert_offsets(counts, bm)
+    records, sizes = container.exact_expert_program("flash_decode.layer0.post", rows, experts, top_k, n, k, block_m=bm)
+    tiles = sizes["TE"] // 4
+    te, tr = orc.expert_tiles(counts, tile_offsets, bm, tiles)
+    a = rng.integers(-128, 128, (slots, k), dtype=np.int8)
+    scale = rng.uniform(0.01, 0.03, slots).astype(np.float16)
+    codes = rng.integers(0, 65536, (experts, n, k // 8), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (experts, n)).astype(np.float16)
+    weights = np.stack([orc.q2_integers(c, orc.basis()) for c in codes])
+    want = orc.grouped_project(a, scale[:, None], weights, ws, counts, offsets).astype(np.float32)
+    want.tofile(tmp_path / "Out.f32")
+    data = {"A": a, "AS": scale, "Book": codebook.nibble_book(), "Counts": counts, "Offsets": offsets, "TC": total, "TE": te,
+            "TR": tr, "P": codebook.q2_to_k64(codebook.q2_to_k_major(codes)), "WS": ws}
+    buffers = []
+    for name, size in sizes.items():
+        if name in data:
+            array = np.ascontiguousarray(data[name])
+            assert array.nbytes == size, name
+            array.tofile(tmp_path / f"{name}.bin")
+            buffers.append({"name": name, "file": f"{name}.bin", "bytes": size})
+        else:
+            buffers.append({"name": name, "bytes": size, "fill": 0})
+    manifest = container.fixture_manifest(buffers, records,
+                                          dict(output="Out", output_dtype="f16", reference="Out.f32",
+                                               relative_l2_tolerance=1e-7, zero_input="A", repetitions=5))
+    (tmp_path / "manifest.json").write_text(json.dumps(manifest))
+    done = subprocess.run([str(build.FIXTURE_RUNNER), str(tmp_path / "manifest.json")], capture_output=True, text=True,
+                          timeout=120)
+    report = json.loads(done.stdout.strip().splitlines()[-1])
+    assert done.returncode == 0 and report["ok"] and report["relative_l2"] == 0, (report, done.stderr)
