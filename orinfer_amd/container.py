@@ -218,16 +218,26 @@ def projection_program(slot, n, k, capacity, *, family="e8p_q4_projection", bind
         while high < capacity and whole.geometry(high + 1)[1:] == (block, shared):
             high += 1
         # the record of a range is resolved at the top of the range: its own dispatch must agree, and the
-        # grid over the range must be one expression per dimension; shrink the range until both hold
-        while True:
-            variant, kernel = handle(high)
-            geometry = {r: kernel.geometry(r) for r in range(low, high + 1)}
-            fits = [None] * 3
-            if all(g[1:] == (block, shared) for g in geometry.values()):
-                fits = [_fit_rows({r: g[0][d] for r, g in geometry.items()}) for d in range(3)]
-            if all(f is not None for f in fits):
-                break
-            high = low + (high - low) // 2
+        # grid over the range must be one expression per dimension; take the longest range for which both hold
+        def attempt(top):
+            variant, kernel = handle(top)
+            geometry = {r: kernel.geometry(r) for r in range(low, top + 1)}
+            if not all(g[1:] == (block, shared) for g in geometry.values()):
+                return None
+            fits = [_fit_rows({r: g[0][d] for r, g in geometry.items()}) for d in range(3)]
+            return (variant, kernel, fits) if all(f is not None for f in fits) else None
+
+        found = attempt(high)
+        if found is None:
+            good, bad = low, high  # a single row count always fits (constants)
+            while bad - good > 1:
+                middle = (good + bad) // 2
+                if attempt(middle) is not None:
+                    good = middle
+                else:
+                    bad = middle
+            high, found = good, attempt(good)
+        variant, kernel, fits = found
         names = kernel.arg_names
         bound = dict(bindings or {a: a for a in names})
         bound["m"] = high

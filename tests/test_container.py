@@ -109,6 +109,18 @@ def test_kernel_records_follow_the_package_schema():
     assert buffer["dtype"] == "u32" and buffer["shape"] == [4, 8] and buffer["access"] == "read"
 
 
+def test_row_ranges_are_the_longest_the_geometry_allows():
+    """One record per stretch of rows with one block size, one LDS size and one grid expression: the scalar Q4 slot of
+    config 1's shape changes kernel at 2, 3, 65, 257 (whole tiles instead of split ones) and 512 rows, nowhere else."""
+    program = container.projection_program("layer0.q", 17408, 5120, 1024, family="q4_projection")
+    assert [k["name"].rsplit("/", 1)[1] for k in program["kernels"]] == ["1-1", "2-2", "3-64", "65-256", "257-511", "512-1024"]
+    for entry in program["dynamic"]:
+        low, high = (int(x) for x in entry["name"].rsplit("/", 1)[1].split("-"))
+        kernel = lib.Kernel("q4_projection", M=high, N=17408, K=5120, dynamic_rows=True, workspace=True)
+        for rows in {low, (low + high) // 2, high}:
+            assert tuple(container.evaluate_rows(e, rows) for e in entry["grid"]) == kernel.geometry(rows)[0]
+
+
 @pytest.mark.gpu
 def test_container_to_records_to_fixture_run(tmp_path):
     """File -> container -> records -> launch through the fixture runner, checked against the oracle."""
