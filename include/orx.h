@@ -29,8 +29,10 @@
  * Single-stage (routed expert) codes are decoded by an XOR identity that needs a basis
  * without zero coordinates, which the E8P basis is (quantization/vq.py:96-118 has the
  * same contract); `integer_vq_grouped` also takes the reference decoder's other options
- * (integer_vq.py:111-258): basis=any (selector ids for zero coordinates), one selector
- * table per expert (shared_table=false, the reference's default: Book is (E,256,1)), patch words (patched=true:
+ * (integer_vq.py:93-258) with its defaults: Book as the (256,2) table of raw int8 basis values, as the (512,4)
+ * table of signed values (shortbook=true) or as (256,1) selector words (shortbook=true, selectorbook=true);
+ * basis=any (selector ids for zero coordinates), one
+ * table per expert (shared_table=false, the reference's default: Book is (E, ...)), patch words (patched=true:
  * Patch is (E,K/128,N) u16), tile lists of 8 or 16 rows and K-major blocks of 64.  These
  * run on the MFMA tile kernel only.  The symbol always lists Patch, as the reference's
  * host ABI does; without patched=true it is never read and may be null.

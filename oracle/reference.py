@@ -113,6 +113,20 @@ def selector_table(table):
     return word.astype(np.uint32).reshape(256, 1)
 
 
+def sign_table(table):
+    """(512, 4) u32: for basis row b at parity p (row p * 256 + b) the words [low half +, low half -, high half +,
+    high half -] of the values +-t + (1 - 2p), int8 wrap-around (python/orinfer_build/quantization/vq.py:44-69)."""
+    t = np.asarray(table, np.int8).astype(np.int16)
+    values = np.empty((512, 8, 2), np.int8)
+    for parity in (0, 1):
+        shift = 1 - 2 * parity
+        values[parity * 256:(parity + 1) * 256, :, 0] = (t + shift).astype(np.int8)
+        values[parity * 256:(parity + 1) * 256, :, 1] = (-t + shift).astype(np.int8)
+    columns = [np.ascontiguousarray(values[:, half * 4:half * 4 + 4, sign]).view("<u4").reshape(512)
+               for half in range(2) for sign in range(2)]
+    return np.stack(columns, axis=-1)
+
+
 def basis_words(table):
     """(256,2) u32 raw int8 basis view used by the single-token Q2 kernel (vq.py:203)."""
     return np.ascontiguousarray(np.asarray(table, np.int8)).view("<u4").reshape(256, 2)

@@ -182,40 +182,65 @@ __device__ __forceinline__ uint2 decode_q2(const Q2ByteTables& t, uint32_t code)
     return make_uint2(b.x ^ m.x, b.y ^ m.y);
 }
 
-// Single-stage decode for any selector table, zero coordinates included (the selector decoder of
-// kernels/cuda/model/integer_vq.py:163-192 takes them; the XOR identity above does not): where the
-// basis value is zero the weight is 1 - 2p whatever the sign bit says, so those bytes are replaced.
+// Single-stage decode for any basis and every form of Book the reference's decoder takes
+// (kernels/cuda/model/integer_vq.py:26-53, 163-192): the (256, 2) table of raw int8 basis values (its default), the
+// (512, 4) table of signed values at both parities (quantization/vq.py:44-69: shortbook) and the (256, 1) selector
+// words (shortbook + selectorbook).  All three become the middle one in LDS: for basis row b at parity p the eight
+// weights with every sign bit clear (+t + 1 - 2p) and with every sign bit set (-t + 1 - 2p), bytes wrapping as int8
+// arithmetic does; a code then picks each byte from one or the other by its sign bits.  A zero coordinate is
+// 1 - 2p either way, any even value decodes as the reference's word arithmetic does, nothing is assumed of the basis.
+enum BookForm { kBookSelector = 0, kBookRaw = 1, kBookSigned = 2 };
+__host__ __device__ constexpr int book_words(int form) { return form == kBookSelector ? 256 : form == kBookRaw ? 512 : 2048; }
+
 struct Q2GeneralTables {
-    uint2 basis[256];  // t
-    uint2 mask[256];   // mask3
-    uint2 zero[256];   // 0xFF where t == 0
+    uint4 value[512];  // [p * 256 + b]: .x/.y all signs clear (coordinates 0-3, 4-7), .z/.w all signs set
+    uint2 pick[256];   // [m]: 0xFF in byte j where sign bit SIGN_BITS[j] of the parity-adjusted low byte m is set
 };
 
-__device__ __forceinline__ uint2 byte_zero_mask(uint32_t selector) {
-    uint32_t lo = 0, hi = 0;
+// bytewise -t + d and t + d of four int8 values
+__device__ __forceinline__ uint32_t bytes_plus(uint32_t t, int d, bool negate) {
+    uint32_t out = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        if (((selector >> (4 * j)) & 3u) == 3u) lo |= 0xFFu << (8 * j);
-        if (((selector >> (4 * (j + 4))) & 3u) == 3u) hi |= 0xFFu << (8 * j);
+        const int v = (int)(int8_t)(t >> (8 * j));
+        out |= (uint32_t)(uint8_t)((negate ? -v : v) + d) << (8 * j);
     }
-    return make_uint2(lo, hi);
+    return out;
 }
 
-__device__ __forceinline__ void build_tables(Q2GeneralTables& t, const uint32_t* __restrict__ book, int tid, int threads) {
-    for (int i = tid; i < 256; i += threads) {
-        const uint32_t s = book[i];
-        t.basis[i] = byte_basis_signed(s);
-        t.zero[i] = byte_zero_mask(s);
-        t.mask[i] = byte_mask_signed((uint32_t)i);
+__device__ __forceinline__ void build_tables(Q2GeneralTables& t, const uint32_t* __restrict__ book, int form, int tid, int threads) {
+    for (int i = tid; i < 512; i += threads) {
+        const int row = i & 255, parity = i >> 8;
+        if (form == kBookSigned) {  // columns: low half +, low half -, high half +, high half - (vq.py:62-69)
+            const uint32_t* words = book + (int64_t)i * 4;
+            t.value[i] = make_uint4(words[0], words[2], words[1], words[3]);
+        } else {
+            uint2 basis;
+            if (form == kBookRaw)
+                basis = make_uint2(book[row * 2], book[row * 2 + 1]);
+            else
+                basis = byte_basis_signed(book[row]);
+            const int d = 1 - 2 * parity;
+            t.value[i] = make_uint4(bytes_plus(basis.x, d, false), bytes_plus(basis.y, d, false), bytes_plus(basis.x, d, true),
+                                    bytes_plus(basis.y, d, true));
+        }
+    }
+    for (int m = tid; m < 256; m += threads) {
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (sign_bit((uint32_t)m, j)) lo |= 0xFFu << (8 * j);
+            if (sign_bit((uint32_t)m, j + 4)) hi |= 0xFFu << (8 * j);
+        }
+        t.pick[m] = make_uint2(lo, hi);
     }
 }
 
 __device__ __forceinline__ uint2 decode_q2(const Q2GeneralTables& t, uint32_t code) {
-    const uint2 b = t.basis[(code >> 8) & 255u];
-    const uint2 m = t.mask[code & 255u];
-    const uint2 z = t.zero[(code >> 8) & 255u];
-    const uint32_t offset = (__popc(code & 255u) & 1u) ? 0xFFFFFFFFu : 0x01010101u;  // 1 - 2p in every byte
-    return make_uint2(((b.x ^ m.x) & ~z.x) | (offset & z.x), ((b.y ^ m.y) & ~z.y) | (offset & z.y));
+    const uint32_t parity = __popc(code & 255u) & 1u;
+    const uint4 v = t.value[parity * 256u + ((code >> 8) & 255u)];
+    const uint2 m = t.pick[(code & 255u) ^ parity];
+    return make_uint2((v.x & ~m.x) | (v.z & m.x), (v.y & ~m.y) | (v.w & m.y));
 }
 
 // Byte offset of the 16-byte chunk `q` (0..3: 32 weights each) of weight row `row` in the 128-wide

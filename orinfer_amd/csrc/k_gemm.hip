@@ -106,7 +106,8 @@ struct GemmParams {
     const __half* ws2;
     // routed single-stage codes, general form
     const uint16_t* patch;         // (E, K/128, N) patch words or null
-    int book_stride;               // selector words between the experts' tables (0: one table for all)
+    int book_stride;               // words between the experts' tables (0: one table for all)
+    int book_form;                 // BookForm of the general decode: selector words, raw int8 basis, signed values
     int direct_rows;               // > 0: no tile list; expert blockIdx.z owns rows [z * direct_rows, (z + 1) * direct_rows)
     uint32_t magnitudes_low, magnitudes_high;  // scalar Q4: the eight magnitudes, one per byte
 };
@@ -192,7 +193,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
         rows_here = min(BM, p.m - row0);
     }
 
-    if constexpr (CODEC == kQ4 || CODEC == kQ2) build_tables(tables, book, tid, 256);
+    if constexpr (GENERAL)
+        build_tables(tables, book, p.book_form, tid, 256);
+    else if constexpr (CODEC == kQ4 || CODEC == kQ2)
+        build_tables(tables, book, tid, 256);
 
     // int8 weights may end in half a K step (K a multiple of 64, int8_projection.py:29): the missing halves of
     // both operands are zeros.  Codes always come in whole steps.
@@ -1416,7 +1420,8 @@ int make_int8_swiglu(const Variant& v, orx_function* f) {
 // flags2: input form (0 int8 rows per slot, 1 int8 token rows gathered by slot, 2 fp16 rows quantised while
 // staged) + 4 * epilogue (0 plain, 1 SwiGLU).  Anything but 0 is a form of the resident kernel.
 // H (integer_vq_grouped only): 1 general decode, 2 patched, 4 one selector table per expert, 8 the list has a Patch.
-enum GroupedForm { kGeneralDecode = 1, kPatched = 2, kExpertTables = 4, kTakesPatch = 8 };
+// bits 4-5: the BookForm of the general decode
+enum GroupedForm { kGeneralDecode = 1, kPatched = 2, kExpertTables = 4, kTakesPatch = 8, kBookFormShift = 4 };
 
 bool grouped_uses_resident(const orx_function& f) {
     if (f.H & kGeneralDecode) return false;
@@ -1473,7 +1478,8 @@ int grouped_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
     if (f.H & kGeneralDecode) {
         p.patch = (f.H & kPatched) ? reinterpret_cast<const uint16_t*>(buffer("Patch")) : nullptr;
-        p.book_stride = (f.H & kExpertTables) ? 256 : 0;
+        p.book_form = (f.H >> kBookFormShift) & 3;
+        p.book_stride = (f.H & kExpertTables) ? book_words(p.book_form) : 0;
         p.tile_rows = f.block_m;
         return launch_mfma_general(f.block_m, p, g, stream);
     }
@@ -1490,7 +1496,7 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     f->tiles = (int)v.integer("tiles", 0, &bad);
     f->N = (int)v.integer("N", 0, &bad);
     f->K = (int)v.integer("K", 0, &bad);
-    f->block_m = (int)v.integer("block_m", 32, &bad);
+    f->block_m = (int)v.integer("block_m", f->symbol == "integer_vq_grouped" ? 16 : 32, &bad);  // integer_vq.py:314
     f->packed_k = (int)v.integer("packed_k", 128, &bad);
     const std::string grouped_algorithm = v.string("algorithm", "auto", &bad);
     const std::string input = v.string("input_dtype", "int8", &bad);
@@ -1501,13 +1507,15 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     const bool patched = vq && v.boolean("patched", false, &bad);
     const bool shared_table = !vq || v.boolean("shared_table", false, &bad);  // the reference's default (integer_vq.py:308)
     const std::string basis = vq ? v.string("basis", "spread29", &bad) : std::string("spread29");
-    // The reference factories' other keywords (integer_vq.py:300-322, e8p_decode.py:36-58): `kind` is e8p; Book is
-    // the (256, 1) selector table, which the reference calls shortbook + selectorbook (its raw-basis and sign-table
-    // forms of Book are not read here); the rest chooses among its own schedules and is accepted as a hint.
+    // The reference factories' other keywords (integer_vq.py:300-322, e8p_decode.py:36-58): `kind` is e8p; Book is the
+    // (256, 2) table of raw basis values unless shortbook (the (512, 4) table of signed values) or shortbook +
+    // selectorbook (the (256, 1) selector words) say otherwise, as in integer_vq.py:93-107; e8p_decode_grouped always
+    // takes selector words (e8p_decode.py:63).  The rest chooses among its own schedules and is accepted as a hint.
     const std::string kind = v.string("kind", "e8p", &bad);
-    const bool selector_book = v.boolean("selectorbook", true, &bad) && v.boolean("shortbook", true, &bad);
-    for (const char* hint : {"block_n", "num_stages", "stages", "byte_permute", "group_n", "warp_decode", "split_k", "parity_xor",
-                             "warp_private"})
+    const bool shortbook = vq ? v.boolean("shortbook", false, &bad) : true;
+    const bool selectorbook = vq ? v.boolean("selectorbook", false, &bad) : true;
+    const bool byte_permute = v.boolean("byte_permute", false, &bad);
+    for (const char* hint : {"block_n", "num_stages", "stages", "group_n", "warp_decode", "split_k", "parity_xor", "warp_private"})
         v.accept(hint);
     // dynamic_rows: the reference's kernel then takes the live row count as a trailing `m` (integer_vq.py:234-258
     // with kernels/shared/rows.py); the tile lists already bound every row these kernels touch, so `m` is taken
@@ -1515,10 +1523,11 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     f->dynamic_rows = v.boolean("dynamic_rows", false, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
-    if (kind != "e8p" || !selector_book) {
-        set_error("%s: kind must be e8p and Book the (256, 1) selector table (shortbook and selectorbook)", name);
+    if (kind != "e8p" || ((selectorbook || byte_permute) && !shortbook)) {  // integer_vq.py:83-97
+        set_error("%s: kind must be e8p; selectorbook and byte_permute need shortbook", name);
         return ORX_ERR_BAD_VARIANT;
     }
+    const int book_form = selectorbook ? kBookSelector : shortbook ? kBookSigned : kBookRaw;
     if (basis != "spread29" && basis != "any") {
         set_error("%s: basis must be spread29 (no zero coordinates: the XOR decoders) or any (selector ids 0-7)", name);
         return ORX_ERR_BAD_VARIANT;
@@ -1555,8 +1564,9 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     }
     // Zero coordinates, per-expert tables, patches, 8- and 16-row tile lists and 64-wide blocks are served by
     // the MFMA tiles with the general decode.
-    const bool general = patched || !shared_table || basis == "any" || small_tile || f->packed_k == 64;
-    f->H = (general ? kGeneralDecode : 0) | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | (vq ? kTakesPatch : 0);
+    const bool general = patched || !shared_table || basis == "any" || small_tile || f->packed_k == 64 || book_form != kBookSelector;
+    f->H = (general ? kGeneralDecode : 0) | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | (vq ? kTakesPatch : 0) |
+           (book_form << kBookFormShift);
     if (general && (f->flags2 != 0 || (f->algorithm != kAuto && f->algorithm != kMfma))) {
         set_error("%s: patched, shared_table=false, basis=any, block_m 8|16 and packed_k=64 run on the MFMA tiles "
                   "(algorithm auto or mfma, int8 rows, plain epilogue)", name);
@@ -1633,7 +1643,8 @@ int vq_direct_launch(const orx_function& f, int rows, const Geometry& g, hipStre
     p.ws = pointer_arg<const __half>(args, 6);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity, p.packed_k = f.packed_k, p.out_f32 = 0;
     p.expert_weight_stride = (int64_t)f.N * (f.K / 8) * 2;
-    p.book_stride = (f.H & kExpertTables) ? 256 : 0;
+    p.book_form = (f.H >> kBookFormShift) & 3;
+    p.book_stride = (f.H & kExpertTables) ? book_words(p.book_form) : 0;
     p.direct_rows = f.M;
     return launch_mfma_general(f.block_m, p, g, stream);
 }
@@ -1644,18 +1655,22 @@ int make_vq_direct(const Variant& v, orx_function* f) {
     f->M = (int)v.integer("M", 0, &bad);
     f->N = (int)v.integer("N", 0, &bad);
     f->K = (int)v.integer("K", 0, &bad);
-    const int block_m = (int)v.integer("block_m", 32, &bad);
+    const int block_m = (int)v.integer("block_m", 16, &bad);  // integer_vq.py:275
     f->packed_k = (int)v.integer("packed_k", 128, &bad);
     const bool patched = v.boolean("patched", false, &bad);
     const bool shared_table = v.boolean("shared_table", false, &bad);  // integer_vq.py:271
     const std::string kind = v.string("kind", "e8p", &bad);
-    const bool selector_book = v.boolean("selectorbook", true, &bad) && v.boolean("shortbook", true, &bad);
-    for (const char* hint : {"block_n", "num_stages", "byte_permute"}) v.accept(hint);
+    // Book (integer_vq.py:93-107): raw basis values (256, 2), signed values (512, 4) with shortbook, selector words
+    // (256, 1) with shortbook + selectorbook
+    const bool shortbook = v.boolean("shortbook", false, &bad), selectorbook = v.boolean("selectorbook", false, &bad);
+    const bool byte_permute = v.boolean("byte_permute", false, &bad);
+    for (const char* hint : {"block_n", "num_stages"}) v.accept(hint);
     if (bad) return ORX_ERR_BAD_VARIANT;
-    if (kind != "e8p" || !selector_book) {
-        set_error("integer_vq: kind must be e8p and Book the (256, 1) selector table (shortbook and selectorbook)");
+    if (kind != "e8p" || ((selectorbook || byte_permute) && !shortbook)) {
+        set_error("integer_vq: kind must be e8p; selectorbook and byte_permute need shortbook");
         return ORX_ERR_BAD_VARIANT;
     }
+    const int book_form = selectorbook ? kBookSelector : shortbook ? kBookSigned : kBookRaw;
     if (f->E <= 0 || f->M <= 0 || f->N <= 0 || f->K <= 0 || f->K % 128 || (int64_t)f->K * 128 * 128 > 2147483647LL ||
         (int64_t)f->E * f->M > 2147483647LL) {
         set_error("integer_vq: invalid integer VQ geometry");  // integer_vq.py:86
@@ -1671,7 +1686,7 @@ int make_vq_direct(const Variant& v, orx_function* f) {
     }
     f->capacity = f->E * f->M;
     f->block_m = block_m < 32 ? 32 : block_m;  // 8 and 16 rows ride in a 32-row tile: the row ranges are the same
-    f->H = kGeneralDecode | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | kTakesPatch;
+    f->H = kGeneralDecode | (patched ? kPatched : 0) | (shared_table ? 0 : kExpertTables) | kTakesPatch | (book_form << kBookFormShift);
     const uint32_t nullable = 0x80000000u;
     f->args = {{"A", ArgPointer, 16}, {"AS", ArgPointer, 2}, {"Book", ArgPointer, 4}, {"C", ArgPointer, 2},
                {"P", ArgPointer, 16}, {"Patch", ArgPointer, patched ? 2u : nullable | 2u}, {"WS", ArgPointer, 2}};
@@ -1860,10 +1875,12 @@ const Registration* gemm_registrations(int* count) {
      "rows, E, tiles, N, K, block_m=32|64|128, packed_k=128|0, dynamic_rows=false, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_vq", make_vq_direct,
-     "E, M (rows of every expert), N, K, block_m=32|8|16|64, packed_k=128|64|0, patched=false, shared_table=false",
+     "E, M (rows of every expert), N, K, block_m=16|8|32|64, packed_k=128|64|0, patched=false, shared_table=false, shortbook=false, "
+     "selectorbook=false (Book: raw basis (256,2) | signed values (512,4) with shortbook | selector words (256,1) with both)",
      "A,AS,Book,C,P,Patch,WS"},
     {"integer_vq_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128|8|16, packed_k=128|64|0, dynamic_rows=false, patched=false, shared_table=false, basis=spread29|any, "
+     "rows, E, tiles, N, K, block_m=16|8|32|64|128, packed_k=128|64|0, dynamic_rows=false, patched=false, shared_table=false, shortbook=false, "
+     "selectorbook=false (Book as for integer_vq), basis=spread29|any, "
      "algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_experts", make_integer_experts,

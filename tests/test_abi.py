@@ -416,26 +416,33 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
         kern = lib.Kernel("integer_vq_grouped", **shape, **extra)
         assert kern.arg_names == want, extra
         grid, block, _ = kern.geometry()
-        if extra != dict(shared_table=True):  # one table per expert is the reference's default (integer_vq.py:308)
-            assert tuple(grid)[:2] == (1, 16) and tuple(block)[0] == 256, extra
+        # the reference's defaults (a raw basis table per expert, 16-row tiles: integer_vq.py:304-314) are the general decode
+        assert tuple(grid)[:2] == (1, 16) and tuple(block)[0] == 256, extra
+    # the selector Book of one table for all on 32-row tiles is what the XOR kernels take
+    xor = lib.Kernel("integer_vq_grouped", **shape, shared_table=True, shortbook=True, selectorbook=True, block_m=32)
+    assert xor.arg_names == want and xor.geometry()[1][0] == 512
     assert "Patch" not in lib.Kernel("e8p_decode_grouped", **shape).arg_names
     for symbol, bad in (("integer_vq_grouped", dict(patched=True, algorithm="stream")),
                         ("integer_vq_grouped", dict(algorithm="stream")),
                         ("integer_vq_grouped", dict(shared_table=True, basis="any", algorithm="resident")),
                         ("integer_vq_grouped", dict(basis="e8")),
                         ("integer_vq_grouped", dict(block_m=24)),
+                        ("integer_vq_grouped", dict(selectorbook=True)),           # integer_vq.py:95-97: needs shortbook
+                        ("integer_vq_grouped", dict(byte_permute=True)),
                         ("integer_vq_grouped", dict(packed_k=32)),
                         ("e8p_decode_grouped", dict(block_m=8)),
                         ("e8p_decode_grouped", dict(packed_k=64))):
         with pytest.raises(lib.OrxError):
             lib.Kernel(symbol, **shape, **bad)
     # the fused forms keep their places around Patch
-    fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", shared_table=True)
+    xor_book = dict(shared_table=True, shortbook=True, selectorbook=True, block_m=32)
+    fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", **xor_book)
     assert fused.arg_names == ["A", "AS", "Book", "C", "Counts", "Offsets", "P", "Patch", "Q", "RowMax", "TileCount",
                                "TileExpert", "TileRow", "WS"]
     with pytest.raises(lib.OrxError):
-        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", shared_table=True,
-                   patched=True)
+        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", patched=True, **xor_book)
+    with pytest.raises(lib.OrxError):  # the fused forms are forms of the XOR kernels: not with the default raw Book
+        lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", shared_table=True)
     # the form without a tile list: every expert multiplies its own M rows (integer_vq.py:217-228)
     direct = lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, block_m=16, patched=True)
     assert direct.arg_names == ["A", "AS", "Book", "C", "P", "Patch", "WS"]
@@ -525,16 +532,21 @@ def test_routed_decode_symbols_take_the_reference_factories_keywords():
     shape = dict(rows=99, E=3, tiles=16, N=65, K=256)
     hints = dict(kind="e8p", shared_table=True, patched=False, block_m=32, block_n=128, shortbook=True, selectorbook=True,
                  num_stages=1, byte_permute=True)
-    assert lib.Kernel("integer_vq_grouped", **shape, **hints).geometry() == lib.Kernel("integer_vq_grouped", **shape, shared_table=True).geometry()
+    assert lib.Kernel("integer_vq_grouped", **shape, **hints).geometry()[1][0] == 512  # the XOR kernels (streaming)
+    assert lib.Kernel("integer_vq_grouped", **shape, shared_table=True).geometry()[1][0] == 256  # raw Book: the general decode
     lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, kind="e8p", shortbook=True, selectorbook=True, num_stages=2, block_n=128, byte_permute=True)
     lib.Kernel("e8p_decode_grouped", **shape, block_n=32, split_k=2, parity_xor=True)
     dynamic = lib.Kernel("integer_vq_grouped", **shape, shared_table=True, dynamic_rows=True)
     assert dynamic.arg_names[-1] == "m" and dynamic.arg_names[:-1] == lib.Kernel("integer_vq_grouped", **shape, shared_table=True).arg_names
-    for bad in (dict(selectorbook=False), dict(shortbook=False), dict(kind="scalar")):
+    for bad in (dict(selectorbook=True, shortbook=False), dict(byte_permute=True, shortbook=False), dict(kind="scalar")):
         with pytest.raises(lib.OrxError):
             lib.Kernel("integer_vq_grouped", **shape, **bad)
         with pytest.raises(lib.OrxError):
             lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, **bad)
+    # the other two forms of Book resolve: signed values (shortbook alone) and raw basis values (the default)
+    for book in (dict(shortbook=True), dict(shortbook=True, byte_permute=True), dict()):
+        lib.Kernel("integer_vq_grouped", **shape, **book)
+        lib.Kernel("integer_vq", E=3, M=17, N=65, K=256, **book)
 
 
 REFERENCE_KEYWORDS = {

@@ -1008,6 +1008,8 @@ def test_five_launches_at_the_largest_gathered_batch_give_the_bits_of_seven():
 @pytest.mark.parametrize("bm,m,patched,shared", [(8, 1, False, True), (8, 3, True, False), (16, 17, True, True),
                                                  (32, 33, False, False), (64, 65, False, True), (128, 130, True, False)])
 def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
+    # Book in each of the reference's three forms (integer_vq.py:93-107), by case: raw basis values, signed values, selectors
+    form = ("raw", "signed", "selector")[(bm // 8 + packed_k // 64) % 3]
     rng = np.random.default_rng(orc.SEED + bm + packed_k)
     e, n, k = 3, 65, 256
     tables, codes, patches = [], [], []
@@ -1020,7 +1022,9 @@ def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
         patches.append(words)
     codes = np.stack(codes)
     patch_np = np.stack([w.T for w in patches])  # (E, K/128, N)
-    book_np = np.stack([orc.selector_table(t) for t in (tables[:1] if shared else tables)])
+    book_of = dict(raw=orc.basis_words, signed=orc.sign_table, selector=orc.selector_table)[form]
+    book_flags = dict(raw={}, signed=dict(shortbook=True), selector=dict(shortbook=True, selectorbook=True))[form]
+    book_np = np.stack([book_of(t) for t in (tables[:1] if shared else tables)])
     weights = np.stack([orc.q2_integers(codes[x], tables[x], patches[x] if patched else None) for x in range(e)])
     ws = np.full((e, n), 0.015625, np.float16)
     counts_np = np.full(e, m, np.int32)
@@ -1033,7 +1037,7 @@ def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
     k128 = np.stack([orc.q2_pack_k128(c) for c in codes])
     stored = codes if packed_k == 0 else k128 if packed_k == 128 else orc.q2_repack_k64(k128)
     kern = gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
-                     patched=patched, shared_table=shared, basis="any")
+                     patched=patched, shared_table=shared, basis="any", **book_flags)
     out = torch.full((rows + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
     book, patch = gu.dev(book_np), gu.dev(patch_np) if patched else None
     counts = gu.dev(counts_np)
@@ -1050,7 +1054,7 @@ def test_integer_vq_grouped_general_decode(bm, m, patched, shared, packed_k):
     small = np.abs(exact) < 2048
     np.testing.assert_array_equal(got[:rows][small].astype(np.float64) * 8192, exact[small])
     # tables and patches are read at launch time: an all-zero table leaves 1 - 2p and the patches
-    book.copy_(gu.dev(np.stack([orc.selector_table(np.zeros((256, 8), np.int8))] * book_np.shape[0])))
+    book.copy_(gu.dev(np.stack([book_of(np.zeros((256, 8), np.int8))] * book_np.shape[0])))
     zero_w = np.stack([orc.q2_integers(codes[x], np.zeros((256, 8), np.int8), patches[x] if patched else None) for x in range(e)])
     kern(**args)
     np.testing.assert_array_equal(gu.host(out)[:rows], orc.grouped_project(a_q, a_s[:, None], zero_w, ws, counts_np, offsets_np))
@@ -1088,7 +1092,8 @@ def test_integer_vq_grouped_default_form_matches_e8p_decode_grouped():
     want = orc.grouped_project(a_q, a_s[:, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np, offsets_np)
     for patch in (None, gu.dev(np.zeros(1, np.uint16))):
         out = torch.full((rows, n), 55.0, dtype=torch.float16, device=gu.DEV)
-        gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, shared_table=True)(
+        gu.kernel("integer_vq_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, shared_table=True, shortbook=True,
+                  selectorbook=True)(
             A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=gu.dev(counts_np), Offsets=gu.dev(offsets_np),
             P=gu.dev(stored), Patch=patch, TileCount=gu.dev(total), TileExpert=gu.dev(te), TileRow=gu.dev(tr), WS=gu.dev(ws))
         np.testing.assert_array_equal(gu.host(out), want)
@@ -1116,9 +1121,13 @@ def test_integer_vq_direct_form(bm, m, patched, shared, packed_k):
     a_s = np.full(e * m, 0.0078125, np.float16)
     k128 = np.stack([orc.q2_pack_k128(c) for c in codes])
     stored = codes if packed_k == 0 else k128 if packed_k == 128 else orc.q2_repack_k64(k128)
-    book_np = np.stack([orc.selector_table(t) for t in (tables[:1] if shared else tables)])
+    form = ("signed", "selector", "raw")[(bm // 8 + packed_k // 64) % 3]  # integer_vq.py:93-107
+    book_of = dict(raw=orc.basis_words, signed=orc.sign_table, selector=orc.selector_table)[form]
+    book_flags = dict(raw={}, signed=dict(shortbook=True, byte_permute=True), selector=dict(shortbook=True, selectorbook=True))[form]
+    book_np = np.stack([book_of(t) for t in (tables[:1] if shared else tables)])
     out = torch.full((e * m + 1, n), 91.0, dtype=torch.float16, device=gu.DEV)
-    kern = gu.kernel("integer_vq", E=e, M=m, N=n, K=k, block_m=bm, packed_k=packed_k, patched=patched, shared_table=shared)
+    kern = gu.kernel("integer_vq", E=e, M=m, N=n, K=k, block_m=bm, packed_k=packed_k, patched=patched, shared_table=shared,
+                     **book_flags)
     kern(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.dev(book_np), C=out, P=gu.dev(stored),
          Patch=gu.dev(np.stack([w.T for w in patches])) if patched else None, WS=gu.dev(ws))
     counts = np.full(e, m, np.int32)
@@ -1143,7 +1152,7 @@ def test_grouped_q2_with_dynamic_rows_takes_m_last(symbol):
     cap = orc.tile_capacity(cap_rows, e, bm)
     te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
     stored = np.stack([orc.q2_pack_k128(c) for c in codes])
-    extra = dict(shared_table=True) if symbol == "integer_vq_grouped" else {}
+    extra = dict(shared_table=True, shortbook=True, selectorbook=True) if symbol == "integer_vq_grouped" else {}
     kern = gu.kernel(symbol, rows=cap_rows, E=e, tiles=cap, N=n, K=k, block_m=bm, dynamic_rows=True, **extra)
     assert kern.arg_names[-1] == "m"
     out = torch.full((cap_rows, n), 55.0, dtype=torch.float16, device=gu.DEV)
@@ -1237,3 +1246,27 @@ def test_router_projection_logits_and_shared_gate(m, h, e):
     for bad in (dict(H=100), dict(block_k=512), dict(block_m=8), dict(stages=3), dict(E=0)):
         with pytest.raises(Exception):
             gu.kernel("router_projection", **{**dict(M=4, H=256, E=8), **bad})
+
+
+def test_integer_vq_raw_basis_with_values_beyond_the_e8p_palette():
+    # the default Book is the (256, 2) table of raw int8 basis values (integer_vq.py:104-107, :188-192): any even value
+    # decodes as +-t + (1 - 2p) in int8 arithmetic, -128 included (its negative wraps to itself, as in the reference's
+    # word arithmetic, integer_vq.py:26-39); the signed-value table gives the same weights
+    rng = np.random.default_rng(orc.SEED + 41)
+    e, m, n, k = 2, 9, 96, 256
+    table = (rng.integers(-64, 64, (256, 8)) * 2).astype(np.int8)
+    table[0] = [-128, 126, 0, -2, 4, 100, -100, 8]
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    codes[0, 0, :4] = [0x0000, 0x00FF, 0x0001, 0x0080]  # row 0 with no sign, every sign, odd parity with one sign each way
+    wide = np.stack([orc.e8p_decode(c, table).reshape(n, k) for c in codes]).astype(np.int64)
+    weights = ((wide + 128) % 256 - 128).astype(np.int8)
+    a_q = rng.integers(-128, 128, (e * m, k), dtype=np.int8)
+    a_s = np.full(e * m, 0.0078125, np.float16)
+    ws = np.full((e, n), 0.015625, np.float16)
+    want = orc.grouped_project(a_q, a_s[:, None], weights, ws, np.full(e, m, np.int32), np.arange(e, dtype=np.int32) * m)
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    for flags, book in ((dict(), orc.basis_words(table)), (dict(shortbook=True), orc.sign_table(table))):
+        out = torch.full((e * m, n), 91.0, dtype=torch.float16, device=gu.DEV)
+        gu.kernel("integer_vq", E=e, M=m, N=n, K=k, shared_table=True, **flags)(
+            A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.dev(book[None]), C=out, P=gu.dev(stored), Patch=None, WS=gu.dev(ws))
+        np.testing.assert_array_equal(gu.host(out), want)

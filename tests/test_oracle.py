@@ -850,3 +850,25 @@ def test_row_q4_every_signed_nibble_and_the_byte_permute_form():
         got[:, i] = byte.astype(np.uint8).view(np.int8)
     want = orc.row_q4_integers(words.astype(np.uint16).reshape(-1, 1), magnitudes)
     np.testing.assert_array_equal(got, want)
+
+
+def test_sign_table_rows_are_the_decodes_with_no_and_with_every_sign(table):
+    """python/orinfer_build/quantization/vq.py:44-69: row p * 256 + b holds +t + (1 - 2p) and -t + (1 - 2p) for the two halves
+    of basis row b, which is what the codes with sign byte 0x00 / 0xFF (even parity) and 0x01 / 0xFE (odd parity: the
+    parity bit itself is flipped back) decode to; a hand-made row with -128 wraps as int8 arithmetic does."""
+    signs = orc.sign_table(table)
+    assert signs.shape == (512, 4) and signs.dtype == np.uint32
+    rows = np.arange(256, dtype=np.uint16) << 8
+    for parity, plain, flipped in ((0, 0x00, 0xFF), (1, 0x01, 0xFE)):
+        positive = orc.e8p_decode(rows | plain, table)
+        negative = orc.e8p_decode(rows | flipped, table)
+        block = signs[parity * 256:(parity + 1) * 256]
+        np.testing.assert_array_equal(block[:, 0], np.ascontiguousarray(positive[:, :4]).view("<u4").reshape(256))
+        np.testing.assert_array_equal(block[:, 1], np.ascontiguousarray(negative[:, :4]).view("<u4").reshape(256))
+        np.testing.assert_array_equal(block[:, 2], np.ascontiguousarray(positive[:, 4:]).view("<u4").reshape(256))
+        np.testing.assert_array_equal(block[:, 3], np.ascontiguousarray(negative[:, 4:]).view("<u4").reshape(256))
+    odd = np.zeros((256, 8), np.int8)
+    odd[0] = [-128, 126, 0, -2, 4, 100, -100, 8]
+    hand = orc.sign_table(odd)
+    assert hand[0, 0] == 0xFF017F81 and hand[0, 1] == 0x03018381  # +t + 1: 81 7F 01 FF;  -t + 1: 81 83 01 03
+    assert hand[256, 0] == 0xFDFF7D7F and hand[256, 1] == 0x01FF817F  # +t - 1: 7F 7D FF FD;  -t - 1: 7F 81 FF 01
