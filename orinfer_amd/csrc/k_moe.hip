@@ -925,7 +925,7 @@ int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStrea
 int make_metadata(const Variant& v, orx_function* f) {
     if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
     bool bad = false;
-    f->block_m = (int)v.integer("block_m", 16, &bad);
+    f->block_m = (int)v.integer("block_m", 8, &bad);  // moe.py:714
     if (bad) return ORX_ERR_BAD_VARIANT;
     // one expert per thread, one route per lane; the reference's own form is decode-only (M <= 1024)
     if (f->M <= 0 || f->E <= 0 || f->E > kMetaThreads || f->top_k <= 0 || f->top_k > f->E || !valid_block_m(f->block_m) ||
@@ -1067,7 +1067,9 @@ int make_dispatch(const Variant& v, orx_function* f) {
     if (!geometry_fields(v, f, true)) return ORX_ERR_BAD_VARIANT;
     bool bad = false;
     f->H = (int)v.integer("H", 0, &bad);
-    f->group = (int)v.integer("scale_group", f->H, &bad);
+    // moe.py:286: 64 channels share a scale unless the record says otherwise (fp16 rows, quantised here, have one per row)
+    const std::string input_kind = v.string("input_dtype", "int8", &bad);
+    f->group = (int)v.integer("scale_group", input_kind == "float16" ? f->H : 64, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     if (f->M <= 0 || f->H <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || f->group <= 0 || f->H % f->group) {
         set_error("expert_dispatch: invalid MoE activation dispatch dimensions");
@@ -1152,7 +1154,7 @@ const Registration* moe_registrations(int* count) {
      "IDs,Offsets,Slots[,m]"},
     {"expert_offsets", make_offsets, "E=512, block_m=16", "Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_tiles", make_tiles, "M, E=512, top_k=10, block_m=16", "Counts,TileExpert,TileOffsets,TileRow"},
-    {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=16, dynamic_rows=false, slot_maps=false",
+    {"route_metadata", make_metadata, "M, E=512, top_k=10, block_m=8, dynamic_rows=false, slot_maps=false",
      "Counts,IDs,RelativeSlot[,RowMax],RowOffsets[,SlotMap,SlotToken],TileCount,TileExpert,TileOffsets,TileRow[,m]"},
     {"single_route_metadata", make_single_metadata, "E=512, top_k=10, capacity=11",
      "Counts,IDs,Offsets,Relative,TileCount,TileExpert,TileOffsets,TileRow"},
@@ -1160,7 +1162,7 @@ const Registration* moe_registrations(int* count) {
      "ColdCount,ColdOffsets,Counts,RowOffsets,TileCount,TileOffsets"},
     {"expert_partition_tiles", make_partition_tiles, "M, experts, top_k, hot_m, cold_m, cold_rows, dynamic_rows=false",
      "ColdExpert,ColdOffsets,ColdRow,Counts,TileExpert,TileOffsets,TileRow[,m]"},
-    {"expert_dispatch", make_dispatch, "M, H, E=512, top_k=10, scale_group=H, dynamic_rows=false",
+    {"expert_dispatch", make_dispatch, "M, H, E=512, top_k=10, scale_group=64, dynamic_rows=false, input_dtype=int8|float16 (one scale per row)",
      "A,D,DS,IDs,RelativeSlot,RowOffsets,Scale,SlotMap[,m]"},
     {"moe_combine", make_combine, "M, H, slots=M*top_k, top_k=10, dynamic_rows=false",
      "Expert,Output,Prob,Shared,SharedGate,SlotMap[,m]"},

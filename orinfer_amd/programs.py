@@ -128,7 +128,7 @@ class MoeLayer:
         # the row layout allows it
         self.fused_dispatch = fused_dispatch and hidden % 8 == 0
         self.k_a8 = Kernel("activation_quantization", K=hidden)
-        self.k_dispatch = Kernel("expert_dispatch", H=hidden, **common,
+        self.k_dispatch = Kernel("expert_dispatch", H=hidden, scale_group=hidden, **common,
                                  **({"input_dtype": "float16"} if self.fused_dispatch else {}))
         # signs: the layer's input is rotated first (block-128 signed Hadamard); rotation, A8 and the
         # scatter to the expert-sorted slots are one launch (kernels/cuda/model/rotation_a8.py:558-604)

@@ -70,8 +70,8 @@ def test_routing_metadata_and_dispatch(m, e, k, bm):
     d = torch.zeros((m * k, h), dtype=torch.int8, device=gu.DEV)
     ds = torch.zeros((m * k, 1), dtype=torch.float16, device=gu.DEV)
     slot = torch.full((m, k), -1, **I32)
-    gu.kernel("expert_dispatch", M=m, H=h, E=e, top_k=k)(A=gu.dev(a_q), D=d, DS=ds, IDs=ids, RelativeSlot=relative,
-                                                       RowOffsets=rows, Scale=gu.dev(a_s), SlotMap=slot)
+    gu.kernel("expert_dispatch", M=m, H=h, E=e, top_k=k, scale_group=h)(A=gu.dev(a_q), D=d, DS=ds, IDs=ids, RelativeSlot=relative,
+                                                                       RowOffsets=rows, Scale=gu.dev(a_s), SlotMap=slot)
     want_d, want_ds, want_slot = orc.expert_dispatch(a_q, a_s, ids_np, want_rel, want_rows)
     np.testing.assert_array_equal(gu.host(slot), want_slot)
     np.testing.assert_array_equal(gu.host(d), want_d)
@@ -811,7 +811,7 @@ def test_rotate_expert_a8_rotates_quantises_and_scatters_in_one_launch(m, e, k, 
     # the two launches it replaces give the same bits
     two = fresh()
     gu.kernel("rotate_activation_a8", **common)(Q=two["q"], S=two["s"], Signs=d_signs, X=d_x, m=m)
-    gu.kernel("expert_dispatch", M=cap, H=h, E=e, top_k=k, dynamic_rows=True)(
+    gu.kernel("expert_dispatch", M=cap, H=h, E=e, top_k=k, scale_group=h, dynamic_rows=True)(
         A=two["q"], D=two["d"], DS=two["ds"], IDs=d_ids, RelativeSlot=d_rel, RowOffsets=d_off, Scale=two["s"],
         SlotMap=two["slot_map"], m=m)
     for name in ("q", "s", "d", "ds", "slot_map"):
@@ -1270,3 +1270,24 @@ def test_integer_vq_raw_basis_with_values_beyond_the_e8p_palette():
         gu.kernel("integer_vq", E=e, M=m, N=n, K=k, shared_table=True, **flags)(
             A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.dev(book[None]), C=out, P=gu.dev(stored), Patch=None, WS=gu.dev(ws))
         np.testing.assert_array_equal(gu.host(out), want)
+
+
+def test_expert_dispatch_default_scale_groups_of_64_channels():
+    # moe.py:286-329: a record without scale_group carries one scale per 64 channels, Scale (M, H / 64) -> DS (slots, H / 64)
+    rng = np.random.default_rng(orc.SEED + 51)
+    m, e, k, h = 13, 8, 3, 192
+    ids_np = np.stack([rng.choice(e, k, replace=False) for _ in range(m)]).astype(np.int32)
+    counts, relative = orc.expert_histogram(ids_np, e)
+    offsets, _, _ = orc.expert_offsets(counts, 16)
+    a_q = rng.integers(-127, 128, (m, h), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.02, (m, h // 64)).astype(np.float16)
+    d = torch.zeros((m * k, h), dtype=torch.int8, device=gu.DEV)
+    ds = torch.zeros((m * k, h // 64), dtype=torch.float16, device=gu.DEV)
+    slot = torch.full((m, k), -1, **I32)
+    gu.kernel("expert_dispatch", M=m, H=h, E=e, top_k=k)(A=gu.dev(a_q), D=d, DS=ds, IDs=gu.dev(ids_np), RelativeSlot=gu.dev(relative),
+                                                       RowOffsets=gu.dev(offsets), Scale=gu.dev(a_s), SlotMap=slot)
+    want_d, want_ds, want_slot = orc.expert_dispatch(a_q, a_s, ids_np, relative, offsets)
+    np.testing.assert_array_equal(gu.host(slot), want_slot)
+    np.testing.assert_array_equal(gu.host(d), want_d)
+    np.testing.assert_array_equal(gu.host(ds), want_ds)
+    assert gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2).geometry() == gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2, block_m=8).geometry()
