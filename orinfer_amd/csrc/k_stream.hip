@@ -113,9 +113,11 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
         if (tile >= p.tile_count[0]) return;
         const int expert = p.tile_expert[tile];
         const int first = p.tile_row[tile];
-        if (PLANES && p.list_rows != p.tile_rows && first % p.tile_rows != 0) return;  // the second of two merged tiles
+        // a tile list in steps of fewer rows than a workgroup takes: the workgroup of the first tile of a stretch takes
+        // them all (tiles of one expert are adjacent and start at multiples of the list's step)
+        if (p.list_rows != p.tile_rows && first % p.tile_rows != 0) return;
         row0 = p.offsets[expert] + first;
-        rows_here = min(PLANES ? p.tile_rows : CB * 32, p.counts[expert] - first);
+        rows_here = min(p.tile_rows, p.counts[expert] - first);
         if (rows_here <= 0) return;
         w_base += (int64_t)expert * p.expert_weight_stride;
         ws += (int64_t)expert * p.n;
@@ -373,6 +375,8 @@ int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, 
     p.n = n, p.k = k, p.stride = n, p.m = 0, p.packed_k = packed_k, p.out_f32 = 0;
     p.counts = counts, p.offsets = offsets, p.tile_expert = tile_expert, p.tile_row = tile_row, p.tile_count = tile_count;
     p.expert_weight_stride = (int64_t)n * (k / 8) * 2;
+    // lists in steps of 8 or 16 rows (the reference's own decode kernels take 8: e8p_decode.py:36-58): 32 rows per workgroup
+    p.tile_rows = block_m <= 32 ? 32 : 64, p.list_rows = block_m < 32 ? block_m : p.tile_rows;
     Geometry g;
     stream_grouped_geometry(n, tiles, &g);
     return launch_codec<kQ2, true, kGroupedSplits>(block_m <= 32 ? 1 : 2, p, dim3(g.grid[0], g.grid[1]), stream);

@@ -422,6 +422,8 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
     xor = lib.Kernel("integer_vq_grouped", **shape, shared_table=True, shortbook=True, selectorbook=True, block_m=32)
     assert xor.arg_names == want and xor.geometry()[1][0] == 512
     assert "Patch" not in lib.Kernel("e8p_decode_grouped", **shape).arg_names
+    # tile lists in steps of 8 rows, as the reference's decode kernel and route_metadata's default build them
+    assert lib.Kernel("e8p_decode_grouped", **shape, block_m=8).geometry()[1][0] == 512
     for symbol, bad in (("integer_vq_grouped", dict(patched=True, algorithm="stream")),
                         ("integer_vq_grouped", dict(algorithm="stream")),
                         ("integer_vq_grouped", dict(shared_table=True, basis="any", algorithm="resident")),
@@ -430,7 +432,9 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
                         ("integer_vq_grouped", dict(selectorbook=True)),           # integer_vq.py:95-97: needs shortbook
                         ("integer_vq_grouped", dict(byte_permute=True)),
                         ("integer_vq_grouped", dict(packed_k=32)),
-                        ("e8p_decode_grouped", dict(block_m=8)),
+                        ("e8p_decode_grouped", dict(block_m=8, algorithm="resident")),  # 8-row lists: the streaming kernel only
+                        ("e8p_decode_grouped", dict(block_m=16, epilogue="swiglu", gather=True)),
+                        ("e8p_decode_grouped", dict(block_m=24)),
                         ("e8p_decode_grouped", dict(packed_k=64))):
         with pytest.raises(lib.OrxError):
             lib.Kernel(symbol, **shape, **bad)

@@ -1291,3 +1291,34 @@ def test_expert_dispatch_default_scale_groups_of_64_channels():
     np.testing.assert_array_equal(gu.host(d), want_d)
     np.testing.assert_array_equal(gu.host(ds), want_ds)
     assert gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2).geometry() == gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2, block_m=8).geometry()
+
+
+@pytest.mark.parametrize("bm", [8, 16])
+def test_e8p_decode_grouped_takes_tile_lists_in_steps_of_8_and_16_rows(bm):
+    # the reference's decode kernel multiplies 8-row tiles (e8p_decode.py:36-58) and route_metadata builds such lists by
+    # default (moe.py:714): here the workgroup of the first tile of every stretch of 32 rows takes the whole stretch
+    rng = np.random.default_rng(orc.SEED + 61 + bm)
+    e, n, k = 6, 160, 512
+    counts_np = np.array([3, 0, 41, 32, 1, 17], np.int32)
+    rows = int(counts_np.sum())
+    codes = rng.integers(0, 65536, (e, n, k // 8), dtype=np.uint16)
+    ws = rng.uniform(0.005, 0.02, (e, n)).astype(np.float16)
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_s = rng.uniform(0.01, 0.03, rows).astype(np.float16)
+    meta = {name: torch.full(shape, -1, **I32) for name, shape in
+            dict(Counts=(e,), RelativeSlot=(rows, 1), RowOffsets=(e,), TileCount=(1,), TileOffsets=(e,)).items()}
+    ids = np.repeat(np.arange(e, dtype=np.int32), counts_np)[:, None]
+    cap = orc.tile_capacity(rows, e, bm)
+    meta["TileExpert"], meta["TileRow"] = torch.full((cap,), -1, **I32), torch.full((cap,), -1, **I32)
+    gu.kernel("route_metadata", M=rows, E=e, top_k=1, block_m=bm)(IDs=gu.dev(ids), **meta)
+    assert int(meta["TileCount"].cpu()[0]) == int(np.sum((counts_np + bm - 1) // bm))
+    out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
+    gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm)(
+        A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=meta["Counts"], Offsets=meta["RowOffsets"],
+        P=gu.dev(np.stack([orc.q2_pack_k128(c) for c in codes])), TileCount=meta["TileCount"], TileExpert=meta["TileExpert"],
+        TileRow=meta["TileRow"], WS=gu.dev(ws))
+    want = orc.grouped_project(a_q, a_s[:, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np,
+                               gu.host(meta["RowOffsets"]))
+    got = gu.host(out)
+    np.testing.assert_array_equal(got[:rows], want)
+    assert (got[rows] == 55).all()
