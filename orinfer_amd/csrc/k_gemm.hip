@@ -1557,18 +1557,18 @@ int make_q2_grouped(const Variant& v, orx_function* f) {
     // route_metadata builds such lists by default): integer_vq_grouped runs them on the MFMA tiles, e8p_decode_grouped on
     // the streaming kernel, whose workgroup takes the stretch of up to 32 rows that starts at a multiple of 32
     const bool small_list = f->block_m == 8 || f->block_m == 16;
-    const bool small_tile = vq && small_list;
+    const bool small_tile = small_list && (vq || f->packed_k == 64);  // 64-wide blocks are read by the MFMA tiles only
     if (f->block_m != 32 && f->block_m != 64 && f->block_m != 128 && !small_list) {
         set_error("%s: block_m must be 8, 16, 32, 64 or 128 (row step of the routed tile list)", name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (small_list && !vq && (f->flags2 != 0 || (f->algorithm != kAuto && f->algorithm != kStream))) {
+    if (small_list && !small_tile && (f->flags2 != 0 || (f->algorithm != kAuto && f->algorithm != kStream))) {
         set_error("%s: tile lists in steps of 8 or 16 rows run on the streaming kernel (algorithm auto or stream, int8 rows, plain epilogue)",
                   name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->packed_k != 128 && f->packed_k != 0 && !(vq && f->packed_k == 64)) {
-        set_error("%s: packed_k must be 128 (K-major)%s or 0 (row-major per expert)", name, vq ? ", 64" : "");
+    if (f->packed_k != 128 && f->packed_k != 64 && f->packed_k != 0) {  // e8p_decode.py:43, integer_vq.py:75
+        set_error("%s: packed_k must be 128 or 64 (K-major blocks) or 0 (row-major per expert)", name);
         return ORX_ERR_BAD_VARIANT;
     }
     // Zero coordinates, per-expert tables, patches, 8- and 16-row tile lists and 64-wide blocks are served by
@@ -1881,7 +1881,7 @@ const Registration* gemm_registrations(int* count) {
     {"int8_swiglu", make_int8_swiglu, "M, N, K, dynamic_rows=false, algorithm=tensor_core|dp4a, block_m, block_n (checked, not used)",
      "A,Gate,GateScale,Output,TokenScale,Up,UpScale[,m]"},
     {"e8p_decode_grouped", make_q2_grouped,
-     "rows, E, tiles, N, K, block_m=32|64|128|8|16 (row step of the tile list), packed_k=128|0, dynamic_rows=false, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
+     "rows, E, tiles, N, K, block_m=32|64|128|8|16 (row step of the tile list), packed_k=128|64|0, dynamic_rows=false, algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_vq", make_vq_direct,
      "E, M (rows of every expert), N, K, block_m=16|8|32|64, packed_k=128|64|0, patched=false, shared_table=false, shortbook=false, "

@@ -435,9 +435,15 @@ def test_integer_vq_grouped_takes_the_reference_patch_buffer():
                         ("e8p_decode_grouped", dict(block_m=8, algorithm="resident")),  # 8-row lists: the streaming kernel only
                         ("e8p_decode_grouped", dict(block_m=16, epilogue="swiglu", gather=True)),
                         ("e8p_decode_grouped", dict(block_m=24)),
-                        ("e8p_decode_grouped", dict(packed_k=64))):
+                        ("e8p_decode_grouped", dict(packed_k=32)),
+                        ("e8p_decode_grouped", dict(packed_k=64, algorithm="stream")),  # 64-wide blocks: the MFMA tiles only
+                        ("e8p_decode_grouped", dict(packed_k=64, algorithm="resident")),
+                        ("e8p_decode_grouped", dict(packed_k=64, epilogue="swiglu"))):
         with pytest.raises(lib.OrxError):
             lib.Kernel(symbol, **shape, **bad)
+    # K-major blocks of 64 codes per channel, which the reference's decode kernel takes too (e8p_decode.py:43), at every list step
+    for bm in (8, 16, 32, 64, 128):
+        assert lib.Kernel("e8p_decode_grouped", **shape, packed_k=64, block_m=bm).geometry()[1][0] == 256
     # the fused forms keep their places around Patch
     xor_book = dict(shared_table=True, shortbook=True, selectorbook=True, block_m=32)
     fused = lib.Kernel("integer_vq_grouped", rows=2048, E=128, tiles=192, N=2048, K=512, input_dtype="float16", **xor_book)

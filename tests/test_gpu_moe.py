@@ -112,7 +112,7 @@ def test_route_metadata_one_launch(m, e, k, bm, repeats):
 
 
 @pytest.mark.parametrize("algorithm", ["auto", "mfma"])
-@pytest.mark.parametrize("packed_k", [128, 0])
+@pytest.mark.parametrize("packed_k", [128, 64, 0])
 @pytest.mark.parametrize("bm", [32, 64, 128])
 def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k, algorithm):
     # count mixes in the spirit of tests/cuda/operators/e8p_exact.py:141-198: empty experts,
@@ -130,6 +130,8 @@ def test_grouped_q2_gemm_counts_tiles_and_masks(bm, packed_k, algorithm):
     cap = orc.tile_capacity(rows, e, bm)
     te, tr = orc.expert_tiles(counts_np, tile_offsets, bm, cap)
     stored = codes if packed_k == 0 else np.stack([orc.q2_pack_k128(c) for c in codes])
+    if packed_k == 64:  # e8p_decode.py:43,62: blocks of 64 codes per channel
+        stored = orc.q2_repack_k64(stored)
     out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
     kern = gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k,
                      algorithm=algorithm)
@@ -1293,8 +1295,9 @@ def test_expert_dispatch_default_scale_groups_of_64_channels():
     assert gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2).geometry() == gu.lib.Kernel("route_metadata", M=64, E=16, top_k=2, block_m=8).geometry()
 
 
+@pytest.mark.parametrize("packed_k", [128, 64])
 @pytest.mark.parametrize("bm", [8, 16])
-def test_e8p_decode_grouped_takes_tile_lists_in_steps_of_8_and_16_rows(bm):
+def test_e8p_decode_grouped_takes_tile_lists_in_steps_of_8_and_16_rows(bm, packed_k):
     # the reference's decode kernel multiplies 8-row tiles (e8p_decode.py:36-58) and route_metadata builds such lists by
     # default (moe.py:714): here the workgroup of the first tile of every stretch of 32 rows takes the whole stretch
     rng = np.random.default_rng(orc.SEED + 61 + bm)
@@ -1313,9 +1316,12 @@ def test_e8p_decode_grouped_takes_tile_lists_in_steps_of_8_and_16_rows(bm):
     gu.kernel("route_metadata", M=rows, E=e, top_k=1, block_m=bm)(IDs=gu.dev(ids), **meta)
     assert int(meta["TileCount"].cpu()[0]) == int(np.sum((counts_np + bm - 1) // bm))
     out = torch.full((rows + 1, n), 55.0, dtype=torch.float16, device=gu.DEV)
-    gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm)(
+    stored = np.stack([orc.q2_pack_k128(c) for c in codes])
+    if packed_k == 64:  # blocks of 64 codes per channel (e8p_decode.py:43,62): the 8- and 16-row tiles of the MFMA kernel
+        stored = orc.q2_repack_k64(stored)
+    gu.kernel("e8p_decode_grouped", rows=rows, E=e, tiles=cap, N=n, K=k, block_m=bm, packed_k=packed_k)(
         A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), C=out, Counts=meta["Counts"], Offsets=meta["RowOffsets"],
-        P=gu.dev(np.stack([orc.q2_pack_k128(c) for c in codes])), TileCount=meta["TileCount"], TileExpert=meta["TileExpert"],
+        P=gu.dev(stored), TileCount=meta["TileCount"], TileExpert=meta["TileExpert"],
         TileRow=meta["TileRow"], WS=gu.dev(ws))
     want = orc.grouped_project(a_q, a_s[:, None], np.stack([orc.q2_integers(c, TABLE) for c in codes]), ws, counts_np,
                                gu.host(meta["RowOffsets"]))
