@@ -101,6 +101,7 @@ struct GemmParams {
     const int* tile_count;
     int64_t expert_weight_stride;  // bytes between experts in w
     int tile_rows;                 // rows a routed tile may hold (0: the kernel's own tile height)
+    int list_split;                // workgroups per listed tile when its rows exceed the kernel's tile (0 or 1: one)
     int* partials;                 // split launches: int32 partial tiles, two slots per workgroup
     const void* w2;                // gate/up + SwiGLU: the Up matrix (w is Gate) and its scales
     const __half* ws2;
@@ -174,10 +175,11 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
             row0 = expert * p.direct_rows + first;
             rows_here = min(BM, p.direct_rows - first);
         } else {
-            const int tile = blockIdx.y;
+            const int split = p.list_split > 1 ? p.list_split : 1;  // a listed tile of split * BM rows: one workgroup per BM
+            const int tile = split > 1 ? blockIdx.y / split : blockIdx.y;
             if (tile >= p.tile_count[0]) return;
             expert = p.tile_expert[tile];
-            first = p.tile_row[tile];
+            first = p.tile_row[tile] + (split > 1 ? (int)(blockIdx.y % split) * BM : 0);
             row0 = p.offsets[expert] + first;
             rows_here = min(p.tile_rows > 0 ? min(BM, p.tile_rows) : BM, p.counts[expert] - first);
         }
@@ -1713,7 +1715,7 @@ int make_vq_direct(const Variant& v, orx_function* f) {
 int experts_geometry(const orx_function& f, int rows, Geometry* g) {
     (void)rows;
     g->grid[0] = ceil_div((uint32_t)f.N, 128u);
-    g->grid[1] = (uint32_t)f.tiles;
+    g->grid[1] = (uint32_t)f.tiles * (f.block_m == 256 ? 2u : 1u);  // a listed tile of 256 rows: two MFMA tiles of 128
     g->block[0] = 256;
     return ORX_OK;
 }
@@ -1734,6 +1736,7 @@ int experts_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     p.ws = pointer_arg<const __half>(args, 10);
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = f.capacity * f.top_k, p.out_f32 = 0;
     p.tile_rows = f.block_m;
+    p.list_split = f.block_m == 256 ? 2 : 0;
     const int bm = f.block_m <= 32 ? 32 : f.block_m <= 64 ? 64 : 128;
     if (f.flags == kQ4) {
         p.packed_k = 128;
@@ -1762,12 +1765,13 @@ int make_integer_experts(const Variant& v, orx_function* f) {
     (void)v.integer("tail_m", 0, &bad);
     if (bad) return ORX_ERR_BAD_VARIANT;
     const bool w8 = codec == "w8";
-    const bool block_m_ok = f->block_m == 8 || f->block_m == 16 || f->block_m == 32 || f->block_m == 64 || f->block_m == 128;
+    const bool block_m_ok = f->block_m == 8 || f->block_m == 16 || f->block_m == 32 || f->block_m == 64 || f->block_m == 128 ||
+                            f->block_m == 256;  // moe.py:77
     if (f->M <= 0 || f->N <= 0 || f->K <= 0 || f->E <= 0 || f->top_k <= 0 || f->top_k > f->E || f->K % 128 || !block_m_ok ||
         (block_n != 32 && block_n != 64 && block_n != 128) || (!w8 && codec != "e8p_q4") ||
         (w8 && (f->block_m == 8 || block_n == 32)) || (block_k != 128 && block_k != 256) || f->K % block_k ||
         (stages != 1 && stages != 2) || minimum_blocks <= 0 || (int64_t)f->K * 128 * 128 > 2147483647LL) {
-        set_error("integer_experts: invalid grouped integer projection geometry (block_m 8..128 here)");
+        set_error("integer_experts: invalid grouped integer projection geometry");
         return ORX_ERR_BAD_VARIANT;
     }
     f->flags = w8 ? kW8 : kQ4;
@@ -1893,7 +1897,7 @@ const Registration* gemm_registrations(int* count) {
      "algorithm=auto|stream|resident|mfma, input_dtype=int8|float16, gather=false, epilogue=none|swiglu",
      "A,AS[,Act],Book,C,Counts,Offsets,P,Patch[,Q][,RowMax][,SlotToken],TileCount,TileExpert,TileRow,WS[,m]"},
     {"integer_experts", make_integer_experts,
-     "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..128), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
+     "M, N, K, E, top_k, codec=e8p_q4|w8, block_m=16 (8..256), dynamic_rows=false, block_n, block_k, stages, tail_m, minimum_blocks",
      "A,AS,Book,Counts,Offsets,Out,TileCount,TileExpert,TileRow,W,WS[,m]"},
     {"e8p_q4_unpack", make_q4_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},
     {"e8p_q2_unpack", make_q2_unpack, "N, K, packed_k=0|64|128", "Book,Output,W"},

@@ -585,10 +585,11 @@ def test_expert_partition_matches_oracle(experts, hot_m, cold_m, cold_rows):
 
 # ---- routed Q4 / W8 banks (integer_experts) -----------------------------------------------------
 @pytest.mark.parametrize("codec,bm", [("e8p_q4", 8), ("e8p_q4", 16), ("e8p_q4", 64), ("e8p_q4", 128), ("w8", 16),
-                                      ("w8", 32), ("w8", 128)])
+                                      ("w8", 32), ("w8", 128), ("e8p_q4", 256), ("w8", 256)])
 def test_integer_experts_q4_and_w8_banks(codec, bm):
     rng = np.random.default_rng(orc.SEED + bm + len(codec))
-    e, n, k, m, top_k = 9, 200, 384, 40, 3
+    e, n, k, top_k = 9, 200, 384, 3
+    m = 300 if bm == 256 else 40  # 256-row lists (moe.py:77): the hot expert fills both halves of a listed tile and a tail
     logits = rng.normal(size=(m, e)).astype(np.float32)
     logits[:, 4] = -50  # an expert nobody picks
     logits[:, 2] += 3   # a hot one
@@ -657,7 +658,7 @@ def test_integer_experts_dynamic_rows_and_refusals():
         want = orc.grouped_project(a_q[:rows], a_s[:rows, None], weights, ws, counts_np, offsets_np)
         np.testing.assert_array_equal(gu.host(out)[:rows], want)
         assert (gu.host(out)[rows:] == 55).all()
-    for variant in (dict(block_m=256), dict(block_m=12), dict(codec="w8", block_m=8), dict(codec="w8", block_n=32),
+    for variant in (dict(block_m=512), dict(block_m=12), dict(codec="w8", block_m=8), dict(codec="w8", block_n=32),
                     dict(codec="q2"), dict(K=192), dict(top_k=7), dict(block_k=256, K=384), dict(stages=3)):
         base = dict(M=8, N=64, K=256, E=6, top_k=2)
         base.update(variant)
