@@ -684,3 +684,34 @@ def test_scalar_q4_symbols_bind_as_the_reference_does_and_refuse_what_it_refuses
     for bad in (dict(block_m=9), dict(BN=32), dict(block_m=0)):
         with pytest.raises(lib.OrxError):
             lib.Kernel("q4_gemv", **{**shape, **bad})
+
+
+# Values that the reference's factories take for a keyword (the `not in (...)` checks of kernels/cuda/model/e8p_q4.py:79-196,
+# e8p_decode.py:43-49, integer_vq.py:87-99, int8_projection.py:33-39, q4_projection.py:143-149, e8p_exact.py:63-66,
+# e8p_prefill.py:167-171, moe.py:77,216,562): each resolves here, on top of the other keywords of the same factory.
+REFERENCE_VALUES = [
+    ("e8p_q4_projection", "block_m", (8, 16, 32, 64, 96, 128, 192, 256)), ("e8p_q4_projection", "block_n", (32, 64, 128)),
+    ("e8p_q4_projection", "split_k", (1, 2, 4)), ("e8p_q4_projection", "group_m", (0, 1, 2, 4, 8)),
+    ("e8p_q4_projection", "packed_k", (0, 64, 128)), ("int8_projection", "block_m", (16, 32, 64, 128, 256)),
+    ("int8_projection", "block_n", (64, 128)), ("int8_projection", "block_k", (64, 128)),
+    ("int8_projection", "group_m", (0, 1, 2, 4, 8)), ("q4_projection", "block_m", (8, 16, 32, 64, 128)),
+    ("q4_projection", "group_m", (0, 1, 2, 4, 8)), ("integer_vq", "block_m", (8, 16, 32, 64)), ("integer_vq", "block_n", (64, 128)),
+    ("integer_vq", "num_stages", (1, 2)), ("integer_vq", "packed_k", (64, 128)), ("integer_vq_grouped", "block_m", (8, 16, 32, 64)),
+    ("integer_vq_grouped", "packed_k", (64, 128)), ("e8p_decode_grouped", "packed_k", (64, 128)),
+    ("e8p_decode_grouped", "block_n", (32, 64, 128)), ("e8p_decode_grouped", "split_k", (1, 2, 4)),
+    ("e8p_exact_grouped", "block_m", (8, 16)), ("e8p_exact_grouped", "stages", (2, 3, 4)),
+    ("integer_experts", "block_m", (8, 16, 32, 64, 128, 256)), ("integer_experts", "codec", ("w8", "e8p_q4")),
+    ("expert_offsets", "block_m", (8, 16, 32, 64, 128, 256)), ("expert_tiles", "block_m", (8, 16, 32, 64, 128, 256)),
+    ("expert_histogram_local", "block", (512, 1024, 2048)), ("router_topk_warp", "warps", (1, 2, 4)),
+    ("activation_quantization", "threads", (128, 256, 512)),
+]
+
+
+@pytest.mark.parametrize("symbol,key,values", REFERENCE_VALUES, ids=[f"{s}-{k}" for s, k, _ in REFERENCE_VALUES])
+def test_every_value_the_reference_factory_takes_resolves(symbol, key, values):
+    for value in values:
+        variant = dict(REFERENCE_KEYWORDS[symbol])
+        variant[key] = value
+        if symbol == "integer_experts" and (variant.get("codec") == "w8") and variant.get("block_m") == 8:
+            variant["block_m"] = 16  # moe.py:80: W8 banks take no 8-row tiles
+        lib.Kernel(symbol, **variant)
