@@ -23,7 +23,7 @@ INT8_PEAK_TOPS = 5000.0        # MI355X published dense int8 MFMA (5.0 POP/s)
 CACHE_BYTES = 256 << 20        # Infinity Cache
 
 # HBM bytes per launch of the contract kernel come from the committed counter summary (two
-# `rocprofv3 --pmc` runs of `bench.py --traffic-probe`: FETCH_SIZE, then WRITE_SIZE, each scaled by what
+# `rocprofv3 --pmc` runs of `bench.py --profile-traffic`: FETCH_SIZE, then WRITE_SIZE, each scaled by what
 # the same counter reads for a device copy of known size in the same run).  The summary records the
 # launch it was taken on; `measured_traffic` gives nothing when that is not what the handle launches now.
 TRAFFIC_SUMMARY = ROOT / "profiles" / "gemv_q4_config1_m1_hbm_traffic.txt"
@@ -57,21 +57,12 @@ def parse():
     p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--no-extra", action="store_true", help="only the contract workload")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    p.add_argument("--rows-probe", type=int, default=0, metavar="ROWS",
-                   help="launch config 1's projection at ROWS rows once per weight copy, eagerly, and exit (for counter runs of "
-                        "the kernel that serves that row count)")
-    p.add_argument("--traffic-probe", action="store_true",
-                   help="for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a plain copy of known size, then the "
+    p.add_argument("--profile-rows", type=int, default=0, metavar="ROWS",
+                   help="workload for a rocprofv3 counter run: config 1's projection at ROWS rows once per weight copy, "
+                        "eagerly, then exit")
+    p.add_argument("--profile-traffic", action="store_true",
+                   help="workload for `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE`: a plain copy of known size, then the "
                         "contract kernel once per weight copy, eagerly; no timing")
-    p.add_argument("--mfma-probe", action="store_true",
-                   help="the int8 matrix pipe alone: v_mfma_i32_32x32x32_i8 back to back from registers, with zero and "
-                        "with random operands (the ceiling the GEMM fractions are read against); no other workload")
-    p.add_argument("--read-probe", action="store_true",
-                   help="a plain streaming read of 12.5, 44.6 and 178 MB (the code bytes of configs 0 and 1 and four times "
-                        "that), rotating more buffers than the caches hold: the rate that bounds the GEMV; no other workload")
-    p.add_argument("--lds-probe", action="store_true",
-                   help="random 4-byte reads of a 256-entry LDS table stored once, 32 and 64 times (what a code's decode "
-                        "lookups cost); no other workload")
     return p.parse_args()
 
 
@@ -161,70 +152,21 @@ def main():
                 self.quantize(s)
                 self.project(i, s)
 
-    if args.mfma_probe:
-        # rates of the matrix pipe by itself; long launches, so that the power controller has settled
-        iterations = 20000
-        out = torch.empty(1024, dtype=torch.int32, device="cuda")
-        report = {}
-        for operands in ("zero", "random"):
-            probe = Kernel("int8_mfma_probe", iterations=iterations, operands=operands)
-            cus = probe.geometry()[0][0]
-            for _ in range(2):
-                probe(stream=stream.cuda_stream, Out=out)
-            torch.cuda.synchronize()
-            seconds = timed_graph(lambda i, s: probe(stream=s, Out=out), 4)
-            ops = cus * 8 * iterations * 8 * 65536.0
-            report[operands] = {"ms_per_launch": round(seconds * 1e3, 3), "TOPS": round(ops / seconds / 1e12, 1),
-                                "frac_int8_peak": round(ops / seconds / 1e12 / INT8_PEAK_TOPS, 4)}
-        print(json.dumps({"int8_mfma_probe": dict(report, compute_units=cus, waves_per_cu=8, iterations=iterations,
-                                                  ops_per_launch=cus * 8 * iterations * 8 * 65536)}))
-        return
-    if args.lds_probe:
-        out = torch.zeros(1, dtype=torch.int32, device="cuda")
-        iterations, report = 2000, {}
-        for copies in (1, 32, 64):
-            probe = Kernel("lds_lookup_probe", iterations=iterations, copies=copies)
-            seconds = timed_graph(lambda i, s: probe(stream=s, Out=out), 8)
-            wave_instructions_per_cu = 16 * iterations * 8
-            report[f"copies_{copies}"] = {"us_per_launch": round(seconds * 1e6, 2),
-                                          "ns_per_wave_lookup_per_cu": round(seconds * 1e9 / wave_instructions_per_cu, 3),
-                                          "lane_lookups_per_ns_per_cu": round(64 * wave_instructions_per_cu / seconds / 1e9, 2)}
-        print(json.dumps({"lds_lookup_probe": dict(report, waves_per_cu=16, iterations=iterations, lookups_per_iteration=8)}))
-        return
-    if args.read_probe:
-        out = torch.zeros(1, dtype=torch.int32, device="cuda")
-        report = {}
-        for label, size in (("config0_codes", 9728 * 2560 // 2), ("config1_codes", 17408 * 5120 // 2),
-                            ("four_times_config1", 4 * 17408 * 5120 // 2)):
-            sources = [torch.empty(size, dtype=torch.uint8, device="cuda").random_(0, 256)
-                       for _ in range(-(-2 * CACHE_BYTES // size))]
-            best = None
-            for per_cu in (4, 8, 16):
-                probe = Kernel("hbm_read_probe", bytes=size, workgroups_per_cu=per_cu)
-                seconds = timed_graph(lambda i, s: probe(stream=s, Out=out, Source=sources[i % len(sources)]),
-                                      max(2 * len(sources), 26))
-                if best is None or seconds < best[0]:
-                    best = (seconds, per_cu)
-            report[label] = {"bytes": size, "us_per_launch": round(best[0] * 1e6, 3), "GBps": round(size / best[0] / 1e9, 1),
-                             "frac_hbm_peak": round(size / best[0] / 1e9 / HBM_PEAK_GBS, 4), "workgroups_per_cu": best[1]}
-            del sources
-        print(json.dumps({"hbm_read_probe": report}))
-        return
     # ---- contract workload: config 1, M=1 ----
     c1 = workloads.config1(1)
     bytes_c1 = workloads.algorithmic_bytes_q4(1, c1["n"], c1["k"])
     copies = -(-2 * CACHE_BYTES // (c1["n"] * c1["k"] // 2))  # aggregate footprint >= 2x the cache
     main_case = Q4Case(c1, copies, fused_input=True)
-    if args.rows_probe:
-        case = Q4Case(workloads.config1(args.rows_probe), copies)
+    if args.profile_rows:
+        case = Q4Case(workloads.config1(args.profile_rows), copies)
         case.quantize(stream.cuda_stream)
         for i in range(copies):
             case.project(i, stream.cuda_stream)
         torch.cuda.synchronize()
-        grid, block, shared = case.proj.geometry(args.rows_probe)
-        print(json.dumps({"rows_probe": {"rows": args.rows_probe, "launches": copies, "grid": list(grid), "block": list(block), "lds": shared}}))
+        grid, block, shared = case.proj.geometry(args.profile_rows)
+        print(json.dumps({"profile_rows": {"rows": args.profile_rows, "launches": copies, "grid": list(grid), "block": list(block), "lds": shared}}))
         return
-    if args.traffic_probe:
+    if args.profile_traffic:
         # counter calibration: a device copy reads and writes exactly `probe.numel()` bytes
         probe = torch.empty(c1["n"] * c1["k"] // 2, dtype=torch.uint8, device="cuda").random_(0, 256)
         target = torch.empty_like(probe)
@@ -234,7 +176,7 @@ def main():
             main_case.step(i, stream.cuda_stream)
         torch.cuda.synchronize()
         grid, block, shared = main_case.fused.geometry(1)
-        print(json.dumps({"traffic_probe": {"copy_bytes_read": probe.numel(), "copy_bytes_written": probe.numel(),
+        print(json.dumps({"profile_traffic": {"copy_bytes_read": probe.numel(), "copy_bytes_written": probe.numel(),
                                             "projection_launches": copies, "algorithmic_bytes": bytes_c1,
                                             "grid": grid[0], "block": block[0], "lds": shared}}))
         return
@@ -261,12 +203,6 @@ def main():
     main_case.quantize(stream.cuda_stream)
     plain_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(min(args.steps, 260), copies))
     traffic_bytes, traffic_kernel = measured_traffic(main_case.fused.geometry(1))
-    # what a read of the same code bytes reaches on this box when nothing is done with them
-    read_probe = Kernel("hbm_read_probe", bytes=c1["n"] * c1["k"] // 2, workgroups_per_cu=4)
-    probe_out = torch.zeros(1, dtype=torch.int32, device="cuda")
-    read_seconds = timed_graph(lambda i, s: read_probe(stream=s, Out=probe_out, Source=main_case.weights[i % copies]),
-                               max(min(args.steps, 260), copies))
-    read_rate = c1["n"] * c1["k"] // 2 / read_seconds / 1e9
     # config 0 (the reference's own CPU-runnable shape) on the same kernel: a second roofline entry
     c0 = workloads.config0()
     b0 = workloads.algorithmic_bytes_q4(1, c0["n"], c0["k"])
@@ -295,9 +231,6 @@ def main():
                      "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "us_per_launch": round(kernel_seconds * 1e6, 3), "traffic": traffic_bytes,
-                     "plain_read_of_the_codes": {"us_per_launch": round(read_seconds * 1e6, 3), "GBps": round(read_rate, 1),
-                                                 "frac": round(read_rate / HBM_PEAK_GBS, 4),
-                                                 "kernel_vs_plain_read": round(achieved / read_rate, 4)},
                      "same_kernel_int8_input": {"us_per_launch": round(plain_seconds * 1e6, 3),
                                                 "achieved": round(bytes_c1 / plain_seconds / 1e9, 1),
                                                 "frac": round(bytes_c1 / plain_seconds / 1e9 / HBM_PEAK_GBS, 4)},

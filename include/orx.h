@@ -92,6 +92,14 @@ int orx_release(orx_fn f);
  * (kernels.rs:150-170): limits the caller validates its launch record against. */
 int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes);
 
+/* The same for the kernel that a launch of `rows` live rows starts (rows <= 0: the variant's own M,
+ * which is what orx_query reports).  A projection handle picks its kernel by the live rows (one-row
+ * GEMV, batched-decode kernels, MFMA tiles): the attributes are read from that kernel, the one whose
+ * grid, block and LDS bytes orx_geometry returns for the same rows, so a record per row range
+ * (crates/orinfer-model-sdk/src/operators/rows.rs:14-58) is validated against its own function as
+ * kernels.rs:150-170 validates a cubin's.  Enqueues nothing. */
+int orx_query_rows(orx_fn f, int32_t rows, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes);
+
 /* The launch geometry a package would record for this kernel: the static grid of a
  * fixed-row kernel, or the RowExpression result of a dynamic one for `rows` live rows
  * (crates/orinfer-model-sdk/src/operators/dynamic.rs:93-118).  rows <= 0 means the
@@ -137,7 +145,11 @@ int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32
  * (orx_workspace_bytes tells) fails with ORX_ERR_WORKSPACE and enqueues nothing.  Calls no
  * allocator.  All calls on one device share that device's array: calls that overlap in time on
  * one device (two streams) race; calls in stream order do not (nothing in the array has to
- * survive from one launch to the next, and nothing has to be zero when a launch starts). */
+ * survive from one launch to the next, and nothing has to be zero when a launch starts).
+ * The array's address is looked up once per device, for the calling thread's current device:
+ * orx_resolve of a workspace handle does it for the device current then, so resolve (or launch
+ * once) with the launch device current before a capture begins; a first launch on a device whose
+ * address is not known yet, on a stream that is capturing, fails with ORX_ERR_BAD_ARGUMENT. */
 int orx_launch_static_scratch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
                               void* hip_stream, void** args);
 

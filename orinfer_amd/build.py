@@ -8,7 +8,7 @@ from pathlib import Path
 HERE = Path(__file__).resolve().parent
 CSRC = HERE / "csrc"
 LIBRARY = HERE / "liborx.so"
-SOURCES = ["orx_api.cpp", "k_quant.hip", "k_gemv.hip", "k_gemm.hip", "k_gemm_big.hip", "k_stream.hip", "k_dense.hip", "k_wide.hip", "k_grouped.hip", "k_moe.hip", "k_planes.hip", "k_rowq4.hip", "k_probe.hip"]
+SOURCES = ["orx_api.cpp", "k_quant.hip", "k_gemv.hip", "k_gemm.hip", "k_gemm_big.hip", "k_stream.hip", "k_dense.hip", "k_wide.hip", "k_grouped.hip", "k_moe.hip", "k_planes.hip", "k_rowq4.hip"]
 # -packed-fp32-ops off: this pool has seen wrong results from compiler-made v_pk_*_f32.
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",

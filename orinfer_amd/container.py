@@ -111,6 +111,11 @@ def kernel_record(name, family, variant, bindings, rows=0):
 
     bindings: argument name -> buffer name | (buffer name, byte offset) | int (scalar).  The grid,
     block and LDS bytes are the library's own for `rows` live rows (0 = the variant's M)."""
+    # An optional buffer that this program does not use (bound to None) leaves the argument list through the
+    # variant's `omit` key: the record's arguments stay within the engine's `Argument` kinds (artifact.rs:184-194).
+    unused = [arg_name for arg_name, bound in bindings.items() if bound is None]
+    if unused:
+        variant = dict(variant, omit=",".join(sorted(unused)))
     kernel = lib.Kernel(family, **variant)
     grid, block, shared = kernel.geometry(rows)
     args = []
@@ -118,9 +123,7 @@ def kernel_record(name, family, variant, bindings, rows=0):
         if arg_name not in bindings:
             raise KeyError(f"{family}: no binding for argument {arg_name}")
         bound = bindings[arg_name]
-        if bound is None:
-            args.append({"kind": "null"})  # an optional buffer that this program does not use
-        elif kind == 1:
+        if kind == 1:
             args.append({"kind": "i32", "value": int(bound)})
         elif isinstance(bound, tuple):
             args.append({"kind": "buffer_slice", "name": bound[0], "offset": int(bound[1])})
@@ -345,8 +348,6 @@ def fixture_manifest(buffers, records, validation, *, rows=None):
                 args.append({"buffer": arg["name"]})
             elif arg["kind"] == "buffer_slice":
                 args.append({"buffer": arg["name"], "offset": arg["offset"]})
-            elif arg["kind"] == "null":
-                args.append({"null": True})
             else:
                 args.append({"i32": arg["value"]})
         entry = {"symbol": record["symbol"], "grid": record["grid"], "block": record["block"],

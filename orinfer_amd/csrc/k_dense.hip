@@ -435,7 +435,7 @@ int launch_shape(const DenseParams& p, hipStream_t stream) {
     });
     if (ready != ORX_OK) return ready;
     const int workgroups = workgroups_for(p.m, p.k);
-    hipLaunchKernelGGL((dense_resident_kernel<W, S, CB, P>), dim3(workgroups), dim3(W * 64), lds_bytes(p.n, workgroups),
+    ORX_LAUNCH((dense_resident_kernel<W, S, CB, P>), dim3(workgroups), dim3(W * 64), lds_bytes(p.n, workgroups),
                        stream, p);
     return hip_check(hipGetLastError(), "launch projection (resident)");
 }
@@ -460,7 +460,7 @@ int launch_specialized_shape(const DenseParams& p, hipStream_t stream) {
                          "hipFuncSetAttribute");
     });
     if (ready != ORX_OK) return ready;
-    hipLaunchKernelGGL((dense_specialized_kernel<S, CB, KM>), dim3(device_compute_units()), dim3(kSpecThreads),
+    ORX_LAUNCH((dense_specialized_kernel<S, CB, KM>), dim3(device_compute_units()), dim3(kSpecThreads),
                        specialized_lds_bytes(p.n, p.k), stream, p);
     return hip_check(hipGetLastError(), "launch projection (resident, loader waves)");
 }

@@ -652,13 +652,13 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
     const dim3 grid(g.grid[0], g.grid[1]), block(256);
     switch (bm) {
         case 32:
-            hipLaunchKernelGGL((gemm_kernel<CODEC, 32, 128, 1, GROUPED>), grid, block, 0, stream, p);
+            ORX_LAUNCH((gemm_kernel<CODEC, 32, 128, 1, GROUPED>), grid, block, 0, stream, p);
             break;
         case 64:
-            hipLaunchKernelGGL((gemm_kernel<CODEC, 64, 128, 2, GROUPED>), grid, block, 0, stream, p);
+            ORX_LAUNCH((gemm_kernel<CODEC, 64, 128, 2, GROUPED>), grid, block, 0, stream, p);
             break;
         default:
-            hipLaunchKernelGGL((gemm_kernel<CODEC, 128, 128, 2, GROUPED>), grid, block, 0, stream, p);
+            ORX_LAUNCH((gemm_kernel<CODEC, 128, 128, 2, GROUPED>), grid, block, 0, stream, p);
             break;
     }
     return hip_check(hipGetLastError(), "launch projection (mfma)");
@@ -668,11 +668,11 @@ int launch_mfma(int bm, const GemmParams& p, const Geometry& g, hipStream_t stre
 int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStream_t stream) {
     const dim3 grid(g.grid[0], g.grid[1], g.grid[2]), block(256);
     if (bm <= 32)
-        hipLaunchKernelGGL((gemm_kernel<kQ2, 32, 128, 1, true, false, true>), grid, block, 0, stream, p);
+        ORX_LAUNCH((gemm_kernel<kQ2, 32, 128, 1, true, false, true>), grid, block, 0, stream, p);
     else if (bm == 64)
-        hipLaunchKernelGGL((gemm_kernel<kQ2, 64, 128, 2, true, false, true>), grid, block, 0, stream, p);
+        ORX_LAUNCH((gemm_kernel<kQ2, 64, 128, 2, true, false, true>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((gemm_kernel<kQ2, 128, 128, 2, true, false, true>), grid, block, 0, stream, p);
+        ORX_LAUNCH((gemm_kernel<kQ2, 128, 128, 2, true, false, true>), grid, block, 0, stream, p);
     return hip_check(hipGetLastError(), "launch routed projection (general decode)");
 }
 
@@ -807,11 +807,11 @@ uint64_t projection_workspace(const orx_function& f, int rows) {
 
 template <int CODEC>
 int launch_split(const GemmParams& p, int groups, hipStream_t stream) {
-    hipLaunchKernelGGL((gemm_split_kernel<CODEC>), dim3(groups), dim3(256), 0, stream, p);
+    ORX_LAUNCH((gemm_split_kernel<CODEC>), dim3(groups), dim3(256), 0, stream, p);
     int code = hip_check(hipGetLastError(), "launch projection (mfma, split K steps)");
     if (code != ORX_OK) return code;
     const uint32_t tiles = ceil_div((uint32_t)p.n, 128u) * ceil_div((uint32_t)p.m, 128u);
-    hipLaunchKernelGGL(gemm_split_finish_kernel, dim3(4 * tiles), dim3(256), 0, stream, p, groups);
+    ORX_LAUNCH(gemm_split_finish_kernel, dim3(4 * tiles), dim3(256), 0, stream, p, groups);
     return hip_check(hipGetLastError(), "launch projection (mfma, sum of split tiles)");
 }
 
@@ -1114,7 +1114,7 @@ __global__ __launch_bounds__(256) void row_q4_unpack_kernel(const uint32_t* __re
 int row_q4_unpack(const void* w, void* out, int n, int k, uint32_t low, uint32_t high, hipStream_t stream) {
     const int64_t pairs = (int64_t)n * (k / 8);
     const int blocks = (int)std::min<int64_t>((pairs + 255) / 256, 4096);
-    hipLaunchKernelGGL(row_q4_unpack_kernel, dim3(blocks), dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(w),
+    ORX_LAUNCH(row_q4_unpack_kernel, dim3(blocks), dim3(256), 0, stream, reinterpret_cast<const uint32_t*>(w),
                        reinterpret_cast<uint2*>(out), pairs, low, high);
     return hip_check(hipGetLastError(), "launch unpack_q4");
 }
@@ -1190,7 +1190,7 @@ int row_q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
         p.partials = pointer_arg<int>(args, f.workspace_arg);
         return launch_split<kS4>(p, split_groups_for(f, rows), stream);
     }
-    hipLaunchKernelGGL((gemm_kernel<kS4, 128, 128, 2, false>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, p);
+    ORX_LAUNCH((gemm_kernel<kS4, 128, 128, 2, false>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, p);
     return hip_check(hipGetLastError(), "launch scalar Q4 projection (mfma)");
 }
 
@@ -1376,9 +1376,9 @@ int int8_swiglu_launch(const orx_function& f, int rows, const Geometry& g, hipSt
     p.n = f.N, p.k = f.K, p.stride = f.N, p.m = rows, p.packed_k = 0, p.out_f32 = 0;
     const dim3 grid(g.grid[0], g.grid[1]), block(256);
     if (rows <= 64)
-        hipLaunchKernelGGL((gemm_kernel<kW8, 64, 128, 2, false, true>), grid, block, 0, stream, p);
+        ORX_LAUNCH((gemm_kernel<kW8, 64, 128, 2, false, true>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((gemm_kernel<kW8, 128, 128, 2, false, true>), grid, block, 0, stream, p);
+        ORX_LAUNCH((gemm_kernel<kW8, 128, 128, 2, false, true>), grid, block, 0, stream, p);
     return hip_check(hipGetLastError(), "launch int8_swiglu");
 }
 
@@ -1803,9 +1803,9 @@ int unpack_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
     uint2* out = pointer_arg<uint2>(args, 1);
     const void* w = pointer_arg<const void>(args, 2);
     if (f.flags == kQ4)
-        hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
+        ORX_LAUNCH((unpack_kernel<kQ4>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
     else
-        hipLaunchKernelGGL((unpack_kernel<kQ2>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
+        ORX_LAUNCH((unpack_kernel<kQ2>), dim3(g.grid[0]), dim3(256), 0, stream, w, book, out, f.N, f.K, f.packed_k, nullptr);
     return hip_check(hipGetLastError(), "launch unpack");
 }
 
@@ -1819,7 +1819,7 @@ int expand_geometry(const orx_function& f, int rows, Geometry* g) {
 }
 int expand_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
-    hipLaunchKernelGGL((unpack_kernel<kQ4>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const void>(args, 3),
+    ORX_LAUNCH((unpack_kernel<kQ4>), dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const void>(args, 3),
                        pointer_arg<const uint32_t>(args, 0), pointer_arg<uint2>(args, 2), f.N, f.K, 128,
                        pointer_arg<const int>(args, 1));
     return hip_check(hipGetLastError(), "launch expand_experts");

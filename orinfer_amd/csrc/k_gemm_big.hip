@@ -466,7 +466,7 @@ int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int
                      hipStream_t stream) {
     const int64_t chunks = (int64_t)n * (k / 32);
     const int blocks = (int)std::min<int64_t>((chunks + 511) / 512, 2048);
-    hipLaunchKernelGGL(q4_expand_kernel, dim3(blocks), dim3(512), 0, stream, reinterpret_cast<const uint4*>(codes), book,
+    ORX_LAUNCH(q4_expand_kernel, dim3(blocks), dim3(512), 0, stream, reinterpret_cast<const uint4*>(codes), book,
                        reinterpret_cast<int8_t*>(weights), n, k, packed_k);
     return hip_check(hipGetLastError(), "launch two-stage weight expansion");
 }
@@ -488,9 +488,9 @@ int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* boo
     p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = packed_k, p.out_f32 = out_f32;
     p.tiles_m = (rows + kTile - 1) / kTile, p.tiles_n = (n + kTile - 1) / kTile;
     if (q4)
-        hipLaunchKernelGGL((gemm_big_kernel<true, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
+        ORX_LAUNCH((gemm_big_kernel<true, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
     else
-        hipLaunchKernelGGL((gemm_big_kernel<false, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
+        ORX_LAUNCH((gemm_big_kernel<false, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
     return hip_check(hipGetLastError(), "launch projection (mfma 256x256)");
 }
 

@@ -758,24 +758,24 @@ int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipSt
     switch (mr_for(rows)) {
         case 1:
             if (f.input_f16 && hold)
-                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true, true>), grid, block, g.shared, stream, a, w,
+                ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, true, true>), grid, block, g.shared, stream, a, w,
                                    book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else if (f.input_f16)
-                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false, true>), grid, block, g.shared, stream, a, w,
+                ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, false, true>), grid, block, g.shared, stream, a, w,
                                    book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else if (hold)
-                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
+                ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
                                    ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             else
-                hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 1, D, LPR, false>), grid, block, g.shared, stream, a, w, book,
+                ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, false>), grid, block, g.shared, stream, a, w, book,
                                    ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
         case 2:
-            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 2, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
+            ORX_LAUNCH((gemv_banked_kernel<kQ4, 2, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
                                as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
         default:
-            hipLaunchKernelGGL((gemv_banked_kernel<kQ4, 4, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
+            ORX_LAUNCH((gemv_banked_kernel<kQ4, 4, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
                                as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
             break;
     }
@@ -809,15 +809,15 @@ int gemv_launch_codec(const orx_function& f, int rows, const Geometry& g, hipStr
     }
     switch (mr_for(rows)) {
         case 1:
-            hipLaunchKernelGGL((gemv_rowmajor_kernel<CODEC, 1>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
+            ORX_LAUNCH((gemv_rowmajor_kernel<CODEC, 1>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
                                f.N, f.K, f.stride, rows, f.block_m, (int)f.out_f32);
             break;
         case 2:
-            hipLaunchKernelGGL((gemv_rowmajor_kernel<CODEC, 2>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
+            ORX_LAUNCH((gemv_rowmajor_kernel<CODEC, 2>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
                                f.N, f.K, f.stride, rows, f.block_m, (int)f.out_f32);
             break;
         default:
-            hipLaunchKernelGGL((gemv_rowmajor_kernel<CODEC, 4>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
+            ORX_LAUNCH((gemv_rowmajor_kernel<CODEC, 4>), grid, block, g.shared, stream, a, wp, book, ws, as, out,
                                f.N, f.K, f.stride, rows, f.block_m, (int)f.out_f32);
             break;
     }
@@ -1068,7 +1068,7 @@ int route_gemv_launch(const orx_function& f, int rows, const Geometry& g, hipStr
     const int x16 = f.input_f16 ? ((f.flags & 2) ? 2 : 1) : 0;
     const dim3 grid(g.grid[0], g.grid[1]), block(kRouteThreads);
 #define ORX_ROUTE_GEMV(LOCAL)                                                                                      \
-    hipLaunchKernelGGL(route_gemv_kernel<LOCAL>, grid, block, g.shared, stream, a, as, book, c, ids, p, ws, f.E, f.N, f.K, \
+    ORX_LAUNCH(route_gemv_kernel<LOCAL>, grid, block, g.shared, stream, a, as, book, c, ids, p, ws, f.E, f.N, f.K, \
                        f.flags & 1, x16, logits, prob, (f.flags >> 3) & 1)
     if (!routing) ORX_ROUTE_GEMV(0);
     else if (f.E <= 64) ORX_ROUTE_GEMV(1);

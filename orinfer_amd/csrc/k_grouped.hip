@@ -634,7 +634,7 @@ int grouped_resident_launch(const GroupedBuffers& b, int n, int k, int tiles, in
     Geometry g;
     grouped_resident_geometry(k, input, epilogue, slots, &g);
     const dim3 grid(g.grid[0]), block(kThreads);
-#define ORX_GROUPED(D, IN, EP) hipLaunchKernelGGL((grouped_resident_kernel<D, IN, EP>), grid, block, g.shared, stream, p)
+#define ORX_GROUPED(D, IN, EP) ORX_LAUNCH((grouped_resident_kernel<D, IN, EP>), grid, block, g.shared, stream, p)
 #define ORX_GROUPED_DEPTH(IN, EP)           \
     do {                                    \
         if (depth == 3) ORX_GROUPED(3, IN, EP); \

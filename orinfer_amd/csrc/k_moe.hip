@@ -661,10 +661,10 @@ int router_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
 #define ORX_ROUTER(LOCAL)                                                                                              \
     do {                                                                                                               \
         if (f.H > 0)                                                                                                   \
-            hipLaunchKernelGGL((router_topk_kernel<LOCAL, true>), grid, block, 0, s, logits, ids, prob, rows, f.E,     \
+            ORX_LAUNCH((router_topk_kernel<LOCAL, true>), grid, block, 0, s, logits, ids, prob, rows, f.E,     \
                                f.top_k, f.flags, x, q, scale, f.H);                                                    \
         else                                                                                                           \
-            hipLaunchKernelGGL((router_topk_kernel<LOCAL, false>), grid, block, 0, s, logits, ids, prob, rows, f.E,    \
+            ORX_LAUNCH((router_topk_kernel<LOCAL, false>), grid, block, 0, s, logits, ids, prob, rows, f.E,    \
                                f.top_k, f.flags, x, q, scale, f.H);                                                    \
     } while (0)
     if (f.E <= 64) ORX_ROUTER(1);
@@ -729,7 +729,7 @@ int histogram_geometry(const orx_function& f, int, Geometry* g) {
     return ORX_OK;
 }
 int histogram_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(expert_histogram_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 1),
+    ORX_LAUNCH(expert_histogram_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 1),
                        pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), rows * f.top_k);
     return hip_check(hipGetLastError(), "launch expert_histogram");
 }
@@ -761,9 +761,9 @@ int router_projection_launch(const orx_function& f, int rows, const Geometry& g,
     float* logits = pointer_arg<float>(args, 0);
     __half* gate = pointer_arg<__half>(args, 1);
     if (rows <= kProjectionSmallRows)
-        hipLaunchKernelGGL(router_projection_kernel<16>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
+        ORX_LAUNCH(router_projection_kernel<16>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
     else
-        hipLaunchKernelGGL(router_projection_kernel<32>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
+        ORX_LAUNCH(router_projection_kernel<32>, grid, block, 0, s, x, w, logits, gate, rows, f.H, f.E);
     return hip_check(hipGetLastError(), "launch router_projection");
 }
 int make_router_projection(const Variant& v, orx_function* f) {
@@ -806,13 +806,13 @@ int segmented_launch(const orx_function& f, int rows, const Geometry& g, hipStre
     const int assignments = rows * f.top_k, segments = (assignments + f.group - 1) / f.group;
     const dim3 grid(g.grid[0], g.grid[1]), block(g.block[0]);
     if (f.algorithm == 0)  // IDs, Partial, Slots
-        hipLaunchKernelGGL(histogram_local_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0), pointer_arg<int>(args, 1),
+        ORX_LAUNCH(histogram_local_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0), pointer_arg<int>(args, 1),
                            pointer_arg<int>(args, 2), assignments, f.group, segments);
     else if (f.algorithm == 1)  // Counts, Offsets, Partial
-        hipLaunchKernelGGL(histogram_offsets_kernel, grid, block, 0, s, pointer_arg<const int>(args, 2),
+        ORX_LAUNCH(histogram_offsets_kernel, grid, block, 0, s, pointer_arg<const int>(args, 2),
                            pointer_arg<int>(args, 1), pointer_arg<int>(args, 0), segments);
     else  // IDs, Offsets, Slots
-        hipLaunchKernelGGL(histogram_finish_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0),
+        ORX_LAUNCH(histogram_finish_kernel, grid, block, 0, s, pointer_arg<const int>(args, 0),
                            pointer_arg<const int>(args, 1), pointer_arg<int>(args, 2), assignments, f.group, segments);
     return hip_check(hipGetLastError(), "launch segmented expert histogram");
 }
@@ -849,7 +849,7 @@ int one_block_geometry(const orx_function&, int, Geometry* g) {
     return ORX_OK;
 }
 int offsets_launch(const orx_function& f, int, const Geometry&, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(expert_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 0),
+    ORX_LAUNCH(expert_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 0),
                        pointer_arg<int>(args, 1), pointer_arg<int>(args, 2), pointer_arg<int>(args, 3), f.E, f.block_m);
     return hip_check(hipGetLastError(), "launch expert_offsets");
 }
@@ -873,7 +873,7 @@ int make_offsets(const Variant& v, orx_function* f) {
 }
 
 int tiles_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(expert_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 0),
+    ORX_LAUNCH(expert_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 0),
                        pointer_arg<int>(args, 1), pointer_arg<const int>(args, 2), pointer_arg<int>(args, 3), f.block_m);
     return hip_check(hipGetLastError(), "launch expert_tiles");
 }
@@ -914,7 +914,7 @@ int metadata_launch(const orx_function& f, int rows, const Geometry& g, hipStrea
     if (ready != ORX_OK) return ready;
     const bool maps = f.flags & 1;
     const int offsets_at = maps ? 4 : 3, tiles_at = maps ? 7 : 4;
-    hipLaunchKernelGGL(route_metadata_kernel, dim3(1), dim3(kMetaThreads), g.shared, s, pointer_arg<const int>(args, 1),
+    ORX_LAUNCH(route_metadata_kernel, dim3(1), dim3(kMetaThreads), g.shared, s, pointer_arg<const int>(args, 1),
                        pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), pointer_arg<int>(args, offsets_at),
                        pointer_arg<int>(args, tiles_at), pointer_arg<int>(args, tiles_at + 1),
                        pointer_arg<int>(args, tiles_at + 2), pointer_arg<int>(args, tiles_at + 3),
@@ -958,7 +958,7 @@ int single_metadata_geometry(const orx_function& f, int, Geometry* g) {
 }
 // Counts, IDs, Offsets, Relative, TileCount, TileExpert, TileOffsets, TileRow (moe.py:674-683 in generated-ABI order)
 int single_metadata_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(single_route_metadata_kernel, dim3(1), dim3(256), g.shared, s, pointer_arg<const int>(args, 1),
+    ORX_LAUNCH(single_route_metadata_kernel, dim3(1), dim3(256), g.shared, s, pointer_arg<const int>(args, 1),
                        pointer_arg<int>(args, 0), pointer_arg<int>(args, 3), pointer_arg<int>(args, 2),
                        pointer_arg<int>(args, 6), pointer_arg<int>(args, 5), pointer_arg<int>(args, 7),
                        pointer_arg<int>(args, 4), f.E, f.top_k);
@@ -1000,7 +1000,7 @@ bool partition_fields(const Variant& v, orx_function* f, const char* who) {
 }
 // ColdCount, ColdOffsets, Counts, RowOffsets, TileCount, TileOffsets (expert_partition.py:21-28 in generated-ABI order)
 int partition_offsets_launch(const orx_function& f, int, const Geometry&, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(partition_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 2),
+    ORX_LAUNCH(partition_offsets_kernel, dim3(1), dim3(256), 0, s, pointer_arg<const int>(args, 2),
                        pointer_arg<int>(args, 3), pointer_arg<int>(args, 5), pointer_arg<int>(args, 4),
                        pointer_arg<int>(args, 1), pointer_arg<int>(args, 0), f.E, f.block_m, f.block_n, f.group);
     return hip_check(hipGetLastError(), "launch expert_partition_offsets");
@@ -1017,7 +1017,7 @@ int make_partition_offsets(const Variant& v, orx_function* f) {
 }
 // ColdExpert, ColdOffsets, ColdRow, Counts, TileExpert, TileOffsets, TileRow[, m] (expert_partition.py:70-78)
 int partition_tiles_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
-    hipLaunchKernelGGL(partition_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 3),
+    ORX_LAUNCH(partition_tiles_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int>(args, 3),
                        pointer_arg<const int>(args, 5), pointer_arg<int>(args, 4), pointer_arg<int>(args, 6),
                        pointer_arg<const int>(args, 1), pointer_arg<int>(args, 0), pointer_arg<int>(args, 2), f.block_m,
                        f.block_n, f.group);
@@ -1051,13 +1051,13 @@ int dispatch_geometry(const orx_function& f, int rows, Geometry* g) {
 }
 int dispatch_launch(const orx_function& f, int, const Geometry& g, hipStream_t s, void** args) {
     if (f.flags & 1) {  // fp16 rows, quantised on the way (Scale is not read)
-        hipLaunchKernelGGL(quantize_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const __half>(args, 0),
+        ORX_LAUNCH(quantize_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const __half>(args, 0),
                            pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 2), pointer_arg<const int>(args, 3),
                            pointer_arg<const int>(args, 4), pointer_arg<const int>(args, 5), pointer_arg<int>(args, 7), f.H,
                            f.top_k);
         return hip_check(hipGetLastError(), "launch expert_dispatch (fp16 rows)");
     }
-    hipLaunchKernelGGL(expert_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int8_t>(args, 0),
+    ORX_LAUNCH(expert_dispatch_kernel, dim3(g.grid[0]), dim3(256), 0, s, pointer_arg<const int8_t>(args, 0),
                        pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 2), pointer_arg<const int>(args, 3),
                        pointer_arg<const int>(args, 4), pointer_arg<const int>(args, 5),
                        pointer_arg<const __half>(args, 6), pointer_arg<int>(args, 7), f.H, f.H / f.group, f.top_k);
@@ -1104,13 +1104,13 @@ int combine_launch(const orx_function& f, int rows, const Geometry& g, hipStream
     // dynamic decode has exactly top_k assignments per live row (moe.py:514-517)
     const int slots = f.dynamic_rows ? rows * f.top_k : f.slots;
     if (f.H % 8 == 0) {
-        hipLaunchKernelGGL(moe_combine_wide_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
+        ORX_LAUNCH(moe_combine_wide_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
                            pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), pointer_arg<const float>(args, 2),
                            pointer_arg<const __half>(args, 3), pointer_arg<const __half>(args, 4),
                            pointer_arg<const int>(args, 5), f.H, slots, f.top_k);
         return hip_check(hipGetLastError(), "launch moe_combine");
     }
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
+    ORX_LAUNCH(moe_combine_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, s,
                        pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), pointer_arg<const float>(args, 2),
                        pointer_arg<const __half>(args, 3), pointer_arg<const __half>(args, 4),
                        pointer_arg<const int>(args, 5), f.H, slots, f.top_k);

@@ -196,8 +196,10 @@ __global__ __launch_bounds__(kPlaneThreads) void plane_gemm_kernel(PlaneGemmPara
     const int expert = p.tile_expert[tile], first = p.tile_row[tile];
     if (p.list_rows != p.tile_rows && first % p.tile_rows != 0) return;  // the second of two merged tiles
     const int row0 = p.offsets[expert] + first;
-    const int rows_here = min(p.tile_rows, p.counts[expert] - first);
-    if (rows_here <= 0) return;
+    // a tile never reaches past the live rows, whatever Counts and Offsets say (e8p_exact.py:127-150 clamps every
+    // plane load to rows - 1 and predicates it on the row being live)
+    const int rows_here = min(min(p.tile_rows, p.counts[expert] - first), p.rows - row0);
+    if (row0 < 0 || rows_here <= 0) return;
     const int n0 = blockIdx.x * kTileChannels;
     const int8_t* codes = reinterpret_cast<const int8_t*>(p.codes) + (int64_t)expert * p.expert_stride;
     const __half* ws = p.ws + (int64_t)expert * p.n;
@@ -349,7 +351,7 @@ int split_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t
             p.sum = pointer_arg<int>(args, 8);
             break;
     }
-    hipLaunchKernelGGL(plane_split_kernel, dim3(g.grid[0]), dim3(g.block[0]), 0, stream, p);
+    ORX_LAUNCH(plane_split_kernel, dim3(g.grid[0]), dim3(g.block[0]), 0, stream, p);
     return hip_check(hipGetLastError(), "launch plane split");
 }
 
@@ -452,7 +454,7 @@ int expand_geometry(const orx_function& f, int rows, Geometry* g) {
 
 // DS, High, Low, Scale, Sources, SrcHigh, SrcLow, SrcSum, Sum, m
 int expand_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
-    hipLaunchKernelGGL(plane_expand_kernel, dim3(g.grid[0], g.grid[1]), dim3(g.block[0]), 0, stream,
+    ORX_LAUNCH(plane_expand_kernel, dim3(g.grid[0], g.grid[1]), dim3(g.block[0]), 0, stream,
                        pointer_arg<const uint32_t>(args, 6), pointer_arg<const uint32_t>(args, 5),
                        pointer_arg<const int>(args, 7), pointer_arg<const __half>(args, 3),
                        pointer_arg<const int>(args, 4), pointer_arg<uint32_t>(args, 2), pointer_arg<uint32_t>(args, 1),
@@ -518,9 +520,9 @@ int plane_gemm_launch(const orx_function& f, int rows, const Geometry& g, hipStr
                                     p.tile_rows, p.list_rows, g, stream);
     const dim3 grid(g.grid[0], g.grid[1]), block(g.block[0]);
     if (f.flags & 2)
-        hipLaunchKernelGGL(plane_gemm_kernel<true>, grid, block, 0, stream, p);
+        ORX_LAUNCH(plane_gemm_kernel<true>, grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL(plane_gemm_kernel<false>, grid, block, 0, stream, p);
+        ORX_LAUNCH(plane_gemm_kernel<false>, grid, block, 0, stream, p);
     return hip_check(hipGetLastError(), "launch grouped GEMM on planes");
 }
 

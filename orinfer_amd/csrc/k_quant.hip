@@ -697,21 +697,21 @@ int a8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     const bool masked = f.flags & 1, fused = f.flags & 2;
     if (a8_per_wave(f)) {
         if (fused)
-            hipLaunchKernelGGL((a8_wave_kernel<true>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
+            ORX_LAUNCH((a8_wave_kernel<true>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
         else
-            hipLaunchKernelGGL((a8_wave_kernel<false>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
+            ORX_LAUNCH((a8_wave_kernel<false>), grid, block, 0, stream, x, q, s, f.K, f.group, groups, rows);
     } else if (g.block[0] == 1024)
-        hipLaunchKernelGGL((a8_kernel<false, false, 1024>), grid, dim3(1024), 0, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<false, false, 1024>), grid, dim3(1024), 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (g.shared > 0)
-        hipLaunchKernelGGL((a8_kernel<false, false, 256, true>), grid, block, g.shared, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<false, false, 256, true>), grid, block, g.shared, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused && masked)
-        hipLaunchKernelGGL((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<true, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (fused)
-        hipLaunchKernelGGL((a8_kernel<true, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<true, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     else if (masked)
-        hipLaunchKernelGGL((a8_kernel<false, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<false, true>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     else
-        hipLaunchKernelGGL((a8_kernel<false, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
+        ORX_LAUNCH((a8_kernel<false, false>), grid, block, 0, stream, x, mask, q, s, f.K, f.group, groups);
     return hip_check(hipGetLastError(), "launch activation_quantization");
 }
 
@@ -763,13 +763,13 @@ int rotate_a8_launch(const orx_function& f, int rows, const Geometry& g, hipStre
     const dim3 grid(g.grid[0]), block(g.block[0]);
     if (g.block[0] == 1024) {
         if (f.flags & 2)
-            hipLaunchKernelGGL((rotate_a8_kernel<true, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+            ORX_LAUNCH((rotate_a8_kernel<true, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
         else
-            hipLaunchKernelGGL((rotate_a8_kernel<false, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+            ORX_LAUNCH((rotate_a8_kernel<false, 1024>), grid, block, g.shared, stream, x, signs, q, s, f.K);
     } else if (f.flags & 2) {
-        hipLaunchKernelGGL((rotate_a8_kernel<true>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+        ORX_LAUNCH((rotate_a8_kernel<true>), grid, block, g.shared, stream, x, signs, q, s, f.K);
     } else {
-        hipLaunchKernelGGL((rotate_a8_kernel<false>), grid, block, g.shared, stream, x, signs, q, s, f.K);
+        ORX_LAUNCH((rotate_a8_kernel<false>), grid, block, g.shared, stream, x, signs, q, s, f.K);
     }
     return hip_check(hipGetLastError(), "launch rotate_activation_a8");
 }
@@ -827,7 +827,7 @@ int rotate_expert_launch(const orx_function& f, int rows, const Geometry& g, hip
     const int group_major = (f.flags & 4) ? 1 : 0;
     const dim3 grid(g.grid[0]), block(g.block[0]);
 #define ORX_ROTATE_EXPERT(SW, TH)                                                                                      \
-    hipLaunchKernelGGL((rotate_expert_kernel<SW, TH>), grid, block, g.shared, stream, x, signs, q, s, d, ds, ids,      \
+    ORX_LAUNCH((rotate_expert_kernel<SW, TH>), grid, block, g.shared, stream, x, signs, q, s, d, ds, ids,      \
                        relative, row_offsets, slot_map, sum, low, high, plane_rows, group_major, f.K, f.top_k, f.algorithm)
     if (g.block[0] == 1024) {
         if (f.flags & 2) ORX_ROTATE_EXPERT(true, 1024);
@@ -921,9 +921,9 @@ int rotate_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
     const __half* x = pointer_arg<const __half>(args, 1);
     __half* y = pointer_arg<__half>(args, 2);
     if (f.flags & 2)
-        hipLaunchKernelGGL((rotate_kernel<true>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
+        ORX_LAUNCH((rotate_kernel<true>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
     else
-        hipLaunchKernelGGL((rotate_kernel<false>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
+        ORX_LAUNCH((rotate_kernel<false>), dim3(g.grid[0]), dim3(256), 0, stream, x, signs, y, f.K);
     return hip_check(hipGetLastError(), "launch rotate_activation");
 }
 int make_rotate(const Variant& v, orx_function* f) {
@@ -962,7 +962,7 @@ int residual_rotate_launch(const orx_function& f, int rows, const Geometry& g, h
     const __half* w = pointer_arg<const __half>(args, 5);
     const __half* x = pointer_arg<const __half>(args, 6);
     __half* y = pointer_arg<__half>(args, 7);
-    hipLaunchKernelGGL(residual_norm_rotate_a8_kernel, dim3(g.grid[0]), dim3(256), g.shared, stream, x, r, w, y, ro, signs,
+    ORX_LAUNCH(residual_norm_rotate_a8_kernel, dim3(g.grid[0]), dim3(256), g.shared, stream, x, r, w, y, ro, signs,
                        q, s, f.K, 1e-6f, (f.flags & 1) ? 1.0f : 0.0f);
     return hip_check(hipGetLastError(), "launch residual_norm_rotate_a8");
 }
@@ -984,9 +984,9 @@ int rotate_tiles_launch(const orx_function& f, int rows, const Geometry& g, hipS
     const dim3 grid(g.grid[0], g.grid[1]), block(256);
     if (f.flags & 2) {
         const int64_t stride = f.slots ? f.K : 2 * (int64_t)f.K, up = f.slots ? (int64_t)f.slots * f.K : f.K;
-        hipLaunchKernelGGL((rotate_tiles_kernel<true>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group, stride, up);
+        ORX_LAUNCH((rotate_tiles_kernel<true>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group, stride, up);
     } else {
-        hipLaunchKernelGGL((rotate_tiles_kernel<false>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group,
+        ORX_LAUNCH((rotate_tiles_kernel<false>), grid, block, 0, stream, x, signs, rotated, maxima, f.K, f.group,
                            (int64_t)f.K, (int64_t)0);
     }
     return hip_check(hipGetLastError(), "launch rotate_activation_tiles");
@@ -994,7 +994,7 @@ int rotate_tiles_launch(const orx_function& f, int rows, const Geometry& g, hipS
 // Maxima, Q, Rotated, S[, m]
 int quantize_tiles_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
-    hipLaunchKernelGGL(quantize_tiles_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const __half>(args, 2),
+    ORX_LAUNCH(quantize_tiles_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream, pointer_arg<const __half>(args, 2),
                        pointer_arg<const float>(args, 0), pointer_arg<int8_t>(args, 1), pointer_arg<__half>(args, 3), f.K, f.group);
     return hip_check(hipGetLastError(), "launch quantize_rotation_tiles");
 }
@@ -1088,7 +1088,7 @@ int q4_embedding_geometry(const orx_function&, int rows, Geometry* g) {
 // Book, IDs, Output, Scale, Signs, Weight, m   (e8p_q4.py:95-102 in generated-ABI order)
 int q4_embedding_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
-    hipLaunchKernelGGL(q4_embedding_kernel, dim3(g.grid[0]), dim3(256), 0, stream, pointer_arg<const int32_t>(args, 1),
+    ORX_LAUNCH(q4_embedding_kernel, dim3(g.grid[0]), dim3(256), 0, stream, pointer_arg<const int32_t>(args, 1),
                        pointer_arg<const uint32_t>(args, 5), pointer_arg<const uint32_t>(args, 0),
                        pointer_arg<const __half>(args, 3), pointer_arg<const int8_t>(args, 4), pointer_arg<__half>(args, 2),
                        f.N, f.K);
@@ -1125,7 +1125,7 @@ int swiglu_geometry(const orx_function& f, int rows, Geometry* g) {
 
 int swiglu_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, void** args) {
     (void)rows;
-    hipLaunchKernelGGL(swiglu_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream,
+    ORX_LAUNCH(swiglu_kernel, dim3(g.grid[0], g.grid[1]), dim3(256), 0, stream,
                        pointer_arg<const __half>(args, 0), pointer_arg<__half>(args, 1), f.N);
     return hip_check(hipGetLastError(), "launch swiglu");
 }

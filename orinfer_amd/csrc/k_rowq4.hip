@@ -158,10 +158,10 @@ int row_q4_gemv_launch(const int8_t* a, const void* w, uint32_t low, uint32_t hi
     p.n = n, p.k = k, p.stride = stride, p.out_f32 = out_f32, p.low = low, p.high = high;
     const dim3 grid(g.grid[0]), block(g.block[0]);
     switch (rows) {
-        case 1: hipLaunchKernelGGL(row_q4_gemv_kernel<1>, grid, block, g.shared, stream, p); break;
-        case 2: hipLaunchKernelGGL(row_q4_gemv_kernel<2>, grid, block, g.shared, stream, p); break;
-        case 3: hipLaunchKernelGGL(row_q4_gemv_kernel<3>, grid, block, g.shared, stream, p); break;
-        default: hipLaunchKernelGGL(row_q4_gemv_kernel<4>, grid, block, g.shared, stream, p); break;
+        case 1: ORX_LAUNCH(row_q4_gemv_kernel<1>, grid, block, g.shared, stream, p); break;
+        case 2: ORX_LAUNCH(row_q4_gemv_kernel<2>, grid, block, g.shared, stream, p); break;
+        case 3: ORX_LAUNCH(row_q4_gemv_kernel<3>, grid, block, g.shared, stream, p); break;
+        default: ORX_LAUNCH(row_q4_gemv_kernel<4>, grid, block, g.shared, stream, p); break;
     }
     return hip_check(hipGetLastError(), "launch scalar Q4 GEMV");
 }

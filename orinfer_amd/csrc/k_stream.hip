@@ -290,9 +290,9 @@ __global__ __launch_bounds__(kThreads) void stream_kernel(StreamParams p) {
 template <int CODEC, bool GROUPED, int SPLITS>
 int launch_codec(int cb, const StreamParams& p, dim3 grid, hipStream_t stream) {
     if (cb == 1)
-        hipLaunchKernelGGL((stream_kernel<CODEC, 1, GROUPED, SPLITS>), grid, dim3(kThreads), 0, stream, p);
+        ORX_LAUNCH((stream_kernel<CODEC, 1, GROUPED, SPLITS>), grid, dim3(kThreads), 0, stream, p);
     else
-        hipLaunchKernelGGL((stream_kernel<CODEC, 2, GROUPED, SPLITS>), grid, dim3(kThreads), 0, stream, p);
+        ORX_LAUNCH((stream_kernel<CODEC, 2, GROUPED, SPLITS>), grid, dim3(kThreads), 0, stream, p);
     return hip_check(hipGetLastError(), "launch projection (stream)");
 }
 
@@ -339,9 +339,9 @@ int stream_planes_launch(bool two_stage, const uint32_t* low, const uint32_t* hi
     p.tile_rows = tile_rows, p.list_rows = list_rows;
     const dim3 grid(g.grid[0], g.grid[1]);
     if (two_stage)
-        hipLaunchKernelGGL((stream_kernel<kQ4, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
+        ORX_LAUNCH((stream_kernel<kQ4, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
     else
-        hipLaunchKernelGGL((stream_kernel<kQ2, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
+        ORX_LAUNCH((stream_kernel<kQ2, 1, true, kGroupedSplits, true>), grid, dim3(kThreads), 0, stream, p);
     return hip_check(hipGetLastError(), "launch routed projection on nibble planes (stream)");
 }
 

@@ -352,9 +352,9 @@ int dense_wide_launch(const int8_t* a, const void* w, const uint32_t* book, cons
     p.a = a, p.w = static_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
     p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k != 0;
     if (packed_k != 0)
-        hipLaunchKernelGGL(wide_kernel<true>, dim3(g.grid[0]), dim3(kThreads), kWideLdsBytes, stream, p);
+        ORX_LAUNCH(wide_kernel<true>, dim3(g.grid[0]), dim3(kThreads), kWideLdsBytes, stream, p);
     else
-        hipLaunchKernelGGL(wide_kernel<false>, dim3(g.grid[0]), dim3(kThreads), kWideLdsBytes, stream, p);
+        ORX_LAUNCH(wide_kernel<false>, dim3(g.grid[0]), dim3(kThreads), kWideLdsBytes, stream, p);
     return hip_check(hipGetLastError(), "launch projection (channel runs)");
 }
 

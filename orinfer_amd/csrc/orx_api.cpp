@@ -31,6 +31,14 @@ int hip_check(hipError_t code, const char* operation) {
     return (int)code;
 }
 
+namespace {
+thread_local std::vector<LaunchRecord>* g_recording = nullptr;
+}
+bool recording_launches() { return g_recording != nullptr; }
+void record_launch(const void* function, dim3 grid, dim3 block, uint32_t shared) {
+    g_recording->push_back({function, grid.x, block.x * block.y * block.z, shared});
+}
+
 int current_device() {
     int device = 0;
     if (hipGetDevice(&device) != hipSuccess) {
@@ -246,14 +254,13 @@ struct Table {
     const Registration* rows;
     int count;
 };
-constexpr int kTables = 6;
+constexpr int kTables = 5;
 void tables(Table out[kTables]) {
     out[0].rows = quant_registrations(&out[0].count);
     out[1].rows = gemv_registrations(&out[1].count);
     out[2].rows = gemm_registrations(&out[2].count);
     out[3].rows = moe_registrations(&out[3].count);
-    out[4].rows = probe_registrations(&out[4].count);
-    out[5].rows = plane_registrations(&out[5].count);
+    out[4].rows = plane_registrations(&out[4].count);
 }
 const Registration* find(const char* symbol) {
     Table t[kTables];
@@ -277,10 +284,22 @@ namespace orx {
 namespace {
 std::atomic<void*> g_scratch_address[64];
 
-// Address of `scratch` on the current device; looked up on the first call per device.
-int static_scratch_address(void** out) {
+// Address of `scratch` on the current device; looked up on the first call per device (the calling thread's
+// current device: a handle is resolved, and launched, with the launch device current).  The lookup is a runtime
+// call that may not run while `stream` is capturing: orx_resolve of a workspace handle does it ahead of time
+// for the device current then, and a first launch on another device under capture is refused.
+int static_scratch_address(void** out, hipStream_t stream = nullptr, bool launching = false) {
     const int slot = current_device() & 63;
     void* address = g_scratch_address[slot].load(std::memory_order_acquire);
+    if (address == nullptr && launching) {
+        hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &status) != hipSuccess) (void)hipGetLastError();
+        if (status != hipStreamCaptureStatusNone) {
+            set_error("orx_launch_static_scratch: the scratch of device %d has not been looked up yet and the stream is "
+                      "capturing: resolve the handle (or launch once) with this device current before the capture", slot);
+            return ORX_ERR_BAD_ARGUMENT;
+        }
+    }
     if (address == nullptr) {
         const int code = hip_check(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
         if (code != ORX_OK) return code;
@@ -369,6 +388,33 @@ int resolve(const char* symbol, const char* variant_json, orx_fn* out) {
     f->symbol = family;
     const int code = r->factory(variant, f.get());
     if (code != ORX_OK) return code;
+    // `omit`: optional buffers that the caller's program does not use leave the argument list (a package record has
+    // no way to say "null", artifact.rs:184-194); the kernel sees a null pointer in their place
+    bool bad_omit = false;
+    const std::string omit = variant.string("omit", "", &bad_omit);
+    if (bad_omit) return ORX_ERR_BAD_VARIANT;
+    for (size_t at = 0; at < omit.size();) {
+        size_t end = omit.find(',', at);
+        if (end == std::string::npos) end = omit.size();
+        const std::string name = omit.substr(at, end - at);
+        at = end + 1;
+        int index = -1;
+        for (size_t i = 0; i < f->args.size(); ++i)
+            if (name == f->args[i].name) index = (int)i;
+        const bool optional = index >= 0 && f->args[index].kind == ArgPointer && (f->args[index].alignment & 0x80000000u) &&
+                              name != "Workspace";
+        if (!optional || std::count(f->omitted.begin(), f->omitted.end(), index)) {
+            set_error("orx_resolve %s: omit names %s, which is not an optional buffer of this variant", family.c_str(),
+                      name.c_str());
+            return ORX_ERR_BAD_VARIANT;
+        }
+        f->omitted.push_back(index);
+    }
+    std::sort(f->omitted.begin(), f->omitted.end());
+    if (!f->omitted.empty() && f->args.size() > 64) {
+        set_error("orx_resolve %s: too many arguments for omit", family.c_str());
+        return ORX_ERR_BAD_VARIANT;
+    }
     for (const auto& field : variant.fields) {
         if (!variant.read->count(field.first)) {
             set_error("orx_resolve %s: unknown variant key %s (keys: %s)", family.c_str(), field.first.c_str(), r->variant_keys);
@@ -456,6 +502,27 @@ int check_launch(const orx_function* f, const uint32_t grid[3], const uint32_t b
     return ORX_OK;
 }
 
+// Index into f->args of the caller's argument `visible` (the list without the omitted buffers), or -1.
+int full_index(const orx_function* f, int visible) {
+    if (visible < 0) return -1;
+    int seen = 0;
+    for (int i = 0; i < (int)f->args.size(); ++i) {
+        if (std::binary_search(f->omitted.begin(), f->omitted.end(), i)) continue;
+        if (seen++ == visible) return i;
+    }
+    return -1;
+}
+
+// The caller's argument list with a null pointer at every omitted buffer.  `storage` must hold 64 entries.
+void** expand_args(const orx_function* f, void** args, void** storage) {
+    static uint64_t null_pointer = 0;  // never written
+    if (f == nullptr || args == nullptr || f->omitted.empty() || f->args.size() > 64) return args;
+    int next = 0;
+    for (int i = 0; i < (int)f->args.size(); ++i)
+        storage[i] = std::binary_search(f->omitted.begin(), f->omitted.end(), i) ? (void*)&null_pointer : args[next++];
+    return storage;
+}
+
 uint64_t workspace_need(const orx_function* f, int rows) {
     return f->takes_workspace && f->workspace_need != nullptr ? f->workspace_need(*f, rows) : 0;
 }
@@ -478,24 +545,65 @@ int orx_release(orx_fn f) {
     return ORX_OK;
 }
 
-int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
+int orx_query_rows(orx_fn f, int32_t rows, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
     if (f == nullptr) {
         set_error("orx_query: null handle");
         return ORX_ERR_BAD_ARGUMENT;
     }
     return guard("orx_query", [&] {
+        const int live = rows <= 0 ? f->capacity : rows;
+        if (live > f->capacity || (!f->dynamic_rows && live != f->capacity)) {
+            set_error("%s: rows %d outside the kernel capacity %d", f->symbol.c_str(), live, f->capacity);
+            return (int)ORX_ERR_ROWS;
+        }
+        const void* function = f->device_function;
+        if (function == nullptr) {
+            // a handle that starts one of several kernels depending on the live rows: run its launch for this row
+            // count with recording on (nothing is enqueued, no argument is dereferenced) and take the kernel whose
+            // grid, block and LDS bytes are the ones orx_geometry reports, i.e. the one a package records
+            Geometry want;
+            int code = f->geometry(*f, live, &want);
+            if (code != ORX_OK) return code;
+            uint64_t zero[64] = {};
+            void* args[64];
+            if (f->args.size() > 64) {
+                set_error("orx_query %s: too many arguments", f->symbol.c_str());
+                return (int)ORX_ERR_INTERNAL;
+            }
+            for (size_t i = 0; i < f->args.size(); ++i) args[i] = &zero[i];
+            if (f->dynamic_rows) *reinterpret_cast<int32_t*>(&zero[f->args.size() - 1]) = live;
+            std::vector<LaunchRecord> seen;
+            g_recording = &seen;
+            try {
+                code = f->launch(*f, live, want, nullptr, args);
+            } catch (...) {
+                g_recording = nullptr;
+                throw;
+            }
+            g_recording = nullptr;
+            if (code != ORX_OK) return code;
+            for (const LaunchRecord& r : seen)
+                if (function == nullptr && r.grid == want.grid[0] && r.block == want.block[0] * want.block[1] * want.block[2] &&
+                    r.shared == want.shared)
+                    function = r.function;
+            if (function == nullptr && !seen.empty()) function = seen.back().function;
+            if (function == nullptr) {
+                set_error("orx_query %s: the launch of %d rows starts no kernel", f->symbol.c_str(), live);
+                return (int)ORX_ERR_INTERNAL;
+            }
+        }
         hipFuncAttributes attr;
         memset(&attr, 0, sizeof attr);
-        if (f->device_function != nullptr) {
-            int code = hip_check(hipFuncGetAttributes(&attr, f->device_function), "hipFuncGetAttributes");
-            if (code != ORX_OK) return code;
-        } else {
-            attr.maxThreadsPerBlock = 1024;
-        }
+        const int code = hip_check(hipFuncGetAttributes(&attr, function), "hipFuncGetAttributes");
+        if (code != ORX_OK) return code;
         if (max_threads_per_block) *max_threads_per_block = (uint32_t)attr.maxThreadsPerBlock;
         if (static_lds_bytes) *static_lds_bytes = (uint32_t)attr.sharedSizeBytes;
         return (int)ORX_OK;
     });
+}
+
+int orx_query(orx_fn f, uint32_t* max_threads_per_block, uint32_t* static_lds_bytes) {
+    return orx_query_rows(f, 0, max_threads_per_block, static_lds_bytes);
 }
 
 int orx_geometry(orx_fn f, int32_t rows, uint32_t grid[3], uint32_t block[3], uint32_t* shared_bytes) {
@@ -545,23 +653,25 @@ int orx_workspace_bytes(orx_fn f, int32_t rows, uint64_t* bytes) {
     });
 }
 
-int orx_arg_count(orx_fn f) { return f ? (int)f->args.size() : 0; }
+int orx_arg_count(orx_fn f) { return f ? (int)(f->args.size() - f->omitted.size()) : 0; }
 
 const char* orx_arg_name(orx_fn f, int index) {
-    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return "";
-    return f->args[index].name;
+    const int at = f ? full_index(f, index) : -1;
+    return at < 0 ? "" : f->args[at].name;
 }
 
 int orx_arg_kind(orx_fn f, int index) {
-    if (f == nullptr || index < 0 || index >= (int)f->args.size()) return -1;
-    return (int)f->args[index].kind;
+    const int at = f ? full_index(f, index) : -1;
+    return at < 0 ? -1 : (int)f->args[at].kind;
 }
 
 int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
                void* hip_stream, void** args) {
-    return guard("orx_launch", [&] {
+    return guard("orx_launch", [&, args]() mutable {
         int rows = 0;
         Geometry want;
+        void* full[64];
+        args = expand_args(f, args, full);
         const int code = check_launch(f, grid, block, shared_bytes, args, true, &rows, &want);
         if (code != ORX_OK) return code;
         const uint64_t need = workspace_need(f, rows);
@@ -576,9 +686,11 @@ int orx_launch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32
 
 int orx_launch_static_scratch(orx_fn f, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes,
                               void* hip_stream, void** args) {
-    return guard("orx_launch_static_scratch", [&] {
+    return guard("orx_launch_static_scratch", [&, args]() mutable {
         int rows = 0;
         Geometry want;
+        void* full[64];
+        args = expand_args(f, args, full);
         const int code = check_launch(f, grid, block, shared_bytes, args, false, &rows, &want);
         if (code != ORX_OK) return code;
         if (!f->takes_workspace)  // nothing to replace: the plain launch
@@ -591,7 +703,7 @@ int orx_launch_static_scratch(orx_fn f, const uint32_t grid[3], const uint32_t b
             return (int)ORX_ERR_WORKSPACE;
         }
         void* address = nullptr;
-        const int found = static_scratch_address(&address);
+        const int found = static_scratch_address(&address, reinterpret_cast<hipStream_t>(hip_stream), true);
         if (found != ORX_OK) return found;
         // the caller's argument list with the Workspace slot pointing at the library's scratch
         const size_t count = f->args.size();

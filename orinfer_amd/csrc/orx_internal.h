@@ -63,6 +63,9 @@ struct Geometry {
 struct orx_function {
     std::string symbol;
     std::vector<orx::ArgSpec> args;
+    // Optional buffers that the variant's `omit` key took out of the caller's argument list (indices into
+    // `args`, ascending): the launch sees a null pointer there.  Empty for most handles.
+    std::vector<int> omitted;
     bool dynamic_rows = false;  // last argument is `int32 m`
     int capacity = 0;           // largest row count (M of the variant)
     // shape / configuration
@@ -92,6 +95,23 @@ namespace orx {
 void set_error(const char* format, ...);
 int hip_check(hipError_t code, const char* operation);
 
+// Every kernel launch of the library goes through ORX_LAUNCH.  While a thread records (orx_query_rows), a launch
+// enqueues nothing and leaves its function, grid, block and dynamic LDS bytes in that thread's list instead: the
+// query then reads the attributes of the very kernel a launch of that row count would start.
+struct LaunchRecord {
+    const void* function;
+    uint32_t grid, block, shared;
+};
+bool recording_launches();
+void record_launch(const void* function, dim3 grid, dim3 block, uint32_t shared);
+#define ORX_LAUNCH(kernel, grid, block, shared, stream, ...)                                                          \
+    do {                                                                                                              \
+        if (::orx::recording_launches())                                                                              \
+            ::orx::record_launch(reinterpret_cast<const void*>(kernel), dim3(grid), dim3(block), (uint32_t)(shared)); \
+        else                                                                                                          \
+            hipLaunchKernelGGL(kernel, grid, block, shared, stream, __VA_ARGS__);                                     \
+    } while (0)
+
 // Each kernel file exports one factory per symbol: fills `f` from the variant or returns an
 // error code after set_error().
 typedef int (*Factory)(const Variant&, orx_function* f);
@@ -107,7 +127,6 @@ const Registration* quant_registrations(int* count);
 const Registration* gemv_registrations(int* count);
 const Registration* gemm_registrations(int* count);
 const Registration* moe_registrations(int* count);
-const Registration* probe_registrations(int* count);
 const Registration* plane_registrations(int* count);
 
 template <typename T>

@@ -302,15 +302,13 @@ int run(const std::string& manifest_path, std::ostringstream& report) {
                             std::to_string(it->second.bytes - offset) + " bytes, the launch needs " + std::to_string(need));
                 }
                 record.pointer_values[a] = reinterpret_cast<uint64_t>(static_cast<char*>(it->second.device) + offset);
-            } else if (arg.get("null")) {
-                record.pointer_values[a] = 0;
             } else if (const Json* value = arg.get("i32")) {
                 if (orx_arg_kind(record.function, (int)a) != 1)
                     die("kernel " + symbol->text + ": argument " + orx_arg_name(record.function, (int)a) + " is a pointer");
                 const int32_t scalar = (int32_t)value->number;
                 std::memcpy(&record.pointer_values[a], &scalar, sizeof scalar);
             } else {
-                die("kernel " + symbol->text + ": argument must be {\"buffer\"}, {\"null\"} or {\"i32\"}");
+                die("kernel " + symbol->text + ": argument must be {\"buffer\"} or {\"i32\"}");
             }
         }
         for (auto& v : record.pointer_values) record.args.push_back(&v);

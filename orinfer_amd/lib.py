@@ -24,7 +24,7 @@ ORX_ERR_INTERNAL = 10007
 EXPORTS = (
     "orx_resolve", "orx_release", "orx_query", "orx_geometry", "orx_arg_count", "orx_arg_name",
     "orx_arg_kind", "orx_launch", "orx_last_error", "orx_catalog", "orx_workspace_bytes",
-    "orx_launch_static_scratch",
+    "orx_launch_static_scratch", "orx_query_rows",
 )
 
 
@@ -59,6 +59,8 @@ def library():
         lib.orx_release.restype = ctypes.c_int
         lib.orx_query.argtypes = [ctypes.c_void_p, u32x3, u32x3]
         lib.orx_query.restype = ctypes.c_int
+        lib.orx_query_rows.argtypes = [ctypes.c_void_p, ctypes.c_int32, u32x3, u32x3]
+        lib.orx_query_rows.restype = ctypes.c_int
         lib.orx_geometry.argtypes = [ctypes.c_void_p, ctypes.c_int32, u32x3, u32x3, u32x3]
         lib.orx_geometry.restype = ctypes.c_int
         lib.orx_arg_count.argtypes = [ctypes.c_void_p]
@@ -123,9 +125,10 @@ class Kernel:
             _lib.orx_release(handle)
             self._handle = None
 
-    def query(self):
+    def query(self, rows=0):
+        """(thread limit, static LDS bytes) of the kernel that a launch of `rows` rows starts (0: the variant's M)."""
         threads, lds = ctypes.c_uint32(), ctypes.c_uint32()
-        _check(library().orx_query(self._handle, ctypes.byref(threads), ctypes.byref(lds)))
+        _check(library().orx_query_rows(self._handle, int(rows), ctypes.byref(threads), ctypes.byref(lds)))
         return threads.value, lds.value
 
     def geometry(self, rows=0):

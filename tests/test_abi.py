@@ -339,27 +339,32 @@ def test_argument_lists_of_the_fused_expert_layer_forms():
         assert err.value.code == lib.ORX_ERR_BAD_VARIANT, (symbol, variant)
 
 
-def test_matrix_pipe_probe_is_a_catalogued_diagnostic():
-    kern = lib.Kernel("int8_mfma_probe", iterations=100, operands="zero")
-    assert kern.arg_names == ["Out"] and kern.geometry()[1][0] == 512
-    for bad in (dict(iterations=0), dict(operands="ones")):
-        with pytest.raises(lib.OrxError):
-            lib.Kernel("int8_mfma_probe", **bad)
+def test_static_scratch_launch_refuses_before_it_enqueues():
+    # host-only checks of orx_launch_static_scratch: nothing reaches a device, so made-up addresses are safe here
+    big = lib.Kernel("e8p_q4_projection", M=8192, N=17408, K=5120, workspace=True)
+    assert big.workspace_bytes(8192) == 17408 * 5120 > 64 << 20
+    grid, block, shared = big.geometry(8192)
+    with pytest.raises(lib.OrxError) as err:  # beyond the static array
+        big.launch_raw(grid, block, shared, 0, [256] * 6 + [None], static_scratch=True)
+    assert err.value.code == lib.ORX_ERR_WORKSPACE and "static scratch" in str(err.value)
+    with pytest.raises(lib.OrxError) as err:  # geometry is checked as orx_launch checks it
+        big.launch_raw((grid[0] + 1, 1, 1), block, shared, 0, [256] * 6 + [None], static_scratch=True)
+    assert err.value.code == lib.ORX_ERR_BAD_GEOMETRY
 
 
-def test_plain_read_probe_is_a_catalogued_diagnostic():
-    kern = lib.Kernel("hbm_read_probe", bytes=44564480, workgroups_per_cu=4)
-    assert kern.arg_names == ["Out", "Source"] and kern.geometry()[1][0] == 256
-    for bad in (dict(bytes=1000), dict(bytes=16384, workgroups_per_cu=0)):
-        with pytest.raises(lib.OrxError):
-            lib.Kernel("hbm_read_probe", **bad)
-
-
-def test_lds_lookup_probe_is_a_catalogued_diagnostic():
-    kern = lib.Kernel("lds_lookup_probe", iterations=10, copies=32)
-    assert kern.arg_names == ["Out"] and kern.geometry()[1:] == ((1024, 1, 1), 256 * 32 * 4)
-    with pytest.raises(lib.OrxError):
-        lib.Kernel("lds_lookup_probe", copies=16)
+def test_omit_takes_optional_buffers_out_of_the_argument_list():
+    # a package record cannot say "null" (artifact.rs:184-194): buffers a program does not use are named in `omit`
+    full = lib.Kernel("moe_combine", M=4, E=8, top_k=2, H=64, slots=8)
+    short = lib.Kernel("moe_combine", M=4, E=8, top_k=2, H=64, slots=8, omit="Shared,SharedGate")
+    assert [n for n in full.arg_names if n not in ("Shared", "SharedGate")] == short.arg_names
+    assert len(short.arg_kinds) == len(short.arg_names)
+    assert short.geometry() == full.geometry()
+    for bad in ("Expert", "Nothing", "Shared,Shared"):  # required, unknown, named twice
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel("moe_combine", M=4, E=8, top_k=2, H=64, slots=8, omit=bad)
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT
+    inline = lib.Kernel("moe_combine?M=4&E=8&top_k=2&H=64&slots=8&omit=Shared,SharedGate")
+    assert inline.arg_names == short.arg_names
 
 
 def test_session_threads_resolve_and_query_concurrently():

@@ -109,6 +109,23 @@ def test_kernel_records_follow_the_package_schema():
     assert buffer["dtype"] == "u32" and buffer["shape"] == [4, 8] and buffer["access"] == "read"
 
 
+def test_every_emitted_argument_is_one_the_engine_deserialises():
+    # crates/orinfer-model-sdk/src/artifact.rs:184-194: `Argument` is tagged by `kind`, denies unknown fields and knows
+    # buffer, buffer_slice, i32, u32, i64, u64 and f32; a program's unused optional buffers are named in `omit`
+    fields = {"buffer": {"kind", "name"}, "buffer_slice": {"kind", "name", "offset"}, "i32": {"kind", "value"},
+              "u32": {"kind", "value"}, "i64": {"kind", "value"}, "u64": {"kind", "value"}, "f32": {"kind", "value"}}
+    layer, _ = container.expert_layer_program("moe.0", 256, 128, 8, 2048, 512)
+    exact, _ = container.exact_expert_program("moe.1", 4, 8, 2, 128, 256)
+    dense = container.projection_program("decoder.0.o", 512, 512, 64)["kernels"]
+    for record in [*layer, *exact, *dense]:
+        for arg in record["args"]:
+            assert arg["kind"] in fields and set(arg) == fields[arg["kind"]], (record["name"], arg)
+        assert len(record["args"]) == len(lib.Kernel(record["symbol"]).arg_names)
+    by_name = {r["name"]: r for r in layer}
+    assert "omit=C" in by_name["moe.0.gate_up"]["symbol"] and "omit=AS,Q" in by_name["moe.0.down"]["symbol"]
+    assert "omit=Shared,SharedGate" in by_name["moe.0.combine"]["symbol"]
+
+
 def test_row_ranges_are_the_longest_the_geometry_allows():
     """One record per stretch of rows with one block size, one LDS size and one grid expression: the scalar Q4 slot of
     config 1's shape changes kernel at 2, 3, 65, 257 (whole tiles instead of split ones) and 512 rows, nowhere else."""

@@ -1115,28 +1115,6 @@ def test_two_handles_on_two_streams_with_their_own_workspaces_stay_bit_exact():
             np.testing.assert_array_equal(gu.host(outs[c, t]), want)
 
 
-def test_diagnostic_probes_run_and_leave_their_inputs_alone():
-    """int8_mfma_probe, hbm_read_probe and lds_lookup_probe are rate probes for bench.py: here only that
-    they launch through the C ABI, finish, and write nothing but their one-word outputs."""
-    out = torch.full((1024,), -1, dtype=torch.int32, device=gu.DEV)
-    probe = gu.kernel("int8_mfma_probe", iterations=50, operands="zero")
-    units = probe.geometry()[0][0]
-    probe(Out=out)
-    gu.sync()
-    assert (gu.host(out)[:units] == 0).all() and (gu.host(out)[units:] == -1).all()  # zero operands fold to zero
-    gu.kernel("int8_mfma_probe", iterations=50, operands="random")(Out=out)
-    gu.sync()
-    assert (gu.host(out)[units:] == -1).all()
-    source = torch.arange(16384 * 4, dtype=torch.int32, device=gu.DEV)
-    before = source.clone()
-    word = torch.full((1,), 5, dtype=torch.int32, device=gu.DEV)
-    gu.kernel("hbm_read_probe", bytes=source.numel() * 4, workgroups_per_cu=2)(Out=word, Source=source)
-    for copies in (1, 32, 64):
-        gu.kernel("lds_lookup_probe", iterations=20, copies=copies)(Out=word)
-    gu.sync()
-    assert torch.equal(source, before) and int(word.item()) == 5
-
-
 @pytest.mark.parametrize("m,k,block_k,swiglu,planes", [(3, 5120, 512, False, False), (1, 17408, 2048, False, False),
                                                        (5, 640, 256, True, False), (4, 1152, 1024, True, True),
                                                        (2, 128, 128, False, False)])

@@ -943,6 +943,22 @@ def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
         for rows in ({1, variant["M"]} if variant.get("dynamic_rows") else {0}):
             block = kern.geometry(rows)[1]
             assert block[0] * block[1] * block[2] <= threads, (symbol, variant, rows, block, threads)
+    # a projection handle starts a different kernel per row range: the limits are those of the kernel that the rows
+    # start (every kernel here is compiled for exactly the block it is launched with), not a device-wide constant
+    for symbol, variant in (("e8p_q4_projection", dict(M=8192, N=17408, K=5120, dynamic_rows=True, workspace=True)),
+                            ("int8_projection", dict(M=8192, N=4096, K=4096, dynamic_rows=True, workspace=True)),
+                            ("e8p_q4_projection", dict(M=4096, N=5120, K=5120, dynamic_rows=True))):
+        kern = gu.lib.Kernel(symbol, **variant)
+        limits = {}
+        for rows in (1, 3, 8, 32, 48, 100, 128, 256, 384, 512, variant["M"]):
+            grid, block, shared = kern.geometry(rows)
+            threads, static_lds = kern.query(rows)
+            assert threads == block[0] * block[1] * block[2], (symbol, rows, block, threads)
+            assert static_lds + shared <= 160 * 1024
+            limits[rows] = threads
+        assert kern.query() == kern.query(variant["M"]) and len(set(limits.values())) >= 3, limits
+        with pytest.raises(gu.lib.OrxError):
+            kern.query(variant["M"] + 1)
 
 
 @pytest.mark.parametrize("e,k,h,i", [(128, 8, 2048, 512), (512, 10, 1024, 384), (64, 64, 256, 128)])
