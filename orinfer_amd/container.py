@@ -170,7 +170,8 @@ def evaluate_rows(expression, rows):
 
 def _fit_rows(values):
     """A RowExpression that gives values[rows] for every key of `values`, or None: a constant,
-    c * ceil(rows / d), or min(cap, c * ceil(rows / d) / 8) (the workgroups of a split launch)."""
+    c * ceil(rows / d), min(cap, c * ceil(rows / d)) (persistent workgroups), or
+    min(cap, c * ceil(rows / d) / 8) (the workgroups of a split launch)."""
     rows = sorted(values)
     if len({values[r] for r in rows}) == 1:
         return _constant(values[rows[0]])
@@ -181,6 +182,15 @@ def _fit_rows(values):
             expr = _ceil_div_rows(d) if c == 1 else {"op": "multiply", "lhs": _constant(c), "rhs": _ceil_div_rows(d)}
             return expr
     cap = max(values.values())
+    # min(cap, c * ceil(rows / d)): persistent workgroups, one per tile up to one per compute unit
+    for d in (32, 64, 128, 256):
+        tiles = {r: -(-r // d) for r in rows}
+        below = [r for r in rows if values[r] < cap]
+        if below and values[below[0]] % tiles[below[0]] == 0:
+            c = values[below[0]] // tiles[below[0]]
+            if all(values[r] == min(cap, c * tiles[r]) for r in rows):
+                return {"op": "minimum", "lhs": _constant(cap),
+                        "rhs": {"op": "multiply", "lhs": _constant(c), "rhs": _ceil_div_rows(d)}}
     for d in (128,):
         below = [r for r in rows if values[r] < cap]
         if not below:

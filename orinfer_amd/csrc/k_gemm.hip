@@ -743,7 +743,7 @@ bool use_resident(const orx_function& f, int rows) {
 // rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
 bool split_preferred_to_big(const orx_function& f, int rows);
 bool use_big(const orx_function& f, int rows) {
-    if (f.K % kBK) return false;  // half a K step at the end: the 32-128 row tiles only
+    if (f.K % kBK || f.K < 2 * kBK) return false;  // half a K step at the end, or a single step: the 32-128 row tiles only
     return f.tiles == 256 || (f.tiles == 0 && rows > 384 && !split_preferred_to_big(f, rows));
 }
 
@@ -1120,7 +1120,7 @@ int row_q4_unpack(const void* w, void* out, int n, int k, uint32_t low, uint32_t
 }
 
 constexpr int kRowQ4BigRows = 512;
-bool row_q4_expands(const orx_function& f, int rows) { return f.takes_workspace && rows >= kRowQ4BigRows; }
+bool row_q4_expands(const orx_function& f, int rows) { return f.takes_workspace && rows >= kRowQ4BigRows && f.K >= 2 * kBK; }
 // 65..511 rows: the K steps of the 128-row tiles dealt evenly to the CUs when whole tiles would not spread evenly
 // (the rule of the other codecs: 8 to 288 tiles that do not divide over the CUs)
 bool row_q4_splits(const orx_function& f, int rows) { return rows > 64 && !row_q4_expands(f, rows) && split_shape_ok(f, rows); }

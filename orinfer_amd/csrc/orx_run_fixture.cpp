@@ -5,7 +5,7 @@
 //
 // Sequence (same order as the reference harness):
 //   1. allocate and upload every buffer, check pointer alignment
-//   2. per kernel record: orx_resolve, orx_query limits, launch record checked against orx_geometry
+//   2. per kernel record: orx_resolve, orx_query_rows limits, launch record checked against orx_geometry
 //   3. launch all records on one stream; compare the named output with an fp32 reference file by
 //      relative L2
 //   4. capture the records in a graph; poison the output with 0xFF, replay, require byte-identical
@@ -258,8 +258,9 @@ int run(const std::string& manifest_path, std::ostringstream& report) {
         orx(orx_resolve(symbol->text.c_str(), variant && variant->kind == Json::Object ? variant->text.c_str() : "{}", &record.function),
             "orx_resolve");
         uint32_t max_threads = 0, static_lds = 0;
-        orx(orx_query(record.function, &max_threads, &static_lds), "orx_query");
         const int rows = (int)as_number(k.get("rows"), 0);
+        // the limits of the kernel that these rows start (a projection handle picks its kernel by the live rows)
+        orx(orx_query_rows(record.function, rows, &max_threads, &static_lds), "orx_query_rows");
         uint32_t grid[3], block[3], shared = 0;
         orx(orx_geometry(record.function, rows, grid, block, &shared), "orx_geometry");
         for (int d = 0; d < 3; ++d) record.grid[d] = grid[d], record.block[d] = block[d];
@@ -308,7 +309,7 @@ int run(const std::string& manifest_path, std::ostringstream& report) {
                 const int32_t scalar = (int32_t)value->number;
                 std::memcpy(&record.pointer_values[a], &scalar, sizeof scalar);
             } else {
-                die("kernel " + symbol->text + ": argument must be {\"buffer\"} or {\"i32\"}");
+                die("kernel " + symbol->text + ": argument must be a buffer or an i32 object");
             }
         }
         for (auto& v : record.pointer_values) record.args.push_back(&v);

@@ -92,8 +92,8 @@ def test_two_record_program_and_rejected_record(tmp_path):
     buffers = [put(tmp_path, "X", x), put(tmp_path, "Weight", weight), put(tmp_path, "WS", ws),
                {"name": "Q", "bytes": m * k, "fill": 0}, {"name": "S", "bytes": m * 2, "fill": 0},
                {"name": "Out", "bytes": m * n * 2, "fill": 0}]
-    quant = {"symbol": "activation_quantization", "variant": {"K": k, "M": m},
-             "args": [{"null": True}, {"buffer": "Q"}, {"buffer": "S"}, {"buffer": "X"}, {"i32": m}], "rows": m}
+    quant = {"symbol": "activation_quantization", "variant": {"K": k, "M": m, "omit": "Mask"},  # no mask: out of the list
+             "args": [{"buffer": "Q"}, {"buffer": "S"}, {"buffer": "X"}, {"i32": m}], "rows": m}
     project = {"symbol": "int8_projection", "variant": {"M": m, "N": n, "K": k},
                "args": [{"buffer": "Q"}, {"buffer": "Out"}, {"buffer": "S"}, {"buffer": "Weight"}, {"buffer": "WS"}]}
     validation = {"output": "Out", "output_dtype": "f16", "reference": "Out.f32", "relative_l2_tolerance": 1e-3,

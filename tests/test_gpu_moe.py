@@ -939,8 +939,8 @@ def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
     ]
     for symbol, variant in forms:
         kern = gu.lib.Kernel(symbol, **variant)
-        threads, _ = kern.query()
         for rows in ({1, variant["M"]} if variant.get("dynamic_rows") else {0}):
+            threads, _ = kern.query(rows)
             block = kern.geometry(rows)[1]
             assert block[0] * block[1] * block[2] <= threads, (symbol, variant, rows, block, threads)
     # a projection handle starts a different kernel per row range: the limits are those of the kernel that the rows
@@ -956,7 +956,7 @@ def test_every_form_reports_a_thread_limit_that_holds_its_own_block():
             assert threads == block[0] * block[1] * block[2], (symbol, rows, block, threads)
             assert static_lds + shared <= 160 * 1024
             limits[rows] = threads
-        assert kern.query() == kern.query(variant["M"]) and len(set(limits.values())) >= 3, limits
+        assert kern.query() == kern.query(variant["M"]) and len(set(limits.values())) >= 2, limits
         with pytest.raises(gu.lib.OrxError):
             kern.query(variant["M"] + 1)
 
