@@ -76,18 +76,13 @@ __device__ __forceinline__ void wait_direct_loads_except() {
 // 16-byte LDS read whose wait is placed by hand.  The compiler waits for EVERY outstanding LDS read before the first
 // multiply that follows a batch of reads (s_waitcnt lgkmcnt(0)), also when those multiplies use fragments that were
 // requested a whole sub-step earlier, which undoes the software pipeline; a read issued from an asm statement is
-// invisible to that pass, and frag_wait<N>() below is the wait: at most N younger LDS requests may still be in flight
-// (LDS requests of a wave complete in order).
+// invisible to that pass, and the wait is an asm statement of its own that names how many younger LDS requests may still
+// be in flight (LDS requests of a wave complete in order).
 template <int OFFSET>
 __device__ __forceinline__ v4i lds_read_16(uint32_t lds_address) {
     v4i value;
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
     return value;
-}
-// The fragments pass through the statement, so no multiply that uses them can move in front of the wait.
-template <int N>
-__device__ __forceinline__ void frag_wait(v4i (&a)[4], v4i (&b)[2]) {
-    asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]) : "n"(N));
 }
 __device__ __forceinline__ uint32_t lds_address_of(const void* pointer) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)pointer;
@@ -428,17 +423,19 @@ __global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigP
 // One workgroup per CU walks a static list of tiles (tile r of workgroup w is number w + r * gridDim.x of the
 // XCD-aware order), and the K steps of all its tiles form ONE software pipeline: the operand requests of the
 // next tile's first steps go out while the current tile's last steps multiply, so no tile after the first pays a
-// prologue.  The epilogue is private to a wave and stays in registers: the two lanes that hold the halves of a row's
-// eight consecutive channels trade words (v_permlane32_swap), after which every lane stores 16-byte pieces of output
-// rows.  It needs no LDS, no workgroup barrier, and leaves both operand stages alone (they already hold the next
-// tile's first steps); its stores are not waited for and drain under the next tile's multiplies.
+// prologue.  The epilogue is private to a wave and stays in registers: lanes that hold neighbouring channels of a
+// row trade words (v_permlane16_swap), after which every lane stores 16-byte pieces of output rows.  It needs no
+// LDS, no workgroup barrier, and leaves both operand stages alone (they already hold the next tile's first
+// steps); its stores are not waited for and drain under the next tile's multiplies.
 //
-// The kernel is bound by power, not by issue slots: the clock inside the K loop settles near 1.2-1.3 GHz, and taking
-// out the operand requests or half of the fragment reads shortens the loop by what they cost in energy (14 % and
-// 10 %), with stalls unchanged.  What pays is fewer bytes moved per multiply: TN = 4 gives a wave 128 x 128 of the
-// tile (four waves, one per SIMD, accumulators in AGPRs), which reads 0.5 KiB of fragments per MFMA instead of
-// 0.75 KiB with 128 x 64 (TN = 2, eight waves).
+// The kernel is bound by power, not by issue slots: on random int8 data the clock inside the K loop settles near
+// 1.2-1.3 GHz, the same launch on zero operands is 30 % shorter, and taking out stalls alone changes nothing at
+// large K.  What pays is less energy per multiply.  v_mfma_i32_16x16x64_i8 does the same work per cycle as
+// v_mfma_i32_32x32x32_i8 with half the accumulator traffic per multiply and sustains 3.83 POP/s on random
+// operands where the 32 x 32 shape sustains 3.37 (back-to-back issue from registers, whole chip); the fragment
+// bytes read from LDS per multiply are the same, so the tile, the stages and the swizzle stay as they were.
 constexpr uint32_t kPersistentLds = 4 * kTileBytes + 2 * kTile * 4;
+constexpr int kPersistentThreads = 512;
 
 struct TileState {
     int row0, col0, rows_here, cols_here;
@@ -455,14 +452,16 @@ __device__ __forceinline__ uint32_t pack_halves(float low, float high) {
     return *reinterpret_cast<const uint32_t*>(&rounded);
 }
 
+// The four fragments pass through the statement, so no multiply that uses them can move in front of the wait: at
+// most N younger LDS requests of this wave may still be in flight behind them (they complete in order).
 template <int N>
-__device__ __forceinline__ void frag_wait_n(v4i (&a)[4], v4i (&b)[2]) {
-    frag_wait<N>(a, b);
+__device__ __forceinline__ void wait_four(v4i (&f)[4]) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]) : "n"(N));
 }
 template <int N>
-__device__ __forceinline__ void frag_wait_n(v4i (&a)[4], v4i (&b)[4]) {
+__device__ __forceinline__ void wait_eight(v4i (&f)[4], v4i (&g)[4]) {
     asm volatile("s_waitcnt lgkmcnt(%8)"
-                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3])
+                 : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(g[0]), "+v"(g[1]), "+v"(g[2]), "+v"(g[3])
                  : "n"(N));
 }
 
@@ -472,31 +471,15 @@ __device__ __forceinline__ const int8_t* uniform_pointer(const int8_t* pointer) 
     return reinterpret_cast<const int8_t*>(((uint64_t)high << 32) | low);
 }
 
-// One multiply-accumulate.  With 128 x 128 per wave the 256 accumulator registers have to live in AGPRs; written with
-// the builtin, the register allocator keeps them as single VGPR values and copies sixteen of them into an AGPR tuple
-// in front of every multiply.  An asm statement with an AGPR constraint pins them there.  The compiler does not know
-// that statement as a matrix instruction, so the one hazard that it would otherwise pad is padded by hand where it
-// can occur: a vector-ALU read of an accumulator right behind the last multiply (settle_accumulators()).
-template <bool AGPR>
-__device__ __forceinline__ void multiply_add(v16i& acc, const v4i& weights, const v4i& tokens) {
-    if constexpr (AGPR)
-        asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(weights), "v"(tokens));
-    else
-        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(weights, tokens, acc, 0, 0, 0);
-}
-__device__ __forceinline__ void settle_accumulators() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
-
-// F32: fp32 output (heads); its own instantiation, so that either kernel holds one epilogue (with both in one kernel
-// the accumulator reads of the two branches are merged and hoisted in front of the branch: 256 live registers).
-template <int TN, bool F32>
-__global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParams p) {
-    constexpr int TM = 4, WAVES_N = 8 / TN, WAVES = 2 * WAVES_N, kThreads = 64 * WAVES, BLOCKS_PER_WAVE = 32 / WAVES;
-    constexpr int READS = TM + TN;  // fragment reads per sub-step
-#ifdef ORX_ASM_MULTIPLY
-    constexpr bool kAsmMultiply = TN == 4;
-#else
-    constexpr bool kAsmMultiply = false;
-#endif
+// F32: fp32 output (heads); its own instantiation, so that either kernel holds one epilogue.
+//
+// Eight waves share the 256 x 256 tile, 128 token rows x 64 channels each: 8 x 4 blocks of 16 x 16, 128 accumulator
+// registers.  A K step of 128 is two MFMA K slices of 64; a slice is multiplied in two phases of 16 multiplies
+// (token blocks 0-3, then 4-7, against the slice's four channel blocks), so that only four token fragments and four
+// weight fragments are live per phase and a second set is on its way from LDS: 64 fragment registers.
+template <bool F32>
+__global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel(BigParams p) {
+    constexpr int WAVES_N = 4, kThreads = kPersistentThreads, BLOCKS_PER_WAVE = 4;
     extern __shared__ __align__(16) int8_t lds[];  // [2 stages][A 32 KiB | W 32 KiB], 512 scales
     float* const lds_as = reinterpret_cast<float*>(lds + 4 * kTileBytes);  // 256 token scales, then 256 weight scales
     float* const lds_ws = lds_as + kTile;
@@ -524,21 +507,17 @@ __global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParam
     // ---- load cursor: the step whose operands are being requested (clamped at this workgroup's last step) ----
     const int load_r8 = lane >> 3, load_slot = lane & 7;
     int load_tile = 0, load_kt = 0;
-    // byte offset of this lane's 16 bytes from the tile's first row: unsigned 32-bit, so that a request is a uniform
-    // 64-bit base plus a 32-bit lane offset and needs no 64-bit address registers
-    uint32_t a_offset[BLOCKS_PER_WAVE], w_offset[BLOCKS_PER_WAVE];
+    // A request is a uniform 64-bit base (the tile's first row, the K step) plus a 32-bit lane offset, computed when
+    // it is issued from two lane registers rather than kept per request: block b of this wave starts 8 b rows below the
+    // lane's first row, and the swizzled chunk of odd blocks is that of even blocks with bit 2 flipped.
+    const int load_row = wave * (BLOCKS_PER_WAVE * 8) + load_r8;                 // row of block 0
+    const uint32_t load_chunk = (uint32_t)((load_slot ^ swizzle(load_row)) * 16);
+    int load_rows = 0, load_cols = 0;  // live rows and channels of the tile being requested
     const int8_t* a_base = nullptr;
     const int8_t* w_base = nullptr;
     auto aim = [&](const TileState& t) {
-#pragma unroll
-        for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
-            const int row = (wave * BLOCKS_PER_WAVE + b) * 8 + load_r8;
-            const int chunk = load_slot ^ swizzle(row);
-            a_offset[b] = (uint32_t)(min(row, t.rows_here - 1) * p.k + chunk * 16);
-            w_offset[b] = (uint32_t)(min(row, t.cols_here - 1) * p.k + chunk * 16);
-        }
-        // (said to be uniform in so many words: the bases then live in scalar registers and a request is
-        // scalar base + 32-bit lane offset)
+        load_rows = t.rows_here, load_cols = t.cols_here;
+        // (said to be uniform in so many words: the bases then live in scalar registers)
         a_base = uniform_pointer(p.a + (int64_t)t.row0 * p.k);
         w_base = uniform_pointer(w8 + (int64_t)t.col0 * p.k);
     };
@@ -553,80 +532,63 @@ __global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParam
     auto issue_one = [&](int id, int stage) {  // id < BLOCKS_PER_WAVE: activations, else weights
         const bool weights = id >= BLOCKS_PER_WAVE;
         const int b = weights ? id - BLOCKS_PER_WAVE : id;
-        // (the offset is made opaque, or base + offset is kept as a 64-bit register pair per request for the whole loop)
-        if (weights) {
-            uint32_t offset = w_offset[b];
-            asm volatile("" : "+v"(offset));
-            direct_load_16(w_base + load_kt * kStep + (uint64_t)offset, stage_w(stage) + (wave * BLOCKS_PER_WAVE + b) * 1024);
-        } else {
-            uint32_t offset = a_offset[b];
-            asm volatile("" : "+v"(offset));
-            direct_load_16(a_base + load_kt * kStep + (uint64_t)offset, stage_a(stage) + (wave * BLOCKS_PER_WAVE + b) * 1024);
-        }
+        // (the row is made opaque, or every request's offset is computed once and kept in a register for the whole loop)
+        int row = load_row;
+        asm volatile("" : "+v"(row));
+        const uint32_t offset = (uint32_t)(min(row + 8 * b, (weights ? load_cols : load_rows) - 1) * p.k) + (load_chunk ^ (uint32_t)((b & 1) * 64));
+        direct_load_16((weights ? w_base : a_base) + load_kt * kStep + (uint64_t)offset,
+                       (weights ? stage_w(stage) : stage_a(stage)) + (wave * BLOCKS_PER_WAVE + b) * 1024);
     };
 
-    // ---- fragment addressing: LDS byte address of this lane's 16 bytes of sub-step ks in stage 0 ----
-    const int frag_row = lane & 31, frag_half = lane >> 5;
-    const int swz = swizzle(frag_row);
-    uint32_t a_frag[4], w_frag[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        const int offset = ((2 * ks + frag_half) ^ swz) * 16;
-        a_frag[ks] = lds_address_of(lds) + (wave_m * TM * 32 + frag_row) * kStep + offset;
-        w_frag[ks] = lds_address_of(lds) + kTileBytes + (wave_n * TN * 32 + frag_row) * kStep + offset;
-    }
+    // ---- fragment addressing: a lane reads K bytes [16 (lane / 16), +16) of K slice s for row lane % 16 of a block ----
+    const int frag_row = lane & 15, frag_chunk = lane >> 4;
+    const int swz = swizzle(frag_row);  // the same in every block of 16 rows
+    // LDS byte address of that piece for K slice 0 in stage 0, first block of the wave; slice 1 is the same address
+    // with bit 6 flipped (chunk 4 + c swizzles to the chunk of c with bit 2 flipped, and rows start at multiples of 128)
+    const uint32_t a_frag = lds_address_of(lds) + (wave_m * 128 + frag_row) * kStep + ((frag_chunk ^ swz) * 16);
+    const uint32_t w_frag = lds_address_of(lds) + kTileBytes + (wave_n * 64 + frag_row) * kStep + ((frag_chunk ^ swz) * 16);
 
-    v16i acc[TM][TN];
+    v4i acc[8][4];  // [token block][channel block]: channels 4 (lane / 16) + {0..3} of the block, token lane % 16
     auto clear = [&]() {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < 8; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                if constexpr (kAsmMultiply) {
-                    // every definition of an accumulator comes from an AGPR-constrained statement, or the values
-                    // travel through VGPRs around the loop: zero = 0 x 0 + 0
-                    const v4i zero = {0, 0, 0, 0};
-                    asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %1, 0" : "=a"(acc[i][j]) : "v"(zero));
-                } else {
-                    acc[i][j] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                }
-            }
+            for (int j = 0; j < 4; ++j) acc[i][j] = v4i{0, 0, 0, 0};
     };
     clear();
 
-    v4i fa[2][TM], fb[2][TN];
-    auto read_fragments = [&](int stage, int ks, int slot) {
-        const uint32_t a = a_frag[ks] + stage * (2 * kTileBytes), w = w_frag[ks] + stage * (2 * kTileBytes);
-        fa[slot][0] = lds_read_16<0>(a);
-        fa[slot][1] = lds_read_16<32 * kStep>(a);
-        fa[slot][2] = lds_read_16<64 * kStep>(a);
-        fa[slot][3] = lds_read_16<96 * kStep>(a);
-        fb[slot][0] = lds_read_16<0>(w);
-        fb[slot][1] = lds_read_16<32 * kStep>(w);
-        if constexpr (TN == 4) {
-            fb[slot][2] = lds_read_16<64 * kStep>(w);
-            fb[slot][3] = lds_read_16<96 * kStep>(w);
-        }
+    v4i ft[2][4], fw[2][4];  // token fragments of a phase, weight fragments of a K slice; two sets each
+    constexpr int kBlockBytes = 16 * kStep;
+    auto read_tokens = [&](int stage, int phase) {  // phase = 2 * slice + half; into set phase % 2
+        const uint32_t a = (a_frag ^ (uint32_t)((phase >> 1) * 64)) + stage * (2 * kTileBytes) + (phase & 1) * 4 * kBlockBytes;
+        v4i(&f)[4] = ft[phase & 1];
+        f[0] = lds_read_16<0>(a);
+        f[1] = lds_read_16<kBlockBytes>(a);
+        f[2] = lds_read_16<2 * kBlockBytes>(a);
+        f[3] = lds_read_16<3 * kBlockBytes>(a);
     };
-    auto multiply = [&](int slot) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                multiply_add<kAsmMultiply>(acc[i][j], fb[slot][j], fa[slot][i]);
+    auto read_weights = [&](int stage, int slice) {  // into set `slice`
+        const uint32_t w = (w_frag ^ (uint32_t)(slice * 64)) + stage * (2 * kTileBytes);
+        v4i(&f)[4] = fw[slice];
+        f[0] = lds_read_16<0>(w);
+        f[1] = lds_read_16<kBlockBytes>(w);
+        f[2] = lds_read_16<2 * kBlockBytes>(w);
+        f[3] = lds_read_16<3 * kBlockBytes>(w);
     };
-    // a wave's requests of a K step go out one at a time behind every second multiply of three groups (a wave cannot
+    // a wave's requests of a K step go out one at a time behind every second multiply of three phases (a wave cannot
     // issue anything while a vector-memory instruction waits for a slot in the CU's memory pipeline)
     constexpr int LOADS = 2 * BLOCKS_PER_WAVE;
     constexpr int PART0 = (LOADS + 2) / 3, PART1 = (LOADS - PART0 + 1) / 2, PART2 = LOADS - PART0 - PART1;
-    static_assert(PART0 <= TM * TN / 2 && PART1 <= TM * TN / 2, "one request after every second multiply of a group");
-    auto multiply_loading = [&](int slot, int first, int count, int stage) {
+    auto multiply_loading = [&](int phase, int first, int count, int stage) {
+        v4i(&tokens)[4] = ft[phase & 1];
+        v4i(&weights)[4] = fw[phase >> 1];
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                multiply_add<kAsmMultiply>(acc[i][j], fb[slot][j], fa[slot][i]);
-                const int index = i * TN + j;
+            for (int j = 0; j < 4; ++j) {
+                v4i& sum = acc[4 * (phase & 1) + i][j];
+                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights[j], tokens[i], sum, 0, 0, 0);
+                const int index = i * 4 + j;
                 if ((index & 1) == 1 && index / 2 < count) {
                     __builtin_amdgcn_sched_barrier(0);
                     issue_one(first + index / 2, stage);
@@ -641,71 +603,62 @@ __global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParam
         // computed once in front of the K loop and held in registers (or spilled) for the whole kernel
         int lane = threadIdx.x & 63;
         asm volatile("" : "+v"(lane));
-        const int half = lane >> 5;
+        const int group = lane >> 4;
         if constexpr (F32) {
             // fp32 heads are rare: 16-byte stores straight from the accumulators
             const bool vector_ok = p.stride % 4 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
+            for (int i = 0; i < 8; ++i) {
+                const int local_row = wave_m * 128 + i * 16 + (lane & 15);
                 if (local_row >= t.rows_here) continue;
                 const int64_t row = t.row0 + local_row;
                 const float token_scale = lds_as[local_row];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) {
+                for (int j = 0; j < 4; ++j) {
+                    const int local_col = wave_n * 64 + j * 16 + 4 * group;
+                    if (local_col >= t.cols_here) continue;
+                    const int col = t.col0 + local_col;
+                    const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
+                    const float value[4] = {rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale),
+                                            rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale)};
+                    float* dst = reinterpret_cast<float*>(p.out) + row * p.stride + col;
+                    if (local_col + 4 <= t.cols_here && vector_ok && (col & 3) == 0) {
+                        *reinterpret_cast<float4*>(dst) = make_float4(value[0], value[1], value[2], value[3]);
+                    } else {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int local_col = (wave_n * TN + j) * 32 + 8 * q + 4 * half;
-                        if (local_col >= t.cols_here) continue;
-                        const int col = t.col0 + local_col;
-                        const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
-                        const float value[4] = {rescale(acc[i][j][4 * q + 0], wscale.x, token_scale),
-                                                rescale(acc[i][j][4 * q + 1], wscale.y, token_scale),
-                                                rescale(acc[i][j][4 * q + 2], wscale.z, token_scale),
-                                                rescale(acc[i][j][4 * q + 3], wscale.w, token_scale)};
-                        float* dst = reinterpret_cast<float*>(p.out) + row * p.stride + col;
-                        if (local_col + 4 <= t.cols_here && vector_ok && (col & 3) == 0) {
-                            *reinterpret_cast<float4*>(dst) = make_float4(value[0], value[1], value[2], value[3]);
-                        } else {
-#pragma unroll
-                            for (int r = 0; r < 4; ++r)
-                                if (local_col + r < t.cols_here) dst[r] = value[r];
-                        }
+                        for (int r = 0; r < 4; ++r)
+                            if (local_col + r < t.cols_here) dst[r] = value[r];
                     }
                 }
             }
             return;
         } else {
-        // Weights are the MFMA row operand, so a lane holds token row (lane & 31) of each 32 x 32 block and, per group
-        // of four accumulator registers, four consecutive output channels 8 q + 4 (lane >> 5) + {0..3}: lanes l and
-        // l + 32 hold the two halves of the same eight channels.  One swap of the upper 32 lanes of group q with the
-        // lower 32 lanes of group q + 2 leaves lane l < 32 with all eight channels of group q and lane l + 32 with those
-        // of group q + 2: 16 contiguous bytes of an output row per lane and store.
-        const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-        const bool whole = aligned && t.rows_here == kTile && t.cols_here == kTile;  // no bounds inside this tile
+            // Weights are the MFMA row operand, so a lane holds token lane % 16 of each 16 x 16 block and four consecutive
+            // output channels 4 (lane / 16) + {0..3}: two words of fp16.  One swap of the odd rows of 16 lanes of channel
+            // block j with the even rows of block j + 1 leaves lane groups 0 and 2 with channels 0-7 and 8-15 of block j
+            // and groups 1 and 3 with those of block j + 1: 16 contiguous bytes of an output row per lane and store, and a
+            // store instruction covers 16 rows x 64 bytes.
+            const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+            const bool whole = aligned && t.rows_here == kTile && t.cols_here == kTile;  // no bounds inside this tile
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
-            const float token_scale = lds_as[local_row];
-            __half* const row_out = reinterpret_cast<__half*>(p.out) + (int64_t)(t.row0 + local_row) * p.stride + t.col0;
+            for (int i = 0; i < 8; ++i) {
+                const int local_row = wave_m * 128 + i * 16 + (lane & 15);
+                const float token_scale = lds_as[local_row];
+                __half* const row_out = reinterpret_cast<__half*>(p.out) + (int64_t)(t.row0 + local_row) * p.stride + t.col0;
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                const int block_col = (wave_n * TN + j) * 32;
-                uint32_t words[4][2];
+                for (int pair = 0; pair < 2; ++pair) {  // channel blocks (0, 1), then (2, 3)
+                    uint32_t words[2][2];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + block_col + 8 * q + 4 * half);
-                    words[q][0] = pack_halves(rescale(acc[i][j][4 * q + 0], wscale.x, token_scale),
-                                              rescale(acc[i][j][4 * q + 1], wscale.y, token_scale));
-                    words[q][1] = pack_halves(rescale(acc[i][j][4 * q + 2], wscale.z, token_scale),
-                                              rescale(acc[i][j][4 * q + 3], wscale.w, token_scale));
-                }
-#pragma unroll
-                for (int pair = 0; pair < 2; ++pair) {  // groups (0, 2), then (1, 3)
-                    const v2u low = __builtin_amdgcn_permlane32_swap(words[pair][0], words[pair + 2][0], false, false);
-                    const v2u high = __builtin_amdgcn_permlane32_swap(words[pair][1], words[pair + 2][1], false, false);
+                    for (int b = 0; b < 2; ++b) {
+                        const int j = 2 * pair + b;
+                        const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + wave_n * 64 + j * 16 + 4 * group);
+                        words[b][0] = pack_halves(rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale));
+                        words[b][1] = pack_halves(rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale));
+                    }
+                    const v2u low = __builtin_amdgcn_permlane16_swap(words[0][0], words[1][0], false, false);
+                    const v2u high = __builtin_amdgcn_permlane16_swap(words[0][1], words[1][1], false, false);
                     const uint4 piece = make_uint4(low.x, high.x, low.y, high.y);
-                    const int local_col = block_col + 8 * (pair + 2 * half);
+                    const int local_col = wave_n * 64 + (2 * pair + (group & 1)) * 16 + (group >> 1) * 8;
                     if (whole) {
                         *reinterpret_cast<uint4*>(row_out + local_col) = piece;
                     } else if (local_row < t.rows_here && local_col < t.cols_here) {
@@ -719,10 +672,9 @@ __global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParam
                                     row_out[local_col + e] = __ushort_as_half((unsigned short)(parts[e >> 1] >> (16 * (e & 1))));
                         }
                     }
+                    __builtin_amdgcn_sched_barrier(0);  // one pair at a time: interleaved pairs cost registers, not time
                 }
-                __builtin_amdgcn_sched_barrier(0);  // one block at a time: interleaved blocks cost registers, not time
             }
-        }
         }
     };
 
@@ -738,78 +690,86 @@ __global__ __launch_bounds__(1024 / TN) void gemm_big_persistent_kernel(BigParam
     }
     wait_direct_loads();
     __syncthreads();
-    read_fragments(0, 0, 0);
+    read_tokens(0, 0);
+    read_weights(0, 0);
 
-    // Step g: sub-steps 0..2 read fragments ks+1 and multiply ks; barrier (step g+1 is complete in LDS and nobody
-    // reads stage `cur` any more); fragments 0 of step g+1; multiplies of sub-step 3 (operands already in registers)
-    // while the requests of step g+2 start into stage `cur`.  The load cursor points at step g+1 until the second
-    // group of requests is out, then at step g+2; at the end of the list it stays on the last step, whose repeated
-    // requests land in a stage that is not read again.  A tile's last step (LAST) also brings the tile's scales into
-    // LDS and keeps its first requests of step g+2 back until the epilogue has read them (a read of LDS waits for
-    // every direct-to-LDS request in flight).
+    // Step g, four phases: each requests the fragments of the next phase, waits for its own (requested a phase
+    // earlier: only the younger batch may still be in flight) and multiplies.  Behind phase 2 comes the barrier (step
+    // g+1 is complete in LDS and nobody reads stage `cur` any more); then the fragments of step g+1's first phase,
+    // and phase 3, whose operands are already in registers, while the requests of step g+2 start into stage `cur`.
+    // The load cursor points at step g+1 until the second group of requests is out, then at step g+2; at the end of
+    // the list it stays on the last step, whose repeated requests land in a stage that is not read again.  A tile's
+    // last step (LAST) also brings the tile's scales into LDS and keeps its first requests of step g+2 back until the
+    // epilogue has read them (a read of LDS waits for every direct-to-LDS request in flight).
     int g = 0;
     auto k_step = [&](auto last_tag) {
         constexpr bool LAST = decltype(last_tag)::value;
         const int cur = g & 1, nxt = cur ^ 1;
-        // this tile's scales (token scales by the first 256 threads, weight scales by the rest, or one of each per
-        // thread of a four-wave workgroup): in LDS before the barrier below, read by the epilogue after it
-        uint32_t scale_bits = 0, more_bits = 0;
+        // this tile's scales, token scales by the first 256 threads and weight scales by the rest: in LDS before the
+        // barrier below, read by the epilogue after it
+        // (which of the two is the same for a whole wave, so the base stays in scalar registers; the lane number is
+        // opaque so that no part of the address is carried through the K loop)
+        uint32_t scale_bits = 0;
+        int scale_index = 0;
         if constexpr (LAST) {
-            const unsigned short* token_bits = reinterpret_cast<const unsigned short*>(p.as) + tile.row0;
-            const unsigned short* weight_bits = reinterpret_cast<const unsigned short*>(p.ws) + tile.col0;
-            if constexpr (kThreads == 2 * kTile) {
-                scale_bits = tid < kTile ? token_bits[min(tid, tile.rows_here - 1)] : weight_bits[min(tid - kTile, tile.cols_here - 1)];
-            } else {
-                scale_bits = token_bits[min(tid, tile.rows_here - 1)];
-                more_bits = weight_bits[min(tid, tile.cols_here - 1)];
-            }
+            int own = threadIdx.x & 63;
+            asm volatile("" : "+v"(own));
+            scale_index = (wave & 3) * 64 + own;
+            if (wave < 4)
+                scale_bits = reinterpret_cast<const unsigned short*>(p.as)[tile.row0 + min(scale_index, tile.rows_here - 1)];
+            else
+                scale_bits = reinterpret_cast<const unsigned short*>(p.ws)[tile.col0 + min(scale_index, tile.cols_here - 1)];
         }
-        // each batch of fragment reads is waited for one sub-step later: one younger batch may still be in flight
-        read_fragments(cur, 1, 1);
-        frag_wait_n<READS>(fa[0], fb[0]);
+        read_tokens(cur, 1);                  // 4 younger requests
+        wait_eight<4>(ft[0], fw[0]);
         __builtin_amdgcn_sched_barrier(0);
         multiply_loading(0, PART0, PART1, nxt);
         __builtin_amdgcn_sched_barrier(0);
-        read_fragments(cur, 2, 0);
-        frag_wait_n<READS>(fa[1], fb[1]);
+        read_tokens(cur, 2);                  // 8 younger requests
+        read_weights(cur, 1);
+        wait_four<8>(ft[1]);
         __builtin_amdgcn_sched_barrier(0);
         multiply_loading(1, PART0 + PART1, PART2, nxt);
         __builtin_amdgcn_sched_barrier(0);
         advance();
-        read_fragments(cur, 3, 1);
-        frag_wait_n<READS>(fa[0], fb[0]);
+        read_tokens(cur, 3);                  // 4 younger requests
+        wait_eight<4>(ft[0], fw[1]);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(0);
+        multiply_loading(2, 0, 0, nxt);
         __builtin_amdgcn_sched_barrier(0);
         wait_loads_and_reads();
-        frag_wait_n<0>(fa[1], fb[1]);
+        wait_four<0>(ft[1]);
         if constexpr (LAST) {
             // (the raw bits stay opaque up to here, or the conversion and with it the wait for the load would move up
             // to the request itself)
-            asm volatile("" : "+v"(scale_bits), "+v"(more_bits));
-            lds_as[tid] = __half2float(__ushort_as_half((unsigned short)scale_bits));  // lds_ws follows lds_as
-            if constexpr (kThreads == kTile) lds_ws[tid] = __half2float(__ushort_as_half((unsigned short)more_bits));
+            asm volatile("" : "+v"(scale_bits));
+            (wave < 4 ? lds_as : lds_ws)[scale_index] = __half2float(__ushort_as_half((unsigned short)scale_bits));
         }
         __syncthreads();
-        if (g + 1 < total_steps) read_fragments(nxt, 0, 0);
+        // (a tile's last step leaves these reads to the tile loop, behind the epilogue: 32 registers less to carry
+        // through it, for one LDS latency per tile)
+        if (!LAST) {
+            read_tokens(nxt, 0);
+            read_weights(nxt, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (LAST)
-            multiply(1);
-        else
-            multiply_loading(1, 0, PART0, cur);
+        multiply_loading(3, 0, LAST ? 0 : PART0, cur);
         __builtin_amdgcn_sched_barrier(0);
         ++g;
     };
     for (int tile_index = 0; tile_index < my_tiles; ++tile_index) {
         for (int kt = 0; kt + 1 < k_tiles; ++kt) k_step(std::false_type{});
         k_step(std::true_type{});
-        if constexpr (kAsmMultiply) settle_accumulators();
         epilogue(tile);
         clear();
         tile = tile_state(tile_index + 1);
         const int cur = (g - 1) & 1;
 #pragma unroll
         for (int id = 0; id < PART0; ++id) issue_one(id, cur);
+        if (g < total_steps) {  // the next tile's first fragments (its first step was published by the last barrier)
+            read_tokens(g & 1, 0);
+            read_weights(g & 1, 0);
+        }
     }
     // a workgroup must not end with direct-to-LDS requests in flight
     wait_direct_loads();
@@ -823,19 +783,15 @@ constexpr uint32_t kBigLdsQ4 = 4 * kTileBytes + sizeof(Q4ByteTables) > kBigLdsEp
                                    : kBigLdsEpilogue;
 
 // wave shape of the shipped kernels
-#ifndef ORX_PERSISTENT_TN
-#define ORX_PERSISTENT_TN 2
-#endif
-constexpr int kPersistentTN = ORX_PERSISTENT_TN;
 constexpr int kTM = ORX_BIG_TM, kTN = ORX_BIG_TN;
 constexpr int kBigThreads = (8 / kTM) * (8 / kTN) * 64;
 
 int prepare_device() {
-    int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_persistent_kernel<kPersistentTN, false>),
+    int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_persistent_kernel<false>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPersistentLds),
                          "hipFuncSetAttribute");
     if (code != ORX_OK) return code;
-    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_persistent_kernel<kPersistentTN, true>),
+    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_persistent_kernel<true>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPersistentLds),
                      "hipFuncSetAttribute");
     if (code != ORX_OK) return code;
@@ -899,7 +855,7 @@ void gemm_big_geometry(int rows, int n, bool q4, Geometry* g) {
     // int8 weights: one persistent workgroup per CU walks the tiles; two-stage codes decoded in the loop: one per tile
     g->grid[0] = q4 ? tiles : std::min(tiles, (uint32_t)device_compute_units());
     g->grid[1] = g->grid[2] = 1;
-    g->block[0] = q4 ? kBigThreads : 1024 / kPersistentTN;
+    g->block[0] = q4 ? kBigThreads : kPersistentThreads;
     g->shared = q4 ? kBigLdsQ4 : kPersistentLds;
 }
 
@@ -920,9 +876,9 @@ int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* boo
         ORX_LAUNCH((gemm_big_kernel<true, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
     else
         if (out_f32)
-            ORX_LAUNCH((gemm_big_persistent_kernel<kPersistentTN, true>), dim3(g.grid[0]), dim3(1024 / kPersistentTN), g.shared, stream, p);
+            ORX_LAUNCH((gemm_big_persistent_kernel<true>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
         else
-            ORX_LAUNCH((gemm_big_persistent_kernel<kPersistentTN, false>), dim3(g.grid[0]), dim3(1024 / kPersistentTN), g.shared, stream, p);
+            ORX_LAUNCH((gemm_big_persistent_kernel<false>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
     return hip_check(hipGetLastError(), "launch projection (mfma 256x256)");
 }
 
