@@ -78,7 +78,9 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2, kS4 = 3 };  // kS4: row-scaled scalar Q4 nibbles (q4_projection.py)
 enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4, kWide = 5 };
-enum Flags2 { kNoSplit = 1, kNoExpand = 2 };  // orx_function::flags2 of a projection
+// orx_function::flags2 of a projection.  kPreferGemv / kNoGemv: the reference's schedule names as hints among the
+// library's own kernels (algorithm=dp4a: its dot-product schedule for few rows; tensor_core: its matrix-unit one).
+enum Flags2 { kNoSplit = 1, kNoExpand = 2, kPreferGemv = 4, kNoGemv = 8 };
 
 constexpr int kBK = 128;        // K bytes per tile step
 constexpr int kPitch = kBK + 16;  // LDS row pitch in bytes
@@ -685,10 +687,18 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
 // 70-83 against 72-74 (N = 28672); 9728 and up: slower (N = 5120, K = 17408: 56-69 against 41).  Below 65
 // rows the batched-decode kernels are as fast or faster except at N = 17408 (30 against 31-34 us), above 128
 // rows a second pass doubles the time (58-62 against 57 us at 160-256 rows).
+// Row tile asked for at `rows` live rows: a block_m this library has a tile for (32, 64, 128, 256) holds at every row
+// count; a reference-only tile (16, 96, 192) was chosen for launches of about that many rows, so it names the tile
+// that holds it (32, 128, 256) while the live rows fit one such tile, and beyond that the row count decides.
+int tile_for(const orx_function& f, int rows) {
+    if (f.tiles) return f.tiles;
+    return f.tile_hint && rows <= f.tile_hint ? f.tile_hint : 0;
+}
+
 bool use_wide(const orx_function& f, int rows) {
     if (f.flags != kQ4 || !dense_wide_eligible(f.N, f.K, f.packed_k)) return false;
     if (f.algorithm == kWide) return true;
-    if (f.algorithm != kAuto || f.tiles != 0 || f.K > 6144) return false;
+    if (f.algorithm != kAuto || tile_for(f, rows) != 0 || f.K > 6144) return false;
     if (rows >= 65 && rows <= 128) return true;
     // 33..64 rows of a large matrix would be two batched-decode launches: one pass here is faster while a CU's
     // run fits one channel pass (N = 17408, K = 5120: 29.9 / 30.2 / 30.4 us at 33 / 48 / 64 rows against 31.2 / 31.8 /
@@ -701,6 +711,9 @@ bool use_gemv(const orx_function& f, int rows) {
     if (use_wide(f, rows)) return false;
     if (f.algorithm == kGemv) return true;
     if (f.algorithm != kAuto) return false;
+    if (f.flags2 & kNoGemv) return false;  // the matrix-unit kernels were asked for: streaming / batched-decode from row 1
+    if ((f.flags2 & kPreferGemv) && f.block_m > 0 && f.tiles == 0)  // the dot-product family wherever it serves the rows
+        return rows <= (f.flags == kW8 ? 2 : 4) && (f.packed_k == 0 || (rows <= 2 && gemv_serves_k_major(f, rows)));
     // K-major codes: 1 row (13.4 us at N=17408, K=5120; the streaming kernel takes 17.2), and 2 rows
     // (16.4 us) where the batched-decode kernel (15.4 us) does not take the shape
     if (f.packed_k != 0) return rows <= 2 && gemv_serves_k_major(f, rows) && !use_resident(f, rows);
@@ -714,7 +727,7 @@ bool use_gemv(const orx_function& f, int rows) {
 // 16 rows: the 32/64/128-row tiles measure 27 / 31 / 40 us at 32 / 48 / 128 rows against 29 / 43 / 94.
 bool use_stream(const orx_function& f, int rows) {
     if (f.algorithm == kStream) return rows <= 64;
-    if (f.algorithm != kAuto || f.tiles != 0) return false;
+    if (f.algorithm != kAuto || tile_for(f, rows) != 0) return false;
     if (f.flags == kQ4) return rows <= 64;
     // W8 with weights that do not stay in cache: up to 32 rows (N = 17408, K = 5120 at 32 rows: 34.8 us
     // against 39.0 us for the 32-row tiles; at 48 rows 49.0 against 42.5), up to 64 rows for matrices of
@@ -734,7 +747,7 @@ bool use_resident(const orx_function& f, int rows) {
     // (the second launch pays for itself only on large matrices: N = 17408, K = 5120 at 48 rows 33 us
     // against 39 us for the streaming kernel, but N = K = 5120 20 against 14.5 us)
     const int limit = (int64_t)f.N * f.K >= ((int64_t)1 << 26) ? 64 : 32;
-    return f.algorithm == kAuto && f.tiles == 0 && rows > 1 && rows <= limit;
+    return f.algorithm == kAuto && tile_for(f, rows) == 0 && rows > 1 && rows <= limit;
 }
 
 // 256x256 tiles once there are enough rows to fill them (or when block_m = 256 is forced)
@@ -744,7 +757,8 @@ bool use_resident(const orx_function& f, int rows) {
 bool split_preferred_to_big(const orx_function& f, int rows);
 bool use_big(const orx_function& f, int rows) {
     if (f.K % kBK || f.K < 2 * kBK) return false;  // half a K step at the end, or a single step: the 32-128 row tiles only
-    return f.tiles == 256 || (f.tiles == 0 && rows > 384 && !split_preferred_to_big(f, rows));
+    const int tile = tile_for(f, rows);
+    return tile == 256 || (tile == 0 && rows > 384 && !split_preferred_to_big(f, rows));
 }
 
 // Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel
@@ -767,7 +781,7 @@ int64_t split_tiles(const orx_function& f, int rows) {
     return (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
 }
 bool split_shape_ok(const orx_function& f, int rows) {
-    if (!f.takes_workspace || (f.flags2 & kNoSplit) || f.tiles != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
+    if (!f.takes_workspace || (f.flags2 & kNoSplit) || tile_for(f, rows) != 0 || (f.algorithm != kAuto && f.algorithm != kMfma)) return false;
     const int64_t tiles = split_tiles(f, rows);
     return tiles >= 8 && tiles <= (int64_t)split_groups() * 9 / 16 && tiles % (split_groups() / 2) != 0;
 }
@@ -839,7 +853,7 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         g->shared = 0;
         return ORX_OK;
     }
-    const int bm = f.tiles ? f.tiles : pick_bm(rows);
+    const int bm = tile_for(f, rows) ? tile_for(f, rows) : pick_bm(rows);
     g->grid[0] = ceil_div((uint32_t)f.N, 128u);
     g->grid[1] = ceil_div((uint32_t)rows, (uint32_t)bm);
     g->block[0] = 256;
@@ -895,7 +909,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         p.partials = static_cast<int*>(workspace);
         return launch_split<kQ4>(p, split_groups_for(f, rows), stream);
     }
-    return launch_mfma<kQ4, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
+    return launch_mfma<kQ4, false>(tile_for(f, rows) ? tile_for(f, rows) : pick_bm(rows), p, g, stream);
 }
 
 // W8A8: A, Output, TokenScale, Weight, WeightScale[, m]   (int8_projection.py:51-57)
@@ -927,7 +941,7 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         p.partials = static_cast<int*>(workspace);
         return launch_split<kW8>(p, split_groups_for(f, rows), stream);
     }
-    return launch_mfma<kW8, false>(f.tiles ? f.tiles : pick_bm(rows), p, g, stream);
+    return launch_mfma<kW8, false>(tile_for(f, rows) ? tile_for(f, rows) : pick_bm(rows), p, g, stream);
 }
 
 int make_projection(const Variant& v, orx_function* f, int codec) {
@@ -945,12 +959,23 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
     if (bad) return ORX_ERR_BAD_VARIANT;
     const char* name = f->symbol.c_str();
     // The reference's factories name their schedules tensor_core, dp4a and int4_direct and take row tiles of
-    // 1-8, 16, 96 and 192 as well (e8p_q4.py:143-215, int8_projection.py:15-48): those are choices among SM87
-    // kernels, so they are accepted and the library picks its own kernel by the live rows.  Its other tile
-    // keys (block_n, block_k, stages, tail_m, group_m, cache_scales, an integer split_k) are not read.
+    // 1-8, 16, 96 and 192 as well (e8p_q4.py:143-215, int8_projection.py:15-48; a package's winners come from
+    // contracts/projection_policy.py:40-101).  They are hints among the library's own kernels: dp4a (the dot-product
+    // schedule) keeps the single-row GEMV family wherever it serves the rows, tensor_core keeps to the kernels built on
+    // the matrix unit at every row count, int4_direct means no preference; a row tile of 16, 96 or 192 asks for the MFMA
+    // tile that holds it (32, 128, 256) for launches whose rows fit one such tile, and tiles of 1-8 rows, which have no
+    // tile kernel here, leave the choice to the row count.  Its other tile keys (block_n, block_k, stages, tail_m, group_m, cache_scales, an integer split_k) are
+    // not read.
+    int schedule_hint = 0;
+    if (algorithm == "dp4a") schedule_hint = kPreferGemv;
+    if (algorithm == "tensor_core") schedule_hint = kNoGemv;
     if (algorithm == "tensor_core" || algorithm == "dp4a" || algorithm == "int4_direct") algorithm = "auto";
     for (const char* hint : {"block_n", "block_k", "stages", "tail_m", "group_m", "cache_scales", "basis_nonzero", "minimum_blocks"}) v.accept(hint);
-    if ((f->tiles >= 1 && f->tiles <= 8) || f->tiles == 16 || f->tiles == 96 || f->tiles == 192) f->tiles = 0;
+    if (f->tiles >= 1 && f->tiles <= 8) f->tiles = 0;
+    if (f->tiles == 16) f->tile_hint = 32;
+    if (f->tiles == 96) f->tile_hint = 128;
+    if (f->tiles == 192) f->tile_hint = f->K % kBK == 0 && f->K >= 2 * kBK ? 256 : 128;
+    if (f->tile_hint) f->tiles = 0;
     // validate_shape + K*128*127 < 2^31 (q4_projection.py:33-35, int8_projection.py:29)
     const bool half_step = codec == kW8 && f->K % kBK == 64;  // int8_projection.py:29 takes K % 64 == 0
     if (f->M <= 0 || f->N <= 0 || f->K <= 0 || (f->K % kBK && !half_step) || (int64_t)f->K * 128 * 128 > 2147483647LL) {
@@ -1037,13 +1062,13 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         const bool split = v.has("split_k") && v.fields.at("split_k").kind == Value::Number ? true : v.boolean("split_k", true, &bad);
         const bool in_gemm = v.boolean("decode_in_gemm", false, &bad);
         if (bad) return ORX_ERR_BAD_VARIANT;
-        f->flags2 = (split && !half_step ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0);
+        f->flags2 = (split && !half_step ? 0 : kNoSplit) | (in_gemm ? kNoExpand : 0) | schedule_hint;
         f->workspace_need = projection_workspace;
     }
     f->geometry = projection_geometry;
     // a projection handle launches one of several kernels depending on the live rows (1024-thread
     // GEMV, 512-thread streaming and 256x256 kernels, 256-thread tiles): no single function's
-    // attributes describe it, so orx_query reports the device-wide limits
+    // attributes describe it: orx_query_rows reports the kernel a row count starts, orx_query the capacity's
     f->device_function = nullptr;
     return ORX_OK;
 }

@@ -71,6 +71,7 @@ struct orx_function {
     // shape / configuration
     int M = 0, N = 0, K = 0, E = 0, top_k = 0, H = 0, stride = 0, group = 0, tiles = 0, slots = 0;
     int block_m = 0, block_n = 0, packed_k = 0, algorithm = 0, flags = 0, flags2 = 0;
+    int tile_hint = 0;  // projections: row tile preferred while the live rows fit one such tile (0 = none)
     bool out_f32 = false;
     bool input_f16 = false;  // single-row projection that quantises its fp16 activations itself
     bool rotate_input = false;  // ... after the signed block-128 rotation (takes a Signs buffer)

@@ -490,20 +490,45 @@ def test_int8_weights_take_k_in_steps_of_64():
 def test_projections_take_the_reference_factories_schedule_names():
     """e8p_q4.projection(algorithm="tensor_core"|"dp4a"|"int4_direct", block_m=8.., split_k=1|2|4, ...) and
     int8_projection(block_m=16.., block_n, block_k, stages, ...) (e8p_q4.py:143-215, int8_projection.py:15-48) pick
-    among SM87 kernels; the same keyword set resolves here to the handle that picks by row count."""
-    plain = lib.Kernel("e8p_q4_projection", M=64, N=512, K=1024, dynamic_rows=True)
-    for extra in (dict(algorithm="tensor_core", block_m=8, block_n=64, block_k=128, stages=2),
-                  dict(algorithm="dp4a", block_m=4, block_n=8),
-                  dict(algorithm="int4_direct", block_m=8, block_n=128, packed_k=128, basis_nonzero=True, split_k=2),
-                  dict(algorithm="tensor_core", block_m=96, group_m=4, cache_scales=True, tail_m=16)):
-        variant = dict(M=64, N=512, K=1024, dynamic_rows=True)
-        variant.update(extra)
-        kern = lib.Kernel("e8p_q4_projection", **variant)
-        if extra.get("packed_k", 0) == 0:
-            for rows in (1, 8, 64):
-                assert kern.geometry(rows) == plain.geometry(rows), (extra, rows)
-    w8 = lib.Kernel("int8_projection", M=256, N=512, K=1024, block_m=16, block_n=64, block_k=64, stages=2)
-    assert w8.geometry() == lib.Kernel("int8_projection", M=256, N=512, K=1024).geometry()
+    among SM87 kernels; the same keyword set resolves here, and the schedule name and the row tile choose among this
+    library's kernels: dp4a keeps the dot-product (GEMV) family where it serves the rows, tensor_core keeps off it,
+    int4_direct and tiles of 1-8 rows leave the choice to the row count, and a tile of 16, 96 or 192 rows asks for the
+    MFMA tile that holds it (32, 128, 256) while the live rows fit one such tile."""
+    shape = dict(M=512, N=17408, K=5120, dynamic_rows=True)
+    plain = lib.Kernel("e8p_q4_projection", **shape)
+
+    def q4(**extra):
+        return lib.Kernel("e8p_q4_projection", **shape, **extra)
+
+    for extra in (dict(algorithm="int4_direct", block_m=8, block_n=128, basis_nonzero=True, split_k=2),
+                  dict(algorithm="int4_direct", block_m=4, group_m=4, cache_scales=True, tail_m=16)):
+        for rows in (1, 3, 8, 64, 100, 200, 512):
+            assert q4(**extra).geometry(rows) == plain.geometry(rows), (extra, rows)
+    gemv = lib.Kernel("e8p_q4_projection", **dict(shape, M=4), algorithm="gemv")
+    mma = q4(algorithm="tensor_core", block_m=8, block_n=64, block_k=128, stages=2)
+    dot = q4(algorithm="dp4a", block_m=4, block_n=8)
+    assert plain.geometry(1) == gemv.geometry(1) == dot.geometry(1) != mma.geometry(1)
+    assert mma.geometry(1) == lib.Kernel("e8p_q4_projection", **dict(shape, M=64), algorithm="stream").geometry(1)
+    for rows in (2, 3, 4):  # by row count these go to the batched-decode kernel; dp4a keeps the GEMV, tensor_core does not
+        assert dot.geometry(rows) == gemv.geometry(rows) != plain.geometry(rows) == mma.geometry(rows), rows
+    for rows in (5, 64, 300):
+        assert dot.geometry(rows) == plain.geometry(rows) == mma.geometry(rows), rows
+    for hint, tile, fits, beyond in ((16, 32, (5, 20, 32), (33, 200)), (96, 128, (20, 100, 128), (129, 400)),
+                                     (192, 256, (20, 200, 256), (257, 300))):
+        hinted, forced = q4(block_m=hint), q4(block_m=tile)
+        for rows in fits:
+            assert hinted.geometry(rows) == forced.geometry(rows), (hint, rows)
+        for rows in beyond:
+            assert hinted.geometry(rows) == plain.geometry(rows), (hint, rows)
+    assert q4(block_m=96).geometry(20) != plain.geometry(20) and q4(block_m=192).geometry(200) != plain.geometry(200)
+    w8_shape = dict(M=256, N=512, K=1024, dynamic_rows=True)
+    w8 = lib.Kernel("int8_projection", **w8_shape, block_m=16, block_n=64, block_k=64, stages=2)
+    assert w8.geometry(20) == lib.Kernel("int8_projection", **w8_shape, block_m=32).geometry(20)
+    assert w8.geometry(200) == lib.Kernel("int8_projection", **w8_shape).geometry(200)
+    # a K of a single step, or one that ends in half a step, has no 256-row tile: 192 then names the 128-row tile
+    short = dict(M=256, N=512, K=192, dynamic_rows=True)
+    assert lib.Kernel("int8_projection", **short, block_m=192).geometry(100) == \
+        lib.Kernel("int8_projection", **short, block_m=128).geometry(100)
 
 
 def test_two_stage_coefficients_other_than_4_1_are_refused():

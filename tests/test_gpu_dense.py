@@ -707,6 +707,29 @@ def test_w8_stream_matches_oracle(m, n, k):
     assert (got[m] == 99).all()
 
 
+@pytest.mark.parametrize("hints", [dict(algorithm="dp4a", block_m=4, block_n=8), dict(algorithm="tensor_core", block_m=8),
+                                   dict(algorithm="int4_direct", block_m=16), dict(algorithm="tensor_core", block_m=96),
+                                   dict(block_m=192)], ids=lambda h: "-".join(str(v) for v in h.values()))
+def test_reference_schedule_names_and_row_tiles_give_the_same_outputs(hints):
+    """The reference's schedule names and row tiles (e8p_q4.py:143-215, int8_projection.py:15-48) choose among this
+    library's kernels; whichever kernel a launch then runs, the output is the oracle's to the bit."""
+    rng = np.random.default_rng(orc.SEED + 77)
+    n, k, capacity = 449, 1024, 300
+    a_q, a_s, packed, scales = q4_case(rng, capacity, n, k)
+    w = orc.q4_integers(packed, TABLE)
+    want = orc.project(a_q, a_s, w, scales)
+    x8 = rng.integers(-128, 128, (capacity, k), dtype=np.int8)
+    w8 = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    want8 = orc.project(x8, a_s, w8, scales)
+    for rows in (1, 2, 4, 5, 20, 33, 100, 129, 200, 300):
+        got = gu.q4_project(gu.dev(a_q[:rows]), gu.dev(a_s[:rows]), gu.dev(packed), gu.dev(scales), dynamic=True,
+                            capacity=capacity, **hints)
+        np.testing.assert_array_equal(gu.host(got), want[:rows], err_msg=f"q4 rows {rows}")
+        got = gu.w8_project(gu.dev(x8[:rows]), gu.dev(a_s[:rows]), gu.dev(w8), gu.dev(scales), dynamic=True,
+                            capacity=capacity, **hints)
+        np.testing.assert_array_equal(gu.host(got), want8[:rows], err_msg=f"w8 rows {rows}")
+
+
 @pytest.mark.parametrize("block_m", [32, 64, 128, 256])
 def test_q4_mfma_tiles_and_accumulators(block_m):
     rng = np.random.default_rng(orc.SEED + block_m)

@@ -332,6 +332,11 @@ def check_layer(c, layer, bm):
                          c["top_k"], bm, signs=None if layer.signs is None else gu.host(layer.signs))["out"].astype(np.float32)
     rel_l2 = np.linalg.norm(got - full) / np.linalg.norm(full)
     assert rel_l2 < 0.003  # flash_next_quantized.py:117-135 accepts the expert FFN at this bar
+    # element by element against the whole oracle chain, at the output tolerance (1e-3 relative + 1e-2 absolute): the
+    # only arithmetic that is not bit-exact in between is exp() inside SwiGLU, which moves a few A8 codes by one step
+    error = np.abs(got - full)
+    beyond = error > 1e-2 + 1e-3 * np.abs(full)
+    assert not beyond.any(), (int(beyond.sum()), beyond.size, float(error.max()))
 
 
 def test_moe_layer_small_end_to_end():
