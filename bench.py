@@ -251,7 +251,7 @@ def main():
                                          "frac_hbm": round(b0 / t0_plain / 1e9 / HBM_PEAK_GBS, 4), "bytes": b0}
         # config 1 sweep
         sweep = {}
-        for rows in (1, 8, 32, 128, 512):
+        for rows in (1, 8, 32, 128, 512, 1024):
             case = Q4Case(workloads.config1(rows), copies)
             t = timed_graph(lambda i, s: case.project(i, s), short_graph)
             b = workloads.algorithmic_bytes_q4(rows, case.n, case.k)

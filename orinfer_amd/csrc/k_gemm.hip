@@ -678,6 +678,14 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
     return hip_check(hipGetLastError(), "launch routed projection (general decode)");
 }
 
+// Row tile asked for at `rows` live rows: a block_m this library has a tile for (32, 64, 128, 256) holds at every row
+// count; a reference-only tile (16, 96, 192) was chosen for launches of about that many rows, so it names the tile
+// that holds it (32, 128, 256) while the live rows fit one such tile, and beyond that the row count decides.
+int tile_for(const orx_function& f, int rows) {
+    if (f.tiles) return f.tiles;
+    return f.tile_hint && rows <= f.tile_hint ? f.tile_hint : 0;
+}
+
 // Channel runs per CU over the whole K (k_wide.hip): two-stage codes, `algorithm=wide` by name, and by
 // `auto` at 65..128 rows (33..64 rows of large matrices) while K is short enough.  Its time is 10 us + 0.4..0.55 us per K step of 128 whatever
 // N is (up to 96 channels per CU), where the split 128 x 128 tiles pay for N K: measured at 65-128 rows,
@@ -687,14 +695,6 @@ int launch_mfma_general(int bm, const GemmParams& p, const Geometry& g, hipStrea
 // 70-83 against 72-74 (N = 28672); 9728 and up: slower (N = 5120, K = 17408: 56-69 against 41).  Below 65
 // rows the batched-decode kernels are as fast or faster except at N = 17408 (30 against 31-34 us), above 128
 // rows a second pass doubles the time (58-62 against 57 us at 160-256 rows).
-// Row tile asked for at `rows` live rows: a block_m this library has a tile for (32, 64, 128, 256) holds at every row
-// count; a reference-only tile (16, 96, 192) was chosen for launches of about that many rows, so it names the tile
-// that holds it (32, 128, 256) while the live rows fit one such tile, and beyond that the row count decides.
-int tile_for(const orx_function& f, int rows) {
-    if (f.tiles) return f.tiles;
-    return f.tile_hint && rows <= f.tile_hint ? f.tile_hint : 0;
-}
-
 bool use_wide(const orx_function& f, int rows) {
     if (f.flags != kQ4 || !dense_wide_eligible(f.N, f.K, f.packed_k)) return false;
     if (f.algorithm == kWide) return true;
@@ -808,13 +808,40 @@ int split_groups_for(const orx_function& f, int rows) {
     return (int)std::max<int64_t>(1, std::min<int64_t>(split_groups(), units / 8));
 }
 
+// A few 256 x 256 tiles more than there are CUs would be a second round with most of the chip idle (1024 rows of
+// N = 17408: 272 tiles; int8, K = 5120: 118 us, against 75 us for the 256 tiles of the first 16384 channels).  The
+// persistent launch then takes the column tiles that fill one round, and the channels behind them go to the
+// 128 x 128 tiles with their K steps split over all CUs (26 us for those 1024 channels: 96 us together).  Only
+// where the second round would hold at most an eighth of the CUs: with more tiles left, or more rounds in front,
+// the half-empty round runs at a higher clock and the split launch gains nothing (2048 rows: 175 against 180 us;
+// 8192 rows of N = 5120, K = 17408: 669 against 657 us).  Returns the channels of the persistent launch (N: all).
+int big_main_channels(const orx_function& f, int rows) {
+    if (!f.takes_workspace || (f.flags2 & kNoSplit) || f.algorithm != kAuto || tile_for(f, rows) != 0) return f.N;
+    const int cus = device_compute_units();
+    const int row_tiles = (int)ceil_div((uint32_t)rows, 256u), column_tiles = (int)ceil_div((uint32_t)f.N, 256u);
+    const int tiles = row_tiles * column_tiles;
+    if (tiles <= cus || tiles > cus + cus / 8 || row_tiles > cus) return f.N;
+    const int main_columns = cus / row_tiles;
+    return main_columns * 256;
+}
+int split_groups_for_channels(int channels, int rows, int k) {
+    const int64_t units = (int64_t)ceil_div((uint32_t)channels, 128u) * ceil_div((uint32_t)rows, 128u) * (k / kBK);
+    return (int)std::max<int64_t>(1, std::min<int64_t>(split_groups(), units / 8));
+}
+uint64_t big_rest_workspace(const orx_function& f, int rows) {
+    const int main_channels = big_main_channels(f, rows);
+    if (main_channels >= f.N) return 0;
+    return (uint64_t)split_groups_for_channels(f.N - main_channels, rows, f.K) * 2 * kSplitSlotInts * sizeof(int);
+}
+
 // Workspace bytes of a launch: the partial slots of a split launch, or the decoded weights of a
-// two-stage launch on the 256-row tiles.
+// two-stage launch on the 256-row tiles (and behind them the partial slots of the channels that the
+// persistent launch leaves to the split tiles).
 uint64_t projection_workspace(const orx_function& f, int rows) {
     if (use_wide(f, rows)) return 0;
     if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows)) return 0;
-    if (use_expand(f, rows)) return (uint64_t)f.N * f.K;
-    if (use_big(f, rows)) return 0;
+    if (use_expand(f, rows)) return (uint64_t)f.N * f.K + big_rest_workspace(f, rows);
+    if (use_big(f, rows)) return f.flags == kW8 ? big_rest_workspace(f, rows) : 0;
     if (use_split(f, rows)) return (uint64_t)split_groups_for(f, rows) * 2 * kSplitSlotInts * sizeof(int);
     return 0;
 }
@@ -844,7 +871,8 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (use_big(f, rows)) {
-        gemm_big_geometry(rows, f.N, f.flags == kQ4 && !use_expand(f, rows), g);
+        const bool decode_in_loop = f.flags == kQ4 && !use_expand(f, rows);
+        gemm_big_geometry(rows, decode_in_loop ? f.N : big_main_channels(f, rows), decode_in_loop, g);
         return ORX_OK;
     }
     if (use_split(f, rows)) {
@@ -859,6 +887,24 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
     g->block[0] = 256;
     g->shared = 0;
     return ORX_OK;
+}
+
+// int8 weights on the 256 x 256 tiles: the persistent launch, and the split 128 x 128 tiles for the channels it
+// leaves (big_main_channels).  `partials`: the workspace bytes behind whatever else the launch keeps there.
+int int8_big_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const GemmParams& p,
+                    const void* weights, void* partials) {
+    const int main_channels = big_main_channels(f, rows);
+    int code = gemm_big_launch(false, p.a, weights, nullptr, p.ws, p.as, p.out, rows, main_channels, f.K, f.stride, 0,
+                               f.out_f32, g, stream);
+    if (code != ORX_OK || main_channels >= f.N) return code;
+    GemmParams rest = p;
+    rest.book = nullptr, rest.packed_k = 0;
+    rest.w = static_cast<const int8_t*>(weights) + (size_t)main_channels * f.K;
+    rest.ws = p.ws + main_channels;
+    rest.out = static_cast<char*>(p.out) + (size_t)main_channels * (f.out_f32 ? 4 : 2);
+    rest.n = f.N - main_channels;
+    rest.partials = static_cast<int*>(partials);
+    return launch_split<kW8>(rest, split_groups_for_channels(rest.n, rows, f.K), stream);
 }
 
 // E8P-Q4: A, AS, Book, Out, S, W[, m]   (e8p_q4.py:248-255 in generated-ABI order)
@@ -899,8 +945,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     if (use_expand(f, rows)) {
         const int code = q4_expand_launch(p.w, p.book, workspace, f.N, f.K, f.packed_k, stream);
         if (code != ORX_OK) return code;
-        return gemm_big_launch(false, p.a, workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0,
-                               f.out_f32, g, stream);
+        return int8_big_launch(f, rows, g, stream, p, workspace, static_cast<char*>(workspace) + (size_t)f.N * f.K);
     }
     if (use_big(f, rows))
         return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
@@ -934,9 +979,7 @@ int w8_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         }
         return ORX_OK;
     }
-    if (use_big(f, rows))
-        return gemm_big_launch(false, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
-                               stream);
+    if (use_big(f, rows)) return int8_big_launch(f, rows, g, stream, p, p.w, workspace);
     if (use_split(f, rows)) {
         p.partials = static_cast<int*>(workspace);
         return launch_split<kW8>(p, split_groups_for(f, rows), stream);

@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int row_in_wave = lane / LPR;
     const int row_bytes = CODEC == kQ4 ? k / 2 : k / 4;
     const int chunks = row_bytes / 16;
-    const int steps = chunks / LPR;              // the host guarantees chunks % LPR == 0
+    const int steps = HOLD ? D : chunks / LPR;   // the host guarantees chunks % LPR == 0 (HOLD: and a quotient of D)
     const int padded = (steps + D - 1) / D * D;  // ring refills happen in whole groups of D
     const int tasks = (n + kRows - 1) / kRows;
     const int task_stride = gridDim.x * (kBankedThreads / 64);

@@ -853,6 +853,52 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
+@pytest.mark.parametrize("codec", ["w8", "q4"])
+def test_a_few_tiles_more_than_cus_go_to_split_tiles(codec):
+    """A handful of 256 x 256 tiles beyond one round of the persistent kernel: it takes the column tiles that fill the
+    round and the channels behind them run as split 128 x 128 tiles from the same Workspace (behind the decoded weights
+    of two-stage codes).  Ragged last tile, output stride, sentinels; rows checked in every row tile."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rows, k = 1000, 256
+    row_tiles = -(-rows // 256)
+    main_columns = cus // row_tiles
+    n = main_columns * 256 + 2 * 256 + 70          # two whole column tiles and a ragged one behind the round
+    assert cus < row_tiles * -(-n // 256) <= cus + cus // 8
+    rng = np.random.default_rng(orc.SEED + 91)
+    scales = rng.uniform(0.005, 0.02, n).astype(np.float16)
+    a_q = rng.integers(-127, 128, (rows, k), dtype=np.int8)
+    a_s = rng.uniform(0.005, 0.02, rows).astype(np.float16)
+    out = torch.full((rows + 1, n + 5), 7.0, dtype=torch.float16, device=gu.DEV)
+    variant = dict(M=rows, N=n, K=k, output_stride=n + 5, workspace=True)
+    if codec == "q4":
+        packed = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+        weights = orc.q4_integers(packed, TABLE)
+        kern = gu.lib.Kernel("e8p_q4_projection", **variant)
+        decoded = n * k
+        args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), Out=out, S=gu.dev(scales), W=gu.dev(packed))
+    else:
+        weights = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        kern = gu.lib.Kernel("int8_projection", **variant)
+        decoded = 0
+        args = dict(A=gu.dev(a_q), Output=out, TokenScale=gu.dev(a_s), Weight=gu.dev(weights), WeightScale=gu.dev(scales))
+    assert kern.geometry(rows)[0][0] == row_tiles * main_columns     # the persistent launch: one round
+    assert kern.workspace_bytes(rows) > decoded                        # partial tiles of the split launch behind it
+    assert gu.lib.Kernel(kern.symbol, **dict(variant, split_k=False)).workspace_bytes(rows) == decoded
+    kern(**args)
+    got = gu.host(out)
+    sample = np.unique(np.concatenate([np.arange(0, rows, 37), [127, 128, 255, 256, 511, 512, 767, 768, rows - 1]]))
+    want = orc.project(a_q[sample], a_s[sample], weights, scales)
+    np.testing.assert_array_equal(got[sample, :n], want)
+    assert (got[rows:] == 7).all() and (got[:rows, n:] == 7).all()
+    # every row and channel was written, and column sums agree with the oracle's on the sampled rows' complement check
+    assert not (got[:rows, :n] == 7).all(axis=0).any()
+    # the whole-tile launch of the same handle family gives the same bits
+    whole = torch.full_like(out, 7.0)
+    other = gu.lib.Kernel(kern.symbol, **dict(variant, split_k=False))
+    other(**dict(args, **({"Out": whole} if codec == "q4" else {"Output": whole})))
+    np.testing.assert_array_equal(gu.host(whole), got)
+
+
 @pytest.mark.parametrize("packed_k", [0, 64, 128])
 @pytest.mark.parametrize("decode_in_gemm", [False, True], ids=["decode-once", "decode-in-gemm"])
 def test_q4_many_rows_both_decode_paths(packed_k, decode_in_gemm):
@@ -1105,7 +1151,10 @@ def test_resolving_handles_takes_no_device_memory():
                for i in range(1000)]
     handles += [gu.lib.Kernel("int8_swiglu", M=512 + i, N=1024, K=2048, dynamic_rows=True) for i in range(100)]
     assert torch.cuda.mem_get_info()[0] == free_before
-    assert handles[0].workspace_bytes(0) == 17408 * 5120
+    # the decoded int8 weights, and at 1024 rows (272 tiles of 256 for 256 CUs) the partial tiles of the channels that
+    # the persistent launch leaves to the split tiles behind them
+    assert handles[0].workspace_bytes(4096) == 17408 * 5120
+    assert 17408 * 5120 <= handles[0].workspace_bytes(0) <= 17408 * 5120 + 512 * 2 * 128 * 128 * 4
 
 
 def test_two_handles_on_two_streams_with_their_own_workspaces_stay_bit_exact():
