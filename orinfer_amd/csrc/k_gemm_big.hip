@@ -586,8 +586,9 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                v4i& sum = acc[4 * (phase & 1) + i][j];
-                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights[j], tokens[i], sum, 0, 0, 0);
+                const int jj = (i & 1) ? 3 - j : j;  // boustrophedon: one operand changes between consecutive multiplies
+                v4i& sum = acc[4 * (phase & 1) + i][jj];
+                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(weights[jj], tokens[i], sum, 0, 0, 0);
                 const int index = i * 4 + j;
                 if ((index & 1) == 1 && index / 2 < count) {
                     __builtin_amdgcn_sched_barrier(0);
