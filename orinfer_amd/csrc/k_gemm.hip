@@ -61,12 +61,14 @@ int stream_grouped_launch(const int8_t* a, const void* w, const uint32_t* book, 
                           const int* tile_count, int n, int k, int tiles, int block_m, int packed_k,
                           hipStream_t stream);
 // from k_gemm_big.hip
-void gemm_big_geometry(int rows, int n, bool q4, Geometry* g);
+void gemm_big_geometry(int rows, int n, Geometry* g);
 int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int n, int k, int packed_k,
                      hipStream_t stream);
-int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                    void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g,
-                    hipStream_t stream);
+void gemm_tall_geometry(int rows, int n, Geometry* g);
+int gemm_tall_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out,
+                     int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g, hipStream_t stream);
+int gemm_big_launch(const int8_t* a, const void* w, const __half* ws, const __half* as, void* out, int rows, int n,
+                    int k, int stride, bool out_f32, const Geometry& g, hipStream_t stream);
 
 namespace {
 
@@ -77,7 +79,7 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 enum Codec { kQ4 = 0, kQ2 = 1, kW8 = 2, kS4 = 3 };  // kS4: row-scaled scalar Q4 nibbles (q4_projection.py)
-enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4, kWide = 5 };
+enum Algorithm { kAuto = 0, kGemv = 1, kMfma = 2, kStream = 3, kResident = 4, kWide = 5, kTall = 6 };
 // orx_function::flags2 of a projection.  kPreferGemv / kNoGemv: the reference's schedule names as hints among the
 // library's own kernels (algorithm=dp4a: its dot-product schedule for few rows; tensor_core: its matrix-unit one).
 enum Flags2 { kNoSplit = 1, kNoExpand = 2, kPreferGemv = 4, kNoGemv = 8 };
@@ -706,9 +708,14 @@ bool use_wide(const orx_function& f, int rows) {
     return rows >= 33 && rows <= 64 && (int64_t)f.N * f.K >= ((int64_t)1 << 26) && f.N <= 96 * device_compute_units();
 }
 
+// 512 x 128 tiles with the decode in the K loop (k_gemm_big.hip): `algorithm=tall` by name
+bool use_tall(const orx_function& f, int rows) {
+    return f.flags == kQ4 && f.algorithm == kTall;
+}
+
 bool use_resident(const orx_function& f, int rows);
 bool use_gemv(const orx_function& f, int rows) {
-    if (use_wide(f, rows)) return false;
+    if (use_wide(f, rows) || use_tall(f, rows)) return false;
     if (f.algorithm == kGemv) return true;
     if (f.algorithm != kAuto) return false;
     if (f.flags2 & kNoGemv) return false;  // the matrix-unit kernels were asked for: streaming / batched-decode from row 1
@@ -838,7 +845,7 @@ uint64_t big_rest_workspace(const orx_function& f, int rows) {
 // two-stage launch on the 256-row tiles (and behind them the partial slots of the channels that the
 // persistent launch leaves to the split tiles).
 uint64_t projection_workspace(const orx_function& f, int rows) {
-    if (use_wide(f, rows)) return 0;
+    if (use_wide(f, rows) || use_tall(f, rows)) return 0;
     if (use_gemv(f, rows) || use_resident(f, rows) || use_stream(f, rows)) return 0;
     if (use_expand(f, rows)) return (uint64_t)f.N * f.K + big_rest_workspace(f, rows);
     if (use_big(f, rows)) return f.flags == kW8 ? big_rest_workspace(f, rows) : 0;
@@ -861,6 +868,10 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         dense_wide_geometry(f.N, g);
         return ORX_OK;
     }
+    if (use_tall(f, rows)) {
+        gemm_tall_geometry(rows, f.N, g);
+        return ORX_OK;
+    }
     if (use_gemv(f, rows)) return gemv_geometry_for(f, rows, g);
     if (use_resident(f, rows)) {
         dense_resident_geometry(rows, f.N, f.K, f.packed_k, g);
@@ -871,8 +882,10 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (use_big(f, rows)) {
-        const bool decode_in_loop = f.flags == kQ4 && !use_expand(f, rows);
-        gemm_big_geometry(rows, decode_in_loop ? f.N : big_main_channels(f, rows), decode_in_loop, g);
+        if (f.flags == kQ4 && !use_expand(f, rows))  // decode in the K loop: the 512 x 128 tiles
+            gemm_tall_geometry(rows, f.N, g);
+        else
+            gemm_big_geometry(rows, big_main_channels(f, rows), g);
         return ORX_OK;
     }
     if (use_split(f, rows)) {
@@ -894,8 +907,7 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
 int int8_big_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t stream, const GemmParams& p,
                     const void* weights, void* partials) {
     const int main_channels = big_main_channels(f, rows);
-    int code = gemm_big_launch(false, p.a, weights, nullptr, p.ws, p.as, p.out, rows, main_channels, f.K, f.stride, 0,
-                               f.out_f32, g, stream);
+    int code = gemm_big_launch(p.a, weights, p.ws, p.as, p.out, rows, main_channels, f.K, f.stride, f.out_f32, g, stream);
     if (code != ORX_OK || main_channels >= f.N) return code;
     GemmParams rest = p;
     rest.book = nullptr, rest.packed_k = 0;
@@ -921,6 +933,8 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
     p.n = f.N, p.k = f.K, p.stride = f.stride, p.m = rows, p.packed_k = f.packed_k, p.out_f32 = f.out_f32;
     if (use_wide(f, rows))
         return dense_wide_launch(p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32, g, stream);
+    if (use_tall(f, rows))
+        return gemm_tall_launch(p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32, g, stream);
     if (use_gemv(f, rows)) return gemv_launch(f, rows, g, stream, p.a, p.w, p.book, p.ws, p.as, p.out, signs);
     if (use_resident(f, rows)) {
         for (int first = 0; first < rows; first += 32) {
@@ -948,8 +962,7 @@ int q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_t st
         return int8_big_launch(f, rows, g, stream, p, workspace, static_cast<char*>(workspace) + (size_t)f.N * f.K);
     }
     if (use_big(f, rows))
-        return gemm_big_launch(true, p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k,
-                               f.out_f32, g, stream);
+        return gemm_tall_launch(p.a, p.w, p.book, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.packed_k, f.out_f32, g, stream);
     if (use_split(f, rows)) {
         p.partials = static_cast<int*>(workspace);
         return launch_split<kQ4>(p, split_groups_for(f, rows), stream);
@@ -1049,10 +1062,15 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
                    : algorithm == "stream"   ? kStream
                    : algorithm == "resident" ? kResident
                    : algorithm == "wide"     ? kWide
+                   : algorithm == "tall"     ? kTall
                    : algorithm == "auto"     ? kAuto
                                              : -1;
     if (f->algorithm < 0) {
-        set_error("%s: algorithm must be auto, gemv, stream, resident, wide or mfma", name);
+        set_error("%s: algorithm must be auto, gemv, stream, resident, wide, tall or mfma", name);
+        return ORX_ERR_BAD_VARIANT;
+    }
+    if (f->algorithm == kTall && (codec != kQ4 || f->K % 128 != 0 || f->K < 256)) {
+        set_error("%s: algorithm=tall serves two-stage codes with K a multiple of 128, at least 256", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->algorithm == kWide && (codec != kQ4 || !dense_wide_eligible(f->N, f->K, f->packed_k))) {
@@ -1215,7 +1233,7 @@ int row_q4_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (row_q4_expands(f, rows)) {
-        gemm_big_geometry(rows, f.N, false, g);
+        gemm_big_geometry(rows, f.N, g);
         return ORX_OK;
     }
     if (row_q4_splits(f, rows)) {
@@ -1251,8 +1269,7 @@ int row_q4_launch(const orx_function& f, int rows, const Geometry& g, hipStream_
         void* workspace = pointer_arg<void>(args, f.workspace_arg);
         const int code = row_q4_unpack(p.w, workspace, f.N, f.K, p.magnitudes_low, p.magnitudes_high, stream);
         if (code != ORX_OK) return code;
-        return gemm_big_launch(false, p.a, workspace, nullptr, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, 0, f.out_f32, g,
-                               stream);
+        return gemm_big_launch(p.a, workspace, p.ws, p.as, p.out, rows, f.N, f.K, f.stride, f.out_f32, g, stream);
     }
     if (row_q4_splits(f, rows)) {
         p.partials = pointer_arg<int>(args, f.workspace_arg);

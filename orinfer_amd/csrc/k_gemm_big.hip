@@ -1,22 +1,17 @@
-// Large-M int8 MFMA projections (prefill): 256 x 256 output tile per workgroup, K step 128.
+// Many-row int8 MFMA projections (prefill).
 //
 // Reference counterparts: the Tensor Core schedules of kernels/cuda/model/integer_core.py:162-272
 // at block_m = 128/256 with grouped tile order (:31-39) for W8A8 (int8_projection.py:15-62) and
 // E8P-Q4 (e8p_q4.py:143-264).  Arithmetic is identical: exact int32 accumulation over full K,
 // then (float(acc)*ws)*as.
 //
-// MI355X design.  Eight wave64 (2 per SIMD) share one 256x256 tile; each wave owns 128x64 of it
-// as 4x2 blocks of v_mfma_i32_32x32x32_i8 (128 accumulator registers).  Both operand tiles are
-// double buffered in LDS (2 x 64 KiB of the 160 KiB).  int8 operands that already exist in HBM
-// (activations, W8 weights) go HBM -> LDS directly with global_load_lds_dwordx4, without touching
-// VGPRs: each wave instruction moves 8 rows x 128 bytes, so global access is whole 128-byte lines,
-// and the 16-byte chunk a lane fetches is XOR-swizzled with its row so that the later
-// ds_read_b128 fragment reads of sixteen consecutive rows fall in sixteen different bank groups.
-// E8P-Q4 weights are decoded from codes in registers (two 8-byte LDS table reads and XORs per
-// code, e8p_device.h) and stored to the same swizzled layout.  Loads for K step t+1 are issued
-// right after the barrier that publishes step t, so they fly under the 32 MFMAs of step t.
-// Workgroup ids are remapped so that the workgroups resident on one XCD (ids congruent mod 8)
-// work on neighbouring tiles and share operand panels in that XCD's L2.
+// Two kernels.  int8 weights (W8A8, and two-stage weights that q4_expand_kernel has decoded once into the
+// caller's scratch): gemm_big_persistent_kernel, one workgroup per CU walking 256 x 256 tiles.  Two-stage codes
+// without scratch: gemm_q4_tall_kernel, 512 x 128 tiles with the decode in the K loop.  In both, eight wave64
+// (2 per SIMD) share a tile, each owning 128 token rows x 64 channels as 8 x 4 blocks of v_mfma_i32_16x16x64_i8
+// (128 accumulator registers); int8 operands that already exist in HBM go HBM -> LDS directly with
+// global_load_lds_dwordx4, without touching VGPRs, and the 16-byte chunk a lane fetches is XOR-swizzled with its
+// row so that the later ds_read_b128 fragment reads of sixteen consecutive rows fall in different bank groups.
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
@@ -24,23 +19,15 @@
 #include "e8p_device.h"
 #include "orx_internal.h"
 
-#ifndef ORX_BIG_TM
-#define ORX_BIG_TM 4
-#define ORX_BIG_TN 2
-#endif
-
 namespace orx {
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned int v4u __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kTile = 256;     // output tile edge
 constexpr int kStep = 128;     // K bytes per step
 constexpr int kTileBytes = kTile * kStep;  // 32 KiB per operand per stage
-constexpr int kImagePitch = kTile + 8;     // halves per row of the fp16 output image (bank skew)
-constexpr int kEpilogueTile = kTile * kImagePitch * 2;  // bytes of the output image in LDS
 
 struct BigParams {
     const int8_t* a;
@@ -66,13 +53,6 @@ __device__ __forceinline__ void direct_load_16(const void* global, void* lds_wav
 // The compiler does not count direct-to-LDS loads as pending at a barrier (they have no register
 // destination), so every barrier that publishes them is preceded by this explicit wait.
 __device__ __forceinline__ void wait_direct_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-// Same, but lets the N youngest vector-memory requests stay in flight (requests retire in order):
-// used when N ordinary loads (weight codes for a later step) were issued after the direct loads.
-template <int N>
-__device__ __forceinline__ void wait_direct_loads_except() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
 // 16-byte LDS read whose wait is placed by hand.  The compiler waits for EVERY outstanding LDS read before the first
 // multiply that follows a batch of reads (s_waitcnt lgkmcnt(0)), also when those multiplies use fragments that were
 // requested a whole sub-step earlier, which undoes the software pipeline; a read issued from an asm statement is
@@ -105,318 +85,6 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int* t
     const int within = logical % group_size;
     *tm = first + within % rows_in_group;
     *tn = within / rows_in_group;
-}
-
-// TM x TN blocks of 32x32 per wave: <4,2> = eight waves of 128x64 (two per SIMD),
-// <4,4> = four waves of 128x128 (one per SIMD, accumulators spill over into AGPRs).
-template <bool Q4, int TM, int TN>
-__global__ __launch_bounds__((8 / TM) * (8 / TN) * 64) void gemm_big_kernel(BigParams p) {
-    constexpr int WAVES_N = 8 / TN;
-    constexpr int WAVES = (8 / TM) * WAVES_N;
-    constexpr int kThreads = WAVES * 64;
-    constexpr int BLOCKS_PER_WAVE = 32 / WAVES;  // 1 KiB blocks of each operand tile per wave
-    constexpr int CODE_CHUNKS = 1024 / kThreads; // 16-byte code chunks per thread per K step
-    extern __shared__ __align__(16) int8_t lds[];  // [2 stages][A 32 KiB | W 32 KiB] (+ Q4 tables)
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-
-    int tile_m, tile_n;
-    tile_of(blockIdx.x, p.tiles_m, p.tiles_n, &tile_m, &tile_n);
-    const int row0 = tile_m * kTile, col0 = tile_n * kTile;
-    const int rows_here = min(kTile, p.m - row0);
-    const int cols_here = min(kTile, p.n - col0);
-
-    // Scales of this tile, one or two per thread, fetched now as raw bits so that the epilogue
-    // does not pay a memory round trip: entries 0..255 token scales, 256..511 weight scales.
-    constexpr int SCALES_PER_THREAD = 2 * kTile / kThreads;
-    unsigned short scale_bits[SCALES_PER_THREAD];
-#pragma unroll
-    for (int e = 0; e < SCALES_PER_THREAD; ++e) {
-        const int i = tid + e * kThreads;
-        scale_bits[e] = i < kTile ? reinterpret_cast<const unsigned short*>(p.as)[row0 + min(i, rows_here - 1)]
-                                  : reinterpret_cast<const unsigned short*>(p.ws)[col0 + min(i - kTile, cols_here - 1)];
-    }
-
-    Q4ByteTables* tables = reinterpret_cast<Q4ByteTables*>(lds + 4 * kTileBytes);
-    if (Q4) build_tables(*tables, p.book, tid, kThreads);
-
-    // ---- global -> LDS: one wave instruction = 8 rows x 128 bytes (1 KiB block) ----
-    // wave w owns BLOCKS_PER_WAVE consecutive blocks of each operand tile (32 blocks of 8 rows)
-    const int load_r8 = lane >> 3, load_slot = lane & 7;
-    auto issue_direct = [&](const int8_t* base, int limit, int origin, int kt, int8_t* stage) {
-#pragma unroll
-        for (int b = 0; b < BLOCKS_PER_WAVE; ++b) {
-            const int block = wave * BLOCKS_PER_WAVE + b;
-            const int row = block * 8 + load_r8;
-            const int chunk = load_slot ^ swizzle(row);
-            const int source_row = origin + min(row, limit - 1);
-            direct_load_16(base + (int64_t)source_row * p.k + kt * kStep + chunk * 16, stage + block * 1024);
-        }
-    };
-    // Q4: one K step of the weight tile is 256 rows x 64 bytes of codes = 1024 chunks of 16 bytes
-    // (4 codes = 32 weights each): CODE_CHUNKS chunks per thread.
-    // Two register sets so that the codes of step t+1 can be in flight while step t is decoded.
-    v4u code_regs[2][CODE_CHUNKS];  // native vectors: an array of HIP's uint4 struct would live in scratch memory
-    auto load_codes = [&](int kt, int set) {
-#pragma unroll
-        for (int i = 0; i < CODE_CHUNKS; ++i) {
-            const int c = tid + kThreads * i;      // chunk id: row = c / 4, quarter = c % 4
-            const int row = min(c >> 2, cols_here - 1), q = c & 3;
-            int64_t byte;
-            if (p.packed_k != 0)
-                byte = q4_k_major_chunk(p.packed_k, p.n, col0 + row, kt, q);
-            else
-                byte = ((int64_t)(col0 + row) * (p.k / kStep) + kt) * 64 + q * 16;
-            code_regs[set][i] = *reinterpret_cast<const v4u*>(reinterpret_cast<const int8_t*>(p.w) + byte);
-        }
-    };
-    // Decode the codes of one K step (4 codes -> 32 weights -> two 16-byte LDS stores per chunk).
-    auto decode_step = [&](int8_t* stage, int set) {
-#pragma unroll
-        for (int i = 0; i < CODE_CHUNKS; ++i) {
-            const int c = tid + kThreads * i;
-            const int row = c >> 2, q = c & 3;
-            const v4u codes = code_regs[set][i];
-            const uint2 d0 = decode_q4(*tables, codes.x), d1 = decode_q4(*tables, codes.y);
-            const uint2 d2 = decode_q4(*tables, codes.z), d3 = decode_q4(*tables, codes.w);
-            int8_t* row_base = stage + row * kStep;
-            const int s = swizzle(row);
-            *reinterpret_cast<uint4*>(row_base + (((2 * q) ^ s) * 16)) = make_uint4(d0.x, d0.y, d1.x, d1.y);
-            *reinterpret_cast<uint4*>(row_base + (((2 * q + 1) ^ s) * 16)) = make_uint4(d2.x, d2.y, d3.x, d3.y);
-        }
-    };
-
-    // ---- fragment addressing ----
-    const int frag_row = lane & 31, frag_half = lane >> 5;
-    const int swz = swizzle(frag_row);  // identical for every 32-row block
-    int frag_offset[4];                 // byte offset inside a row for K sub-step ks
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) frag_offset[ks] = ((2 * ks + frag_half) ^ swz) * 16;
-    const int a_lane = (wave_m * TM * 32 + frag_row) * kStep;
-    const int w_lane = (wave_n * TN * 32 + frag_row) * kStep;
-
-    v16i acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    const int k_tiles = p.k / kStep;
-    auto stage_a = [&](int stage) { return lds + stage * 2 * kTileBytes; };
-    auto stage_w = [&](int stage) { return lds + kTileBytes + stage * 2 * kTileBytes; };
-
-    // Software pipeline over K steps (two LDS stages, two fragment register slots):
-    //   prologue   steps 0 and 1 requested, step 0 published, its first fragments read
-    //   step kt    sub-steps 0..2: read fragments ks+1, issue MFMAs ks
-    //              barrier: step kt+1 is complete in LDS and nobody reads stage `cur` any more
-    //              read fragments 0 of step kt+1, issue MFMAs of sub-step 3 (their operands are
-    //              already in registers), request step kt+2 into stage `cur`
-    // so the matrix pipe always holds queued work while waves meet at the barrier.
-    const int8_t* w8 = reinterpret_cast<const int8_t*>(p.w);
-    issue_direct(p.a, rows_here, row0, 0, stage_a(0));
-    if (!Q4) issue_direct(w8, cols_here, col0, 0, stage_w(0));
-    if (k_tiles > 1) {
-        issue_direct(p.a, rows_here, row0, 1, stage_a(1));
-        if (!Q4) issue_direct(w8, cols_here, col0, 1, stage_w(1));
-    }
-    if (Q4) {
-        load_codes(0, 0);
-        if (k_tiles > 1) load_codes(1, 1);
-        __syncthreads();  // tables
-        decode_step(stage_w(0), 0);
-        if (k_tiles > 2) load_codes(2, 0);
-        if (k_tiles > 1) decode_step(stage_w(1), 1);
-        if (k_tiles > 3) load_codes(3, 1);
-    }
-    wait_direct_loads();
-    __syncthreads();
-
-    v4i fa[2][TM], fb[2][TN];
-    auto read_fragments = [&](int stage, int ks, int slot) {
-        const int8_t* la = stage_a(stage) + a_lane;
-        const int8_t* lw = stage_w(stage) + w_lane;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const v4i*>(la + i * 32 * kStep + frag_offset[ks]);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) fb[slot][j] = *reinterpret_cast<const v4i*>(lw + j * 32 * kStep + frag_offset[ks]);
-    };
-    auto multiply = [&](int slot) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
-    };
-    // W8: a wave's 2*BLOCKS_PER_WAVE load instructions per K step are threaded one by one between
-    // MFMAs and spread over three MFMA groups.  A wave cannot issue anything while a vector-memory
-    // instruction waits for a slot in the CU's memory pipeline, and eight waves that all request
-    // their 8 KiB right after the barrier queue up there for most of an MFMA group; a single
-    // request at a time leaves the wave's next MFMAs issuable almost at once.
-    constexpr int LOADS = 2 * BLOCKS_PER_WAVE;
-    constexpr int PART0 = (LOADS + 2) / 3, PART1 = (LOADS - PART0 + 1) / 2, PART2 = LOADS - PART0 - PART1;
-    static_assert(PART0 <= TM * TN / 2 && PART1 <= TM * TN / 2, "one request after every second MFMA of a group");
-    auto issue_one = [&](int id, int kt_target, int stage) {  // id < BLOCKS_PER_WAVE: activations, else weights
-        const bool weights = id >= BLOCKS_PER_WAVE;
-        const int block = wave * BLOCKS_PER_WAVE + (weights ? id - BLOCKS_PER_WAVE : id);
-        const int row = block * 8 + load_r8;
-        const int chunk = load_slot ^ swizzle(row);
-        const int source_row = weights ? col0 + min(row, cols_here - 1) : row0 + min(row, rows_here - 1);
-        direct_load_16((weights ? w8 : p.a) + (int64_t)source_row * p.k + kt_target * kStep + chunk * 16,
-                       (weights ? stage_w(stage) : stage_a(stage)) + block * 1024);
-    };
-    // Requests are unconditional: a step past the end is clamped to the last one and lands in a
-    // stage that is not read again (the epilogue waits for it before it reuses LDS), which keeps
-    // branches out of the MFMA stream.
-    auto multiply_loading = [&](int slot, int first, int count, int kt_target, int stage) {
-        kt_target = min(kt_target, k_tiles - 1);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
-                const int index = i * TN + j;
-                if ((index & 1) == 1 && index / 2 < count) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (!Q4) issue_one(first + index / 2, kt_target, stage);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-    };
-    // Q4: the whole weight tile of step kt+2 is decoded in one piece right after MFMA group 3 of
-    // step kt, into the stage the barrier of step kt has just released.  (Threading the decode
-    // between the MFMAs of a group, with or without pipelined table reads, measured 20 % slower:
-    // the LDS waits of the decode then sit in the MFMA issue stream.)
-    read_fragments(0, 0, 0);
-    for (int kt = 0; kt < k_tiles; ++kt) {
-        const int cur = kt & 1, nxt = cur ^ 1;
-        // the rest of step kt+1 (its first part went out behind the previous barrier; in step 0 this
-        // repeats part of the prologue's request for step 1, byte for byte)
-        read_fragments(cur, 1, 1);
-        __builtin_amdgcn_sched_barrier(0);  // reads above stay ahead of the MFMAs below
-        multiply_loading(0, PART0, PART1, kt + 1, nxt);
-        __builtin_amdgcn_sched_barrier(0);
-        read_fragments(cur, 2, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply_loading(1, PART0 + PART1, PART2, kt + 1, nxt);
-        __builtin_amdgcn_sched_barrier(0);
-        read_fragments(cur, 3, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(0);
-        __builtin_amdgcn_sched_barrier(0);
-        // this wave's part of step kt+1; the code loads issued after it (Q4, step kt+3) may stay
-        // in flight: a barrier should not wait for HBM
-        if (Q4 && kt + 3 < k_tiles)
-            wait_direct_loads_except<CODE_CHUNKS>();
-        else
-            wait_direct_loads();
-        __syncthreads();
-        if (Q4 && kt + 2 < k_tiles) issue_direct(p.a, rows_here, row0, kt + 2, stage_a(cur));
-        if (kt + 1 < k_tiles) read_fragments(nxt, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply_loading(1, 0, PART0, kt + 2, cur);
-        __builtin_amdgcn_sched_barrier(0);
-        if (Q4 && kt + 2 < k_tiles) {
-            decode_step(stage_w(cur), cur);
-            if (kt + 4 < k_tiles) load_codes(kt + 4, cur);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    }
-
-    // ---- epilogue ----
-    // the clamped requests of the last two steps may still be writing LDS (and a workgroup must
-    // not end with direct-to-LDS loads in flight)
-    if (!Q4) wait_direct_loads();
-    // Weights are the MFMA row operand, so a lane holds token row (lane & 31) of each 32x32 block
-    // and, per group of four accumulator registers, four CONSECUTIVE output channels
-    // 8*q + 4*(lane >> 5) + {0..3}.
-    const int half = lane >> 5;
-    if (p.out_f32) {
-        // fp32 heads are rare: 16-byte stores straight from the accumulators
-        const bool vector_ok = p.stride % 4 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
-            if (local_row >= rows_here) continue;
-            const int64_t row = row0 + local_row;
-            const float token_scale = __half2float(p.as[row]);
-#pragma unroll
-            for (int j = 0; j < TN; ++j) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int local_col = (wave_n * TN + j) * 32 + 8 * q + 4 * half;
-                    if (local_col >= cols_here) continue;
-                    const int col = col0 + local_col;
-                    float value[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        value[r] = rescale(acc[i][j][4 * q + r], __half2float(p.ws[min(col + r, p.n - 1)]), token_scale);
-                    float* dst = reinterpret_cast<float*>(p.out) + row * p.stride + col;
-                    if (local_col + 4 <= cols_here && vector_ok && (col & 3) == 0) {
-                        *reinterpret_cast<float4*>(dst) = make_float4(value[0], value[1], value[2], value[3]);
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (local_col + r < cols_here) dst[r] = value[r];
-                    }
-                }
-            }
-        }
-        return;
-    }
-    // fp16: rescale into an LDS image of the tile (8-byte writes), then store whole 16-byte pieces
-    // of output rows.  The operand stages are dead after the last K step, so their LDS is reused.
-    __syncthreads();
-    float* lds_as = reinterpret_cast<float*>(lds + kEpilogueTile);  // 256 token scales
-    float* lds_ws = lds_as + kTile;                                  // 256 weight scales
-#pragma unroll
-    for (int e = 0; e < SCALES_PER_THREAD; ++e)
-        lds_as[tid + e * kThreads] = __half2float(__ushort_as_half(scale_bits[e]));  // lds_ws follows lds_as
-    __syncthreads();
-    __half* image = reinterpret_cast<__half*>(lds);
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int local_row = (wave_m * TM + i) * 32 + (lane & 31);
-        const float token_scale = lds_as[local_row];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int local_col = (wave_n * TN + j) * 32 + 8 * q + 4 * half;
-                const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
-                const __half2 lo = __halves2half2(__float2half_rn(rescale(acc[i][j][4 * q + 0], wscale.x, token_scale)),
-                                                  __float2half_rn(rescale(acc[i][j][4 * q + 1], wscale.y, token_scale)));
-                const __half2 hi = __halves2half2(__float2half_rn(rescale(acc[i][j][4 * q + 2], wscale.z, token_scale)),
-                                                  __float2half_rn(rescale(acc[i][j][4 * q + 3], wscale.w, token_scale)));
-                uint2 packed;
-                packed.x = *reinterpret_cast<const uint32_t*>(&lo);
-                packed.y = *reinterpret_cast<const uint32_t*>(&hi);
-                *reinterpret_cast<uint2*>(image + local_row * kImagePitch + local_col) = packed;
-            }
-        }
-    }
-    __syncthreads();
-    // each thread moves 16 bytes: kThreads/32 rows x 512 bytes per pass
-    const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0) && (col0 % 8 == 0);
-    const int piece = tid & 31, piece_row = tid >> 5;
-    constexpr int ROWS_PER_PASS = kThreads / 32;
-#pragma unroll 4
-    for (int pass = 0; pass < kTile / ROWS_PER_PASS; ++pass) {
-        const int local = pass * ROWS_PER_PASS + piece_row;
-        if (local >= rows_here) break;
-        const uint4 value = *reinterpret_cast<const uint4*>(image + local * kImagePitch + piece * 8);
-        __half* dst = reinterpret_cast<__half*>(p.out) + (int64_t)(row0 + local) * p.stride + col0 + piece * 8;
-        if (aligned && piece * 8 + 8 <= cols_here) {
-            *reinterpret_cast<uint4*>(dst) = value;
-        } else {
-            const __half* h = reinterpret_cast<const __half*>(&value);
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (piece * 8 + e < cols_here) dst[e] = h[e];
-        }
-    }
 }
 
 // ---- int8 weights: persistent workgroups ------------------------------------------------------------
@@ -479,7 +147,7 @@ __device__ __forceinline__ const int8_t* uniform_pointer(const int8_t* pointer) 
 // weight fragments are live per phase and a second set is on its way from LDS: 64 fragment registers.
 template <bool F32>
 __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel(BigParams p) {
-    constexpr int WAVES_N = 4, kThreads = kPersistentThreads, BLOCKS_PER_WAVE = 4;
+    constexpr int WAVES_N = 4, BLOCKS_PER_WAVE = 4;
     extern __shared__ __align__(16) int8_t lds[];  // [2 stages][A 32 KiB | W 32 KiB], 512 scales
     float* const lds_as = reinterpret_cast<float*>(lds + 4 * kTileBytes);  // 256 token scales, then 256 weight scales
     float* const lds_ws = lds_as + kTile;
@@ -776,16 +444,326 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
     wait_direct_loads();
 }
 
-// operand stages (128 KiB, + 8 KiB of decode tables for Q4) or the epilogue's output image + scales
-constexpr uint32_t kBigLdsEpilogue = kEpilogueTile + 2 * kTile * 4;
-constexpr uint32_t kBigLds = 4 * kTileBytes > kBigLdsEpilogue ? 4 * kTileBytes : kBigLdsEpilogue;
-constexpr uint32_t kBigLdsQ4 = 4 * kTileBytes + sizeof(Q4ByteTables) > kBigLdsEpilogue
-                                   ? 4 * kTileBytes + sizeof(Q4ByteTables)
-                                   : kBigLdsEpilogue;
+// ---- two-stage codes, up to 512 rows: 512 x 128 tiles with the decode in the K loop ----------------------------
+// Between 385 and 512 rows the 256 x 256 tiles need the weights decoded once into scratch first (1.5 bytes of HBM
+// traffic per weight, a launch of its own) and then leave half the CUs idle at N = 17408; decoding inside those
+// tiles instead repeats the decode for every row tile.  A tile of 512 token rows x 128 channels holds the same
+// multiplies per workgroup, decodes every weight once, and needs no scratch.  The price is LDS: 512 rows of a
+// 128-byte K step would be 64 KiB per stage, so the K step here is one MFMA slice of 64: three stages of token
+// rows (32 KiB each, requested two steps ahead with direct-to-LDS loads), two stages of decoded weights (8 KiB),
+// the byte tables and the tile's scales.
+//
+// Eight waves, 4 x 2, of 128 token rows x 64 channels each (the wave tile, fragment layout and epilogue of the
+// persistent kernel above).  A thread owns one 16-byte chunk of the decoded weight stage per step: channel
+// tid / 4, K bytes [16 (tid % 4), +16) of the slice, i.e. two code words; it holds the four words of its channel
+// and quarter for a K block of 128 (two steps) in registers, a second set for the block after it.
+//
+// Step s:   read the token fragments of the step's second half; wait for the first half and the weights;
+//           16 multiplies, with the requests for step s + 2 (and, in odd steps, the codes two blocks ahead) between
+//           them; eight table lookups for step s + 1's weights, combined and written while the multiplies run;
+//           barrier (step s + 1's token rows have landed, its weights are written, nobody reads what step s + 2's
+//           requests overwrite); read the first fragments of step s + 1; the other 16 multiplies.
+// Every LDS access of the loop is an asm statement with hand-placed waits: the compiler would wait for all
+// direct-to-LDS requests in flight before any LDS access it can see.
+constexpr int kTallRows = 512, kTallCols = 128, kTallStep = 64, kTallThreads = 512, kTallStagesA = 3;
+constexpr uint32_t kTallStageA = kTallRows * kTallStep, kTallStageW = kTallCols * kTallStep;
+constexpr uint32_t kTallWeights = kTallStagesA * kTallStageA;          // byte offsets in dynamic LDS
+constexpr uint32_t kTallTables = kTallWeights + kTallStagesA * kTallStageW;
+constexpr uint32_t kTallScales = kTallTables + (uint32_t)sizeof(Q4ByteTables);
+constexpr uint32_t kTallLds = kTallScales + (kTallRows + kTallCols) * 4;
 
-// wave shape of the shipped kernels
-constexpr int kTM = ORX_BIG_TM, kTN = ORX_BIG_TN;
-constexpr int kBigThreads = (8 / kTM) * (8 / kTN) * 64;
+typedef unsigned int v2w __attribute__((ext_vector_type(2)));
+
+template <int OFFSET>
+__device__ __forceinline__ v2w lds_read_8(uint32_t lds_address) {
+    v2w value;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
+    return value;
+}
+// 8 bytes from global memory that the compiler keeps no count for: whoever uses them waits by hand
+__device__ __forceinline__ void load_8(v2w& destination, uint32_t lane_offset, const int8_t* uniform_base) {
+    asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(destination) : "v"(lane_offset), "s"(uniform_base) : "memory");
+}
+__device__ __forceinline__ void lds_write_16(uint32_t lds_address, v4u value) {
+    asm volatile("ds_write_b128 %0, %1" ::"v"(lds_address), "v"(value) : "memory");
+}
+// rows of 64 bytes: four chunks of 16; chunk c of row r sits at position c ^ ((r / 4) % 4), so that the 16 rows a
+// fragment read touches per chunk spread over all banks
+__device__ __forceinline__ int tall_swizzle(int row) { return (row >> 2) & 3; }
+
+template <bool F32>
+__global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p) {
+    extern __shared__ __align__(16) int8_t lds[];
+    float* const lds_as = reinterpret_cast<float*>(lds + kTallScales);
+    float* const lds_ws = lds_as + kTallRows;
+    Q4ByteTables* const tables = reinterpret_cast<Q4ByteTables*>(lds + kTallTables);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int tn = (int)blockIdx.x % p.tiles_n, tm = (int)blockIdx.x / p.tiles_n;
+    TileState t;
+    t.row0 = tm * kTallRows, t.col0 = tn * kTallCols;
+    t.rows_here = min(kTallRows, p.m - t.row0), t.cols_here = min(kTallCols, p.n - t.col0);
+    const int steps = p.k / kTallStep, blocks = p.k / 128;
+    const uint32_t lds_base = lds_address_of(lds);
+
+    // ---- codes: words 2q, 2q+1 (first step of a K block) and 8+2q, 8+2q+1 (second step) of channel tid / 4 ----
+    const int channel = tid >> 2, quarter = tid & 3;
+    const int code_row = t.col0 + min(channel, t.cols_here - 1);
+    // The loads are asm statements: the compiler then keeps no count for them, and the waits in front of the barriers
+    // (which let only the current step's requests stay in flight) are what guarantees that a set has arrived two
+    // steps after it was requested.  Sets and halves are compile-time indices everywhere, so that no select or copy
+    // touches a register whose load is still in flight.
+    v2w codes[2][2];  // [set][half of the K block]
+    // address = uniform base of the K block (+ uniform step to its second half) + a lane offset, for all three layouts:
+    // row-major (N, K/8) words, K-major blocks of 128 (K/128, N, 16) and of 64 (K/64, N, 8)
+    const uint32_t piece = (uint32_t)((quarter >> 1) * 16 + (quarter & 1) * 8);
+    const uint32_t code_lane = (uint32_t)code_row * (uint32_t)(p.packed_k == 0 ? blocks * 64 : p.packed_k == 128 ? 64 : 32) + piece;
+    const int64_t block_stride = p.packed_k == 0 ? 64 : (int64_t)p.n * 64;
+    const int64_t half_stride = p.packed_k == 64 ? (int64_t)p.n * 32 : 32;
+    auto load_codes = [&](int block, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
+        const int8_t* const base = uniform_pointer(reinterpret_cast<const int8_t*>(p.w) + (int64_t)min(block, blocks - 1) * block_stride);
+        load_8(codes[SET][0], code_lane, base);
+        load_8(codes[SET][1], code_lane, base + half_stride);
+    };
+    load_codes(0, std::integral_constant<int, 0>{});
+    load_codes(1, std::integral_constant<int, 1>{});
+
+    // ---- tables and scales, written before any direct-to-LDS request is in flight ----
+    build_tables(*tables, p.book, tid, kTallThreads);
+    lds_as[tid] = __half2float(p.as[t.row0 + min(tid, t.rows_here - 1)]);
+    if (tid < kTallCols) lds_ws[tid] = __half2float(p.ws[t.col0 + min(tid, t.cols_here - 1)]);
+    __syncthreads();
+
+    // ---- token rows: a wave requests rows [64 wave, +64) of a step, four 1 KiB blocks of 16 rows ----
+    const int load_row = wave * 64 + (lane >> 2);
+    const uint32_t load_chunk = (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);  // (row / 4) % 4 = (lane / 16) % 4 in every block
+    const int8_t* const a_base = uniform_pointer(p.a + (int64_t)t.row0 * p.k);
+    auto issue_tokens = [&](int b, int step, int stage) {
+        int row = load_row;
+        asm volatile("" : "+v"(row));  // or every request's offset is kept in a register for the whole loop
+        const uint32_t offset = (uint32_t)(min(row + 16 * b, t.rows_here - 1) * p.k) + load_chunk;
+        direct_load_16(a_base + min(step, steps - 1) * kTallStep + (uint64_t)offset,
+                       lds + stage * kTallStageA + (wave * 4 + b) * 1024);
+    };
+
+    // ---- fragments: a lane reads K bytes [16 (lane / 16), +16) of the slice for row lane % 16 of a block ----
+    const int frag_row = lane & 15, frag_chunk = lane >> 4;
+    const uint32_t frag_offset = (uint32_t)(frag_row * kTallStep + ((frag_chunk ^ tall_swizzle(frag_row)) * 16));
+    const uint32_t a_frag = lds_base + wave_m * 128 * kTallStep + frag_offset;
+    const uint32_t w_frag = lds_base + kTallWeights + wave_n * 64 * kTallStep + frag_offset;
+    v4i ft[2][4], fw[2][4];  // token fragments of a step's halves; weight fragments of even and odd steps
+    constexpr int kBlock = 16 * kTallStep;
+    auto read_tokens = [&](int stage, int half) {
+        const uint32_t a = a_frag + stage * kTallStageA + half * 4 * kBlock;
+        v4i(&f)[4] = ft[half];
+        f[0] = lds_read_16<0>(a);
+        f[1] = lds_read_16<kBlock>(a);
+        f[2] = lds_read_16<2 * kBlock>(a);
+        f[3] = lds_read_16<3 * kBlock>(a);
+    };
+    auto read_weights = [&](int stage, int parity) {  // register set by the parity of the step
+        const uint32_t w = w_frag + stage * kTallStageW;
+        v4i(&f)[4] = fw[parity];
+        f[0] = lds_read_16<0>(w);
+        f[1] = lds_read_16<kBlock>(w);
+        f[2] = lds_read_16<2 * kBlock>(w);
+        f[3] = lds_read_16<3 * kBlock>(w);
+    };
+
+    // ---- decode: this thread's chunk of a weight stage ----
+    const uint32_t table_base = lds_base + kTallTables;
+    const uint32_t write_offset = kTallWeights + (uint32_t)(channel * kTallStep + ((quarter ^ tall_swizzle(channel)) * 16));
+    v2w looked[8];
+    auto lookups = [&](v2w pair) {  // two code words: basis0, mask0, basis1, mask1 of each
+        asm volatile("" : "+v"(pair));  // nothing computed from the words moves above this point
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const uint32_t code = pair[i];
+            looked[4 * i + 0] = lds_read_8<0>(table_base + ((code >> 5) & 0x7F8u));       // basis0[(code >> 8) & 255]
+            looked[4 * i + 1] = lds_read_8<2048>(table_base + ((code << 3) & 0x7F8u));    // mask0[code & 255]
+            looked[4 * i + 2] = lds_read_8<4096>(table_base + ((code >> 21) & 0x7F8u));   // basis1[code >> 24]
+            looked[4 * i + 3] = lds_read_8<6144>(table_base + ((code >> 13) & 0x7F8u));   // mask1[(code >> 16) & 255]
+        }
+    };
+    auto write_decoded = [&](int stage) {
+        // every LDS request of this wave has returned (the lookups are the youngest)
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
+                       "+v"(looked[6]), "+v"(looked[7]));
+        v4u chunk;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            chunk[2 * i + 0] = ((looked[4 * i][0] ^ looked[4 * i + 1][0]) + (looked[4 * i + 2][0] ^ looked[4 * i + 3][0]) + 0x35353535u) ^ 0x80808080u;
+            chunk[2 * i + 1] = ((looked[4 * i][1] ^ looked[4 * i + 1][1]) + (looked[4 * i + 2][1] ^ looked[4 * i + 3][1]) + 0x35353535u) ^ 0x80808080u;
+        }
+        lds_write_16(lds_base + write_offset + stage * kTallStageW, chunk);
+    };
+
+    v4i acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    auto multiply = [&](int half, int parity, auto between) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int jj = (i & 1) ? 3 - j : j;
+                v4i& sum = acc[4 * half + i][jj];
+                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[parity][jj], ft[half][i], sum, 0, 0, 0);
+                between(i * 4 + j);
+            }
+    };
+
+    // ---- prologue: steps 0 and 1 requested, their weights decoded (block 0), step 0's first fragments read ----
+#pragma unroll
+    for (int b = 0; b < 4; ++b) issue_tokens(b, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) issue_tokens(b, 1, 1);
+    asm volatile("s_waitcnt vmcnt(8)" : "+v"(codes[0][0]), "+v"(codes[0][1]), "+v"(codes[1][0]), "+v"(codes[1][1]));
+    lookups(codes[0][0]);
+    write_decoded(0);
+    lookups(codes[0][1]);
+    write_decoded(1);
+    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    read_tokens(0, 0);
+    read_weights(0, 0);
+
+    // One step.  The weights are decoded two steps ahead, behind the barrier: step s writes the stage of step s + 2
+    // (block (s + 2) / 2, held in set ((s + 2) / 2) % 2; an even step decodes the first half of the next block, an odd
+    // step the second half of the same), its lookups issued in front of the second 16 multiplies and combined behind
+    // them, so that no table latency stands between a multiply and a barrier.  Even steps also request the codes of
+    // block s / 2 + 2 into the set that block s / 2 has just left.  The waits name how many younger requests may
+    // stay in flight: vector memory retires in order, and this step's 4 token requests (and the 2 code requests of
+    // an even step) are younger than step s + 1's rows.
+    auto step = [&](int s, auto set_tag, auto odd_tag) {
+        constexpr int SET = decltype(set_tag)::value, ODD = decltype(odd_tag)::value;  // SET: of the block being decoded
+        const int stage = s % kTallStagesA, next_stage = (s + 1) % kTallStagesA, load_stage = (s + 2) % kTallStagesA;
+        read_tokens(stage, 1);                                // 4 younger requests than the first half and the weights
+        wait_eight<4>(ft[0], fw[ODD]);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(0, ODD, [&](int index) {
+            if ((index & 3) == 3) {
+                __builtin_amdgcn_sched_barrier(0);
+                issue_tokens(index >> 2, s + 2, load_stage);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!ODD) load_codes((s >> 1) + 2, std::integral_constant<int, 1 - SET>{});
+        wait_four<0>(ft[1]);
+        if constexpr (!ODD)
+            asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        read_tokens(next_stage, 0);
+        read_weights(next_stage, 1 - ODD);
+        lookups(codes[SET][ODD]);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1, ODD, [](int) {});
+        __builtin_amdgcn_sched_barrier(0);
+        write_decoded(load_stage);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // steps 4 g .. 4 g + 3 decode blocks 2 g + 1 (set 1: steps 4 g, 4 g + 1) and 2 g + 2 (set 0: steps 4 g + 2, 4 g + 3)
+    std::integral_constant<int, 0> zero;
+    std::integral_constant<int, 1> one;
+    int s = 0;
+    for (; s + 3 < steps; s += 4) {
+        step(s, one, zero);       // requests block 2 g + 2 into set 0
+        step(s + 1, one, one);
+        step(s + 2, zero, zero);  // requests block 2 g + 3 into set 1
+        step(s + 3, zero, one);
+    }
+    if (s < steps) {  // K = 128 x an odd number: one block left
+        step(s, one, zero);
+        step(s + 1, one, one);
+    }
+    // The last steps request code words, token rows and fragments that nobody consumes (clamped addresses; the waits above
+    // count on every step issuing the same requests).  Their destination registers are named here, behind the wait:
+    // a register whose value the compiler believes dead is free for reuse while its load is still in flight, and the
+    // data would land on whatever lives there by then.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)"
+                 : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(ft[1][0]), "+v"(ft[1][1]), "+v"(ft[1][2]),
+                   "+v"(ft[1][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]), "+v"(fw[0][3]), "+v"(fw[1][0]), "+v"(fw[1][1]),
+                   "+v"(fw[1][2]), "+v"(fw[1][3])
+                 :
+                 : "memory");
+    asm volatile("" : "+v"(codes[0][0]), "+v"(codes[0][1]), "+v"(codes[1][0]), "+v"(codes[1][1]));
+
+    // ---- epilogue: as in the persistent kernel, private to a wave and in registers ----
+    int own = threadIdx.x & 63;
+    asm volatile("" : "+v"(own));
+    const int group = own >> 4;
+    if constexpr (F32) {
+        const bool vector_ok = p.stride % 4 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int local_row = wave_m * 128 + i * 16 + (own & 15);
+            if (local_row >= t.rows_here) continue;
+            const int64_t row = t.row0 + local_row;
+            const float token_scale = lds_as[local_row];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int local_col = wave_n * 64 + j * 16 + 4 * group;
+                if (local_col >= t.cols_here) continue;
+                const int col = t.col0 + local_col;
+                const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
+                const float value[4] = {rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale),
+                                        rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale)};
+                float* dst = reinterpret_cast<float*>(p.out) + row * p.stride + col;
+                if (local_col + 4 <= t.cols_here && vector_ok && (col & 3) == 0) {
+                    *reinterpret_cast<float4*>(dst) = make_float4(value[0], value[1], value[2], value[3]);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (local_col + r < t.cols_here) dst[r] = value[r];
+                }
+            }
+        }
+    } else {
+        const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
+        const bool whole = aligned && t.rows_here == kTallRows && t.cols_here == kTallCols;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int local_row = wave_m * 128 + i * 16 + (own & 15);
+            const float token_scale = lds_as[local_row];
+            __half* const row_out = reinterpret_cast<__half*>(p.out) + (int64_t)(t.row0 + local_row) * p.stride + t.col0;
+#pragma unroll
+            for (int pair = 0; pair < 2; ++pair) {
+                uint32_t words[2][2];
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const int j = 2 * pair + b;
+                    const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + wave_n * 64 + j * 16 + 4 * group);
+                    words[b][0] = pack_halves(rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale));
+                    words[b][1] = pack_halves(rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale));
+                }
+                const v2u low = __builtin_amdgcn_permlane16_swap(words[0][0], words[1][0], false, false);
+                const v2u high = __builtin_amdgcn_permlane16_swap(words[0][1], words[1][1], false, false);
+                const uint4 piece = make_uint4(low.x, high.x, low.y, high.y);
+                const int local_col = wave_n * 64 + (2 * pair + (group & 1)) * 16 + (group >> 1) * 8;
+                if (whole) {
+                    *reinterpret_cast<uint4*>(row_out + local_col) = piece;
+                } else if (local_row < t.rows_here && local_col < t.cols_here) {
+                    if (aligned && local_col + 8 <= t.cols_here) {
+                        *reinterpret_cast<uint4*>(row_out + local_col) = piece;
+                    } else {
+                        const uint32_t parts[4] = {piece.x, piece.y, piece.z, piece.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (local_col + e < t.cols_here)
+                                row_out[local_col + e] = __ushort_as_half((unsigned short)(parts[e >> 1] >> (16 * (e & 1))));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+}
 
 int prepare_device() {
     int code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_persistent_kernel<false>),
@@ -796,8 +774,12 @@ int prepare_device() {
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPersistentLds),
                      "hipFuncSetAttribute");
     if (code != ORX_OK) return code;
-    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel<true, kTM, kTN>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsQ4),
+    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q4_tall_kernel<false>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTallLds),
+                     "hipFuncSetAttribute");
+    if (code != ORX_OK) return code;
+    code = hip_check(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_q4_tall_kernel<true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kTallLds),
                      "hipFuncSetAttribute");
     return code;
 }
@@ -851,36 +833,59 @@ int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int
     return hip_check(hipGetLastError(), "launch two-stage weight expansion");
 }
 
-void gemm_big_geometry(int rows, int n, bool q4, Geometry* g) {
+// int8 weights: one persistent workgroup per CU walks the 256 x 256 tiles
+void gemm_big_geometry(int rows, int n, Geometry* g) {
     const uint32_t tiles = ceil_div((uint32_t)rows, (uint32_t)kTile) * ceil_div((uint32_t)n, (uint32_t)kTile);
-    // int8 weights: one persistent workgroup per CU walks the tiles; two-stage codes decoded in the loop: one per tile
-    g->grid[0] = q4 ? tiles : std::min(tiles, (uint32_t)device_compute_units());
+    g->grid[0] = std::min(tiles, (uint32_t)device_compute_units());
     g->grid[1] = g->grid[2] = 1;
-    g->block[0] = q4 ? kBigThreads : kPersistentThreads;
-    g->shared = q4 ? kBigLdsQ4 : kPersistentLds;
+    g->block[0] = kPersistentThreads;
+    g->shared = kPersistentLds;
 }
 
-int gemm_big_launch(bool q4, const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as,
-                    void* out, int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g,
-                    hipStream_t stream) {
+int gemm_big_launch(const int8_t* a, const void* w, const __half* ws, const __half* as, void* out, int rows, int n,
+                    int k, int stride, bool out_f32, const Geometry& g, hipStream_t stream) {
     const int ready = prepare();
     if (ready != ORX_OK) return ready;
     BigParams p = {};
-    p.a = a, p.w = w, p.book = book, p.ws = ws, p.as = as, p.out = out;
-    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = packed_k, p.out_f32 = out_f32;
+    p.a = a, p.w = w, p.book = nullptr, p.ws = ws, p.as = as, p.out = out;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = 0, p.out_f32 = out_f32;
     p.tiles_m = (rows + kTile - 1) / kTile, p.tiles_n = (n + kTile - 1) / kTile;
-    if (!q4 && k < 2 * kStep) {
+    if (k < 2 * kStep) {
         set_error("projection (mfma 256x256): the persistent int8 kernel needs K >= 256");
         return ORX_ERR_BAD_VARIANT;
     }
-    if (q4)
-        ORX_LAUNCH((gemm_big_kernel<true, kTM, kTN>), dim3(g.grid[0]), dim3(kBigThreads), g.shared, stream, p);
+    if (out_f32)
+        ORX_LAUNCH((gemm_big_persistent_kernel<true>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
     else
-        if (out_f32)
-            ORX_LAUNCH((gemm_big_persistent_kernel<true>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
-        else
-            ORX_LAUNCH((gemm_big_persistent_kernel<false>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
+        ORX_LAUNCH((gemm_big_persistent_kernel<false>), dim3(g.grid[0]), dim3(kPersistentThreads), g.shared, stream, p);
     return hip_check(hipGetLastError(), "launch projection (mfma 256x256)");
+}
+
+// two-stage codes on 512 x 128 tiles with the decode in the K loop (K a multiple of 128)
+void gemm_tall_geometry(int rows, int n, Geometry* g) {
+    g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTallRows) * ceil_div((uint32_t)n, (uint32_t)kTallCols);
+    g->grid[1] = g->grid[2] = 1;
+    g->block[0] = kTallThreads;
+    g->shared = kTallLds;
+}
+
+int gemm_tall_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out,
+                     int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g, hipStream_t stream) {
+    const int ready = prepare();
+    if (ready != ORX_OK) return ready;
+    if (k % 128 != 0 || k < 256) {
+        set_error("projection (mfma 512x128): K must be a multiple of 128, at least 256");
+        return ORX_ERR_BAD_VARIANT;
+    }
+    BigParams p = {};
+    p.a = a, p.w = w, p.book = book, p.ws = ws, p.as = as, p.out = out;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = packed_k, p.out_f32 = out_f32;
+    p.tiles_m = (rows + kTallRows - 1) / kTallRows, p.tiles_n = (n + kTallCols - 1) / kTallCols;
+    if (out_f32)
+        ORX_LAUNCH((gemm_q4_tall_kernel<true>), dim3(g.grid[0]), dim3(kTallThreads), g.shared, stream, p);
+    else
+        ORX_LAUNCH((gemm_q4_tall_kernel<false>), dim3(g.grid[0]), dim3(kTallThreads), g.shared, stream, p);
+    return hip_check(hipGetLastError(), "launch projection (mfma 512x128, decode in the loop)");
 }
 
 }  // namespace orx

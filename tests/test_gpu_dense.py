@@ -853,6 +853,26 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
+@pytest.mark.parametrize("packed_k", [0, 64, 128])
+@pytest.mark.parametrize("m,n,k", [(512, 256, 512), (500, 333, 640), (700, 130, 256), (3, 128, 384)])
+def test_q4_tall_tiles_decode_in_the_k_loop(m, n, k, packed_k):
+    """512 x 128 tiles with the decode in the K loop (`algorithm=tall`; what a handle without a Workspace runs from 385
+    rows on): K of an even and an odd number of 128-blocks, one and two row tiles, ragged rows and channels, every
+    layout, fp16 and fp32 output with a stride and sentinels."""
+    rng = np.random.default_rng(orc.SEED + m + n + k + packed_k)
+    a_q, a_s, packed, scales = q4_case(rng, m, n, k)
+    a_q[0, :2] = [-128, 127]
+    stored = packed if packed_k == 0 else orc.q4_pack_k(packed, packed_k)
+    weights = orc.q4_integers(packed, TABLE)
+    for dtype, np_dtype in ((torch.float16, np.float16), (torch.float32, np.float32)):
+        storage = torch.full((m + 2, n + 8), 91.0, dtype=dtype, device=gu.DEV)
+        gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 8, dtype=dtype,
+                      algorithm="tall", packed_k=packed_k)
+        got = gu.host(storage)
+        np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, weights, scales, np_dtype))
+        assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+
+
 @pytest.mark.parametrize("codec", ["w8", "q4"])
 def test_a_few_tiles_more_than_cus_go_to_split_tiles(codec):
     """A handful of 256 x 256 tiles beyond one round of the persistent kernel: it takes the column tiles that fill the
