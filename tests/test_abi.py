@@ -535,6 +535,26 @@ def test_projections_take_the_reference_factories_schedule_names():
         lib.Kernel("int8_projection", **short, block_m=128).geometry(100)
 
 
+def test_tall_tiles_by_name_and_for_handles_without_scratch():
+    """512 x 128 tiles with the decode in the K loop: by name at any row count, and what a two-stage handle without a
+    Workspace (or with decode_in_gemm) launches from 385 rows; K in whole blocks of 128, two-stage codes only."""
+    shape = dict(M=1024, N=17408, K=5120, dynamic_rows=True)
+    tall = lib.Kernel("e8p_q4_projection", **shape, algorithm="tall")
+    plain = lib.Kernel("e8p_q4_projection", **shape)
+    in_loop = lib.Kernel("e8p_q4_projection", **shape, workspace=True, decode_in_gemm=True)
+    for rows, row_tiles in ((3, 1), (512, 1), (513, 2), (1024, 2)):
+        grid, block, lds = tall.geometry(rows)
+        assert grid == (row_tiles * 136, 1, 1) and block == (512, 1, 1) and 128 * 1024 < lds <= 160 * 1024
+    for rows in (385, 512, 1024):
+        assert plain.geometry(rows) == tall.geometry(rows) == in_loop.geometry(rows)
+        assert in_loop.workspace_bytes(rows) == 0
+    assert plain.geometry(384) != tall.geometry(384)
+    for symbol, bad in (("int8_projection", dict(M=8, N=256, K=512)), ("e8p_q4_projection", dict(M=8, N=256, K=128))):
+        with pytest.raises(lib.OrxError) as err:
+            lib.Kernel(symbol, **bad, algorithm="tall")
+        assert err.value.code == lib.ORX_ERR_BAD_VARIANT and "tall" in str(err.value)
+
+
 def test_two_stage_coefficients_other_than_4_1_are_refused():
     """quantization/e8p_q4.py:19-29 allows other coprime pairs, the model builder only [4, 1]
     (models/qwen35/test_build.py:695-709): the kernels decode 4 * coarse + residual and say so."""
