@@ -917,6 +917,16 @@ def test_a_few_tiles_more_than_cus_go_to_split_tiles(codec):
     other = gu.lib.Kernel(kern.symbol, **dict(variant, split_k=False))
     other(**dict(args, **({"Out": whole} if codec == "q4" else {"Output": whole})))
     np.testing.assert_array_equal(gu.host(whole), got)
+    # a dynamic handle of larger capacity: one Workspace sized for any row count serves this launch and a shorter one
+    dynamic = gu.lib.Kernel(kern.symbol, **dict(variant, M=1024, dynamic_rows=True))
+    space = torch.empty(dynamic.workspace_bytes(0), dtype=torch.uint8, device=gu.DEV)
+    assert dynamic.workspace_bytes(0) >= dynamic.workspace_bytes(rows) == kern.workspace_bytes(rows)
+    for live in (rows, 300):
+        again = torch.full_like(out, 7.0)
+        dynamic(**dict(args, Workspace=space, m=live, **({"Out": again} if codec == "q4" else {"Output": again})))
+        result = gu.host(again)
+        np.testing.assert_array_equal(result[:live], got[:live])
+        assert (result[live:] == 7).all()
 
 
 @pytest.mark.parametrize("packed_k", [0, 64, 128])
