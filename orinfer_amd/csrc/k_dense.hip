@@ -268,7 +268,10 @@ __global__ __launch_bounds__(kSpecThreads) void dense_specialized_kernel(DensePa
                 // i (16 bytes each) holds row i/4, piece (i%4) ^ ((i/8)&3): with that swizzle the
                 // decoders' reads of one piece of 16 different rows fall into different bank groups.
                 const int row = lane >> 2, piece = (lane & 3) ^ ((lane >> 3) & 3);
-                const uint8_t* src = p.w + ((int64_t)first_row + start + row) * 64 + piece * 16;
+                // (blocks of 64: the K block's two halves lie N rows x 32 bytes apart, 512 contiguous bytes each)
+                const uint8_t* src = p.k_major == 2 ? p.w + ((int64_t)first_row + start + row) * 32 + (piece & 1) * 16 +
+                                                          (int64_t)(piece >> 1) * p.n * 32
+                                                    : p.w + ((int64_t)first_row + start + row) * 64 + piece * 16;
 #pragma unroll
                 for (int i = 0; i < kPerLoader; ++i) {
                     const int kb = loader + kLoaders * i;
@@ -448,7 +451,7 @@ uint32_t specialized_lds_bytes(int n, int k) {
 // Loader-wave kernel: K a multiple of 512 up to 5120 (a decoder wave holds the token fragments of K/8).
 bool specialized_fits(int n, int k, int packed_k) {
     if (k % 512 != 0 || k / 512 > 10 || specialized_lds_bytes(n, k) > kLdsLimit) return false;
-    return packed_k == 0 || (packed_k == 128 && k % 1024 == 0);
+    return packed_k == 0 || ((packed_k == 128 || packed_k == 64) && k % 1024 == 0);
 }
 
 template <int S, int CB, bool KM>
@@ -510,7 +513,7 @@ int dense_resident_launch(const int8_t* a, const void* w, const uint32_t* book, 
     }
     DenseParams p = {};
     p.a = a, p.w = reinterpret_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
-    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k != 0;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k == 64 ? 2 : packed_k != 0;  // 1: blocks of 128, 2: blocks of 64
     if (specialized_fits(n, k, packed_k)) {
         switch (k / 512) {
             case 1: return launch_specialized<1>(p, stream);

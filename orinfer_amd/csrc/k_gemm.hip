@@ -1074,7 +1074,7 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         return ORX_ERR_BAD_VARIANT;
     }
     if (f->algorithm == kWide && (codec != kQ4 || !dense_wide_eligible(f->N, f->K, f->packed_k))) {
-        set_error("%s: algorithm=wide serves two-stage codes, row-major or K-major in blocks of 128", name);
+        set_error("%s: algorithm=wide serves two-stage codes, row-major or K-major", name);
         return ORX_ERR_BAD_VARIANT;
     }
     if (half_step) {
@@ -1095,12 +1095,12 @@ int make_projection(const Variant& v, orx_function* f, int codec) {
         set_error("%s: the stream algorithm serves up to 64 rows, variant asks for %d", name, f->capacity);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv && f->packed_k != 0 && (codec != kQ4 || f->packed_k != 128 || f->K % 256 != 0)) {
-        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0), or K-major two-stage codes in 128-wide blocks with K a multiple of 256",
+    if (f->algorithm == kGemv && f->packed_k != 0 && (codec != kQ4 || f->K % 256 != 0)) {
+        set_error("%s: the gemv algorithm reads row-major codes (packed_k = 0), or K-major two-stage codes (blocks of 128 or 64) with K a multiple of 256",
                   name);
         return ORX_ERR_BAD_VARIANT;
     }
-    if (f->algorithm == kGemv || (f->algorithm == kAuto && (f->packed_k == 0 || (codec == kQ4 && f->packed_k == 128 && f->K % 256 == 0)))) {
+    if (f->algorithm == kGemv || (f->algorithm == kAuto && (f->packed_k == 0 || (codec == kQ4 && f->K % 256 == 0)))) {
         orx_function probe = *f;
         if (probe.capacity > 4) probe.capacity = 4;
         int code = gemv_configure(&probe, codec, passes);

@@ -327,8 +327,9 @@ template <int CODEC, int MR, int D, int LAYOUT, bool HOLD, bool X16 = false>
 __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     const int8_t* __restrict__ a, const uint4* __restrict__ w, const uint32_t* __restrict__ book,
     const __half* __restrict__ ws, const __half* __restrict__ as, void* __restrict__ out, int n, int k, int stride,
-    int m, int out_f32, const int8_t* __restrict__ signs) {
+    int m, int flags, const int8_t* __restrict__ signs) {
     extern __shared__ __align__(16) uint32_t lds[];
+    const bool out_f32 = flags & 1;  // bit 1: K-major blocks of 64 instead of 128
     constexpr int LPR = LAYOUT & (kKMajorLayout - 1);
     constexpr bool kKMajor = LAYOUT >= kKMajorLayout;
     constexpr int kRows = 64 / LPR;  // rows per wave task
@@ -351,17 +352,20 @@ __global__ __launch_bounds__(kBankedThreads) void gemv_banked_kernel(
     // plus one 32-bit lane offset: no vector arithmetic per load.
     const int first_task = __builtin_amdgcn_readfirstlane(wave) * gridDim.x + blockIdx.x;
     const char* stream = reinterpret_cast<const char*>(w);
-    // K-major codes (K/128 blocks of N rows x 64 bytes): a task is still 64/LPR adjacent rows, a step
-    // is LPR/4 K blocks, and the lanes of one K block read the task's rows as one contiguous run of
-    // 64 bytes per row.  A lane still owns chunk sub + step * LPR of its row, so everything below the
-    // addressing is shared with the row-major form.
-    const size_t task_bytes = kKMajor ? (size_t)kRows * 64 : (size_t)kRows * row_bytes;
-    const size_t step_bytes = kKMajor ? (size_t)n * 64 * (LPR / 4) : (size_t)LPR * 16;
+    // K-major codes (K/128 blocks of N rows x 64 bytes, or K/64 blocks of N rows x 32 bytes): a task is still
+    // 64/LPR adjacent rows, a step is LPR/4 (LPR/2) K blocks, and the lanes of one K block read the task's rows as
+    // one contiguous run of 64 (32) bytes per row.  A lane still owns chunk sub + step * LPR of its row, so
+    // everything below the addressing is shared with the row-major form.
+    const int block_shift = (flags & 2) ? 1 : 2;  // log2 of the 16-byte chunks a row holds per K block
+    const int block_bytes = 16 << block_shift;
+    const size_t task_bytes = kKMajor ? (size_t)kRows * block_bytes : (size_t)kRows * row_bytes;
+    const size_t step_bytes = kKMajor ? (size_t)n * 16 * LPR : (size_t)LPR * 16;
     auto base_of = [&](int task) { return stream + (size_t)min(task, tasks - 1) * task_bytes; };
     auto lane_offset = [&](int task) {  // rows past the end re-read the task's first row and are not stored
         const int row = min(task, tasks - 1) * kRows + row_in_wave;
         const int local_row = row < n ? row_in_wave : 0;
-        if (kKMajor) return (uint32_t)((sub >> 2) * n * 64 + local_row * 64 + (sub & 3) * 16);
+        if (kKMajor)
+            return (uint32_t)(((sub >> block_shift) * n + local_row) * block_bytes + (sub & ((1 << block_shift) - 1)) * 16);
         return (uint32_t)(local_row * row_bytes + sub * 16);
     };
     auto fetch = [&](const char* base, uint32_t offset, int step) {
@@ -759,24 +763,24 @@ int gemv_launch_banked(const orx_function& f, int rows, const Geometry& g, hipSt
         case 1:
             if (f.input_f16 && hold)
                 ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, true, true>), grid, block, g.shared, stream, a, w,
-                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             else if (f.input_f16)
                 ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, false, true>), grid, block, g.shared, stream, a, w,
-                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                                   book, ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             else if (hold)
                 ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, true>), grid, block, g.shared, stream, a, w, book,
-                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             else
                 ORX_LAUNCH((gemv_banked_kernel<kQ4, 1, D, LPR, false>), grid, block, g.shared, stream, a, w, book,
-                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                                   ws, as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             break;
         case 2:
             ORX_LAUNCH((gemv_banked_kernel<kQ4, 2, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
-                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             break;
         default:
             ORX_LAUNCH((gemv_banked_kernel<kQ4, 4, D, LPR, false>), grid, block, g.shared, stream, a, w, book, ws,
-                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32, pending_signs);
+                               as, out, f.N, f.K, f.stride, rows, (int)f.out_f32 | (f.packed_k == 64 ? 2 : 0), pending_signs);
             break;
     }
     return hip_check(hipGetLastError(), "launch projection (gemv, replicated tables)");
@@ -1142,7 +1146,7 @@ int gemv_prepare_device();
 
 // K-major two-stage codes are only served by the replicated-table kernel.
 bool gemv_serves_k_major(const orx_function& f, int rows) {
-    return f.flags == kQ4 && f.packed_k == 128 && ((uint32_t)f.slots >> 8) >= (uint32_t)kKMajorLayout && use_banked(f, mr_for(rows));
+    return f.flags == kQ4 && (f.packed_k == 128 || f.packed_k == 64) && ((uint32_t)f.slots >> 8) >= (uint32_t)kKMajorLayout && use_banked(f, mr_for(rows));
 }
 
 // Launchers used by the projection factories.  Argument order is the caller's business:
@@ -1198,7 +1202,7 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
         int lanes_per_row = chunks % 32 == 0 ? 32 : chunks % 16 == 0 ? 16 : 0;
         // K-major codes: 16 lanes per row measure best (13.4 us at N=17408, K=5120 against 15.1 with 8
         // and 15.0 with 32), 8 for a K that is a multiple of 256 only
-        if (f->packed_k == 128) lanes_per_row = chunks % 16 == 0 ? 16 : chunks % 8 == 0 ? 8 : 0;
+        if (f->packed_k != 0) lanes_per_row = chunks % 16 == 0 ? 16 : chunks % 8 == 0 ? 8 : 0;
         if (lanes_per_row) {
             const int steps = chunks / lanes_per_row;
             int best_pad = 1 << 30, depth = 4;
@@ -1207,7 +1211,7 @@ int gemv_configure(orx_function* f, int codec, int passes_override) {
                 if (pad < best_pad) best_pad = pad, depth = candidate;
             }
             // the overflow flags hold one bit per step in a 64-bit word per lane column
-            if (steps <= 64) f->slots = depth | (lanes_per_row + (f->packed_k == 128 ? kKMajorLayout : 0)) << 8;
+            if (steps <= 64) f->slots = depth | (lanes_per_row + (f->packed_k != 0 ? kKMajorLayout : 0)) << 8;
         }
     }
     if (gemv_lds_bytes(*f, 4) > kLdsLimit) {

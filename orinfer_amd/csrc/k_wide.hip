@@ -170,8 +170,10 @@ __global__ __launch_bounds__(kThreads) void wide_kernel(WideParams p) {
             const int channel = dl >> 2, quarter = dl & 3;
             const bool active = channel < channels;
             const int source_channel = channel0 + min(channel, channels - 1);
-            const uint8_t* codes = KM ? p.w + (int64_t)source_channel * 64 + quarter * 16
-                                      : p.w + (int64_t)source_channel * (p.k / 2) + quarter * 16;
+            // (K-major blocks of 64: the two halves of a K step lie N rows x 32 bytes apart)
+            const uint8_t* codes = !KM              ? p.w + (int64_t)source_channel * (p.k / 2) + quarter * 16
+                                   : p.k_major == 2 ? p.w + (int64_t)source_channel * 32 + (quarter & 1) * 16 + (int64_t)(quarter >> 1) * p.n * 32
+                                                    : p.w + (int64_t)source_channel * 64 + quarter * 16;
             const int64_t step_bytes = KM ? (int64_t)p.n * 64 : 64;
             const int swz = chunk_swizzle(channel);
             uint8_t* mine = lds + kWeightBase + channel * kStep;
@@ -325,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void wide_kernel(WideParams p) {
 
 // Shapes: two-stage codes, row-major or K-major in blocks of 128.
 bool dense_wide_eligible(int n, int k, int packed_k) {
-    return n > 0 && k > 0 && k % kStep == 0 && (packed_k == 0 || packed_k == 128);
+    return n > 0 && k > 0 && k % kStep == 0 && (packed_k == 0 || packed_k == 128 || packed_k == 64);
 }
 
 void dense_wide_geometry(int n, Geometry* g) {
@@ -350,7 +352,7 @@ int dense_wide_launch(const int8_t* a, const void* w, const uint32_t* book, cons
     if (ready != ORX_OK) return ready;
     WideParams p;
     p.a = a, p.w = static_cast<const uint8_t*>(w), p.book = book, p.ws = ws, p.as = as, p.out = out;
-    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k != 0;
+    p.n = n, p.k = k, p.stride = stride, p.m = rows, p.out_f32 = out_f32, p.k_major = packed_k == 64 ? 2 : packed_k != 0;  // 1: blocks of 128, 2: blocks of 64
     if (packed_k != 0)
         ORX_LAUNCH(wide_kernel<true>, dim3(g.grid[0]), dim3(kThreads), kWideLdsBytes, stream, p);
     else

@@ -134,10 +134,12 @@ def test_resolve_errors():
             lib.Kernel("e8p_q4_projection", **variant)
         assert err.value.code == lib.ORX_ERR_BAD_VARIANT, variant
         assert "e8p_q4_projection" in str(err.value) or "variant" in str(err.value)
-    # K-major blocks of 64 resolve (e8p_q4.py:78-80); the one-row GEMV by name does not read them
+    # K-major blocks of 64 resolve (e8p_q4.py:78-80), for the one-row GEMV by name as well while K is a multiple of 256
     assert lib.Kernel("e8p_q4_projection", M=8, N=128, K=256, packed_k=64).arg_names[-1] == "W"
+    by_name = lib.Kernel("e8p_q4_projection", M=1, N=128, K=256, packed_k=64, algorithm="gemv")
+    assert by_name.geometry(1) == lib.Kernel("e8p_q4_projection", M=1, N=128, K=256, packed_k=128, algorithm="gemv").geometry(1)
     with pytest.raises(lib.OrxError) as err:
-        lib.Kernel("e8p_q4_projection", M=1, N=128, K=256, packed_k=64, algorithm="gemv")
+        lib.Kernel("e8p_q4_projection", M=1, N=128, K=384, packed_k=64, algorithm="gemv")
     assert err.value.code == lib.ORX_ERR_BAD_VARIANT
     with pytest.raises(lib.OrxError):
         lib.Kernel("int8_projection", M=8, N=128, K=256, packed_k=64)

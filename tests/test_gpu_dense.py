@@ -518,35 +518,36 @@ def test_q4_gemv_matches_oracle(m, n, k):
     np.testing.assert_array_equal(gu.host(got), want)
 
 
+@pytest.mark.parametrize("blocks_of", [128, 64])
 @pytest.mark.parametrize("m", [1, 2, 3, 4])
 @pytest.mark.parametrize("n,k", [(65, 256), (257, 2560), (1024, 5120), (130, 16384), (33, 8192 + 512), (7, 1536), (17408, 5120),
                                  (40, 17408), (9, 768)])
-def test_q4_gemv_k_major_codes_match_oracle(m, n, k):
-    """The reference's storage layout (K/128 blocks of N rows): 16 lanes per row and tasks of 4 adjacent rows, or 8 lanes
-    and 8 rows when K is a multiple of 256 only."""
+def test_q4_gemv_k_major_codes_match_oracle(m, n, k, blocks_of):
+    """The reference's storage layouts (K/128 blocks of N rows, or K/64: e8p_q4.py:78-80): 16 lanes per row and tasks of 4
+    adjacent rows, or 8 lanes and 8 rows when K is a multiple of 256 only."""
     rng = np.random.default_rng(orc.SEED + 500 + m + n)
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :4] = [-128, -1, 0, 127]
-    stored = orc.q4_pack_k(packed, 128)
+    stored = orc.q4_pack_k(packed, blocks_of)
     w = orc.q4_integers(packed, TABLE)
     acc = orc.int_dot(a_q, w)
     ones_n, ones_m = np.ones(n, np.float16), np.ones(m, np.float16)
     planes_fit = 131072 + (1 if m == 1 else 2 if m == 2 else 4) * (k // 8) * 12 + 256 + k // 32 + 16 <= 160 * 1024
     if not planes_fit:  # the activation planes of so many rows do not fit beside the tables: refused at launch
         with pytest.raises(Exception, match="K-major"):
-            gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), algorithm="gemv", packed_k=128)
+            gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), algorithm="gemv", packed_k=blocks_of)
         return
     got_acc = gu.q4_project(gu.dev(a_q), gu.dev(ones_m), gu.dev(stored), gu.dev(ones_n), dtype=torch.float32,
-                            algorithm="gemv", packed_k=128)
+                            algorithm="gemv", packed_k=blocks_of)
     np.testing.assert_array_equal(gu.host(got_acc).astype(np.int64), acc.astype(np.int64))
     storage = torch.full((m + 1, n + 5), 91.0, dtype=torch.float16, device=gu.DEV)
     gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 5,
-                  algorithm="gemv", packed_k=128)
+                  algorithm="gemv", packed_k=blocks_of)
     got = gu.host(storage)
     np.testing.assert_array_equal(got[:m, :n], orc.rescale(acc, scales, a_s))
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
     if m <= 2:  # what `auto` picks for K-major codes at 1 and 2 rows
-        auto = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=128)
+        auto = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=blocks_of)
         np.testing.assert_array_equal(gu.host(auto), orc.rescale(acc, scales, a_s))
 
 
@@ -658,20 +659,21 @@ def test_q4_resident_rows_blocks_and_tails(m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(3, 97, 1024), (16, 300, 2048), (17, 1000, 3072), (8, 5000, 4096), (32, 17408, 5120),
                                    (64, 2050, 5120), (5, 40, 2048)])
-def test_q4_resident_k_major_codes(m, n, k):
-    """The loader/decoder kernel on the reference's storage layout (K/128 blocks of N rows x 64 bytes)."""
+@pytest.mark.parametrize("blocks_of", [128, 64])
+def test_q4_resident_k_major_codes(m, n, k, blocks_of):
+    """The loader/decoder kernel on the reference's storage layouts (K/128 blocks of N rows x 64 bytes, K/64 x 32)."""
     rng = np.random.default_rng(orc.SEED + 400 + m + n)
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :2] = [-128, 127]
-    stored = orc.q4_pack_k(packed, 128)
+    stored = orc.q4_pack_k(packed, blocks_of)
     w = orc.q4_integers(packed, TABLE)
     storage = torch.full((m + 2, n + 3), 91.0, dtype=torch.float32, device=gu.DEV)
     gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), out=storage, stride=n + 3,
-                  dtype=torch.float32, algorithm="resident", packed_k=128)
+                  dtype=torch.float32, algorithm="resident", packed_k=blocks_of)
     got = gu.host(storage)
     np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, w, scales, np.float32))
     assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
-    half = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=128)  # what `auto` picks
+    half = gu.q4_project(gu.dev(a_q), gu.dev(a_s), gu.dev(stored), gu.dev(scales), packed_k=blocks_of)  # what `auto` picks
     np.testing.assert_array_equal(gu.host(half), orc.project(a_q, a_s, w, scales))
 
 
@@ -819,7 +821,7 @@ def test_w8_k_ends_in_half_a_step(m, k):
 # Channel runs per CU over the whole K (`algorithm=wide`): one and two row passes, a last pass of one row,
 # runs of 2, 97 (two channel passes, the second with one channel) and 100 channels per CU, a K of one step
 # and of many, both code layouts, strided fp32 output with sentinels, extremes outside the A8 range.
-@pytest.mark.parametrize("packed_k", [0, 128])
+@pytest.mark.parametrize("packed_k", [0, 128, 64])
 @pytest.mark.parametrize("m,n,k", [(33, 300, 384), (64, 24832, 128), (100, 1000, 640), (128, 300, 5120), (129, 515, 256),
                                    (200, 25600, 256), (256, 300, 1024)])
 def test_q4_channel_run_kernel(m, n, k, packed_k):
