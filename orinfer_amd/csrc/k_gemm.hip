@@ -762,10 +762,24 @@ bool use_resident(const orx_function& f, int rows) {
 // K=5120 against 86..93 us for decode-once + 256x256, and 54..60 us against 58..62 us for W8; at 512
 // rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
 bool split_preferred_to_big(const orx_function& f, int rows);
+// Two-stage codes without scratch: 512 x 128 tiles with the decode in the K loop against whole 128 x 128 tiles, which
+// decode every weight once per 128 rows but come four to the 512 rows.  Measured at K = 5120 (times scale with K):
+// the tall tiles take 87 us per round of the CUs (N = 17408: 91 / 172 / 263 us at 512 / 1024 / 2048 rows), the small
+// ones 40 us + 32 us per tile and CU (105 / 171 / 314 us); N = 5120: 86 / 87 / 88 against 57 / 78 / 107 us.
+bool tall_beats_whole_tiles(const orx_function& f, int rows) {
+    const int64_t cus = device_compute_units();
+    const int64_t columns = ceil_div((uint32_t)f.N, 128u);
+    const int64_t tall = columns * ceil_div((uint32_t)rows, 512u), small = columns * ceil_div((uint32_t)rows, 128u);
+    return 87 * ((tall + cus - 1) / cus) * cus < 40 * cus + 32 * small;
+}
 bool use_big(const orx_function& f, int rows) {
     if (f.K % kBK || f.K < 2 * kBK) return false;  // half a K step at the end, or a single step: the 32-128 row tiles only
     const int tile = tile_for(f, rows);
-    return tile == 256 || (tile == 0 && rows > 384 && !split_preferred_to_big(f, rows));
+    if (tile == 256) return true;
+    if (tile != 0 || rows <= 384 || split_preferred_to_big(f, rows)) return false;
+    const bool decodes_once = f.takes_workspace && (f.flags2 & kNoExpand) == 0;
+    if (f.flags == kQ4 && !decodes_once) return tall_beats_whole_tiles(f, rows);
+    return true;
 }
 
 // Two-stage weights are decoded once into the handle's scratch and multiplied by the int8 kernel

@@ -155,7 +155,11 @@ def test_dynamic_geometry_follows_live_rows():
     one, many, big = kernel.geometry(1), kernel.geometry(64), lib.Kernel(
         "e8p_q4_projection", M=512, N=9728, K=2560, dynamic_rows=True).geometry(512)
     assert one != many                        # batch-1 and batch-64 take different kernels
-    assert big[0][0] * big[0][1] * big[0][2] == 2 * 38
+    # no scratch: 76 tall tiles (512 x 128, decode in the loop) would be one round of 87 us-per-5120-K, the 304 whole
+    # 128 x 128 tiles are a little faster at this size; at N = 17408 the tall tiles win
+    assert big[0][0] * big[0][1] * big[0][2] == 76 * 4 and big[1] == (256, 1, 1)
+    tall = lib.Kernel("e8p_q4_projection", M=512, N=17408, K=5120, dynamic_rows=True).geometry(512)
+    assert tall[0] == (136, 1, 1) and tall[1] == (512, 1, 1)
     with pytest.raises(lib.OrxError) as err:
         kernel.geometry(65)
     assert err.value.code == lib.ORX_ERR_ROWS
