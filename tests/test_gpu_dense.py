@@ -1076,6 +1076,20 @@ def test_config1_full_size_bit_exact(rows):
     np.testing.assert_array_equal(gu.host(out), want)
 
 
+def test_config1_full_size_512_rows_without_scratch():
+    """The same 512 rows through a handle without a Workspace: 512 x 128 tiles with the decode in the K loop, K-major
+    codes as the package stores them, against the oracle on every row."""
+    c = workloads.config1(512)
+    a_q, a_s = gu.a8(gu.dev(c["x"]))
+    wq, ws = orc.a8(c["x"])
+    stored = orc.q4_pack_k(c["packed"], 128)
+    kern = gu.lib.Kernel("e8p_q4_projection", M=512, N=c["n"], K=c["k"], packed_k=128)
+    assert kern.geometry(512)[1] == (512, 1, 1) and kern.geometry(512)[0] == (c["n"] // 128, 1, 1)
+    out = torch.empty((512, c["n"]), dtype=torch.float16, device=gu.DEV)
+    kern(A=a_q, AS=a_s, Book=gu.book(), Out=out, S=gu.dev(c["scales"]), W=gu.dev(stored))
+    np.testing.assert_array_equal(gu.host(out), orc.project(wq, ws[:, 0], _config1_weights(c), c["scales"]))
+
+
 _weights_cache = {}
 
 
