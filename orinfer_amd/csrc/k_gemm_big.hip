@@ -444,14 +444,13 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
     wait_direct_loads();
 }
 
-// ---- two-stage codes, up to 512 rows: 512 x 128 tiles with the decode in the K loop ----------------------------
-// Between 385 and 512 rows the 256 x 256 tiles need the weights decoded once into scratch first (1.5 bytes of HBM
-// traffic per weight, a launch of its own) and then leave half the CUs idle at N = 17408; decoding inside those
-// tiles instead repeats the decode for every row tile.  A tile of 512 token rows x 128 channels holds the same
-// multiplies per workgroup, decodes every weight once, and needs no scratch.  The price is LDS: 512 rows of a
-// 128-byte K step would be 64 KiB per stage, so the K step here is one MFMA slice of 64: three stages of token
-// rows (32 KiB each, requested two steps ahead with direct-to-LDS loads), two stages of decoded weights (8 KiB),
-// the byte tables and the tile's scales.
+// ---- two-stage codes without scratch: 512 x 128 tiles with the decode in the K loop ----------------------------
+// From 385 rows on the 256 x 256 tiles need the weights decoded once into scratch first (1.5 bytes of HBM traffic
+// per weight, a launch of its own); decoding inside those tiles instead repeats the decode for every 256 rows.  A
+// tile of 512 token rows x 128 channels holds the same multiplies per workgroup, decodes every weight once per 512
+// rows, and needs no scratch.  The price is LDS: 512 rows of a 128-byte K step would be 64 KiB per stage, so the K
+// step here is one MFMA slice of 64: three stages of token rows (32 KiB each, requested two steps ahead with
+// direct-to-LDS loads), three stages of decoded weights (8 KiB each), the byte tables and the tile's scales.
 //
 // Eight waves, 4 x 2, of 128 token rows x 64 channels each (the wave tile, fragment layout and epilogue of the
 // persistent kernel above).  A thread owns one 16-byte chunk of the decoded weight stage per step: channel
@@ -459,10 +458,11 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
 // and quarter for a K block of 128 (two steps) in registers, a second set for the block after it.
 //
 // Step s:   read the token fragments of the step's second half; wait for the first half and the weights;
-//           16 multiplies, with the requests for step s + 2 (and, in odd steps, the codes two blocks ahead) between
-//           them; eight table lookups for step s + 1's weights, combined and written while the multiplies run;
-//           barrier (step s + 1's token rows have landed, its weights are written, nobody reads what step s + 2's
-//           requests overwrite); read the first fragments of step s + 1; the other 16 multiplies.
+//           16 multiplies, with the requests for the token rows of step s + 2 (and, in even steps, the codes two
+//           blocks ahead) between them; barrier (step s + 1's token rows have landed, its weights were written a
+//           step ago, nobody reads what step s + 2's requests and weights overwrite); read the first fragments of
+//           step s + 1; eight table lookups for the weights of step s + 2; the other 16 multiplies; the lookups
+//           combined and written.
 // Every LDS access of the loop is an asm statement with hand-placed waits: the compiler would wait for all
 // direct-to-LDS requests in flight before any LDS access it can see.
 constexpr int kTallRows = 512, kTallCols = 128, kTallStep = 64, kTallThreads = 512, kTallStagesA = 3;
