@@ -65,6 +65,7 @@ void gemm_big_geometry(int rows, int n, Geometry* g);
 int q4_expand_launch(const void* codes, const uint32_t* book, void* weights, int n, int k, int packed_k,
                      hipStream_t stream);
 void gemm_tall_geometry(int rows, int n, Geometry* g);
+uint32_t gemm_tall_units(int n);
 int gemm_tall_launch(const int8_t* a, const void* w, const uint32_t* book, const __half* ws, const __half* as, void* out,
                      int rows, int n, int k, int stride, int packed_k, bool out_f32, const Geometry& g, hipStream_t stream);
 int gemm_big_launch(const int8_t* a, const void* w, const __half* ws, const __half* as, void* out, int rows, int n,
@@ -708,9 +709,25 @@ bool use_wide(const orx_function& f, int rows) {
     return rows >= 33 && rows <= 64 && (int64_t)f.N * f.K >= ((int64_t)1 << 26) && f.N <= 96 * device_compute_units();
 }
 
-// 512 x 128 tiles with the decode in the K loop (k_gemm_big.hip): `algorithm=tall` by name
+// Two-stage codes on 512 rows x channel runs with the decode in the K loop (k_gemm_big.hip): `algorithm=tall` by
+// name, and `auto` from 257 to 512 rows, with or without scratch, when the runs fill their five blocks of 16
+// channels well enough.  A launch costs 0.76 us per 64 of K and round of the CUs whatever N is (every CU reads all
+// token rows), so it pays when the matrix gives every CU enough channels.  Measured against the kernels `auto` had
+// at 384 / 512 rows (128 x 128 tiles / decode once + 256 x 256 tiles; us, 256 CUs): N x K = 17408 x 5120 (4.25
+// blocks per CU) 64 / 66 against 77 / 86, 34816 x 5120 (two rounds of 4.25) 131 / 135 against 142 / 158,
+// 14336 x 4096 (3.5) 52 / 53 against 64 / 65, 12288 x 3072 (3) 41 / 42 against 46 / 55, 9728 x 2560 (2.4) 35 / 34
+// against 40 / 44; 7168 x 5120 (1.75) 59 / 59 against 44 / 51, 28672 x 8192 (two rounds of 3.5) 189 / 194 against
+// 158 / 194.  Up to 256 rows the split 128 x 128 tiles tie or win (60-63 against 62-65 at config 1's shape).
+bool tall_runs_fill(int n) {
+    const int64_t blocks = ceil_div((uint32_t)n, 16u), cus = device_compute_units();
+    const int64_t rounds = (blocks + 5 * cus - 1) / (5 * cus);
+    return rounds == 1 ? 4 * blocks >= 9 * cus : blocks >= 4 * rounds * cus;
+}
 bool use_tall(const orx_function& f, int rows) {
-    return f.flags == kQ4 && f.algorithm == kTall;
+    if (f.flags != kQ4) return false;
+    if (f.algorithm == kTall) return true;
+    if (f.algorithm != kAuto || tile_for(f, rows) != 0 || f.K % 128 != 0 || f.K < 256) return false;
+    return rows > 256 && rows <= 512 && tall_runs_fill(f.N);
 }
 
 bool use_resident(const orx_function& f, int rows);
@@ -762,15 +779,15 @@ bool use_resident(const orx_function& f, int rows) {
 // K=5120 against 86..93 us for decode-once + 256x256, and 54..60 us against 58..62 us for W8; at 512
 // rows the 256x256 kernel wins, 92 against 104 us and 61 against 79 us)
 bool split_preferred_to_big(const orx_function& f, int rows);
-// Two-stage codes without scratch: 512 x 128 tiles with the decode in the K loop against whole 128 x 128 tiles, which
+// Two-stage codes above 384 rows without scratch: the 512-row channel runs against whole 128 x 128 tiles, which
 // decode every weight once per 128 rows but come four to the 512 rows.  Measured at K = 5120 (times scale with K):
-// the tall tiles take 87 us per round of the CUs (N = 17408: 91 / 172 / 263 us at 512 / 1024 / 2048 rows), the small
-// ones 40 us + 32 us per tile and CU (105 / 171 / 314 us); N = 5120: 86 / 87 / 88 against 57 / 78 / 107 us.
+// the runs take 66 us per row tile and round of the CUs (N = 17408: 66 / 124 / 132 us at 512 / 768 / 1024 rows),
+// the small tiles 40 us + 32 us per tile and CU (105 / 141 / 171 us); N = 5120: 61 / 113 / 113 against 55 / 56 / 77 us.
 bool tall_beats_whole_tiles(const orx_function& f, int rows) {
     const int64_t cus = device_compute_units();
-    const int64_t columns = ceil_div((uint32_t)f.N, 128u);
-    const int64_t tall = columns * ceil_div((uint32_t)rows, 512u), small = columns * ceil_div((uint32_t)rows, 128u);
-    return 87 * ((tall + cus - 1) / cus) * cus < 40 * cus + 32 * small;
+    const int64_t tall = (int64_t)gemm_tall_units(f.N) * ceil_div((uint32_t)rows, 512u);
+    const int64_t small = (int64_t)ceil_div((uint32_t)f.N, 128u) * ceil_div((uint32_t)rows, 128u);
+    return 66 * ((tall + cus - 1) / cus) * cus < 40 * cus + 32 * small;
 }
 bool use_big(const orx_function& f, int rows) {
     if (f.K % kBK || f.K < 2 * kBK) return false;  // half a K step at the end, or a single step: the 32-128 row tiles only
@@ -896,7 +913,7 @@ int projection_geometry(const orx_function& f, int rows, Geometry* g) {
         return ORX_OK;
     }
     if (use_big(f, rows)) {
-        if (f.flags == kQ4 && !use_expand(f, rows))  // decode in the K loop: the 512 x 128 tiles
+        if (f.flags == kQ4 && !use_expand(f, rows))  // decode in the K loop: the 512-row channel runs
             gemm_tall_geometry(rows, f.N, g);
         else
             gemm_big_geometry(rows, big_main_channels(f, rows), g);

@@ -6,12 +6,13 @@
 // then (float(acc)*ws)*as.
 //
 // Two kernels.  int8 weights (W8A8, and two-stage weights that q4_expand_kernel has decoded once into the
-// caller's scratch): gemm_big_persistent_kernel, one workgroup per CU walking 256 x 256 tiles.  Two-stage codes
-// without scratch: gemm_q4_tall_kernel, 512 x 128 tiles with the decode in the K loop.  In both, eight wave64
-// (2 per SIMD) share a tile, each owning 128 token rows x 64 channels as 8 x 4 blocks of v_mfma_i32_16x16x64_i8
-// (128 accumulator registers); int8 operands that already exist in HBM go HBM -> LDS directly with
-// global_load_lds_dwordx4, without touching VGPRs, and the 16-byte chunk a lane fetches is XOR-swizzled with its
-// row so that the later ds_read_b128 fragment reads of sixteen consecutive rows fall in different bank groups.
+// caller's scratch): gemm_big_persistent_kernel, one workgroup per CU walking 256 x 256 tiles, eight wave64 of
+// 128 token rows x 64 channels each.  Two-stage codes without scratch: gemm_q4_tall_kernel, 512 token rows x a run
+// of up to 80 channels per workgroup with the decode in the K loop, eight wave64 of 64 rows x the run.  Both
+// multiply with v_mfma_i32_16x16x64_i8 from two waves per SIMD; int8 operands that already exist in HBM go
+// HBM -> LDS directly with global_load_lds_dwordx4, without touching VGPRs, and the 16-byte chunk a lane fetches is
+// XOR-swizzled with its row so that the later ds_read_b128 fragment reads of sixteen consecutive rows fall in
+// different bank groups.
 #include <hip/hip_fp16.h>
 
 #include <type_traits>
@@ -444,40 +445,52 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
     wait_direct_loads();
 }
 
-// ---- two-stage codes without scratch: 512 x 128 tiles with the decode in the K loop ----------------------------
-// From 385 rows on the 256 x 256 tiles need the weights decoded once into scratch first (1.5 bytes of HBM traffic
-// per weight, a launch of its own); decoding inside those tiles instead repeats the decode for every 256 rows.  A
-// tile of 512 token rows x 128 channels holds the same multiplies per workgroup, decodes every weight once per 512
-// rows, and needs no scratch.  The price is LDS: 512 rows of a 128-byte K step would be 64 KiB per stage, so the K
-// step here is one MFMA slice of 64: three stages of token rows (32 KiB each, requested two steps ahead with
-// direct-to-LDS loads), three stages of decoded weights (8 KiB each), the byte tables and the tile's scales.
+// ---- two-stage codes without scratch: 512 rows x a run of channels, the decode in the K loop ---------------------
+// From 257 rows on the other kernels either decode every weight once per 128- or 256-row tile, or need the weights
+// decoded once into scratch first (1.5 bytes of HBM traffic per weight, a launch of its own).  Here a workgroup owns
+// up to 512 token rows and a run of at most five blocks of 16 channels over the whole K; the blocks of the matrix
+// are dealt evenly to whole rounds of the CUs (N = 17408 on 256 CUs: 1088 blocks, 4 or 5 per workgroup, one
+// round), so every weight is decoded once per 512 rows and nothing goes through scratch.
 //
-// Eight waves, 4 x 2, of 128 token rows x 64 channels each (the wave tile, fragment layout and epilogue of the
-// persistent kernel above).  A thread owns one 16-byte chunk of the decoded weight stage per step: channel
-// tid / 4, K bytes [16 (tid % 4), +16) of the slice, i.e. two code words; it holds the four words of its channel
-// and quarter for a K block of 128 (two steps) in registers, a second set for the block after it.
-//
-// Step s:   read the token fragments of the step's second half; wait for the first half and the weights;
-//           16 multiplies, with the requests for the token rows of step s + 2 (and, in even steps, the codes two
-//           blocks ahead) between them; barrier (step s + 1's token rows have landed, its weights were written a
-//           step ago, nobody reads what step s + 2's requests and weights overwrite); read the first fragments of
-//           step s + 1; eight table lookups for the weights of step s + 2; the other 16 multiplies; the lookups
-//           combined and written.
-// Every LDS access of the loop is an asm statement with hand-placed waits: the compiler would wait for all
-// direct-to-LDS requests in flight before any LDS access it can see.
-constexpr int kTallRows = 512, kTallCols = 128, kTallStep = 64, kTallThreads = 512, kTallStagesA = 3;
-constexpr uint32_t kTallStageA = kTallRows * kTallStep, kTallStageW = kTallCols * kTallStep;
-constexpr uint32_t kTallWeights = kTallStagesA * kTallStageA;          // byte offsets in dynamic LDS
-constexpr uint32_t kTallTables = kTallWeights + kTallStagesA * kTallStageW;
-constexpr uint32_t kTallScales = kTallTables + (uint32_t)sizeof(Q4ByteTables);
+// Eight waves; wave w owns token rows [64 w, +64) and all channels of the run: 4 x 5 blocks of
+// v_mfma_i32_16x16x64_i8 (80 accumulator registers), weights as the row operand, so a lane holds four consecutive
+// channels of one token.  K advances in MFMA slices of 64.
+//   token rows   two slots of 512 rows x 128 bytes of K (64 KiB each): a wave requests its own 64 rows of a K chunk
+//                of 128 with eight direct-to-LDS loads of 8 rows x 128 bytes, whole cache lines (requests of half
+//                lines, one 64-byte slice per step, cost twice the traffic between L2 and the CU: the other half
+//                of a line has left the L1 by the next step).  Nobody but the wave itself reads those rows, so
+//                they need no barrier, only the wave's own wait.
+//   weights      a thread of the first five waves owns one 16-byte chunk of the decoded stage per step (channel
+//                tid / 4, K bytes [16 (tid % 4), +16) of the slice: two code words); it holds the four words of
+//                its channel and quarter for a K block of 128 in registers, a second set for the block after it.
+//                Every code word costs four 4-byte lookups (biased nibbles of the basis row, sign mask, for either
+//                stage; tables of 1 KiB each) and a few byte-parallel operations.  Four stages of 5 KiB.
+//   step s       the fragments of step s are in registers on entry.  Between its 20 multiplies the wave issues the
+//                eight lookups for the weights of step s + 2, the nine fragment reads of step s + 1, in odd steps
+//                the eight requests for the token rows of steps s + 3 and s + 4 (the slot that steps s - 1 and s
+//                have left), then combines the lookups and writes its chunk; in even steps it requests the codes
+//                two blocks ahead (every wave does, so that all count the same requests).  One barrier per step
+//                publishes the decoded stage.
+// All LDS traffic and the code loads of the loop are asm statements with hand-placed waits: the compiler would
+// wait for every direct-to-LDS request in flight before an LDS access it can see.  The loop is bound by the LDS
+// pipe (per step and CU: 72 fragment reads of 1 KiB, 32 KiB of token rows landing, 40 wave lookups, 5 KiB written)
+// at about 70 % of its rate, above the floor that the token rows set (every CU reads all rows once: 2.6 MB per CU
+// at 512 x 5120, which 256 CUs together pull out of the L2 in 37 us).
+constexpr int kTallBlocks = 5;  // blocks of 16 channels per workgroup, at most
+constexpr int kTallRows = 512, kTallCols = 16 * kTallBlocks, kTallStep = 64, kTallThreads = 512, kTallStagesW = 4;
+constexpr uint32_t kTallSlotA = kTallRows * 128;  // token rows of a K chunk of 128
+constexpr uint32_t kTallStageW = kTallCols * kTallStep;
+constexpr uint32_t kTallWeights = 2 * kTallSlotA;  // byte offsets in dynamic LDS
+constexpr uint32_t kTallTables = kTallWeights + kTallStagesW * kTallStageW;
+constexpr uint32_t kTallScales = kTallTables + 2048;  // nib[256], msk[256]
 constexpr uint32_t kTallLds = kTallScales + (kTallRows + kTallCols) * 4;
 
 typedef unsigned int v2w __attribute__((ext_vector_type(2)));
 
 template <int OFFSET>
-__device__ __forceinline__ v2w lds_read_8(uint32_t lds_address) {
-    v2w value;
-    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
+__device__ __forceinline__ uint32_t lds_read_4(uint32_t lds_address) {
+    uint32_t value;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
     return value;
 }
 // 8 bytes from global memory that the compiler keeps no count for: whoever uses them waits by hand
@@ -496,14 +509,18 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     extern __shared__ __align__(16) int8_t lds[];
     float* const lds_as = reinterpret_cast<float*>(lds + kTallScales);
     float* const lds_ws = lds_as + kTallRows;
-    Q4ByteTables* const tables = reinterpret_cast<Q4ByteTables*>(lds + kTallTables);
+    uint32_t* const nib = reinterpret_cast<uint32_t*>(lds + kTallTables);  // biased nibbles of the basis rows, then the sign masks
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave_m = wave >> 1, wave_n = wave & 1;
-    const int tn = (int)blockIdx.x % p.tiles_n, tm = (int)blockIdx.x / p.tiles_n;
+    // unit u of a row tile owns the channel blocks [u B / U, (u + 1) B / U) of the B blocks of 16 channels
+    const int unit = (int)blockIdx.x % p.tiles_n, tm = (int)blockIdx.x / p.tiles_n;
+    const int channel_blocks = (p.n + 15) >> 4;
+    const int first_block = (int)((int64_t)unit * channel_blocks / p.tiles_n);
+    const int end_block = (int)((int64_t)(unit + 1) * channel_blocks / p.tiles_n);
     TileState t;
-    t.row0 = tm * kTallRows, t.col0 = tn * kTallCols;
-    t.rows_here = min(kTallRows, p.m - t.row0), t.cols_here = min(kTallCols, p.n - t.col0);
+    t.row0 = tm * kTallRows, t.col0 = first_block * 16;
+    t.rows_here = min(kTallRows, p.m - t.row0), t.cols_here = min((end_block - first_block) * 16, p.n - t.col0);
+    const bool decoder = wave < kTallBlocks;  // threads 0 .. 64 blocks - 1 own the chunks of the weight stage
     const int steps = p.k / kTallStep, blocks = p.k / 128;
     const uint32_t lds_base = lds_address_of(lds);
 
@@ -511,8 +528,8 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     const int channel = tid >> 2, quarter = tid & 3;
     const int code_row = t.col0 + min(channel, t.cols_here - 1);
     // The loads are asm statements: the compiler then keeps no count for them, and the waits in front of the barriers
-    // (which let only the current step's requests stay in flight) are what guarantees that a set has arrived two
-    // steps after it was requested.  Sets and halves are compile-time indices everywhere, so that no select or copy
+    // (which let only the youngest requests stay in flight) are what guarantees that a set has arrived two steps
+    // after it was requested.  Sets and halves are compile-time indices everywhere, so that no select or copy
     // touches a register whose load is still in flight.
     v2w codes[2][2];  // [set][half of the K block]
     // address = uniform base of the K block (+ uniform step to its second half) + a lane offset, for all three layouts:
@@ -531,141 +548,174 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     load_codes(1, std::integral_constant<int, 1>{});
 
     // ---- tables and scales, written before any direct-to-LDS request is in flight ----
-    build_tables(*tables, p.book, tid, kTallThreads);
+    if (tid < 256) nib[tid] = nibble_basis_word(p.book[tid], 8u), nib[256 + tid] = nibble_mask_word((uint32_t)tid);
     lds_as[tid] = __half2float(p.as[t.row0 + min(tid, t.rows_here - 1)]);
     if (tid < kTallCols) lds_ws[tid] = __half2float(p.ws[t.col0 + min(tid, t.cols_here - 1)]);
     __syncthreads();
 
-    // ---- token rows: a wave requests rows [64 wave, +64) of a step, four 1 KiB blocks of 16 rows ----
-    const int load_row = wave * 64 + (lane >> 2);
-    const uint32_t load_chunk = (uint32_t)(((lane & 3) ^ ((lane >> 4) & 3)) * 16);  // (row / 4) % 4 = (lane / 16) % 4 in every block
+    // ---- token rows: K chunks of 128 (whole cache lines), two slots of 512 rows x 128 bytes; a wave requests its own
+    // rows [64 wave, +64) of a chunk as eight 1 KiB blocks of 8 rows; 16-byte piece c of row r sits at position
+    // c ^ ((r / 2) % 8) of the row, as in the persistent kernel ----
+    const int load_row = wave * 64 + (lane >> 3);
+    const uint32_t load_chunk = (uint32_t)(((lane & 7) ^ swizzle(load_row)) * 16);
     const int8_t* const a_base = uniform_pointer(p.a + (int64_t)t.row0 * p.k);
-    auto issue_tokens = [&](int b, int step, int stage) {
+    auto issue_tokens = [&](int b, int chunk, int slot) {
         int row = load_row;
         asm volatile("" : "+v"(row));  // or every request's offset is kept in a register for the whole loop
-        const uint32_t offset = (uint32_t)(min(row + 16 * b, t.rows_here - 1) * p.k) + load_chunk;
-        direct_load_16(a_base + min(step, steps - 1) * kTallStep + (uint64_t)offset,
-                       lds + stage * kTallStageA + (wave * 4 + b) * 1024);
+        const uint32_t offset = (uint32_t)(min(row + 8 * b, t.rows_here - 1) * p.k) + (load_chunk ^ (uint32_t)((b & 1) * 64));
+        direct_load_16(a_base + min(chunk, blocks - 1) * 128 + (uint64_t)offset, lds + slot * kTallSlotA + (wave * 8 + b) * 1024);
     };
 
     // ---- fragments: a lane reads K bytes [16 (lane / 16), +16) of the slice for row lane % 16 of a block ----
     const int frag_row = lane & 15, frag_chunk = lane >> 4;
-    const uint32_t frag_offset = (uint32_t)(frag_row * kTallStep + ((frag_chunk ^ tall_swizzle(frag_row)) * 16));
-    const uint32_t a_frag = lds_base + wave_m * 128 * kTallStep + frag_offset;
-    const uint32_t w_frag = lds_base + kTallWeights + wave_n * 64 * kTallStep + frag_offset;
-    v4i ft[2][4], fw[2][4];  // token fragments of a step's halves; weight fragments of even and odd steps
+    const uint32_t a_frag = lds_base + (wave * 64 + frag_row) * 128 + ((frag_chunk ^ swizzle(frag_row)) * 16);
+    const uint32_t w_frag = lds_base + kTallWeights + (uint32_t)(frag_row * kTallStep + ((frag_chunk ^ tall_swizzle(frag_row)) * 16));
+    v4i ft[2][4], fw[2][kTallBlocks];  // token and weight fragments of even and odd steps
     constexpr int kBlock = 16 * kTallStep;
-    auto read_tokens = [&](int stage, int half) {
-        const uint32_t a = a_frag + stage * kTallStageA + half * 4 * kBlock;
-        v4i(&f)[4] = ft[half];
+    // slice step % 2 of chunk step / 2, which sits in slot (step / 2) % 2; the second slice of a row is the first
+    // with address bit 6 flipped (piece 4 + c swizzles to the position of piece c with bit 2 flipped)
+    auto read_tokens = [&](int step, int parity) {
+        const uint32_t a = (a_frag ^ (uint32_t)((step & 1) * 64)) + ((step >> 1) & 1) * kTallSlotA;
+        v4i(&f)[4] = ft[parity];
         f[0] = lds_read_16<0>(a);
-        f[1] = lds_read_16<kBlock>(a);
-        f[2] = lds_read_16<2 * kBlock>(a);
-        f[3] = lds_read_16<3 * kBlock>(a);
+        f[1] = lds_read_16<2048>(a);
+        f[2] = lds_read_16<4096>(a);
+        f[3] = lds_read_16<6144>(a);
     };
     auto read_weights = [&](int stage, int parity) {  // register set by the parity of the step
         const uint32_t w = w_frag + stage * kTallStageW;
-        v4i(&f)[4] = fw[parity];
+        v4i(&f)[kTallBlocks] = fw[parity];
         f[0] = lds_read_16<0>(w);
         f[1] = lds_read_16<kBlock>(w);
         f[2] = lds_read_16<2 * kBlock>(w);
         f[3] = lds_read_16<3 * kBlock>(w);
+        f[4] = lds_read_16<4 * kBlock>(w);
     };
 
     // ---- decode: this thread's chunk of a weight stage ----
     const uint32_t table_base = lds_base + kTallTables;
     const uint32_t write_offset = kTallWeights + (uint32_t)(channel * kTallStep + ((quarter ^ tall_swizzle(channel)) * 16));
-    v2w looked[8];
-    auto lookups = [&](v2w pair) {  // two code words: basis0, mask0, basis1, mask1 of each
+    uint32_t looked[8];
+    auto lookups = [&](v2w pair) {  // two code words: nibbles and signs of either stage
         asm volatile("" : "+v"(pair));  // nothing computed from the words moves above this point
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t code = pair[i];
-            looked[4 * i + 0] = lds_read_8<0>(table_base + ((code >> 5) & 0x7F8u));       // basis0[(code >> 8) & 255]
-            looked[4 * i + 1] = lds_read_8<2048>(table_base + ((code << 3) & 0x7F8u));    // mask0[code & 255]
-            looked[4 * i + 2] = lds_read_8<4096>(table_base + ((code >> 21) & 0x7F8u));   // basis1[code >> 24]
-            looked[4 * i + 3] = lds_read_8<6144>(table_base + ((code >> 13) & 0x7F8u));   // mask1[(code >> 16) & 255]
+            looked[4 * i + 0] = lds_read_4<0>(table_base + ((code >> 6) & 0x3FCu));       // nib[(code >> 8) & 255]
+            looked[4 * i + 1] = lds_read_4<1024>(table_base + ((code << 2) & 0x3FCu));    // msk[code & 255]
+            looked[4 * i + 2] = lds_read_4<0>(table_base + ((code >> 22) & 0x3FCu));      // nib[code >> 24]
+            looked[4 * i + 3] = lds_read_4<1024>(table_base + ((code >> 14) & 0x3FCu));   // msk[(code >> 16) & 255]
         }
     };
-    auto write_decoded = [&](int stage) {
-        // every LDS request of this wave has returned (the lookups are the youngest)
+    v4u chunk;
+    // (LDS requests of a wave return in order)
+    auto wait_lookups = [&]() {
         asm volatile("s_waitcnt lgkmcnt(0)"
                      : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
                        "+v"(looked[6]), "+v"(looked[7]));
-        v4u chunk;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            chunk[2 * i + 0] = ((looked[4 * i][0] ^ looked[4 * i + 1][0]) + (looked[4 * i + 2][0] ^ looked[4 * i + 3][0]) + 0x35353535u) ^ 0x80808080u;
-            chunk[2 * i + 1] = ((looked[4 * i][1] ^ looked[4 * i + 1][1]) + (looked[4 * i + 2][1] ^ looked[4 * i + 3][1]) + 0x35353535u) ^ 0x80808080u;
-        }
-        lds_write_16(lds_base + write_offset + stage * kTallStageW, chunk);
+    };
+    auto wait_lookups_before_fragments = [&]() {  // the 9 fragment reads of a step are younger
+        asm volatile("s_waitcnt lgkmcnt(9)"
+                     : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
+                       "+v"(looked[6]), "+v"(looked[7]));
+    };
+    // code word i -> 8 weights.  x0, x1: v + 8 of either stage in the nibbles (coordinates 0..3 in the low nibbles of
+    // the bytes, 4..7 in the high ones); w + 128 = 8 (v0 + 8) + 2 (v1 + 8) + 53 in every byte, in [73, 183]: no carry
+    // between bytes, and the XOR turns offset binary into two's complement (what decode_q4 computes from byte tables)
+    auto combine = [&](int i) {
+        const uint32_t x0 = looked[4 * i] ^ looked[4 * i + 1], x1 = looked[4 * i + 2] ^ looked[4 * i + 3];
+        chunk[2 * i + 0] = (((x0 << 3) & 0x78787878u) + ((x1 << 1) & 0x1E1E1E1Eu) + 0x35353535u) ^ 0x80808080u;
+        chunk[2 * i + 1] = (((x0 >> 1) & 0x78787878u) + ((x1 >> 3) & 0x1E1E1E1Eu) + 0x35353535u) ^ 0x80808080u;
+    };
+    auto write_chunk = [&](int stage) { lds_write_16(lds_base + write_offset + stage * kTallStageW, chunk); };
+    auto write_decoded = [&](int stage) {
+        wait_lookups();
+        combine(0);
+        combine(1);
+        write_chunk(stage);
     };
 
-    v4i acc[8][4];
+    v4i acc[4][kTallBlocks];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = v4i{0, 0, 0, 0};
-    auto multiply = [&](int half, int parity, auto between) {
+        for (int j = 0; j < kTallBlocks; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    // 4 x 5 multiplies of a step, one operand changing between consecutive instructions
+    auto multiply = [&](int parity, auto between) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int jj = (i & 1) ? 3 - j : j;
-                v4i& sum = acc[4 * half + i][jj];
-                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[parity][jj], ft[half][i], sum, 0, 0, 0);
-                between(i * 4 + j);
+            for (int j = 0; j < kTallBlocks; ++j) {
+                const int jj = (i & 1) ? kTallBlocks - 1 - j : j;
+                v4i& sum = acc[i][jj];
+                sum = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[parity][jj], ft[parity][i], sum, 0, 0, 0);
+                between(i * kTallBlocks + j);
             }
     };
 
-    // ---- prologue: steps 0 and 1 requested, their weights decoded (block 0), step 0's first fragments read ----
+    // ---- prologue: K chunks 0 and 1 requested, the weights of steps 0 and 1 decoded (block 0), step 0's fragments read ----
 #pragma unroll
-    for (int b = 0; b < 4; ++b) issue_tokens(b, 0, 0);
+    for (int b = 0; b < 8; ++b) issue_tokens(b, 0, 0);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) issue_tokens(b, 1, 1);
-    asm volatile("s_waitcnt vmcnt(8)" : "+v"(codes[0][0]), "+v"(codes[0][1]), "+v"(codes[1][0]), "+v"(codes[1][1]));
-    lookups(codes[0][0]);
-    write_decoded(0);
-    lookups(codes[0][1]);
-    write_decoded(1);
-    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int b = 0; b < 8; ++b) issue_tokens(b, 1, 1);
+    asm volatile("s_waitcnt vmcnt(16)" : "+v"(codes[0][0]), "+v"(codes[0][1]), "+v"(codes[1][0]), "+v"(codes[1][1]));
+    if (decoder) {
+        lookups(codes[0][0]);
+        write_decoded(0);
+        lookups(codes[0][1]);
+        write_decoded(1);
+    }
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     read_tokens(0, 0);
     read_weights(0, 0);
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]),
+                   "+v"(fw[0][3]), "+v"(fw[0][4])
+                 :
+                 : "memory");
 
-    // One step.  The weights are decoded two steps ahead, behind the barrier: step s writes the stage of step s + 2
-    // (block (s + 2) / 2, held in set ((s + 2) / 2) % 2; an even step decodes the first half of the next block, an odd
-    // step the second half of the same), its lookups issued in front of the second 16 multiplies and combined behind
-    // them, so that no table latency stands between a multiply and a barrier.  Even steps also request the codes of
-    // block s / 2 + 2 into the set that block s / 2 has just left.  The waits name how many younger requests may
-    // stay in flight: vector memory retires in order, and this step's 4 token requests (and the 2 code requests of
-    // an even step) are younger than step s + 1's rows.
+    // Step s.  On entry the fragments of step s are in registers, the rows of step s + 1 (this wave's own requests)
+    // have landed and its weights were written in front of the last barrier.  Everything else of the step sits
+    // between its 20 multiplies, so that the matrix pipe works while the LDS pipe and the vector ALU serve the rest:
+    // the lookups for the weights of step s + 2 first, then the fragment reads of step s + 1 (so the lookups return
+    // first), the row requests of an odd step, and behind the tenth multiply the lookups combined and written.
+    // K chunk c (steps 2 c, 2 c + 1) is requested in step 2 c - 3 into the slot that chunk c - 2 left when step
+    // 2 c - 4 read its last fragments, and has two steps to land.  The wait in front of the barrier names how many
+    // younger requests may stay in flight (vector memory retires in order): behind an even step its 2 code requests,
+    // behind an odd step its 8 row requests.
     auto step = [&](int s, auto set_tag, auto odd_tag) {
         constexpr int SET = decltype(set_tag)::value, ODD = decltype(odd_tag)::value;  // SET: of the block being decoded
-        const int stage = s % kTallStagesA, next_stage = (s + 1) % kTallStagesA, load_stage = (s + 2) % kTallStagesA;
-        read_tokens(stage, 1);                                // 4 younger requests than the first half and the weights
-        wait_eight<4>(ft[0], fw[ODD]);
+        const int next_stage = (s + 1) % kTallStagesW, decode_stage = (s + 2) % kTallStagesW;
         __builtin_amdgcn_sched_barrier(0);
-        multiply(0, ODD, [&](int index) {
-            if ((index & 3) == 3) {
-                __builtin_amdgcn_sched_barrier(0);
-                issue_tokens(index >> 2, s + 2, load_stage);
-                __builtin_amdgcn_sched_barrier(0);
+        multiply(ODD, [&](int index) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (index == 0 && decoder) lookups(codes[SET][ODD]);
+            if (index == 2) read_tokens(s + 1, 1 - ODD);
+            if (index == 4) read_weights(next_stage, 1 - ODD);
+            if (ODD && (index & 1) == 1 && index < 16)  // chunk (s + 3) / 2 into the slot that chunk (s - 1) / 2 has left
+                issue_tokens(index >> 1, (s + 3) >> 1, ((s + 3) >> 1) & 1);
+            if (index >= 10 && index <= 14 && (index & 1) == 0 && decoder) {
+                if (index == 10) wait_lookups_before_fragments();
+                if (index == 10) combine(0);
+                if (index == 12) combine(1);
+                if (index == 14) write_chunk(decode_stage);
             }
+            __builtin_amdgcn_sched_barrier(0);
         });
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!ODD) load_codes((s >> 1) + 2, std::integral_constant<int, 1 - SET>{});
-        wait_four<0>(ft[1]);
         if constexpr (!ODD)
-            asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(ft[1][0]), "+v"(ft[1][1]), "+v"(ft[1][2]), "+v"(ft[1][3]), "+v"(fw[1][0]), "+v"(fw[1][1]),
+                           "+v"(fw[1][2]), "+v"(fw[1][3]), "+v"(fw[1][4])
+                         :
+                         : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        read_tokens(next_stage, 0);
-        read_weights(next_stage, 1 - ODD);
-        lookups(codes[SET][ODD]);
-        __builtin_amdgcn_sched_barrier(0);
-        multiply(1, ODD, [](int) {});
-        __builtin_amdgcn_sched_barrier(0);
-        write_decoded(load_stage);
+            asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
+                         : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(fw[0][0]), "+v"(fw[0][1]),
+                           "+v"(fw[0][2]), "+v"(fw[0][3]), "+v"(fw[0][4])
+                         :
+                         : "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
     // steps 4 g .. 4 g + 3 decode blocks 2 g + 1 (set 1: steps 4 g, 4 g + 1) and 2 g + 2 (set 0: steps 4 g + 2, 4 g + 3)
@@ -688,27 +738,27 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     // data would land on whatever lives there by then.
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)"
                  : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(ft[1][0]), "+v"(ft[1][1]), "+v"(ft[1][2]),
-                   "+v"(ft[1][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]), "+v"(fw[0][3]), "+v"(fw[1][0]), "+v"(fw[1][1]),
-                   "+v"(fw[1][2]), "+v"(fw[1][3])
+                   "+v"(ft[1][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]), "+v"(fw[0][3]), "+v"(fw[0][4]), "+v"(fw[1][0]),
+                   "+v"(fw[1][1]), "+v"(fw[1][2]), "+v"(fw[1][3]), "+v"(fw[1][4])
                  :
                  : "memory");
     asm volatile("" : "+v"(codes[0][0]), "+v"(codes[0][1]), "+v"(codes[1][0]), "+v"(codes[1][1]));
 
-    // ---- epilogue: as in the persistent kernel, private to a wave and in registers ----
+    // ---- epilogue: private to a wave and in registers; a lane holds four consecutive channels of one token ----
     int own = threadIdx.x & 63;
     asm volatile("" : "+v"(own));
     const int group = own >> 4;
     if constexpr (F32) {
         const bool vector_ok = p.stride % 4 == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int local_row = wave_m * 128 + i * 16 + (own & 15);
+        for (int i = 0; i < 4; ++i) {
+            const int local_row = wave * 64 + i * 16 + (own & 15);
             if (local_row >= t.rows_here) continue;
             const int64_t row = t.row0 + local_row;
             const float token_scale = lds_as[local_row];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int local_col = wave_n * 64 + j * 16 + 4 * group;
+            for (int j = 0; j < kTallBlocks; ++j) {
+                const int local_col = j * 16 + 4 * group;
                 if (local_col >= t.cols_here) continue;
                 const int col = t.col0 + local_col;
                 const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
@@ -726,35 +776,53 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
         }
     } else {
         const bool aligned = (p.stride % 8 == 0) && ((reinterpret_cast<uintptr_t>(p.out) & 15) == 0);
-        const bool whole = aligned && t.rows_here == kTallRows && t.cols_here == kTallCols;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int local_row = wave_m * 128 + i * 16 + (own & 15);
+        for (int i = 0; i < 4; ++i) {
+            const int local_row = wave * 64 + i * 16 + (own & 15);
             const float token_scale = lds_as[local_row];
             __half* const row_out = reinterpret_cast<__half*>(p.out) + (int64_t)(t.row0 + local_row) * p.stride + t.col0;
+            // blocks 0..3 in pairs: a lane swap turns two 4-channel pieces into one of 8 channels (16 bytes)
 #pragma unroll
             for (int pair = 0; pair < 2; ++pair) {
                 uint32_t words[2][2];
 #pragma unroll
                 for (int b = 0; b < 2; ++b) {
                     const int j = 2 * pair + b;
-                    const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + wave_n * 64 + j * 16 + 4 * group);
+                    const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + j * 16 + 4 * group);
                     words[b][0] = pack_halves(rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale));
                     words[b][1] = pack_halves(rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale));
                 }
                 const v2u low = __builtin_amdgcn_permlane16_swap(words[0][0], words[1][0], false, false);
                 const v2u high = __builtin_amdgcn_permlane16_swap(words[0][1], words[1][1], false, false);
                 const uint4 piece = make_uint4(low.x, high.x, low.y, high.y);
-                const int local_col = wave_n * 64 + (2 * pair + (group & 1)) * 16 + (group >> 1) * 8;
-                if (whole) {
-                    *reinterpret_cast<uint4*>(row_out + local_col) = piece;
-                } else if (local_row < t.rows_here && local_col < t.cols_here) {
+                const int local_col = (2 * pair + (group & 1)) * 16 + (group >> 1) * 8;
+                if (local_row < t.rows_here && local_col < t.cols_here) {
                     if (aligned && local_col + 8 <= t.cols_here) {
                         *reinterpret_cast<uint4*>(row_out + local_col) = piece;
                     } else {
                         const uint32_t parts[4] = {piece.x, piece.y, piece.z, piece.w};
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
+                            if (local_col + e < t.cols_here)
+                                row_out[local_col + e] = __ushort_as_half((unsigned short)(parts[e >> 1] >> (16 * (e & 1))));
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // the fifth block: four channels (8 bytes) per lane
+            {
+                constexpr int j = kTallBlocks - 1;
+                const int local_col = j * 16 + 4 * group;
+                const float4 wscale = *reinterpret_cast<const float4*>(lds_ws + local_col);
+                const uint2 piece = make_uint2(pack_halves(rescale(acc[i][j][0], wscale.x, token_scale), rescale(acc[i][j][1], wscale.y, token_scale)),
+                                               pack_halves(rescale(acc[i][j][2], wscale.z, token_scale), rescale(acc[i][j][3], wscale.w, token_scale)));
+                if (local_row < t.rows_here && local_col < t.cols_here) {
+                    if (aligned && local_col + 4 <= t.cols_here) {
+                        *reinterpret_cast<uint2*>(row_out + local_col) = piece;
+                    } else {
+                        const uint32_t parts[2] = {piece.x, piece.y};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
                             if (local_col + e < t.cols_here)
                                 row_out[local_col + e] = __ushort_as_half((unsigned short)(parts[e >> 1] >> (16 * (e & 1))));
                     }
@@ -861,9 +929,16 @@ int gemm_big_launch(const int8_t* a, const void* w, const __half* ws, const __ha
     return hip_check(hipGetLastError(), "launch projection (mfma 256x256)");
 }
 
-// two-stage codes on 512 x 128 tiles with the decode in the K loop (K a multiple of 128)
+// Two-stage codes on 512 rows x channel runs with the decode in the K loop (K a multiple of 128).
+// Workgroups per row tile: the blocks of 16 channels are dealt evenly over whole rounds of the CUs, at most kTallBlocks
+// to a workgroup.
+uint32_t gemm_tall_units(int n) {
+    const uint32_t blocks = ceil_div((uint32_t)n, 16u), cus = (uint32_t)device_compute_units();
+    const uint32_t rounds = ceil_div(blocks, (uint32_t)kTallBlocks * cus);
+    return std::min(blocks, rounds * cus);
+}
 void gemm_tall_geometry(int rows, int n, Geometry* g) {
-    g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTallRows) * ceil_div((uint32_t)n, (uint32_t)kTallCols);
+    g->grid[0] = ceil_div((uint32_t)rows, (uint32_t)kTallRows) * gemm_tall_units(n);
     g->grid[1] = g->grid[2] = 1;
     g->block[0] = kTallThreads;
     g->shared = kTallLds;
@@ -874,18 +949,18 @@ int gemm_tall_launch(const int8_t* a, const void* w, const uint32_t* book, const
     const int ready = prepare();
     if (ready != ORX_OK) return ready;
     if (k % 128 != 0 || k < 256) {
-        set_error("projection (mfma 512x128): K must be a multiple of 128, at least 256");
+        set_error("projection (mfma, 512-row channel runs): K must be a multiple of 128, at least 256");
         return ORX_ERR_BAD_VARIANT;
     }
     BigParams p = {};
     p.a = a, p.w = w, p.book = book, p.ws = ws, p.as = as, p.out = out;
     p.n = n, p.k = k, p.stride = stride, p.m = rows, p.packed_k = packed_k, p.out_f32 = out_f32;
-    p.tiles_m = (rows + kTallRows - 1) / kTallRows, p.tiles_n = (n + kTallCols - 1) / kTallCols;
+    p.tiles_m = (rows + kTallRows - 1) / kTallRows, p.tiles_n = (int)gemm_tall_units(n);
     if (out_f32)
         ORX_LAUNCH((gemm_q4_tall_kernel<true>), dim3(g.grid[0]), dim3(kTallThreads), g.shared, stream, p);
     else
         ORX_LAUNCH((gemm_q4_tall_kernel<false>), dim3(g.grid[0]), dim3(kTallThreads), g.shared, stream, p);
-    return hip_check(hipGetLastError(), "launch projection (mfma 512x128, decode in the loop)");
+    return hip_check(hipGetLastError(), "launch projection (mfma, 512-row channel runs, decode in the loop)");
 }
 
 }  // namespace orx

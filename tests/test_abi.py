@@ -155,11 +155,14 @@ def test_dynamic_geometry_follows_live_rows():
     one, many, big = kernel.geometry(1), kernel.geometry(64), lib.Kernel(
         "e8p_q4_projection", M=512, N=9728, K=2560, dynamic_rows=True).geometry(512)
     assert one != many                        # batch-1 and batch-64 take different kernels
-    # no scratch: 76 tall tiles (512 x 128, decode in the loop) would be one round of 87 us-per-5120-K, the 304 whole
-    # 128 x 128 tiles are a little faster at this size; at N = 17408 the tall tiles win
-    assert big[0][0] * big[0][1] * big[0][2] == 76 * 4 and big[1] == (256, 1, 1)
+    # 257..512 rows of a matrix that gives every CU at least 2.25 blocks of 16 channels: one workgroup per CU (256 where
+    # no device answers) owns all rows and a run of channels, the decode in its K loop (608 and 1088 blocks here)
+    assert big[0] == (256, 1, 1) and big[1] == (512, 1, 1)
     tall = lib.Kernel("e8p_q4_projection", M=512, N=17408, K=5120, dynamic_rows=True).geometry(512)
-    assert tall[0] == (136, 1, 1) and tall[1] == (512, 1, 1)
+    assert tall[0] == (256, 1, 1) and tall[1] == (512, 1, 1)
+    # a narrow matrix (320 blocks) keeps the 128 x 128 tiles
+    narrow = lib.Kernel("e8p_q4_projection", M=512, N=5120, K=5120, dynamic_rows=True).geometry(512)
+    assert narrow[1] == (256, 1, 1)
     with pytest.raises(lib.OrxError) as err:
         kernel.geometry(65)
     assert err.value.code == lib.ORX_ERR_ROWS
@@ -542,19 +545,24 @@ def test_projections_take_the_reference_factories_schedule_names():
 
 
 def test_tall_tiles_by_name_and_for_handles_without_scratch():
-    """512 x 128 tiles with the decode in the K loop: by name at any row count, and what a two-stage handle without a
-    Workspace (or with decode_in_gemm) launches from 385 rows; K in whole blocks of 128, two-stage codes only."""
+    """512 rows x channel runs with the decode in the K loop: by name at any row count; what `auto` launches from 257
+    to 512 rows of a wide matrix whether or not there is a Workspace; and what a two-stage handle without one (or with
+    decode_in_gemm) launches above 512 rows.  K in whole blocks of 128, two-stage codes only."""
     shape = dict(M=1024, N=17408, K=5120, dynamic_rows=True)
     tall = lib.Kernel("e8p_q4_projection", **shape, algorithm="tall")
     plain = lib.Kernel("e8p_q4_projection", **shape)
     in_loop = lib.Kernel("e8p_q4_projection", **shape, workspace=True, decode_in_gemm=True)
+    scratch = lib.Kernel("e8p_q4_projection", **shape, workspace=True)
     for rows, row_tiles in ((3, 1), (512, 1), (513, 2), (1024, 2)):
         grid, block, lds = tall.geometry(rows)
-        assert grid == (row_tiles * 136, 1, 1) and block == (512, 1, 1) and 128 * 1024 < lds <= 160 * 1024
-    for rows in (385, 512, 1024):
+        assert grid == (row_tiles * 256, 1, 1) and block == (512, 1, 1) and 128 * 1024 < lds <= 160 * 1024
+    for rows in (257, 385, 512, 1024):
         assert plain.geometry(rows) == tall.geometry(rows) == in_loop.geometry(rows)
         assert in_loop.workspace_bytes(rows) == 0
-    assert plain.geometry(384) != tall.geometry(384)
+    for rows in (257, 384, 512):
+        assert scratch.geometry(rows) == tall.geometry(rows) and scratch.workspace_bytes(rows) == 0
+    assert scratch.geometry(513) != tall.geometry(513) and scratch.workspace_bytes(513) >= 17408 * 5120
+    assert plain.geometry(256) != tall.geometry(256) and scratch.geometry(256) != tall.geometry(256)
     for symbol, bad in (("int8_projection", dict(M=8, N=256, K=512)), ("e8p_q4_projection", dict(M=8, N=256, K=128))):
         with pytest.raises(lib.OrxError) as err:
             lib.Kernel(symbol, **bad, algorithm="tall")

@@ -856,11 +856,11 @@ def test_q4_big_tile_tails_stride_sentinels(packed_k):
 
 
 @pytest.mark.parametrize("packed_k", [0, 64, 128])
-@pytest.mark.parametrize("m,n,k", [(512, 256, 512), (500, 333, 640), (700, 130, 256), (3, 128, 384)])
+@pytest.mark.parametrize("m,n,k", [(512, 256, 512), (500, 333, 640), (700, 130, 256), (3, 128, 384), (300, 17400, 256)])
 def test_q4_tall_tiles_decode_in_the_k_loop(m, n, k, packed_k):
-    """512 x 128 tiles with the decode in the K loop (`algorithm=tall`; what a handle without a Workspace runs from 385
-    rows on): K of an even and an odd number of 128-blocks, one and two row tiles, ragged rows and channels, every
-    layout, fp16 and fp32 output with a stride and sentinels."""
+    """512 rows x channel runs with the decode in the K loop (`algorithm=tall`): K of an even and an odd number of
+    128-blocks, one and two row tiles, ragged rows and channels, runs of one block and (N = 17400 on 256 CUs) of four
+    and five blocks with a ragged last block, every layout, fp16 and fp32 output with a stride and sentinels."""
     rng = np.random.default_rng(orc.SEED + m + n + k + packed_k)
     a_q, a_s, packed, scales = q4_case(rng, m, n, k)
     a_q[0, :2] = [-128, 127]
@@ -873,6 +873,39 @@ def test_q4_tall_tiles_decode_in_the_k_loop(m, n, k, packed_k):
         got = gu.host(storage)
         np.testing.assert_array_equal(got[:m, :n], orc.project(a_q, a_s, weights, scales, np_dtype))
         assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
+
+
+@pytest.mark.parametrize("workspace", [False, True])
+def test_q4_auto_takes_channel_runs_from_257_rows_of_a_wide_matrix(workspace):
+    """257..512 rows of a matrix with at least 2.25 blocks of 16 channels per CU: `auto` decodes in the K loop of the
+    512-row channel runs and leaves the Workspace alone; 256 rows and a narrow matrix keep the other kernels."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n, k = 16 * (9 * cus // 4) + 16 + 8, 256
+    rng = np.random.default_rng(orc.SEED + 77 + workspace)
+    a_q, a_s, packed, scales = q4_case(rng, 512, n, k)
+    weights = orc.q4_integers(packed, TABLE)
+    variant = dict(M=512, N=n, K=k, dynamic_rows=True, output_stride=n + 8)
+    if workspace:
+        variant["workspace"] = True
+    kern = gu.lib.Kernel("e8p_q4_projection", **variant)
+    by_name = gu.lib.Kernel("e8p_q4_projection", **variant, algorithm="tall")
+    narrow = [gu.lib.Kernel("e8p_q4_projection", **dict(variant, N=16 * 2 * cus), **extra) for extra in ({}, {"algorithm": "tall"})]
+    scratch = torch.zeros(max(kern.workspace_bytes(0), 16), dtype=torch.uint8, device=gu.DEV) if workspace else None
+    assert narrow[0].geometry(257) != narrow[1].geometry(257)      # two blocks per CU: the 128 x 128 tiles
+    out = torch.full((513, n + 8), 7.0, dtype=torch.float16, device=gu.DEV)
+    for rows in (257, 400, 512, 256):
+        same = kern.geometry(rows) == by_name.geometry(rows)
+        assert same == (rows > 256)
+        if rows > 256:
+            assert kern.workspace_bytes(rows) == 0
+        out.fill_(7.0)
+        args = dict(A=gu.dev(a_q), AS=gu.dev(a_s), Book=gu.book(), Out=out, S=gu.dev(scales), W=gu.dev(packed), m=rows)
+        if workspace:
+            args["Workspace"] = scratch
+        kern(**args)
+        got = gu.host(out)
+        np.testing.assert_array_equal(got[:rows, :n], orc.project(a_q[:rows], a_s[:rows], weights, scales))
+        assert (got[rows:] == 7).all() and (got[:rows, n:] == 7).all()
 
 
 @pytest.mark.parametrize("codec", ["w8", "q4"])
@@ -1077,14 +1110,15 @@ def test_config1_full_size_bit_exact(rows):
 
 
 def test_config1_full_size_512_rows_without_scratch():
-    """The same 512 rows through a handle without a Workspace: 512 x 128 tiles with the decode in the K loop, K-major
-    codes as the package stores them, against the oracle on every row."""
+    """The same 512 rows through a handle without a Workspace: the same 512-row channel runs with the decode in the K
+    loop (one workgroup per CU), K-major codes as the package stores them, against the oracle on every row."""
     c = workloads.config1(512)
     a_q, a_s = gu.a8(gu.dev(c["x"]))
     wq, ws = orc.a8(c["x"])
     stored = orc.q4_pack_k(c["packed"], 128)
     kern = gu.lib.Kernel("e8p_q4_projection", M=512, N=c["n"], K=c["k"], packed_k=128)
-    assert kern.geometry(512)[1] == (512, 1, 1) and kern.geometry(512)[0] == (c["n"] // 128, 1, 1)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    assert kern.geometry(512)[1] == (512, 1, 1) and kern.geometry(512)[0] == (min(c["n"] // 16, cus), 1, 1)
     out = torch.empty((512, c["n"]), dtype=torch.float16, device=gu.DEV)
     kern(A=a_q, AS=a_s, Book=gu.book(), Out=out, S=gu.dev(c["scales"]), W=gu.dev(stored))
     np.testing.assert_array_equal(gu.host(out), orc.project(wq, ws[:, 0], _config1_weights(c), c["scales"]))
