@@ -463,8 +463,9 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
 //   weights      a thread of the first five waves owns one 16-byte chunk of the decoded stage per step (channel
 //                tid / 4, K bytes [16 (tid % 4), +16) of the slice: two code words); it holds the four words of
 //                its channel and quarter for a K block of 128 in registers, a second set for the block after it.
-//                Every code word costs four 4-byte lookups (biased nibbles of the basis row, sign mask, for either
-//                stage; tables of 1 KiB each) and a few byte-parallel operations.  Four stages of 5 KiB.
+//                Every code word costs four 8-byte lookups in the compact byte tables (8 KiB at the start of the
+//                LDS, so a lookup's address is its entry's offset and the table is the instruction's offset
+//                field) and four byte-parallel operations per output word.  Four stages of 5 KiB.
 //   step s       the fragments of step s are in registers on entry.  Between its 20 multiplies the wave issues the
 //                eight lookups for the weights of step s + 2, the nine fragment reads of step s + 1, in odd steps
 //                the eight requests for the token rows of steps s + 3 and s + 4 (the slot that steps s - 1 and s
@@ -472,25 +473,29 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
 //                two blocks ahead (every wave does, so that all count the same requests).  One barrier per step
 //                publishes the decoded stage.
 // All LDS traffic and the code loads of the loop are asm statements with hand-placed waits: the compiler would
-// wait for every direct-to-LDS request in flight before an LDS access it can see.  The loop is bound by the LDS
-// pipe (per step and CU: 72 fragment reads of 1 KiB, 32 KiB of token rows landing, 40 wave lookups, 5 KiB written)
-// at about 70 % of its rate, above the floor that the token rows set (every CU reads all rows once: 2.6 MB per CU
-// at 512 x 5120, which 256 CUs together pull out of the L2 in 37 us).
+// wait for every direct-to-LDS request in flight before an LDS access it can see.  What a step issues has to come
+// back within the step, and per step and CU that is 72 fragment reads of 1 KiB (8 clocks each), 32 KiB of token
+// rows landing, 5 KiB written and 40 wave lookups whose random addresses collide in the banks (counters: bank
+// conflicts are 0.4 of the LDS pipe's busy cycles, all of them lookups; tables stored several times would not fit
+// beside the token slots): about 1 350 clocks of LDS work in a step of 1 550.  The floor under it is what the token
+// rows cost: every CU reads all of them once, 2.6 MB per CU at 512 x 5120, which 256 CUs together pull out of the
+// L2 in 37 us.
 constexpr int kTallBlocks = 5;  // blocks of 16 channels per workgroup, at most
 constexpr int kTallRows = 512, kTallCols = 16 * kTallBlocks, kTallStep = 64, kTallThreads = 512, kTallStagesW = 4;
 constexpr uint32_t kTallSlotA = kTallRows * 128;  // token rows of a K chunk of 128
 constexpr uint32_t kTallStageW = kTallCols * kTallStep;
-constexpr uint32_t kTallWeights = 2 * kTallSlotA;  // byte offsets in dynamic LDS
-constexpr uint32_t kTallTables = kTallWeights + kTallStagesW * kTallStageW;
-constexpr uint32_t kTallScales = kTallTables + 2048;  // nib[256], msk[256]
+// byte offsets in dynamic LDS: the tables first, so that a lookup's address is its table index alone
+constexpr uint32_t kTallTokens = (uint32_t)sizeof(Q4ByteTables);
+constexpr uint32_t kTallWeights = kTallTokens + 2 * kTallSlotA;
+constexpr uint32_t kTallScales = kTallWeights + kTallStagesW * kTallStageW;
 constexpr uint32_t kTallLds = kTallScales + (kTallRows + kTallCols) * 4;
 
 typedef unsigned int v2w __attribute__((ext_vector_type(2)));
 
 template <int OFFSET>
-__device__ __forceinline__ uint32_t lds_read_4(uint32_t lds_address) {
-    uint32_t value;
-    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
+__device__ __forceinline__ v2w lds_read_8(uint32_t lds_address) {
+    v2w value;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(value) : "v"(lds_address), "n"(OFFSET));
     return value;
 }
 // 8 bytes from global memory that the compiler keeps no count for: whoever uses them waits by hand
@@ -509,7 +514,7 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     extern __shared__ __align__(16) int8_t lds[];
     float* const lds_as = reinterpret_cast<float*>(lds + kTallScales);
     float* const lds_ws = lds_as + kTallRows;
-    uint32_t* const nib = reinterpret_cast<uint32_t*>(lds + kTallTables);  // biased nibbles of the basis rows, then the sign masks
+    Q4ByteTables* const tables = reinterpret_cast<Q4ByteTables*>(lds);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // unit u of a row tile owns the channel blocks [u B / U, (u + 1) B / U) of the B blocks of 16 channels
@@ -548,7 +553,7 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     load_codes(1, std::integral_constant<int, 1>{});
 
     // ---- tables and scales, written before any direct-to-LDS request is in flight ----
-    if (tid < 256) nib[tid] = nibble_basis_word(p.book[tid], 8u), nib[256 + tid] = nibble_mask_word((uint32_t)tid);
+    build_tables(*tables, p.book, tid, kTallThreads);
     lds_as[tid] = __half2float(p.as[t.row0 + min(tid, t.rows_here - 1)]);
     if (tid < kTallCols) lds_ws[tid] = __half2float(p.ws[t.col0 + min(tid, t.cols_here - 1)]);
     __syncthreads();
@@ -559,16 +564,20 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     const int load_row = wave * 64 + (lane >> 3);
     const uint32_t load_chunk = (uint32_t)(((lane & 7) ^ swizzle(load_row)) * 16);
     const int8_t* const a_base = uniform_pointer(p.a + (int64_t)t.row0 * p.k);
+    // (the eight offsets stay in registers: computing them on issue is a multiply and five more instructions per
+    // request, and the vector ALU of the SIMD that hosts two decoding waves is what the loop waits for)
+    uint32_t load_offset[8];
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+        load_offset[b] = (uint32_t)(min(load_row + 8 * b, t.rows_here - 1) * p.k) + (load_chunk ^ (uint32_t)((b & 1) * 64));
     auto issue_tokens = [&](int b, int chunk, int slot) {
-        int row = load_row;
-        asm volatile("" : "+v"(row));  // or every request's offset is kept in a register for the whole loop
-        const uint32_t offset = (uint32_t)(min(row + 8 * b, t.rows_here - 1) * p.k) + (load_chunk ^ (uint32_t)((b & 1) * 64));
-        direct_load_16(a_base + min(chunk, blocks - 1) * 128 + (uint64_t)offset, lds + slot * kTallSlotA + (wave * 8 + b) * 1024);
+        direct_load_16(a_base + min(chunk, blocks - 1) * 128 + (uint64_t)load_offset[b],
+                       lds + kTallTokens + slot * kTallSlotA + (wave * 8 + b) * 1024);
     };
 
     // ---- fragments: a lane reads K bytes [16 (lane / 16), +16) of the slice for row lane % 16 of a block ----
     const int frag_row = lane & 15, frag_chunk = lane >> 4;
-    const uint32_t a_frag = lds_base + (wave * 64 + frag_row) * 128 + ((frag_chunk ^ swizzle(frag_row)) * 16);
+    const uint32_t a_frag = lds_base + kTallTokens + (wave * 64 + frag_row) * 128 + ((frag_chunk ^ swizzle(frag_row)) * 16);
     const uint32_t w_frag = lds_base + kTallWeights + (uint32_t)(frag_row * kTallStep + ((frag_chunk ^ tall_swizzle(frag_row)) * 16));
     v4i ft[2][4], fw[2][kTallBlocks];  // token and weight fragments of even and odd steps
     constexpr int kBlock = 16 * kTallStep;
@@ -593,18 +602,19 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     };
 
     // ---- decode: this thread's chunk of a weight stage ----
-    const uint32_t table_base = lds_base + kTallTables;
     const uint32_t write_offset = kTallWeights + (uint32_t)(channel * kTallStep + ((quarter ^ tall_swizzle(channel)) * 16));
-    uint32_t looked[8];
-    auto lookups = [&](v2w pair) {  // two code words: nibbles and signs of either stage
+    // (the dynamic LDS of a kernel without static LDS starts at address 0, where the tables sit: a lookup's address
+    // is the byte offset of its entry, the table chosen by the instruction's offset field)
+    v2w looked[8];
+    auto lookups = [&](v2w pair) {  // two code words: basis0, mask0, basis1, mask1 of each
         asm volatile("" : "+v"(pair));  // nothing computed from the words moves above this point
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const uint32_t code = pair[i];
-            looked[4 * i + 0] = lds_read_4<0>(table_base + ((code >> 6) & 0x3FCu));       // nib[(code >> 8) & 255]
-            looked[4 * i + 1] = lds_read_4<1024>(table_base + ((code << 2) & 0x3FCu));    // msk[code & 255]
-            looked[4 * i + 2] = lds_read_4<0>(table_base + ((code >> 22) & 0x3FCu));      // nib[code >> 24]
-            looked[4 * i + 3] = lds_read_4<1024>(table_base + ((code >> 14) & 0x3FCu));   // msk[(code >> 16) & 255]
+            looked[4 * i + 0] = lds_read_8<0>(lds_base + ((code >> 5) & 0x7F8u));       // basis0[(code >> 8) & 255]
+            looked[4 * i + 1] = lds_read_8<2048>(lds_base + ((code << 3) & 0x7F8u));    // mask0[code & 255]
+            looked[4 * i + 2] = lds_read_8<4096>(lds_base + ((code >> 21) & 0x7F8u));   // basis1[code >> 24]
+            looked[4 * i + 3] = lds_read_8<6144>(lds_base + ((code >> 13) & 0x7F8u));   // mask1[(code >> 16) & 255]
         }
     };
     v4u chunk;
@@ -619,13 +629,10 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
                      : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
                        "+v"(looked[6]), "+v"(looked[7]));
     };
-    // code word i -> 8 weights.  x0, x1: v + 8 of either stage in the nibbles (coordinates 0..3 in the low nibbles of
-    // the bytes, 4..7 in the high ones); w + 128 = 8 (v0 + 8) + 2 (v1 + 8) + 53 in every byte, in [73, 183]: no carry
-    // between bytes, and the XOR turns offset binary into two's complement (what decode_q4 computes from byte tables)
+    // code word i -> 8 weights, as decode_q4 combines the four entries
     auto combine = [&](int i) {
-        const uint32_t x0 = looked[4 * i] ^ looked[4 * i + 1], x1 = looked[4 * i + 2] ^ looked[4 * i + 3];
-        chunk[2 * i + 0] = (((x0 << 3) & 0x78787878u) + ((x1 << 1) & 0x1E1E1E1Eu) + 0x35353535u) ^ 0x80808080u;
-        chunk[2 * i + 1] = (((x0 >> 1) & 0x78787878u) + ((x1 >> 3) & 0x1E1E1E1Eu) + 0x35353535u) ^ 0x80808080u;
+        chunk[2 * i + 0] = ((looked[4 * i][0] ^ looked[4 * i + 1][0]) + (looked[4 * i + 2][0] ^ looked[4 * i + 3][0]) + 0x35353535u) ^ 0x80808080u;
+        chunk[2 * i + 1] = ((looked[4 * i][1] ^ looked[4 * i + 1][1]) + (looked[4 * i + 2][1] ^ looked[4 * i + 3][1]) + 0x35353535u) ^ 0x80808080u;
     };
     auto write_chunk = [&](int stage) { lds_write_16(lds_base + write_offset + stage * kTallStageW, chunk); };
     auto write_decoded = [&](int stage) {
