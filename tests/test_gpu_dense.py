@@ -875,6 +875,35 @@ def test_q4_tall_tiles_decode_in_the_k_loop(m, n, k, packed_k):
         assert (got[m:] == 91).all() and (got[:m, n:] == 91).all()
 
 
+def test_q4_tall_tiles_two_rounds_of_units_and_graph_replay():
+    """More blocks of 16 channels than five per CU: the units come in two rounds.  One handle, live rows from a trailing
+    scalar, replayed from a graph while the weight bits change in place and the row count changes between captures."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    n, k = 16 * (5 * cus + 9) + 3, 256
+    rng = np.random.default_rng(orc.SEED + 123)
+    a_q, a_s, packed, scales = q4_case(rng, 512, n, k)
+    other = rng.integers(0, 2**32, packed.shape, dtype=np.uint32)
+    kern = gu.lib.Kernel("e8p_q4_projection", M=512, N=n, K=k, dynamic_rows=True, algorithm="tall")
+    assert kern.geometry(300)[0] == (2 * cus, 1, 1)
+    d_a, d_as, d_s, d_book, d_w = gu.dev(a_q), gu.dev(a_s), gu.dev(scales), gu.book(), gu.dev(packed)
+    out = torch.full((512, n), 7.0, dtype=torch.float16, device=gu.DEV)
+    side = torch.cuda.Stream()
+    for rows in (300, 512):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                kern(stream=side.cuda_stream, A=d_a, AS=d_as, Book=d_book, Out=out, S=d_s, W=d_w, m=rows)
+        for bits in (other, packed, other):
+            d_w.copy_(gu.dev(bits))
+            out.fill_(7.0)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = gu.host(out)
+            np.testing.assert_array_equal(got[:rows], orc.project(a_q[:rows], a_s[:rows], orc.q4_integers(bits, TABLE), scales))
+            assert (got[rows:] == 7).all()
+
+
 @pytest.mark.parametrize("workspace", [False, True])
 def test_q4_auto_takes_channel_runs_from_257_rows_of_a_wide_matrix(workspace):
     """257..512 rows of a matrix with at least 2.25 blocks of 16 channels per CU: `auto` decodes in the K loop of the
