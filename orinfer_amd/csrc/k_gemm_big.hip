@@ -565,7 +565,7 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     const uint32_t load_chunk = (uint32_t)(((lane & 7) ^ swizzle(load_row)) * 16);
     const int8_t* const a_base = uniform_pointer(p.a + (int64_t)t.row0 * p.k);
     // (the eight offsets stay in registers: computing them on issue is a multiply and five more instructions per
-    // request, and the vector ALU of the SIMD that hosts two decoding waves is what the loop waits for)
+    // request)
     uint32_t load_offset[8];
 #pragma unroll
     for (int b = 0; b < 8; ++b)
