@@ -62,6 +62,8 @@ def parse():
     p.add_argument("--warmup", type=int, default=100)
     p.add_argument("--no-extra", action="store_true", help="only the contract workload")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--settle", type=float, default=CLOCK_WARMUP_SECONDS, metavar="SECONDS",
+                   help="untimed graph replays in front of every timed region (0 under a profiler: they only add dispatches)")
     p.add_argument("--profile-rows", type=int, default=0, metavar="ROWS",
                    help="workload for a rocprofv3 counter run: config 1's projection at ROWS rows once per weight copy, "
                         "eagerly, then exit")
@@ -97,7 +99,7 @@ def main():
         while True:
             graph.replay()
             torch.cuda.synchronize()
-            if time.perf_counter() - t0 >= CLOCK_WARMUP_SECONDS:
+            if time.perf_counter() - t0 >= args.settle:
                 return
 
     def timed_graph(enqueue, launches, replays=3):
@@ -240,7 +242,7 @@ def main():
         "config": {"workload": "BASELINE config 1: Q4A8 linear K=5120 N=17408, M=1 decode GEMV, step = A8 + projection "
                                "of one fp16 row (one launch: the GEMV quantises the row during its set-up)",
                    "weight_copies_rotated": copies, "algorithmic_bytes_per_step": bytes_c1,
-                   "untimed_replays_before_timing_seconds": CLOCK_WARMUP_SECONDS},
+                   "untimed_replays_before_timing_seconds": args.settle},
         "roofline": {"bound": "hbm", "kernel": traffic_kernel or "gemv_banked_kernel<Q4, 1 row, fp16 input>",
                      "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),

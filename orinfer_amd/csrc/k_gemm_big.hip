@@ -97,9 +97,9 @@ __device__ __forceinline__ void tile_of(int id, int tiles_m, int tiles_n, int* t
 // LDS, no workgroup barrier, and leaves both operand stages alone (they already hold the next tile's first
 // steps); its stores are not waited for and drain under the next tile's multiplies.
 //
-// The kernel is bound by power, not by issue slots: on random int8 data the clock inside the K loop settles near
-// 1.2-1.3 GHz, the same launch on zero operands is 30 % shorter, and taking out stalls alone changes nothing at
-// large K.  What pays is less energy per multiply.  v_mfma_i32_16x16x64_i8 does the same work per cycle as
+// The kernel is bound by power, not by issue slots: on random int8 data the clock inside the K loop is 1.9 GHz in a
+// sustained run (1.2-1.3 GHz in a launch that follows a pause), the same launch on zero operands is 30 % shorter, and
+// taking out stalls alone changes nothing at large K.  What pays is less energy per multiply.  v_mfma_i32_16x16x64_i8 does the same work per cycle as
 // v_mfma_i32_32x32x32_i8 with half the accumulator traffic per multiply and sustains 3.83 POP/s on random
 // operands where the 32 x 32 shape sustains 3.37 (back-to-back issue from registers, whole chip); the fragment
 // bytes read from LDS per multiply are the same, so the tile, the stages and the swizzle stay as they were.
