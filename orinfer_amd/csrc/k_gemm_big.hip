@@ -473,13 +473,14 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
 //                two blocks ahead (every wave does, so that all count the same requests).  One barrier per step
 //                publishes the decoded stage.
 // All LDS traffic and the code loads of the loop are asm statements with hand-placed waits: the compiler would
-// wait for every direct-to-LDS request in flight before an LDS access it can see.  What a step issues has to come
-// back within the step, and per step and CU that is 72 fragment reads of 1 KiB (8 clocks each), 32 KiB of token
-// rows landing, 5 KiB written and 40 wave lookups whose random addresses collide in the banks (counters: bank
-// conflicts are 0.4 of the LDS pipe's busy cycles, all of them lookups; tables stored several times would not fit
-// beside the token slots): about 1 350 clocks of LDS work in a step of 1 550.  The floor under it is what the token
-// rows cost: every CU reads all of them once, 2.6 MB per CU at 512 x 5120, which 256 CUs together pull out of the
-// L2 in 37 us.
+// wait for every direct-to-LDS request in flight before an LDS access it can see.  Per step and CU the LDS pipe
+// serves 72 fragment reads of 1 KiB (8 clocks each), 32 KiB of token rows landing, 5 KiB written and 40 wave
+// lookups whose random addresses collide in the banks, and no unit is full: the matrix pipe is busy in 0.35 of
+// the cycles, the LDS pipe in about 0.6.  Taking out any one part of a step shortens the loop by 5-25 % (the
+// decode most), while lookups made cheaper (4-byte nibble tables, also stored 8 and 4 times) measure the same:
+// what a step issues has to come back within the step, and the parts queue behind one another.  The floor under
+// it is what the token rows cost: every CU reads all of them once, 2.6 MB per CU at 512 x 5120, which 256 CUs
+// together pull out of the L2 in 37 us.
 constexpr int kTallBlocks = 5;  // blocks of 16 channels per workgroup, at most
 constexpr int kTallRows = 512, kTallCols = 16 * kTallBlocks, kTallStep = 64, kTallThreads = 512, kTallStagesW = 4;
 constexpr uint32_t kTallSlotA = kTallRows * 128;  // token rows of a K chunk of 128
