@@ -466,12 +466,12 @@ __global__ __launch_bounds__(kPersistentThreads) void gemm_big_persistent_kernel
 //                Every code word costs four 8-byte lookups in the compact byte tables (8 KiB at the start of the
 //                LDS, so a lookup's address is its entry's offset and the table is the instruction's offset
 //                field) and four byte-parallel operations per output word.  Four stages of 5 KiB.
-//   step s       the fragments of step s are in registers on entry.  Between its 20 multiplies the wave issues the
-//                eight lookups for the weights of step s + 2, the nine fragment reads of step s + 1, in odd steps
-//                the eight requests for the token rows of steps s + 3 and s + 4 (the slot that steps s - 1 and s
-//                have left), then combines the lookups and writes its chunk; in even steps it requests the codes
-//                two blocks ahead (every wave does, so that all count the same requests).  One barrier per step
-//                publishes the decoded stage.
+//   step s       between its 20 multiplies the wave issues the eight lookups for the weights of step s + 2, combines
+//                them and writes its chunk, then requests the nine fragments of step s + 1, which cross the
+//                step's barrier and are waited for in front of the next step's first multiply; in odd steps the
+//                eight requests for the token rows of steps s + 3 and s + 4 (the slot that steps s - 1 and s have
+//                left); in even steps the codes two blocks ahead (every wave does, so that all count the same
+//                requests).  One barrier per step publishes the decoded stage.
 // All LDS traffic and the code loads of the loop are asm statements with hand-placed waits: the compiler would
 // wait for every direct-to-LDS request in flight before an LDS access it can see.  Per step and CU the LDS pipe
 // serves 72 fragment reads of 1 KiB (8 clocks each), 32 KiB of token rows landing, 5 KiB written and 40 wave
@@ -625,11 +625,6 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
                      : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
                        "+v"(looked[6]), "+v"(looked[7]));
     };
-    auto wait_lookups_before_fragments = [&]() {  // the 9 fragment reads of a step are younger
-        asm volatile("s_waitcnt lgkmcnt(9)"
-                     : "+v"(looked[0]), "+v"(looked[1]), "+v"(looked[2]), "+v"(looked[3]), "+v"(looked[4]), "+v"(looked[5]),
-                       "+v"(looked[6]), "+v"(looked[7]));
-    };
     // code word i -> 8 weights, as decode_q4 combines the four entries
     auto combine = [&](int i) {
         chunk[2 * i + 0] = ((looked[4 * i][0] ^ looked[4 * i + 1][0]) + (looked[4 * i + 2][0] ^ looked[4 * i + 3][0]) + 0x35353535u) ^ 0x80808080u;
@@ -661,7 +656,7 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
             }
     };
 
-    // ---- prologue: K chunks 0 and 1 requested, the weights of steps 0 and 1 decoded (block 0), step 0's fragments read ----
+    // ---- prologue: K chunks 0 and 1 requested, the weights of steps 0 and 1 decoded (block 0), step 0's fragments requested ----
 #pragma unroll
     for (int b = 0; b < 8; ++b) issue_tokens(b, 0, 0);
 #pragma unroll
@@ -676,54 +671,61 @@ __global__ __launch_bounds__(kTallThreads) void gemm_q4_tall_kernel(BigParams p)
     asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     read_tokens(0, 0);
     read_weights(0, 0);
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]),
-                   "+v"(fw[0][3]), "+v"(fw[0][4])
-                 :
-                 : "memory");
 
-    // Step s.  On entry the fragments of step s are in registers, the rows of step s + 1 (this wave's own requests)
-    // have landed and its weights were written in front of the last barrier.  Everything else of the step sits
-    // between its 20 multiplies, so that the matrix pipe works while the LDS pipe and the vector ALU serve the rest:
-    // the lookups for the weights of step s + 2 first, then the fragment reads of step s + 1 (so the lookups return
-    // first), the row requests of an odd step, and behind the tenth multiply the lookups combined and written.
+    // Step s.  On entry the fragments of step s are on their way into registers (requested late in step s - 1, waited
+    // for here), the rows of step s + 1 (this wave's own requests) have landed and its weights were written in front
+    // of the last barrier.  Everything else of the step sits between its 20 multiplies, so that the matrix pipe works
+    // while the LDS pipe and the vector ALU serve the rest: the lookups for the weights of step s + 2 first, behind
+    // the fifth multiply their combination and the write of the chunk, and only then the nine fragment reads of step
+    // s + 1.  LDS requests of a wave return in order, so the wait in front of the barrier can name the nine reads as
+    // what may stay in flight: the chunk has landed, which is all the barrier has to publish, and the reads cross the
+    // barrier (the LDS pipe has work while the waves meet; with the reads waited for in front of the barrier the
+    // loop measured 5 % longer).  The stages they read are not written again before two more barriers.
     // K chunk c (steps 2 c, 2 c + 1) is requested in step 2 c - 3 into the slot that chunk c - 2 left when step
-    // 2 c - 4 read its last fragments, and has two steps to land.  The wait in front of the barrier names how many
-    // younger requests may stay in flight (vector memory retires in order): behind an even step its 2 code requests,
-    // behind an odd step its 8 row requests.
+    // 2 c - 3 waited for its last fragments, and has two steps to land.  The vector-memory part of the wait names
+    // how many younger requests may stay in flight (vector memory retires in order): behind an even step its 2 code
+    // requests, behind an odd step its 8 row requests.
+    auto wait_fragments_even = [&]() {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(fw[0][0]), "+v"(fw[0][1]), "+v"(fw[0][2]),
+                       "+v"(fw[0][3]), "+v"(fw[0][4])
+                     :
+                     : "memory");
+    };
+    auto wait_fragments_odd = [&]() {
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(ft[1][0]), "+v"(ft[1][1]), "+v"(ft[1][2]), "+v"(ft[1][3]), "+v"(fw[1][0]), "+v"(fw[1][1]), "+v"(fw[1][2]),
+                       "+v"(fw[1][3]), "+v"(fw[1][4])
+                     :
+                     : "memory");
+    };
     auto step = [&](int s, auto set_tag, auto odd_tag) {
         constexpr int SET = decltype(set_tag)::value, ODD = decltype(odd_tag)::value;  // SET: of the block being decoded
         const int next_stage = (s + 1) % kTallStagesW, decode_stage = (s + 2) % kTallStagesW;
+        if constexpr (ODD) wait_fragments_odd(); else wait_fragments_even();
         __builtin_amdgcn_sched_barrier(0);
         multiply(ODD, [&](int index) {
             __builtin_amdgcn_sched_barrier(0);
             if (index == 0 && decoder) lookups(codes[SET][ODD]);
-            if (index == 2) read_tokens(s + 1, 1 - ODD);
-            if (index == 4) read_weights(next_stage, 1 - ODD);
             if (ODD && (index & 1) == 1 && index < 16)  // chunk (s + 3) / 2 into the slot that chunk (s - 1) / 2 has left
                 issue_tokens(index >> 1, (s + 3) >> 1, ((s + 3) >> 1) & 1);
-            if (index >= 10 && index <= 14 && (index & 1) == 0 && decoder) {
-                if (index == 10) wait_lookups_before_fragments();
-                if (index == 10) combine(0);
-                if (index == 12) combine(1);
-                if (index == 14) write_chunk(decode_stage);
+            if (index >= 4 && index <= 8 && (index & 1) == 0 && decoder) {
+                if (index == 4) wait_lookups();
+                if (index == 4) combine(0);
+                if (index == 6) combine(1);
+                if (index == 8) write_chunk(decode_stage);
             }
+            if (index == 10) read_tokens(s + 1, 1 - ODD);
+            if (index == 12) read_weights(next_stage, 1 - ODD);
             __builtin_amdgcn_sched_barrier(0);
         });
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!ODD) load_codes((s >> 1) + 2, std::integral_constant<int, 1 - SET>{});
+        // the 9 fragment reads may stay in flight over the barrier; the chunk written before them has landed
         if constexpr (!ODD)
-            asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(ft[1][0]), "+v"(ft[1][1]), "+v"(ft[1][2]), "+v"(ft[1][3]), "+v"(fw[1][0]), "+v"(fw[1][1]),
-                           "+v"(fw[1][2]), "+v"(fw[1][3]), "+v"(fw[1][4])
-                         :
-                         : "memory");
+            asm volatile("s_waitcnt vmcnt(2) lgkmcnt(9)\n\ts_barrier" ::: "memory");
         else
-            asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
-                         : "+v"(ft[0][0]), "+v"(ft[0][1]), "+v"(ft[0][2]), "+v"(ft[0][3]), "+v"(fw[0][0]), "+v"(fw[0][1]),
-                           "+v"(fw[0][2]), "+v"(fw[0][3]), "+v"(fw[0][4])
-                         :
-                         : "memory");
+            asm volatile("s_waitcnt vmcnt(8) lgkmcnt(9)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
     // steps 4 g .. 4 g + 3 decode blocks 2 g + 1 (set 1: steps 4 g, 4 g + 1) and 2 g + 2 (set 0: steps 4 g + 2, 4 g + 3)
