@@ -710,24 +710,28 @@ bool use_wide(const orx_function& f, int rows) {
 }
 
 // Two-stage codes on 512 rows x channel runs with the decode in the K loop (k_gemm_big.hip): `algorithm=tall` by
-// name, and `auto` from 257 to 512 rows, with or without scratch, when the runs fill their five blocks of 16
-// channels well enough.  A launch costs 0.76 us per 64 of K and round of the CUs whatever N is (every CU reads all
+// name, and `auto` from 257 (the widest matrices: 129) to 512 rows, with or without scratch, when the runs fill
+// their five blocks of 16 channels well enough.  A launch costs 0.76 us per 64 of K and round of the CUs whatever N is (every CU reads all
 // token rows), so it pays when the matrix gives every CU enough channels.  Measured against the kernels `auto` had
 // at 384 / 512 rows (128 x 128 tiles / decode once + 256 x 256 tiles; us, 256 CUs): N x K = 17408 x 5120 (4.25
 // blocks per CU) 64 / 66 against 77 / 86, 34816 x 5120 (two rounds of 4.25) 131 / 135 against 142 / 158,
 // 14336 x 4096 (3.5) 52 / 53 against 64 / 65, 12288 x 3072 (3) 41 / 42 against 46 / 55, 9728 x 2560 (2.4) 35 / 34
 // against 40 / 44; 7168 x 5120 (1.75) 59 / 59 against 44 / 51, 28672 x 8192 (two rounds of 3.5) 189 / 194 against
-// 158 / 194.  Up to 256 rows the split 128 x 128 tiles tie or win (60-63 against 62-65 at config 1's shape).
-bool tall_runs_fill(int n) {
+// 158 / 194.  At 129..256 rows the runs cost what they cost at 512 and the 128 x 128 tiles half as much: only a
+// matrix with 4.25 blocks per CU in one round gains (17408 x 5120 at 130 / 192 / 256 rows: 56 / 57 / 56 us against
+// 57 / 59 / 59 for the split tiles and 69 / 76 / 76 for whole tiles, what a handle without scratch had; 14336 x 4096
+// at 3.5 blocks per CU: 51 against 45 and 47).
+bool tall_runs_fill(int n, int rows) {
     const int64_t blocks = ceil_div((uint32_t)n, 16u), cus = device_compute_units();
     const int64_t rounds = (blocks + 5 * cus - 1) / (5 * cus);
+    if (rows <= 256) return rounds == 1 && 4 * blocks >= 17 * cus;
     return rounds == 1 ? 4 * blocks >= 9 * cus : blocks >= 4 * rounds * cus;
 }
 bool use_tall(const orx_function& f, int rows) {
     if (f.flags != kQ4) return false;
     if (f.algorithm == kTall) return true;
     if (f.algorithm != kAuto || tile_for(f, rows) != 0 || f.K % 128 != 0 || f.K < 256) return false;
-    return rows > 256 && rows <= 512 && tall_runs_fill(f.N);
+    return rows > 128 && rows <= 512 && tall_runs_fill(f.N, rows);
 }
 
 bool use_resident(const orx_function& f, int rows);

@@ -243,8 +243,9 @@ def test_handles_own_no_device_memory_and_say_what_workspace_they_need():
     assert err.value.code == lib.ORX_ERR_BAD_ARGUMENT
     handles = [lib.Kernel("e8p_q4_projection", M=64 + i, N=17408, K=5120, dynamic_rows=True, workspace=True)
                for i in range(1000)]
-    # up to 128 rows no launch of such a handle needs scratch (K = 5120: the channel-run kernel serves 65..128 rows)
-    assert all(h.workspace_bytes(0) == 0 for h in handles[:65]) and all(h.workspace_bytes(0) > 0 for h in handles[65:])
+    # up to 512 rows no launch of such a handle needs scratch (K = 5120: the channel-run kernel serves 65..128 rows, and
+    # this matrix gives every CU 4.25 blocks of 16 channels: the 512-row channel runs serve 129..512)
+    assert all(h.workspace_bytes(0) == 0 for h in handles[:449]) and all(h.workspace_bytes(0) > 0 for h in handles[449:])
     assert lib.library().orx_workspace_bytes(None, 0, None) == lib.ORX_ERR_BAD_ARGUMENT
 
 
@@ -533,7 +534,7 @@ def test_projections_take_the_reference_factories_schedule_names():
             assert hinted.geometry(rows) == forced.geometry(rows), (hint, rows)
         for rows in beyond:
             assert hinted.geometry(rows) == plain.geometry(rows), (hint, rows)
-    assert q4(block_m=96).geometry(20) != plain.geometry(20) and q4(block_m=192).geometry(200) != plain.geometry(200)
+    assert q4(block_m=96).geometry(20) != plain.geometry(20) and q4(block_m=192).geometry(100) != plain.geometry(100)
     w8_shape = dict(M=256, N=512, K=1024, dynamic_rows=True)
     w8 = lib.Kernel("int8_projection", **w8_shape, block_m=16, block_n=64, block_k=64, stages=2)
     assert w8.geometry(20) == lib.Kernel("int8_projection", **w8_shape, block_m=32).geometry(20)
@@ -562,7 +563,12 @@ def test_tall_tiles_by_name_and_for_handles_without_scratch():
     for rows in (257, 384, 512):
         assert scratch.geometry(rows) == tall.geometry(rows) and scratch.workspace_bytes(rows) == 0
     assert scratch.geometry(513) != tall.geometry(513) and scratch.workspace_bytes(513) >= 17408 * 5120
-    assert plain.geometry(256) != tall.geometry(256) and scratch.geometry(256) != tall.geometry(256)
+    # 129..256 rows: only where every CU gets 4.25 blocks of 16 channels in one round (17408 = 16 * 4.25 * 256)
+    for rows in (129, 256):
+        assert plain.geometry(rows) == tall.geometry(rows) == scratch.geometry(rows) and scratch.workspace_bytes(rows) == 0
+    assert plain.geometry(128) != tall.geometry(128) and scratch.geometry(128) != tall.geometry(128)
+    narrower = lib.Kernel("e8p_q4_projection", **dict(shape, N=17408 - 16))
+    assert narrower.geometry(256) != tall.geometry(256) and narrower.geometry(257)[1] == (512, 1, 1)
     for symbol, bad in (("int8_projection", dict(M=8, N=256, K=512)), ("e8p_q4_projection", dict(M=8, N=256, K=128))):
         with pytest.raises(lib.OrxError) as err:
             lib.Kernel(symbol, **bad, algorithm="tall")

@@ -412,9 +412,9 @@ def test_mid_row_projections_split_k_steps_evenly(codec, m, n, k, dtype):
         symbol, stored = "int8_projection", gu.dev(weights)
         call = lambda kern, out: kern(A=gu.dev(a), Output=out, TokenScale=gu.dev(a_s), Weight=stored, WeightScale=gu.dev(scales))
     variant = dict(M=m, N=n, K=k, output_dtype=dtype, output_stride=stride)
-    if m <= 64 or (codec == "q4" and m <= 128):
-        # `auto` gives so few rows of so small a matrix to the streaming kernel, and 65..128 rows of two-stage
-        # codes with a short K to the channel-run kernel
+    if m <= 64 or codec == "q4":
+        # `auto` gives so few rows of so small a matrix to the streaming kernel, 65..128 rows of two-stage codes with a
+        # short K to the channel-run kernel, and more rows of a matrix this wide to the 512-row channel runs
         variant["algorithm"] = "mfma"
     split = gu.kernel(symbol, **variant)
     whole = gu.kernel(symbol, split_k=False, **variant)
