@@ -212,11 +212,13 @@ def main():
     torch.cuda.synchronize()
     step_seconds = (time.perf_counter() - t0) / args.steps
     # the step is one launch: the GEMV that quantises its fp16 row during set-up
-    kernel_seconds = timed_graph(lambda i, s: main_case.project_fp16(i, s), max(min(args.steps, 260), copies))
+    # (260 launches per graph whatever K is: the events bracket the graph's own launch as well, which is 0.3 us per
+    # kernel in a graph of 20 and nothing in one of 260)
+    kernel_seconds = timed_graph(lambda i, s: main_case.project_fp16(i, s), max(260, copies))
     achieved = bytes_c1 / kernel_seconds / 1e9
     # for comparison: the same GEMV on a row that is already int8 (the quantiser is then a launch of its own)
     main_case.quantize(stream.cuda_stream)
-    plain_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(min(args.steps, 260), copies))
+    plain_seconds = timed_graph(lambda i, s: main_case.project(i, s), max(260, copies))
     traffic_bytes, traffic_kernel = measured_traffic(main_case.fused.geometry(1))
     # config 0 (the reference's own CPU-runnable shape) on the same kernel: a second roofline entry
     c0 = workloads.config0()
